@@ -1,0 +1,252 @@
+"""CPU oracle for the TOSA tensor-op hot path -- TEST INFRASTRUCTURE ONLY.
+
+numpy front end of ``libtosa_oracle.so`` (``tosa_oracle.c``), the plain-C restatement of the TOSA
+reference model's CONV2D / DEPTHWISE_CONV2D / MATMUL / RESCALE / CLAMP arithmetic.  Only the tests,
+the smoke test and the benchmark's CPU-baseline leg may import this package; the shipped library
+never does.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtosa_oracle.so")
+
+VALID, UNPREDICTABLE, ERROR = 0, 1, 2
+ROUND_SINGLE, ROUND_INEXACT, ROUND_DOUBLE = 1, 2, 3
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc (make).  Returns the path of the shared object."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _HERE], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+class ConvShape(ctypes.Structure):
+    _fields_ = [
+        ("N", ctypes.c_int32), ("IH", ctypes.c_int32), ("IW", ctypes.c_int32), ("IC", ctypes.c_int32),
+        ("OC", ctypes.c_int32), ("KH", ctypes.c_int32), ("KW", ctypes.c_int32),
+        ("OH", ctypes.c_int32), ("OW", ctypes.c_int32),
+        ("pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("dilation", ctypes.c_int32 * 2),
+        ("bias_len", ctypes.c_int32),
+    ]
+
+
+class RescaleAttr(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "in_bits", "out_bits", "scale32", "rounding_mode", "per_channel",
+        "input_unsigned", "output_unsigned", "in_zp", "out_zp")]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+        _lib.orc_apply_scale_32.restype = ctypes.c_int32
+        _lib.orc_apply_scale_32.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int,
+                                            ctypes.POINTER(ctypes.c_int)]
+        _lib.orc_apply_scale_16.restype = ctypes.c_int32
+        _lib.orc_apply_scale_16.argtypes = [ctypes.c_int64, ctypes.c_int16, ctypes.c_int32,
+                                            ctypes.POINTER(ctypes.c_int)]
+    return _lib
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(a), dtype=dtype)
+
+
+def conv_out_hw(ih, iw, kh, kw, pad, stride, dilation):
+    """Output height/width rule of check_conv_attribute (tensor_ops.cpp:203-223); None if inexact."""
+    fh = ih - 1 + pad[0] + pad[1] - (kh - 1) * dilation[0]
+    fw = iw - 1 + pad[2] + pad[3] - (kw - 1) * dilation[1]
+    if fh % stride[0] or fw % stride[1] or fh < 0 or fw < 0:
+        return None
+    return fh // stride[0] + 1, fw // stride[1] + 1
+
+
+def _shape(inp, kh, kw, oc, bias, pad, stride, dilation, out_hw=None) -> ConvShape:
+    n, ih, iw, ic = inp.shape
+    if out_hw is None:
+        out_hw = conv_out_hw(ih, iw, kh, kw, pad, stride, dilation) or (-1, -1)
+    s = ConvShape()
+    s.N, s.IH, s.IW, s.IC = n, ih, iw, ic
+    s.OC, s.KH, s.KW = oc, kh, kw
+    s.OH, s.OW = out_hw
+    s.pad[:] = list(pad)
+    s.stride[:] = list(stride)
+    s.dilation[:] = list(dilation)
+    s.bias_len = int(np.asarray(bias).shape[0])
+    return s
+
+
+class OracleStatus(Exception):
+    def __init__(self, status):
+        super().__init__(f"oracle status {status}")
+        self.status = status
+
+
+def _check(rc, allow=(VALID,)):
+    if rc not in allow:
+        raise OracleStatus(rc)
+    return rc
+
+
+_KINDS = {
+    "i8": (np.int8, np.int32, np.int32),      # element dtype, bias dtype, output dtype
+    "i32": (np.int32, np.int32, np.int32),
+    "f32": (np.float32, np.float32, np.float32),
+    "f64": (np.float64, np.float64, np.float64),
+}
+
+
+def conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0,
+           abs_mode=False, out_hw=None):
+    """CONV2D.  inp NHWC, w OHWI, bias [1] or [OC].  kind in i8/i32/f32/f64."""
+    et, bt, ot = _KINDS[kind]
+    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    oc, kh, kw, _ = w.shape
+    s = _shape(inp, kh, kw, oc, bias, pad, stride, dilation, out_hw)
+    if w.shape[3] != inp.shape[3]:
+        raise OracleStatus(ERROR)
+    out = np.zeros((s.N, max(s.OH, 0), max(s.OW, 0), oc), dtype=ot)
+    L = lib()
+    if kind in ("i8", "i32"):
+        fn = L.orc_conv2d_i8 if kind == "i8" else L.orc_conv2d_i32
+        rc = fn(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp), ctypes.c_int32(w_zp),
+                _ptr(out))
+    elif kind == "f32":
+        rc = L.orc_conv2d_f32(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), _ptr(out))
+    else:
+        rc = L.orc_conv2d_f64(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int(int(abs_mode)),
+                              _ptr(out))
+    _check(rc)
+    return out
+
+
+def depthwise_conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0,
+                     abs_mode=False, out_hw=None):
+    """DEPTHWISE_CONV2D.  inp NHWC, w [KH,KW,C,M], bias [1] or [C*M]."""
+    et, bt, ot = _KINDS[kind]
+    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    kh, kw, c, m = w.shape
+    if c != inp.shape[3]:
+        raise OracleStatus(ERROR)
+    s = _shape(inp, kh, kw, c * m, bias, pad, stride, dilation, out_hw)
+    out = np.zeros((s.N, max(s.OH, 0), max(s.OW, 0), c * m), dtype=ot)
+    L = lib()
+    if kind in ("i8", "i32"):
+        fn = L.orc_depthwise_i8 if kind == "i8" else L.orc_depthwise_i32
+        rc = fn(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp),
+                ctypes.c_int32(w_zp), _ptr(out))
+    elif kind == "f32":
+        rc = L.orc_depthwise_f32(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias), _ptr(out))
+    else:
+        rc = L.orc_depthwise_f64(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias),
+                                 ctypes.c_int(int(abs_mode)), _ptr(out))
+    _check(rc)
+    return out
+
+
+def matmul(kind, a, b, a_zp=0, b_zp=0, abs_mode=False):
+    """MATMUL a[N,H,C] x b[N,C,W] -> [N,H,W]."""
+    et, _, ot = _KINDS[kind]
+    a, b = _c(a, et), _c(b, et)
+    n, h, c = a.shape
+    if b.shape[0] != n or b.shape[1] != c:
+        raise OracleStatus(ERROR)
+    w = b.shape[2]
+    out = np.zeros((n, h, w), dtype=ot)
+    L = lib()
+    dims = [ctypes.c_int32(v) for v in (n, h, c, w)]
+    if kind in ("i8", "i32"):
+        fn = L.orc_matmul_i8 if kind == "i8" else L.orc_matmul_i32
+        rc = fn(*dims, _ptr(a), _ptr(b), ctypes.c_int32(a_zp), ctypes.c_int32(b_zp), _ptr(out))
+    elif kind == "f32":
+        rc = L.orc_matmul_f32(*dims, _ptr(a), _ptr(b), _ptr(out))
+    else:
+        rc = L.orc_matmul_f64(*dims, _ptr(a), _ptr(b), ctypes.c_int(int(abs_mode)), _ptr(out))
+    _check(rc)
+    return out
+
+
+def apply_scale_32(value, multiplier, shift, double_round=True):
+    """Returns (result, status)."""
+    st = ctypes.c_int(VALID)
+    r = lib().orc_apply_scale_32(int(value), int(multiplier), int(shift), int(bool(double_round)), ctypes.byref(st))
+    return int(r), st.value
+
+
+def apply_scale_16(value, multiplier, shift):
+    st = ctypes.c_int(VALID)
+    r = lib().orc_apply_scale_16(int(value), int(multiplier), int(shift), ctypes.byref(st))
+    return int(r), st.value
+
+
+_BITS = {np.dtype(np.int8): 8, np.dtype(np.uint8): 8, np.dtype(np.int16): 16, np.dtype(np.uint16): 16,
+         np.dtype(np.int32): 32}
+
+
+def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale32=True,
+            rounding_mode=ROUND_DOUBLE, per_channel=True, input_unsigned=False, output_unsigned=False):
+    """RESCALE.  Returns (out, status); out has dtype out_dtype (bit pattern of the stored value)."""
+    inp = np.asarray(inp)
+    out_dtype = np.dtype(out_dtype)
+    a = RescaleAttr()
+    a.in_bits, a.out_bits = _BITS[inp.dtype], _BITS[out_dtype]
+    a.scale32, a.rounding_mode, a.per_channel = int(scale32), int(rounding_mode), int(per_channel)
+    a.input_unsigned, a.output_unsigned = int(input_unsigned), int(output_unsigned)
+    # the zero-point tensors hold the stored (sign-interpreted) value of their dtype
+    a.in_zp = int(np.array(in_zp).astype(np.int64).astype(_signed(inp.dtype)))
+    a.out_zp = int(np.array(out_zp).astype(np.int64).astype(_signed(out_dtype)))
+    rank = inp.ndim
+    C = inp.shape[-1] if rank > 0 else 1
+    rows = int(np.prod(inp.shape[:-1], dtype=np.int64)) if rank > 0 else 1
+    stored = _c(inp.view(_signed(inp.dtype)) if inp.dtype.kind == "u" else inp, np.int32)
+    mult = _c(np.atleast_1d(multiplier), np.int32)
+    sh = _c(np.atleast_1d(shift), np.int32)
+    out = np.zeros(inp.shape, dtype=np.int32)
+    rc = lib().orc_rescale(ctypes.byref(a), ctypes.c_int64(rows), ctypes.c_int32(C), _ptr(stored), _ptr(mult),
+                           _ptr(sh), ctypes.c_int32(mult.size), ctypes.c_int32(sh.size), ctypes.c_int32(rank),
+                           _ptr(out))
+    # narrow to the output dtype keeping the low bits (uint16 32832 is stored as such)
+    narrowed = out.astype(np.int64).astype(_signed(out_dtype), casting="unsafe") if out_dtype.kind != "u" else \
+        (out.astype(np.int64) & ((1 << (8 * out_dtype.itemsize)) - 1)).astype(out_dtype)
+    return narrowed, rc
+
+
+def _signed(dt):
+    dt = np.dtype(dt)
+    return {1: np.int8, 2: np.int16, 4: np.int32}[dt.itemsize]
+
+
+def clamp(inp, lo, hi, nan_mode=1):
+    """CLAMP; integer dtypes go through the int32 storage path, floats through float32 storage."""
+    inp = np.asarray(inp)
+    if inp.dtype.kind in "iu":
+        x = _c(inp, np.int32)
+        out = np.zeros_like(x)
+        rc = lib().orc_clamp_i32(ctypes.c_int64(x.size), _ptr(x), ctypes.c_int32(int(lo)), ctypes.c_int32(int(hi)),
+                                 _ptr(out))
+        _check(rc)
+        return out.astype(inp.dtype)
+    x = _c(inp, np.float32)
+    out = np.zeros_like(x)
+    rc = lib().orc_clamp_f32(ctypes.c_int64(x.size), _ptr(x), ctypes.c_float(lo), ctypes.c_float(hi),
+                             ctypes.c_int(nan_mode), _ptr(out))
+    _check(rc)
+    return out.astype(inp.dtype)

@@ -1,0 +1,524 @@
+/*
+ * CPU oracle for the TOSA tensor-op hot path.  TEST INFRASTRUCTURE ONLY: the checker for the parity
+ * tests and the timed CPU baseline; never linked into, loaded by or called from the shipped library.
+ *
+ * Each function restates one piece of the TOSA reference model on flat row-major buffers, keeping
+ * the reference's loop nest, its storage types (int32 per INT8 element, float per FP16/BF16
+ * element, double in precise mode) and its accumulator types.  Build with -fno-strict-overflow /
+ * -fwrapv: the reference is built with -fno-strict-overflow and its int32 accumulators wrap.
+ */
+#include "tosa_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------------------------------
+ * check_conv_attribute (reference_model/src/ops/tensor_ops.cpp:120-226) and the ERROR_IFs that
+ * open OpConv2d::eval / OpDepthwiseConv2d::eval (tensor_ops.cpp:742-748, 1191-1197).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m)
+{
+    for (int i = 0; i < 4; i++)
+        if (s->pad[i] < 0)
+            return ORC_ERROR;
+    for (int i = 0; i < 2; i++)
+        if (s->stride[i] < 1 || s->dilation[i] < 1)
+            return ORC_ERROR;
+
+    const int32_t full_h = s->IH - 1 + s->pad[0] + s->pad[1] - (s->KH - 1) * s->dilation[0];
+    const int32_t full_w = s->IW - 1 + s->pad[2] + s->pad[3] - (s->KW - 1) * s->dilation[1];
+    if ((full_h % s->stride[0]) != 0 || (full_w % s->stride[1]) != 0)
+        return ORC_ERROR;
+    if (s->OH != full_h / s->stride[0] + 1 || s->OW != full_w / s->stride[1] + 1)
+        return ORC_ERROR;
+
+    if (depthwise_m > 0 && s->IC * depthwise_m != s->OC)
+        return ORC_ERROR;
+    if (s->bias_len != s->OC && s->bias_len != 1)
+        return ORC_ERROR;
+    return ORC_VALID;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpConv2d::eval (tensor_ops.cpp:723-882).
+ * The reference materialises a copy padded with input_zp (:807-808), initialises the output with the
+ * broadcast bias (:814-823), then runs ob,oy,ox,oc x ky,kx x ic, skipping out-of-image taps
+ * (:845-852; bounds mode visits them, where the padded value minus input_zp contributes zero) and
+ * finally stores bias + acc (:868-869).
+ * ---------------------------------------------------------------------------------------------- */
+#define ORC_DEFINE_CONV2D(NAME, T, ABS_EXPR)                                                                       \
+    static int NAME(const orc_conv_shape_t* s, const T* in, const T* w, const T* bias, T in_zp, T w_zp,          \
+                    int abs_mode, T* out)                                                                          \
+    {                                                                                                              \
+        if (orc_conv_check(s, 0) != ORC_VALID)                                                                     \
+            return ORC_ERROR;                                                                                      \
+        const int N = s->N, IH = s->IH, IW = s->IW, IC = s->IC, OC = s->OC, KH = s->KH, KW = s->KW;                \
+        const int OH = s->OH, OW = s->OW;                                                                          \
+        const int pt = s->pad[0], pb = s->pad[1], pl = s->pad[2], pr = s->pad[3];                                  \
+        const int sy = s->stride[0], sx = s->stride[1], dy = s->dilation[0], dx = s->dilation[1];                  \
+        const int PH = IH + pt + pb, PW = IW + pl + pr;                                                            \
+        const size_t n_w = (size_t)OC * KH * KW * IC;                                                              \
+        T* padded        = (T*)malloc(sizeof(T) * (size_t)N * PH * PW * IC + 1);                                   \
+        T* wv            = (T*)malloc(sizeof(T) * n_w + 1);                                                        \
+        if (!padded || !wv)                                                                                        \
+        {                                                                                                          \
+            free(padded);                                                                                          \
+            free(wv);                                                                                              \
+            return ORC_ERROR;                                                                                      \
+        }                                                                                                          \
+        for (size_t i = 0; i < n_w; i++)                                                                           \
+            wv[i] = abs_mode ? ABS_EXPR(w[i]) : w[i];                                                              \
+        for (int n = 0; n < N; n++)                                                                                \
+            for (int y = 0; y < PH; y++)                                                                           \
+                for (int x = 0; x < PW; x++)                                                                       \
+                    for (int c = 0; c < IC; c++)                                                                   \
+                    {                                                                                              \
+                        const int iy = y - pt, ix = x - pl;                                                        \
+                        T v = in_zp;                                                                               \
+                        if (iy >= 0 && iy < IH && ix >= 0 && ix < IW)                                              \
+                        {                                                                                          \
+                            v = in[(((size_t)n * IH + iy) * IW + ix) * IC + c];                                    \
+                            if (abs_mode)                                                                          \
+                                v = ABS_EXPR(v);                                                                   \
+                        }                                                                                          \
+                        padded[(((size_t)n * PH + y) * PW + x) * IC + c] = v;                                      \
+                    }                                                                                              \
+        for (int ob = 0; ob < N; ob++)                                                                             \
+            for (int oy = 0; oy < OH; oy++)                                                                        \
+                for (int ox = 0; ox < OW; ox++)                                                                    \
+                    for (int oc = 0; oc < OC; oc++)                                                                \
+                    {                                                                                              \
+                        T acc = 0;                                                                                 \
+                        for (int ky = 0; ky < KH; ky++)                                                            \
+                        {                                                                                          \
+                            const int iy_pad = oy * sy + ky * dy;                                                  \
+                            for (int kx = 0; kx < KW; kx++)                                                        \
+                            {                                                                                      \
+                                const int ix_pad = ox * sx + kx * dx;                                              \
+                                const int y = iy_pad - pt, x = ix_pad - pl;                                        \
+                                const int in_scope = (0 <= x && x < IW) && (0 <= y && y < IH);                     \
+                                if (!in_scope && !abs_mode)                                                        \
+                                    continue;                                                                      \
+                                const T* ip = padded + (((size_t)ob * PH + iy_pad) * PW + ix_pad) * IC;            \
+                                const T* wp = wv + (((size_t)oc * KH + ky) * KW + kx) * IC;                        \
+                                for (int ic = 0; ic < IC; ic++)                                                    \
+                                    acc += (ip[ic] - in_zp) * (wp[ic] - w_zp);                                     \
+                            }                                                                                      \
+                        }                                                                                          \
+                        T b = bias[s->bias_len == 1 ? 0 : oc];                                                     \
+                        if (abs_mode)                                                                              \
+                            b = ABS_EXPR(b);                                                                       \
+                        out[(((size_t)ob * OH + oy) * OW + ox) * OC + oc] = b + acc;                               \
+                    }                                                                                              \
+        free(padded);                                                                                              \
+        free(wv);                                                                                                  \
+        return ORC_VALID;                                                                                          \
+    }
+
+#define ORC_ABS_I32(v) ((v) < 0 ? -(v) : (v))
+#define ORC_ABS_F32(v) fabsf(v)
+#define ORC_ABS_F64(v) fabs(v)
+
+ORC_DEFINE_CONV2D(conv2d_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_CONV2D(conv2d_f32_impl, float, ORC_ABS_F32)
+ORC_DEFINE_CONV2D(conv2d_f64_impl, double, ORC_ABS_F64)
+
+int orc_conv2d_i32(const orc_conv_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                   int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    return conv2d_i32_impl(s, in, w, bias, in_zp, w_zp, 0, out);
+}
+
+int orc_conv2d_f32(const orc_conv_shape_t* s, const float* in, const float* w, const float* bias, float* out)
+{
+    return conv2d_f32_impl(s, in, w, bias, 0.0f, 0.0f, 0, out);
+}
+
+int orc_conv2d_f64(const orc_conv_shape_t* s, const double* in, const double* w, const double* bias, int abs_mode,
+                   double* out)
+{
+    return conv2d_f64_impl(s, in, w, bias, 0.0, 0.0, abs_mode, out);
+}
+
+static int32_t* widen_i8(const int8_t* p, size_t n)
+{
+    int32_t* r = (int32_t*)malloc(sizeof(int32_t) * n + 4);
+    if (r)
+        for (size_t i = 0; i < n; i++)
+            r[i] = (int32_t)p[i];
+    return r;
+}
+
+int orc_conv2d_i8(const orc_conv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias, int32_t in_zp,
+                  int32_t w_zp, int32_t* out)
+{
+    if (orc_conv_check(s, 0) != ORC_VALID)
+        return ORC_ERROR;
+    int32_t* in32 = widen_i8(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int32_t* w32  = widen_i8(w, (size_t)s->OC * s->KH * s->KW * s->IC);
+    int rc        = (in32 && w32) ? orc_conv2d_i32(s, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
+    free(in32);
+    free(w32);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpDepthwiseConv2d::eval (tensor_ops.cpp:1172-1334): ob,oy,ox,ic,km x ky,kx; an out-of-image tap
+ * contributes zero (:1302-1313); weight [KH,KW,IC,M]; output channel ic*M+km (:1320).
+ * ---------------------------------------------------------------------------------------------- */
+#define ORC_DEFINE_DEPTHWISE(NAME, T, ABS_EXPR)                                                                    \
+    static int NAME(const orc_conv_shape_t* s, int32_t M, const T* in, const T* w, const T* bias, T in_zp,        \
+                    T w_zp, int abs_mode, T* out)                                                                  \
+    {                                                                                                              \
+        if (M < 1 || orc_conv_check(s, M) != ORC_VALID)                                                            \
+            return ORC_ERROR;                                                                                      \
+        const int N = s->N, IH = s->IH, IW = s->IW, IC = s->IC, OC = s->OC, KH = s->KH, KW = s->KW;                \
+        const int OH = s->OH, OW = s->OW;                                                                          \
+        const int pt = s->pad[0], pl = s->pad[2];                                                                  \
+        const int sy = s->stride[0], sx = s->stride[1], dy = s->dilation[0], dx = s->dilation[1];                  \
+        for (int ob = 0; ob < N; ob++)                                                                             \
+            for (int oy = 0; oy < OH; oy++)                                                                        \
+                for (int ox = 0; ox < OW; ox++)                                                                    \
+                    for (int ic = 0; ic < IC; ic++)                                                                \
+                        for (int km = 0; km < M; km++)                                                             \
+                        {                                                                                          \
+                            T acc        = 0;                                                                      \
+                            const int iy = oy * sy - pt, ix = ox * sx - pl;                                        \
+                            for (int ky = 0; ky < KH; ky++)                                                        \
+                                for (int kx = 0; kx < KW; kx++)                                                    \
+                                {                                                                                  \
+                                    const int y = iy + ky * dy, x = ix + kx * dx;                                  \
+                                    const int in_scope = (0 <= y && y < IH) && (0 <= x && x < IW);                 \
+                                    if (!in_scope)                                                                 \
+                                        continue;                                                                  \
+                                    T a = in[(((size_t)ob * IH + y) * IW + x) * IC + ic];                          \
+                                    T b = w[(((size_t)ky * KW + kx) * IC + ic) * M + km];                          \
+                                    if (abs_mode)                                                                  \
+                                    {                                                                              \
+                                        a = ABS_EXPR(a);                                                           \
+                                        b = ABS_EXPR(b);                                                           \
+                                    }                                                                              \
+                                    acc += (a - in_zp) * (b - w_zp);                                               \
+                                }                                                                                  \
+                            const int oc = ic * M + km;                                                            \
+                            T bv         = bias[s->bias_len == 1 ? 0 : oc];                                        \
+                            if (abs_mode)                                                                          \
+                                bv = ABS_EXPR(bv);                                                                 \
+                            out[(((size_t)ob * OH + oy) * OW + ox) * OC + oc] = bv + acc;                          \
+                        }                                                                                          \
+        return ORC_VALID;                                                                                          \
+    }
+
+ORC_DEFINE_DEPTHWISE(depthwise_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_DEPTHWISE(depthwise_f32_impl, float, ORC_ABS_F32)
+ORC_DEFINE_DEPTHWISE(depthwise_f64_impl, double, ORC_ABS_F64)
+
+int orc_depthwise_i32(const orc_conv_shape_t* s, int32_t M, const int32_t* in, const int32_t* w,
+                      const int32_t* bias, int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    return depthwise_i32_impl(s, M, in, w, bias, in_zp, w_zp, 0, out);
+}
+
+int orc_depthwise_i8(const orc_conv_shape_t* s, int32_t M, const int8_t* in, const int8_t* w, const int32_t* bias,
+                     int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    if (M < 1 || orc_conv_check(s, M) != ORC_VALID)
+        return ORC_ERROR;
+    int32_t* in32 = widen_i8(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int32_t* w32  = widen_i8(w, (size_t)s->KH * s->KW * s->IC * M);
+    int rc        = (in32 && w32) ? orc_depthwise_i32(s, M, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
+    free(in32);
+    free(w32);
+    return rc;
+}
+
+int orc_depthwise_f32(const orc_conv_shape_t* s, int32_t M, const float* in, const float* w, const float* bias,
+                      float* out)
+{
+    return depthwise_f32_impl(s, M, in, w, bias, 0.0f, 0.0f, 0, out);
+}
+
+int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, const double* w, const double* bias,
+                      int abs_mode, double* out)
+{
+    return depthwise_f64_impl(s, M, in, w, bias, 0.0, 0.0, abs_mode, out);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpMatMul::eval (tensor_ops.cpp:1423-1492): per batch, widen to the accumulator type, subtract the
+ * zero points, contract over C.  Integer sums are order independent modulo 2^32; the floating-point
+ * summation order of Eigen's contraction is not restated (sequential in c here).
+ * ---------------------------------------------------------------------------------------------- */
+#define ORC_DEFINE_MATMUL(NAME, T, ABS_EXPR)                                                                       \
+    static int NAME(int32_t N, int32_t H, int32_t C, int32_t W, const T* a, const T* b, T a_zp, T b_zp,           \
+                    int abs_mode, T* out)                                                                          \
+    {                                                                                                              \
+        if (N < 0 || H < 0 || C < 0 || W < 0)                                                                      \
+            return ORC_ERROR;                                                                                      \
+        T* row = (T*)malloc(sizeof(T) * (size_t)(W > 0 ? W : 1));                                                  \
+        if (!row)                                                                                                  \
+            return ORC_ERROR;                                                                                      \
+        for (int n = 0; n < N; n++)                                                                                \
+            for (int h = 0; h < H; h++)                                                                            \
+            {                                                                                                      \
+                for (int x = 0; x < W; x++)                                                                        \
+                    row[x] = 0;                                                                                    \
+                for (int c = 0; c < C; c++)                                                                        \
+                {                                                                                                  \
+                    T av = a[((size_t)n * H + h) * C + c];                                                         \
+                    if (abs_mode)                                                                                  \
+                        av = ABS_EXPR(av);                                                                         \
+                    av -= a_zp;                                                                                    \
+                    const T* bp = b + ((size_t)n * C + c) * W;                                                     \
+                    for (int x = 0; x < W; x++)                                                                    \
+                    {                                                                                              \
+                        T bv = bp[x];                                                                              \
+                        if (abs_mode)                                                                              \
+                            bv = ABS_EXPR(bv);                                                                     \
+                        row[x] += av * (bv - b_zp);                                                                \
+                    }                                                                                              \
+                }                                                                                                  \
+                memcpy(out + ((size_t)n * H + h) * W, row, sizeof(T) * (size_t)W);                                 \
+            }                                                                                                      \
+        free(row);                                                                                                 \
+        return ORC_VALID;                                                                                          \
+    }
+
+ORC_DEFINE_MATMUL(matmul_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_MATMUL(matmul_f32_impl, float, ORC_ABS_F32)
+ORC_DEFINE_MATMUL(matmul_f64_impl, double, ORC_ABS_F64)
+
+int orc_matmul_i32(int32_t N, int32_t H, int32_t C, int32_t W, const int32_t* a, const int32_t* b, int32_t a_zp,
+                   int32_t b_zp, int32_t* out)
+{
+    return matmul_i32_impl(N, H, C, W, a, b, a_zp, b_zp, 0, out);
+}
+
+int orc_matmul_i8(int32_t N, int32_t H, int32_t C, int32_t W, const int8_t* a, const int8_t* b, int32_t a_zp,
+                  int32_t b_zp, int32_t* out)
+{
+    int32_t* a32 = widen_i8(a, (size_t)N * H * C);
+    int32_t* b32 = widen_i8(b, (size_t)N * C * W);
+    int rc       = (a32 && b32) ? orc_matmul_i32(N, H, C, W, a32, b32, a_zp, b_zp, out) : ORC_ERROR;
+    free(a32);
+    free(b32);
+    return rc;
+}
+
+int orc_matmul_f32(int32_t N, int32_t H, int32_t C, int32_t W, const float* a, const float* b, float* out)
+{
+    return matmul_f32_impl(N, H, C, W, a, b, 0.0f, 0.0f, 0, out);
+}
+
+int orc_matmul_f64(int32_t N, int32_t H, int32_t C, int32_t W, const double* a, const double* b, int abs_mode,
+                   double* out)
+{
+    return matmul_f64_impl(N, H, C, W, a, b, 0.0, 0.0, abs_mode, out);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * QuantUtil::apply_scale_32 / apply_scale_16 (reference_model/src/quant_util.h:45-108).
+ * ---------------------------------------------------------------------------------------------- */
+int32_t orc_apply_scale_32(int32_t value, int32_t multiplier, int32_t shift, int double_round, int* status)
+{
+    if (multiplier < 0 || shift < 2 || shift > 62)
+    {
+        *status = ORC_UNPREDICTABLE;
+        return 0;
+    }
+    const int64_t low_val  = -(INT64_C(1) << (shift - 1));
+    const int64_t high_val = INT64_C(1) << (shift - 1);
+    if ((int64_t)value < low_val || (int64_t)value >= high_val)
+    {
+        *status = ORC_UNPREDICTABLE;
+        return 0;
+    }
+    int64_t round = INT64_C(1) << (shift - 1);
+    if (double_round)
+    {
+        if (shift > 31 && value >= 0)
+            round += INT64_C(1) << 30;
+        if (shift > 31 && value < 0)
+            round -= INT64_C(1) << 30;
+    }
+    int64_t result = (int64_t)value * (int64_t)multiplier + round;
+    result         = result >> shift;
+    if (result < -(INT64_C(1) << 31) || result >= (INT64_C(1) << 31))
+    {
+        *status = ORC_UNPREDICTABLE;
+        return 0;
+    }
+    return (int32_t)result;
+}
+
+int32_t orc_apply_scale_16(int64_t value, int16_t multiplier, int32_t shift, int* status)
+{
+    if (multiplier < 0 || shift < 2 || shift > 62)
+    {
+        *status = ORC_UNPREDICTABLE;
+        return 0;
+    }
+    const int64_t round = INT64_C(1) << (shift - 1);
+    int64_t result      = (int64_t)((uint64_t)value * (uint64_t)(int64_t)multiplier + (uint64_t)round);
+    result              = result >> shift;
+    if (result < -(INT64_C(1) << 31) || result >= (INT64_C(1) << 31))
+    {
+        *status = ORC_UNPREDICTABLE;
+        return 0;
+    }
+    return (int32_t)result;
+}
+
+/* value_extend64_impl (reference_model/src/ops/type_conversion.cpp:183-221) for 8/16/32-bit types. */
+static int64_t value_extend64(int32_t val, int bits, int is_unsigned)
+{
+    switch (bits)
+    {
+        case 8:
+            return is_unsigned ? (int64_t)(uint8_t)(int8_t)val : (int64_t)(int8_t)(uint8_t)(val & 0xFF);
+        case 16:
+            return is_unsigned ? (int64_t)(uint16_t)(int16_t)val : (int64_t)(int16_t)(uint16_t)(val & 0xFFFF);
+        case 32:
+            return is_unsigned ? (int64_t)(uint32_t)val : (int64_t)val;
+        default:
+            return (int64_t)val;
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpRescale::checkTensorAttributes + eval (type_conversion.cpp:72-154, 224-421).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
+                const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out)
+{
+    const int i8in = a->in_bits == 8, i16in = a->in_bits == 16, i32in = a->in_bits == 32;
+    const int i8out = a->out_bits == 8, i16out = a->out_bits == 16, i32out = a->out_bits == 32;
+    if (!(i8in || i16in || i32in) || !(i8out || i16out || i32out))
+        return ORC_ERROR;
+
+    /* checkTensorAttributes :118-151 */
+    if (a->rounding_mode != ORC_ROUND_SINGLE && a->rounding_mode != ORC_ROUND_DOUBLE &&
+        a->rounding_mode != ORC_ROUND_INEXACT)
+        return ORC_ERROR;
+    if (!a->scale32 && a->rounding_mode == ORC_ROUND_DOUBLE)
+        return ORC_ERROR;
+    if (a->input_unsigned && a->output_unsigned)
+        return ORC_ERROR;
+    if (i32out && a->input_unsigned)
+        return ORC_ERROR;
+    if (i32in && a->output_unsigned)
+        return ORC_ERROR;
+    if (i32in && a->input_unsigned)
+        return ORC_ERROR;
+    if (i32out && a->output_unsigned)
+        return ORC_ERROR;
+    if (a->per_channel)
+    {
+        if (rank < 1 || n_mult != C || n_shift != C)
+            return ORC_ERROR;
+    }
+    else if (n_mult != 1 || n_shift != 1)
+        return ORC_ERROR;
+
+    /* eval :242-255 */
+    const int64_t out_zp_ext = value_extend64(a->out_zp, a->out_bits, a->output_unsigned);
+    const int64_t in_zp_ext  = value_extend64(a->in_zp, a->in_bits, a->input_unsigned);
+    if (!i8in && !(i16in && a->input_unsigned) && in_zp_ext != 0)
+        return ORC_ERROR;
+    if (!i8out && !(i16out && a->output_unsigned) && out_zp_ext != 0)
+        return ORC_ERROR;
+    if (i16in && a->input_unsigned && in_zp_ext != 0 && in_zp_ext != 32768)
+        return ORC_ERROR;
+    if (i16out && a->output_unsigned && out_zp_ext != 0 && out_zp_ext != 32768)
+        return ORC_ERROR;
+
+    /* getSigned/UnsignedMinimum/Maximum for the output type (type_conversion.cpp:61-64) */
+    int64_t qmin, qmax;
+    if (a->output_unsigned)
+    {
+        qmin = 0;
+        qmax = i8out ? 255 : (i16out ? 65535 : (int64_t)INT32_MAX); /* u32 max is capped to int32 max by applyClip */
+    }
+    else
+    {
+        qmin = i8out ? -128 : (i16out ? -32768 : (int64_t)INT32_MIN);
+        qmax = i8out ? 127 : (i16out ? 32767 : (int64_t)INT32_MAX);
+    }
+
+    const int double_round = a->rounding_mode == ORC_ROUND_DOUBLE;
+    const int inexact      = a->rounding_mode == ORC_ROUND_INEXACT;
+    int status             = ORC_VALID;
+
+    /* The reference walks channel by channel when per_channel is set (:381-394) and stops at the first
+     * throw; results after a REQUIRE failure are unspecified, so the element order here is free. */
+    for (int64_t r = 0; r < rows && status == ORC_VALID; r++)
+        for (int32_t c = 0; c < C; c++)
+        {
+            const int32_t m  = a->per_channel ? multiplier[c] : multiplier[0];
+            const int32_t sh = a->per_channel ? shift[c] : shift[0];
+            const int64_t v  = value_extend64(in[r * C + c], a->in_bits, a->input_unsigned) - in_zp_ext;
+            int32_t scaled;
+            if (!inexact)
+            {
+                if (a->scale32)
+                    scaled = orc_apply_scale_32((int32_t)v, m, sh, double_round, &status);
+                else
+                    scaled = orc_apply_scale_16(v, (int16_t)m, sh, &status);
+            }
+            else
+            {
+                /* INEXACT_ROUND with FP32 maths (:318-324), round to nearest even */
+                volatile float t = (float)v * (float)m;
+                volatile float u = t * exp2f((float)(-sh));
+                scaled           = (int32_t)rintf(u);
+            }
+            if (status != ORC_VALID)
+                break;
+            const int64_t res = (int64_t)scaled + out_zp_ext;
+            if (res > (int64_t)INT32_MAX || res < (int64_t)INT32_MIN)
+            {
+                status = ORC_UNPREDICTABLE;
+                break;
+            }
+            int64_t clipped = res < qmin ? qmin : res;
+            clipped         = clipped > qmax ? qmax : clipped;
+            out[r * C + c]  = (int32_t)clipped;
+        }
+    return status;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpClamp (reference_model/src/ops/activation_funcs.cpp:27-125) through applyClip
+ * (reference_model/src/arith_util.h:389-413).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out)
+{
+    if (hi < lo)
+        return ORC_ERROR;
+    for (int64_t i = 0; i < n; i++)
+    {
+        int32_t v = in[i] >= lo ? in[i] : lo;
+        out[i]    = v < hi ? v : hi;
+    }
+    return ORC_VALID;
+}
+
+int orc_clamp_f32(int64_t n, const float* in, float lo, float hi, int nan_mode, float* out)
+{
+    if (hi < lo || isnan(lo) || isnan(hi))
+        return ORC_ERROR;
+    for (int64_t i = 0; i < n; i++)
+    {
+        float v = in[i];
+        if (isnan(v))
+            v = (nan_mode == 1) ? NAN : lo; /* IGNORE: max(NaN, lo) -> lo, then min(lo, hi) -> lo */
+        else
+        {
+            v = v >= lo ? v : lo;
+            v = v < hi ? v : hi;
+        }
+        out[i] = v;
+    }
+    return ORC_VALID;
+}

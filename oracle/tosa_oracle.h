@@ -1,0 +1,127 @@
+/*
+ * CPU oracle for the TOSA tensor-op hot path (CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the arithmetic of the TOSA reference
+ * model, used as the checker in the parity tests, in the smoke test and as the timed CPU baseline.
+ * Nothing in the shipped library may call, link or load it.
+ *
+ * Every function works on flat row-major buffers.  Status codes follow the reference's GraphStatus
+ * (reference_model/include/graph_status.h:18-23): 0 = valid, 1 = unpredictable, 2 = error.
+ *
+ * Parity pins (see tests/test_oracle_*.py):
+ *   - conv2d int8 + rescale double-round per-channel: the reference's stored golden of
+ *     examples/test_conv2d_1x1_1x32x32x8_qi8_st11_padSAME_dilat11 (bit exact).
+ *   - conv2d / depthwise / matmul zero points and bias broadcast: the literal vectors of
+ *     reference_model/test/ref_model_tests/tensor_ops_tests.cpp:622-683,736-798.
+ *   - rescale: type_conversion_tests.cpp:324-405 literals, Python big-integer brute force of
+ *     quant_util.h:45-84 and the boundary operands of generate_int_special.cpp:119-131.
+ *   - large shapes: independent numpy int64 einsum / float64 convolution.
+ *   - fp accumulate order of MATMUL (Eigen contraction order): parity unpinned (tolerance covered).
+ */
+#ifndef TOSA_ORACLE_H
+#define TOSA_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum
+{
+    ORC_VALID         = 0,
+    ORC_UNPREDICTABLE = 1,
+    ORC_ERROR         = 2
+};
+
+/* rounding_mode values as serialized in RescaleAttribute */
+enum
+{
+    ORC_ROUND_SINGLE  = 1,
+    ORC_ROUND_INEXACT = 2,
+    ORC_ROUND_DOUBLE  = 3
+};
+
+typedef struct
+{
+    int32_t N, IH, IW, IC; /* input  NHWC */
+    int32_t OC, KH, KW;    /* weight OHWI (conv2d) ; depthwise: KH,KW,IC,M with OC = IC*M */
+    int32_t OH, OW;        /* declared output height/width */
+    int32_t pad[4];        /* top, bottom, left, right */
+    int32_t stride[2];     /* y, x */
+    int32_t dilation[2];   /* y, x */
+    int32_t bias_len;      /* 1 (broadcast) or OC */
+} orc_conv_shape_t;
+
+/* check_conv_attribute + the ERROR_IFs at the top of eval().  depthwise_m = 0 for CONV2D, else the
+ * channel multiplier M.  Returns ORC_VALID or ORC_ERROR. */
+int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m);
+
+/* CONV2D.  Elements are given in the reference's storage type (int32 for INT8, float for FP16/BF16/FP32,
+ * double in precise mode); accumulate in the same type as the reference's AccEigenType for that
+ * instantiation (int32 wraps; float; double).  abs_mode != 0 selects the bounds pass
+ * (|in|, |w|, |bias|, local_bound = true). */
+int orc_conv2d_i32(const orc_conv_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                   int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_conv2d_f32(const orc_conv_shape_t* s, const float* in, const float* w, const float* bias, float* out);
+int orc_conv2d_f64(const orc_conv_shape_t* s, const double* in, const double* w, const double* bias, int abs_mode,
+                   double* out);
+
+/* Same arithmetic on packed int8 operands (1 byte per element, as they sit in .npy files and in HBM),
+ * widened to the reference's int32 storage inside.  Convenience for tests; identical results. */
+int orc_conv2d_i8(const orc_conv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias, int32_t in_zp,
+                  int32_t w_zp, int32_t* out);
+
+/* DEPTHWISE_CONV2D, weight [KH,KW,IC,M], out channel = ic*M + m. */
+int orc_depthwise_i32(const orc_conv_shape_t* s, int32_t M, const int32_t* in, const int32_t* w,
+                      const int32_t* bias, int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_depthwise_i8(const orc_conv_shape_t* s, int32_t M, const int8_t* in, const int8_t* w, const int32_t* bias,
+                     int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_depthwise_f32(const orc_conv_shape_t* s, int32_t M, const float* in, const float* w, const float* bias,
+                      float* out);
+int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, const double* w, const double* bias,
+                      int abs_mode, double* out);
+
+/* MATMUL a[N,H,C] x b[N,C,W] -> out[N,H,W]. */
+int orc_matmul_i32(int32_t N, int32_t H, int32_t C, int32_t W, const int32_t* a, const int32_t* b, int32_t a_zp,
+                   int32_t b_zp, int32_t* out);
+int orc_matmul_i8(int32_t N, int32_t H, int32_t C, int32_t W, const int8_t* a, const int8_t* b, int32_t a_zp,
+                  int32_t b_zp, int32_t* out);
+int orc_matmul_f32(int32_t N, int32_t H, int32_t C, int32_t W, const float* a, const float* b, float* out);
+int orc_matmul_f64(int32_t N, int32_t H, int32_t C, int32_t W, const double* a, const double* b, int abs_mode,
+                   double* out);
+
+/* QuantUtil::apply_scale_32 / apply_scale_16.  *status is set to ORC_UNPREDICTABLE where the
+ * reference throws (the throw becomes a REQUIRE failure in OpRescale::eval). */
+int32_t orc_apply_scale_32(int32_t value, int32_t multiplier, int32_t shift, int double_round, int* status);
+int32_t orc_apply_scale_16(int64_t value, int16_t multiplier, int32_t shift, int* status);
+
+typedef struct
+{
+    int32_t in_bits;  /* 8, 16 or 32: nominal width of the input dtype  */
+    int32_t out_bits; /* 8, 16 or 32: nominal width of the output dtype */
+    int32_t scale32;
+    int32_t rounding_mode;
+    int32_t per_channel;
+    int32_t input_unsigned;
+    int32_t output_unsigned;
+    int32_t in_zp;  /* stored value of the input_zp tensor  (storage type int32) */
+    int32_t out_zp; /* stored value of the output_zp tensor (storage type int32) */
+} orc_rescale_attr_t;
+
+/* RESCALE on a tensor viewed as [rows, C] (C = last dimension, 1 for rank 0).  in/out hold one stored
+ * value per element in the reference's int32 storage type.  n_scale = number of multiplier / shift
+ * entries supplied.  Returns ORC_ERROR for the attribute/shape violations that the reference rejects,
+ * ORC_UNPREDICTABLE when a REQUIRE fires (output contents then unspecified), else ORC_VALID. */
+int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
+                const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out);
+
+/* CLAMP for the integer instantiations: min(max(x, lo), hi); ORC_ERROR when hi < lo. */
+int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out);
+/* CLAMP for float storage; nan_mode 1 = PROPAGATE, 2 = IGNORE. */
+int orc_clamp_f32(int64_t n, const float* in, float lo, float hi, int nan_mode, float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
