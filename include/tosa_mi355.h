@@ -1,0 +1,207 @@
+/*
+ * tosa_mi355.h -- C ABI of the MI355X (gfx950) implementation of the TOSA reference model's tensor-op
+ * hot path: CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP and their fused forms.
+ *
+ * The TOSA reference model has no C ABI for built-in operators: each operator is a C++ GraphNode
+ * subclass whose virtual eval() is called by SubgraphTraverser::evaluateNextNode()
+ * (reference_model/src/graph_node.h:176-179, reference_model/src/subgraph_traverser.cpp:856).  The entry
+ * points below are what a GraphNode adapter for these operators binds: one call per eval(), operands
+ * given as device pointers to packed row-major tensors, attributes as plain structs, and the
+ * reference's GraphStatus integer (reference_model/include/graph_status.h:18-23) as the return value.
+ *
+ * Conventions
+ *   - Every function returns TMI_VALID (0), TMI_UNPREDICTABLE (1) or TMI_ERROR (2); none throws.
+ *     TMI_ERROR corresponds to the reference's ERROR_IF / validation failures and is detected on the
+ *     host before anything is launched; tmi_last_error() then holds the message.
+ *   - Kernels are enqueued on the context's stream and the call returns without waiting.  The
+ *     conditions that the reference turns into REQUIRE failures while evaluating RESCALE
+ *     (reference_model/src/quant_util.h:48-82, reference_model/src/ops/type_conversion.cpp:348-360) are
+ *     detected on the device and latched in a per-context flag word; tmi_ctx_sync() waits for the
+ *     stream and returns TMI_UNPREDICTABLE if any was raised since the previous sync.
+ *   - Tensors are packed: INT8 1 byte, INT16/FP16/BF16 2 bytes, INT32/FP32 4 bytes per element
+ *     (the reference widens INT8 to int32 and FP16/BF16 to float in host memory:
+ *     reference_model/src/ops/template_types.h:67-163).  Layouts are those of the TOSA operators:
+ *     input/output NHWC, CONV2D weight OHWI, DEPTHWISE_CONV2D weight [KH,KW,C,M], MATMUL [N,H,C]x[N,C,W].
+ *   - Pointers named *_dev must be device memory (from tmi_buf_alloc or any other HIP allocation on the
+ *     context's device), 16-byte aligned for whole tensors.
+ *   - One context serves one host thread at a time (the reference is single threaded and keeps its
+ *     configuration in process globals: reference_model/src/model_runner.cpp:22-23).
+ */
+#ifndef TOSA_MI355_H
+#define TOSA_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GraphStatus values: reference_model/include/graph_status.h:18-23 */
+enum
+{
+    TMI_VALID         = 0,
+    TMI_UNPREDICTABLE = 1,
+    TMI_ERROR         = 2
+};
+
+/* Element types; the numbers are those of the serialized TOSA DType enum so that a graph loader can
+ * pass them through (INT8 = 3 and INT32 = 5 as found in the reference's example graphs). */
+enum
+{
+    TMI_INT8  = 3,
+    TMI_INT16 = 4,
+    TMI_INT32 = 5,
+    TMI_FP32  = 7,
+    TMI_FP16  = 8,
+    TMI_BF16  = 9
+};
+
+/* RescaleAttribute.rounding_mode as serialized (reference_model/src/ops/type_conversion.cpp:118-120) */
+enum
+{
+    TMI_ROUND_SINGLE  = 1,
+    TMI_ROUND_INEXACT = 2,
+    TMI_ROUND_DOUBLE  = 3
+};
+
+/* Bits of the device flag word reported by tmi_ctx_flags(): which REQUIRE condition fired. */
+enum
+{
+    TMI_FLAG_SCALE_MULTIPLIER = 1u << 0, /* multiplier < 0                      quant_util.h:48-52  */
+    TMI_FLAG_SCALE_SHIFT      = 1u << 1, /* shift outside [2,62]                quant_util.h:53-58  */
+    TMI_FLAG_SCALE_VALUE      = 1u << 2, /* value outside [-2^(s-1), 2^(s-1))   quant_util.h:59-67  */
+    TMI_FLAG_SCALE_RESULT     = 1u << 3, /* scaled result exceeds int32         quant_util.h:78-82  */
+    TMI_FLAG_ZP_RESULT        = 1u << 4  /* result + output_zp exceeds int32    type_conversion.cpp:352-360 */
+};
+
+typedef struct tmi_ctx tmi_ctx_t;
+
+/* ---- context -------------------------------------------------------------------------------------- */
+
+/* Creates a context on HIP device `device` with its own stream.  Replaces nothing in the reference
+ * (which has no device); plays the role of SubgraphTraverser as owner of per-graph state
+ * (reference_model/src/subgraph_traverser.cpp:56-80). */
+int tmi_ctx_create(tmi_ctx_t** out_ctx, int device);
+int tmi_ctx_destroy(tmi_ctx_t* ctx);
+
+/* Makes the context enqueue on a stream owned by the caller (a hipStream_t passed as void*; NULL selects
+ * the device's default stream).  The context never destroys a borrowed stream. */
+int tmi_ctx_set_stream(tmi_ctx_t* ctx, void* hip_stream);
+
+/* Waits for all enqueued work.  Returns TMI_UNPREDICTABLE if a device-side REQUIRE condition was latched
+ * since the last sync (and clears the latch), TMI_ERROR on a HIP failure, else TMI_VALID.
+ * Counterpart of reading SubgraphTraverser::getGraphStatus() after evaluateAll()
+ * (reference_model/src/model_runner_impl.cpp:56-126). */
+int tmi_ctx_sync(tmi_ctx_t* ctx);
+
+/* Flag bits (TMI_FLAG_*) seen by the most recent tmi_ctx_sync(). */
+uint32_t tmi_ctx_flags(const tmi_ctx_t* ctx);
+
+/* Message of the most recent TMI_ERROR on this context ("" if none).  The reference prints these with
+ * printNodeValidationError / ERROR_IF (reference_model/include/func_debug.h:143-158). */
+const char* tmi_last_error(const tmi_ctx_t* ctx);
+
+/* Name of the kernel variant chosen by the most recent operator call (for tests and profiling). */
+const char* tmi_last_kernel(const tmi_ctx_t* ctx);
+
+/* ---- device memory (replaces Tensor::allocate / deallocate and the element-wise host copies of
+ *      reference_model/src/tensor.cpp:993-1015, 4722-4736) -------------------------------------------- */
+int tmi_buf_alloc(tmi_ctx_t* ctx, size_t bytes, void** out_dev);
+int tmi_buf_free(tmi_ctx_t* ctx, void* dev);
+int tmi_upload(tmi_ctx_t* ctx, void* dst_dev, const void* src_host, size_t bytes);   /* synchronous */
+int tmi_download(tmi_ctx_t* ctx, void* dst_host, const void* src_dev, size_t bytes); /* synchronous */
+
+/* ---- operator descriptors ----------------------------------------------------------------------- */
+
+/* Shapes and Conv2dAttribute / DepthwiseConv2dAttribute fields as read at the top of
+ * OpConv2d::eval / OpDepthwiseConv2d::eval (reference_model/src/ops/tensor_ops.cpp:725-758, 1174-1207). */
+typedef struct
+{
+    int32_t in_dtype;    /* TMI_INT8, TMI_FP16 or TMI_BF16 (weight has the same type)               */
+    int32_t out_dtype;   /* TMI_INT32 for INT8 input; TMI_FP16 / TMI_BF16 (same as input) otherwise  */
+    int32_t N, IH, IW, IC;
+    int32_t OC;          /* CONV2D: weight dim 0.  DEPTHWISE: IC * M (output channels)               */
+    int32_t KH, KW;
+    int32_t OH, OW;      /* declared output shape; checked against the reference's shape rule        */
+    int32_t pad[4];      /* top, bottom, left, right */
+    int32_t stride[2];   /* y, x */
+    int32_t dilation[2]; /* y, x */
+    int32_t bias_len;    /* 1 (broadcast) or OC */
+} tmi_conv_desc_t;
+
+/* RescaleAttribute plus the operand facts OpRescale::checkTensorAttributes / eval read
+ * (reference_model/src/ops/type_conversion.cpp:111-151, 226-255). */
+typedef struct
+{
+    int32_t in_dtype;        /* TMI_INT8 / TMI_INT16 / TMI_INT32 (bit pattern width; signedness below) */
+    int32_t out_dtype;       /* TMI_INT8 / TMI_INT16 / TMI_INT32 */
+    int32_t scale32;         /* 1: multiplier tensor is INT32; 0: INT16 */
+    int32_t rounding_mode;   /* TMI_ROUND_* */
+    int32_t per_channel;
+    int32_t input_unsigned;
+    int32_t output_unsigned;
+    int32_t in_zp;           /* stored value of the input_zp tensor  (sign-interpreted, as the reference holds it) */
+    int32_t out_zp;          /* stored value of the output_zp tensor */
+    int32_t n_multiplier;    /* element count of the multiplier tensor */
+    int32_t n_shift;         /* element count of the shift tensor      */
+} tmi_rescale_desc_t;
+
+/* ---- operators --------------------------------------------------------------------------------- */
+
+/* OpConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:723-882 (checks :120-226, :690-720).
+ * INT8 x INT8 -> INT32 with int32 accumulation, or FP16 / BF16 with fp32 accumulation and an output of
+ * the input type.  in_zp / w_zp are the values of operands 3 and 4 (must be 0 for non-INT8). */
+int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
+
+/* OpDepthwiseConv2d::eval, reference_model/src/ops/tensor_ops.cpp:1172-1334.  M = d->OC / d->IC. */
+int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
+
+/* OpMatMul::eval, reference_model/src/ops/tensor_ops.cpp:1423-1492 (checks :1347-1420).
+ * in_dtype TMI_INT8 -> INT32 output; TMI_FP16 / TMI_BF16 -> FP32 output (fp32 accumulation). */
+int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
+               const void* b_dev, int32_t a_zp, int32_t b_zp, void* out_dev);
+
+/* OpRescale::eval, reference_model/src/ops/type_conversion.cpp:224-421, on a tensor of `rank` dimensions
+ * viewed as [rows, C] (C = last dimension, or 1 for rank 0).  multiplier_dev holds INT32 (scale32) or
+ * INT16 values, shift_dev INT8 values. */
+int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64_t rows, int32_t C,
+                const void* in_dev, const void* multiplier_dev, const void* shift_dev, void* out_dev);
+
+/* OpClamp::eval for INT8 / INT16 (reference_model/src/ops/activation_funcs.cpp:27-125 with applyClip,
+ * reference_model/src/arith_util.h:389-413).  TMI_ERROR when max_val < min_val. */
+int tmi_clamp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, int32_t min_val, int32_t max_val,
+              void* out_dev);
+
+/* CONV2D -> RESCALE (-> CLAMP) evaluated as one kernel: the int32 convolution result never reaches HBM.
+ * Same results as tmi_conv2d + tmi_rescale (+ tmi_clamp) on the same operands.  The rescale input is the
+ * INT32 convolution output (r->in_dtype must be TMI_INT32, r->in_zp 0); per-channel constants have OC
+ * entries.  has_clamp = 0 skips the clamp. */
+int tmi_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                             const void* bias_dev, int32_t in_zp, int32_t w_zp, const tmi_rescale_desc_t* r,
+                             const void* multiplier_dev, const void* shift_dev, int32_t has_clamp,
+                             int32_t clamp_min, int32_t clamp_max, void* out_dev);
+
+/* DEPTHWISE_CONV2D -> RESCALE (-> CLAMP) as one kernel; see tmi_conv2d_rescale_clamp. */
+int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev,
+                                       const void* weight_dev, const void* bias_dev, int32_t in_zp, int32_t w_zp,
+                                       const tmi_rescale_desc_t* r, const void* multiplier_dev,
+                                       const void* shift_dev, int32_t has_clamp, int32_t clamp_min,
+                                       int32_t clamp_max, void* out_dev);
+
+/* ---- tuning / test hooks ------------------------------------------------------------------------- */
+
+/* Forces a kernel family for the following operator calls: 0 = automatic choice, 1 = direct (one output
+ * element per lane, any shape), 2 = MFMA (TMI_ERROR if the shape is not eligible).  Used by the parity
+ * tests to check every kernel on the same operands. */
+int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
+
+/* Library build identification, e.g. "tosa_mi355 gfx950". */
+const char* tmi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TOSA_MI355_H */

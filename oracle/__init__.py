@@ -74,7 +74,7 @@ def conv_out_hw(ih, iw, kh, kw, pad, stride, dilation):
     """Output height/width rule of check_conv_attribute (tensor_ops.cpp:203-223); None if inexact."""
     fh = ih - 1 + pad[0] + pad[1] - (kh - 1) * dilation[0]
     fw = iw - 1 + pad[2] + pad[3] - (kw - 1) * dilation[1]
-    if fh % stride[0] or fw % stride[1] or fh < 0 or fw < 0:
+    if stride[0] < 1 or stride[1] < 1 or fh % stride[0] or fw % stride[1] or fh < 0 or fw < 0:
         return None
     return fh // stride[0] + 1, fw // stride[1] + 1
 

@@ -1,0 +1,161 @@
+// RESCALE and CLAMP as stand-alone bandwidth kernels.
+//
+// RESCALE reads 1/2/4 bytes and writes 1/2/4 bytes per element and does ~20 integer instructions per
+// element, so it is bound by HBM.  Each lane handles VEC consecutive elements of one row with a single
+// vector load and a single vector store; the per-channel constants come from the L1/L2-resident
+// multiplier and shift arrays.
+#include "tmi_kernels.h"
+
+namespace tmi
+{
+
+template <typename T, int N>
+struct alignas(sizeof(T) * N) Pack
+{
+    T v[N];
+};
+
+template <typename InT, typename OutT, int VEC>
+__global__ __launch_bounds__(256) void rescale_vec_kernel(RescaleParams p, const InT* __restrict__ in,
+                                                          OutT* __restrict__ out, int64_t n_vec, int32_t C,
+                                                          uint32_t* flag_word)
+{
+    // C % VEC == 0, so a pack never straddles a row and its channels are c0 .. c0+VEC-1
+    uint32_t flags       = 0;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride)
+    {
+        const Pack<InT, VEC> a = reinterpret_cast<const Pack<InT, VEC>*>(in)[i];
+        const int c0           = (int)((i * VEC) % C);
+        Pack<OutT, VEC> r;
+#pragma unroll
+        for (int j = 0; j < VEC; j++)
+        {
+            const int32_t m = load_multiplier(p, c0 + j);
+            const int32_t s = load_shift(p, c0 + j);
+            r.v[j]          = (OutT)rescale_value(p, (int32_t)a.v[j], m, s, flags);
+        }
+        reinterpret_cast<Pack<OutT, VEC>*>(out)[i] = r;
+    }
+    raise_flags(flag_word, flags);
+}
+
+template <typename InT, typename OutT>
+__global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, const InT* __restrict__ in,
+                                                             OutT* __restrict__ out, int64_t n, int32_t C,
+                                                             uint32_t* flag_word)
+{
+    uint32_t flags       = 0;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    {
+        const int c     = (int)(i % C);
+        const int32_t m = load_multiplier(p, c);
+        const int32_t s = load_shift(p, c);
+        out[i]          = (OutT)rescale_value(p, (int32_t)in[i], m, s, flags);
+    }
+    raise_flags(flag_word, flags);
+}
+
+static int grid_for(int64_t work_items)
+{
+    // 256 CUs x 8 blocks of 256 lanes keep every SIMD busy; beyond that the loop strides.
+    int64_t blocks = (work_items + 255) / 256;
+    if (blocks < 1)
+        blocks = 1;
+    if (blocks > 256 * 8)
+        blocks = 256 * 8;
+    return (int)blocks;
+}
+
+template <typename InT, typename OutT>
+static const char* launch_rescale_t(hipStream_t st, const RescaleParams& p, const void* in, void* out, int64_t n,
+                                    int32_t C, uint32_t* flag_word)
+{
+    constexpr int VEC = 16 / (sizeof(InT) > sizeof(OutT) ? sizeof(InT) : sizeof(OutT)) >= 4
+                            ? 16 / (sizeof(InT) > sizeof(OutT) ? sizeof(InT) : sizeof(OutT))
+                            : 4;
+    const bool aligned = ((uintptr_t)in % (sizeof(InT) * VEC) == 0) && ((uintptr_t)out % (sizeof(OutT) * VEC) == 0);
+    if (n == 0)
+        return "rescale_empty";
+    if (aligned && C % VEC == 0)
+    {
+        const int64_t n_vec = n / VEC;
+        hipLaunchKernelGGL((rescale_vec_kernel<InT, OutT, VEC>), dim3(grid_for(n_vec)), dim3(256), 0, st, p,
+                           (const InT*)in, (OutT*)out, n_vec, C, flag_word);
+        return "rescale_vec";
+    }
+    hipLaunchKernelGGL((rescale_scalar_kernel<InT, OutT>), dim3(grid_for(n)), dim3(256), 0, st, p, (const InT*)in,
+                       (OutT*)out, n, C, flag_word);
+    return "rescale_scalar";
+}
+
+const char* launch_rescale(hipStream_t st, const RescaleParams& p, int32_t in_dtype, int32_t out_dtype,
+                           const void* in, void* out, int64_t n, int32_t C, uint32_t* flag_word)
+{
+#define TMI_RESCALE_CASE(ID, IT, OD, OT)                                                                            \
+    if (in_dtype == ID && out_dtype == OD)                                                                          \
+        return launch_rescale_t<IT, OT>(st, p, in, out, n, C, flag_word);
+    TMI_RESCALE_CASE(TMI_INT8, int8_t, TMI_INT8, int8_t)
+    TMI_RESCALE_CASE(TMI_INT8, int8_t, TMI_INT16, int16_t)
+    TMI_RESCALE_CASE(TMI_INT8, int8_t, TMI_INT32, int32_t)
+    TMI_RESCALE_CASE(TMI_INT16, int16_t, TMI_INT8, int8_t)
+    TMI_RESCALE_CASE(TMI_INT16, int16_t, TMI_INT16, int16_t)
+    TMI_RESCALE_CASE(TMI_INT16, int16_t, TMI_INT32, int32_t)
+    TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT8, int8_t)
+    TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT16, int16_t)
+    TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT32, int32_t)
+#undef TMI_RESCALE_CASE
+    return nullptr;
+}
+
+// ------------------------------------------------------------------------------------------------
+// CLAMP on INT8 / INT16: min(max(x, lo), hi), 16 bytes per lane.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void clamp_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t n,
+                                                    int32_t lo, int32_t hi, int vectorised)
+{
+    constexpr int VEC    = 16 / sizeof(T);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t n_vec  = vectorised ? n / VEC : 0;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride)
+    {
+        Pack<T, VEC> a = reinterpret_cast<const Pack<T, VEC>*>(in)[i];
+#pragma unroll
+        for (int j = 0; j < VEC; j++)
+        {
+            int32_t v = a.v[j];
+            v         = v >= lo ? v : lo;
+            v         = v < hi ? v : hi;
+            a.v[j]    = (T)v;
+        }
+        reinterpret_cast<Pack<T, VEC>*>(out)[i] = a;
+    }
+    for (int64_t i = n_vec * VEC + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    {
+        int32_t v = in[i];
+        v         = v >= lo ? v : lo;
+        v         = v < hi ? v : hi;
+        out[i]    = (T)v;
+    }
+}
+
+const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, int32_t lo,
+                         int32_t hi)
+{
+    if (n == 0)
+        return "clamp_empty";
+    const int vec = ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 16 == 0);
+    if (dtype == TMI_INT8)
+        hipLaunchKernelGGL(clamp_kernel<int8_t>, dim3(grid_for((n + 15) / 16)), dim3(256), 0, st, (const int8_t*)in,
+                           (int8_t*)out, n, lo, hi, vec);
+    else if (dtype == TMI_INT16)
+        hipLaunchKernelGGL(clamp_kernel<int16_t>, dim3(grid_for((n + 7) / 8)), dim3(256), 0, st,
+                           (const int16_t*)in, (int16_t*)out, n, lo, hi, vec);
+    else
+        return nullptr;
+    return "clamp_vec";
+}
+
+}    // namespace tmi

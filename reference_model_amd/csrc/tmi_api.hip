@@ -1,0 +1,558 @@
+// C ABI of the library: context, device memory, operand validation and kernel selection.
+// Validation follows the reference operator's checkTensorAttributes()/eval() checks so that the same
+// malformed node is rejected with the same status; arithmetic lives in the kernel files.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "tmi_kernels.h"
+
+struct tmi_ctx
+{
+    int device            = 0;
+    hipStream_t stream    = nullptr;
+    bool owns_stream      = false;
+    uint32_t* flags_dev   = nullptr;    // latched REQUIRE conditions
+    uint32_t* flags_host  = nullptr;    // pinned staging word
+    uint32_t last_flags   = 0;
+    int32_t kernel_choice = 0;
+    std::string last_error;
+    const char* last_kernel = "";
+};
+
+namespace
+{
+
+using namespace tmi;
+
+int fail(tmi_ctx* ctx, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    if (ctx)
+        ctx->last_error = buf;
+    return TMI_ERROR;
+}
+
+int hip_fail(tmi_ctx* ctx, hipError_t e, const char* what)
+{
+    return fail(ctx, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define TMI_HIP(ctx, call)                                                                                          \
+    do                                                                                                              \
+    {                                                                                                               \
+        hipError_t e_ = (call);                                                                                     \
+        if (e_ != hipSuccess)                                                                                       \
+            return hip_fail(ctx, e_, #call);                                                                        \
+    } while (0)
+
+int after_launch(tmi_ctx* ctx, const char* kernel_name)
+{
+    if (!kernel_name)
+        return fail(ctx, "no kernel implements this operand type combination");
+    ctx->last_kernel = kernel_name;
+    hipError_t e     = hipGetLastError();
+    if (e != hipSuccess)
+        return hip_fail(ctx, e, kernel_name);
+    return TMI_VALID;
+}
+
+int dtype_bits(int32_t dt)
+{
+    switch (dt)
+    {
+        case TMI_INT8:
+            return 8;
+        case TMI_INT16:
+        case TMI_FP16:
+        case TMI_BF16:
+            return 16;
+        case TMI_INT32:
+        case TMI_FP32:
+            return 32;
+        default:
+            return 0;
+    }
+}
+
+bool is_int_dtype(int32_t dt)
+{
+    return dt == TMI_INT8 || dt == TMI_INT16 || dt == TMI_INT32;
+}
+
+// check_conv_attribute (tensor_ops.cpp:120-226) and the ERROR_IFs of eval (:742-748, :805, :811;
+// depthwise :1191-1197, :1237, :1241).
+int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool depthwise, int32_t in_zp,
+                  int32_t w_zp, ConvGeom& g)
+{
+    if (!d)
+        return fail(ctx, "%s: null descriptor", op);
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+        return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
+    const int32_t want_out = d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype;
+    if (d->out_dtype != want_out)
+        return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1 || d->OH < 0 ||
+        d->OW < 0)
+        return fail(ctx, "%s: negative tensor dimension", op);
+    for (int i = 0; i < 4; i++)
+        if (d->pad[i] < 0)
+            return fail(ctx, "%s: At least one pad is smaller than zero", op);
+    for (int i = 0; i < 2; i++)
+        if (d->stride[i] < 1)
+            return fail(ctx, "%s: At least one stride dimension is smaller than one", op);
+    for (int i = 0; i < 2; i++)
+        if (d->dilation[i] < 1)
+            return fail(ctx, "%s: At least one dilation dimension is smaller than one", op);
+
+    const int64_t full_h = (int64_t)d->IH - 1 + d->pad[0] + d->pad[1] - (int64_t)(d->KH - 1) * d->dilation[0];
+    const int64_t full_w = (int64_t)d->IW - 1 + d->pad[2] + d->pad[3] - (int64_t)(d->KW - 1) * d->dilation[1];
+    if ((full_h % d->stride[0]) != 0 || (full_w % d->stride[1]) != 0)
+        return fail(ctx, "%s: Parameters must yield exact integer output dimensions", op);
+    if (d->OH != full_h / d->stride[0] + 1 || d->OW != full_w / d->stride[1] + 1)
+        return fail(ctx, "%s: Mismatch between output shape provided and expected output shape (%lld,%lld)", op,
+                    (long long)(full_h / d->stride[0] + 1), (long long)(full_w / d->stride[1] + 1));
+
+    int32_t M = 1;
+    if (depthwise)
+    {
+        if (d->IC == 0 || d->OC % d->IC != 0)
+            return fail(ctx, "%s: tensor output channel mismatch %d != %d", op, d->IC, d->OC);
+        M = d->OC / d->IC;
+        if (M < 1)
+            return fail(ctx, "%s: tensor output channel mismatch %d != %d", op, d->IC, d->OC);
+    }
+    if (d->bias_len != d->OC && d->bias_len != 1)
+        return fail(ctx, "%s: bias channel mismatch %d != %d", op, d->bias_len, d->OC);
+    if (d->in_dtype != TMI_INT8 && in_zp != 0)
+        return fail(ctx, "%s: Input zero point must be zero for non int8_t data", op);
+    if (d->in_dtype != TMI_INT8 && w_zp != 0)
+        return fail(ctx, "%s: Weight zero point must be zero for non int8_t data", op);
+    if (in_zp < -128 || in_zp > 127 || w_zp < -128 || w_zp > 127)
+        return fail(ctx, "%s: zero point outside the int8 range", op);
+
+    g.N = d->N, g.IH = d->IH, g.IW = d->IW, g.IC = d->IC, g.OC = d->OC, g.KH = d->KH, g.KW = d->KW;
+    g.OH = d->OH, g.OW = d->OW;
+    g.pad_top = d->pad[0], g.pad_left = d->pad[2];
+    g.stride_y = d->stride[0], g.stride_x = d->stride[1], g.dil_y = d->dilation[0], g.dil_x = d->dilation[1];
+    g.bias_len = d->bias_len;
+    g.M        = M;
+    return TMI_VALID;
+}
+
+int64_t extend(int32_t v, int bits, bool is_unsigned)
+{
+    if (bits == 8)
+        return is_unsigned ? (int64_t)(uint8_t)v : (int64_t)(int8_t)v;
+    if (bits == 16)
+        return is_unsigned ? (int64_t)(uint16_t)v : (int64_t)(int16_t)v;
+    return is_unsigned ? (int64_t)(uint32_t)v : (int64_t)v;
+}
+
+// OpRescale::checkTensorAttributes (type_conversion.cpp:111-151) and the zero-point ERROR_IFs of eval
+// (:242-255).  Fills the kernel parameters.
+int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, int32_t C, const void* mult,
+                     const void* shift, RescaleParams& p)
+{
+    if (!r)
+        return fail(ctx, "OpRescale: null descriptor");
+    if (!is_int_dtype(r->in_dtype) || !is_int_dtype(r->out_dtype))
+        return fail(ctx, "OpRescale: unsupported data type");
+    const bool i32in = r->in_dtype == TMI_INT32, i32out = r->out_dtype == TMI_INT32;
+    const bool i8in = r->in_dtype == TMI_INT8, i8out = r->out_dtype == TMI_INT8;
+    const bool i16in = r->in_dtype == TMI_INT16, i16out = r->out_dtype == TMI_INT16;
+    const bool in_u = r->input_unsigned != 0, out_u = r->output_unsigned != 0;
+
+    if (r->rounding_mode != TMI_ROUND_SINGLE && r->rounding_mode != TMI_ROUND_DOUBLE &&
+        r->rounding_mode != TMI_ROUND_INEXACT)
+        return fail(ctx, "OpRescale: Unsupported rounding mode");
+    if (!r->scale32 && r->rounding_mode == TMI_ROUND_DOUBLE)
+        return fail(ctx, "OpRescale: Scale set to false but rounding mode set to double round");
+    if (in_u && out_u)
+        return fail(ctx, "OpRescale: input_unsigned and output_unsigned set to true");
+    if (i32out && in_u)
+        return fail(ctx, "OpRescale: Output signed int32 and input_unsigned set to true");
+    if (i32in && out_u)
+        return fail(ctx, "OpRescale: Input signed int32 and output_unsigned set to true");
+    if (i32in && in_u)
+        return fail(ctx, "OpRescale: Input unsigned int32");
+    if (i32out && out_u)
+        return fail(ctx, "OpRescale: Output unsigned int32");
+    if (r->per_channel)
+    {
+        if (rank < 1)
+            return fail(ctx, "OpRescale: per_channel set to true and rank of input < 1");
+        if (r->n_multiplier != C)
+            return fail(ctx, "OpRescale: wrong size multiplier array for per_channel=true");
+        if (r->n_shift != C)
+            return fail(ctx, "OpRescale: wrong size shift array for per_channel=true");
+    }
+    else
+    {
+        if (r->n_multiplier != 1)
+            return fail(ctx, "OpRescale: wrong size multiplier array for per_channel=false");
+        if (r->n_shift != 1)
+            return fail(ctx, "OpRescale: wrong size shift array for per_channel=false");
+    }
+
+    const int64_t out_zp = extend(r->out_zp, dtype_bits(r->out_dtype), out_u);
+    const int64_t in_zp  = extend(r->in_zp, dtype_bits(r->in_dtype), in_u);
+    if (!i8in && !(i16in && in_u) && in_zp != 0)
+        return fail(ctx, "OpRescale: Input TOSA_REF_TYPE not INT8/UINT8/UINT16 and zero point not 0");
+    if (!i8out && !(i16out && out_u) && out_zp != 0)
+        return fail(ctx, "OpRescale: Output TOSA_REF_TYPE not INT8/UINT8/UINT16 and zero point not 0");
+    if (i16in && in_u && in_zp != 0 && in_zp != 32768)
+        return fail(ctx, "OpRescale: Input unsigned int16 and zero point (%lld) not 0 or 32768", (long long)in_zp);
+    if (i16out && out_u && out_zp != 0 && out_zp != 32768)
+        return fail(ctx, "OpRescale: Output unsigned int16 and zero point (%lld) not 0 or 32768",
+                    (long long)out_zp);
+    if (!mult || !shift)
+        return fail(ctx, "OpRescale: null multiplier or shift tensor");
+
+    p               = RescaleParams{};
+    p.multiplier    = mult;
+    p.shift         = reinterpret_cast<const int8_t*>(shift);
+    p.in_zp         = (int32_t)in_zp;
+    p.out_zp        = (int32_t)out_zp;
+    p.qmin          = out_u ? 0 : (i8out ? -128 : (i16out ? -32768 : INT32_MIN));
+    p.qmax          = out_u ? (i8out ? 255 : 65535) : (i8out ? 127 : (i16out ? 32767 : INT32_MAX));
+    p.scale32       = r->scale32 != 0;
+    p.double_round  = r->rounding_mode == TMI_ROUND_DOUBLE;
+    p.inexact_round = r->rounding_mode == TMI_ROUND_INEXACT;
+    p.per_channel   = r->per_channel != 0;
+    p.in_bits       = (uint8_t)dtype_bits(r->in_dtype);
+    p.in_unsigned   = in_u;
+    p.has_clamp     = 0;
+    p.enabled       = 1;
+    return TMI_VALID;
+}
+
+int validate_fused_rescale(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, const tmi_rescale_desc_t* r,
+                           const void* mult, const void* shift, int32_t has_clamp, int32_t clamp_min,
+                           int32_t clamp_max, RescaleParams& p)
+{
+    if (!r)
+        return fail(ctx, "%s: null rescale descriptor", op);
+    if (d->in_dtype != TMI_INT8)
+        return fail(ctx, "%s: the fused rescale needs an INT8 convolution", op);
+    if (r->in_dtype != TMI_INT32)
+        return fail(ctx, "%s: the fused rescale consumes the INT32 convolution output", op);
+    int rc = validate_rescale(ctx, r, 4, d->OC, mult, shift, p);
+    if (rc != TMI_VALID)
+        return rc;
+    if (has_clamp)
+    {
+        // OpClamp::register_fcn: ERROR_IF(max < min) (activation_funcs.cpp:91)
+        if (clamp_max < clamp_min)
+            return fail(ctx, "OpClamp: max smaller than min");
+        p.has_clamp = 1;
+        p.clamp_min = clamp_min;
+        p.clamp_max = clamp_max;
+    }
+    return TMI_VALID;
+}
+
+int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in, const void* w,
+             const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, int32_t out_dtype, void* out)
+{
+    ConvGeom g;
+    int rc = validate_conv(ctx, op, d, depthwise, in_zp, w_zp, g);
+    if (rc != TMI_VALID)
+        return rc;
+    const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
+    if (total > 0 && (!in || !w || !bias || !out))
+        return fail(ctx, "%s: null tensor pointer", op);
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+
+    const char* name = nullptr;
+    if (ctx->kernel_choice == 2)
+        return fail(ctx, "%s: no MFMA kernel is eligible for this shape", op);
+    if (depthwise)
+        name = launch_depthwise_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                       ctx->flags_dev);
+    else
+        name = launch_conv2d_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                    ctx->flags_dev);
+    return after_launch(ctx, name);
+}
+
+}    // namespace
+
+extern "C" {
+
+const char* tmi_version(void)
+{
+    return "tosa_mi355 0.1 gfx950";
+}
+
+int tmi_ctx_create(tmi_ctx_t** out_ctx, int device)
+{
+    if (!out_ctx)
+        return TMI_ERROR;
+    *out_ctx = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count)
+        return TMI_ERROR;
+    tmi_ctx* ctx = new tmi_ctx();
+    ctx->device  = device;
+    if (hipSetDevice(device) != hipSuccess || hipStreamCreate(&ctx->stream) != hipSuccess)
+    {
+        delete ctx;
+        return TMI_ERROR;
+    }
+    ctx->owns_stream = true;
+    if (hipMalloc((void**)&ctx->flags_dev, 256) != hipSuccess ||
+        hipHostMalloc((void**)&ctx->flags_host, 256, hipHostMallocDefault) != hipSuccess ||
+        hipMemset(ctx->flags_dev, 0, 256) != hipSuccess)
+    {
+        tmi_ctx_destroy(ctx);
+        return TMI_ERROR;
+    }
+    *ctx->flags_host = 0;
+    *out_ctx         = ctx;
+    return TMI_VALID;
+}
+
+int tmi_ctx_destroy(tmi_ctx_t* ctx)
+{
+    if (!ctx)
+        return TMI_VALID;
+    // teardown is best effort: there is nobody left to report a failure to
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->flags_dev)
+        (void)hipFree(ctx->flags_dev);
+    if (ctx->flags_host)
+        (void)hipHostFree(ctx->flags_host);
+    if (ctx->owns_stream && ctx->stream)
+        (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return TMI_VALID;
+}
+
+int tmi_ctx_set_stream(tmi_ctx_t* ctx, void* hip_stream)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->owns_stream && ctx->stream)
+        TMI_HIP(ctx, hipStreamDestroy(ctx->stream));
+    ctx->stream      = (hipStream_t)hip_stream;
+    ctx->owns_stream = false;
+    return TMI_VALID;
+}
+
+int tmi_ctx_sync(tmi_ctx_t* ctx)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipMemcpyAsync(ctx->flags_host, ctx->flags_dev, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                ctx->stream));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    ctx->last_flags = *ctx->flags_host;
+    if (ctx->last_flags)
+    {
+        // cleared with a plain stream-ordered memset: nothing captures this path into a graph
+        TMI_HIP(ctx, hipMemsetAsync(ctx->flags_dev, 0, sizeof(uint32_t), ctx->stream));
+        TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return TMI_UNPREDICTABLE;
+    }
+    return TMI_VALID;
+}
+
+uint32_t tmi_ctx_flags(const tmi_ctx_t* ctx)
+{
+    return ctx ? ctx->last_flags : 0;
+}
+
+const char* tmi_last_error(const tmi_ctx_t* ctx)
+{
+    return ctx ? ctx->last_error.c_str() : "null context";
+}
+
+const char* tmi_last_kernel(const tmi_ctx_t* ctx)
+{
+    return ctx ? ctx->last_kernel : "";
+}
+
+int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
+{
+    if (!ctx || choice < 0 || choice > 2)
+        return TMI_ERROR;
+    ctx->kernel_choice = choice;
+    return TMI_VALID;
+}
+
+int tmi_buf_alloc(tmi_ctx_t* ctx, size_t bytes, void** out_dev)
+{
+    if (!ctx || !out_dev)
+        return TMI_ERROR;
+    *out_dev = nullptr;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipMalloc(out_dev, bytes ? bytes : 16));
+    return TMI_VALID;
+}
+
+int tmi_buf_free(tmi_ctx_t* ctx, void* dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (!dev)
+        return TMI_VALID;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    TMI_HIP(ctx, hipFree(dev));
+    return TMI_VALID;
+}
+
+int tmi_upload(tmi_ctx_t* ctx, void* dst_dev, const void* src_host, size_t bytes)
+{
+    if (!ctx || (bytes && (!dst_dev || !src_host)))
+        return fail(ctx, "tmi_upload: null pointer");
+    if (!bytes)
+        return TMI_VALID;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TMI_VALID;
+}
+
+int tmi_download(tmi_ctx_t* ctx, void* dst_host, const void* src_dev, size_t bytes)
+{
+    if (!ctx || (bytes && (!dst_host || !src_dev)))
+        return fail(ctx, "tmi_download: null pointer");
+    if (!bytes)
+        return TMI_VALID;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TMI_VALID;
+}
+
+int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    RescaleParams none{};
+    return run_conv(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, none,
+                    d ? d->out_dtype : 0, out_dev);
+}
+
+int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    RescaleParams none{};
+    return run_conv(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, none,
+                    d ? d->out_dtype : 0, out_dev);
+}
+
+int tmi_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                             const void* bias_dev, int32_t in_zp, int32_t w_zp, const tmi_rescale_desc_t* r,
+                             const void* multiplier_dev, const void* shift_dev, int32_t has_clamp,
+                             int32_t clamp_min, int32_t clamp_max, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (!d)
+        return fail(ctx, "OpConv2d: null descriptor");
+    RescaleParams rp;
+    int rc = validate_fused_rescale(ctx, "OpConv2d+OpRescale", d, r, multiplier_dev, shift_dev, has_clamp,
+                                    clamp_min, clamp_max, rp);
+    if (rc != TMI_VALID)
+        return rc;
+    return run_conv(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp, r->out_dtype, out_dev);
+}
+
+int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev,
+                                       const void* weight_dev, const void* bias_dev, int32_t in_zp, int32_t w_zp,
+                                       const tmi_rescale_desc_t* r, const void* multiplier_dev,
+                                       const void* shift_dev, int32_t has_clamp, int32_t clamp_min,
+                                       int32_t clamp_max, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (!d)
+        return fail(ctx, "OpDepthwiseConv2d: null descriptor");
+    RescaleParams rp;
+    int rc = validate_fused_rescale(ctx, "OpDepthwiseConv2d+OpRescale", d, r, multiplier_dev, shift_dev, has_clamp,
+                                    clamp_min, clamp_max, rp);
+    if (rc != TMI_VALID)
+        return rc;
+    return run_conv(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp, r->out_dtype,
+                    out_dev);
+}
+
+int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
+               const void* b_dev, int32_t a_zp, int32_t b_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
+        return fail(ctx, "OpMatMul: input data type not supported for this configuration of operator");
+    if (N < 0 || H < 0 || C < 0 || W < 0)
+        return fail(ctx, "OpMatMul: negative tensor dimension");
+    // tensor_ops.cpp:1433-1434
+    if (in_dtype != TMI_INT8 && a_zp != 0)
+        return fail(ctx, "OpMatMul: A zeropoint must be zero for non int8_t data");
+    if (in_dtype != TMI_INT8 && b_zp != 0)
+        return fail(ctx, "OpMatMul: B zeropoint must be zero for non int8_t data");
+    if (a_zp < -128 || a_zp > 127 || b_zp < -128 || b_zp > 127)
+        return fail(ctx, "OpMatMul: zero point outside the int8 range");
+    const int64_t total = (int64_t)N * H * W;
+    if (total > 0 && (!out_dev || ((int64_t)C > 0 && (!a_dev || !b_dev))))
+        return fail(ctx, "OpMatMul: null tensor pointer");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    if (ctx->kernel_choice == 2)
+        return fail(ctx, "OpMatMul: no MFMA kernel is eligible for this shape");
+    const char* name = launch_matmul_direct(ctx->stream, in_dtype, N, H, C, W, a_dev, b_dev, a_zp, b_zp, out_dev);
+    return after_launch(ctx, name);
+}
+
+int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64_t rows, int32_t C,
+                const void* in_dev, const void* multiplier_dev, const void* shift_dev, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (rank < 0 || rank > 6)
+        return fail(ctx, "OpRescale: rank outside [0,6]");
+    if (rows < 0 || C < 0)
+        return fail(ctx, "OpRescale: negative tensor dimension");
+    RescaleParams p;
+    int rc = validate_rescale(ctx, r, rank, C, multiplier_dev, shift_dev, p);
+    if (rc != TMI_VALID)
+        return rc;
+    const int64_t n = rows * (int64_t)C;
+    if (n > 0 && (!in_dev || !out_dev))
+        return fail(ctx, "OpRescale: null tensor pointer");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    const char* name = launch_rescale(ctx->stream, p, r->in_dtype, r->out_dtype, in_dev, out_dev, n, C > 0 ? C : 1,
+                                      ctx->flags_dev);
+    return after_launch(ctx, name);
+}
+
+int tmi_clamp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, int32_t min_val, int32_t max_val,
+              void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (dtype != TMI_INT8 && dtype != TMI_INT16)
+        return fail(ctx, "OpClamp: unsupported TOSA_REF_TYPE");
+    if (max_val < min_val)
+        return fail(ctx, "OpClamp: max smaller than min");
+    if (n < 0 || (n > 0 && (!in_dev || !out_dev)))
+        return fail(ctx, "OpClamp: bad tensor");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    return after_launch(ctx, launch_clamp(ctx->stream, dtype, in_dev, out_dev, n, min_val, max_val));
+}
+
+}    // extern "C"

@@ -1,0 +1,130 @@
+// Device-side helpers shared by every kernel: the RESCALE arithmetic and the epilogue that turns an
+// int32 accumulator into the stored output element.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tosa_mi355.h"
+
+namespace tmi
+{
+
+// Everything a kernel needs to apply RESCALE (and an optional CLAMP) to one value.  Filled on the host
+// after validation, passed by value.
+struct RescaleParams
+{
+    const void* multiplier;    // int32[n] when scale32 else int16[n]
+    const int8_t* shift;       // int8[n]
+    int32_t in_zp;             // sign/zero-extended input zero point
+    int32_t out_zp;            // sign/zero-extended output zero point
+    int32_t qmin, qmax;        // clip range of the output type
+    int32_t clamp_min, clamp_max;
+    uint8_t scale32, double_round, inexact_round, per_channel;
+    uint8_t in_bits, in_unsigned, has_clamp, enabled;
+};
+
+// value_extend64_impl of the reference (type_conversion.cpp:183-221) for 8/16/32-bit storage.
+__device__ __forceinline__ int64_t value_extend(int32_t v, int bits, bool is_unsigned)
+{
+    if (bits == 8)
+        return is_unsigned ? (int64_t)(uint8_t)v : (int64_t)(int8_t)v;
+    if (bits == 16)
+        return is_unsigned ? (int64_t)(uint16_t)v : (int64_t)(int16_t)v;
+    return is_unsigned ? (int64_t)(uint32_t)v : (int64_t)v;
+}
+
+// QuantUtil::apply_scale_32 (quant_util.h:45-84).  Violated preconditions set bits in `flags`.
+__device__ __forceinline__ int32_t apply_scale_32(int32_t value, int32_t multiplier, int32_t shift,
+                                                  bool double_round, uint32_t& flags)
+{
+    if (multiplier < 0)
+        flags |= TMI_FLAG_SCALE_MULTIPLIER;
+    if (shift < 2 || shift > 62)
+    {
+        flags |= TMI_FLAG_SCALE_SHIFT;
+        return 0;
+    }
+    if (shift <= 31)
+    {
+        const int32_t high = 1 << (shift - 1);
+        if (value < -high || value >= high)
+            flags |= TMI_FLAG_SCALE_VALUE;
+    }
+    int64_t round = int64_t(1) << (shift - 1);
+    if (double_round && shift > 31)
+        round += (value >= 0) ? (int64_t(1) << 30) : -(int64_t(1) << 30);
+    int64_t result = (int64_t)value * (int64_t)multiplier + round;
+    result >>= shift;
+    if (result < -(int64_t(1) << 31) || result >= (int64_t(1) << 31))
+        flags |= TMI_FLAG_SCALE_RESULT;
+    return (int32_t)result;
+}
+
+// QuantUtil::apply_scale_16 (quant_util.h:86-108).
+__device__ __forceinline__ int32_t apply_scale_16(int64_t value, int32_t multiplier, int32_t shift, uint32_t& flags)
+{
+    if (multiplier < 0)
+        flags |= TMI_FLAG_SCALE_MULTIPLIER;
+    if (shift < 2 || shift > 62)
+    {
+        flags |= TMI_FLAG_SCALE_SHIFT;
+        return 0;
+    }
+    int64_t result = (int64_t)((uint64_t)value * (uint64_t)(int64_t)multiplier + (uint64_t(1) << (shift - 1)));
+    result >>= shift;
+    if (result < -(int64_t(1) << 31) || result >= (int64_t(1) << 31))
+        flags |= TMI_FLAG_SCALE_RESULT;
+    return (int32_t)result;
+}
+
+// The rescale_func lambda of OpRescale::eval (type_conversion.cpp:305-370) followed by the optional
+// CLAMP (arith_util.h:389-413).  `stored` is the raw stored input value, `m`/`s` the channel's constants.
+__device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int32_t stored, int32_t m, int32_t s,
+                                                 uint32_t& flags)
+{
+    const int64_t v = value_extend(stored, p.in_bits, p.in_unsigned) - (int64_t)p.in_zp;
+    int32_t scaled;
+    if (p.inexact_round)
+    {
+        const float t = (float)v * (float)m;
+        scaled        = (int32_t)rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
+    }
+    else if (p.scale32)
+        scaled = apply_scale_32((int32_t)v, m, s, p.double_round, flags);
+    else
+        scaled = apply_scale_16(v, m, s, flags);
+    const int64_t res = (int64_t)scaled + (int64_t)p.out_zp;
+    if (res > (int64_t)INT32_MAX || res < (int64_t)INT32_MIN)
+        flags |= TMI_FLAG_ZP_RESULT;
+    int32_t r = (int32_t)res;
+    r         = r < p.qmin ? p.qmin : r;
+    r         = r > p.qmax ? p.qmax : r;
+    if (p.has_clamp)
+    {
+        r = r >= p.clamp_min ? r : p.clamp_min;
+        r = r < p.clamp_max ? r : p.clamp_max;
+    }
+    return r;
+}
+
+__device__ __forceinline__ int32_t load_multiplier(const RescaleParams& p, int c)
+{
+    const int i = p.per_channel ? c : 0;
+    return p.scale32 ? reinterpret_cast<const int32_t*>(p.multiplier)[i]
+                     : (int32_t) reinterpret_cast<const int16_t*>(p.multiplier)[i];
+}
+
+__device__ __forceinline__ int32_t load_shift(const RescaleParams& p, int c)
+{
+    return (int32_t)p.shift[p.per_channel ? c : 0];
+}
+
+// Latches REQUIRE conditions into the context's flag word (one vector atomic per lane that saw one).
+__device__ __forceinline__ void raise_flags(uint32_t* flag_word, uint32_t flags)
+{
+    if (flags)
+        atomicOr(flag_word, flags);
+}
+
+}    // namespace tmi

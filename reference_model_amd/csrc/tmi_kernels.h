@@ -1,0 +1,72 @@
+// Host-callable launchers of every kernel family.  Each returns the name of the kernel variant it
+// enqueued (nullptr if the combination is not implemented) and never synchronises.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tmi_device.h"
+
+namespace tmi
+{
+
+// Validated geometry of a CONV2D / DEPTHWISE_CONV2D call.
+struct ConvGeom
+{
+    int32_t N, IH, IW, IC, OC, KH, KW, OH, OW;
+    int32_t pad_top, pad_left, stride_y, stride_x, dil_y, dil_x;
+    int32_t bias_len;
+    int32_t M;    // depthwise channel multiplier (unused by CONV2D)
+};
+
+// bf16 carried as its bit pattern
+struct bf16_t
+{
+    uint16_t bits;
+};
+
+__host__ __device__ inline float bf16_to_float(bf16_t v)
+{
+    union
+    {
+        uint32_t u;
+        float f;
+    } x;
+    x.u = (uint32_t)v.bits << 16;
+    return x.f;
+}
+
+__host__ __device__ inline bf16_t float_to_bf16(float f)
+{
+    union
+    {
+        uint32_t u;
+        float f;
+    } x;
+    x.f = f;
+    bf16_t r;
+    if ((x.u & 0x7fffffffu) > 0x7f800000u)    // NaN: keep it quiet
+        r.bits = (uint16_t)((x.u >> 16) | 0x0040u);
+    else
+        r.bits = (uint16_t)((x.u + 0x7fffu + ((x.u >> 16) & 1u)) >> 16);    // round to nearest even
+    return r;
+}
+
+// elementwise.hip
+const char* launch_rescale(hipStream_t st, const RescaleParams& p, int32_t in_dtype, int32_t out_dtype,
+                           const void* in, void* out, int64_t n, int32_t C, uint32_t* flag_word);
+const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, int32_t lo,
+                         int32_t hi);
+
+// direct.hip: one output element per lane, any legal shape.  out_dtype is the stored output type
+// (INT32 without rescale; the rescale output type with it; FP16/BF16/FP32 for floating point).
+const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
+                                 const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
+                                 const RescaleParams& rp, void* out, uint32_t* flag_word);
+const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
+                                    const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
+                                    const RescaleParams& rp, void* out, uint32_t* flag_word);
+const char* launch_matmul_direct(hipStream_t st, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
+                                 const void* a, const void* b, int32_t a_zp, int32_t b_zp, void* out);
+
+}    // namespace tmi

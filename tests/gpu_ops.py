@@ -1,0 +1,108 @@
+"""numpy-in / numpy-out helpers over the C ABI for the GPU parity tests (upload, run, download)."""
+from __future__ import annotations
+
+import numpy as np
+
+import oracle
+from reference_model_amd import capi
+
+_TMI = {np.dtype(np.int8): capi.INT8, np.dtype(np.uint8): capi.INT8, np.dtype(np.int16): capi.INT16,
+        np.dtype(np.uint16): capi.INT16, np.dtype(np.int32): capi.INT32, np.dtype(np.float16): capi.FP16}
+
+
+def _conv_common(ctx, x, w_shape_khkwoc, bias, pad, stride, dilation, in_dtype, out_hw):
+    kh, kw, oc = w_shape_khkwoc
+    if out_hw is None:
+        out_hw = oracle.conv_out_hw(x.shape[1], x.shape[2], kh, kw, pad, stride, dilation) or (0, 0)
+    out_dtype = capi.INT32 if in_dtype == capi.INT8 else in_dtype
+    d = ctx.conv_desc(in_dtype, out_dtype, x.shape, oc, kh, kw, out_hw, pad, stride, dilation, bias.shape[0])
+    return d, out_hw, out_dtype
+
+
+def conv2d(ctx, x, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0, out_hw=None,
+           depthwise=False, dtype=None, rescale=None, clamp=None):
+    """Runs CONV2D / DEPTHWISE_CONV2D (optionally fused with RESCALE[/CLAMP]); returns (out, status).
+
+    rescale = dict(mult, shift, out_zp, out_dtype(np), rounding_mode, scale32, per_channel, output_unsigned)."""
+    in_dtype = dtype or _TMI[x.dtype]
+    if depthwise:
+        kh, kw, c, m = w.shape
+        oc = c * m
+    else:
+        oc, kh, kw, _ = w.shape
+    d, out_hw, out_dtype = _conv_common(ctx, x, (kh, kw, oc), bias, pad, stride, dilation, in_dtype, out_hw)
+    tx, tw, tb = ctx.upload(x, in_dtype), ctx.upload(w, in_dtype), ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
+    shape = (x.shape[0], out_hw[0], out_hw[1], oc)
+    try:
+        if rescale is None:
+            np_out = {capi.INT32: np.int32, capi.FP16: np.float16, capi.BF16: np.uint16}[out_dtype]
+            to = ctx.empty(shape, out_dtype, np_out)
+            fn = ctx.depthwise_conv2d if depthwise else ctx.conv2d
+            fn(d, tx, tw, tb, in_zp, w_zp, to)
+        else:
+            od = np.dtype(rescale.get("out_dtype", np.int8))
+            mult, shift = np.atleast_1d(rescale["mult"]), np.atleast_1d(rescale["shift"]).astype(np.int8)
+            scale32 = rescale.get("scale32", True)
+            tm = ctx.upload(mult.astype(np.int32 if scale32 else np.int16))
+            ts = ctx.upload(shift)
+            r = ctx.rescale_desc(capi.INT32, _TMI[od], mult.size, shift.size, 0, rescale.get("out_zp", 0), scale32,
+                                 rescale.get("rounding_mode", capi.ROUND_DOUBLE), rescale.get("per_channel", True),
+                                 False, rescale.get("output_unsigned", False))
+            to = ctx.empty(shape, _TMI[od], od)
+            fn = ctx.depthwise_conv2d_rescale_clamp if depthwise else ctx.conv2d_rescale_clamp
+            fn(d, tx, tw, tb, in_zp, w_zp, r, tm, ts, to, clamp)
+        st = ctx.sync()
+        return to.numpy(), st
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+
+def matmul(ctx, a, b, a_zp=0, b_zp=0, dtype=None):
+    in_dtype = dtype or _TMI[a.dtype]
+    n, h, c = a.shape
+    w = b.shape[2]
+    ta, tb = ctx.upload(a, in_dtype), ctx.upload(b, in_dtype)
+    to = ctx.empty((n, h, w), capi.INT32 if in_dtype == capi.INT8 else capi.FP32)
+    try:
+        ctx.matmul(in_dtype, n, h, c, w, ta, tb, a_zp, b_zp, to)
+        st = ctx.sync()
+        return to.numpy(), st
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+
+def rescale(ctx, x, mult, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale32=True,
+            rounding_mode=capi.ROUND_DOUBLE, per_channel=True, input_unsigned=False, output_unsigned=False):
+    x = np.asarray(x)
+    od = np.dtype(out_dtype)
+    mult, shift = np.atleast_1d(mult), np.atleast_1d(shift).astype(np.int8)
+    rank = x.ndim
+    C = x.shape[-1] if rank else 1
+    rows = int(np.prod(x.shape[:-1], dtype=np.int64)) if rank else 1
+    try:
+        tx = ctx.upload(x)
+        tm = ctx.upload(mult.astype(np.int32 if scale32 else np.int16))
+        ts = ctx.upload(shift)
+        to = ctx.empty(x.shape, _TMI[od], od)
+        r = ctx.rescale_desc(_TMI[x.dtype], _TMI[od], mult.size, shift.size, in_zp, out_zp, scale32, rounding_mode,
+                             per_channel, input_unsigned, output_unsigned)
+        ctx.rescale(r, rank, rows, C, tx, tm, ts, to)
+        st = ctx.sync()
+        return to.numpy(), st
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+
+def clamp(ctx, x, lo, hi):
+    try:
+        tx = ctx.upload(x)
+        to = ctx.empty(x.shape, _TMI[x.dtype], x.dtype)
+        ctx.clamp(_TMI[x.dtype], x.size, tx, lo, hi, to)
+        st = ctx.sync()
+        return to.numpy(), st
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)

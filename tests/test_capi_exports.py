@@ -1,0 +1,48 @@
+"""The C-ABI library loads and exports every symbol that include/tosa_mi355.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tosa_mi355.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_path():
+    names = declared_functions()
+    for want in ("tmi_conv2d", "tmi_depthwise_conv2d", "tmi_matmul", "tmi_rescale", "tmi_clamp",
+                 "tmi_conv2d_rescale_clamp", "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_create",
+                 "tmi_ctx_sync", "tmi_buf_alloc", "tmi_upload", "tmi_download"):
+        assert want in names
+
+
+def test_library_exports_every_declared_symbol():
+    from reference_model_amd import capi
+    lib = capi.load_library()
+    missing = [n for n in declared_functions() if not hasattr(lib, n)]
+    assert not missing, f"declared in the header but not exported: {missing}"
+    assert sorted(capi.EXPORTS) == declared_functions()
+    assert b"gfx950" in lib.tmi_version()
+
+
+def test_structs_match_header_sizes():
+    from reference_model_amd import capi
+    assert ctypes.sizeof(capi.ConvDesc) == 4 * 20
+    assert ctypes.sizeof(capi.RescaleDesc) == 4 * 11
+
+
+def test_no_cpu_fallback_without_device():
+    """Without a GPU the context refuses to come up instead of computing anything on the host."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from reference_model_amd import Context
+    with pytest.raises(RuntimeError):
+        Context(0)
