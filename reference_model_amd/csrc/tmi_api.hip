@@ -270,12 +270,20 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     TMI_HIP(ctx, hipSetDevice(ctx->device));
 
     const char* name = nullptr;
-    if (ctx->kernel_choice == 2)
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    if (!depthwise && ctx->kernel_choice != 1)
+        name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                  ctx->flags_dev);
+    if (!name && ctx->kernel_choice == 2)
         return fail(ctx, "%s: no MFMA kernel is eligible for this shape", op);
-    if (depthwise)
+    if (!name && depthwise)
         name = launch_depthwise_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                        ctx->flags_dev);
-    else
+    else if (!name)
         name = launch_conv2d_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
     return after_launch(ctx, name);

@@ -1,0 +1,168 @@
+"""GPU parity of the MFMA CONV2D kernel (implicit GEMM with fused bias / zero-point / RESCALE / CLAMP
+epilogue) against the CPU oracle, through the C ABI.  int8 results are compared bit for bit; fp16 / bf16
+results with the reference's DOT_PRODUCT bound against the fp64 oracle (tolerance printed in the assert)."""
+import numpy as np
+import pytest
+
+import cases
+import dot_product_check as dp
+import gpu_ops
+import oracle
+from reference_model_amd import Context, TmiError, capi
+from test_oracle_kats import CONV_SHAPES
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = Context(0)
+    c.set_kernel_choice(capi.KERNEL_MFMA)
+    yield c
+    c.close()
+
+
+MFMA_SHAPES = CONV_SHAPES + [
+    # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
+    (1, 32, 32, 8, 16, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),       # config 1 geometry
+    (2, 14, 14, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # config 3 geometry, small
+    (1, 9, 9, 16, 16, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),
+    (1, 10, 10, 32, 40, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilation, OC not a multiple of 16
+    (1, 6, 200, 24, 20, 1, 3, (0, 0, 1, 1), (1, 1), (1, 1)),      # wide rows split into two tiles
+    (1, 7, 7, 160, 96, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),       # three channel blocks, two OC blocks
+    (2, 5, 5, 100, 33, 2, 2, (0, 1, 0, 1), (1, 1), (1, 1)),       # ragged channel tail (100 = 64 + 36)
+    (1, 3, 65, 3, 8, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+    (1, 16, 16, 48, 64, 5, 5, (2, 2, 2, 2), (1, 1), (1, 1)),
+    (1, 1, 1, 1, 1, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("shape", MFMA_SHAPES)
+@pytest.mark.parametrize("zps", [(-7, 3), (5, 0), (0, -4), (0, 0), (-128, 127)])
+def test_conv2d_i8_mfma_bit_exact(ctx, shape, zps):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(sum(shape[:7]) + 1000 * (zps[0] + 128) + zps[1] + 128)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
+    bias = rng.integers(-65536, 65536, oc).astype(np.int32)
+    want = oracle.conv2d("i8", x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=zps[1])
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=zps[1])
+    assert ctx.last_kernel == "conv2d_mfma_i8"
+    assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+
+
+@pytest.mark.parametrize("shape", MFMA_SHAPES[5:9])
+def test_conv2d_i8_mfma_broadcast_bias(ctx, shape):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(77)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-127, 128, (oc, kh, kw, ic)).astype(np.int8)
+    bias = np.array([-12345], np.int32)
+    want = oracle.conv2d("i8", x, w, bias, pad, stride, dil, in_zp=2, w_zp=0)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=2, w_zp=0)
+    assert st == capi.VALID and np.array_equal(got, want)
+
+
+def _fused_expect(c, out_dtype=np.int8):
+    acc = oracle.conv2d("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
+    want, st = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype)
+    assert st == oracle.VALID
+    if c["clamp"] is not None:
+        want = oracle.clamp(want, *c["clamp"])
+    return want
+
+
+def _fused_run(ctx, c, out_dtype=np.int8):
+    return gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"],
+                          rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype),
+                          clamp=c["clamp"])
+
+
+def test_config1_conv_rescale(ctx):
+    c = cases.c1()
+    got, st = _fused_run(ctx, c)
+    assert ctx.last_kernel == "conv2d_mfma_i8_rescale"
+    assert st == capi.VALID and np.array_equal(got, _fused_expect(c))
+
+
+def test_config3_resnet_conv_rescale_clamp_full_size(ctx):
+    c = cases.c3()
+    got, st = _fused_run(ctx, c)
+    want = _fused_expect(c)
+    assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert got.min() == 0 and got.max() == 127  # the clamp range is exercised on both ends
+
+
+@pytest.mark.parametrize("out_dtype", [np.int8, np.int16, np.int32])
+def test_fused_rescale_output_types_and_ragged_channels(ctx, out_dtype):
+    rng = np.random.default_rng(5)
+    c = dict(x=rng.integers(-128, 128, (2, 9, 13, 20)).astype(np.int8),
+             w=rng.integers(-127, 128, (37, 3, 3, 20)).astype(np.int8),
+             bias=rng.integers(-5000, 5000, 37).astype(np.int32), in_zp=-11, w_zp=0, pad=(1, 1, 1, 1), stride=(1, 1),
+             dilation=(1, 1), mult=rng.integers(1 << 30, 1 << 31, 37).astype(np.int32),
+             shift=rng.integers(33, 44, 37).astype(np.int8), out_zp=0 if out_dtype != np.int8 else -6,
+             clamp=None)
+    got, st = _fused_run(ctx, c, out_dtype)
+    assert st == capi.VALID and np.array_equal(got, _fused_expect(c, out_dtype))
+
+
+def test_fused_rescale_require_condition_is_reported(ctx):
+    c = cases.c1()
+    c["shift"] = np.full(16, 12, np.int8)  # |acc| exceeds 2^11: apply_scale_32's value range (quant_util.h:59-67)
+    _, st = _fused_run(ctx, c)
+    assert st == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
+
+
+def test_property_linearity_in_bias_and_zero_weights(ctx):
+    """Size-independent properties at the full config-3 shape: zero weights give exactly the bias, and adding
+    a constant to the bias adds it to every int32 output."""
+    c = cases.c3()
+    z = np.zeros_like(c["w"])
+    out0, _ = gpu_ops.conv2d(ctx, c["x"], z, c["bias"], c["pad"], in_zp=c["in_zp"])
+    assert np.array_equal(out0, np.broadcast_to(c["bias"], out0.shape))
+    a, _ = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], in_zp=c["in_zp"])
+    b, _ = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"] + 1000, c["pad"], in_zp=c["in_zp"])
+    assert np.array_equal(b - a, np.full_like(a, 1000))
+    # an input equal to the zero point everywhere contributes nothing, padding included
+    flat = np.full_like(c["x"], c["in_zp"])
+    out1, _ = gpu_ops.conv2d(ctx, flat, c["w"], c["bias"], c["pad"], in_zp=c["in_zp"])
+    assert np.array_equal(out1, np.broadcast_to(c["bias"], out1.shape))
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 8, 8, 32, 48, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+                                   (1, 9, 9, 24, 20, 3, 3, (0, 0, 0, 0), (2, 2), (1, 1)),
+                                   (1, 7, 7, 256, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1))])
+def test_conv2d_fp_mfma_within_dot_product_bound(ctx, kind, shape):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(31 + ic)
+    x = rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float32)
+    w = rng.normal(0, 1 / np.sqrt(kh * kw * ic), (oc, kh, kw, ic)).astype(np.float32)
+    b = rng.normal(0, 0.1, oc).astype(np.float32)
+    if kind == "fp16":
+        xs, ws, bs = x.astype(np.float16), w.astype(np.float16), b.astype(np.float16)
+        xf, wf, bf = (v.astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.FP16
+    else:
+        xs, ws, bs = (cases.float_to_bf16_bits(v) for v in (x, w, b))
+        xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.BF16
+    ref = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil)
+    bnd = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True)
+    got, st = gpu_ops.conv2d(ctx, xs, ws, bs, pad, stride, dil, dtype=dtype)
+    assert ctx.last_kernel == ("conv2d_mfma_f16" if kind == "fp16" else "conv2d_mfma_bf16")
+    imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
+    ksb = dp.kernel_size_bound(kh * kw * ic, kind)
+    res = dp.check(imp, ref, bnd, kind, ksb)
+    # tolerance: |imp-ref| <= 2*ksb * max(bnd*2^-(1+frac), normal_min) per element, sum err^2 <= 1.6*ksb*T
+    assert st == capi.VALID and res["ok"], res
+    assert res["max_ulp"] <= 2.0, res  # fp32 accumulation: the result is the correctly rounded value +- 1 ulp
+
+
+def test_mfma_not_eligible_is_an_error_when_forced(ctx):
+    # a 31x31 kernel with 64 output channels needs a 4.9 MB weight slab: no MFMA tiling fits LDS
+    x = np.zeros((1, 31, 31, 64), np.int8)
+    w = np.zeros((64, 31, 31, 64), np.int8)
+    with pytest.raises(TmiError) as e:
+        gpu_ops.conv2d(ctx, x, w, np.zeros(1, np.int32))
+    assert "no MFMA kernel" in e.value.message
