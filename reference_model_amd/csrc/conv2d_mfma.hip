@@ -156,6 +156,7 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
     using acc_t            = typename M::acc_t;
     constexpr int EB       = sizeof(T);
     constexpr int OCB      = 16 * OCT;
+    constexpr int STAGE_U  = 8;    // global loads in flight per lane while staging
     const ConvGeom& g      = a.g;
     const int tid          = threadIdx.x;
     const int lane         = tid & 63;
@@ -173,6 +174,9 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
     uint8_t* wl        = lds + tab_bytes;
     uint8_t* pl        = wl + (size_t)taps * OCB * a.wstride;
 
+#ifdef TMI_X_EARLY_RETURN
+    if (a.ksteps < 1000) return;
+#endif
     // ---- which tile --------------------------------------------------------------------------------
     int bid = blockIdx.x;
     if (a.xcd_remap)
@@ -233,47 +237,82 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
         const int ic_off = icb * blk_bytes;
         if (icb)
             __syncthreads();
-        // ---- stage weights: [tap][row][CH chunks] --------------------------------------------------
+        // ---- stage weights [tap][row][CH chunks] and the input patch [py][px][CH chunks] ------------------
+        // Loads are issued in batches of STAGE_U per lane before any of them is written to LDS, so that
+        // the HBM/L2 latency is paid once per batch rather than once per chunk.
+#ifndef TMI_X_NO_STAGE
         {
-            const int total = OCB * taps * a.CH;
-            for (int idx = tid; idx < total; idx += 256)
+            const int w_total = OCB * taps * a.CH;
+            const int p_total = a.PH * a.PW * a.CH;
+            for (int base = tid; base < w_total; base += 256 * STAGE_U)
             {
-                const int cc  = idx & (a.CH - 1);
-                const int r2  = idx >> ch_shift;
-                const int tap = r2 % taps;
-                const int ocl = r2 / taps;
-                v4i v         = v4i{ 0, 0, 0, 0 };
-                if (oc0 + ocl < g.OC)
-                    v = load_chunk(a.w + ((size_t)(oc0 + ocl) * taps + tap) * row_bytes, ic_off + cc * 16, row_bytes,
-                                   vec_ok);
-                const int grp = ocl / (4 * OCT), rem = ocl % (4 * OCT);
-                const int row = (rem >> 2) * 16 + grp * 4 + (rem & 3);
-                *reinterpret_cast<v4i*>(wl + (size_t)(tap * OCB + row) * a.wstride + cc * 16) = v;
+                v4i v[STAGE_U];
+                int dst[STAGE_U];
+#pragma unroll
+                for (int u = 0; u < STAGE_U; u++)
+                {
+                    const int idx = base + u * 256;
+                    v[u]          = v4i{ 0, 0, 0, 0 };
+                    dst[u]        = -1;
+                    if (idx < w_total)
+                    {
+                        const int cc  = idx & (a.CH - 1);
+                        const int r2  = idx >> ch_shift;
+                        const int ocl = r2 / taps;
+                        const int tap = r2 - ocl * taps;
+                        if (oc0 + ocl < g.OC)
+                            v[u] = load_chunk(a.w + ((size_t)(oc0 + ocl) * taps + tap) * row_bytes, ic_off + cc * 16,
+                                              row_bytes, vec_ok);
+                        const int grp = ocl / (4 * OCT), rem = ocl % (4 * OCT);
+                        const int row = (rem >> 2) * 16 + grp * 4 + (rem & 3);
+                        dst[u]        = (tap * OCB + row) * a.wstride + cc * 16;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < STAGE_U; u++)
+                    if (dst[u] >= 0)
+                        *reinterpret_cast<v4i*>(wl + dst[u]) = v[u];
+            }
+            for (int base = tid; base < p_total; base += 256 * STAGE_U)
+            {
+                v4i v[STAGE_U];
+                int dst[STAGE_U];
+#pragma unroll
+                for (int u = 0; u < STAGE_U; u++)
+                {
+                    const int idx = base + u * 256;
+                    v[u]          = v4i{ 0, 0, 0, 0 };
+                    dst[u]        = -1;
+                    if (idx < p_total)
+                    {
+                        const int cc  = idx & (a.CH - 1);
+                        const int pix = idx >> ch_shift;
+                        const int py  = pix / a.PW;
+                        const int px  = pix - py * a.PW;
+                        const int iy = y0 + py, ix = x0 + px;
+                        if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW)
+                            v[u] = load_chunk(a.in + (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes,
+                                              ic_off + cc * 16, row_bytes, vec_ok);
+                        else
+                            v[u] = fill_chunk(ic_off + cc * 16, row_bytes, M::is_int ? a.za : 0);
+                        dst[u] = pix * a.pstride + cc * 16;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < STAGE_U; u++)
+                    if (dst[u] >= 0)
+                        *reinterpret_cast<v4i*>(pl + dst[u]) = v[u];
             }
         }
-        // ---- stage the input patch: [py][px][CH chunks] ----------------------------------------------
-        {
-            const int total = a.PH * a.PW * a.CH;
-            for (int idx = tid; idx < total; idx += 256)
-            {
-                const int cc  = idx & (a.CH - 1);
-                const int pix = idx >> ch_shift;
-                const int py  = pix / a.PW;
-                const int px  = pix - py * a.PW;
-                const int iy = y0 + py, ix = x0 + px;
-                v4i v;
-                if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW)
-                    v = load_chunk(a.in + (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes, ic_off + cc * 16,
-                                   row_bytes, vec_ok);
-                else
-                    v = fill_chunk(ic_off + cc * 16, row_bytes, M::is_int ? a.za : 0);
-                *reinterpret_cast<v4i*>(pl + (size_t)pix * a.pstride + cc * 16) = v;
-            }
-        }
+#endif
         __syncthreads();
 
         // ---- MFMA over the (tap, chunk) pairs of this channel block -----------------------------------
+#ifndef TMI_X_NO_MFMA
         if (wave_active)
+#else
+        if (wave_active && a.ksteps > 1000)
+#endif
         {
             for (int s = 0; s < a.ksteps; s++)
             {
@@ -312,6 +351,9 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
 
     if (!wave_active)
         return;
+#ifdef TMI_X_NO_EPILOGUE_AT_ALL
+    if (a.ksteps < 1000) { if (acc[0][0][0] == 0x12345678) a.flag_word[1] = 1; return; }
+#endif
 
     // ---- epilogue -------------------------------------------------------------------------------------
     uint32_t flags = 0;
@@ -343,6 +385,10 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
                     corr[t][r] = 0;
         }
         const int kzz = g.KH * g.KW * g.IC * a.za * a.zw;
+        // per pixel group: validity, output offset and the zero-point term that depends on the pixel
+        bool pix_ok[PXT];
+        size_t obase[PXT];
+        int pcorr[PXT];
 #pragma unroll
         for (int i = 0; i < PXT; i++)
         {
@@ -352,80 +398,150 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
                 sa += __shfl_xor(sa, 16);
                 sa += __shfl_xor(sa, 32);
             }
-            const int p = (wave * PXT + i) * 16 + li;
+            pcorr[i]     = kzz - a.zw * sa;
+            const int p  = (wave * PXT + i) * 16 + li;
             const int ty = p / a.TW, tx = p - ty * a.TW;
             const int oy = oy0 + ty, ox = ox0 + tx;
-            const bool pix_ok = p < P && oy < g.OH && ox < g.OW;
-            if (!pix_ok)
-                continue;
-            const size_t obase = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
-            int32_t res[4 * OCT];
+            pix_ok[i]    = p < P && oy < g.OH && ox < g.OW;
+            obase[i]     = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
+        }
+        const bool full    = (oc0 + ocl0 + 4 * OCT <= g.OC);
+        const bool vec_out = full && (g.OC % (4 * OCT)) == 0 && ((uintptr_t)a.out & 15) == 0;
+        // bias / multiplier / shift / int32 output rows of four channels can be moved as one vector
+        const bool vec_par = full && (g.OC & 3) == 0 && (oc0 + ocl0) % 4 == 0 &&
+                             (((uintptr_t)a.bias | (uintptr_t)a.out | (a.rp.enabled ? (uintptr_t)a.rp.multiplier : 0)) & 15) == 0 &&
+                             (!a.rp.enabled || ((uintptr_t)a.rp.shift & 3) == 0);
+        int packed[PXT][OCT];    // int8 results, four channels per word
+
+        // channel tile by channel tile: fetch the four channels' constants once, use them for every pixel
 #pragma unroll
-            for (int t = 0; t < OCT; t++)
+        for (int t = 0; t < OCT; t++)
+        {
+            const int c0 = oc0 + ocl0 + 4 * t;
+            int32_t bias4[4], mult4[4], shift4[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                bias4[r] = mult4[r] = 0, shift4[r] = 32;    // neutral: every value legal, result 0
+            if (g.bias_len == 1)
+            {
+                const int32_t b = reinterpret_cast<const int32_t*>(a.bias)[0];
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                {
-                    const int oc = oc0 + ocl0 + 4 * t + r;
-                    int32_t v    = acc[i][t][r] - a.zw * sa - corr[t][r] + kzz;
-                    if (oc < g.OC)
-                    {
-                        v += reinterpret_cast<const int32_t*>(a.bias)[g.bias_len == 1 ? 0 : oc];
-                        if (a.rp.enabled)
-                            v = rescale_value(a.rp, v, load_multiplier(a.rp, oc), load_shift(a.rp, oc), flags);
-                    }
-                    res[4 * t + r] = v;
-                }
-            const bool full = (oc0 + ocl0 + 4 * OCT <= g.OC);
-            if (a.out_dtype == TMI_INT32)
-            {
-                int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase;
-                if (full && (g.OC & 3) == 0)
-                {
-#pragma unroll
-                    for (int t = 0; t < OCT; t++)
-                        *reinterpret_cast<v4i*>(o + 4 * t) = v4i{ res[4 * t], res[4 * t + 1], res[4 * t + 2],
-                                                                  res[4 * t + 3] };
-                }
-                else
-                {
-#pragma unroll
-                    for (int j = 0; j < 4 * OCT; j++)
-                        if (oc0 + ocl0 + j < g.OC)
-                            o[j] = res[j];
-                }
+                    bias4[r] = b;
             }
-            else if (a.out_dtype == TMI_INT8)
+            else if (vec_par)
             {
-                int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase;
-                if (full && (g.OC % (4 * OCT)) == 0)
-                {
-                    int packed[OCT];
-#pragma unroll
-                    for (int t = 0; t < OCT; t++)
-                        packed[t] = (res[4 * t] & 0xff) | ((res[4 * t + 1] & 0xff) << 8) |
-                                    ((res[4 * t + 2] & 0xff) << 16) | ((res[4 * t + 3] & 0xff) << 24);
-                    if constexpr (OCT == 4)
-                        *reinterpret_cast<v4i*>(o) = v4i{ packed[0], packed[1], packed[2], packed[3] };
-                    else
-#pragma unroll
-                        for (int t = 0; t < OCT; t++)
-                            reinterpret_cast<int*>(o)[t] = packed[t];
-                }
-                else
-                {
-#pragma unroll
-                    for (int j = 0; j < 4 * OCT; j++)
-                        if (oc0 + ocl0 + j < g.OC)
-                            o[j] = (int8_t)res[j];
-                }
+                const v4i b = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(a.bias) + c0);
+                bias4[0] = b.x, bias4[1] = b.y, bias4[2] = b.z, bias4[3] = b.w;
             }
             else
             {
-                int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase;
 #pragma unroll
-                for (int j = 0; j < 4 * OCT; j++)
-                    if (oc0 + ocl0 + j < g.OC)
-                        o[j] = (int16_t)res[j];
+                for (int r = 0; r < 4; r++)
+                    if (c0 + r < g.OC)
+                        bias4[r] = reinterpret_cast<const int32_t*>(a.bias)[c0 + r];
+            }
+            ChannelScale cs[4];
+            if (a.rp.enabled)
+            {
+                if (vec_par && a.rp.per_channel && a.rp.scale32)
+                {
+                    const v4i m = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(a.rp.multiplier) + c0);
+                    const int sh = *reinterpret_cast<const int*>(a.rp.shift + c0);
+                    mult4[0] = m.x, mult4[1] = m.y, mult4[2] = m.z, mult4[3] = m.w;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        shift4[r] = (int32_t)(int8_t)(sh >> (8 * r));
+                }
+                else
+                {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (c0 + r < g.OC)
+                            mult4[r] = load_multiplier(a.rp, c0 + r), shift4[r] = load_shift(a.rp, c0 + r);
+                }
+                if (a.rp.fast)
+                {
+                    // channels past OC carry the neutral constants (0, 32) set above and raise nothing
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        cs[r] = make_channel_scale(mult4[r], shift4[r], a.rp.double_round, flags);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+            {
+                int32_t res[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                {
+                    int32_t v = acc[i][t][r] + pcorr[i] - corr[t][r] + bias4[r];
+#ifndef TMI_X_NO_EPI
+                    if (a.rp.enabled)
+                    {
+                        if (a.rp.fast)
+                        {
+                            uint32_t f = 0;
+                            v          = fast_rescale(v, cs[r], a.rp.out_zp, a.rp.lo, a.rp.hi, f);
+                            flags |= pix_ok[i] ? f : 0u;    // pixels outside the image must not raise anything
+                        }
+                        else if (pix_ok[i] && c0 + r < g.OC)
+                            v = rescale_value(a.rp, v, mult4[r], shift4[r], flags);
+                    }
+#endif
+                    res[r] = v;
+                }
+                if (!pix_ok[i])
+                    continue;
+                if (a.out_dtype == TMI_INT32)
+                {
+                    int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase[i] + 4 * t;
+                    if (vec_par)
+                        *reinterpret_cast<v4i*>(o) = v4i{ res[0], res[1], res[2], res[3] };
+                    else
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (c0 + r < g.OC)
+                                o[r] = res[r];
+                }
+                else if (a.out_dtype == TMI_INT8)
+                {
+                    if (vec_out)
+                        packed[i][t] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
+                                       ((res[3] & 0xff) << 24);
+                    else
+                    {
+                        int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i] + 4 * t;
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            if (c0 + r < g.OC)
+                                o[r] = (int8_t)res[r];
+                    }
+                }
+                else
+                {
+                    int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase[i] + 4 * t;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        if (c0 + r < g.OC)
+                            o[r] = (int16_t)res[r];
+                }
+            }
+        }
+        if (a.out_dtype == TMI_INT8 && vec_out)
+        {
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+            {
+                if (!pix_ok[i])
+                    continue;
+                int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i];
+                if constexpr (OCT == 4)
+                    *reinterpret_cast<v4i*>(o) = v4i{ packed[i][0], packed[i][1], packed[i][2], packed[i][3] };
+                else
+#pragma unroll
+                    for (int t = 0; t < OCT; t++)
+                        reinterpret_cast<int*>(o)[t] = packed[i][t];
             }
         }
         raise_flags(a.flag_word, flags);

@@ -154,6 +154,21 @@ int64_t extend(int32_t v, int bits, bool is_unsigned)
     return is_unsigned ? (int64_t)(uint32_t)v : (int64_t)v;
 }
 
+// Decides whether the kernels may use fast_rescale(): signed INT32 input, no input zero point, 32-bit scale
+// with SINGLE or DOUBLE rounding, and an output clip / CLAMP pair that merges into one range.
+void set_fast_path(RescaleParams& p)
+{
+    p.lo = p.qmin, p.hi = p.qmax;
+    bool merged = true;
+    if (p.has_clamp)
+    {
+        p.lo   = p.qmin > p.clamp_min ? p.qmin : p.clamp_min;
+        p.hi   = p.qmax < p.clamp_max ? p.qmax : p.clamp_max;
+        merged = p.lo <= p.hi;
+    }
+    p.fast = merged && p.scale32 && !p.inexact_round && p.in_bits == 32 && !p.in_unsigned && p.in_zp == 0;
+}
+
 // OpRescale::checkTensorAttributes (type_conversion.cpp:111-151) and the zero-point ERROR_IFs of eval
 // (:242-255).  Fills the kernel parameters.
 int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, int32_t C, const void* mult,
@@ -229,6 +244,7 @@ int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, in
     p.in_unsigned   = in_u;
     p.has_clamp     = 0;
     p.enabled       = 1;
+    set_fast_path(p);
     return TMI_VALID;
 }
 
@@ -253,6 +269,7 @@ int validate_fused_rescale(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* 
         p.has_clamp = 1;
         p.clamp_min = clamp_min;
         p.clamp_max = clamp_max;
+        set_fast_path(p);
     }
     return TMI_VALID;
 }

@@ -22,6 +22,19 @@ struct RescaleParams
     int32_t clamp_min, clamp_max;
     uint8_t scale32, double_round, inexact_round, per_channel;
     uint8_t in_bits, in_unsigned, has_clamp, enabled;
+    // Set by the host when the input is a signed INT32 value with zero input_zp, scale32 is on and the
+    // rounding is SINGLE or DOUBLE: the kernels may then use fast_rescale() with the merged range [lo, hi]
+    // (output clip followed by CLAMP) instead of the general rescale_value().
+    uint8_t fast;
+    int32_t lo, hi;
+};
+
+// Per-channel constants of the fast path, derived once per channel and reused for every pixel.
+struct ChannelScale
+{
+    int32_t m, s;
+    int64_t rnd_pos, rnd_neg;    // rounding constant for value >= 0 / value < 0 (double round folded in)
+    uint32_t lim, lim2;          // value v is legal iff (uint32)(v + lim) <= lim2
 };
 
 // value_extend64_impl of the reference (type_conversion.cpp:183-221) for 8/16/32-bit storage.
@@ -105,6 +118,42 @@ __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int32_t
         r = r >= p.clamp_min ? r : p.clamp_min;
         r = r < p.clamp_max ? r : p.clamp_max;
     }
+    return r;
+}
+
+__device__ __forceinline__ ChannelScale make_channel_scale(int32_t m, int32_t s, bool double_round, uint32_t& flags)
+{
+    if (m < 0)
+        flags |= TMI_FLAG_SCALE_MULTIPLIER;
+    if (s < 2 || s > 62)
+    {
+        flags |= TMI_FLAG_SCALE_SHIFT;
+        s = 2;
+    }
+    ChannelScale c;
+    c.m               = m;
+    c.s               = s;
+    const int64_t rnd = int64_t(1) << (s - 1);
+    const int64_t adj = (double_round && s > 31) ? (int64_t(1) << 30) : 0;
+    c.rnd_pos         = rnd + adj;
+    c.rnd_neg         = rnd - adj;
+    c.lim             = s <= 31 ? (1u << (s - 1)) : 0x80000000u;
+    c.lim2            = 2u * c.lim - 1u;    // 0xffffffff when every int32 value is legal
+    return c;
+}
+
+// apply_scale_32 + output_zp + clip (+ CLAMP) for a signed int32 value with zero input_zp.  With a legal
+// value |v| < 2^(s-1) and m < 2^31 the scaled result is below 2^30 in magnitude, so neither of the
+// reference's int32 range checks (quant_util.h:78-82, type_conversion.cpp:352-360) can fire here.
+__device__ __forceinline__ int32_t fast_rescale(int32_t v, const ChannelScale& c, int32_t out_zp, int32_t lo,
+                                                int32_t hi, uint32_t& flags)
+{
+    if ((uint32_t)v + c.lim > c.lim2)
+        flags |= TMI_FLAG_SCALE_VALUE;
+    const int64_t p = (int64_t)v * (int64_t)c.m + (v >= 0 ? c.rnd_pos : c.rnd_neg);
+    int32_t r       = (int32_t)(p >> c.s) + out_zp;
+    r               = r < lo ? lo : r;
+    r               = r > hi ? hi : r;
     return r;
 }
 
