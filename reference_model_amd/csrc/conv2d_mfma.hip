@@ -1,35 +1,71 @@
 // CONV2D as an implicit GEMM on the matrix cores (MFMA), with the bias / zero-point / RESCALE / CLAMP
 // epilogue fused so that the int32 accumulators never reach HBM.
 //
-// One workgroup (4 waves) computes a TH x TW tile of output pixels of one image for a block of OCB =
-// 16*OCT output channels.  Per block of 64 bytes of input channels it stages in LDS
+// One workgroup (8 waves) computes a TH x TW tile of output pixels of one image for a block of OCB =
+// 32*WOC output channels; wave w owns channel tile w / (8/WOC) and PXT pixel tiles of 32 pixels.  Two waves
+// per SIMD is what hides LDS and VALU latency here: the named shapes are far too small to fill the chip with
+// bigger per-wave tiles.  Per block of 64 bytes of input channels the workgroup stages in LDS
 //   - the input patch that the tile needs (PH x PW pixels, out-of-image pixels filled with input_zp, so the
-//     zero-point identity below holds with the full K), each pixel a row of CH 16-byte chunks, and
-//   - the weight slab [tap][channel row][CH chunks],
-// both with a row stride chosen so that the 16 lanes of a ds_read_b128 phase hit distinct banks.
+//     zero-point identity below holds with the full K): one row of CH 16-byte chunks per pixel, and
+//   - the weight slab: one row per output channel holding its KH*KW*CH chunks in (tap, chunk) order, which
+//     is the order they have in HBM.
 // Every input byte is read from HBM/L2 once per workgroup (plus the halo) and reused KH*KW*OCB times
 // from LDS.
 //
-// MFMA operand roles: the weights are the "A" operand (rows of D = output channels), the pixels the "B"
-// operand (columns of D = pixels).  With the 16x16 accumulator layout (lane l, register r) = D[4*(l/16)+r]
-// [l%16], assigning output channel 4*OCT*(i/4) + 4*t + i%4 to row i of channel tile t makes every lane own
-// 4*OCT consecutive channels of one pixel, i.e. one 16-byte store of int8 results for OCT = 4.
+// The MFMA is the 32x32 shape (v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x16_{f16,bf16}), which on this chip
+// runs at the full int8 rate while the 16x16x64 shape does not.  A fragment gives every lane 16 bytes: lane
+// l holds row l%32, K half l/32.  Both LDS row strides are kept congruent to 16 modulo 32 bytes, the layout
+// for which ds_read_b128 of such a fragment runs at the full LDS rate (measured: 16/48/80/.. bytes reach
+// ~230 B/clk/CU, 32/64/96 bytes half or less).
 //
-// A K-step feeds each lane 16 bytes of one (tap, channel chunk) pair; lane group g = l/16 takes pair
-// 4*step+g.  Integer dot products are order independent, so which pair lands in which lane group does not
-// matter as long as both operands agree.
+// Operand roles: the weights are the "A" operand (rows of D = output channels), the pixels the "B" operand
+// (columns of D = pixels).  With the 32x32 accumulator layout (lane l, register 4q+j) = D[8q + 4(l/32) + j]
+// [l%32], giving row 8q+4h+j of a channel tile the output channel 16h + 4q + j makes every lane own 16
+// consecutive channels of one pixel: its int8 results leave as one 16-byte store.
+//
+// A K-step feeds each lane 16 bytes of one (tap, chunk) pair; lane half h takes pair 2*step+h.  The K loop is
+// software pipelined three deep (fragments of step s+2 are requested before the MFMAs of step s issue) and a
+// dead pair (odd pair count) is read from a zeroed LDS chunk so that no instruction has to touch a fragment
+// between its load and its MFMA.  Integer dot
+// products are order independent, so the assignment of pairs to lanes is free as long as both operands
+// agree; the floating-point variants are compared against fp64 with the reference's DOT_PRODUCT bound.
 //
 // Zero points: sum((a-za)(w-zw)) = sum(a*w) - zw*sum(a) - za*sum(w) + K*za*zw.  sum(w) per channel and
 // sum(a) per pixel are accumulated from the very fragments fed to the MFMA with v_dot4 against 0x01010101.
+//
+// Epilogue: the per-channel constants (bias, multiplier, shift and the 64-bit rounding terms derived from
+// them) are computed once per workgroup by OCB lanes while the staging loads are in flight and kept in an
+// LDS table; every lane then spends about ten instructions per output element.
 #include "tmi_kernels.h"
 
 namespace tmi
 {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+
+// n / d for n*d < 2^32 as one multiply-high (magic = floor(2^32/d) + 1; d == 1 is special-cased).
+struct FastDiv
+{
+    uint32_t magic, d;
+};
+
+static FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f;
+    f.d     = d;
+    f.magic = d <= 1 ? 0u : (uint32_t)((uint64_t(1) << 32) / d) + 1u;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f)
+{
+    return f.d <= 1 ? n : __umulhi(n, f.magic);
+}
 
 struct PatchArgs
 {
@@ -41,15 +77,16 @@ struct PatchArgs
     uint32_t* flag_word;
     RescaleParams rp;
     int32_t za, zw;
-    int32_t TH, TW, tiles_y, tiles_x, oc_blocks;
+    int32_t TH, TW, tiles_y, tiles_x;
     int32_t PH, PW;
-    int32_t CH;               // 16-byte chunks per pixel row in LDS (1, 2 or 4)
-    int32_t pstride, wstride; // LDS row strides in bytes
-    int32_t n_icb;            // blocks of CH*16 bytes along the input channels
-    int32_t ksteps;           // MFMA K-steps per channel block = ceil(taps*CH/4)
-    int32_t n_tiles;          // N * tiles_y * tiles_x
+    int32_t CH;                  // 16-byte chunks per pixel row in LDS (1, 2 or 4)
+    int32_t pstride, wstride;    // LDS row strides in bytes, both = 16 (mod 32)
+    int32_t n_icb;               // blocks of CH*16 bytes along the input channels
+    int32_t ksteps;              // MFMA K-steps per channel block = ceil(taps*CH/2)
+    int32_t n_tiles;             // N * tiles_y * tiles_x
     int32_t out_dtype;
     int32_t xcd_remap;
+    FastDiv div_tw, div_pw, div_rch, div_tiles_x, div_tiles_y, div_n_tiles, div_kw;
 };
 
 template <typename T>
@@ -58,32 +95,32 @@ struct Mma;
 template <>
 struct Mma<int8_t>
 {
-    using acc_t                  = v4i;
+    using acc_t                  = v16i;
     static constexpr bool is_int = true;
-    __device__ static v4i mma(v4i a, v4i b, v4i c)
+    __device__ static v16i mma(v4i a, v4i b, v16i c)
     {
-        return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
     }
 };
 template <>
 struct Mma<_Float16>
 {
-    using acc_t                  = v4f;
+    using acc_t                  = v16f;
     static constexpr bool is_int = false;
-    __device__ static v4f mma(v4i a, v4i b, v4f c)
+    __device__ static v16f mma(v4i a, v4i b, v16f c)
     {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0,
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0,
                                                       0, 0);
     }
 };
 template <>
 struct Mma<bf16_t>
 {
-    using acc_t                  = v4f;
+    using acc_t                  = v16f;
     static constexpr bool is_int = false;
-    __device__ static v4f mma(v4i a, v4i b, v4f c)
+    __device__ static v16f mma(v4i a, v4i b, v16f c)
     {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, a), __builtin_bit_cast(v8b, b), c, 0,
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b, a), __builtin_bit_cast(v8b, b), c, 0,
                                                        0, 0);
     }
 };
@@ -96,377 +133,446 @@ __device__ __forceinline__ int dot4_ones(v4i v)
     return __builtin_amdgcn_sdot4(v.w, 0x01010101, s, false);
 }
 
-// 16 bytes starting at byte offset `off` of a row of `row_bytes` bytes; bytes past the row end read as 0.
-// `vec_ok` says that every row start and `off` are 16-byte aligned and the row length is a multiple of 16.
-__device__ __forceinline__ v4i load_chunk(const uint8_t* row, int off, int row_bytes, bool vec_ok)
+// Byte-wise version of a chunk load for channel vectors whose length is not a multiple of 16 bytes
+// (rows are then unaligned): bytes past the row end read as 0.  The rare path.
+__device__ __forceinline__ v4i load_chunk_bytes(const uint8_t* row, int off, int row_bytes)
 {
-    if (vec_ok)
+    v4i r;
+#pragma unroll
+    for (int k = 0; k < 4; k++)
     {
-        if (off < row_bytes)
-            return *reinterpret_cast<const v4i*>(row + off);
-        return v4i{ 0, 0, 0, 0 };
+        uint32_t word = 0;
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            if (off + 4 * k + b < row_bytes)
+                word |= (uint32_t)row[off + 4 * k + b] << (8 * b);
+        r[k] = (int)word;
     }
-    union
-    {
-        v4i v;
-        uint8_t b[16];
-    } u;
-    u.v = v4i{ 0, 0, 0, 0 };
-    for (int j = 0; j < 16; j++)
-        if (off + j < row_bytes)
-            u.b[j] = row[off + j];
-    return u.v;
+    return r;
 }
 
-// 16 bytes of the fill value (input_zp in every byte) limited to the row, zero beyond it.
+// 16 bytes of the fill byte limited to the row, zero beyond it.
 __device__ __forceinline__ v4i fill_chunk(int off, int row_bytes, int fill_byte)
 {
     const int word = (fill_byte & 0xff) * 0x01010101;
-    if (off + 16 <= row_bytes)
+    const int n    = row_bytes - off;    // bytes of this chunk that belong to the row
+    if (n >= 16)
         return v4i{ word, word, word, word };
-    union
+    v4i r;
+#pragma unroll
+    for (int k = 0; k < 4; k++)
     {
-        v4i v;
-        uint8_t b[16];
-    } u;
-    u.v = v4i{ 0, 0, 0, 0 };
-    for (int j = 0; j < 16; j++)
-        if (off + j < row_bytes)
-            u.b[j] = (uint8_t)fill_byte;
-    return u.v;
+        const int m = n - 4 * k;    // bytes of word k inside the row
+        r[k]        = m >= 4 ? word : (m <= 0 ? 0 : (word & ((1 << (8 * m)) - 1)));
+    }
+    return r;
 }
 
-template <typename OutT>
-__device__ __forceinline__ OutT to_out(float v);
+template <typename T>
+__device__ __forceinline__ float load_as_float(const void* p, int i);
 template <>
-__device__ __forceinline__ _Float16 to_out<_Float16>(float v)
+__device__ __forceinline__ float load_as_float<_Float16>(const void* p, int i)
 {
-    return (_Float16)v;
+    return (float)reinterpret_cast<const _Float16*>(p)[i];
 }
 template <>
-__device__ __forceinline__ bf16_t to_out<bf16_t>(float v)
+__device__ __forceinline__ float load_as_float<bf16_t>(const void* p, int i)
 {
-    return float_to_bf16(v);
+    return bf16_to_float(reinterpret_cast<const bf16_t*>(p)[i]);
+}
+template <>
+__device__ __forceinline__ float load_as_float<int8_t>(const void*, int)
+{
+    return 0.0f;
 }
 
-template <typename T, int OCT, int PXT>
-__global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
+__device__ __forceinline__ void store_from_float(_Float16* p, float v)
 {
-    using M                = Mma<T>;
-    using acc_t            = typename M::acc_t;
-    constexpr int EB       = sizeof(T);
-    constexpr int OCB      = 16 * OCT;
-    constexpr int STAGE_U  = 8;    // global loads in flight per lane while staging
-    const ConvGeom& g      = a.g;
-    const int tid          = threadIdx.x;
-    const int lane         = tid & 63;
-    const int wave         = tid >> 6;
-    const int li           = lane & 15;    // row of the A fragment / column (pixel) of D
-    const int lg           = lane >> 4;    // K chunk taken by this lane / row group of D
-    const int taps         = g.KH * g.KW;
-    const int row_bytes    = g.IC * EB;    // bytes of one pixel's (or one weight tap's) channel vector
-    const int blk_bytes    = a.CH * 16;
-    const bool vec_ok      = (row_bytes % 16) == 0;
+    *p = (_Float16)v;
+}
+__device__ __forceinline__ void store_from_float(bf16_t* p, float v)
+{
+    *p = float_to_bf16(v);
+}
+__device__ __forceinline__ void store_from_float(int8_t*, float)
+{}
 
+enum
+{
+    EPI_PLAIN   = 0,    // int32 (or floating-point) result stored as is
+    EPI_FAST    = 1,    // RESCALE (+CLAMP) through fast_rescale()
+    EPI_GENERIC = 2     // any other RESCALE, staged through LDS
+};
+
+// Per-channel constants of the integer epilogues, one 32-byte LDS entry per channel of the block.
+struct alignas(16) ChanEntry
+{
+    int32_t m, s, bias;
+    uint32_t lim;
+    int64_t rnd_pos, rnd_neg;
+};
+
+template <typename T, int WOC, int PXT, int EPI, bool VEC>
+__global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
+{
+    using M              = Mma<T>;
+    using acc_t          = typename M::acc_t;
+    constexpr int EB     = sizeof(T);
+    constexpr int NT     = 512;          // lanes per workgroup
+    constexpr int WPX    = 8 / WOC;      // waves along the pixel dimension
+    constexpr int OCB    = 32 * WOC;     // output channels per workgroup
+    constexpr int WU     = 5;            // weight chunks in flight per lane in one staging round
+    constexpr int PU     = 2;            // patch chunks in flight per lane in one staging round
+    const ConvGeom& g    = a.g;
+    const int tid        = threadIdx.x;
+    const int lane       = tid & 63;
+    const int wave       = tid >> 6;
+    const int woc        = wave / WPX;   // channel tile of this wave
+    const int wpx        = wave % WPX;   // first pixel tile of this wave is wpx*PXT
+    const int li         = lane & 31;    // row of the A fragment / column (pixel) of D
+    const int lh         = lane >> 5;    // K half taken by this lane / row half of D
+    const int taps       = g.KH * g.KW;
+    const int row_bytes  = g.IC * EB;    // bytes of one pixel's (or one weight tap's) channel vector
+    const int blk_bytes  = a.CH * 16;
+    const int ch_shift   = a.CH == 4 ? 2 : (a.CH == 2 ? 1 : 0);
+    const int n_pairs    = taps * a.CH;  // (tap, chunk) pairs per channel block = chunks per weight row
+
+    // LDS: [channel table][16 zero bytes][pair offset table][weight rows][input patch]
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    int* tapoff        = reinterpret_cast<int*>(lds);
-    const int tab_bytes = (taps * 4 + 15) & ~15;
-    uint8_t* wl        = lds + tab_bytes;
-    uint8_t* pl        = wl + (size_t)taps * OCB * a.wstride;
+    ChanEntry* ctab        = reinterpret_cast<ChanEntry*>(lds);
+    float* ftab            = reinterpret_cast<float*>(lds);    // floating point: bias as float
+    constexpr int kCtab    = OCB * (int)sizeof(ChanEntry);
+    uint8_t* zero_chunk    = lds + kCtab;
+    int* pairoff           = reinterpret_cast<int*>(lds + kCtab + 16);
+    const int tab_entries  = n_pairs + 12;    // slack: the pipeline reads a few entries past the end
+    const int tab_bytes    = (tab_entries * 4 + 15) & ~15;
+    uint8_t* wl            = lds + kCtab + 16 + tab_bytes;
+    uint8_t* pl            = wl + OCB * a.wstride;
 
-#ifdef TMI_X_EARLY_RETURN
-    if (a.ksteps < 1000) return;
-#endif
-    // ---- which tile --------------------------------------------------------------------------------
-    int bid = blockIdx.x;
+    // ---- which tile ------------------------------------------------------------------------------------
+    uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
     {
         // consecutive workgroups are dealt to the 8 XCDs in turn; give each XCD a contiguous run of tiles
         // so that neighbouring tiles (which share halo rows) share an L2
-        const int per = gridDim.x >> 3;
-        bid           = (bid & 7) * per + (bid >> 3);
+        const uint32_t per = gridDim.x >> 3;
+        bid                = (bid & 7) * per + (bid >> 3);
     }
-    const int ocb   = bid / a.n_tiles;
-    int tile        = bid - ocb * a.n_tiles;
-    const int txi   = tile % a.tiles_x;
-    tile /= a.tiles_x;
-    const int tyi   = tile % a.tiles_y;
-    const int n     = tile / a.tiles_y;
-    const int oy0   = tyi * a.TH;
-    const int ox0   = txi * a.TW;
-    const int oc0   = ocb * OCB;
-    const int y0    = oy0 * g.stride_y - g.pad_top;
-    const int x0    = ox0 * g.stride_x - g.pad_left;
-    const int P     = a.TH * a.TW;
+    const uint32_t ocb  = fdiv(bid, a.div_n_tiles);
+    uint32_t tile       = bid - ocb * a.n_tiles;
+    const uint32_t trow = fdiv(tile, a.div_tiles_x);
+    const int txi       = tile - trow * a.tiles_x;
+    const int n         = fdiv(trow, a.div_tiles_y);
+    const int tyi       = trow - n * a.tiles_y;
+    const int oy0       = tyi * a.TH;
+    const int ox0       = txi * a.TW;
+    const int oc0       = ocb * OCB;
+    const int y0        = oy0 * g.stride_y - g.pad_top;
+    const int x0        = ox0 * g.stride_x - g.pad_left;
+    const int P         = a.TH * a.TW;
 
-    for (int t = tid; t < taps; t += 256)
-        tapoff[t] = ((t / g.KW) * g.dil_y * a.PW + (t % g.KW) * g.dil_x) * a.pstride;
+    // ---- tables ----------------------------------------------------------------------------------------
+    uint32_t flags = 0;
+    if (tid < 4)
+        reinterpret_cast<int*>(zero_chunk)[tid] = 0;
+    for (int q = tid; q < tab_entries; q += NT)
+    {
+        int off = 0;
+        if (q < n_pairs)
+        {
+            const int tap = q >> ch_shift;
+            const int ky  = fdiv(tap, a.div_kw);
+            const int kx  = tap - ky * g.KW;
+            off           = (ky * g.dil_y * a.PW + kx * g.dil_x) * a.pstride + (q & (a.CH - 1)) * 16;
+        }
+        pairoff[q] = off;
+    }
+    if (tid < OCB)
+    {
+        const int oc  = oc0 + tid;
+        const bool ok = oc < g.OC;
+        if constexpr (M::is_int)
+        {
+            ChanEntry e;
+            e.bias = ok ? reinterpret_cast<const int32_t*>(a.bias)[g.bias_len == 1 ? 0 : oc] : 0;
+            e.m = 0, e.s = 32, e.lim = 0x80000000u, e.rnd_pos = e.rnd_neg = 0;
+            if constexpr (EPI == EPI_FAST)
+            {
+                // channels past OC get neutral constants (0, 32): every value legal, nothing raised
+                const int32_t m       = ok ? load_multiplier(a.rp, oc) : 0;
+                const int32_t sh      = ok ? load_shift(a.rp, oc) : 32;
+                const ChannelScale cs = make_channel_scale(m, sh, a.rp.double_round, flags);
+                e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos, e.rnd_neg = cs.rnd_neg;
+            }
+            ctab[tid] = e;
+        }
+        else
+            ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : oc) : 0.0f;
+    }
 
-    // ---- per-lane pixel bases ----------------------------------------------------------------------
+    // ---- per-lane pixel bases --------------------------------------------------------------------------
     int pbase[PXT];
 #pragma unroll
     for (int i = 0; i < PXT; i++)
     {
-        int p = (wave * PXT + i) * 16 + li;
+        int p = (wpx * PXT + i) * 32 + li;
         if (p >= P)
             p = 0;
-        pbase[i] = ((p / a.TW) * g.stride_y * a.PW + (p % a.TW) * g.stride_x) * a.pstride;
+        const int ty = fdiv(p, a.div_tw);
+        pbase[i]     = (ty * g.stride_y * a.PW + (p - ty * a.TW) * g.stride_x) * a.pstride;
     }
 
-    acc_t acc[PXT][OCT];
+    acc_t acc[PXT];
 #pragma unroll
     for (int i = 0; i < PXT; i++)
 #pragma unroll
-        for (int t = 0; t < OCT; t++)
-            acc[i][t] = acc_t{ 0, 0, 0, 0 };
-    int wsum[OCT];
+        for (int r = 0; r < 16; r++)
+            acc[i][r] = 0;
+    int wsum = 0;
     int asum[PXT];
-#pragma unroll
-    for (int t = 0; t < OCT; t++)
-        wsum[t] = 0;
 #pragma unroll
     for (int i = 0; i < PXT; i++)
         asum[i] = 0;
 
-    const int ch_shift = a.CH == 4 ? 2 : (a.CH == 2 ? 1 : 0);
-    const int n_pairs  = taps * a.CH;
-    const bool wave_active = wave * PXT * 16 < P;
+    const bool wave_active = wpx * PXT * 32 < P;
 
     for (int icb = 0; icb < a.n_icb; icb++)
     {
         const int ic_off = icb * blk_bytes;
         if (icb)
             __syncthreads();
-        // ---- stage weights [tap][row][CH chunks] and the input patch [py][px][CH chunks] ------------------
-        // Loads are issued in batches of STAGE_U per lane before any of them is written to LDS, so that
-        // the HBM/L2 latency is paid once per batch rather than once per chunk.
-#ifndef TMI_X_NO_STAGE
+        // ---- stage the weight rows and the input patch ---------------------------------------------------
+        // Nothing hides memory latency here except the loads themselves: every round issues up to WU weight
+        // chunks and PU patch chunks per lane before any of them is written to LDS, so a round costs one trip
+        // to HBM/L2.  The 3x3 / 64-channel shape needs a single round.  In the VEC instantiation (channel
+        // vectors are whole, aligned 16-byte chunks) the loads are unconditional: out-of-range work items read
+        // a clamped, valid address and the result is replaced afterwards, which keeps the round free of
+        // branches so that its loads really are in flight together.
         {
-            const int w_total = OCB * taps * a.CH;
+            const int w_total = OCB * n_pairs;
             const int p_total = a.PH * a.PW * a.CH;
-            for (int base = tid; base < w_total; base += 256 * STAGE_U)
+            for (int wbase = tid, pbase_idx = tid; wbase < w_total || pbase_idx < p_total;
+                 wbase += NT * WU, pbase_idx += NT * PU)
             {
-                v4i v[STAGE_U];
-                int dst[STAGE_U];
+                v4i wv[WU], pv[PU];
+                int wdst[WU], pdst[PU];
 #pragma unroll
-                for (int u = 0; u < STAGE_U; u++)
+                for (int u = 0; u < PU; u++)
                 {
-                    const int idx = base + u * 256;
-                    v[u]          = v4i{ 0, 0, 0, 0 };
-                    dst[u]        = -1;
-                    if (idx < w_total)
+                    const int idx  = pbase_idx + u * NT;
+                    const bool ok  = idx < p_total;
+                    const int idc  = ok ? idx : 0;
+                    const int cc   = idc & (a.CH - 1);
+                    const int pix  = idc >> ch_shift;
+                    const int py   = fdiv(pix, a.div_pw);
+                    const int px   = pix - py * a.PW;
+                    const int iy = y0 + py, ix = x0 + px;
+                    const int off  = ic_off + cc * 16;
+                    const bool img = iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW;
+                    pdst[u]        = ok ? pix * a.pstride + cc * 16 : -1;
+                    if constexpr (VEC)
                     {
-                        const int cc  = idx & (a.CH - 1);
-                        const int r2  = idx >> ch_shift;
-                        const int ocl = r2 / taps;
-                        const int tap = r2 - ocl * taps;
-                        if (oc0 + ocl < g.OC)
-                            v[u] = load_chunk(a.w + ((size_t)(oc0 + ocl) * taps + tap) * row_bytes, ic_off + cc * 16,
-                                              row_bytes, vec_ok);
-                        const int grp = ocl / (4 * OCT), rem = ocl % (4 * OCT);
-                        const int row = (rem >> 2) * 16 + grp * 4 + (rem & 3);
-                        dst[u]        = (tap * OCB + row) * a.wstride + cc * 16;
+                        const bool ld    = img && off < row_bytes;
+                        const size_t src = ld ? (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes + off : 0;
+                        const v4i v      = *reinterpret_cast<const v4i*>(a.in + src);
+                        const v4i f      = fill_chunk(off, row_bytes, M::is_int ? a.za : 0);
+                        pv[u]            = ld ? v : (img ? v4i{ 0, 0, 0, 0 } : f);
+                    }
+                    else
+                    {
+                        pv[u] = v4i{ 0, 0, 0, 0 };
+                        if (ok)
+                            pv[u] = img ? load_chunk_bytes(a.in + (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes,
+                                                           off, row_bytes)
+                                        : fill_chunk(off, row_bytes, M::is_int ? a.za : 0);
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < STAGE_U; u++)
-                    if (dst[u] >= 0)
-                        *reinterpret_cast<v4i*>(wl + dst[u]) = v[u];
-            }
-            for (int base = tid; base < p_total; base += 256 * STAGE_U)
-            {
-                v4i v[STAGE_U];
-                int dst[STAGE_U];
-#pragma unroll
-                for (int u = 0; u < STAGE_U; u++)
+                for (int u = 0; u < WU; u++)
                 {
-                    const int idx = base + u * 256;
-                    v[u]          = v4i{ 0, 0, 0, 0 };
-                    dst[u]        = -1;
-                    if (idx < p_total)
+                    const int idx = wbase + u * NT;
+                    const bool ok = idx < w_total;
+                    const int idc = ok ? idx : 0;
+                    const int ocl = fdiv(idc, a.div_rch);
+                    const int j   = idc - ocl * n_pairs;    // (tap, chunk) pair inside the row
+                    const int off = ic_off + (j & (a.CH - 1)) * 16;
+                    const bool ld = oc0 + ocl < g.OC && off < row_bytes;
+                    // output channel -> row of the MFMA operand (see the header comment)
+                    const int r32 = ocl & 31;
+                    const int row = (ocl & ~31) + ((r32 >> 2) & 3) * 8 + (r32 >> 4) * 4 + (r32 & 3);
+                    wdst[u]       = ok ? row * a.wstride + j * 16 : -1;
+                    if constexpr (VEC)
                     {
-                        const int cc  = idx & (a.CH - 1);
-                        const int pix = idx >> ch_shift;
-                        const int py  = pix / a.PW;
-                        const int px  = pix - py * a.PW;
-                        const int iy = y0 + py, ix = x0 + px;
-                        if (iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW)
-                            v[u] = load_chunk(a.in + (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes,
-                                              ic_off + cc * 16, row_bytes, vec_ok);
-                        else
-                            v[u] = fill_chunk(ic_off + cc * 16, row_bytes, M::is_int ? a.za : 0);
-                        dst[u] = pix * a.pstride + cc * 16;
+                        const size_t src = ld ? ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes + off : 0;
+                        const v4i v      = *reinterpret_cast<const v4i*>(a.w + src);
+                        wv[u]            = ld ? v : v4i{ 0, 0, 0, 0 };
+                    }
+                    else
+                    {
+                        wv[u] = v4i{ 0, 0, 0, 0 };
+                        if (ok && ld)
+                            wv[u] = load_chunk_bytes(a.w + ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes,
+                                                     off, row_bytes);
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < STAGE_U; u++)
-                    if (dst[u] >= 0)
-                        *reinterpret_cast<v4i*>(pl + dst[u]) = v[u];
+                for (int u = 0; u < PU; u++)
+                    if (pdst[u] >= 0)
+                        *reinterpret_cast<v4i*>(pl + pdst[u]) = pv[u];
+#pragma unroll
+                for (int u = 0; u < WU; u++)
+                    if (wdst[u] >= 0)
+                        *reinterpret_cast<v4i*>(wl + wdst[u]) = wv[u];
             }
         }
-#endif
         __syncthreads();
 
         // ---- MFMA over the (tap, chunk) pairs of this channel block -----------------------------------
-#ifndef TMI_X_NO_MFMA
         if (wave_active)
-#else
-        if (wave_active && a.ksteps > 1000)
-#endif
         {
-            for (int s = 0; s < a.ksteps; s++)
-            {
-                const int q     = 4 * s + lg;
+            const uint8_t* wrow = wl + (woc * 32 + li) * a.wstride;
+            // requests the fragments of K-step s; `po` is the pair's patch offset read from the table earlier
+            auto issue = [&](int s, int po, v4i& fa, v4i(&fb)[PXT]) {
+                const int q     = 2 * s + lh;
                 const bool live = q < n_pairs;
-                const int tap   = live ? (q >> ch_shift) : 0;
-                const int cc    = q & (a.CH - 1);
-                v4i af[OCT], bf[PXT];
-                const uint8_t* wp = wl + (size_t)(tap * OCB + li) * a.wstride + cc * 16;
-#pragma unroll
-                for (int t = 0; t < OCT; t++)
-                    af[t] = live ? *reinterpret_cast<const v4i*>(wp + t * 16 * a.wstride) : v4i{ 0, 0, 0, 0 };
-                const int to = tapoff[tap] + cc * 16;
+                fa              = *reinterpret_cast<const v4i*>(live ? wrow + q * 16 : zero_chunk);
 #pragma unroll
                 for (int i = 0; i < PXT; i++)
-                    bf[i] = live ? *reinterpret_cast<const v4i*>(pl + pbase[i] + to) : v4i{ 0, 0, 0, 0 };
+                    fb[i] = *reinterpret_cast<const v4i*>(live ? pl + pbase[i] + po : zero_chunk);
+            };
+            auto compute = [&](const v4i& fa, const v4i(&fb)[PXT]) {
 #pragma unroll
                 for (int i = 0; i < PXT; i++)
-#pragma unroll
-                    for (int t = 0; t < OCT; t++)
-                        acc[i][t] = M::mma(af[t], bf[i], acc[i][t]);
+                    acc[i] = M::mma(fa, fb[i], acc[i]);
                 if constexpr (M::is_int)
                 {
                     if (a.za != 0)
-#pragma unroll
-                        for (int t = 0; t < OCT; t++)
-                            wsum[t] += dot4_ones(af[t]);
+                        wsum += dot4_ones(fa);
                     if (a.zw != 0)
 #pragma unroll
                         for (int i = 0; i < PXT; i++)
-                            asum[i] += dot4_ones(bf[i]);
+                            asum[i] += dot4_ones(fb[i]);
+                }
+            };
+            const int* tab = pairoff + lh;
+            int po0 = tab[0], po1 = tab[2], po2 = tab[4];
+            v4i fa0, fa1, fa2, fb0[PXT], fb1[PXT], fb2[PXT];
+            issue(0, po0, fa0, fb0);
+            po0 = tab[6];
+            issue(1, po1, fa1, fb1);
+            po1 = tab[8];
+            for (int s = 0; s < a.ksteps; s += 3)
+            {
+                issue(s + 2, po2, fa2, fb2);
+                po2 = tab[2 * (s + 5)];
+                compute(fa0, fb0);
+                if (s + 1 < a.ksteps)
+                {
+                    issue(s + 3, po0, fa0, fb0);
+                    po0 = tab[2 * (s + 6)];
+                    compute(fa1, fb1);
+                }
+                if (s + 2 < a.ksteps)
+                {
+                    issue(s + 4, po1, fa1, fb1);
+                    po1 = tab[2 * (s + 7)];
+                    compute(fa2, fb2);
                 }
             }
         }
     }
 
-    if (!wave_active)
-        return;
-#ifdef TMI_X_NO_EPILOGUE_AT_ALL
-    if (a.ksteps < 1000) { if (acc[0][0][0] == 0x12345678) a.flag_word[1] = 1; return; }
-#endif
-
     // ---- epilogue -------------------------------------------------------------------------------------
-    uint32_t flags = 0;
-    const int ocl0 = 4 * OCT * lg;    // first of this lane's 4*OCT consecutive channels inside the block
-    if constexpr (M::is_int)
-    {
-        // finish the K-chunk reduction of the side sums (lanes li, li+16, li+32, li+48 hold partials)
-        int corr[OCT][4];
-        if (a.za != 0)
-        {
+    // per pixel tile: validity and output offset of this lane's pixel; the lane owns channels
+    // [ocl0, ocl0 + 16) of the block
+    bool pix_ok[PXT];
+    size_t obase[PXT];
+    const int ocl0 = woc * 32 + 16 * lh;
 #pragma unroll
-            for (int t = 0; t < OCT; t++)
+    for (int i = 0; i < PXT; i++)
+    {
+        const int p  = (wpx * PXT + i) * 32 + li;
+        const int ty = fdiv(p, a.div_tw);
+        const int oy = oy0 + ty, ox = ox0 + (p - ty * a.TW);
+        pix_ok[i]    = wave_active && p < P && oy < g.OH && ox < g.OW;
+        obase[i]     = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
+    }
+    const bool full = (oc0 + ocl0 + 16 <= g.OC);
+
+    if constexpr (!M::is_int)
+    {
+        // floating point: out = bias + acc, rounded to the output type; 16 channels = 32 bytes per pixel
+        const bool vec_out = full && (g.OC & 7) == 0 && ((uintptr_t)a.out & 15) == 0;
+#pragma unroll
+        for (int i = 0; i < PXT; i++)
+        {
+            union
             {
-                int v = wsum[t];
-                v += __shfl_xor(v, 16);
-                v += __shfl_xor(v, 32);
-                // D row 4*lg + r of tile t is weight row (A fragment lane) 4*lg + r
+                v4i v[2];
+                T e[16];
+            } u;
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+            {
+                const v4f b = *reinterpret_cast<const v4f*>(ftab + ocl0 + 4 * q);
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                    corr[t][r] = __shfl(v, 4 * lg + r) * a.za;
+                    store_from_float(&u.e[4 * q + r], b[r] + acc[i][4 * q + r]);
+            }
+            if (!pix_ok[i])
+                continue;
+            T* o = reinterpret_cast<T*>(a.out) + obase[i];
+            if (vec_out)
+            {
+                reinterpret_cast<v4i*>(o)[0] = u.v[0];
+                reinterpret_cast<v4i*>(o)[1] = u.v[1];
+            }
+            else
+            {
+#pragma unroll
+                for (int j = 0; j < 16; j++)
+                    if (oc0 + ocl0 + j < g.OC)
+                        o[j] = u.e[j];
             }
         }
-        else
-        {
-#pragma unroll
-            for (int t = 0; t < OCT; t++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    corr[t][r] = 0;
-        }
+    }
+    else
+    {
         const int kzz = g.KH * g.KW * g.IC * a.za * a.zw;
-        // per pixel group: validity, output offset and the zero-point term that depends on the pixel
-        bool pix_ok[PXT];
-        size_t obase[PXT];
-        int pcorr[PXT];
+        int pcorr[PXT];    // the zero-point terms that depend on the pixel only
 #pragma unroll
         for (int i = 0; i < PXT; i++)
         {
             int sa = asum[i];
             if (a.zw != 0)
-            {
-                sa += __shfl_xor(sa, 16);
                 sa += __shfl_xor(sa, 32);
-            }
-            pcorr[i]     = kzz - a.zw * sa;
-            const int p  = (wave * PXT + i) * 16 + li;
-            const int ty = p / a.TW, tx = p - ty * a.TW;
-            const int oy = oy0 + ty, ox = ox0 + tx;
-            pix_ok[i]    = p < P && oy < g.OH && ox < g.OW;
-            obase[i]     = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
+            pcorr[i] = kzz - a.zw * sa;
         }
-        const bool full    = (oc0 + ocl0 + 4 * OCT <= g.OC);
-        const bool vec_out = full && (g.OC % (4 * OCT)) == 0 && ((uintptr_t)a.out & 15) == 0;
-        // bias / multiplier / shift / int32 output rows of four channels can be moved as one vector
-        const bool vec_par = full && (g.OC & 3) == 0 && (oc0 + ocl0) % 4 == 0 &&
-                             (((uintptr_t)a.bias | (uintptr_t)a.out | (a.rp.enabled ? (uintptr_t)a.rp.multiplier : 0)) & 15) == 0 &&
-                             (!a.rp.enabled || ((uintptr_t)a.rp.shift & 3) == 0);
-        int packed[PXT][OCT];    // int8 results, four channels per word
+        // finish the K-half reduction of sum(w): afterwards lane i (either half) holds za * the total of
+        // operand row i of the wave's channel tile
+        if (a.za != 0)
+            wsum = (wsum + __shfl_xor(wsum, 32)) * a.za;
+        // int32 rows of four channels can be stored as one vector; int8 rows of 16 channels likewise
+        const bool vec4  = full && (g.OC & 3) == 0 && ((uintptr_t)a.out & 15) == 0;
+        const bool vec16 = full && (g.OC & 15) == 0 && ((uintptr_t)a.out & 15) == 0;
+        int packed[PXT][4];    // int8 results, four channels per word
 
-        // channel tile by channel tile: fetch the four channels' constants once, use them for every pixel
+        if constexpr (EPI == EPI_GENERIC)
+            __syncthreads();    // every wave is done reading the operands: LDS becomes the staging area
+        int32_t* stage = reinterpret_cast<int32_t*>(lds + kCtab);    // [pixel of the tile][channel of the block]
+
+        // four channels at a time: fetch their constants once, use them for every pixel of the lane
 #pragma unroll
-        for (int t = 0; t < OCT; t++)
+        for (int q = 0; q < 4; q++)
         {
-            const int c0 = oc0 + ocl0 + 4 * t;
-            int32_t bias4[4], mult4[4], shift4[4];
+            const int c0 = oc0 + ocl0 + 4 * q;
+            ChanEntry ce[4];
+            int32_t cb[4];    // bias minus the weight-sum term of the zero-point correction
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                bias4[r] = mult4[r] = 0, shift4[r] = 32;    // neutral: every value legal, result 0
-            if (g.bias_len == 1)
             {
-                const int32_t b = reinterpret_cast<const int32_t*>(a.bias)[0];
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    bias4[r] = b;
-            }
-            else if (vec_par)
-            {
-                const v4i b = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(a.bias) + c0);
-                bias4[0] = b.x, bias4[1] = b.y, bias4[2] = b.z, bias4[3] = b.w;
-            }
-            else
-            {
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (c0 + r < g.OC)
-                        bias4[r] = reinterpret_cast<const int32_t*>(a.bias)[c0 + r];
-            }
-            ChannelScale cs[4];
-            if (a.rp.enabled)
-            {
-                if (vec_par && a.rp.per_channel && a.rp.scale32)
-                {
-                    const v4i m = *reinterpret_cast<const v4i*>(reinterpret_cast<const int32_t*>(a.rp.multiplier) + c0);
-                    const int sh = *reinterpret_cast<const int*>(a.rp.shift + c0);
-                    mult4[0] = m.x, mult4[1] = m.y, mult4[2] = m.z, mult4[3] = m.w;
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        shift4[r] = (int32_t)(int8_t)(sh >> (8 * r));
-                }
-                else
-                {
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        if (c0 + r < g.OC)
-                            mult4[r] = load_multiplier(a.rp, c0 + r), shift4[r] = load_shift(a.rp, c0 + r);
-                }
-                if (a.rp.fast)
-                {
-                    // channels past OC carry the neutral constants (0, 32) set above and raise nothing
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        cs[r] = make_channel_scale(mult4[r], shift4[r], a.rp.double_round, flags);
-                }
+                ce[r] = ctab[ocl0 + 4 * q + r];
+                cb[r] = ce[r].bias - (a.za != 0 ? __shfl(wsum, 8 * q + 4 * lh + r) : 0);
             }
 #pragma unroll
             for (int i = 0; i < PXT; i++)
@@ -475,28 +581,32 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                 {
-                    int32_t v = acc[i][t][r] + pcorr[i] - corr[t][r] + bias4[r];
-#ifndef TMI_X_NO_EPI
-                    if (a.rp.enabled)
+                    int32_t v = acc[i][4 * q + r] + pcorr[i] + cb[r];
+                    if constexpr (EPI == EPI_FAST)
                     {
-                        if (a.rp.fast)
-                        {
-                            uint32_t f = 0;
-                            v          = fast_rescale(v, cs[r], a.rp.out_zp, a.rp.lo, a.rp.hi, f);
-                            flags |= pix_ok[i] ? f : 0u;    // pixels outside the image must not raise anything
-                        }
-                        else if (pix_ok[i] && c0 + r < g.OC)
-                            v = rescale_value(a.rp, v, mult4[r], shift4[r], flags);
+                        if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
+                            flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
+                        const int64_t pr = (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
+                        v                = (int32_t)(pr >> ce[r].s) + a.rp.out_zp;
+                        v                = v < a.rp.lo ? a.rp.lo : v;
+                        v                = v > a.rp.hi ? a.rp.hi : v;
                     }
-#endif
                     res[r] = v;
+                }
+                if constexpr (EPI == EPI_GENERIC)
+                {
+                    const int p = (wpx * PXT + i) * 32 + li;
+                    if (wave_active && p < P)
+                        *reinterpret_cast<v4i*>(stage + (size_t)p * OCB + ocl0 + 4 * q) =
+                            v4i{ res[0], res[1], res[2], res[3] };
+                    continue;
                 }
                 if (!pix_ok[i])
                     continue;
-                if (a.out_dtype == TMI_INT32)
+                if (EPI == EPI_PLAIN || a.out_dtype == TMI_INT32)
                 {
-                    int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase[i] + 4 * t;
-                    if (vec_par)
+                    int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase[i] + 4 * q;
+                    if (vec4)
                         *reinterpret_cast<v4i*>(o) = v4i{ res[0], res[1], res[2], res[3] };
                     else
 #pragma unroll
@@ -506,12 +616,12 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
                 }
                 else if (a.out_dtype == TMI_INT8)
                 {
-                    if (vec_out)
-                        packed[i][t] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
+                    if (vec16)
+                        packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
                                        ((res[3] & 0xff) << 24);
                     else
                     {
-                        int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i] + 4 * t;
+                        int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i] + 4 * q;
 #pragma unroll
                         for (int r = 0; r < 4; r++)
                             if (c0 + r < g.OC)
@@ -520,7 +630,7 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
                 }
                 else
                 {
-                    int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase[i] + 4 * t;
+                    int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase[i] + 4 * q;
 #pragma unroll
                     for (int r = 0; r < 4; r++)
                         if (c0 + r < g.OC)
@@ -528,55 +638,45 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
                 }
             }
         }
-        if (a.out_dtype == TMI_INT8 && vec_out)
+        if constexpr (EPI == EPI_FAST)
         {
-#pragma unroll
-            for (int i = 0; i < PXT; i++)
+            if (a.out_dtype == TMI_INT8 && vec16)
             {
-                if (!pix_ok[i])
-                    continue;
-                int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i];
-                if constexpr (OCT == 4)
-                    *reinterpret_cast<v4i*>(o) = v4i{ packed[i][0], packed[i][1], packed[i][2], packed[i][3] };
-                else
 #pragma unroll
-                    for (int t = 0; t < OCT; t++)
-                        reinterpret_cast<int*>(o)[t] = packed[i][t];
+                for (int i = 0; i < PXT; i++)
+                    if (pix_ok[i])
+                        *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + obase[i]) =
+                            v4i{ packed[i][0], packed[i][1], packed[i][2], packed[i][3] };
+            }
+        }
+        if constexpr (EPI == EPI_GENERIC)
+        {
+            // the general RESCALE (16-bit scale, inexact rounding, split clip/clamp ranges, ...): every lane
+            // takes elements of the staged int32 tile in turn
+            __syncthreads();
+            const int total = P * OCB;
+#pragma nounroll
+            for (int idx = tid; idx < total; idx += NT)
+            {
+                const int p   = idx / OCB;
+                const int ocl = idx % OCB;
+                const int oc  = oc0 + ocl;
+                const int ty  = fdiv(p, a.div_tw);
+                const int oy = oy0 + ty, ox = ox0 + (p - ty * a.TW);
+                if (oc >= g.OC || oy >= g.OH || ox >= g.OW)
+                    continue;
+                const int32_t r =
+                    rescale_value(a.rp, stage[idx], load_multiplier(a.rp, oc), load_shift(a.rp, oc), flags);
+                const size_t o = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc;
+                if (a.out_dtype == TMI_INT8)
+                    reinterpret_cast<int8_t*>(a.out)[o] = (int8_t)r;
+                else if (a.out_dtype == TMI_INT16)
+                    reinterpret_cast<int16_t*>(a.out)[o] = (int16_t)r;
+                else
+                    reinterpret_cast<int32_t*>(a.out)[o] = r;
             }
         }
         raise_flags(a.flag_word, flags);
-    }
-    else
-    {
-#pragma unroll
-        for (int i = 0; i < PXT; i++)
-        {
-            const int p = (wave * PXT + i) * 16 + li;
-            const int ty = p / a.TW, tx = p - ty * a.TW;
-            const int oy = oy0 + ty, ox = ox0 + tx;
-            if (!(p < P && oy < g.OH && ox < g.OW))
-                continue;
-            const size_t obase = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
-            T* o               = reinterpret_cast<T*>(a.out) + obase;
-            const T* bias      = reinterpret_cast<const T*>(a.bias);
-#pragma unroll
-            for (int t = 0; t < OCT; t++)
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                {
-                    const int j  = 4 * t + r;
-                    const int oc = oc0 + ocl0 + j;
-                    if (oc < g.OC)
-                    {
-                        float b;
-                        if constexpr (sizeof(T) == 2 && !__is_same(T, bf16_t))
-                            b = (float)bias[g.bias_len == 1 ? 0 : oc];
-                        else
-                            b = bf16_to_float(reinterpret_cast<const bf16_t*>(a.bias)[g.bias_len == 1 ? 0 : oc]);
-                        o[j] = to_out<T>(b + acc[i][t][r]);
-                    }
-                }
-        }
     }
 }
 
@@ -584,10 +684,10 @@ __global__ __launch_bounds__(256) void conv2d_patch_kernel(PatchArgs a)
 
 static constexpr int kMaxLds = 160 * 1024;
 
-template <typename T, int OCT, int PXT>
+template <typename T, int WOC, int PXT, int EPI, bool VEC>
 static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blocks)
 {
-    auto kern = conv2d_patch_kernel<T, OCT, PXT>;
+    auto kern                = conv2d_patch_kernel<T, WOC, PXT, EPI, VEC>;
     static size_t configured = 0;    // largest dynamic LDS size this instantiation was configured for
     if (lds_bytes > configured)
     {
@@ -596,7 +696,7 @@ static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blo
             return false;
         configured = lds_bytes;
     }
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds_bytes, st, a);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
     return true;
 }
 
@@ -605,42 +705,48 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
                                         const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                         const RescaleParams& rp, void* out, uint32_t* flag_word, const char* label)
 {
-    constexpr int EB  = sizeof(T);
-    constexpr int PXT = 2;
+    constexpr int EB    = sizeof(T);
     const int row_bytes = g.IC * EB;
-    if (row_bytes <= 0 || g.OC <= 0 || (int64_t)g.N * g.OH * g.OW == 0)
+    const int64_t n_px  = (int64_t)g.N * g.OH * g.OW;
+    if (row_bytes <= 0 || g.OC <= 0 || n_px == 0)
         return nullptr;
 
     PatchArgs a{};
     a.g = g, a.in = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = bias, a.out = out;
     a.flag_word = flag_word, a.rp = rp, a.za = in_zp, a.zw = w_zp, a.out_dtype = out_dtype;
-    a.CH      = row_bytes <= 16 ? 1 : (row_bytes <= 32 ? 2 : 4);
-    a.pstride = a.CH == 1 ? 16 : a.CH * 16 + 16;
-    a.wstride = a.pstride;
-    a.n_icb   = (row_bytes + a.CH * 16 - 1) / (a.CH * 16);
+    a.CH           = row_bytes <= 16 ? 1 : (row_bytes <= 32 ? 2 : 4);
+    a.pstride      = a.CH == 1 ? 16 : a.CH * 16 + 16;    // 16, 48, 80: all = 16 (mod 32)
+    a.n_icb        = (row_bytes + a.CH * 16 - 1) / (a.CH * 16);
     const int taps = g.KH * g.KW;
-    a.ksteps  = (taps * a.CH + 3) / 4;
+    const int rch  = taps * a.CH;    // chunks per weight row
+    a.wstride      = rch * 16 + ((rch & 1) ? 0 : 16);
+    a.ksteps       = (rch + 1) / 2;
 
-    const int OCT = g.OC > 32 ? 4 : (g.OC > 16 ? 2 : 1);
-    const int OCB = 16 * OCT;
-    a.oc_blocks   = (g.OC + OCB - 1) / OCB;
+    const int WOC           = g.OC > 32 ? 2 : 1;
+    const int OCB           = 32 * WOC;
+    const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
 
-    // tile: up to 4 waves x PXT groups x 16 pixels; prefer full output rows
-    const int max_px = 4 * PXT * 16;
+    // channel vectors made of whole, aligned 16-byte chunks take the branch-free staging path
+    const bool vec = (row_bytes & 15) == 0 && (((uintptr_t)in | (uintptr_t)w) & 15) == 0;
+    // Pixel tiles per wave: two when that still leaves at least two workgroups per CU, else one.
+    const int max_px1 = 32 * (8 / WOC);
+    const int PXT     = (vec && n_px * oc_blocks >= (int64_t)256 * 2 * 2 * max_px1) ? 2 : 1;
+    const int max_px  = max_px1 * PXT;
+    // tile: prefer full output rows
     int TW = g.OW < max_px ? g.OW : max_px;
     int TH = max_px / TW;
     if (TH > g.OH)
         TH = g.OH;
     if (TH < 1)
         TH = 1;
-    const size_t tab_bytes = ((size_t)taps * 4 + 15) & ~(size_t)15;
-    const size_t w_bytes   = (size_t)taps * OCB * a.wstride;
-    size_t lds_bytes       = 0;
+    const size_t fixed_bytes = (size_t)OCB * 32 + 16 + ((((size_t)rch + 12) * 4 + 15) & ~(size_t)15);
+    const size_t w_bytes     = (size_t)OCB * a.wstride;
+    size_t lds_bytes         = 0;
     for (;;)
     {
         a.PH      = (TH - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
         a.PW      = (TW - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
-        lds_bytes = tab_bytes + w_bytes + (size_t)a.PH * a.PW * a.pstride;
+        lds_bytes = fixed_bytes + w_bytes + (size_t)a.PH * a.PW * a.pstride;
         if (lds_bytes <= (size_t)kMaxLds)
             break;
         if (TH > 1)
@@ -654,25 +760,74 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     a.tiles_y = (g.OH + TH - 1) / TH;
     a.tiles_x = (g.OW + TW - 1) / TW;
     const int64_t n_tiles = (int64_t)g.N * a.tiles_y * a.tiles_x;
-    const int64_t blocks  = n_tiles * a.oc_blocks;
-    if (blocks > 0x7fffffff)
+    const int64_t blocks  = n_tiles * oc_blocks;
+    if (blocks > 0x3fffffff || (int64_t)a.PH * a.PW * a.CH > (1 << 20))
         return nullptr;
-    a.n_tiles   = (int)n_tiles;
-    a.xcd_remap = (blocks % 8) == 0 && blocks >= 16;
+    a.n_tiles     = (int)n_tiles;
+    a.xcd_remap   = (blocks % 8) == 0 && blocks >= 16;
+    a.div_tw      = make_fastdiv(TW);
+    a.div_pw      = make_fastdiv(a.PW);
+    a.div_rch     = make_fastdiv(rch);
+    a.div_tiles_x = make_fastdiv(a.tiles_x);
+    a.div_tiles_y = make_fastdiv(a.tiles_y);
+    a.div_n_tiles = make_fastdiv(a.n_tiles);
+    a.div_kw      = make_fastdiv(g.KW);
+    // fdiv is exact for n*d < 2^32: every dividend but the block index is bounded by the LDS capacity;
+    // guard the products that involve the block index
+    if ((uint64_t)blocks * (uint64_t)a.n_tiles >= (uint64_t(1) << 32) ||
+        (uint64_t)n_tiles * (uint64_t)a.tiles_x >= (uint64_t(1) << 32) ||
+        (uint64_t)(n_tiles / a.tiles_x + 1) * (uint64_t)a.tiles_y >= (uint64_t(1) << 32))
+        return nullptr;
 
-    bool ok = false;
-    switch (OCT)
+    const int epi = !rp.enabled ? EPI_PLAIN : (rp.fast ? EPI_FAST : EPI_GENERIC);
+    if (epi == EPI_GENERIC)
     {
-        case 4:
-            ok = launch_patch<T, 4, PXT>(st, a, lds_bytes, (int)blocks);
-            break;
-        case 2:
-            ok = launch_patch<T, 2, PXT>(st, a, lds_bytes, (int)blocks);
-            break;
-        default:
-            ok = launch_patch<T, 1, PXT>(st, a, lds_bytes, (int)blocks);
-            break;
+        // the int32 tile is staged in LDS (behind the channel table) before the general RESCALE
+        const size_t stage_bytes = (size_t)OCB * 32 + (size_t)TH * TW * OCB * 4;
+        if (stage_bytes > lds_bytes)
+            lds_bytes = stage_bytes;
+        if (lds_bytes > (size_t)kMaxLds)
+            return nullptr;
     }
+    bool ok = false;
+#define TMI_PATCH_CASE(O, P, E)                                                                                      \
+    if (WOC == O && PXT == P && epi == E)                                                                            \
+        ok = launch_patch<T, O, P, E, true>(st, a, lds_bytes, (int)blocks);
+#define TMI_PATCH_CASE_BYTES(O, E)                                                                                   \
+    if (WOC == O && epi == E)                                                                                        \
+        ok = launch_patch<T, O, 1, E, false>(st, a, lds_bytes, (int)blocks);
+    if (vec)
+    {
+        TMI_PATCH_CASE(1, 1, EPI_PLAIN)
+        TMI_PATCH_CASE(1, 2, EPI_PLAIN)
+        TMI_PATCH_CASE(2, 1, EPI_PLAIN)
+        TMI_PATCH_CASE(2, 2, EPI_PLAIN)
+        if constexpr (Mma<T>::is_int)
+        {
+            TMI_PATCH_CASE(1, 1, EPI_FAST)
+            TMI_PATCH_CASE(1, 2, EPI_FAST)
+            TMI_PATCH_CASE(2, 1, EPI_FAST)
+            TMI_PATCH_CASE(2, 2, EPI_FAST)
+            TMI_PATCH_CASE(1, 1, EPI_GENERIC)
+            TMI_PATCH_CASE(1, 2, EPI_GENERIC)
+            TMI_PATCH_CASE(2, 1, EPI_GENERIC)
+            TMI_PATCH_CASE(2, 2, EPI_GENERIC)
+        }
+    }
+    else
+    {
+        TMI_PATCH_CASE_BYTES(1, EPI_PLAIN)
+        TMI_PATCH_CASE_BYTES(2, EPI_PLAIN)
+        if constexpr (Mma<T>::is_int)
+        {
+            TMI_PATCH_CASE_BYTES(1, EPI_FAST)
+            TMI_PATCH_CASE_BYTES(2, EPI_FAST)
+            TMI_PATCH_CASE_BYTES(1, EPI_GENERIC)
+            TMI_PATCH_CASE_BYTES(2, EPI_GENERIC)
+        }
+    }
+#undef TMI_PATCH_CASE_BYTES
+#undef TMI_PATCH_CASE
     return ok ? label : nullptr;
 }
 
