@@ -86,6 +86,7 @@ struct PatchArgs
     int32_t n_tiles;             // N * tiles_y * tiles_x
     int32_t out_dtype;
     int32_t xcd_remap;
+    int64_t w_batch_stride;    // bytes between the weights of consecutive images (0: shared; MATMUL: per batch)
     FastDiv div_tw, div_pw, div_rch, div_tiles_x, div_tiles_y, div_n_tiles, div_kw;
 };
 
@@ -270,6 +271,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const int y0        = oy0 * g.stride_y - g.pad_top;
     const int x0        = ox0 * g.stride_x - g.pad_left;
     const int P         = a.TH * a.TW;
+    const uint8_t* wbase_ptr = a.w + (size_t)n * a.w_batch_stride;
 
     // ---- tables ----------------------------------------------------------------------------------------
     uint32_t flags = 0;
@@ -404,14 +406,14 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                     if constexpr (VEC)
                     {
                         const size_t src = ld ? ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes + off : 0;
-                        const v4i v      = *reinterpret_cast<const v4i*>(a.w + src);
+                        const v4i v      = *reinterpret_cast<const v4i*>(wbase_ptr + src);
                         wv[u]            = ld ? v : v4i{ 0, 0, 0, 0 };
                     }
                     else
                     {
                         wv[u] = v4i{ 0, 0, 0, 0 };
                         if (ok && ld)
-                            wv[u] = load_chunk_bytes(a.w + ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes,
+                            wv[u] = load_chunk_bytes(wbase_ptr + ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes,
                                                      off, row_bytes);
                     }
                 }
@@ -501,11 +503,35 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 
     if constexpr (!M::is_int)
     {
-        // floating point: out = bias + acc, rounded to the output type; 16 channels = 32 bytes per pixel
+        // floating point: out = bias + acc, rounded to the output type (16 channels = 32 bytes per pixel), or
+        // kept in fp32 (MATMUL: 64 bytes per pixel)
         const bool vec_out = full && (g.OC & 7) == 0 && ((uintptr_t)a.out & 15) == 0;
 #pragma unroll
         for (int i = 0; i < PXT; i++)
         {
+            if (a.out_dtype == TMI_FP32)
+            {
+                float* o = reinterpret_cast<float*>(a.out) + obase[i];
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                {
+                    const v4f b = *reinterpret_cast<const v4f*>(ftab + ocl0 + 4 * q);
+                    v4f r;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        r[j] = b[j] + acc[i][4 * q + j];
+                    if (!pix_ok[i])
+                        continue;
+                    if (vec_out)
+                        *reinterpret_cast<v4f*>(o + 4 * q) = r;
+                    else
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            if (oc0 + ocl0 + 4 * q + j < g.OC)
+                                o[4 * q + j] = r[j];
+                }
+                continue;
+            }
             union
             {
                 v4i v[2];
@@ -703,7 +729,8 @@ static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blo
 template <typename T>
 static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32_t out_dtype, const void* in,
                                         const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
-                                        const RescaleParams& rp, void* out, uint32_t* flag_word, const char* label)
+                                        const RescaleParams& rp, void* out, uint32_t* flag_word, const char* label,
+                                        int64_t w_batch_stride)
 {
     constexpr int EB    = sizeof(T);
     const int row_bytes = g.IC * EB;
@@ -714,6 +741,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     PatchArgs a{};
     a.g = g, a.in = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = bias, a.out = out;
     a.flag_word = flag_word, a.rp = rp, a.za = in_zp, a.zw = w_zp, a.out_dtype = out_dtype;
+    a.w_batch_stride = w_batch_stride;
     a.CH           = row_bytes <= 16 ? 1 : (row_bytes <= 32 ? 2 : 4);
     a.pstride      = a.CH == 1 ? 16 : a.CH * 16 + 16;    // 16, 48, 80: all = 16 (mod 32)
     a.n_icb        = (row_bytes + a.CH * 16 - 1) / (a.CH * 16);
@@ -833,17 +861,17 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
 
 const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                               void* out, uint32_t* flag_word)
+                               void* out, uint32_t* flag_word, int64_t w_batch_stride)
 {
     if (in_dtype == TMI_INT8)
         return launch_conv2d_mfma_t<int8_t>(st, g, out_dtype, in, w, bias, in_zp, w_zp, rp, out, flag_word,
-                                            rp.enabled ? "conv2d_mfma_i8_rescale" : "conv2d_mfma_i8");
-    if (in_dtype == TMI_FP16 && out_dtype == TMI_FP16)
+                                            rp.enabled ? "conv2d_mfma_i8_rescale" : "conv2d_mfma_i8", w_batch_stride);
+    if (in_dtype == TMI_FP16 && (out_dtype == TMI_FP16 || out_dtype == TMI_FP32))
         return launch_conv2d_mfma_t<_Float16>(st, g, out_dtype, in, w, bias, 0, 0, rp, out, flag_word,
-                                              "conv2d_mfma_f16");
-    if (in_dtype == TMI_BF16 && out_dtype == TMI_BF16)
+                                              "conv2d_mfma_f16", w_batch_stride);
+    if (in_dtype == TMI_BF16 && (out_dtype == TMI_BF16 || out_dtype == TMI_FP32))
         return launch_conv2d_mfma_t<bf16_t>(st, g, out_dtype, in, w, bias, 0, 0, rp, out, flag_word,
-                                            "conv2d_mfma_bf16");
+                                            "conv2d_mfma_bf16", w_batch_stride);
     return nullptr;
 }
 

@@ -158,4 +158,41 @@ const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* ou
     return "clamp_vec";
 }
 
+// ------------------------------------------------------------------------------------------------
+// Batched transpose [N, R, C] -> [N, C, R] through a padded 64x64 LDS tile: rows are read and written as
+// contiguous runs along the fastest dimension of their side.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(int32_t R, int32_t C, const T* __restrict__ in,
+                                                        T* __restrict__ out)
+{
+    __shared__ T tile[64][64 + 4 / sizeof(T)];
+    const size_t base = (size_t)blockIdx.z * R * C;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4)
+        if (r0 + i < R && c0 + tx < C)
+            tile[i][tx] = in[base + (size_t)(r0 + i) * C + c0 + tx];
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4)
+        if (c0 + i < C && r0 + tx < R)
+            out[base + (size_t)(c0 + i) * R + r0 + tx] = tile[tx][i];
+}
+
+const char* launch_transpose(hipStream_t st, int32_t elem_bytes, int32_t N, int32_t R, int32_t C, const void* in,
+                             void* out)
+{
+    if ((int64_t)N * R * C == 0)
+        return "transpose_empty";
+    const dim3 grid((C + 63) / 64, (R + 63) / 64, N);
+    if (elem_bytes == 1)
+        hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, st, R, C, (const uint8_t*)in, (uint8_t*)out);
+    else if (elem_bytes == 2)
+        hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, st, R, C, (const uint16_t*)in,
+                           (uint16_t*)out);
+    else
+        return nullptr;
+    return "transpose";
+}
+
 }    // namespace tmi

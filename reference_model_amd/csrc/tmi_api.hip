@@ -15,6 +15,8 @@ struct tmi_ctx
     bool owns_stream      = false;
     uint32_t* flags_dev   = nullptr;    // latched REQUIRE conditions
     uint32_t* flags_host  = nullptr;    // pinned staging word
+    void* workspace       = nullptr;    // scratch for operand re-layout (MATMUL's transposed B)
+    size_t workspace_size = 0;
     uint32_t last_flags   = 0;
     int32_t kernel_choice = 0;
     std::string last_error;
@@ -59,6 +61,21 @@ int after_launch(tmi_ctx* ctx, const char* kernel_name)
     hipError_t e     = hipGetLastError();
     if (e != hipSuccess)
         return hip_fail(ctx, e, kernel_name);
+    return TMI_VALID;
+}
+
+// Grows the context's scratch buffer; the old one is released only after the stream has drained.
+int ensure_workspace(tmi_ctx* ctx, size_t bytes)
+{
+    if (bytes <= ctx->workspace_size)
+        return TMI_VALID;
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->workspace)
+        TMI_HIP(ctx, hipFree(ctx->workspace));
+    ctx->workspace      = nullptr;
+    ctx->workspace_size = 0;
+    TMI_HIP(ctx, hipMalloc(&ctx->workspace, bytes));
+    ctx->workspace_size = bytes;
     return TMI_VALID;
 }
 
@@ -350,6 +367,8 @@ int tmi_ctx_destroy(tmi_ctx_t* ctx)
     // teardown is best effort: there is nobody left to report a failure to
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->workspace)
+        (void)hipFree(ctx->workspace);
     if (ctx->flags_dev)
         (void)hipFree(ctx->flags_dev);
     if (ctx->flags_host)
@@ -537,9 +556,39 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
     if (total > 0 && (!out_dev || ((int64_t)C > 0 && (!a_dev || !b_dev))))
         return fail(ctx, "OpMatMul: null tensor pointer");
     TMI_HIP(ctx, hipSetDevice(ctx->device));
-    if (ctx->kernel_choice == 2)
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    const char* name = nullptr;
+    if (ctx->kernel_choice != 1 && C > 0)
+    {
+        // MFMA path: make B K-contiguous ([N,C,W] -> [N,W,C]) in the context's scratch buffer, then run the
+        // implicit-GEMM kernel with one "image" per batch: pixels = rows of A, output channels = columns of
+        // B, 1x1 taps, per-image weights.  The bias operand is the permanently zero word kept after the flags.
+        const int eb       = in_dtype == TMI_INT8 ? 1 : 2;
+        const size_t bytes = (size_t)N * C * W * eb;
+        int rc             = ensure_workspace(ctx, bytes);
+        if (rc != TMI_VALID)
+            return rc;
+        ConvGeom g{};
+        g.N = N, g.IH = H, g.IW = 1, g.IC = C, g.OC = W, g.KH = 1, g.KW = 1, g.OH = H, g.OW = 1;
+        g.stride_y = g.stride_x = g.dil_y = g.dil_x = 1;
+        g.bias_len = 1, g.M = 1;
+        RescaleParams none{};
+        if (!launch_transpose(ctx->stream, eb, N, C, W, b_dev, ctx->workspace))
+            return fail(ctx, "OpMatMul: transpose launch failed");
+        name = launch_conv2d_mfma(ctx->stream, in_dtype, in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32, g, a_dev,
+                                  ctx->workspace, ctx->flags_dev + 16, a_zp, b_zp, none, out_dev, ctx->flags_dev,
+                                  (int64_t)W * C * eb);
+        if (name)
+            name = in_dtype == TMI_INT8 ? "matmul_mfma_i8" : (in_dtype == TMI_FP16 ? "matmul_mfma_f16" : "matmul_mfma_bf16");
+    }
+    if (!name && ctx->kernel_choice == 2)
         return fail(ctx, "OpMatMul: no MFMA kernel is eligible for this shape");
-    const char* name = launch_matmul_direct(ctx->stream, in_dtype, N, H, C, W, a_dev, b_dev, a_zp, b_zp, out_dev);
+    if (!name)
+        name = launch_matmul_direct(ctx->stream, in_dtype, N, H, C, W, a_dev, b_dev, a_zp, b_zp, out_dev);
     return after_launch(ctx, name);
 }
 

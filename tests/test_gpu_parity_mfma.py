@@ -166,3 +166,56 @@ def test_mfma_not_eligible_is_an_error_when_forced(ctx):
     with pytest.raises(TmiError) as e:
         gpu_ops.conv2d(ctx, x, w, np.zeros(1, np.int32))
     assert "no MFMA kernel" in e.value.message
+
+
+# ---- MATMUL on the matrix cores ----------------------------------------------------------------------
+MATMUL_SHAPES = [(1, 2, 2, 2), (3, 17, 29, 11), (2, 128, 64, 128), (1, 33, 100, 65), (2, 70, 256, 40),
+                 (1, 1, 1024, 1), (4, 96, 48, 200)]
+
+
+@pytest.mark.parametrize("shape", MATMUL_SHAPES)
+@pytest.mark.parametrize("zps", [(-5, 3), (0, 0), (127, -128)])
+def test_matmul_i8_mfma_bit_exact(ctx, shape, zps):
+    n, h, c, w = shape
+    rng = np.random.default_rng(n * 1000 + h + c + w)
+    a = rng.integers(-128, 128, (n, h, c)).astype(np.int8)
+    b = rng.integers(-128, 128, (n, c, w)).astype(np.int8)
+    got, st = gpu_ops.matmul(ctx, a, b, *zps)
+    assert ctx.last_kernel == "matmul_mfma_i8"
+    assert st == capi.VALID and np.array_equal(got, oracle.matmul("i8", a, b, *zps))
+
+
+def test_config2_matmul_full_size(ctx):
+    """[8,1024,1024] x [8,1024,1024] -> int32, a_zp -5, b_zp 3: every element against a float64 BLAS product
+    (exact: |sum| < 2^53), one batch against the scalar oracle, plus the transposition property
+    (A.B)^T = B^T.A^T computed by the same kernel."""
+    c = cases.c2()
+    got, st = gpu_ops.matmul(ctx, c["a"], c["b"], c["a_zp"], c["b_zp"])
+    assert st == capi.VALID and ctx.last_kernel == "matmul_mfma_i8"
+    want = np.matmul(c["a"].astype(np.float64) - c["a_zp"], c["b"].astype(np.float64) - c["b_zp"])
+    assert np.array_equal(got, want.astype(np.int64).astype(np.int32))
+    assert np.array_equal(got[5], oracle.matmul("i8", c["a"][5:6], c["b"][5:6], c["a_zp"], c["b_zp"])[0])
+    at = np.ascontiguousarray(c["a"].transpose(0, 2, 1))
+    bt = np.ascontiguousarray(c["b"].transpose(0, 2, 1))
+    got_t, _ = gpu_ops.matmul(ctx, bt, at, c["b_zp"], c["a_zp"])
+    assert np.array_equal(got_t, got.transpose(0, 2, 1))
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+def test_matmul_fp_mfma_within_dot_product_bound(ctx, kind):
+    rng = np.random.default_rng(8)
+    n, h, c, w = 2, 96, 512, 72
+    a = rng.normal(0, 1 / 8, (n, h, c)).astype(np.float32)
+    b = rng.normal(0, 1 / 8, (n, c, w)).astype(np.float32)
+    if kind == "fp16":
+        a_s, b_s, dtype = a.astype(np.float16), b.astype(np.float16), capi.FP16
+        af, bf = a_s.astype(np.float64), b_s.astype(np.float64)
+    else:
+        a_s, b_s, dtype = cases.float_to_bf16_bits(a), cases.float_to_bf16_bits(b), capi.BF16
+        af, bf = cases.bf16_bits_to_float(a_s).astype(np.float64), cases.bf16_bits_to_float(b_s).astype(np.float64)
+    got, st = gpu_ops.matmul(ctx, a_s, b_s, dtype=dtype)
+    assert st == capi.VALID and got.dtype == np.float32
+    ref, bnd = np.matmul(af, bf), np.matmul(np.abs(af), np.abs(bf))
+    res = dp.check(got, ref, bnd, "fp32", dp.kernel_size_bound(c, "fp32", has_bias=False))
+    # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
+    assert res["ok"], res
