@@ -309,11 +309,14 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         ctx->last_kernel = "empty";
         return TMI_VALID;
     }
+    if (depthwise && ctx->kernel_choice != 1)
+        name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                    ctx->flags_dev);
     if (!depthwise && ctx->kernel_choice != 1)
         name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                   ctx->flags_dev);
     if (!name && ctx->kernel_choice == 2)
-        return fail(ctx, "%s: no MFMA kernel is eligible for this shape", op);
+        return fail(ctx, "%s: no MFMA / vector kernel is eligible for this shape", op);
     if (!name && depthwise)
         name = launch_depthwise_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                        ctx->flags_dev);

@@ -165,7 +165,7 @@ def test_mfma_not_eligible_is_an_error_when_forced(ctx):
     w = np.zeros((64, 31, 31, 64), np.int8)
     with pytest.raises(TmiError) as e:
         gpu_ops.conv2d(ctx, x, w, np.zeros(1, np.int32))
-    assert "no MFMA kernel" in e.value.message
+    assert "kernel is eligible" in e.value.message
 
 
 # ---- MATMUL on the matrix cores ----------------------------------------------------------------------
@@ -219,3 +219,70 @@ def test_matmul_fp_mfma_within_dot_product_bound(ctx, kind):
     res = dp.check(got, ref, bnd, "fp32", dp.kernel_size_bound(c, "fp32", has_bias=False))
     # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
     assert res["ok"], res
+
+
+# ---- DEPTHWISE_CONV2D, 16-channel vector kernel ------------------------------------------------------
+@pytest.mark.parametrize("shape", [  # n, ih, iw, c, kh, kw, pad, stride, dilation
+    (2, 10, 8, 16, 3, 3, (0, 1, 0, 1), (2, 2), (1, 1)),
+    (1, 9, 9, 48, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 12, 7, 32, 5, 3, (2, 2, 1, 1), (1, 1), (1, 1)),
+    (3, 8, 8, 96, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),
+])
+@pytest.mark.parametrize("zps", [(4, 0), (-3, 7), (0, 0)])
+def test_depthwise_vec16_bit_exact(ctx, shape, zps):
+    n, ih, iw, c, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(c + kh)
+    x = rng.integers(-128, 128, (n, ih, iw, c)).astype(np.int8)
+    w = rng.integers(-127, 128, (kh, kw, c, 1)).astype(np.int8)
+    for bias in (rng.integers(-30000, 30000, c).astype(np.int32), np.array([-77], np.int32)):
+        want = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, *zps)
+        got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, *zps, depthwise=True)
+        assert ctx.last_kernel == "depthwise_vec16_i8"
+        assert st == capi.VALID and np.array_equal(got, want)
+
+
+def _dw_expect(c, out_dtype=np.int8):
+    acc = oracle.depthwise_conv2d("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                                  c["w_zp"])
+    want, st = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype)
+    assert st == oracle.VALID
+    return want if c["clamp"] is None else oracle.clamp(want, *c["clamp"])
+
+
+def test_config4_depthwise_rescale_full_size(ctx):
+    c = cases.c4()
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                             c["w_zp"], depthwise=True, rescale=dict(mult=c["mult"], shift=c["shift"],
+                                                                     out_zp=c["out_zp"]))
+    assert ctx.last_kernel == "depthwise_vec16_i8_rescale"
+    want = _dw_expect(c)
+    assert st == capi.VALID and got.shape == (8, 56, 56, 96) and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("out_dtype", [np.int16, np.int32])
+def test_depthwise_rescale_other_outputs_and_clamp(ctx, out_dtype):
+    c = cases.c4(n=1, hw=16, c=32)
+    c["clamp"] = None
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                             c["w_zp"], depthwise=True, rescale=dict(mult=c["mult"], shift=c["shift"],
+                                                                     out_zp=0, out_dtype=out_dtype))
+    assert st == capi.VALID and np.array_equal(got, _dw_expect(c, out_dtype))
+    c["clamp"] = (-5, 60)
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                             c["w_zp"], depthwise=True, clamp=c["clamp"],
+                             rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=0))
+    assert st == capi.VALID and np.array_equal(got, _dw_expect(c))
+
+
+def test_depthwise_multiplier_falls_back_to_direct_kernel():
+    c2 = Context(0)
+    try:
+        rng = np.random.default_rng(1)
+        x = rng.integers(-128, 128, (1, 6, 6, 16)).astype(np.int8)
+        w = rng.integers(-127, 128, (3, 3, 16, 2)).astype(np.int8)
+        bias = rng.integers(-100, 100, 32).astype(np.int32)
+        got, st = gpu_ops.conv2d(c2, x, w, bias, (1, 1, 1, 1), in_zp=3, depthwise=True)
+        assert c2.last_kernel == "depthwise_direct_i8"
+        assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, (1, 1, 1, 1), in_zp=3))
+    finally:
+        c2.close()
