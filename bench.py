@@ -1,14 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-A step is one pass of the fused INT8 CONV2D -> RESCALE -> CLAMP operator (one C-ABI call) over one batch of
-the ResNet-style 3x3 configuration: input NHWC [8,56,56,64] int8 (input_zp -7), weight OHWI [64,3,3,64],
-bias int32, stride 1, pad 1, per-channel double-round RESCALE (shift 38) to int8, CLAMP [0,127].
-Operands are seeded synthetic tensors, resident in HBM before the timed region starts.
+A step is one pass of one operator (one C-ABI call) over one batch of seeded synthetic operands that are
+resident in HBM before the timed region starts.  The default workload is the one BASELINE.json's metric is
+quoted on:
 
-Prints one JSON line: metric / value in int8 TOPS (2 x dense MACs, padded taps counted), the roofline
-object for the convolution kernel (MFMA bound, dense int8 peak 5.0 POP/s) and the CPU baseline (the scalar
-C oracle, 1 core).
+  c3   INT8 CONV2D 3x3 [8,56,56,64]x[64,3,3,64] s1 p1 + per-channel RESCALE (shift 38, double_round) +
+       CLAMP [0,127], fused (default; unit TOPS, MFMA roofline)
+
+and --config selects the other BASELINE configurations, each reported against the roofline that bounds it:
+
+  c2   INT8 MATMUL [8,1024,1024]x[8,1024,1024] -> int32            (TOPS; HBM roofline, int32 result)
+  c4   INT8 DEPTHWISE_CONV2D [8,112,112,96] s2 + RESCALE, fused     (GB/s; HBM roofline)
+  c5a  FP16 CONV2D 3x3 [16,28,28,256]x[256,3,3,256], fp32 accumulate (TFLOPS; MFMA roofline)
+  c5b  BF16 MATMUL [4,2048,4096]x[4,4096,2048] -> fp32              (TFLOPS; MFMA roofline)
+
+One JSON line is printed: value = whole-job throughput over the timed steps (host clock), roofline.achieved =
+algorithmic work per launch / average launch duration from HIP events recorded on the launch stream, and
+cpu_baseline = the scalar C oracle (1 core) on a bounded sample of the same workload.
 """
 from __future__ import annotations
 
@@ -23,18 +32,19 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8, published
-# HBM bytes per launch of the convolution kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (profiles/conv2d_mfma_i8_rescale_c3_pmc.txt); None until measured.
-MEASURED_TRAFFIC_BYTES = None
+PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X, published)
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a
+# plain copy kernel of known size (see profiles/*_pmc.txt); None where not measured.
+MEASURED_TRAFFIC_BYTES = {"c3": 3693001, "c2": 174113648, "c4": 17376255, "c5a": 34578561, "c5b": 3126818328}
 
 
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "copy"])
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1",
@@ -51,82 +61,192 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     dev = torch.device("cuda:0")
-    c = cases.c3()
-    n, ih, iw, ic = c["x"].shape
-    oc, kh, kw, _ = c["w"].shape
-    oh, ow = ih, iw
-    macs = n * oh * ow * oc * kh * kw * ic
-    ops = 2 * macs
-    algo_bytes = c["x"].nbytes + c["w"].nbytes + c["bias"].nbytes + c["mult"].nbytes + c["shift"].nbytes + n * oh * ow * oc
-
-    t = {k: torch.from_numpy(np.ascontiguousarray(c[k])).to(dev) for k in ("x", "w", "bias", "mult", "shift")}
-    out = torch.empty((n, oh, ow, oc), dtype=torch.int8, device=dev)
-
     ctx = Context(0)
     stream = torch.cuda.current_stream()
     ctx.set_stream(stream.cuda_stream)
-    d = ctx.conv_desc(capi.INT8, capi.INT32, (n, ih, iw, ic), oc, kh, kw, (oh, ow), c["pad"], c["stride"],
-                      c["dilation"], c["bias"].shape[0])
-    r = ctx.rescale_desc(capi.INT32, capi.INT8, oc, oc, 0, c["out_zp"], True, capi.ROUND_DOUBLE, True)
 
-    def step():
-        ctx.conv2d_rescale_clamp(d, t["x"], t["w"], t["bias"], c["in_zp"], c["w_zp"], r, t["mult"], t["shift"], out,
-                                 c["clamp"])
+    def to_dev(a):
+        a = np.ascontiguousarray(a)
+        if a.dtype == np.uint16:  # bf16 bit patterns
+            return torch.from_numpy(a.view(np.int16)).to(dev)
+        return torch.from_numpy(a).to(dev)
 
-    for _ in range(args.warmup):
+    cfg = args.config
+    if cfg == "copy":
+        # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size
+        nbytes = 64 << 20
+        src = torch.zeros(nbytes, dtype=torch.int8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(args.steps or 20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": nbytes,
+                          "bytes_written_per_launch": nbytes}))
+        ctx.close()
+        return 0
+    W = {}  # workload description filled below
+    if cfg in ("c3", "c4"):
+        c = cases.c3() if cfg == "c3" else cases.c4()
+        depthwise = cfg == "c4"
+        n, ih, iw, ic = c["x"].shape
+        if depthwise:
+            kh, kw, _, m = c["w"].shape
+            oc = ic * m
+        else:
+            oc, kh, kw, _ = c["w"].shape
+        import oracle
+        oh, ow = oracle.conv_out_hw(ih, iw, kh, kw, c["pad"], c["stride"], c["dilation"])
+        macs = n * oh * ow * oc * kh * kw * (1 if depthwise else ic)
+        t = {k: to_dev(c[k]) for k in ("x", "w", "bias", "mult", "shift")}
+        out = torch.empty((n, oh, ow, oc), dtype=torch.int8, device=dev)
+        d = ctx.conv_desc(capi.INT8, capi.INT32, (n, ih, iw, ic), oc, kh, kw, (oh, ow), c["pad"], c["stride"],
+                          c["dilation"], c["bias"].shape[0])
+        r = ctx.rescale_desc(capi.INT32, capi.INT8, oc, oc, 0, c["out_zp"], True, capi.ROUND_DOUBLE, True)
+        fn = ctx.depthwise_conv2d_rescale_clamp if depthwise else ctx.conv2d_rescale_clamp
+
+        def step():
+            fn(d, t["x"], t["w"], t["bias"], c["in_zp"], c["w_zp"], r, t["mult"], t["shift"], out, c["clamp"])
+
+        def cpu_ref():
+            f = oracle.depthwise_conv2d if depthwise else oracle.conv2d
+            acc = f("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
+            ref, _ = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
+            return ref if c["clamp"] is None else oracle.clamp(ref, *c["clamp"])
+
+        W = dict(ops=2 * macs, bytes=sum(c[k].nbytes for k in ("x", "w", "bias", "mult", "shift")) + out.numel(),
+                 exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0, result=lambda: out.cpu().numpy(), dtype="int8")
+        if cfg == "c3":
+            W.update(metric="int8 CONV2D+RESCALE TOPS at 3x3 ResNet shape; % int8 MFMA peak; bit-exact", unit="TOPS",
+                     bound="mfma", peak=PEAK["int8_mfma"], runit="TOP/s",
+                     workload="configs[2]: INT8 CONV2D ResNet-style 3x3 [8,56,56,64]x[64,3,3,64] s1 p1 + per-channel "
+                              "RESCALE (shift 38, double_round) + CLAMP [0,127], fused")
+        else:
+            W.update(metric="int8 DEPTHWISE_CONV2D+RESCALE GB/s at MobileNetV2 shape; % HBM peak; bit-exact",
+                     unit="GB/s", bound="hbm", peak=PEAK["hbm"], runit="GB/s",
+                     workload="configs[3]: INT8 DEPTHWISE_CONV2D [8,112,112,96] 3x3 s2 pad [0,1,0,1] + per-channel "
+                              "RESCALE (shift 34..40, double_round), fused")
+    elif cfg in ("c2", "c5b"):
+        c = cases.c2() if cfg == "c2" else cases.c5_matmul()
+        n, h, k = c["a"].shape
+        w = c["b"].shape[2]
+        in_dtype = capi.INT8 if cfg == "c2" else capi.BF16
+        ta, tb = to_dev(c["a"]), to_dev(c["b"])
+        out = torch.empty((n, h, w), dtype=torch.int32 if cfg == "c2" else torch.float32, device=dev)
+        a_zp, b_zp = (c["a_zp"], c["b_zp"]) if cfg == "c2" else (0, 0)
+
+        def step():
+            ctx.matmul(in_dtype, n, h, k, w, ta, tb, a_zp, b_zp, out)
+
+        import oracle
+        rows = 64 if cfg == "c2" else 8  # bounded CPU sample: the first `rows` rows of batch 0
+
+        def cpu_ref():
+            if cfg == "c2":
+                return oracle.matmul("i8", c["a"][:1, :rows], c["b"][:1], a_zp, b_zp)
+            return oracle.matmul("f32", cases.bf16_bits_to_float(c["a"][:1, :rows]), cases.bf16_bits_to_float(c["b"][:1]))
+
+        W = dict(ops=2 * n * h * k * w, bytes=c["a"].nbytes + c["b"].nbytes + out.numel() * 4, exact=cfg == "c2",
+                 cpu_ref=cpu_ref, cpu_fraction=rows / (n * h), result=lambda: out[:1, :rows].cpu().numpy(),
+                 dtype="int8" if cfg == "c2" else "bf16")
+        if cfg == "c2":
+            W.update(metric="int8 MATMUL TOPS [8,1024,1024]x[8,1024,1024]; bit-exact", unit="TOPS", bound="hbm",
+                     peak=PEAK["hbm"], runit="GB/s",
+                     workload="configs[1]: INT8 MATMUL [8,1024,1024]x[8,1024,1024] -> int32, a_zp -5, b_zp 3")
+        else:
+            W.update(metric="bf16 MATMUL TFLOPS [4,2048,4096]x[4,4096,2048], fp32 accumulate", unit="TFLOPS",
+                     bound="mfma", peak=PEAK["f16_mfma"], runit="TFLOP/s",
+                     workload="configs[4b]: BF16 MATMUL [4,2048,4096]x[4,4096,2048] -> fp32")
+    else:  # c5a
+        c = cases.c5_conv()
+        n, ih, iw, ic = c["x"].shape
+        oc, kh, kw, _ = c["w"].shape
+        tx, tw, tb = to_dev(c["x"]), to_dev(c["w"]), to_dev(c["bias"])
+        out = torch.empty((n, ih, iw, oc), dtype=torch.float16, device=dev)
+        d = ctx.conv_desc(capi.FP16, capi.FP16, (n, ih, iw, ic), oc, kh, kw, (ih, iw), c["pad"], c["stride"],
+                          c["dilation"], oc)
+
+        def step():
+            ctx.conv2d(d, tx, tw, tb, 0, 0, out)
+
+        import oracle
+
+        def cpu_ref():  # bounded CPU sample: image 0 only
+            return oracle.conv2d("f32", c["x"][:1], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"])
+
+        W = dict(ops=2 * n * ih * iw * oc * kh * kw * ic, bytes=c["x"].nbytes + c["w"].nbytes + c["bias"].nbytes +
+                 out.numel() * 2, exact=False, cpu_ref=cpu_ref, cpu_fraction=1.0 / n,
+                 result=lambda: out[:1].cpu().numpy(), dtype="fp16",
+                 metric="fp16 CONV2D TFLOPS 3x3 [16,28,28,256]x[256,3,3,256], fp32 accumulate", unit="TFLOPS",
+                 bound="mfma", peak=PEAK["f16_mfma"], runit="TFLOP/s",
+                 workload="configs[4a]: FP16 CONV2D 3x3 [16,28,28,256]x[256,3,3,256] s1 p1, fp32 accumulate")
+
+    big = cfg in ("c5b",)
+    steps = args.steps if args.steps is not None else (200 if big else 2000)
+    warmup = args.warmup if args.warmup is not None else (20 if big else 200)
+
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record(stream)
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     ev1.record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     status = ctx.sync()
     kernel = ctx.last_kernel
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    ev_ms_per_launch = ev0.elapsed_time(ev1) / args.steps
-    tops = ops / (ms_per_step * 1e-3) / 1e12
-    achieved = ops / (ev_ms_per_launch * 1e-3) / 1e12
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    ev_s_per_launch = ev0.elapsed_time(ev1) * 1e-3 / steps
 
-    # parity of what was just timed, against the CPU oracle (bit exact)
-    result = {"metric": "int8 CONV2D+RESCALE TOPS at 3x3 ResNet shape; % int8 MFMA peak; bit-exact",
-              "value": round(tops, 3), "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-              "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-              "dtype": "int8", "data": "synthetic",
-              "config": {"workload": "configs[2]: INT8 CONV2D ResNet-style 3x3 [8,56,56,64]x[64,3,3,64] s1 p1 "
-                                     "+ per-channel RESCALE (shift 38, double_round) + CLAMP [0,127], fused",
-                         "kernel": kernel, "ops_per_step": ops, "algorithmic_bytes_per_step": algo_bytes,
-                         "graph_status": status},
-              "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": INT8_MFMA_PEAK_TOPS,
-                           "unit": "TOP/s", "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 5),
-                           "traffic": MEASURED_TRAFFIC_BYTES, "us_per_launch": round(ev_ms_per_launch * 1e3, 3)}}
+    work = W["bytes"] / 1e9 if W["unit"] == "GB/s" else W["ops"] / 1e12
+    value = work / (ms_per_step * 1e-3)
+    rwork = W["bytes"] / 1e9 if W["bound"] == "hbm" else W["ops"] / 1e12
+    achieved = rwork / ev_s_per_launch
 
+    result = {"metric": W["metric"], "value": round(value, 3), "unit": W["unit"], "n_gpus": 1, "steps": steps,
+              "warmup": warmup, "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak",
+              "vs_baseline": None, "dtype": W["dtype"], "data": "synthetic",
+              "config": {"workload": W["workload"], "kernel": kernel, "ops_per_step": W["ops"],
+                         "algorithmic_bytes_per_step": W["bytes"], "graph_status": status},
+              "roofline": {"bound": W["bound"], "achieved": round(achieved, 3), "peak": W["peak"], "unit": W["runit"],
+                           "frac": round(achieved / W["peak"], 5), "traffic": MEASURED_TRAFFIC_BYTES[cfg],
+                           "us_per_launch": round(ev_s_per_launch * 1e6, 3)}}
+    if W["bound"] == "hbm" and W["unit"] != "GB/s":
+        result["roofline"]["mfma_frac"] = round(W["ops"] / 1e12 / ev_s_per_launch / PEAK["int8_mfma"], 5)
+
+    rc = 0
     if not args.no_cpu_baseline:
-        import oracle
-        best = None
+        best, ref = None, None
         for _ in range(3):
             c0 = time.perf_counter()
-            acc = oracle.conv2d("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
-                                c["w_zp"])
-            ref, _ = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
-            ref = oracle.clamp(ref, *c["clamp"])
+            ref = W["cpu_ref"]()
             dt = time.perf_counter() - c0
             best = dt if best is None else min(best, dt)
-        bit_exact = bool(np.array_equal(out.cpu().numpy(), ref))
-        result["config"]["bit_exact_vs_oracle"] = bit_exact
-        result["cpu_baseline"] = {"value": round(ops / best / 1e12, 6), "unit": "TOPS", "cores": 1, "kind": "port",
-                                  "sample": "the full config (1 batch of [8,56,56,64]), min of 3 runs of the scalar "
-                                            "C oracle (conv2d + rescale + clamp), %.2f s per run" % best}
-        if not bit_exact:
+            if best > 10.0:
+                break
+        got = W["result"]()
+        if W["exact"]:
+            ok = bool(np.array_equal(got, ref))
+            result["config"]["bit_exact_vs_oracle"] = ok
+        else:
+            g64 = got.astype(np.float64)
+            r64 = np.asarray(ref, np.float64)
+            err = float(np.max(np.abs(g64 - r64) / np.maximum(np.abs(r64), 1e-3)))
+            ok = err < 2e-2  # sanity only: the DOT_PRODUCT-bound check against fp64 lives in the tests
+            result["config"]["max_rel_err_vs_fp32_oracle"] = err
+        cpu_work = work * W["cpu_fraction"]
+        result["cpu_baseline"] = {"value": round(cpu_work / best, 6), "unit": W["unit"], "cores": 1, "kind": "port",
+                                  "sample": "%.4g of one step's work (%s), min of up to 3 runs of the scalar C oracle, "
+                                            "%.2f s per run" % (W["cpu_fraction"], "whole batch" if W["cpu_fraction"] == 1.0
+                                                                else "leading rows / first image", best)}
+        if not ok:
             print("bench.py: GPU result differs from the oracle", file=sys.stderr)
-            print(json.dumps(result))
-            return 1
+            rc = 1
     print(json.dumps(result))
     ctx.close()
-    return 0
+    return rc
 
 
 if __name__ == "__main__":
