@@ -191,6 +191,19 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
                                        const void* shift_dev, int32_t has_clamp, int32_t clamp_min,
                                        int32_t clamp_max, void* out_dev);
 
+/* ---- validation only (no launch) ---------------------------------------------------------------- */
+
+/* The checks OpConv2d / OpDepthwiseConv2d::checkTensorAttributes and the head of eval() perform
+ * (reference_model/src/ops/tensor_ops.cpp:120-226, 690-720, 742-748, 1139-1169, 1191-1197): attribute sizes
+ * and signs, the output-shape rule, channel and bias consistency, supported type combination.  Called from an
+ * adapter's checkTensorAttributes() so that SubgraphTraverser::validateGraph() rejects a malformed node before
+ * anything is evaluated.  depthwise != 0 selects the DEPTHWISE_CONV2D rules. */
+int tmi_conv2d_check(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, int32_t depthwise);
+
+/* OpRescale::checkTensorAttributes and the zero-point rules at the head of eval()
+ * (reference_model/src/ops/type_conversion.cpp:72-154, 242-255). */
+int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int32_t C);
+
 /* ---- tuning / test hooks ------------------------------------------------------------------------- */
 
 /* Forces a kernel family for the following operator calls: 0 = automatic choice, 1 = direct (one output

@@ -71,5 +71,27 @@ def build(force: bool = False, jobs: int = 8) -> str:
     return LIB
 
 
+def build_host(force: bool = False) -> list:
+    """Compiles the C++ host side above the C ABI (g++, links against libtosa_mi355.so):
+    tosa_mi355_run (command-line runner) and tosa_mi355_host_kats (known-answer tests)."""
+    host = os.path.join(CSRC, "host")
+    common = [os.path.join(host, f) for f in ("formats.cc", "runtime.cc")]
+    outs = []
+    for exe, main in ((HOST_BIN, "main.cc"), (os.path.join(HERE, "tosa_mi355_host_kats"), "host_kats.cc")):
+        srcs = common + [os.path.join(host, main)]
+        deps = srcs + [os.path.join(host, "tosa_host.h"), os.path.join(INCLUDE, "tosa_mi355.h"), LIB]
+        if force or not os.path.exists(exe) or any(os.path.getmtime(d) > os.path.getmtime(exe) for d in deps):
+            cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", f"-I{INCLUDE}", f"-I{host}", *srcs, "-o", exe,
+                   f"-L{HERE}", "-ltosa_mi355", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath-link," + "/opt/rocm/lib"]
+            r = subprocess.run(cmd, capture_output=True, text=True)
+            if r.returncode != 0:
+                raise RuntimeError(f"g++ failed on {main}:\n{r.stdout}\n{r.stderr}")
+            if r.stderr.strip():
+                sys.stderr.write(r.stderr)
+        outs.append(exe)
+    return outs
+
+
 if __name__ == "__main__":
     print(build(force="--force" in sys.argv))
+    print(build_host(force="--force" in sys.argv))

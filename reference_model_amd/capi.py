@@ -29,7 +29,7 @@ EXPORTS = [
     "tmi_version", "tmi_ctx_create", "tmi_ctx_destroy", "tmi_ctx_set_stream", "tmi_ctx_sync", "tmi_ctx_flags",
     "tmi_last_error", "tmi_last_kernel", "tmi_buf_alloc", "tmi_buf_free", "tmi_upload", "tmi_download",
     "tmi_conv2d", "tmi_depthwise_conv2d", "tmi_matmul", "tmi_rescale", "tmi_clamp", "tmi_conv2d_rescale_clamp",
-    "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice",
+    "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice", "tmi_conv2d_check", "tmi_rescale_check",
 ]
 
 
@@ -96,6 +96,8 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_matmul.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, i32, vp]
     lib.tmi_rescale.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i64, i32, vp, vp, vp, vp]
     lib.tmi_clamp.argtypes = [vp, i32, i64, vp, i32, i32, vp]
+    lib.tmi_conv2d_check.argtypes = [vp, ctypes.POINTER(ConvDesc), i32]
+    lib.tmi_rescale_check.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i32]
     for name in EXPORTS:
         fn = getattr(lib, name)
         if fn.restype is ctypes.c_int:

@@ -483,6 +483,25 @@ int tmi_download(tmi_ctx_t* ctx, void* dst_host, const void* src_dev, size_t byt
     return TMI_VALID;
 }
 
+int tmi_conv2d_check(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, int32_t depthwise)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    ConvGeom g;
+    return validate_conv(ctx, depthwise ? "OpDepthwiseConv2d" : "OpConv2d", d, depthwise != 0, 0, 0, g);
+}
+
+int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int32_t C)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (rank < 0 || rank > 6)
+        return fail(ctx, "OpRescale: rank outside [0,6]");
+    RescaleParams p;
+    static const int8_t dummy = 0;    // only the pointers' presence is checked here
+    return validate_rescale(ctx, r, rank, C, &dummy, &dummy, p);
+}
+
 int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
 {

@@ -1,0 +1,181 @@
+"""The C++ host side (GraphNode-shaped adapters + graph runtime + file readers) through its two executables.
+
+CPU part: the test-only FlatBuffers writer round-trips through the test-only reader, and the runner refuses to
+run without a GPU (no CPU fall-back).  GPU part: the reference-style known-answer binary, the reference's
+int8 example directory end to end (with and without operator fusion), and synthetic graphs against the oracle,
+including the UNPREDICTABLE and ERROR exit codes."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import cases
+import oracle
+import tosa_fb_writer as W
+import tosa_flatbuffer as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+RUN = os.path.join(ROOT, "reference_model_amd", "tosa_mi355_run")
+KATS = os.path.join(ROOT, "reference_model_amd", "tosa_mi355_host_kats")
+
+
+def _write_case(tmp_path, raw_graph, inputs, ofm_names):
+    (tmp_path / "graph.tosa").write_bytes(raw_graph)
+    desc = {"tosa_file": "graph.tosa", "ifm_name": [], "ifm_file": [], "ofm_name": [], "ofm_file": []}
+    for name, arr in inputs.items():
+        np.save(tmp_path / f"{name}.npy", arr)
+        desc["ifm_name"].append(name)
+        desc["ifm_file"].append(f"{name}.npy")
+    for name in ofm_names:
+        desc["ofm_name"].append(name)
+        desc["ofm_file"].append(f"{name}_out.npy")
+    (tmp_path / "desc.json").write_text(json.dumps(desc))
+    return str(tmp_path / "desc.json")
+
+
+def _run(desc, *extra):
+    return subprocess.run([RUN, f"--test_desc={desc}", *extra], capture_output=True, text=True, timeout=120)
+
+
+def _conv_graph(c, depthwise=False, with_clamp=True, shift_override=None):
+    x, w = c["x"], c["w"]
+    oc = w.shape[2] * w.shape[3] if depthwise else w.shape[0]
+    kh, kw = (w.shape[0], w.shape[1]) if depthwise else (w.shape[1], w.shape[2])
+    oh, ow = oracle.conv_out_hw(x.shape[1], x.shape[2], kh, kw, c["pad"], c["stride"], c["dilation"])
+    shift = c["shift"] if shift_override is None else shift_override
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", w.shape, np.int8, w), W.tensor("bias", c["bias"].shape, np.int32, c["bias"]),
+          W.tensor("izp", [1], np.int8, [c["in_zp"]]), W.tensor("wzp", [1], np.int8, [c["w_zp"]]),
+          W.tensor("acc", [x.shape[0], oh, ow, oc], np.int32), W.tensor("mult", [oc], np.int32, c["mult"]),
+          W.tensor("shift", [oc], np.int8, shift), W.tensor("rizp", [1], np.int32, [0]),
+          W.tensor("rozp", [1], np.int8, [c["out_zp"]]), W.tensor("q", [x.shape[0], oh, ow, oc], np.int8),
+          W.tensor("y", [x.shape[0], oh, ow, oc], np.int8)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "izp", "wzp", "mult", "shift", "rizp", "rozp")]
+    ops.append(W.operator(R.OP_DEPTHWISE_CONV2D if depthwise else R.OP_CONV2D, ["x", "w", "bias", "izp", "wzp"], ["acc"],
+                          W.conv_attr(c["pad"], c["stride"], c["dilation"])))
+    ops.append(W.operator(R.OP_RESCALE, ["acc", "mult", "shift", "rizp", "rozp"], ["q"], W.rescale_attr()))
+    out = "q"
+    if with_clamp and c["clamp"] is not None:
+        ops.append(W.operator(R.OP_CLAMP, ["q"], ["y"], W.clamp_attr(*c["clamp"])))
+        out = "y"
+    return W.graph(ts, ops, ["x"], [out]), out
+
+
+def _expect(c, depthwise=False):
+    f = oracle.depthwise_conv2d if depthwise else oracle.conv2d
+    acc = f("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
+    want, _ = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
+    return want if c["clamp"] is None else oracle.clamp(want, *c["clamp"])
+
+
+# ---- CPU ----------------------------------------------------------------------------------------------------
+def test_writer_round_trips_through_reader(tmp_path):
+    c = cases.c3(n=1, hw=6)
+    raw, out = _conv_graph(c)
+    p = tmp_path / "g.tosa"
+    p.write_bytes(raw)
+    tensors, ops, ins, outs = R.load_main_block(str(p))
+    assert ins == ["x"] and outs == [out]
+    assert [o["op"] for o in ops][-3:] == [R.OP_CONV2D, R.OP_RESCALE, R.OP_CLAMP]
+    assert np.array_equal(tensors["w"]["data"], c["w"]) and np.array_equal(tensors["mult"]["data"], c["mult"])
+    assert R.conv_attr(ops[-3]["attr"])["pad"] == [1, 1, 1, 1]
+    assert R.rescale_attr(ops[-2]["attr"]) == dict(scale32=True, rounding_mode=3, per_channel=True,
+                                                   input_unsigned=False, output_unsigned=False)
+
+
+def test_runner_refuses_to_run_without_a_gpu(golden_dir):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    assert os.path.exists(RUN), "build the host side first: python -m reference_model_amd.build"
+    r = _run(os.path.join(golden_dir, "qi8_conv2d_1x1", "desc.json"), "--ofm_file=/tmp/should_not_exist.npy")
+    assert r.returncode == 2 and "no CPU fall-back" in r.stderr
+    assert not os.path.exists("/tmp/should_not_exist.npy")
+
+
+# ---- GPU ----------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_reference_style_known_answer_binary():
+    r = subprocess.run([KATS], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("PASS") == 23 and "FAIL" not in r.stdout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fusion", [True, False])
+def test_reference_qi8_example_directory(golden_dir, tmp_path, fusion):
+    out = str(tmp_path / "out.npy")
+    args = [f"--ofm_file={out}"] + ([] if fusion else ["--no_fusion"])
+    r = _run(os.path.join(golden_dir, "qi8_conv2d_1x1", "desc.json"), *args)
+    assert r.returncode == 0, r.stderr
+    want = np.load(os.path.join(golden_dir, "qi8_conv2d_1x1", "tflite_result.npy"))
+    got = np.load(out)
+    assert got.dtype == np.int8 and np.array_equal(got, want)
+    assert ("kernels launched: 1, nodes folded into a producer: 1" if fusion else
+            "kernels launched: 2, nodes folded into a producer: 0") in r.stderr
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("which", ["conv_rescale_clamp", "depthwise_rescale"])
+def test_synthetic_graphs_match_oracle(tmp_path, which):
+    depthwise = which == "depthwise_rescale"
+    c = cases.c4(n=2, hw=20, c=32) if depthwise else cases.c3(n=2, hw=14)
+    raw, out = _conv_graph(c, depthwise=depthwise)
+    desc = _write_case(tmp_path, raw, {"x": c["x"]}, [out])
+    for extra in ([], ["--no_fusion"]):
+        r = _run(desc, *extra)
+        assert r.returncode == 0, r.stderr
+        assert np.array_equal(np.load(tmp_path / f"{out}_out.npy"), _expect(c, depthwise)), extra
+    assert "nodes folded into a producer: 0" in r.stderr
+
+
+@pytest.mark.gpu
+def test_matmul_graph(tmp_path):
+    rng = np.random.default_rng(4)
+    a = rng.integers(-128, 128, (2, 40, 96)).astype(np.int8)
+    b = rng.integers(-128, 128, (2, 96, 24)).astype(np.int8)
+    ts = [W.tensor("a", a.shape, np.int8), W.tensor("b", b.shape, np.int8), W.tensor("azp", [1], np.int8, [-5]),
+          W.tensor("bzp", [1], np.int8, [3]), W.tensor("o", [2, 40, 24], np.int32)]
+    ops = [W.operator(R.OP_CONST, [], ["azp"]), W.operator(R.OP_CONST, [], ["bzp"]),
+           W.operator(R.OP_MATMUL, ["a", "b", "azp", "bzp"], ["o"])]
+    desc = _write_case(tmp_path, W.graph(ts, ops, ["a", "b"], ["o"]), {"a": a, "b": b}, ["o"])
+    r = _run(desc)
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(tmp_path / "o_out.npy"), oracle.matmul("i8", a, b, -5, 3))
+
+
+@pytest.mark.gpu
+def test_exit_codes_unpredictable_and_error(tmp_path):
+    c = cases.c1()
+    # shift 12 admits |acc| < 2^11 only: apply_scale_32's value REQUIRE fires -> exit code 1, output still written
+    raw, out = _conv_graph(c, shift_override=np.full(16, 12, np.int8))
+    d1 = tmp_path / "u"
+    d1.mkdir()
+    r = _run(_write_case(d1, raw, {"x": c["x"]}, [out]))
+    assert r.returncode == 1 and "UNPREDICTABLE" in r.stderr
+    # declared output shape that violates the convolution shape rule -> rejected by validateGraph, exit code 2
+    bad = dict(c)
+    bad["pad"] = (1, 0, 0, 0)
+    raw_bad, out = _conv_graph(bad)
+    raw_ok, _ = _conv_graph(c)
+    d2 = tmp_path / "e"
+    d2.mkdir()
+    # take the good graph's tensors but the bad attribute by rebuilding with mismatching pad vs declared output
+    ts_ops = _conv_graph(c)  # noqa: F841  (documented intent; the mismatch below is what is tested)
+    x = c["x"]
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", c["w"].shape, np.int8, c["w"]),
+          W.tensor("bias", [16], np.int32, c["bias"]), W.tensor("z", [1], np.int8, [0]),
+          W.tensor("acc", [1, 32, 32, 16], np.int32)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "z")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "bias", "z", "z"], ["acc"], W.conv_attr([1, 0, 0, 0], [1, 1], [1, 1])))
+    r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["acc"]), {"x": x}, ["acc"]))
+    assert r.returncode == 2 and "Mismatch between output shape provided and expected output shape" in r.stderr
+    assert not (d2 / "acc_out.npy").exists()
+    # an operator outside the accelerated path (ADD = 15) is refused loudly rather than evaluated on the host
+    ts = [W.tensor("x", [4], np.int32), W.tensor("y", [4], np.int32)]
+    d3 = tmp_path / "o"
+    d3.mkdir()
+    r = _run(_write_case(d3, W.graph(ts, [W.operator(15, ["x", "x"], ["y"])], ["x"], ["y"]),
+                         {"x": np.arange(4, dtype=np.int32)}, ["y"]))
+    assert r.returncode == 2 and "outside the accelerated path" in r.stderr
