@@ -36,6 +36,8 @@
 // Epilogue: the per-channel constants (bias, multiplier, shift and the 64-bit rounding terms derived from
 // them) are computed once per workgroup by OCB lanes while the staging loads are in flight and kept in an
 // LDS table; every lane then spends about ten instructions per output element.
+#include <type_traits>
+
 #include "tmi_kernels.h"
 
 namespace tmi
@@ -227,7 +229,9 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const ConvGeom& g    = a.g;
     const int tid        = threadIdx.x;
     const int lane       = tid & 63;
-    const int wave       = tid >> 6;
+    // wave-uniform values are made scalar explicitly: with two waves per SIMD the vector ALU (4 cycles per
+    // wave64 instruction) is the scarce resource, so everything uniform must run on the scalar unit
+    const int wave       = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int woc        = wave / WPX;   // channel tile of this wave
     const int wpx        = wave % WPX;   // first pixel tile of this wave is wpx*PXT
     const int li         = lane & 31;    // row of the A fragment / column (pixel) of D
@@ -237,6 +241,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const int blk_bytes  = a.CH * 16;
     const int ch_shift   = a.CH == 4 ? 2 : (a.CH == 2 ? 1 : 0);
     const int n_pairs    = taps * a.CH;  // (tap, chunk) pairs per channel block = chunks per weight row
+    const int fill_word  = M::is_int ? (a.za & 0xff) * 0x01010101 : 0;    // out-of-image pixels hold input_zp
 
     // LDS: [channel table][16 zero bytes][pair offset table][weight rows][input patch]
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -245,7 +250,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     constexpr int kCtab    = OCB * (int)sizeof(ChanEntry);
     uint8_t* zero_chunk    = lds + kCtab;
     int* pairoff           = reinterpret_cast<int*>(lds + kCtab + 16);
-    const int tab_entries  = n_pairs + 12;    // slack: the pipeline reads a few entries past the end
+    const int tab_entries  = n_pairs + 32;    // 2*(ksteps + 3G) + 1 < n_pairs + 32 for G = 3    // slack: the pipeline reads a few entries past the end
     const int tab_bytes    = (tab_entries * 4 + 15) & ~15;
     uint8_t* wl            = lds + kCtab + 16 + tab_bytes;
     uint8_t* pl            = wl + OCB * a.wstride;
@@ -277,6 +282,10 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     uint32_t flags = 0;
     if (tid < 4)
         reinterpret_cast<int*>(zero_chunk)[tid] = 0;
+    // An odd pair count leaves the upper K half of the last step empty: the spare chunk behind every weight
+    // row is zero, so that half contributes nothing whatever the pixel operand holds.
+    if ((n_pairs & 1) && tid < OCB)
+        *reinterpret_cast<v4i*>(wl + tid * a.wstride + n_pairs * 16) = v4i{ 0, 0, 0, 0 };
     for (int q = tid; q < tab_entries; q += NT)
     {
         int off = 0;
@@ -330,7 +339,6 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 #pragma unroll
         for (int r = 0; r < 16; r++)
             acc[i][r] = 0;
-    int wsum = 0;
     int asum[PXT];
 #pragma unroll
     for (int i = 0; i < PXT; i++)
@@ -377,7 +385,8 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                         const bool ld    = img && off < row_bytes;
                         const size_t src = ld ? (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes + off : 0;
                         const v4i v      = *reinterpret_cast<const v4i*>(a.in + src);
-                        const v4i f      = fill_chunk(off, row_bytes, M::is_int ? a.za : 0);
+                        const int fw     = off < row_bytes ? fill_word : 0;    // whole chunks only in this path
+                        const v4i f      = v4i{ fw, fw, fw, fw };
                         pv[u]            = ld ? v : (img ? v4i{ 0, 0, 0, 0 } : f);
                     }
                     else
@@ -429,58 +438,111 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         }
         __syncthreads();
 
+        // ---- sum(w) per output channel, for the zero-point correction -----------------------------------------
+        // NT/OCB lanes share a weight row: each adds up the bytes of its chunks with v_dot4, a butterfly
+        // finishes the row, and -za*sum(w) goes straight into the channel table's bias (one LDS atomic per row,
+        // all rows distinct).  Doing this once per block keeps the K loop free of side computations.
+        if constexpr (M::is_int)
+        {
+            if (a.za != 0)
+            {
+                constexpr int LPR = NT / OCB;    // lanes per row: 8 or 16
+                const int row     = tid / LPR;   // row of the staged operand: tile*32 + 8q + 4h + j
+                const int part    = tid % LPR;
+                const uint8_t* rp = wl + row * a.wstride;
+                int sum           = 0;
+                for (int j = part; j < n_pairs; j += LPR)
+                    sum += dot4_ones(*reinterpret_cast<const v4i*>(rp + j * 16));
+#pragma unroll
+                for (int m = 1; m < LPR; m <<= 1)
+                    sum += __shfl_xor(sum, m);
+                if (part == 0)
+                {
+                    const int r32 = row & 31;    // 8q + 4h + j  ->  channel 16h + 4q + j
+                    const int ch  = (row & ~31) + ((r32 >> 2) & 1) * 16 + (r32 >> 3) * 4 + (r32 & 3);
+                    atomicAdd(&ctab[ch].bias, -a.za * sum);
+                }
+            }
+        }
+
         // ---- MFMA over the (tap, chunk) pairs of this channel block -----------------------------------
         if (wave_active)
         {
-            const uint8_t* wrow = wl + (woc * 32 + li) * a.wstride;
-            // requests the fragments of K-step s; `po` is the pair's patch offset read from the table earlier
-            auto issue = [&](int s, int po, v4i& fa, v4i(&fb)[PXT]) {
-                const int q     = 2 * s + lh;
-                const bool live = q < n_pairs;
-                fa              = *reinterpret_cast<const v4i*>(live ? wrow + q * 16 : zero_chunk);
+            // Double buffered in groups of G steps: at the top of a round the fragments of the next group are
+            // requested (their patch offsets were read from the table one round earlier), then the current
+            // group's MFMAs issue, so the wait in front of an MFMA only meets loads that have had a whole
+            // group of matrix instructions to complete.  The main loop runs on whole pairs of groups and has no
+            // branch in its body; what is left (fewer than 2G steps) goes through the checked tail.  Loads past
+            // the last step are clamped to it and never used.
+            constexpr int G     = 3;
+            const uint8_t* wrow = wl + (woc * 32 + li) * a.wstride + lh * 16;
+            const int* tab      = pairoff + lh;
+            const int last_step = a.ksteps - 1;
+            v4i fa[2][G], fb[2][G][PXT];
+            int po[G];
+            auto load_group = [&](int s0, v4i(&ga)[G], v4i(&gb)[G][PXT]) {
 #pragma unroll
-                for (int i = 0; i < PXT; i++)
-                    fb[i] = *reinterpret_cast<const v4i*>(live ? pl + pbase[i] + po : zero_chunk);
-            };
-            auto compute = [&](const v4i& fa, const v4i(&fb)[PXT]) {
-#pragma unroll
-                for (int i = 0; i < PXT; i++)
-                    acc[i] = M::mma(fa, fb[i], acc[i]);
-                if constexpr (M::is_int)
+                for (int u = 0; u < G; u++)
                 {
-                    if (a.za != 0)
-                        wsum += dot4_ones(fa);
-                    if (a.zw != 0)
+                    const int sc = s0 + u < last_step ? s0 + u : last_step;
+                    ga[u]        = *reinterpret_cast<const v4i*>(wrow + sc * 32);
+#pragma unroll
+                    for (int i = 0; i < PXT; i++)
+                        gb[u][i] = *reinterpret_cast<const v4i*>(pl + pbase[i] + po[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < G; u++)
+                    po[u] = tab[2 * (s0 + G + u)];    // offsets of the group after that one
+            };
+            // ZW: the weight zero point is non-zero, so sum(a) per pixel is needed as well; it is accumulated
+            // from the pixel fragments here (the upper K half of an odd last step holds no pair)
+            auto run = [&](auto zw_tag) {
+                constexpr bool ZW = decltype(zw_tag)::value;
+                auto compute = [&](int s, const v4i& ga, const v4i(&gb)[PXT]) {
+#pragma unroll
+                    for (int i = 0; i < PXT; i++)
+                        acc[i] = M::mma(ga, gb[i], acc[i]);
+                    if constexpr (ZW)
+                    {
+                        const bool live = 2 * s + lh < n_pairs;
 #pragma unroll
                         for (int i = 0; i < PXT; i++)
-                            asum[i] += dot4_ones(fb[i]);
+                            asum[i] += live ? dot4_ones(gb[i]) : 0;
+                    }
+                };
+#pragma unroll
+                for (int u = 0; u < G; u++)
+                    po[u] = tab[2 * u];
+                load_group(0, fa[0], fb[0]);
+                int s = 0;
+                for (; s + 2 * G <= a.ksteps; s += 2 * G)
+                {
+                    load_group(s + G, fa[1], fb[1]);
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        compute(s + u, fa[0][u], fb[0][u]);
+                    load_group(s + 2 * G, fa[0], fb[0]);
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        compute(s + G + u, fa[1][u], fb[1][u]);
+                }
+                if (s < a.ksteps)
+                {
+                    load_group(s + G, fa[1], fb[1]);
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        if (s + u < a.ksteps)
+                            compute(s + u, fa[0][u], fb[0][u]);
+#pragma unroll
+                    for (int u = 0; u < G; u++)
+                        if (s + G + u < a.ksteps)
+                            compute(s + G + u, fa[1][u], fb[1][u]);
                 }
             };
-            const int* tab = pairoff + lh;
-            int po0 = tab[0], po1 = tab[2], po2 = tab[4];
-            v4i fa0, fa1, fa2, fb0[PXT], fb1[PXT], fb2[PXT];
-            issue(0, po0, fa0, fb0);
-            po0 = tab[6];
-            issue(1, po1, fa1, fb1);
-            po1 = tab[8];
-            for (int s = 0; s < a.ksteps; s += 3)
-            {
-                issue(s + 2, po2, fa2, fb2);
-                po2 = tab[2 * (s + 5)];
-                compute(fa0, fb0);
-                if (s + 1 < a.ksteps)
-                {
-                    issue(s + 3, po0, fa0, fb0);
-                    po0 = tab[2 * (s + 6)];
-                    compute(fa1, fb1);
-                }
-                if (s + 2 < a.ksteps)
-                {
-                    issue(s + 4, po1, fa1, fb1);
-                    po1 = tab[2 * (s + 7)];
-                    compute(fa2, fb2);
-                }
-            }
+            if (M::is_int && a.zw != 0)
+                run(std::true_type{});
+            else
+                run(std::false_type{});
         }
     }
 
@@ -574,10 +636,9 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 sa += __shfl_xor(sa, 32);
             pcorr[i] = kzz - a.zw * sa;
         }
-        // finish the K-half reduction of sum(w): afterwards lane i (either half) holds za * the total of
-        // operand row i of the wave's channel tile
+        // -za*sum(w) was added to the channel table's bias after staging: make it visible to every wave
         if (a.za != 0)
-            wsum = (wsum + __shfl_xor(wsum, 32)) * a.za;
+            __syncthreads();
         // int32 rows of four channels can be stored as one vector; int8 rows of 16 channels likewise
         const bool vec4  = full && (g.OC & 3) == 0 && ((uintptr_t)a.out & 15) == 0;
         const bool vec16 = full && (g.OC & 15) == 0 && ((uintptr_t)a.out & 15) == 0;
@@ -593,12 +654,12 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         {
             const int c0 = oc0 + ocl0 + 4 * q;
             ChanEntry ce[4];
-            int32_t cb[4];    // bias minus the weight-sum term of the zero-point correction
+            int32_t cb[4];    // bias minus za * sum(w)
 #pragma unroll
             for (int r = 0; r < 4; r++)
             {
                 ce[r] = ctab[ocl0 + 4 * q + r];
-                cb[r] = ce[r].bias - (a.za != 0 ? __shfl(wsum, 8 * q + 4 * lh + r) : 0);
+                cb[r] = ce[r].bias;
             }
 #pragma unroll
             for (int i = 0; i < PXT; i++)
@@ -747,7 +808,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     a.n_icb        = (row_bytes + a.CH * 16 - 1) / (a.CH * 16);
     const int taps = g.KH * g.KW;
     const int rch  = taps * a.CH;    // chunks per weight row
-    a.wstride      = rch * 16 + ((rch & 1) ? 0 : 16);
+    a.wstride      = (rch + (rch & 1)) * 16 + 16;    // room for a spare zero chunk; = 16 (mod 32)
     a.ksteps       = (rch + 1) / 2;
 
     const int WOC           = g.OC > 32 ? 2 : 1;
@@ -767,7 +828,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
         TH = g.OH;
     if (TH < 1)
         TH = 1;
-    const size_t fixed_bytes = (size_t)OCB * 32 + 16 + ((((size_t)rch + 12) * 4 + 15) & ~(size_t)15);
+    const size_t fixed_bytes = (size_t)OCB * 32 + 16 + ((((size_t)rch + 32) * 4 + 15) & ~(size_t)15);
     const size_t w_bytes     = (size_t)OCB * a.wstride;
     size_t lds_bytes         = 0;
     for (;;)
