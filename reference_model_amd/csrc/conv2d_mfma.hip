@@ -249,10 +249,11 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     float* ftab            = reinterpret_cast<float*>(lds);    // floating point: bias as float
     constexpr int kCtab    = OCB * (int)sizeof(ChanEntry);
     uint8_t* zero_chunk    = lds + kCtab;
-    int* pairoff           = reinterpret_cast<int*>(lds + kCtab + 16);
+    int* need_check        = reinterpret_cast<int*>(lds + kCtab + 16);    // set when some channel has shift < 32
+    int* pairoff           = reinterpret_cast<int*>(lds + kCtab + 32);
     const int tab_entries  = n_pairs + 32;    // 2*(ksteps + 3G) + 1 < n_pairs + 32 for G = 3    // slack: the pipeline reads a few entries past the end
     const int tab_bytes    = (tab_entries * 4 + 15) & ~15;
-    uint8_t* wl            = lds + kCtab + 16 + tab_bytes;
+    uint8_t* wl            = lds + kCtab + 32 + tab_bytes;
     uint8_t* pl            = wl + OCB * a.wstride;
 
     // ---- which tile ------------------------------------------------------------------------------------
@@ -313,7 +314,14 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 const int32_t m       = ok ? load_multiplier(a.rp, oc) : 0;
                 const int32_t sh      = ok ? load_shift(a.rp, oc) : 32;
                 const ChannelScale cs = make_channel_scale(m, sh, a.rp.double_round, flags);
-                e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos, e.rnd_neg = cs.rnd_neg;
+                // (p + rnd) >> s + zp == (p + rnd + zp * 2^s) >> s: the output zero point rides in the rounding term
+                const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
+                e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos + zp_term, e.rnd_neg = cs.rnd_neg + zp_term;
+                // a shift below 32 somewhere: apply_scale_32's value range can be violated and must be checked.
+                // All table lanes sit in wave 0, so one ballot decides and a single lane writes the word.
+                const int any_check = __any(cs.lim != 0x80000000u);
+                if (tid == 0)
+                    *need_check = any_check;
             }
             ctab[tid] = e;
         }
@@ -349,6 +357,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     for (int icb = 0; icb < a.n_icb; icb++)
     {
         const int ic_off = icb * blk_bytes;
+        int staged_w_sum = 0;
         if (icb)
             __syncthreads();
         // ---- stage the weight rows and the input patch ---------------------------------------------------
@@ -359,10 +368,18 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         // a clamped, valid address and the result is replaced afterwards, which keeps the round free of
         // branches so that its loads really are in flight together.
         {
-            const int w_total = OCB * n_pairs;
+            // weight rows: NT/OCB lanes share a row and walk its chunks, so no division is needed
+            constexpr int LPR = NT / OCB;
+            const int w_ocl   = tid / LPR;
+            const int w_part  = tid % LPR;
+            const int w_r32   = w_ocl & 31;    // output channel -> row of the MFMA operand (see the header comment)
+            const int w_row   = (w_ocl & ~31) + ((w_r32 >> 2) & 3) * 8 + (w_r32 >> 4) * 4 + (w_r32 & 3);
+            const bool w_oc_ok = oc0 + w_ocl < g.OC;
+            const size_t w_src_row = (size_t)(oc0 + w_ocl) * taps * row_bytes;
+            int w_sum = 0;
             const int p_total = a.PH * a.PW * a.CH;
-            for (int wbase = tid, pbase_idx = tid; wbase < w_total || pbase_idx < p_total;
-                 wbase += NT * WU, pbase_idx += NT * PU)
+            for (int wj0 = w_part, pbase_idx = tid; wj0 < n_pairs || pbase_idx < p_total;
+                 wj0 += LPR * WU, pbase_idx += NT * PU)
             {
                 v4i wv[WU], pv[PU];
                 int wdst[WU], pdst[PU];
@@ -401,29 +418,24 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 #pragma unroll
                 for (int u = 0; u < WU; u++)
                 {
-                    const int idx = wbase + u * NT;
-                    const bool ok = idx < w_total;
-                    const int idc = ok ? idx : 0;
-                    const int ocl = fdiv(idc, a.div_rch);
-                    const int j   = idc - ocl * n_pairs;    // (tap, chunk) pair inside the row
-                    const int off = ic_off + (j & (a.CH - 1)) * 16;
-                    const bool ld = oc0 + ocl < g.OC && off < row_bytes;
-                    // output channel -> row of the MFMA operand (see the header comment)
-                    const int r32 = ocl & 31;
-                    const int row = (ocl & ~31) + ((r32 >> 2) & 3) * 8 + (r32 >> 4) * 4 + (r32 & 3);
-                    wdst[u]       = ok ? row * a.wstride + j * 16 : -1;
+                    const int j   = wj0 + u * LPR;    // (tap, chunk) pair inside the row
+                    const bool ok = j < n_pairs;
+                    const int jc  = ok ? j : 0;
+                    const int off = ic_off + (jc & (a.CH - 1)) * 16;
+                    const bool ld = ok && w_oc_ok && off < row_bytes;
+                    wdst[u]       = ok ? w_row * a.wstride + j * 16 : -1;
+                    const size_t src = w_src_row + (size_t)(jc >> ch_shift) * row_bytes + off;
                     if constexpr (VEC)
                     {
-                        const size_t src = ld ? ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes + off : 0;
-                        const v4i v      = *reinterpret_cast<const v4i*>(wbase_ptr + src);
-                        wv[u]            = ld ? v : v4i{ 0, 0, 0, 0 };
+                        const v4i v = *reinterpret_cast<const v4i*>(wbase_ptr + (ld ? src : 0));
+                        wv[u]       = ld ? v : v4i{ 0, 0, 0, 0 };
                     }
                     else
                     {
                         wv[u] = v4i{ 0, 0, 0, 0 };
-                        if (ok && ld)
-                            wv[u] = load_chunk_bytes(wbase_ptr + ((size_t)(oc0 + ocl) * taps + (j >> ch_shift)) * row_bytes,
-                                                     off, row_bytes);
+                        if (ld)
+                            wv[u] = load_chunk_bytes(wbase_ptr + w_src_row + (size_t)(jc >> ch_shift) * row_bytes, off,
+                                                     row_bytes);
                     }
                 }
 #pragma unroll
@@ -434,34 +446,32 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 for (int u = 0; u < WU; u++)
                     if (wdst[u] >= 0)
                         *reinterpret_cast<v4i*>(wl + wdst[u]) = wv[u];
+                // sum(w) of this lane's share of its weight row, taken while the chunks are in registers
+                if constexpr (M::is_int)
+                    if (a.za != 0)
+#pragma unroll
+                        for (int u = 0; u < WU; u++)
+                            w_sum += dot4_ones(wv[u]);
+                staged_w_sum = w_sum;
             }
         }
         __syncthreads();
 
         // ---- sum(w) per output channel, for the zero-point correction -----------------------------------------
-        // NT/OCB lanes share a weight row: each adds up the bytes of its chunks with v_dot4, a butterfly
-        // finishes the row, and -za*sum(w) goes straight into the channel table's bias (one LDS atomic per row,
-        // all rows distinct).  Doing this once per block keeps the K loop free of side computations.
+        // The NT/OCB lanes that share a weight row finish its byte sum with a butterfly and -za*sum(w) goes
+        // straight into the channel table's bias (one LDS atomic per row, all rows distinct; the table was
+        // written before the barrier above).  The K loop stays free of side computations.
         if constexpr (M::is_int)
         {
             if (a.za != 0)
             {
                 constexpr int LPR = NT / OCB;    // lanes per row: 8 or 16
-                const int row     = tid / LPR;   // row of the staged operand: tile*32 + 8q + 4h + j
-                const int part    = tid % LPR;
-                const uint8_t* rp = wl + row * a.wstride;
-                int sum           = 0;
-                for (int j = part; j < n_pairs; j += LPR)
-                    sum += dot4_ones(*reinterpret_cast<const v4i*>(rp + j * 16));
+                int sum           = staged_w_sum;
 #pragma unroll
                 for (int m = 1; m < LPR; m <<= 1)
                     sum += __shfl_xor(sum, m);
-                if (part == 0)
-                {
-                    const int r32 = row & 31;    // 8q + 4h + j  ->  channel 16h + 4q + j
-                    const int ch  = (row & ~31) + ((r32 >> 2) & 1) * 16 + (r32 >> 3) * 4 + (r32 & 3);
-                    atomicAdd(&ctab[ch].bias, -a.za * sum);
-                }
+                if ((tid % LPR) == 0)
+                    atomicAdd(&ctab[tid / LPR].bias, -a.za * sum);    // the lanes of row group r staged channel r
             }
         }
 
@@ -648,7 +658,53 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             __syncthreads();    // every wave is done reading the operands: LDS becomes the staging area
         int32_t* stage = reinterpret_cast<int32_t*>(lds + kCtab);    // [pixel of the tile][channel of the block]
 
-        // four channels at a time: fetch their constants once, use them for every pixel of the lane
+        // The common case -- RESCALE to int8, whole aligned 16-channel rows -- as straight-line code: about ten
+        // vector instructions per element and no branch; `checked` adds apply_scale_32's value-range test and
+        // is only taken when some channel's shift is below 32.
+        const bool fast_i8 = EPI == EPI_FAST && a.out_dtype == TMI_INT8 && vec16;
+        if constexpr (EPI == EPI_FAST)
+        {
+            if (fast_i8)
+            {
+                auto rows = [&](auto checked_tag) {
+                    constexpr bool CHECKED = decltype(checked_tag)::value;
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                    {
+                        ChanEntry ce[4];
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            ce[r] = ctab[ocl0 + 4 * q + r];
+#pragma unroll
+                        for (int i = 0; i < PXT; i++)
+                        {
+                            int32_t res[4];
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                            {
+                                const int32_t v = acc[i][4 * q + r] + pcorr[i] + ce[r].bias;
+                                if constexpr (CHECKED)
+                                    if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
+                                        flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
+                                const int64_t pr = (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
+                                int32_t o        = (int32_t)(pr >> ce[r].s);
+                                o                = o < a.rp.lo ? a.rp.lo : o;
+                                res[r]           = o > a.rp.hi ? a.rp.hi : o;
+                            }
+                            packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
+                                           ((res[3] & 0xff) << 24);
+                        }
+                    }
+                };
+                if (*need_check)
+                    rows(std::true_type{});
+                else
+                    rows(std::false_type{});
+            }
+        }
+
+        // every other combination: four channels at a time, constants fetched once and used for every pixel
+        if (!fast_i8)
 #pragma unroll
         for (int q = 0; q < 4; q++)
         {
@@ -674,7 +730,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                         if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
                             flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
                         const int64_t pr = (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                        v                = (int32_t)(pr >> ce[r].s) + a.rp.out_zp;
+                        v                = (int32_t)(pr >> ce[r].s);    // output_zp rides in the rounding term
                         v                = v < a.rp.lo ? a.rp.lo : v;
                         v                = v > a.rp.hi ? a.rp.hi : v;
                     }
@@ -828,7 +884,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
         TH = g.OH;
     if (TH < 1)
         TH = 1;
-    const size_t fixed_bytes = (size_t)OCB * 32 + 16 + ((((size_t)rch + 32) * 4 + 15) & ~(size_t)15);
+    const size_t fixed_bytes = (size_t)OCB * 32 + 32 + ((((size_t)rch + 32) * 4 + 15) & ~(size_t)15);
     const size_t w_bytes     = (size_t)OCB * a.wstride;
     size_t lds_bytes         = 0;
     for (;;)
