@@ -2,15 +2,22 @@
 // epilogue fused so that the int32 accumulators never reach HBM.
 //
 // One workgroup (8 waves) computes a TH x TW tile of output pixels of one image for a block of OCB =
-// 32*WOC output channels; wave w owns channel tile w / (8/WOC) and PXT pixel tiles of 32 pixels.  Two waves
-// per SIMD is what hides LDS and VALU latency here: the named shapes are far too small to fill the chip with
-// bigger per-wave tiles.  Per block of 64 bytes of input channels the workgroup stages in LDS
+// 32*OCT*WOC output channels.  The waves form a WOC x (8/WOC) grid; each owns OCT channel tiles and PXT pixel
+// tiles of 32, i.e. OCT*PXT accumulator tiles.  The small instantiations (one or two accumulator tiles per
+// wave) are for layers too small to fill the chip otherwise, the 2x2 one for GEMM-sized work, where it
+// halves the LDS traffic per MFMA.  Per block of CH*16 bytes of input channels the workgroup stages in LDS
 //   - the input patch that the tile needs (PH x PW pixels, out-of-image pixels filled with input_zp, so the
 //     zero-point identity below holds with the full K): one row of CH 16-byte chunks per pixel, and
 //   - the weight slab: one row per output channel holding its KH*KW*CH chunks in (tap, chunk) order, which
 //     is the order they have in HBM.
 // Every input byte is read from HBM/L2 once per workgroup (plus the halo) and reused KH*KW*OCB times
 // from LDS.
+//
+// When the input channels need more than one block and a block is at most WU weight chunks and PU patch
+// chunks per lane, the blocks are software pipelined: LDS holds two buffers, the global loads of block b+1
+// are issued before the MFMA loop of block b and written to the other buffer after it, and one barrier per
+// block remains.  Otherwise (single block, or blocks too large for the registers) a block is staged in
+// rounds into a single buffer.
 //
 // The MFMA is the 32x32 shape (v_mfma_i32_32x32x32_i8, v_mfma_f32_32x32x16_{f16,bf16}), which on this chip
 // runs at the full int8 rate while the 16x16x64 shape does not.  A fragment gives every lane 16 bytes: lane
@@ -24,14 +31,15 @@
 // consecutive channels of one pixel: its int8 results leave as one 16-byte store.
 //
 // A K-step feeds each lane 16 bytes of one (tap, chunk) pair; lane half h takes pair 2*step+h.  The K loop is
-// software pipelined three deep (fragments of step s+2 are requested before the MFMAs of step s issue) and a
-// dead pair (odd pair count) is read from a zeroed LDS chunk so that no instruction has to touch a fragment
-// between its load and its MFMA.  Integer dot
-// products are order independent, so the assignment of pairs to lanes is free as long as both operands
-// agree; the floating-point variants are compared against fp64 with the reference's DOT_PRODUCT bound.
+// double buffered in groups of G steps and a dead pair (odd pair count) is read from a zeroed LDS chunk so
+// that no instruction has to touch a fragment between its load and its MFMA.  Integer dot products are order
+// independent, so the assignment of pairs to lanes is free as long as both operands agree; the
+// floating-point variants are compared against fp64 with the reference's DOT_PRODUCT bound.
 //
-// Zero points: sum((a-za)(w-zw)) = sum(a*w) - zw*sum(a) - za*sum(w) + K*za*zw.  sum(w) per channel and
-// sum(a) per pixel are accumulated from the very fragments fed to the MFMA with v_dot4 against 0x01010101.
+// Zero points: sum((a-za)(w-zw)) = sum(a*w) - zw*sum(a) - za*sum(w) + K*za*zw.  sum(w) per channel is taken
+// with v_dot4 against 0x01010101 from the registers that stage the weights, sum(a) per pixel from the patch
+// chunks as they are staged (only when zw != 0; kept per patch pixel in LDS and summed over the window in
+// the epilogue).
 //
 // Epilogue: the per-channel constants (bias, multiplier, shift and the 64-bit rounding terms derived from
 // them) are computed once per workgroup by OCB lanes while the staging loads are in flight and kept in an
@@ -81,15 +89,20 @@ struct PatchArgs
     int32_t za, zw;
     int32_t TH, TW, tiles_y, tiles_x;
     int32_t PH, PW;
-    int32_t CH;                  // 16-byte chunks per pixel row in LDS (1, 2 or 4)
+    int32_t CH;                  // 16-byte chunks per pixel row in LDS (a power of two up to 16)
+    int32_t ch_shift;            // log2(CH)
     int32_t pstride, wstride;    // LDS row strides in bytes, both = 16 (mod 32)
     int32_t n_icb;               // blocks of CH*16 bytes along the input channels
     int32_t ksteps;              // MFMA K-steps per channel block = ceil(taps*CH/2)
     int32_t n_tiles;             // N * tiles_y * tiles_x
+    int32_t n_ocb;               // blocks of output channels
     int32_t out_dtype;
     int32_t xcd_remap;
+    int32_t rounds;              // staging rounds per channel block
+    int32_t pipelined;           // two LDS buffers, loads of the next block in flight during the MFMA loop
+    int32_t buf_bytes;           // size of one LDS operand buffer (weight rows + patch)
     int64_t w_batch_stride;    // bytes between the weights of consecutive images (0: shared; MATMUL: per batch)
-    FastDiv div_tw, div_pw, div_rch, div_tiles_x, div_tiles_y, div_n_tiles, div_kw;
+    FastDiv div_tw, div_pw, div_tiles_x, div_tiles_y, div_group, div_kw;
 };
 
 template <typename T>
@@ -215,46 +228,68 @@ struct alignas(16) ChanEntry
     int64_t rnd_pos, rnd_neg;
 };
 
-template <typename T, int WOC, int PXT, int EPI, bool VEC>
+// Per-lane chunk budget of one staging round (weights, patch) and K-loop group size of an instantiation.
+template <int OCT, int PXT>
+struct TileTraits
+{
+    static constexpr bool big = OCT * PXT >= 4;
+    static constexpr int WU   = 5;
+    static constexpr int PU   = big ? 8 : 2;
+    static constexpr int G    = big ? 1 : 3;
+};
+
+// Source descriptors of the staging: a byte offset below kFill is loaded, kFill is an out-of-image pixel
+// (filled with input_zp), kNone reads as zero.  Tensors this kernel takes are smaller than kFill bytes.
+static constexpr uint32_t kNone = 0xffffffffu;
+static constexpr uint32_t kFill = 0xfffffffeu;
+
+template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC>
 __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 {
     using M              = Mma<T>;
     using acc_t          = typename M::acc_t;
+    using TT             = TileTraits<OCT, PXT>;
     constexpr int EB     = sizeof(T);
-    constexpr int NT     = 512;          // lanes per workgroup
-    constexpr int WPX    = 8 / WOC;      // waves along the pixel dimension
-    constexpr int OCB    = 32 * WOC;     // output channels per workgroup
-    constexpr int WU     = 5;            // weight chunks in flight per lane in one staging round
-    constexpr int PU     = 2;            // patch chunks in flight per lane in one staging round
+    constexpr int NT     = 512;                // lanes per workgroup
+    constexpr int WPX    = 8 / WOC;            // waves along the pixel dimension
+    constexpr int OCB    = 32 * OCT * WOC;     // output channels per workgroup
+    constexpr int WU     = TT::WU;             // weight chunks in flight per lane in one staging round
+    constexpr int PU     = TT::PU;             // patch chunks in flight per lane in one staging round
+    constexpr int LPR    = NT / OCB;           // lanes that share a weight row while staging: 4, 8 or 16
     const ConvGeom& g    = a.g;
     const int tid        = threadIdx.x;
     const int lane       = tid & 63;
     // wave-uniform values are made scalar explicitly: with two waves per SIMD the vector ALU (4 cycles per
     // wave64 instruction) is the scarce resource, so everything uniform must run on the scalar unit
     const int wave       = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int woc        = wave / WPX;   // channel tile of this wave
+    const int woc        = wave / WPX;   // first channel tile of this wave is woc*OCT
     const int wpx        = wave % WPX;   // first pixel tile of this wave is wpx*PXT
     const int li         = lane & 31;    // row of the A fragment / column (pixel) of D
     const int lh         = lane >> 5;    // K half taken by this lane / row half of D
     const int taps       = g.KH * g.KW;
     const int row_bytes  = g.IC * EB;    // bytes of one pixel's (or one weight tap's) channel vector
     const int blk_bytes  = a.CH * 16;
-    const int ch_shift   = a.CH == 4 ? 2 : (a.CH == 2 ? 1 : 0);
+    const int ch_shift   = a.ch_shift;
     const int n_pairs    = taps * a.CH;  // (tap, chunk) pairs per channel block = chunks per weight row
     const int fill_word  = M::is_int ? (a.za & 0xff) * 0x01010101 : 0;    // out-of-image pixels hold input_zp
 
-    // LDS: [channel table][16 zero bytes][pair offset table][weight rows][input patch]
+    // LDS: [channel table][16 zero bytes][check words][1 KB dump area][pair offset table][patch byte sums]
+    // [buffer 0][buffer 1 when pipelined], a buffer being the weight rows followed by the input patch
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     ChanEntry* ctab        = reinterpret_cast<ChanEntry*>(lds);
     float* ftab            = reinterpret_cast<float*>(lds);    // floating point: bias as float
     constexpr int kCtab    = OCB * (int)sizeof(ChanEntry);
     uint8_t* zero_chunk    = lds + kCtab;
-    int* need_check        = reinterpret_cast<int*>(lds + kCtab + 16);    // set when some channel has shift < 32
-    int* pairoff           = reinterpret_cast<int*>(lds + kCtab + 32);
-    const int tab_entries  = n_pairs + 32;    // 2*(ksteps + 3G) + 1 < n_pairs + 32 for G = 3    // slack: the pipeline reads a few entries past the end
+    int* need_check        = reinterpret_cast<int*>(lds + kCtab + 16);    // two words, one per table wave
+    uint8_t* dump          = lds + kCtab + 32 + lane * 16;    // where staging work items without a destination write
+    constexpr int kFixed   = kCtab + 32 + 1024;
+    int* pairoff           = reinterpret_cast<int*>(lds + kFixed);
+    const int tab_entries  = n_pairs + 32;    // slack: the pipeline reads up to 4G + 1 < 32 entries past the end
     const int tab_bytes    = (tab_entries * 4 + 15) & ~15;
-    uint8_t* wl            = lds + kCtab + 32 + tab_bytes;
-    uint8_t* pl            = wl + OCB * a.wstride;
+    int* psum              = reinterpret_cast<int*>(lds + kFixed + tab_bytes);    // per patch pixel: sum of its bytes
+    const int psum_bytes   = M::is_int ? ((a.PH * a.PW * 4 + 15) & ~15) : 0;
+    uint8_t* buf0          = lds + kFixed + tab_bytes + psum_bytes;
+    const int w_bytes      = OCB * a.wstride;
 
     // ---- which tile ------------------------------------------------------------------------------------
     uint32_t bid = blockIdx.x;
@@ -265,8 +300,16 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         const uint32_t per = gridDim.x >> 3;
         bid                = (bid & 7) * per + (bid >> 3);
     }
-    const uint32_t ocb  = fdiv(bid, a.div_n_tiles);
-    uint32_t tile       = bid - ocb * a.n_tiles;
+    // Grouped order: a run of kGroup pixel tiles times all channel blocks, the pixel tile running fastest.
+    // The workgroups that are resident on an XCD together then share a few patches and a few weight blocks
+    // instead of one weight block and many patches, which is what keeps GEMM-sized operands in L2.
+    constexpr uint32_t kGroup = 4;
+    const uint32_t grp        = fdiv(bid, a.div_group);
+    const uint32_t first      = grp * kGroup;
+    const uint32_t in_grp     = bid - grp * kGroup * a.n_ocb;
+    const uint32_t rows       = a.n_tiles - first < kGroup ? a.n_tiles - first : kGroup;
+    const uint32_t ocb        = rows == kGroup ? in_grp / kGroup : in_grp / rows;
+    const uint32_t tile       = first + in_grp - ocb * rows;
     const uint32_t trow = fdiv(tile, a.div_tiles_x);
     const int txi       = tile - trow * a.tiles_x;
     const int n         = fdiv(trow, a.div_tiles_y);
@@ -277,7 +320,183 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const int y0        = oy0 * g.stride_y - g.pad_top;
     const int x0        = ox0 * g.stride_x - g.pad_left;
     const int P         = a.TH * a.TW;
-    const uint8_t* wbase_ptr = a.w + (size_t)n * a.w_batch_stride;
+    const uint8_t* w_n  = a.w + (size_t)n * a.w_batch_stride;                 // weights of this image
+    const uint8_t* in_n = a.in + (size_t)n * g.IH * g.IW * row_bytes;        // this image
+
+    // ---- per-lane pixel bases --------------------------------------------------------------------------
+    int pidx[PXT];    // patch pixel under tap (0, 0) of this lane's output pixel
+#pragma unroll
+    for (int i = 0; i < PXT; i++)
+    {
+        int p = (wpx * PXT + i) * 32 + li;
+        if (p >= P)
+            p = 0;
+        const int ty = fdiv(p, a.div_tw);
+        pidx[i]      = ty * g.stride_y * a.PW + (p - ty * a.TW) * g.stride_x;
+    }
+
+    acc_t acc[PXT][OCT];
+#pragma unroll
+    for (int i = 0; i < PXT; i++)
+#pragma unroll
+        for (int t = 0; t < OCT; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[i][t][r] = 0;
+    const bool wave_active = wpx * PXT * 32 < P;
+
+    // ---- staging ---------------------------------------------------------------------------------------
+    // A round moves up to WU weight chunks and PU patch chunks per lane: describe() works out where they come
+    // from and go to (independent of the channel block), issue() starts the global loads of one channel block
+    // and commit() writes them to an LDS buffer.  Nothing but the loads themselves hides memory latency inside
+    // a round, so all of a round's loads are issued before any is used; in the VEC instantiation (channel
+    // vectors are whole, aligned 16-byte chunks) they are unconditional: a work item without a source reads a
+    // clamped, valid address and its result is replaced in commit(), which keeps the round free of branches.
+    // Weight rows: LPR lanes share a row and walk its chunks, so no division is needed.
+    const int w_ocl        = tid / LPR;
+    const int w_part       = tid % LPR;
+    const int w_r32        = w_ocl & 31;    // output channel -> row of the MFMA operand (see the header comment)
+    const int w_row        = (w_ocl & ~31) + ((w_r32 >> 2) & 3) * 8 + (w_r32 >> 4) * 4 + (w_r32 & 3);
+    const bool w_oc_ok     = oc0 + w_ocl < g.OC;
+    const uint32_t w_src_row = (uint32_t)(oc0 + w_ocl) * (uint32_t)(taps * row_bytes);
+    const int p_total      = a.PH * a.PW * a.CH;
+    const int p_cc16       = (tid & (a.CH - 1)) * 16;    // NT is a multiple of CH: one chunk column per lane
+
+    uint32_t wsrc[WU], psrc[PU];
+    int wdst[WU], ppix[PU];
+    v4i wv[WU], pv[PU];
+
+    auto describe = [&](int round) {
+#pragma unroll
+        for (int u = 0; u < PU; u++)
+        {
+            const int idx  = tid + (round * PU + u) * NT;
+            const bool ok  = idx < p_total;
+            const int pix  = (ok ? idx : 0) >> ch_shift;
+            const int py   = fdiv(pix, a.div_pw);
+            const int px   = pix - py * a.PW;
+            const int iy = y0 + py, ix = x0 + px;
+            const bool img = iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW;
+            ppix[u]        = ok ? pix : -1;
+            psrc[u]        = !ok ? kNone : (img ? (uint32_t)(iy * g.IW + ix) * (uint32_t)row_bytes + (uint32_t)p_cc16 : kFill);
+        }
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            const int j   = w_part + (round * WU + u) * LPR;    // (tap, chunk) pair inside the row
+            const bool ok = j < n_pairs;
+            const int jc  = ok ? j : 0;
+            wdst[u]       = ok ? w_row * a.wstride + j * 16 : -1;
+            wsrc[u]       = (ok && w_oc_ok)
+                                ? w_src_row + (uint32_t)((jc >> ch_shift) * row_bytes + (jc & (a.CH - 1)) * 16)
+                                : kNone;
+        }
+    };
+    // chunk column (byte offset inside the channel block) of weight work item u of a round
+    auto w_cc16 = [&](int round, int u) { return ((w_part + (round * WU + u) * LPR) & (a.CH - 1)) * 16; };
+
+    auto issue = [&](int round, int ic_off) {
+#pragma unroll
+        for (int u = 0; u < PU; u++)
+        {
+            const bool in_row = ic_off + p_cc16 < row_bytes;
+            if constexpr (VEC)
+            {
+                const bool ld = psrc[u] < kFill && in_row;
+                pv[u]         = *reinterpret_cast<const v4i*>(in_n + (ld ? psrc[u] + (uint32_t)ic_off : 0u));
+            }
+            else
+            {
+                pv[u] = v4i{ 0, 0, 0, 0 };
+                if (psrc[u] < kFill)
+                    pv[u] = load_chunk_bytes(in_n + (psrc[u] - p_cc16), ic_off + p_cc16, row_bytes);
+                else if (psrc[u] == kFill)
+                    pv[u] = fill_chunk(ic_off + p_cc16, row_bytes, M::is_int ? a.za : 0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            const int cc16 = w_cc16(round, u);
+            if constexpr (VEC)
+            {
+                const bool ld = wsrc[u] != kNone && ic_off + cc16 < row_bytes;
+                wv[u]         = *reinterpret_cast<const v4i*>(w_n + (ld ? wsrc[u] + (uint32_t)ic_off : 0u));
+            }
+            else
+            {
+                wv[u] = v4i{ 0, 0, 0, 0 };
+                if (wsrc[u] != kNone)
+                    wv[u] = load_chunk_bytes(w_n + (wsrc[u] - cc16), ic_off + cc16, row_bytes);
+            }
+        }
+    };
+
+    // Writes a round to LDS.  Work items without a destination write to the dump area, so the round has no
+    // branch.  Returns the byte sum of the weight chunks written (for the zero-point correction); with a
+    // non-zero weight zero point the byte sum of every patch pixel is accumulated in psum as well: the CH
+    // lanes that hold a pixel's chunks add them up and the first of them owns the pixel's entry.
+    auto commit = [&](int round, int ic_off, uint8_t* wl, uint8_t* pl, bool first_block) {
+        int w_sum = 0;
+#pragma unroll
+        for (int u = 0; u < PU; u++)
+        {
+            v4i v = pv[u];
+            if constexpr (VEC)
+            {
+                const bool in_row = ic_off + p_cc16 < row_bytes;
+                const bool ld     = psrc[u] < kFill && in_row;
+                const int fw      = (psrc[u] == kFill && in_row) ? fill_word : 0;    // whole chunks only here
+                v                 = ld ? v : v4i{ fw, fw, fw, fw };
+            }
+            uint8_t* dst = ppix[u] >= 0 ? pl + ppix[u] * a.pstride + p_cc16 : dump;
+            *reinterpret_cast<v4i*>(dst) = v;
+            if constexpr (M::is_int)
+                if (a.zw != 0)
+                {
+                    int sum = dot4_ones(v);
+                    for (int m = 1; m < a.CH; m <<= 1)
+                        sum += __shfl_xor(sum, m);
+                    if (p_cc16 == 0 && ppix[u] >= 0)
+                        psum[ppix[u]] = first_block ? sum : psum[ppix[u]] + sum;
+                }
+        }
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            v4i v = wv[u];
+            if constexpr (VEC)
+            {
+                const bool ld = wsrc[u] != kNone && ic_off + w_cc16(round, u) < row_bytes;
+                v             = ld ? v : v4i{ 0, 0, 0, 0 };
+            }
+            uint8_t* dst = wdst[u] >= 0 ? wl + wdst[u] : dump;
+            *reinterpret_cast<v4i*>(dst) = v;
+            if constexpr (M::is_int)
+                if (a.za != 0)
+                    w_sum += dot4_ones(v);    // work items without a source hold zeros
+        }
+        return w_sum;
+    };
+
+    // The channel blocks are taken in an order rotated by the workgroup's position: workgroups that run side
+    // by side would otherwise all read the same 16*CH-byte column of every row at the same time, which lands
+    // on a fraction of the memory channels when the row length is a power of two.  (Integer sums do not depend
+    // on the order; the floating-point bound holds for any order.)
+    const int rot = a.n_icb > 1 ? (int)((tile + ocb) % (uint32_t)a.n_icb) : 0;
+    auto block_offset = [&](int icb) {
+        const int b = icb + rot;
+        return (b >= a.n_icb ? b - a.n_icb : b) * blk_bytes;
+    };
+
+    // With one round per block the first block's loads are started before anything else, so that the table
+    // set-up below (which has global loads of its own) runs in their shadow.
+    const bool one_round = a.rounds == 1;
+    if (one_round)
+    {
+        describe(0);
+        issue(0, block_offset(0));
+    }
 
     // ---- tables ----------------------------------------------------------------------------------------
     uint32_t flags = 0;
@@ -286,7 +505,11 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     // An odd pair count leaves the upper K half of the last step empty: the spare chunk behind every weight
     // row is zero, so that half contributes nothing whatever the pixel operand holds.
     if ((n_pairs & 1) && tid < OCB)
-        *reinterpret_cast<v4i*>(wl + tid * a.wstride + n_pairs * 16) = v4i{ 0, 0, 0, 0 };
+    {
+        *reinterpret_cast<v4i*>(buf0 + tid * a.wstride + n_pairs * 16) = v4i{ 0, 0, 0, 0 };
+        if (a.pipelined)
+            *reinterpret_cast<v4i*>(buf0 + a.buf_bytes + tid * a.wstride + n_pairs * 16) = v4i{ 0, 0, 0, 0 };
+    }
     for (int q = tid; q < tab_entries; q += NT)
     {
         int off = 0;
@@ -299,10 +522,10 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         }
         pairoff[q] = off;
     }
-    if (tid < OCB)
+    if (tid < 128)    // the first two waves; OCB <= 128
     {
         const int oc  = oc0 + tid;
-        const bool ok = oc < g.OC;
+        const bool ok = oc < g.OC && tid < OCB;
         if constexpr (M::is_int)
         {
             ChanEntry e;
@@ -318,162 +541,64 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
                 e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos + zp_term, e.rnd_neg = cs.rnd_neg + zp_term;
                 // a shift below 32 somewhere: apply_scale_32's value range can be violated and must be checked.
-                // All table lanes sit in wave 0, so one ballot decides and a single lane writes the word.
+                // One ballot per table wave; each wave's first lane writes that wave's word.
                 const int any_check = __any(cs.lim != 0x80000000u);
-                if (tid == 0)
-                    *need_check = any_check;
+                if (lane == 0)
+                    need_check[wave] = any_check;
             }
-            ctab[tid] = e;
+            if (tid < OCB)
+                ctab[tid] = e;
         }
-        else
+        else if (tid < OCB)
             ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : oc) : 0.0f;
     }
 
-    // ---- per-lane pixel bases --------------------------------------------------------------------------
-    int pbase[PXT];
-#pragma unroll
-    for (int i = 0; i < PXT; i++)
-    {
-        int p = (wpx * PXT + i) * 32 + li;
-        if (p >= P)
-            p = 0;
-        const int ty = fdiv(p, a.div_tw);
-        pbase[i]     = (ty * g.stride_y * a.PW + (p - ty * a.TW) * g.stride_x) * a.pstride;
-    }
-
-    acc_t acc[PXT];
-#pragma unroll
-    for (int i = 0; i < PXT; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[i][r] = 0;
-    int asum[PXT];
-#pragma unroll
-    for (int i = 0; i < PXT; i++)
-        asum[i] = 0;
-
-    const bool wave_active = wpx * PXT * 32 < P;
-
     for (int icb = 0; icb < a.n_icb; icb++)
     {
-        const int ic_off = icb * blk_bytes;
+        const int ic_off = block_offset(icb);
+        uint8_t* wl      = buf0 + ((a.pipelined && (icb & 1)) ? a.buf_bytes : 0);
+        uint8_t* pl      = wl + w_bytes;
         int staged_w_sum = 0;
-        if (icb)
-            __syncthreads();
-        // ---- stage the weight rows and the input patch ---------------------------------------------------
-        // Nothing hides memory latency here except the loads themselves: every round issues up to WU weight
-        // chunks and PU patch chunks per lane before any of them is written to LDS, so a round costs one trip
-        // to HBM/L2.  The 3x3 / 64-channel shape needs a single round.  In the VEC instantiation (channel
-        // vectors are whole, aligned 16-byte chunks) the loads are unconditional: out-of-range work items read
-        // a clamped, valid address and the result is replaced afterwards, which keeps the round free of
-        // branches so that its loads really are in flight together.
+        if (a.pipelined)
         {
-            // weight rows: NT/OCB lanes share a row and walk its chunks, so no division is needed
-            constexpr int LPR = NT / OCB;
-            const int w_ocl   = tid / LPR;
-            const int w_part  = tid % LPR;
-            const int w_r32   = w_ocl & 31;    // output channel -> row of the MFMA operand (see the header comment)
-            const int w_row   = (w_ocl & ~31) + ((w_r32 >> 2) & 3) * 8 + (w_r32 >> 4) * 4 + (w_r32 & 3);
-            const bool w_oc_ok = oc0 + w_ocl < g.OC;
-            const size_t w_src_row = (size_t)(oc0 + w_ocl) * taps * row_bytes;
-            int w_sum = 0;
-            const int p_total = a.PH * a.PW * a.CH;
-            for (int wj0 = w_part, pbase_idx = tid; wj0 < n_pairs || pbase_idx < p_total;
-                 wj0 += LPR * WU, pbase_idx += NT * PU)
+            // this block's chunks were requested one block ago; its buffer was last read two blocks ago, and
+            // every wave has passed a barrier since
+            staged_w_sum = commit(0, ic_off, wl, pl, icb == 0);
+        }
+        else
+        {
+            if (icb)
+                __syncthreads();    // every wave is done reading the buffer
+            for (int round = 0; round < a.rounds; round++)
             {
-                v4i wv[WU], pv[PU];
-                int wdst[WU], pdst[PU];
-#pragma unroll
-                for (int u = 0; u < PU; u++)
-                {
-                    const int idx  = pbase_idx + u * NT;
-                    const bool ok  = idx < p_total;
-                    const int idc  = ok ? idx : 0;
-                    const int cc   = idc & (a.CH - 1);
-                    const int pix  = idc >> ch_shift;
-                    const int py   = fdiv(pix, a.div_pw);
-                    const int px   = pix - py * a.PW;
-                    const int iy = y0 + py, ix = x0 + px;
-                    const int off  = ic_off + cc * 16;
-                    const bool img = iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW;
-                    pdst[u]        = ok ? pix * a.pstride + cc * 16 : -1;
-                    if constexpr (VEC)
-                    {
-                        const bool ld    = img && off < row_bytes;
-                        const size_t src = ld ? (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes + off : 0;
-                        const v4i v      = *reinterpret_cast<const v4i*>(a.in + src);
-                        const int fw     = off < row_bytes ? fill_word : 0;    // whole chunks only in this path
-                        const v4i f      = v4i{ fw, fw, fw, fw };
-                        pv[u]            = ld ? v : (img ? v4i{ 0, 0, 0, 0 } : f);
-                    }
-                    else
-                    {
-                        pv[u] = v4i{ 0, 0, 0, 0 };
-                        if (ok)
-                            pv[u] = img ? load_chunk_bytes(a.in + (((size_t)n * g.IH + iy) * g.IW + ix) * row_bytes,
-                                                           off, row_bytes)
-                                        : fill_chunk(off, row_bytes, M::is_int ? a.za : 0);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < WU; u++)
-                {
-                    const int j   = wj0 + u * LPR;    // (tap, chunk) pair inside the row
-                    const bool ok = j < n_pairs;
-                    const int jc  = ok ? j : 0;
-                    const int off = ic_off + (jc & (a.CH - 1)) * 16;
-                    const bool ld = ok && w_oc_ok && off < row_bytes;
-                    wdst[u]       = ok ? w_row * a.wstride + j * 16 : -1;
-                    const size_t src = w_src_row + (size_t)(jc >> ch_shift) * row_bytes + off;
-                    if constexpr (VEC)
-                    {
-                        const v4i v = *reinterpret_cast<const v4i*>(wbase_ptr + (ld ? src : 0));
-                        wv[u]       = ld ? v : v4i{ 0, 0, 0, 0 };
-                    }
-                    else
-                    {
-                        wv[u] = v4i{ 0, 0, 0, 0 };
-                        if (ld)
-                            wv[u] = load_chunk_bytes(wbase_ptr + w_src_row + (size_t)(jc >> ch_shift) * row_bytes, off,
-                                                     row_bytes);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < PU; u++)
-                    if (pdst[u] >= 0)
-                        *reinterpret_cast<v4i*>(pl + pdst[u]) = pv[u];
-#pragma unroll
-                for (int u = 0; u < WU; u++)
-                    if (wdst[u] >= 0)
-                        *reinterpret_cast<v4i*>(wl + wdst[u]) = wv[u];
-                // sum(w) of this lane's share of its weight row, taken while the chunks are in registers
-                if constexpr (M::is_int)
-                    if (a.za != 0)
-#pragma unroll
-                        for (int u = 0; u < WU; u++)
-                            w_sum += dot4_ones(wv[u]);
-                staged_w_sum = w_sum;
+                if (!one_round)
+                    describe(round);
+                if (!one_round || icb)
+                    issue(round, ic_off);
+                staged_w_sum += commit(round, ic_off, wl, pl, icb == 0);
             }
         }
         __syncthreads();
 
         // ---- sum(w) per output channel, for the zero-point correction -----------------------------------------
-        // The NT/OCB lanes that share a weight row finish its byte sum with a butterfly and -za*sum(w) goes
+        // The LPR lanes that share a weight row finish its byte sum with a butterfly and -za*sum(w) goes
         // straight into the channel table's bias (one LDS atomic per row, all rows distinct; the table was
         // written before the barrier above).  The K loop stays free of side computations.
         if constexpr (M::is_int)
         {
             if (a.za != 0)
             {
-                constexpr int LPR = NT / OCB;    // lanes per row: 8 or 16
-                int sum           = staged_w_sum;
+                int sum = staged_w_sum;
 #pragma unroll
                 for (int m = 1; m < LPR; m <<= 1)
                     sum += __shfl_xor(sum, m);
-                if ((tid % LPR) == 0)
-                    atomicAdd(&ctab[tid / LPR].bias, -a.za * sum);    // the lanes of row group r staged channel r
+                if (w_part == 0)
+                    atomicAdd(&ctab[w_ocl].bias, -a.za * sum);
             }
         }
+
+        if (a.pipelined && icb + 1 < a.n_icb)
+            issue(0, block_offset(icb + 1));
 
         // ---- MFMA over the (tap, chunk) pairs of this channel block -----------------------------------
         if (wave_active)
@@ -483,85 +608,79 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             // group's MFMAs issue, so the wait in front of an MFMA only meets loads that have had a whole
             // group of matrix instructions to complete.  The main loop runs on whole pairs of groups and has no
             // branch in its body; what is left (fewer than 2G steps) goes through the checked tail.  Loads past
-            // the last step are clamped to it and never used.
-            constexpr int G     = 3;
-            const uint8_t* wrow = wl + (woc * 32 + li) * a.wstride + lh * 16;
+            // the last step are clamped to it and never used.  Nothing but loads and MFMAs is in the loop: the
+            // zero-point sums are taken while staging.
+            constexpr int G     = TT::G;
+            const uint8_t* wrow = wl + (woc * OCT * 32 + li) * a.wstride + lh * 16;
             const int* tab      = pairoff + lh;
             const int last_step = a.ksteps - 1;
-            v4i fa[2][G], fb[2][G][PXT];
+            const int wtile     = 32 * a.wstride;
+            const uint8_t* prow[PXT];
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+                prow[i] = pl + pidx[i] * a.pstride;
+            v4i fa[2][G][OCT], fb[2][G][PXT];
             int po[G];
-            auto load_group = [&](int s0, v4i(&ga)[G], v4i(&gb)[G][PXT]) {
+            auto load_group = [&](int s0, v4i(&ga)[G][OCT], v4i(&gb)[G][PXT]) {
 #pragma unroll
                 for (int u = 0; u < G; u++)
                 {
                     const int sc = s0 + u < last_step ? s0 + u : last_step;
-                    ga[u]        = *reinterpret_cast<const v4i*>(wrow + sc * 32);
+#pragma unroll
+                    for (int t = 0; t < OCT; t++)
+                        ga[u][t] = *reinterpret_cast<const v4i*>(wrow + t * wtile + sc * 32);
 #pragma unroll
                     for (int i = 0; i < PXT; i++)
-                        gb[u][i] = *reinterpret_cast<const v4i*>(pl + pbase[i] + po[u]);
+                        gb[u][i] = *reinterpret_cast<const v4i*>(prow[i] + po[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < G; u++)
                     po[u] = tab[2 * (s0 + G + u)];    // offsets of the group after that one
             };
-            // ZW: the weight zero point is non-zero, so sum(a) per pixel is needed as well; it is accumulated
-            // from the pixel fragments here (the upper K half of an odd last step holds no pair)
-            auto run = [&](auto zw_tag) {
-                constexpr bool ZW = decltype(zw_tag)::value;
-                auto compute = [&](int s, const v4i& ga, const v4i(&gb)[PXT]) {
+            auto compute = [&](const v4i(&ga)[OCT], const v4i(&gb)[PXT]) {
 #pragma unroll
-                    for (int i = 0; i < PXT; i++)
-                        acc[i] = M::mma(ga, gb[i], acc[i]);
-                    if constexpr (ZW)
-                    {
-                        const bool live = 2 * s + lh < n_pairs;
+                for (int i = 0; i < PXT; i++)
 #pragma unroll
-                        for (int i = 0; i < PXT; i++)
-                            asum[i] += live ? dot4_ones(gb[i]) : 0;
-                    }
-                };
+                    for (int t = 0; t < OCT; t++)
+                        acc[i][t] = M::mma(ga[t], gb[i], acc[i][t]);
+            };
+#pragma unroll
+            for (int u = 0; u < G; u++)
+                po[u] = tab[2 * u];
+            load_group(0, fa[0], fb[0]);
+            int s = 0;
+            for (; s + 2 * G <= a.ksteps; s += 2 * G)
+            {
+                load_group(s + G, fa[1], fb[1]);
 #pragma unroll
                 for (int u = 0; u < G; u++)
-                    po[u] = tab[2 * u];
-                load_group(0, fa[0], fb[0]);
-                int s = 0;
-                for (; s + 2 * G <= a.ksteps; s += 2 * G)
-                {
-                    load_group(s + G, fa[1], fb[1]);
+                    compute(fa[0][u], fb[0][u]);
+                load_group(s + 2 * G, fa[0], fb[0]);
 #pragma unroll
-                    for (int u = 0; u < G; u++)
-                        compute(s + u, fa[0][u], fb[0][u]);
-                    load_group(s + 2 * G, fa[0], fb[0]);
+                for (int u = 0; u < G; u++)
+                    compute(fa[1][u], fb[1][u]);
+            }
+            if (s < a.ksteps)
+            {
+                load_group(s + G, fa[1], fb[1]);
 #pragma unroll
-                    for (int u = 0; u < G; u++)
-                        compute(s + G + u, fa[1][u], fb[1][u]);
-                }
-                if (s < a.ksteps)
-                {
-                    load_group(s + G, fa[1], fb[1]);
+                for (int u = 0; u < G; u++)
+                    if (s + u < a.ksteps)
+                        compute(fa[0][u], fb[0][u]);
 #pragma unroll
-                    for (int u = 0; u < G; u++)
-                        if (s + u < a.ksteps)
-                            compute(s + u, fa[0][u], fb[0][u]);
-#pragma unroll
-                    for (int u = 0; u < G; u++)
-                        if (s + G + u < a.ksteps)
-                            compute(s + G + u, fa[1][u], fb[1][u]);
-                }
-            };
-            if (M::is_int && a.zw != 0)
-                run(std::true_type{});
-            else
-                run(std::false_type{});
+                for (int u = 0; u < G; u++)
+                    if (s + G + u < a.ksteps)
+                        compute(fa[1][u], fb[1][u]);
+            }
         }
     }
 
     // ---- epilogue -------------------------------------------------------------------------------------
-    // per pixel tile: validity and output offset of this lane's pixel; the lane owns channels
-    // [ocl0, ocl0 + 16) of the block
+    // per pixel tile: validity and output offset of this lane's pixel; in channel tile t the lane owns
+    // channels [ocl0 + 32t, ocl0 + 32t + 16) of the block
     bool pix_ok[PXT];
     size_t obase[PXT];
-    const int ocl0 = woc * 32 + 16 * lh;
+    const int ocl0 = woc * OCT * 32 + 16 * lh;
 #pragma unroll
     for (int i = 0; i < PXT; i++)
     {
@@ -571,225 +690,240 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         pix_ok[i]    = wave_active && p < P && oy < g.OH && ox < g.OW;
         obase[i]     = (((size_t)n * g.OH + oy) * g.OW + ox) * g.OC + oc0 + ocl0;
     }
-    const bool full = (oc0 + ocl0 + 16 <= g.OC);
 
     if constexpr (!M::is_int)
     {
         // floating point: out = bias + acc, rounded to the output type (16 channels = 32 bytes per pixel), or
         // kept in fp32 (MATMUL: 64 bytes per pixel)
-        const bool vec_out = full && (g.OC & 7) == 0 && ((uintptr_t)a.out & 15) == 0;
 #pragma unroll
-        for (int i = 0; i < PXT; i++)
+        for (int t = 0; t < OCT; t++)
         {
-            if (a.out_dtype == TMI_FP32)
+            const int oclt     = ocl0 + 32 * t;
+            const bool full    = (oc0 + oclt + 16 <= g.OC);
+            const bool vec_out = full && (g.OC & 7) == 0 && ((uintptr_t)a.out & 15) == 0;
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
             {
-                float* o = reinterpret_cast<float*>(a.out) + obase[i];
+                if (a.out_dtype == TMI_FP32)
+                {
+                    float* o = reinterpret_cast<float*>(a.out) + obase[i] + 32 * t;
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                    {
+                        const v4f b = *reinterpret_cast<const v4f*>(ftab + oclt + 4 * q);
+                        v4f r;
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            r[j] = b[j] + acc[i][t][4 * q + j];
+                        if (!pix_ok[i])
+                            continue;
+                        if (vec_out)
+                            *reinterpret_cast<v4f*>(o + 4 * q) = r;
+                        else
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+                                if (oc0 + oclt + 4 * q + j < g.OC)
+                                    o[4 * q + j] = r[j];
+                    }
+                    continue;
+                }
+                union
+                {
+                    v4i v[2];
+                    T e[16];
+                } u;
 #pragma unroll
                 for (int q = 0; q < 4; q++)
                 {
-                    const v4f b = *reinterpret_cast<const v4f*>(ftab + ocl0 + 4 * q);
-                    v4f r;
+                    const v4f b = *reinterpret_cast<const v4f*>(ftab + oclt + 4 * q);
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        r[j] = b[j] + acc[i][4 * q + j];
-                    if (!pix_ok[i])
-                        continue;
-                    if (vec_out)
-                        *reinterpret_cast<v4f*>(o + 4 * q) = r;
-                    else
-#pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            if (oc0 + ocl0 + 4 * q + j < g.OC)
-                                o[4 * q + j] = r[j];
+                    for (int r = 0; r < 4; r++)
+                        store_from_float(&u.e[4 * q + r], b[r] + acc[i][t][4 * q + r]);
                 }
-                continue;
-            }
-            union
-            {
-                v4i v[2];
-                T e[16];
-            } u;
+                if (!pix_ok[i])
+                    continue;
+                T* o = reinterpret_cast<T*>(a.out) + obase[i] + 32 * t;
+                if (vec_out)
+                {
+                    reinterpret_cast<v4i*>(o)[0] = u.v[0];
+                    reinterpret_cast<v4i*>(o)[1] = u.v[1];
+                }
+                else
+                {
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-            {
-                const v4f b = *reinterpret_cast<const v4f*>(ftab + ocl0 + 4 * q);
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    store_from_float(&u.e[4 * q + r], b[r] + acc[i][4 * q + r]);
-            }
-            if (!pix_ok[i])
-                continue;
-            T* o = reinterpret_cast<T*>(a.out) + obase[i];
-            if (vec_out)
-            {
-                reinterpret_cast<v4i*>(o)[0] = u.v[0];
-                reinterpret_cast<v4i*>(o)[1] = u.v[1];
-            }
-            else
-            {
-#pragma unroll
-                for (int j = 0; j < 16; j++)
-                    if (oc0 + ocl0 + j < g.OC)
-                        o[j] = u.e[j];
+                    for (int j = 0; j < 16; j++)
+                        if (oc0 + oclt + j < g.OC)
+                            o[j] = u.e[j];
+                }
             }
         }
     }
     else
     {
         const int kzz = g.KH * g.KW * g.IC * a.za * a.zw;
-        int pcorr[PXT];    // the zero-point terms that depend on the pixel only
+        int pcorr[PXT];    // the zero-point terms that depend on the pixel only: K*za*zw - zw*sum(a)
 #pragma unroll
         for (int i = 0; i < PXT; i++)
         {
-            int sa = asum[i];
-            if (a.zw != 0)
-                sa += __shfl_xor(sa, 32);
+            int sa = 0;
+            if (a.zw != 0)    // sum(a) over the window of this pixel from the per-pixel byte sums (complete since the
+                              // barrier that followed the last block's staging)
+                for (int ky = 0; ky < g.KH; ky++)
+                    for (int kx = 0; kx < g.KW; kx++)
+                        sa += psum[pidx[i] + ky * g.dil_y * a.PW + kx * g.dil_x];
             pcorr[i] = kzz - a.zw * sa;
         }
         // -za*sum(w) was added to the channel table's bias after staging: make it visible to every wave
         if (a.za != 0)
             __syncthreads();
-        // int32 rows of four channels can be stored as one vector; int8 rows of 16 channels likewise
-        const bool vec4  = full && (g.OC & 3) == 0 && ((uintptr_t)a.out & 15) == 0;
-        const bool vec16 = full && (g.OC & 15) == 0 && ((uintptr_t)a.out & 15) == 0;
-        int packed[PXT][4];    // int8 results, four channels per word
-
         if constexpr (EPI == EPI_GENERIC)
             __syncthreads();    // every wave is done reading the operands: LDS becomes the staging area
         int32_t* stage = reinterpret_cast<int32_t*>(lds + kCtab);    // [pixel of the tile][channel of the block]
-
-        // The common case -- RESCALE to int8, whole aligned 16-channel rows -- as straight-line code: about ten
-        // vector instructions per element and no branch; `checked` adds apply_scale_32's value-range test and
-        // is only taken when some channel's shift is below 32.
-        const bool fast_i8 = EPI == EPI_FAST && a.out_dtype == TMI_INT8 && vec16;
+        bool check     = false;
         if constexpr (EPI == EPI_FAST)
+            check = (need_check[0] | need_check[1]) != 0;
+
+#pragma unroll
+        for (int t = 0; t < OCT; t++)
         {
-            if (fast_i8)
+            const int oclt  = ocl0 + 32 * t;
+            const bool full = (oc0 + oclt + 16 <= g.OC);
+            // int32 rows of four channels can be stored as one vector; int8 rows of 16 channels likewise
+            const bool vec4  = full && (g.OC & 3) == 0 && ((uintptr_t)a.out & 15) == 0;
+            const bool vec16 = full && (g.OC & 15) == 0 && ((uintptr_t)a.out & 15) == 0;
+            int packed[PXT][4];    // int8 results, four channels per word
+
+            // The common case -- RESCALE to int8, whole aligned 16-channel rows -- as straight-line code: about
+            // ten vector instructions per element and no branch; `checked` adds apply_scale_32's value-range
+            // test and is only taken when some channel's shift is below 32.
+            const bool fast_i8 = EPI == EPI_FAST && a.out_dtype == TMI_INT8 && vec16;
+            if constexpr (EPI == EPI_FAST)
             {
-                auto rows = [&](auto checked_tag) {
-                    constexpr bool CHECKED = decltype(checked_tag)::value;
+                if (fast_i8)
+                {
+                    auto rows = [&](auto checked_tag) {
+                        constexpr bool CHECKED = decltype(checked_tag)::value;
 #pragma unroll
-                    for (int q = 0; q < 4; q++)
-                    {
-                        ChanEntry ce[4];
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            ce[r] = ctab[ocl0 + 4 * q + r];
-#pragma unroll
-                        for (int i = 0; i < PXT; i++)
+                        for (int q = 0; q < 4; q++)
                         {
-                            int32_t res[4];
+                            ChanEntry ce[4];
 #pragma unroll
                             for (int r = 0; r < 4; r++)
+                                ce[r] = ctab[oclt + 4 * q + r];
+#pragma unroll
+                            for (int i = 0; i < PXT; i++)
                             {
-                                const int32_t v = acc[i][4 * q + r] + pcorr[i] + ce[r].bias;
-                                if constexpr (CHECKED)
-                                    if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
-                                        flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
-                                const int64_t pr = (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                                int32_t o        = (int32_t)(pr >> ce[r].s);
-                                o                = o < a.rp.lo ? a.rp.lo : o;
-                                res[r]           = o > a.rp.hi ? a.rp.hi : o;
+                                int32_t res[4];
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                {
+                                    const int32_t v = acc[i][t][4 * q + r] + pcorr[i] + ce[r].bias;
+                                    if constexpr (CHECKED)
+                                        if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
+                                            flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
+                                    const int64_t pr =
+                                        (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
+                                    int32_t o = (int32_t)(pr >> ce[r].s);
+                                    o         = o < a.rp.lo ? a.rp.lo : o;
+                                    res[r]    = o > a.rp.hi ? a.rp.hi : o;
+                                }
+                                packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
+                                               ((res[3] & 0xff) << 24);
                             }
-                            packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
-                                           ((res[3] & 0xff) << 24);
                         }
-                    }
-                };
-                if (*need_check)
-                    rows(std::true_type{});
-                else
-                    rows(std::false_type{});
+                    };
+                    if (check)
+                        rows(std::true_type{});
+                    else
+                        rows(std::false_type{});
+                }
             }
-        }
 
-        // every other combination: four channels at a time, constants fetched once and used for every pixel
-        if (!fast_i8)
+            // every other combination: four channels at a time, constants fetched once and used for every pixel
+            if (!fast_i8)
 #pragma unroll
-        for (int q = 0; q < 4; q++)
-        {
-            const int c0 = oc0 + ocl0 + 4 * q;
-            ChanEntry ce[4];
-            int32_t cb[4];    // bias minus za * sum(w)
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-            {
-                ce[r] = ctab[ocl0 + 4 * q + r];
-                cb[r] = ce[r].bias;
-            }
-#pragma unroll
-            for (int i = 0; i < PXT; i++)
-            {
-                int32_t res[4];
-#pragma unroll
-                for (int r = 0; r < 4; r++)
+                for (int q = 0; q < 4; q++)
                 {
-                    int32_t v = acc[i][4 * q + r] + pcorr[i] + cb[r];
-                    if constexpr (EPI == EPI_FAST)
-                    {
-                        if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
-                            flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
-                        const int64_t pr = (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                        v                = (int32_t)(pr >> ce[r].s);    // output_zp rides in the rounding term
-                        v                = v < a.rp.lo ? a.rp.lo : v;
-                        v                = v > a.rp.hi ? a.rp.hi : v;
-                    }
-                    res[r] = v;
-                }
-                if constexpr (EPI == EPI_GENERIC)
-                {
-                    const int p = (wpx * PXT + i) * 32 + li;
-                    if (wave_active && p < P)
-                        *reinterpret_cast<v4i*>(stage + (size_t)p * OCB + ocl0 + 4 * q) =
-                            v4i{ res[0], res[1], res[2], res[3] };
-                    continue;
-                }
-                if (!pix_ok[i])
-                    continue;
-                if (EPI == EPI_PLAIN || a.out_dtype == TMI_INT32)
-                {
-                    int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase[i] + 4 * q;
-                    if (vec4)
-                        *reinterpret_cast<v4i*>(o) = v4i{ res[0], res[1], res[2], res[3] };
-                    else
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (c0 + r < g.OC)
-                                o[r] = res[r];
-                }
-                else if (a.out_dtype == TMI_INT8)
-                {
-                    if (vec16)
-                        packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
-                                       ((res[3] & 0xff) << 24);
-                    else
-                    {
-                        int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i] + 4 * q;
-#pragma unroll
-                        for (int r = 0; r < 4; r++)
-                            if (c0 + r < g.OC)
-                                o[r] = (int8_t)res[r];
-                    }
-                }
-                else
-                {
-                    int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase[i] + 4 * q;
+                    const int c0 = oc0 + oclt + 4 * q;
+                    ChanEntry ce[4];
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        if (c0 + r < g.OC)
-                            o[r] = (int16_t)res[r];
-                }
-            }
-        }
-        if constexpr (EPI == EPI_FAST)
-        {
-            if (a.out_dtype == TMI_INT8 && vec16)
-            {
+                        ce[r] = ctab[oclt + 4 * q + r];
 #pragma unroll
-                for (int i = 0; i < PXT; i++)
-                    if (pix_ok[i])
-                        *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + obase[i]) =
-                            v4i{ packed[i][0], packed[i][1], packed[i][2], packed[i][3] };
+                    for (int i = 0; i < PXT; i++)
+                    {
+                        int32_t res[4];
+#pragma unroll
+                        for (int r = 0; r < 4; r++)
+                        {
+                            int32_t v = acc[i][t][4 * q + r] + pcorr[i] + ce[r].bias;    // bias minus za*sum(w)
+                            if constexpr (EPI == EPI_FAST)
+                            {
+                                if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
+                                    flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
+                                const int64_t pr =
+                                    (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
+                                v = (int32_t)(pr >> ce[r].s);    // output_zp rides in the rounding term
+                                v = v < a.rp.lo ? a.rp.lo : v;
+                                v = v > a.rp.hi ? a.rp.hi : v;
+                            }
+                            res[r] = v;
+                        }
+                        if constexpr (EPI == EPI_GENERIC)
+                        {
+                            const int p = (wpx * PXT + i) * 32 + li;
+                            if (wave_active && p < P)
+                                *reinterpret_cast<v4i*>(stage + (size_t)p * OCB + oclt + 4 * q) =
+                                    v4i{ res[0], res[1], res[2], res[3] };
+                            continue;
+                        }
+                        if (!pix_ok[i])
+                            continue;
+                        if (EPI == EPI_PLAIN || a.out_dtype == TMI_INT32)
+                        {
+                            int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase[i] + 32 * t + 4 * q;
+                            if (vec4)
+                                *reinterpret_cast<v4i*>(o) = v4i{ res[0], res[1], res[2], res[3] };
+                            else
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                    if (c0 + r < g.OC)
+                                        o[r] = res[r];
+                        }
+                        else if (a.out_dtype == TMI_INT8)
+                        {
+                            if (vec16)
+                                packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
+                                               ((res[3] & 0xff) << 24);
+                            else
+                            {
+                                int8_t* o = reinterpret_cast<int8_t*>(a.out) + obase[i] + 32 * t + 4 * q;
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                    if (c0 + r < g.OC)
+                                        o[r] = (int8_t)res[r];
+                            }
+                        }
+                        else
+                        {
+                            int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase[i] + 32 * t + 4 * q;
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                if (c0 + r < g.OC)
+                                    o[r] = (int16_t)res[r];
+                        }
+                    }
+                }
+            if constexpr (EPI == EPI_FAST)
+            {
+                if (a.out_dtype == TMI_INT8 && vec16)
+                {
+#pragma unroll
+                    for (int i = 0; i < PXT; i++)
+                        if (pix_ok[i])
+                            *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + obase[i] + 32 * t) =
+                                v4i{ packed[i][0], packed[i][1], packed[i][2], packed[i][3] };
+                }
             }
         }
         if constexpr (EPI == EPI_GENERIC)
@@ -827,10 +961,10 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 
 static constexpr int kMaxLds = 160 * 1024;
 
-template <typename T, int WOC, int PXT, int EPI, bool VEC>
+template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC>
 static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blocks)
 {
-    auto kern                = conv2d_patch_kernel<T, WOC, PXT, EPI, VEC>;
+    auto kern                = conv2d_patch_kernel<T, WOC, OCT, PXT, EPI, VEC>;
     static size_t configured = 0;    // largest dynamic LDS size this instantiation was configured for
     if (lds_bytes > configured)
     {
@@ -841,6 +975,11 @@ static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blo
     }
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
     return true;
+}
+
+static int ceil_div(int a, int b)
+{
+    return (a + b - 1) / b;
 }
 
 template <typename T>
@@ -854,53 +993,113 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     const int64_t n_px  = (int64_t)g.N * g.OH * g.OW;
     if (row_bytes <= 0 || g.OC <= 0 || n_px == 0)
         return nullptr;
+    const int taps = g.KH * g.KW;
+    // the staging addresses one image and one image's weights with 32-bit byte offsets
+    if ((int64_t)g.IH * g.IW * row_bytes >= 0xfffffff0ll || (int64_t)g.OC * taps * row_bytes >= 0xfffffff0ll)
+        return nullptr;
 
     PatchArgs a{};
     a.g = g, a.in = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = bias, a.out = out;
     a.flag_word = flag_word, a.rp = rp, a.za = in_zp, a.zw = w_zp, a.out_dtype = out_dtype;
     a.w_batch_stride = w_batch_stride;
-    a.CH           = row_bytes <= 16 ? 1 : (row_bytes <= 32 ? 2 : 4);
-    a.pstride      = a.CH == 1 ? 16 : a.CH * 16 + 16;    // 16, 48, 80: all = 16 (mod 32)
-    a.n_icb        = (row_bytes + a.CH * 16 - 1) / (a.CH * 16);
-    const int taps = g.KH * g.KW;
-    const int rch  = taps * a.CH;    // chunks per weight row
-    a.wstride      = (rch + (rch & 1)) * 16 + 16;    // room for a spare zero chunk; = 16 (mod 32)
-    a.ksteps       = (rch + 1) / 2;
-
-    const int WOC           = g.OC > 32 ? 2 : 1;
-    const int OCB           = 32 * WOC;
-    const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
 
     // channel vectors made of whole, aligned 16-byte chunks take the branch-free staging path
     const bool vec = (row_bytes & 15) == 0 && (((uintptr_t)in | (uintptr_t)w) & 15) == 0;
-    // Pixel tiles per wave: two when that still leaves at least two workgroups per CU, else one.
-    const int max_px1 = 32 * (8 / WOC);
-    const int PXT     = (vec && n_px * oc_blocks >= (int64_t)256 * 2 * 2 * max_px1) ? 2 : 1;
-    const int max_px  = max_px1 * PXT;
-    // tile: prefer full output rows
+
+    // ---- workgroup shape: WOC x OCT channel tiles, PXT pixel tiles per wave -------------------------------
+    // The 128-channel x 256-pixel shape when that still gives every CU a workgroup; else 64 (or 32) channels
+    // with two pixel tiles per wave when that leaves two workgroups per CU; else the smallest.
+    int WOC = g.OC > 32 ? 2 : 1, OCT = 1, PXT = 1;
+    if (vec && g.OC > 64 && n_px * ((g.OC + 127) / 128) >= (int64_t)256 * 256)
+        OCT = 2, PXT = 2;
+    else if (vec && n_px * ((g.OC + 32 * WOC - 1) / (32 * WOC)) >= (int64_t)256 * 2 * 2 * 32 * (8 / WOC))
+        PXT = 2;
+    const int OCB           = 32 * OCT * WOC;
+    const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
+    const int max_px        = 32 * (8 / WOC) * PXT;
+    const int WU = 5, PU = (OCT * PXT >= 4) ? 8 : 2;    // the values of TileTraits<OCT, PXT>
+    const int LPR = 512 / OCB;
+
+    // ---- pixel tile: full output rows when they fit, and rows spread evenly over the tiles ------------------
     int TW = g.OW < max_px ? g.OW : max_px;
+    TW     = ceil_div(g.OW, ceil_div(g.OW, TW));
     int TH = max_px / TW;
     if (TH > g.OH)
         TH = g.OH;
     if (TH < 1)
         TH = 1;
-    const size_t fixed_bytes = (size_t)OCB * 32 + 32 + ((((size_t)rch + 32) * 4 + 15) & ~(size_t)15);
-    const size_t w_bytes     = (size_t)OCB * a.wstride;
-    size_t lds_bytes         = 0;
-    for (;;)
+    TH = ceil_div(g.OH, ceil_div(g.OH, TH));
+
+    // ---- channel block ------------------------------------------------------------------------------------
+    // Candidates from the largest block down.  A single block that covers the whole channel vector is staged
+    // in rounds into one buffer; several blocks are software pipelined over two LDS buffers when a block fits
+    // one staging round per lane.  If no candidate qualifies, blocks of at most 64 bytes go through a single
+    // buffer one after the other, with the tile shrunk until it fits.
+    const int ch_needed = row_bytes <= 16 ? 1 : (row_bytes <= 32 ? 2 : (row_bytes <= 64 ? 4 : (row_bytes <= 128 ? 8 : 16)));
+    auto set_block = [&](int CH) {
+        a.CH       = CH;
+        a.ch_shift = CH == 16 ? 4 : (CH == 8 ? 3 : (CH == 4 ? 2 : (CH == 2 ? 1 : 0)));
+        a.pstride  = CH == 1 ? 16 : CH * 16 + 16;    // all = 16 (mod 32)
+        a.n_icb    = ceil_div(row_bytes, CH * 16);
+        const int rch = taps * CH;                   // chunks per weight row
+        a.wstride  = (rch + (rch & 1)) * 16 + 16;    // room for a spare zero chunk; = 16 (mod 32)
+        a.ksteps   = (rch + 1) / 2;
+    };
+    auto fixed_bytes = [&]() {    // channel table, zero chunk, check words, dump area, pair table, patch byte sums
+        return (size_t)OCB * 32 + 32 + 1024 + ((((size_t)taps * a.CH + 32) * 4 + 15) & ~(size_t)15) +
+               (Mma<T>::is_int ? (((size_t)a.PH * a.PW * 4 + 15) & ~(size_t)15) : 0);
+    };
+    auto buf_bytes   = [&]() { return (size_t)OCB * a.wstride + (size_t)a.PH * a.PW * a.pstride; };
+    auto set_patch   = [&]() {
+        a.PH = (TH - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+        a.PW = (TW - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
+    };
+    auto set_rounds = [&]() {
+        const int w_rounds = ceil_div(ceil_div(taps * a.CH, LPR), WU);
+        const int p_rounds = ceil_div(ceil_div(a.PH * a.PW * a.CH, 512), PU);
+        a.rounds           = w_rounds > p_rounds ? w_rounds : p_rounds;
+    };
+    set_patch();
+    size_t lds_bytes = 0;
+    bool chosen      = false;
+    if (vec)
+        for (int CH = ch_needed; CH >= 1 && !chosen; CH >>= 1)
+        {
+            set_block(CH);
+            set_rounds();
+            if (a.n_icb == 1)
+            {
+                lds_bytes = fixed_bytes() + buf_bytes();
+                if (lds_bytes <= (size_t)kMaxLds)
+                    a.pipelined = 0, chosen = true;
+                continue;
+            }
+            if (a.rounds > 1)
+                continue;
+            lds_bytes = fixed_bytes() + 2 * buf_bytes();
+            if (lds_bytes <= (size_t)kMaxLds)
+                a.pipelined = 1, chosen = true;
+        }
+    if (!chosen)
     {
-        a.PH      = (TH - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
-        a.PW      = (TW - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
-        lds_bytes = fixed_bytes + w_bytes + (size_t)a.PH * a.PW * a.pstride;
-        if (lds_bytes <= (size_t)kMaxLds)
-            break;
-        if (TH > 1)
-            TH = (TH + 1) / 2;
-        else if (TW > 16)
-            TW = (TW + 1) / 2;
-        else
-            return nullptr;    // the weight slab alone does not fit: not eligible
+        set_block(ch_needed > 4 ? 4 : ch_needed);
+        for (;;)
+        {
+            set_patch();
+            lds_bytes = fixed_bytes() + buf_bytes();
+            if (lds_bytes <= (size_t)kMaxLds)
+                break;
+            if (TH > 1)
+                TH = (TH + 1) / 2;
+            else if (TW > 16)
+                TW = (TW + 1) / 2;
+            else
+                return nullptr;    // the weight slab alone does not fit: not eligible
+        }
+        a.pipelined = 0;
+        set_rounds();
     }
+    a.buf_bytes = (int)buf_bytes();
     a.TH = TH, a.TW = TW;
     a.tiles_y = (g.OH + TH - 1) / TH;
     a.tiles_x = (g.OW + TW - 1) / TW;
@@ -912,14 +1111,14 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     a.xcd_remap   = (blocks % 8) == 0 && blocks >= 16;
     a.div_tw      = make_fastdiv(TW);
     a.div_pw      = make_fastdiv(a.PW);
-    a.div_rch     = make_fastdiv(rch);
     a.div_tiles_x = make_fastdiv(a.tiles_x);
     a.div_tiles_y = make_fastdiv(a.tiles_y);
-    a.div_n_tiles = make_fastdiv(a.n_tiles);
+    a.n_ocb       = (int)oc_blocks;
+    a.div_group   = make_fastdiv(4 * a.n_ocb);    // kGroup of the kernel
     a.div_kw      = make_fastdiv(g.KW);
     // fdiv is exact for n*d < 2^32: every dividend but the block index is bounded by the LDS capacity;
     // guard the products that involve the block index
-    if ((uint64_t)blocks * (uint64_t)a.n_tiles >= (uint64_t(1) << 32) ||
+    if ((uint64_t)blocks * (uint64_t)(4 * oc_blocks) >= (uint64_t(1) << 32) ||
         (uint64_t)n_tiles * (uint64_t)a.tiles_x >= (uint64_t(1) << 32) ||
         (uint64_t)(n_tiles / a.tiles_x + 1) * (uint64_t)a.tiles_y >= (uint64_t(1) << 32))
         return nullptr;
@@ -935,28 +1134,25 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
             return nullptr;
     }
     bool ok = false;
-#define TMI_PATCH_CASE(O, P, E)                                                                                      \
-    if (WOC == O && PXT == P && epi == E)                                                                            \
-        ok = launch_patch<T, O, P, E, true>(st, a, lds_bytes, (int)blocks);
+#define TMI_PATCH_CASE(O, C, P, E)                                                                                   \
+    if (WOC == O && OCT == C && PXT == P && epi == E)                                                                \
+        ok = launch_patch<T, O, C, P, E, true>(st, a, lds_bytes, (int)blocks);
 #define TMI_PATCH_CASE_BYTES(O, E)                                                                                   \
     if (WOC == O && epi == E)                                                                                        \
-        ok = launch_patch<T, O, 1, E, false>(st, a, lds_bytes, (int)blocks);
+        ok = launch_patch<T, O, 1, 1, E, false>(st, a, lds_bytes, (int)blocks);
+#define TMI_PATCH_SHAPES(E)                                                                                          \
+    TMI_PATCH_CASE(1, 1, 1, E)                                                                                       \
+    TMI_PATCH_CASE(1, 1, 2, E)                                                                                       \
+    TMI_PATCH_CASE(2, 1, 1, E)                                                                                       \
+    TMI_PATCH_CASE(2, 1, 2, E)                                                                                       \
+    TMI_PATCH_CASE(2, 2, 2, E)
     if (vec)
     {
-        TMI_PATCH_CASE(1, 1, EPI_PLAIN)
-        TMI_PATCH_CASE(1, 2, EPI_PLAIN)
-        TMI_PATCH_CASE(2, 1, EPI_PLAIN)
-        TMI_PATCH_CASE(2, 2, EPI_PLAIN)
+        TMI_PATCH_SHAPES(EPI_PLAIN)
         if constexpr (Mma<T>::is_int)
         {
-            TMI_PATCH_CASE(1, 1, EPI_FAST)
-            TMI_PATCH_CASE(1, 2, EPI_FAST)
-            TMI_PATCH_CASE(2, 1, EPI_FAST)
-            TMI_PATCH_CASE(2, 2, EPI_FAST)
-            TMI_PATCH_CASE(1, 1, EPI_GENERIC)
-            TMI_PATCH_CASE(1, 2, EPI_GENERIC)
-            TMI_PATCH_CASE(2, 1, EPI_GENERIC)
-            TMI_PATCH_CASE(2, 2, EPI_GENERIC)
+            TMI_PATCH_SHAPES(EPI_FAST)
+            TMI_PATCH_SHAPES(EPI_GENERIC)
         }
     }
     else
@@ -971,6 +1167,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
             TMI_PATCH_CASE_BYTES(2, EPI_GENERIC)
         }
     }
+#undef TMI_PATCH_SHAPES
 #undef TMI_PATCH_CASE_BYTES
 #undef TMI_PATCH_CASE
     return ok ? label : nullptr;

@@ -84,3 +84,27 @@ def c5_matmul(n=4, h=2048, c=4096, w=2048):
     a = float_to_bf16_bits(r.normal(0, 1 / 64, (n, h, c)).astype(np.float32))
     b = float_to_bf16_bits(r.normal(0, 1 / 64, (n, c, w)).astype(np.float32))
     return dict(a=a, b=b)
+
+
+def conv2d_exact_blas(x, w, bias, pad, stride, dilation, in_zp=0, w_zp=0):
+    """int8 CONV2D (NHWC x OHWI, int32 result) as one float64 BLAS product per kernel tap.  Every partial
+    sum is an integer far below 2^53, so the float64 arithmetic is exact; the int32 result wraps like the
+    accumulator of the oracle does.  For operands too large for the scalar oracle to finish in seconds;
+    the CPU suite checks this helper against the oracle on small shapes."""
+    n, ih, iw, ic = x.shape
+    oc, kh, kw, _ = w.shape
+    pt, pb, pl, pr = pad
+    sy, sx = stride
+    dy, dx = dilation
+    oh = (ih - 1 + pt + pb - (kh - 1) * dy) // sy + 1
+    ow = (iw - 1 + pl + pr - (kw - 1) * dx) // sx + 1
+    xp = np.zeros((n, ih + pt + pb, iw + pl + pr, ic), np.float64)       # (x - in_zp), zero outside the image
+    xp[:, pt:pt + ih, pl:pl + iw, :] = x.astype(np.float64) - in_zp
+    wf = w.astype(np.float64) - w_zp
+    acc = np.zeros((n * oh * ow, oc), np.float64)
+    for ky in range(kh):
+        for kx in range(kw):
+            win = xp[:, ky * dy: ky * dy + (oh - 1) * sy + 1: sy, kx * dx: kx * dx + (ow - 1) * sx + 1: sx, :]
+            acc += win.reshape(-1, ic) @ wf[:, ky, kx, :].T
+    acc += (bias.astype(np.float64) if bias.shape[0] == oc else float(bias[0]))
+    return acc.astype(np.int64).astype(np.int32).reshape(n, oh, ow, oc)

@@ -159,6 +159,64 @@ def test_conv2d_fp_mfma_within_dot_product_bound(ctx, kind, shape):
     assert res["max_ulp"] <= 2.0, res  # fp32 accumulation: the result is the correctly rounded value +- 1 ulp
 
 
+# ---- GEMM-sized work: the 128-channel x 256-pixel workgroup shape and pipelined channel blocks ---------------
+BIG_SHAPES = [
+    # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
+    (1, 256, 256, 128, 128, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),    # one 128-byte channel block
+    (2, 128, 128, 128, 200, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),    # 3x3, four pipelined blocks, ragged OC
+    (1, 300, 220, 528, 96, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),     # 528 = 4*128 + 16: short last block
+    (4, 131, 131, 64, 136, 3, 3, (0, 0, 0, 0), (2, 2), (1, 1)),     # stride 2, rows that do not fill a tile
+    (16, 28, 28, 256, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # 64-channel shape with pipelined blocks
+]
+
+
+@pytest.mark.parametrize("shape", BIG_SHAPES)
+@pytest.mark.parametrize("zps", [(-7, 3), (11, 0)])
+def test_conv2d_i8_mfma_gemm_sized_bit_exact(ctx, shape, zps):
+    """Expected values from the float64-BLAS restatement (checked against the oracle by the CPU suite), plus the
+    scalar oracle itself on the first image's first rows."""
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(sum(shape[:7]) + zps[0])
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
+    bias = rng.integers(-65536, 65536, oc).astype(np.int32)
+    want = cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, *zps)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=zps[1])
+    assert ctx.last_kernel == "conv2d_mfma_i8"
+    assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    rows = 2 * stride[0] + (kh - 1) * dil[0] + 1 - pad[0]    # input rows behind the first three output rows
+    sl = oracle.conv2d("i8", x[:1, :rows], w, bias, (pad[0], 0, pad[2], pad[3]), stride, dil, in_zp=zps[0],
+                       w_zp=zps[1])
+    assert np.array_equal(got[0, :3], sl[0])
+
+
+@pytest.mark.parametrize("mode", ["fast", "generic16", "int16out"])
+def test_conv2d_i8_gemm_sized_fused_rescale(ctx, mode):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = BIG_SHAPES[1]
+    rng = np.random.default_rng(99)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = np.clip(np.rint(rng.normal(0, 20, (oc, kh, kw, ic))), -127, 127).astype(np.int8)
+    bias = rng.integers(-65536, 65536, oc).astype(np.int32)
+    acc = cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, -7, 0)
+    if mode == "generic16":
+        # a 16-bit multiplier on the int32 accumulator: not the fast path, the staged general RESCALE
+        mult, shift, scale32 = rng.integers(1 << 13, 1 << 15, oc).astype(np.int32), np.full(oc, 26, np.int8), False
+        rounding = capi.ROUND_SINGLE
+    else:
+        mult, shift, scale32 = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32), rng.integers(37, 41, oc).astype(np.int8), True
+        rounding = capi.ROUND_DOUBLE
+    od = np.int16 if mode == "int16out" else np.int8
+    out_zp = 0 if mode == "int16out" else -3    # a non-zero output_zp is an ERROR_IF for int16
+    want, wst = oracle.rescale(acc, mult, shift, in_zp=0, out_zp=out_zp, out_dtype=od, scale32=scale32,
+                               rounding_mode=oracle.ROUND_DOUBLE if scale32 else oracle.ROUND_SINGLE, per_channel=True)
+    assert wst == oracle.VALID
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=-7, w_zp=0,
+                             rescale=dict(mult=mult, shift=shift, out_zp=out_zp, out_dtype=od, scale32=scale32,
+                                          rounding_mode=rounding))
+    assert ctx.last_kernel == "conv2d_mfma_i8_rescale"
+    assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+
+
 def test_mfma_not_eligible_is_an_error_when_forced(ctx):
     # a 31x31 kernel with 64 output channels needs a 4.9 MB weight slab: no MFMA tiling fits LDS
     x = np.zeros((1, 31, 31, 64), np.int8)

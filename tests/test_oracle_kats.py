@@ -353,3 +353,17 @@ def _np_conv_f64(x, w, b):
         for kx in range(3):
             out += np.einsum("nhwc,oc->nhwo", xp[:, ky:ky + 6, kx:kx + 7], w[:, ky, kx].astype(np.float64))
     return out + b.astype(np.float64)
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES)
+def test_blas_conv_helper_equals_oracle(shape):
+    """The float64-BLAS restatement used for GEMM-sized GPU cases gives the oracle's int32 results."""
+    import cases
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(4242 + sum(shape[:7]))
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
+    bias = rng.integers(-(1 << 30), 1 << 30, oc).astype(np.int32)
+    for zps in [(0, 0), (-128, 127), (9, -3)]:
+        want = oracle.conv2d("i8", x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=zps[1])
+        assert np.array_equal(cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, *zps), want)
