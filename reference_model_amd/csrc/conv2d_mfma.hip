@@ -58,25 +58,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 
-// n / d for n*d < 2^32 as one multiply-high (magic = floor(2^32/d) + 1; d == 1 is special-cased).
-struct FastDiv
-{
-    uint32_t magic, d;
-};
-
-static FastDiv make_fastdiv(uint32_t d)
-{
-    FastDiv f;
-    f.d     = d;
-    f.magic = d <= 1 ? 0u : (uint32_t)((uint64_t(1) << 32) / d) + 1u;
-    return f;
-}
-
-__device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f)
-{
-    return f.d <= 1 ? n : __umulhi(n, f.magic);
-}
-
 struct PatchArgs
 {
     ConvGeom g;

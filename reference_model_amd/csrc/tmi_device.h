@@ -10,6 +10,25 @@
 namespace tmi
 {
 
+// n / d for n*d < 2^32 as one multiply-high (magic = floor(2^32/d) + 1; d == 1 is special-cased).
+struct FastDiv
+{
+    uint32_t magic, d;
+};
+
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    FastDiv f;
+    f.d     = d;
+    f.magic = d <= 1 ? 0u : (uint32_t)((uint64_t(1) << 32) / d) + 1u;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f)
+{
+    return f.d <= 1 ? n : __umulhi(n, f.magic);
+}
+
 // Everything a kernel needs to apply RESCALE (and an optional CLAMP) to one value.  Filled on the host
 // after validation, passed by value.
 struct RescaleParams

@@ -73,7 +73,7 @@ const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dty
 // elementwise.hip: [N, R, C] -> [N, C, R] for 1- or 2-byte elements (MATMUL's second operand becomes K-contiguous).
 const char* launch_transpose(hipStream_t st, int32_t elem_bytes, int32_t N, int32_t R, int32_t C, const void* in,
                              void* out);
-// depthwise.hip: 16 channels per lane, fused epilogue; nullptr when not eligible.
+// depthwise.hip: 4 channels per lane, dot4 across taps, fused epilogue; nullptr when not eligible.
 const char* launch_depthwise_vec(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                  const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                  const RescaleParams& rp, void* out, uint32_t* flag_word);

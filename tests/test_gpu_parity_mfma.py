@@ -279,15 +279,19 @@ def test_matmul_fp_mfma_within_dot_product_bound(ctx, kind):
     assert res["ok"], res
 
 
-# ---- DEPTHWISE_CONV2D, 16-channel vector kernel ------------------------------------------------------
+# ---- DEPTHWISE_CONV2D, four channels per lane with dot4 across taps ---------------------------------------
 @pytest.mark.parametrize("shape", [  # n, ih, iw, c, kh, kw, pad, stride, dilation
     (2, 10, 8, 16, 3, 3, (0, 1, 0, 1), (2, 2), (1, 1)),
     (1, 9, 9, 48, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
     (1, 12, 7, 32, 5, 3, (2, 2, 1, 1), (1, 1), (1, 1)),
     (3, 8, 8, 96, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),
+    (1, 11, 13, 20, 5, 5, (2, 2, 2, 2), (1, 1), (1, 1)),      # 25 taps, channels a multiple of 4 only
+    (2, 7, 9, 4, 1, 1, (0, 0, 0, 0), (2, 2), (1, 1)),         # one tap, one channel group
+    (1, 6, 40, 260, 2, 2, (0, 0, 1, 1), (1, 1), (1, 1)),      # 65 channel groups: three pixels per iteration
+    (1, 70, 70, 1024, 1, 2, (0, 0, 0, 1), (1, 1), (1, 1)),    # a whole workgroup per pixel, several iterations
 ])
 @pytest.mark.parametrize("zps", [(4, 0), (-3, 7), (0, 0)])
-def test_depthwise_vec16_bit_exact(ctx, shape, zps):
+def test_depthwise_dot4_bit_exact(ctx, shape, zps):
     n, ih, iw, c, kh, kw, pad, stride, dil = shape
     rng = np.random.default_rng(c + kh)
     x = rng.integers(-128, 128, (n, ih, iw, c)).astype(np.int8)
@@ -295,7 +299,7 @@ def test_depthwise_vec16_bit_exact(ctx, shape, zps):
     for bias in (rng.integers(-30000, 30000, c).astype(np.int32), np.array([-77], np.int32)):
         want = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, *zps)
         got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, *zps, depthwise=True)
-        assert ctx.last_kernel == "depthwise_vec16_i8"
+        assert ctx.last_kernel == "depthwise_dot4_i8"
         assert st == capi.VALID and np.array_equal(got, want)
 
 
@@ -312,7 +316,7 @@ def test_config4_depthwise_rescale_full_size(ctx):
     got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
                              c["w_zp"], depthwise=True, rescale=dict(mult=c["mult"], shift=c["shift"],
                                                                      out_zp=c["out_zp"]))
-    assert ctx.last_kernel == "depthwise_vec16_i8_rescale"
+    assert ctx.last_kernel == "depthwise_dot4_i8_rescale"
     want = _dw_expect(c)
     assert st == capi.VALID and got.shape == (8, 56, 56, 96) and np.array_equal(got, want)
 
@@ -330,6 +334,24 @@ def test_depthwise_rescale_other_outputs_and_clamp(ctx, out_dtype):
                              c["w_zp"], depthwise=True, clamp=c["clamp"],
                              rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=0))
     assert st == capi.VALID and np.array_equal(got, _dw_expect(c))
+
+
+def test_depthwise_small_shifts_take_the_checked_path(ctx):
+    """Shifts below 32 switch on apply_scale_32's value-range test (quant_util.h:59-67): legal values stay VALID
+    and bit-exact, a violation is reported as UNPREDICTABLE."""
+    c = cases.c4(n=1, hw=16, c=32)
+    c["mult"] = np.full(32, 1 << 20, np.int32)
+    c["shift"] = np.full(32, 24, np.int8)    # |acc| < 2^23 holds: 9 * 128 * 132 + 2^15 < 2^18
+    kw = dict(depthwise=True, rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"]))
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                             c["w_zp"], **kw)
+    assert ctx.last_kernel == "depthwise_dot4_i8_rescale"
+    assert st == capi.VALID and np.array_equal(got, _dw_expect(c))
+    c["shift"] = np.full(32, 10, np.int8)    # now |acc| exceeds 2^9 somewhere
+    kw["rescale"]["shift"] = c["shift"]
+    _, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                           c["w_zp"], **kw)
+    assert st == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
 
 
 def test_depthwise_multiplier_falls_back_to_direct_kernel():
