@@ -224,7 +224,8 @@ struct TileTraits
 static constexpr uint32_t kNone = 0xffffffffu;
 static constexpr uint32_t kFill = 0xfffffffeu;
 
-template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC>
+// MULTI: the input channels take more than one block (the block loop's bookkeeping is compiled in)
+template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC, bool MULTI>
 __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 {
     using M              = Mma<T>;
@@ -343,9 +344,15 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const int p_total      = a.PH * a.PW * a.CH;
     const int p_cc16       = (tid & (a.CH - 1)) * 16;    // NT is a multiple of CH: one chunk column per lane
 
-    uint32_t wsrc[WU], psrc[PU];
-    int wdst[WU], ppix[PU];
+    uint32_t wsrc[WU], psrc[PU];    // byte offsets of the sources (chunk column included), or kNone / kFill
+    int wdst[WU], pdst[PU];         // byte offsets inside the weight rows / the patch, or -1
+    int ppix[PU];                   // patch pixel of the slot, or -1
     v4i wv[WU], pv[PU];
+    int wacc = 0;                   // byte sum of this lane's share of its weight row, over all blocks
+    int pacc[PU];                   // byte sums of the lane's patch chunks over all blocks (one round per block only)
+#pragma unroll
+    for (int u = 0; u < PU; u++)
+        pacc[u] = 0;
 
     auto describe = [&](int round) {
 #pragma unroll
@@ -359,6 +366,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             const int iy = y0 + py, ix = x0 + px;
             const bool img = iy >= 0 && iy < g.IH && ix >= 0 && ix < g.IW;
             ppix[u]        = ok ? pix : -1;
+            pdst[u]        = ok ? pix * a.pstride + p_cc16 : -1;
             psrc[u]        = !ok ? kNone : (img ? (uint32_t)(iy * g.IW + ix) * (uint32_t)row_bytes + (uint32_t)p_cc16 : kFill);
         }
 #pragma unroll
@@ -375,11 +383,40 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     };
     // chunk column (byte offset inside the channel block) of weight work item u of a round
     auto w_cc16 = [&](int round, int u) { return ((w_part + (round * WU + u) * LPR) & (a.CH - 1)) * 16; };
-
-    auto issue = [&](int round, int ic_off) {
+    // Per slot and wave: `void` if no lane has a destination (the slot is skipped), `plain` if every lane has a
+    // source and a destination.  A plain slot of a channel block that lies wholly inside the channel vector
+    // needs no per-item test: the load takes a scalar base plus the item's offset and the data goes to LDS as
+    // it arrived.  The masks are wave-uniform; they are only known when a block is one round.
+    uint32_t p_plain = 0, p_void = 0, w_plain = 0, w_void = 0;
+    auto classify = [&]() {
 #pragma unroll
         for (int u = 0; u < PU; u++)
         {
+            p_plain |= (__all(psrc[u] < kFill) ? 1u : 0u) << u;
+            p_void |= (__all(ppix[u] < 0) ? 1u : 0u) << u;
+        }
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            w_plain |= (__all(wsrc[u] != kNone) ? 1u : 0u) << u;
+            w_void |= (__all(wdst[u] < 0) ? 1u : 0u) << u;
+        }
+    };
+
+    // `whole`: the channel block [ic_off, ic_off + blk_bytes) ends inside the channel vector
+    auto issue = [&](int round, int ic_off, bool whole) {
+        const uint8_t* pb = in_n + ic_off;
+        const uint8_t* wb = w_n + ic_off;
+#pragma unroll
+        for (int u = 0; u < PU; u++)
+        {
+            if (MULTI && ((p_void >> u) & 1u))
+                continue;
+            if (MULTI && VEC && whole && ((p_plain >> u) & 1u))
+            {
+                pv[u] = *reinterpret_cast<const v4i*>(pb + psrc[u]);
+                continue;
+            }
             const bool in_row = ic_off + p_cc16 < row_bytes;
             if constexpr (VEC)
             {
@@ -398,6 +435,13 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 #pragma unroll
         for (int u = 0; u < WU; u++)
         {
+            if (MULTI && ((w_void >> u) & 1u))
+                continue;
+            if (MULTI && VEC && whole && ((w_plain >> u) & 1u))
+            {
+                wv[u] = *reinterpret_cast<const v4i*>(wb + wsrc[u]);
+                continue;
+            }
             const int cc16 = w_cc16(round, u);
             if constexpr (VEC)
             {
@@ -413,59 +457,78 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
         }
     };
 
-    // Writes a round to LDS.  Work items without a destination write to the dump area, so the round has no
-    // branch.  Returns the byte sum of the weight chunks written (for the zero-point correction); with a
-    // non-zero weight zero point the byte sum of every patch pixel is accumulated in psum as well: the CH
-    // lanes that hold a pixel's chunks add them up and the first of them owns the pixel's entry.
-    auto commit = [&](int round, int ic_off, uint8_t* wl, uint8_t* pl, bool first_block) {
-        int w_sum = 0;
+    // Writes a round to LDS.  Work items without a destination write to the dump area, so a slot has no
+    // divergent branch.  The byte sums for the zero-point correction are taken here, from the registers: sum(w)
+    // of the lane's share of its weight row goes to wacc; with a non-zero weight zero point the byte sum of
+    // every patch chunk goes to pacc (`defer`: one round per block, flushed to psum once after the last block)
+    // or, when the slots change from round to round, straight to psum: the CH lanes that hold a pixel's chunks
+    // add them up and the first of them owns the pixel's entry.
+    auto commit = [&](int round, int ic_off, uint8_t* wl, uint8_t* pl, bool first_block, bool whole, bool defer) {
 #pragma unroll
         for (int u = 0; u < PU; u++)
         {
+            if (MULTI && ((p_void >> u) & 1u))
+                continue;
             v4i v = pv[u];
-            if constexpr (VEC)
+            uint8_t* dst = pl + pdst[u];
+            if (!(MULTI && whole && ((p_plain >> u) & 1u)))
             {
-                const bool in_row = ic_off + p_cc16 < row_bytes;
-                const bool ld     = psrc[u] < kFill && in_row;
-                const int fw      = (psrc[u] == kFill && in_row) ? fill_word : 0;    // whole chunks only here
-                v                 = ld ? v : v4i{ fw, fw, fw, fw };
+                if constexpr (VEC)
+                {
+                    const bool in_row = ic_off + p_cc16 < row_bytes;
+                    const bool ld     = psrc[u] < kFill && in_row;
+                    const int fw      = (psrc[u] == kFill && in_row) ? fill_word : 0;    // whole chunks only here
+                    v                 = ld ? v : v4i{ fw, fw, fw, fw };
+                }
+                dst = pdst[u] >= 0 ? dst : dump;
             }
-            uint8_t* dst = ppix[u] >= 0 ? pl + ppix[u] * a.pstride + p_cc16 : dump;
             *reinterpret_cast<v4i*>(dst) = v;
             if constexpr (M::is_int)
                 if (a.zw != 0)
                 {
                     int sum = dot4_ones(v);
-                    for (int m = 1; m < a.CH; m <<= 1)
-                        sum += __shfl_xor(sum, m);
-                    if (p_cc16 == 0 && ppix[u] >= 0)
-                        psum[ppix[u]] = first_block ? sum : psum[ppix[u]] + sum;
+                    if (defer)
+                        pacc[u] += sum;
+                    else
+                    {
+                        for (int m = 1; m < a.CH; m <<= 1)
+                            sum += __shfl_xor(sum, m);
+                        if (p_cc16 == 0 && ppix[u] >= 0)
+                            psum[ppix[u]] = first_block ? sum : psum[ppix[u]] + sum;
+                    }
                 }
         }
 #pragma unroll
         for (int u = 0; u < WU; u++)
         {
+            if (MULTI && ((w_void >> u) & 1u))
+                continue;
             v4i v = wv[u];
-            if constexpr (VEC)
+            uint8_t* dst = wl + wdst[u];
+            if (!(MULTI && whole && ((w_plain >> u) & 1u)))
             {
-                const bool ld = wsrc[u] != kNone && ic_off + w_cc16(round, u) < row_bytes;
-                v             = ld ? v : v4i{ 0, 0, 0, 0 };
+                if constexpr (VEC)
+                {
+                    const bool ld = wsrc[u] != kNone && ic_off + w_cc16(round, u) < row_bytes;
+                    v             = ld ? v : v4i{ 0, 0, 0, 0 };
+                }
+                dst = wdst[u] >= 0 ? dst : dump;
             }
-            uint8_t* dst = wdst[u] >= 0 ? wl + wdst[u] : dump;
             *reinterpret_cast<v4i*>(dst) = v;
             if constexpr (M::is_int)
                 if (a.za != 0)
-                    w_sum += dot4_ones(v);    // work items without a source hold zeros
+                    wacc += dot4_ones(v);    // work items without a source hold zeros
         }
-        return w_sum;
     };
 
     // The channel blocks are taken in an order rotated by the workgroup's position: workgroups that run side
     // by side would otherwise all read the same 16*CH-byte column of every row at the same time, which lands
     // on a fraction of the memory channels when the row length is a power of two.  (Integer sums do not depend
     // on the order; the floating-point bound holds for any order.)
-    const int rot = a.n_icb > 1 ? (int)((tile + ocb) % (uint32_t)a.n_icb) : 0;
+    const int rot = MULTI ? (int)((tile + ocb) % (uint32_t)a.n_icb) : 0;
     auto block_offset = [&](int icb) {
+        if constexpr (!MULTI)
+            return 0;
         const int b = icb + rot;
         return (b >= a.n_icb ? b - a.n_icb : b) * blk_bytes;
     };
@@ -473,10 +536,14 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     // With one round per block the first block's loads are started before anything else, so that the table
     // set-up below (which has global loads of its own) runs in their shadow.
     const bool one_round = a.rounds == 1;
+    // a block is whole when it ends inside the channel vector; only the last one in memory order may not be
+    auto block_is_whole = [&](int off) { return off + blk_bytes <= row_bytes; };
     if (one_round)
     {
         describe(0);
-        issue(0, block_offset(0));
+        if constexpr (MULTI)
+            classify();
+        issue(0, block_offset(0), block_is_whole(block_offset(0)));
     }
 
     // ---- tables ----------------------------------------------------------------------------------------
@@ -534,17 +601,18 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : oc) : 0.0f;
     }
 
-    for (int icb = 0; icb < a.n_icb; icb++)
+    const int n_icb = MULTI ? a.n_icb : 1;
+    for (int icb = 0; icb < n_icb; icb++)
     {
-        const int ic_off = block_offset(icb);
-        uint8_t* wl      = buf0 + ((a.pipelined && (icb & 1)) ? a.buf_bytes : 0);
-        uint8_t* pl      = wl + w_bytes;
-        int staged_w_sum = 0;
-        if (a.pipelined)
+        const int ic_off   = block_offset(icb);
+        const bool whole   = block_is_whole(ic_off);
+        uint8_t* wl        = buf0 + ((a.pipelined && (icb & 1)) ? a.buf_bytes : 0);
+        uint8_t* pl        = wl + w_bytes;
+        if (MULTI && a.pipelined)
         {
             // this block's chunks were requested one block ago; its buffer was last read two blocks ago, and
             // every wave has passed a barrier since
-            staged_w_sum = commit(0, ic_off, wl, pl, icb == 0);
+            commit(0, ic_off, wl, pl, icb == 0, whole, true);
         }
         else
         {
@@ -555,31 +623,17 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 if (!one_round)
                     describe(round);
                 if (!one_round || icb)
-                    issue(round, ic_off);
-                staged_w_sum += commit(round, ic_off, wl, pl, icb == 0);
+                    issue(round, ic_off, whole);
+                commit(round, ic_off, wl, pl, icb == 0, whole, one_round);
             }
         }
         __syncthreads();
 
-        // ---- sum(w) per output channel, for the zero-point correction -----------------------------------------
-        // The LPR lanes that share a weight row finish its byte sum with a butterfly and -za*sum(w) goes
-        // straight into the channel table's bias (one LDS atomic per row, all rows distinct; the table was
-        // written before the barrier above).  The K loop stays free of side computations.
-        if constexpr (M::is_int)
+        if (MULTI && a.pipelined && icb + 1 < n_icb)
         {
-            if (a.za != 0)
-            {
-                int sum = staged_w_sum;
-#pragma unroll
-                for (int m = 1; m < LPR; m <<= 1)
-                    sum += __shfl_xor(sum, m);
-                if (w_part == 0)
-                    atomicAdd(&ctab[w_ocl].bias, -a.za * sum);
-            }
+            const int next = block_offset(icb + 1);
+            issue(0, next, block_is_whole(next));
         }
-
-        if (a.pipelined && icb + 1 < a.n_icb)
-            issue(0, block_offset(icb + 1));
 
         // ---- MFMA over the (tap, chunk) pairs of this channel block -----------------------------------
         if (wave_active)
@@ -652,6 +706,37 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 for (int u = 0; u < G; u++)
                     if (s + G + u < a.ksteps)
                         compute(fa[1][u], fb[1][u]);
+            }
+        }
+    }
+
+    // ---- zero-point sums ---------------------------------------------------------------------------------
+    // sum(w) per output channel: the LPR lanes that share a weight row finish its byte sum with a butterfly and
+    // -za*sum(w) goes into the channel table's bias (one LDS atomic per row, all rows distinct; the table was
+    // written before the first barrier).  sum(a) per patch pixel, when it was kept in registers: the CH lanes
+    // that hold a pixel's chunks add up and the first writes the pixel's entry.  The barrier in the epilogue
+    // makes both visible.
+    if constexpr (M::is_int)
+    {
+        if (a.za != 0)
+        {
+            int sum = wacc;
+#pragma unroll
+            for (int m = 1; m < LPR; m <<= 1)
+                sum += __shfl_xor(sum, m);
+            if (w_part == 0)
+                atomicAdd(&ctab[w_ocl].bias, -a.za * sum);
+        }
+        if (a.zw != 0 && one_round)
+        {
+#pragma unroll
+            for (int u = 0; u < PU; u++)
+            {
+                int sum = pacc[u];
+                for (int m = 1; m < a.CH; m <<= 1)
+                    sum += __shfl_xor(sum, m);
+                if (p_cc16 == 0 && ppix[u] >= 0)
+                    psum[ppix[u]] = sum;
             }
         }
     }
@@ -741,22 +826,21 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     }
     else
     {
+        // the zero-point sums were written after the last block: make them visible to every wave
+        if (a.za != 0 || a.zw != 0)
+            __syncthreads();
         const int kzz = g.KH * g.KW * g.IC * a.za * a.zw;
         int pcorr[PXT];    // the zero-point terms that depend on the pixel only: K*za*zw - zw*sum(a)
 #pragma unroll
         for (int i = 0; i < PXT; i++)
         {
             int sa = 0;
-            if (a.zw != 0)    // sum(a) over the window of this pixel from the per-pixel byte sums (complete since the
-                              // barrier that followed the last block's staging)
+            if (a.zw != 0)    // sum(a) over the window of this pixel from the per-pixel byte sums
                 for (int ky = 0; ky < g.KH; ky++)
                     for (int kx = 0; kx < g.KW; kx++)
                         sa += psum[pidx[i] + ky * g.dil_y * a.PW + kx * g.dil_x];
             pcorr[i] = kzz - a.zw * sa;
         }
-        // -za*sum(w) was added to the channel table's bias after staging: make it visible to every wave
-        if (a.za != 0)
-            __syncthreads();
         if constexpr (EPI == EPI_GENERIC)
             __syncthreads();    // every wave is done reading the operands: LDS becomes the staging area
         int32_t* stage = reinterpret_cast<int32_t*>(lds + kCtab);    // [pixel of the tile][channel of the block]
@@ -942,10 +1026,10 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 
 static constexpr int kMaxLds = 160 * 1024;
 
-template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC>
+template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC, bool MULTI>
 static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blocks)
 {
-    auto kern                = conv2d_patch_kernel<T, WOC, OCT, PXT, EPI, VEC>;
+    auto kern                = conv2d_patch_kernel<T, WOC, OCT, PXT, EPI, VEC, MULTI>;
     static size_t configured = 0;    // largest dynamic LDS size this instantiation was configured for
     if (lds_bytes > configured)
     {
@@ -1117,10 +1201,12 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     bool ok = false;
 #define TMI_PATCH_CASE(O, C, P, E)                                                                                   \
     if (WOC == O && OCT == C && PXT == P && epi == E)                                                                \
-        ok = launch_patch<T, O, C, P, E, true>(st, a, lds_bytes, (int)blocks);
+        ok = a.n_icb > 1 ? launch_patch<T, O, C, P, E, true, true>(st, a, lds_bytes, (int)blocks)                      \
+                         : launch_patch<T, O, C, P, E, true, false>(st, a, lds_bytes, (int)blocks);
 #define TMI_PATCH_CASE_BYTES(O, E)                                                                                   \
     if (WOC == O && epi == E)                                                                                        \
-        ok = launch_patch<T, O, 1, 1, E, false>(st, a, lds_bytes, (int)blocks);
+        ok = a.n_icb > 1 ? launch_patch<T, O, 1, 1, E, false, true>(st, a, lds_bytes, (int)blocks)                     \
+                         : launch_patch<T, O, 1, 1, E, false, false>(st, a, lds_bytes, (int)blocks);
 #define TMI_PATCH_SHAPES(E)                                                                                          \
     TMI_PATCH_CASE(1, 1, 1, E)                                                                                       \
     TMI_PATCH_CASE(1, 1, 2, E)                                                                                       \
