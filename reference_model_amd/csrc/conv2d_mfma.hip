@@ -1025,6 +1025,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 // ---- host side: tile choice and launch -----------------------------------------------------------------
 
 static constexpr int kMaxLds = 160 * 1024;
+static constexpr int kCUs    = 256;
 
 template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC, bool MULTI>
 static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blocks)
@@ -1072,28 +1073,50 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     const bool vec = (row_bytes & 15) == 0 && (((uintptr_t)in | (uintptr_t)w) & 15) == 0;
 
     // ---- workgroup shape: WOC x OCT channel tiles, PXT pixel tiles per wave -------------------------------
-    // The 128-channel x 256-pixel shape when that still gives every CU a workgroup; else 64 (or 32) channels
-    // with two pixel tiles per wave when that leaves two workgroups per CU; else the smallest.
-    int WOC = g.OC > 32 ? 2 : 1, OCT = 1, PXT = 1;
-    if (vec && g.OC > 64 && n_px * ((g.OC + 127) / 128) >= (int64_t)256 * 256)
-        OCT = 2, PXT = 2;
-    else if (vec && n_px * ((g.OC + 32 * WOC - 1) / (32 * WOC)) >= (int64_t)256 * 2 * 2 * 32 * (8 / WOC))
-        PXT = 2;
+    // Each candidate is priced in SIMD cycles: rounds of workgroups over the CUs times (MFMA time of one
+    // workgroup + the cost of staging its operands + a fixed start-up); the cheapest wins.  The pixel tile
+    // prefers full output rows and spreads the rows evenly over the tiles.
+    const int WOC = g.OC > 32 ? 2 : 1;
+    auto tile_for = [&](int max_px, int& TH, int& TW) {
+        TW = g.OW < max_px ? g.OW : max_px;
+        TW = ceil_div(g.OW, ceil_div(g.OW, TW));
+        TH = max_px / TW;
+        if (TH > g.OH)
+            TH = g.OH;
+        if (TH < 1)
+            TH = 1;
+        TH = ceil_div(g.OH, ceil_div(g.OH, TH));
+    };
+    int OCT = 1, PXT = 1;
+    if (vec)
+    {
+        static const int cand[3][2] = { { 1, 1 }, { 1, 2 }, { 2, 2 } };
+        double best = 0;
+        for (int c = 0; c < 3; c++)
+        {
+            const int oct = cand[c][0], pxt = cand[c][1];
+            if (oct == 2 && g.OC <= 64)
+                continue;
+            const int ocb = 32 * oct * WOC, max_px = 32 * (8 / WOC) * pxt;
+            int th, tw;
+            tile_for(max_px, th, tw);
+            const double wgs    = (double)g.N * ceil_div(g.OH, th) * ceil_div(g.OW, tw) * ceil_div(g.OC, ocb);
+            const double rounds = (double)(int64_t)((wgs + kCUs - 1) / kCUs);
+            const double ksteps = (double)taps * ceil_div(row_bytes, 32);             // 32 bytes of K per MFMA and lane half
+            const double mfma   = 2.0 * oct * pxt * ksteps * 32;                      // two waves per SIMD
+            const double stage  = (double)(ocb + max_px) * taps * row_bytes / 16 / 512 * 2 * 40;
+            const double cost   = rounds * (mfma + stage + 3000);
+            if (c == 0 || cost < best)
+                best = cost, OCT = oct, PXT = pxt;
+        }
+    }
     const int OCB           = 32 * OCT * WOC;
     const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
     const int max_px        = 32 * (8 / WOC) * PXT;
     const int WU = 5, PU = (OCT * PXT >= 4) ? 8 : 2;    // the values of TileTraits<OCT, PXT>
     const int LPR = 512 / OCB;
-
-    // ---- pixel tile: full output rows when they fit, and rows spread evenly over the tiles ------------------
-    int TW = g.OW < max_px ? g.OW : max_px;
-    TW     = ceil_div(g.OW, ceil_div(g.OW, TW));
-    int TH = max_px / TW;
-    if (TH > g.OH)
-        TH = g.OH;
-    if (TH < 1)
-        TH = 1;
-    TH = ceil_div(g.OH, ceil_div(g.OH, TH));
+    int TH, TW;
+    tile_for(max_px, TH, TW);
 
     // ---- channel block ------------------------------------------------------------------------------------
     // Candidates from the largest block down.  A single block that covers the whole channel vector is staged
