@@ -210,12 +210,12 @@ struct alignas(16) ChanEntry
 };
 
 // Per-lane chunk budget of one staging round (weights, patch) and K-loop group size of an instantiation.
-template <int OCT, int PXT>
+template <int OCT, int PXT, bool MULTI>
 struct TileTraits
 {
     static constexpr bool big = OCT * PXT >= 4;
     static constexpr int WU   = 5;
-    static constexpr int PU   = big ? 8 : 2;
+    static constexpr int PU   = big ? 8 : (MULTI ? 4 : 2);
     static constexpr int G    = big ? 1 : 3;
 };
 
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 {
     using M              = Mma<T>;
     using acc_t          = typename M::acc_t;
-    using TT             = TileTraits<OCT, PXT>;
+    using TT             = TileTraits<OCT, PXT, MULTI>;
     constexpr int EB     = sizeof(T);
     constexpr int NT     = 512;                // lanes per workgroup
     constexpr int WPX    = 8 / WOC;            // waves along the pixel dimension
@@ -1113,7 +1113,8 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     const int OCB           = 32 * OCT * WOC;
     const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
     const int max_px        = 32 * (8 / WOC) * PXT;
-    const int WU = 5, PU = (OCT * PXT >= 4) ? 8 : 2;    // the values of TileTraits<OCT, PXT>
+    const int WU = 5;                                   // the values of TileTraits<OCT, PXT, n_icb > 1>
+    auto PU_for  = [&](int n_icb) { return (OCT * PXT >= 4) ? 8 : (n_icb > 1 ? 4 : 2); };
     const int LPR = 512 / OCB;
     int TH, TW;
     tile_for(max_px, TH, TW);
@@ -1144,7 +1145,7 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     };
     auto set_rounds = [&]() {
         const int w_rounds = ceil_div(ceil_div(taps * a.CH, LPR), WU);
-        const int p_rounds = ceil_div(ceil_div(a.PH * a.PW * a.CH, 512), PU);
+        const int p_rounds = ceil_div(ceil_div(a.PH * a.PW * a.CH, 512), PU_for(a.n_icb));
         a.rounds           = w_rounds > p_rounds ? w_rounds : p_rounds;
     };
     set_patch();

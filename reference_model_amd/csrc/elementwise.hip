@@ -179,13 +179,94 @@ __global__ __launch_bounds__(256) void transpose_kernel(int32_t R, int32_t C, co
             out[base + (size_t)(c0 + i) * R + r0 + tx] = tile[tx][i];
 }
 
+// The same for shapes made of whole, aligned pieces (C*EB a multiple of 4 bytes, R*EB a multiple of 16): dwords in,
+// small blocks transposed in registers with byte permutes, 16-byte rows out.  A 64x64-element tile per workgroup.
+typedef int tr_v4i __attribute__((ext_vector_type(4)));
+
+template <int EB>
+__global__ __launch_bounds__(256) void transpose_vec_kernel(int32_t R, int32_t C, const uint8_t* __restrict__ in,
+                                                            uint8_t* __restrict__ out)
+{
+    constexpr int kRow = 64 * EB + 16;    // LDS row: 64 elements along R, padded
+    __shared__ __attribute__((aligned(16))) uint8_t tile[64 * kRow];    // [c][r]
+    const size_t base = (size_t)blockIdx.z * R * C * EB;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tid = threadIdx.x;
+    if constexpr (EB == 1)
+    {
+        // a thread takes a 4x4 block: four dwords (one per row), transposed to four dwords (one per column)
+        const int tx = tid & 15, ty = tid >> 4;
+        int d[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+        {
+            const bool ok = r0 + 4 * ty + j < R && c0 + 4 * tx < C;
+            d[j] = *reinterpret_cast<const int*>(in + base + (ok ? (size_t)(r0 + 4 * ty + j) * C + c0 + 4 * tx : 0));
+        }
+        const int t01_lo = __builtin_amdgcn_perm(d[1], d[0], 0x05010400);
+        const int t01_hi = __builtin_amdgcn_perm(d[1], d[0], 0x07030602);
+        const int t23_lo = __builtin_amdgcn_perm(d[3], d[2], 0x05010400);
+        const int t23_hi = __builtin_amdgcn_perm(d[3], d[2], 0x07030602);
+        int e[4];
+        e[0] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x05040100);
+        e[1] = __builtin_amdgcn_perm(t23_lo, t01_lo, 0x07060302);
+        e[2] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x05040100);
+        e[3] = __builtin_amdgcn_perm(t23_hi, t01_hi, 0x07060302);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            *reinterpret_cast<int*>(tile + (4 * tx + j) * kRow + 4 * ty) = e[j];
+    }
+    else
+    {
+        // 2-byte elements: 2x2 blocks, four per thread
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+        {
+            const int b  = tid + 256 * k;    // block index: 32 x 32 blocks
+            const int bx = b & 31, by = b >> 5;
+            int d[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                const bool ok = r0 + 2 * by + j < R && c0 + 2 * bx < C;
+                d[j] = *reinterpret_cast<const int*>(
+                    in + base + (ok ? ((size_t)(r0 + 2 * by + j) * C + c0 + 2 * bx) * 2 : 0));
+            }
+            const int lo = __builtin_amdgcn_perm(d[1], d[0], 0x05040100);    // column 2bx: rows 2by, 2by+1
+            const int hi = __builtin_amdgcn_perm(d[1], d[0], 0x07060302);
+            *reinterpret_cast<int*>(tile + (2 * bx) * kRow + 4 * by)     = lo;
+            *reinterpret_cast<int*>(tile + (2 * bx + 1) * kRow + 4 * by) = hi;
+        }
+    }
+    __syncthreads();
+    // 16-byte pieces of the transposed rows: 4 * EB pieces per row
+    constexpr int kPieces = 4 * EB;
+#pragma unroll
+    for (int k = 0; k < EB; k++)
+    {
+        const int idx  = tid + 256 * k;
+        const int c    = idx / kPieces;
+        const int part = idx % kPieces;
+        const int r    = r0 + part * (16 / EB);
+        if (c0 + c < C && r < R)
+            *reinterpret_cast<tr_v4i*>(out + base + ((size_t)(c0 + c) * R + r) * EB) =
+                *reinterpret_cast<const tr_v4i*>(tile + c * kRow + part * 16);
+    }
+}
+
 const char* launch_transpose(hipStream_t st, int32_t elem_bytes, int32_t N, int32_t R, int32_t C, const void* in,
                              void* out)
 {
     if ((int64_t)N * R * C == 0)
         return "transpose_empty";
     const dim3 grid((C + 63) / 64, (R + 63) / 64, N);
-    if (elem_bytes == 1)
+    const bool pieces = (elem_bytes == 1 || elem_bytes == 2) && ((int64_t)C * elem_bytes) % 4 == 0 &&
+                        ((int64_t)R * elem_bytes) % 16 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0;
+    if (pieces && elem_bytes == 1)
+        hipLaunchKernelGGL(transpose_vec_kernel<1>, grid, dim3(256), 0, st, R, C, (const uint8_t*)in, (uint8_t*)out);
+    else if (pieces)
+        hipLaunchKernelGGL(transpose_vec_kernel<2>, grid, dim3(256), 0, st, R, C, (const uint8_t*)in, (uint8_t*)out);
+    else if (elem_bytes == 1)
         hipLaunchKernelGGL(transpose_kernel<uint8_t>, grid, dim3(256), 0, st, R, C, (const uint8_t*)in, (uint8_t*)out);
     else if (elem_bytes == 2)
         hipLaunchKernelGGL(transpose_kernel<uint16_t>, grid, dim3(256), 0, st, R, C, (const uint16_t*)in,
