@@ -35,7 +35,7 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X, published)
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by a
 # plain copy kernel of known size (see profiles/*_pmc.txt); None where not measured.
-MEASURED_TRAFFIC_BYTES = {"c3": 3693001, "c2": 174113648, "c4": 17376255, "c5a": 34578561, "c5b": 3126818328}
+MEASURED_TRAFFIC_BYTES = {"c3": 3718552, "c2": 78442023, "c4": 12187828, "c5a": 22517189, "c5b": 492198669}
 
 
 def main() -> int:
