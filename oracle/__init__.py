@@ -1,7 +1,7 @@
 """CPU oracle for the TOSA tensor-op hot path -- TEST INFRASTRUCTURE ONLY.
 
 numpy front end of ``libtosa_oracle.so`` (``tosa_oracle.c``), the plain-C restatement of the TOSA
-reference model's CONV2D / DEPTHWISE_CONV2D / MATMUL / RESCALE / CLAMP arithmetic.  Only the tests,
+reference model's CONV2D / DEPTHWISE_CONV2D / MATMUL / RESCALE / CLAMP (and CONV3D / TRANSPOSE_CONV2D) arithmetic.  Only the tests,
 the smoke test and the benchmark's CPU-baseline leg may import this package; the shipped library
 never does.
 """
@@ -160,6 +160,81 @@ def depthwise_conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilati
                                  ctypes.c_int(int(abs_mode)), _ptr(out))
     _check(rc)
     return out
+
+
+class Conv3dShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("N", "ID", "IH", "IW", "IC", "OC", "KD", "KH", "KW", "OD", "OH", "OW")] + [
+        ("pad", ctypes.c_int32 * 6), ("stride", ctypes.c_int32 * 3), ("dilation", ctypes.c_int32 * 3),
+        ("bias_len", ctypes.c_int32)]
+
+
+class TconvShape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("N", "IH", "IW", "IC", "OC", "KH", "KW", "OH", "OW")] + [
+        ("out_pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("bias_len", ctypes.c_int32)]
+
+
+def conv3d_out_dhw(idhw, kdhw, pad, stride, dilation):
+    """Output depth/height/width rule of check_conv_attribute for three dimensions; None if inexact."""
+    out = []
+    for i in range(3):
+        full = idhw[i] - 1 + pad[2 * i] + pad[2 * i + 1] - (kdhw[i] - 1) * dilation[i]
+        if stride[i] < 1 or full < 0 or full % stride[i]:
+            return None
+        out.append(full // stride[i] + 1)
+    return tuple(out)
+
+
+def _dispatch(prefix, kind, s, inp, w, bias, in_zp, w_zp, abs_mode, out):
+    L = lib()
+    if kind in ("i8", "i32"):
+        rc = getattr(L, f"{prefix}_{kind}")(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp),
+                                            ctypes.c_int32(w_zp), _ptr(out))
+    elif kind == "f32":
+        rc = getattr(L, f"{prefix}_f32")(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), _ptr(out))
+    else:
+        rc = getattr(L, f"{prefix}_f64")(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias),
+                                         ctypes.c_int(int(abs_mode)), _ptr(out))
+    _check(rc)
+    return out
+
+
+def conv3d(kind, inp, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), in_zp=0, w_zp=0,
+           abs_mode=False, out_dhw=None):
+    """CONV3D.  inp [N,D,H,W,C], w [OC,KD,KH,KW,C], bias [1] or [OC]."""
+    et, bt, ot = _KINDS[kind]
+    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    if w.shape[4] != inp.shape[4]:
+        raise OracleStatus(ERROR)
+    if out_dhw is None:
+        out_dhw = conv3d_out_dhw(inp.shape[1:4], w.shape[1:4], pad, stride, dilation) or (-1, -1, -1)
+    s = Conv3dShape()
+    s.N, s.ID, s.IH, s.IW, s.IC = inp.shape
+    s.OC, s.KD, s.KH, s.KW = w.shape[:4]
+    s.OD, s.OH, s.OW = out_dhw
+    s.pad[:], s.stride[:], s.dilation[:] = list(pad), list(stride), list(dilation)
+    s.bias_len = int(bias.shape[0])
+    out = np.zeros((s.N,) + tuple(max(v, 0) for v in out_dhw) + (s.OC,), dtype=ot)
+    return _dispatch("orc_conv3d", kind, s, inp, w, bias, in_zp, w_zp, abs_mode, out)
+
+
+def transpose_conv2d(kind, inp, w, bias, out_pad=(0, 0, 0, 0), stride=(1, 1), in_zp=0, w_zp=0, abs_mode=False,
+                     out_hw=None):
+    """TRANSPOSE_CONV2D.  inp NHWC, w OHWI, bias [1] or [OC]."""
+    et, bt, ot = _KINDS[kind]
+    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    if w.shape[3] != inp.shape[3]:
+        raise OracleStatus(ERROR)
+    n, ih, iw, ic = inp.shape
+    oc, kh, kw, _ = w.shape
+    if out_hw is None:
+        out_hw = ((ih - 1) * stride[0] + out_pad[0] + out_pad[1] + kh, (iw - 1) * stride[1] + out_pad[2] + out_pad[3] + kw)
+    s = TconvShape()
+    s.N, s.IH, s.IW, s.IC, s.OC, s.KH, s.KW = n, ih, iw, ic, oc, kh, kw
+    s.OH, s.OW = out_hw
+    s.out_pad[:], s.stride[:] = list(out_pad), list(stride)
+    s.bias_len = int(bias.shape[0])
+    out = np.zeros((n, max(out_hw[0], 0), max(out_hw[1], 0), oc), dtype=ot)
+    return _dispatch("orc_transpose_conv2d", kind, s, inp, w, bias, in_zp, w_zp, abs_mode, out)
 
 
 def matmul(kind, a, b, a_zp=0, b_zp=0, abs_mode=False):

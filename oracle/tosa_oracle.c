@@ -164,6 +164,205 @@ int orc_conv2d_i8(const orc_conv_shape_t* s, const int8_t* in, const int8_t* w, 
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * OpConv3d (tensor_ops.cpp:901-1120): check_conv_attribute with conv_dimension 3 (:120-226), then
+ * ob,od,oy,ox,oc x kd,ky,kx x ic on a copy padded with input_zp, out-of-volume taps skipped
+ * (:1079-1087; bounds mode visits them, contributing zero), out = bias + acc (:1104-1105).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_conv3d_check(const orc_conv3d_shape_t* s)
+{
+    for (int i = 0; i < 6; i++)
+        if (s->pad[i] < 0)
+            return ORC_ERROR;
+    for (int i = 0; i < 3; i++)
+        if (s->stride[i] < 1 || s->dilation[i] < 1)
+            return ORC_ERROR;
+    const int32_t full_d = s->ID - 1 + s->pad[0] + s->pad[1] - (s->KD - 1) * s->dilation[0];
+    const int32_t full_h = s->IH - 1 + s->pad[2] + s->pad[3] - (s->KH - 1) * s->dilation[1];
+    const int32_t full_w = s->IW - 1 + s->pad[4] + s->pad[5] - (s->KW - 1) * s->dilation[2];
+    if ((full_d % s->stride[0]) != 0 || (full_h % s->stride[1]) != 0 || (full_w % s->stride[2]) != 0)
+        return ORC_ERROR;
+    if (s->OD != full_d / s->stride[0] + 1 || s->OH != full_h / s->stride[1] + 1 || s->OW != full_w / s->stride[2] + 1)
+        return ORC_ERROR;
+    if (s->bias_len != s->OC && s->bias_len != 1)
+        return ORC_ERROR;
+    return ORC_VALID;
+}
+
+#define ORC_DEFINE_CONV3D(NAME, T, ABS_EXPR)                                                                       \
+    static int NAME(const orc_conv3d_shape_t* s, const T* in, const T* w, const T* bias, T in_zp, T w_zp,        \
+                    int abs_mode, T* out)                                                                          \
+    {                                                                                                              \
+        if (orc_conv3d_check(s) != ORC_VALID)                                                                      \
+            return ORC_ERROR;                                                                                      \
+        const int N = s->N, ID = s->ID, IH = s->IH, IW = s->IW, IC = s->IC, OC = s->OC;                            \
+        const int KD = s->KD, KH = s->KH, KW = s->KW, OD = s->OD, OH = s->OH, OW = s->OW;                          \
+        for (int ob = 0; ob < N; ob++)                                                                             \
+            for (int od = 0; od < OD; od++)                                                                        \
+                for (int oy = 0; oy < OH; oy++)                                                                    \
+                    for (int ox = 0; ox < OW; ox++)                                                                \
+                        for (int oc = 0; oc < OC; oc++)                                                            \
+                        {                                                                                          \
+                            T acc = 0;                                                                             \
+                            for (int kd = 0; kd < KD; kd++)                                                        \
+                                for (int ky = 0; ky < KH; ky++)                                                    \
+                                    for (int kx = 0; kx < KW; kx++)                                                \
+                                    {                                                                              \
+                                        const int d = od * s->stride[0] + kd * s->dilation[0] - s->pad[0];         \
+                                        const int y = oy * s->stride[1] + ky * s->dilation[1] - s->pad[2];         \
+                                        const int x = ox * s->stride[2] + kx * s->dilation[2] - s->pad[4];         \
+                                        const int in_scope =                                                       \
+                                            0 <= x && x < IW && 0 <= y && y < IH && 0 <= d && d < ID;              \
+                                        if (!in_scope)                                                             \
+                                            continue; /* the padded value is input_zp: contributes zero */         \
+                                        const T* ip = in + ((((size_t)ob * ID + d) * IH + y) * IW + x) * IC;       \
+                                        const T* wp = w + ((((size_t)oc * KD + kd) * KH + ky) * KW + kx) * IC;     \
+                                        for (int ic = 0; ic < IC; ic++)                                            \
+                                        {                                                                          \
+                                            T a = ip[ic], b = wp[ic];                                              \
+                                            if (abs_mode)                                                          \
+                                                a = ABS_EXPR(a), b = ABS_EXPR(b);                                  \
+                                            acc += (a - in_zp) * (b - w_zp);                                       \
+                                        }                                                                          \
+                                    }                                                                              \
+                            T b = bias[s->bias_len == 1 ? 0 : oc];                                                 \
+                            if (abs_mode)                                                                          \
+                                b = ABS_EXPR(b);                                                                   \
+                            out[((((size_t)ob * OD + od) * OH + oy) * OW + ox) * OC + oc] = b + acc;               \
+                        }                                                                                          \
+        return ORC_VALID;                                                                                          \
+    }
+
+ORC_DEFINE_CONV3D(conv3d_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_CONV3D(conv3d_f32_impl, float, ORC_ABS_F32)
+ORC_DEFINE_CONV3D(conv3d_f64_impl, double, ORC_ABS_F64)
+
+int orc_conv3d_i32(const orc_conv3d_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                   int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    return conv3d_i32_impl(s, in, w, bias, in_zp, w_zp, 0, out);
+}
+
+int orc_conv3d_f32(const orc_conv3d_shape_t* s, const float* in, const float* w, const float* bias, float* out)
+{
+    return conv3d_f32_impl(s, in, w, bias, 0.0f, 0.0f, 0, out);
+}
+
+int orc_conv3d_f64(const orc_conv3d_shape_t* s, const double* in, const double* w, const double* bias, int abs_mode,
+                   double* out)
+{
+    return conv3d_f64_impl(s, in, w, bias, 0.0, 0.0, abs_mode, out);
+}
+
+int orc_conv3d_i8(const orc_conv3d_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias, int32_t in_zp,
+                  int32_t w_zp, int32_t* out)
+{
+    if (orc_conv3d_check(s) != ORC_VALID)
+        return ORC_ERROR;
+    int32_t* in32 = widen_i8(in, (size_t)s->N * s->ID * s->IH * s->IW * s->IC);
+    int32_t* w32  = widen_i8(w, (size_t)s->OC * s->KD * s->KH * s->KW * s->IC);
+    int rc        = (in32 && w32) ? orc_conv3d_i32(s, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
+    free(in32);
+    free(w32);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * OpTransposeConv2d (tensor_ops.cpp:1982-2197): out_pad > -kernel (:2037-2041), output size
+ * (IH-1)*stride + out_pad + kernel (:2043-2053); eval: for every output element and tap (ky,kx) the
+ * input position y = oy - out_pad_top - ky, x = ox - out_pad_left - kx is used when it is inside
+ * [0, IH*sy) x [0, IW*sx) and a multiple of the stride (:2155-2165); out = acc + bias (:2183-2184).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_tconv_check(const orc_tconv_shape_t* s)
+{
+    if (s->stride[0] < 1 || s->stride[1] < 1)
+        return ORC_ERROR;
+    if (s->out_pad[0] <= -s->KH || s->out_pad[1] <= -s->KH || s->out_pad[2] <= -s->KW || s->out_pad[3] <= -s->KW)
+        return ORC_ERROR;
+    if (s->OH != (s->IH - 1) * s->stride[0] + s->out_pad[0] + s->out_pad[1] + s->KH ||
+        s->OW != (s->IW - 1) * s->stride[1] + s->out_pad[2] + s->out_pad[3] + s->KW)
+        return ORC_ERROR;
+    if (s->bias_len != s->OC && s->bias_len != 1)
+        return ORC_ERROR;
+    return ORC_VALID;
+}
+
+#define ORC_DEFINE_TCONV(NAME, T, ABS_EXPR)                                                                        \
+    static int NAME(const orc_tconv_shape_t* s, const T* in, const T* w, const T* bias, T in_zp, T w_zp,         \
+                    int abs_mode, T* out)                                                                          \
+    {                                                                                                              \
+        if (orc_tconv_check(s) != ORC_VALID)                                                                       \
+            return ORC_ERROR;                                                                                      \
+        const int N = s->N, IH = s->IH, IW = s->IW, IC = s->IC, OC = s->OC, KH = s->KH, KW = s->KW;                \
+        const int OH = s->OH, OW = s->OW, sy = s->stride[0], sx = s->stride[1];                                    \
+        for (int ob = 0; ob < N; ob++)                                                                             \
+            for (int oy = 0; oy < OH; oy++)                                                                        \
+                for (int ox = 0; ox < OW; ox++)                                                                    \
+                    for (int oc = 0; oc < OC; oc++)                                                                \
+                    {                                                                                              \
+                        const int iy = oy - s->out_pad[0], ix = ox - s->out_pad[2];                                \
+                        T acc = 0;                                                                                 \
+                        for (int ky = 0; ky < KH; ky++)                                                            \
+                            for (int kx = 0; kx < KW; kx++)                                                        \
+                            {                                                                                      \
+                                const int y = iy - ky, x = ix - kx;                                                \
+                                const int in_scope = 0 <= y && y < IH * sy && 0 <= x && x < IW * sx &&             \
+                                                     (y % sy) == 0 && (x % sx) == 0;                               \
+                                if (!in_scope)                                                                     \
+                                    continue; /* extra multiplies would add 0 * weight */                          \
+                                const T* ip = in + (((size_t)ob * IH + y / sy) * IW + x / sx) * IC;                \
+                                const T* wp = w + (((size_t)oc * KH + ky) * KW + kx) * IC;                         \
+                                for (int ic = 0; ic < IC; ic++)                                                    \
+                                {                                                                                  \
+                                    T a = ip[ic], b = wp[ic];                                                      \
+                                    if (abs_mode)                                                                  \
+                                        a = ABS_EXPR(a), b = ABS_EXPR(b);                                          \
+                                    acc += (a - in_zp) * (b - w_zp);                                               \
+                                }                                                                                  \
+                            }                                                                                      \
+                        T b = bias[s->bias_len == 1 ? 0 : oc];                                                     \
+                        if (abs_mode)                                                                              \
+                            b = ABS_EXPR(b);                                                                       \
+                        out[(((size_t)ob * OH + oy) * OW + ox) * OC + oc] = acc + b;                               \
+                    }                                                                                              \
+        return ORC_VALID;                                                                                          \
+    }
+
+ORC_DEFINE_TCONV(tconv_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_TCONV(tconv_f32_impl, float, ORC_ABS_F32)
+ORC_DEFINE_TCONV(tconv_f64_impl, double, ORC_ABS_F64)
+
+int orc_transpose_conv2d_i32(const orc_tconv_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                             int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    return tconv_i32_impl(s, in, w, bias, in_zp, w_zp, 0, out);
+}
+
+int orc_transpose_conv2d_f32(const orc_tconv_shape_t* s, const float* in, const float* w, const float* bias,
+                             float* out)
+{
+    return tconv_f32_impl(s, in, w, bias, 0.0f, 0.0f, 0, out);
+}
+
+int orc_transpose_conv2d_f64(const orc_tconv_shape_t* s, const double* in, const double* w, const double* bias,
+                             int abs_mode, double* out)
+{
+    return tconv_f64_impl(s, in, w, bias, 0.0, 0.0, abs_mode, out);
+}
+
+int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias,
+                            int32_t in_zp, int32_t w_zp, int32_t* out)
+{
+    if (orc_tconv_check(s) != ORC_VALID)
+        return ORC_ERROR;
+    int32_t* in32 = widen_i8(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int32_t* w32  = widen_i8(w, (size_t)s->OC * s->KH * s->KW * s->IC);
+    int rc        = (in32 && w32) ? orc_transpose_conv2d_i32(s, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
+    free(in32);
+    free(w32);
+    return rc;
+}
+
+/* ------------------------------------------------------------------------------------------------
  * OpDepthwiseConv2d::eval (tensor_ops.cpp:1172-1334): ob,oy,ox,ic,km x ky,kx; an out-of-image tap
  * contributes zero (:1302-1313); weight [KH,KW,IC,M]; output channel ic*M+km (:1320).
  * ---------------------------------------------------------------------------------------------- */

@@ -1,5 +1,6 @@
 /*
- * CPU oracle for the TOSA tensor-op hot path (CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP).
+ * CPU oracle for the TOSA tensor-op hot path (CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP) and its
+ * neighbours CONV3D and TRANSPOSE_CONV2D.
  *
  * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the arithmetic of the TOSA reference
  * model, used as the checker in the parity tests, in the smoke test and as the timed CPU baseline.
@@ -15,6 +16,9 @@
  *     reference_model/test/ref_model_tests/tensor_ops_tests.cpp:622-683,736-798.
  *   - rescale: type_conversion_tests.cpp:324-405 literals, Python big-integer brute force of
  *     quant_util.h:45-84 and the boundary operands of generate_int_special.cpp:119-131.
+ *   - conv3d / transpose_conv2d: the literal vectors of tensor_ops_tests.cpp:268-446,622-766 (zero points,
+ *     bias broadcast) and an independent numpy restatement (correlation of the zero-upsampled input with the
+ *     flipped kernel for TRANSPOSE_CONV2D; per-depth-tap sums of 2-D convolutions for CONV3D).
  *   - large shapes: independent numpy int64 einsum / float64 convolution.
  *   - fp accumulate order of MATMUL (Eigen contraction order): parity unpinned (tolerance covered).
  */
@@ -81,6 +85,47 @@ int orc_depthwise_f32(const orc_conv_shape_t* s, int32_t M, const float* in, con
                       float* out);
 int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, const double* w, const double* bias,
                       int abs_mode, double* out);
+
+/* CONV3D (tensor_ops.cpp:901-1120): input [N,ID,IH,IW,IC], weight [OC,KD,KH,KW,IC], output [N,OD,OH,OW,OC]. */
+typedef struct
+{
+    int32_t N, ID, IH, IW, IC;
+    int32_t OC, KD, KH, KW;
+    int32_t OD, OH, OW;
+    int32_t pad[6];      /* d0, d1, top, bottom, left, right */
+    int32_t stride[3];   /* d, y, x */
+    int32_t dilation[3]; /* d, y, x */
+    int32_t bias_len;
+} orc_conv3d_shape_t;
+int orc_conv3d_check(const orc_conv3d_shape_t* s);
+int orc_conv3d_i32(const orc_conv3d_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                   int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_conv3d_i8(const orc_conv3d_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias, int32_t in_zp,
+                  int32_t w_zp, int32_t* out);
+int orc_conv3d_f32(const orc_conv3d_shape_t* s, const float* in, const float* w, const float* bias, float* out);
+int orc_conv3d_f64(const orc_conv3d_shape_t* s, const double* in, const double* w, const double* bias, int abs_mode,
+                   double* out);
+
+/* TRANSPOSE_CONV2D (tensor_ops.cpp:1982-2197): input NHWC, weight OHWI, OH = (IH-1)*sy + out_pad_top +
+ * out_pad_bottom + KH. */
+typedef struct
+{
+    int32_t N, IH, IW, IC;
+    int32_t OC, KH, KW;
+    int32_t OH, OW;
+    int32_t out_pad[4]; /* top, bottom, left, right; each > -kernel size */
+    int32_t stride[2];  /* y, x */
+    int32_t bias_len;
+} orc_tconv_shape_t;
+int orc_tconv_check(const orc_tconv_shape_t* s);
+int orc_transpose_conv2d_i32(const orc_tconv_shape_t* s, const int32_t* in, const int32_t* w, const int32_t* bias,
+                             int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias,
+                            int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_transpose_conv2d_f32(const orc_tconv_shape_t* s, const float* in, const float* w, const float* bias,
+                             float* out);
+int orc_transpose_conv2d_f64(const orc_tconv_shape_t* s, const double* in, const double* w, const double* bias,
+                             int abs_mode, double* out);
 
 /* MATMUL a[N,H,C] x b[N,C,W] -> out[N,H,W]. */
 int orc_matmul_i32(int32_t N, int32_t H, int32_t C, int32_t W, const int32_t* a, const int32_t* b, int32_t a_zp,
