@@ -130,6 +130,34 @@ typedef struct
     int32_t bias_len;    /* 1 (broadcast) or OC */
 } tmi_conv_desc_t;
 
+/* TransposeConv2dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:1982-2056).
+ * input NHWC, weight OHWI, output [N,OH,OW,OC] with OH = (IH-1)*stride_y + out_pad_top + out_pad_bottom + KH. */
+typedef struct
+{
+    int32_t in_dtype;    /* TMI_INT8 / TMI_FP16 / TMI_BF16 */
+    int32_t out_dtype;   /* TMI_INT32 for INT8, else the input type */
+    int32_t N, IH, IW, IC;
+    int32_t OC, KH, KW;
+    int32_t OH, OW;
+    int32_t out_pad[4];  /* top, bottom, left, right; each > -kernel size */
+    int32_t stride[2];   /* y, x */
+    int32_t bias_len;    /* 1 (broadcast) or OC */
+} tmi_tconv_desc_t;
+
+/* Conv3dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:901-933, check :120-226).
+ * input [N,ID,IH,IW,IC], weight [OC,KD,KH,KW,IC], output [N,OD,OH,OW,OC]. */
+typedef struct
+{
+    int32_t in_dtype, out_dtype;
+    int32_t N, ID, IH, IW, IC;
+    int32_t OC, KD, KH, KW;
+    int32_t OD, OH, OW;
+    int32_t pad[6];      /* d0, d1, top, bottom, left, right */
+    int32_t stride[3];   /* d, y, x */
+    int32_t dilation[3]; /* d, y, x */
+    int32_t bias_len;
+} tmi_conv3d_desc_t;
+
 /* RescaleAttribute plus the operand facts OpRescale::checkTensorAttributes / eval read
  * (reference_model/src/ops/type_conversion.cpp:111-151, 226-255). */
 typedef struct
@@ -190,6 +218,17 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
                                        const tmi_rescale_desc_t* r, const void* multiplier_dev,
                                        const void* shift_dev, int32_t has_clamp, int32_t clamp_min,
                                        int32_t clamp_max, void* out_dev);
+
+/* OpTransposeConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:2058-2197 (checks :1982-2056).
+ * Evaluated as a stride-1 CONV2D with flipped taps over the input with stride-1 holes filled with input_zp;
+ * the re-laid-out operands live in the context's scratch buffer. */
+int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
+
+/* OpConv3d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:935-1120 (checks :901-933, :120-226).
+ * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side. */
+int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
+               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
 /* ---- validation only (no launch) ---------------------------------------------------------------- */
 

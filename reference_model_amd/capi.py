@@ -30,6 +30,7 @@ EXPORTS = [
     "tmi_last_error", "tmi_last_kernel", "tmi_buf_alloc", "tmi_buf_free", "tmi_upload", "tmi_download",
     "tmi_conv2d", "tmi_depthwise_conv2d", "tmi_matmul", "tmi_rescale", "tmi_clamp", "tmi_conv2d_rescale_clamp",
     "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice", "tmi_conv2d_check", "tmi_rescale_check",
+    "tmi_transpose_conv2d", "tmi_conv3d",
 ]
 
 
@@ -42,6 +43,19 @@ class ConvDesc(ctypes.Structure):
         ("pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("dilation", ctypes.c_int32 * 2),
         ("bias_len", ctypes.c_int32),
     ]
+
+
+class TconvDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("in_dtype", "out_dtype", "N", "IH", "IW", "IC", "OC", "KH", "KW", "OH",
+                                              "OW")] + [
+        ("out_pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("bias_len", ctypes.c_int32)]
+
+
+class Conv3dDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("in_dtype", "out_dtype", "N", "ID", "IH", "IW", "IC", "OC", "KD", "KH",
+                                              "KW", "OD", "OH", "OW")] + [
+        ("pad", ctypes.c_int32 * 6), ("stride", ctypes.c_int32 * 3), ("dilation", ctypes.c_int32 * 3),
+        ("bias_len", ctypes.c_int32)]
 
 
 class RescaleDesc(ctypes.Structure):
@@ -241,6 +255,14 @@ class Context:
     # -- operators (device pointers in, status out) ------------------------------------------
     def conv2d(self, d: ConvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias),
+                                               in_zp, w_zp, _ptr(out)))
+
+    def transpose_conv2d(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
+        return self._check(self.lib.tmi_transpose_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
+                                                         _ptr(bias), in_zp, w_zp, _ptr(out)))
+
+    def conv3d(self, d: Conv3dDesc, inp, w, bias, in_zp, w_zp, out) -> int:
+        return self._check(self.lib.tmi_conv3d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias),
                                                in_zp, w_zp, _ptr(out)))
 
     def depthwise_conv2d(self, d: ConvDesc, inp, w, bias, in_zp, w_zp, out) -> int:

@@ -512,6 +512,160 @@ int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, con
                     d ? d->out_dtype : 0, out_dev);
 }
 
+static size_t align256(size_t v)
+{
+    return (v + 255) & ~(size_t)255;
+}
+
+int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    const char* op = "OpTransposeConv2d";
+    if (!d)
+        return fail(ctx, "%s: null descriptor", op);
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+        return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
+    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
+        return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1)
+        return fail(ctx, "%s: negative tensor dimension", op);
+    // checkTensorAttributes (tensor_ops.cpp:2017-2053)
+    for (int i = 0; i < 2; i++)
+        if (d->stride[i] < 1)
+            return fail(ctx, "%s: At least one stride is smaller than one", op);
+    for (int i = 0; i < 4; i++)
+        if (d->out_pad[i] <= -(i < 2 ? d->KH : d->KW))
+            return fail(ctx, "%s: At least one out_pad value is larger than kernel size", op);
+    const int64_t H = (int64_t)(d->IH - 1) * d->stride[0] + d->out_pad[0] + d->out_pad[1] + d->KH;
+    const int64_t W = (int64_t)(d->IW - 1) * d->stride[1] + d->out_pad[2] + d->out_pad[3] + d->KW;
+    if (d->OH != H || d->OW != W)
+        return fail(ctx, "%s: Mismatch between output shape provided and expected output shape (%lld,%lld)", op,
+                    (long long)H, (long long)W);
+    if (d->bias_len != d->OC && d->bias_len != 1)
+        return fail(ctx, "%s: bias channels mismatch %d != %d", op, d->bias_len, d->OC);
+    if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
+        return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    const int64_t total = (int64_t)d->N * d->OH * d->OW * d->OC;
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    if (!in_dev || !weight_dev || !bias_dev || !out_dev)
+        return fail(ctx, "%s: null tensor pointer", op);
+    if (d->IH == 0 || d->IW == 0 || d->IC == 0)
+        return fail(ctx, "%s: empty input with a non-empty output", op);
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+
+    // the equivalent CONV2D: flipped taps, stride 1, pads KH-1+out_pad, input with holes between its pixels
+    const int eb         = dtype_bits(d->in_dtype) / 8;
+    const int row_bytes  = d->IC * eb;
+    const bool holes     = d->stride[0] > 1 || d->stride[1] > 1;
+    const int32_t UH     = (d->IH - 1) * d->stride[0] + 1, UW = (d->IW - 1) * d->stride[1] + 1;
+    const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * row_bytes);
+    const size_t u_bytes = holes ? align256((size_t)d->N * UH * UW * row_bytes) : 0;
+    int rc               = ensure_workspace(ctx, w_bytes + u_bytes);
+    if (rc != TMI_VALID)
+        return rc;
+    uint8_t* w_flip = (uint8_t*)ctx->workspace;
+    uint8_t* u      = w_flip + w_bytes;
+    if (!launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip))
+        return fail(ctx, "%s: weight re-layout launch failed", op);
+    if (holes && !launch_upsample(ctx->stream, row_bytes, d->N, d->IH, d->IW, d->stride[0], d->stride[1], in_zp,
+                                  in_dev, u))
+        return fail(ctx, "%s: input re-layout launch failed", op);
+    tmi_conv_desc_t c{};
+    c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
+    c.N = d->N, c.IH = UH, c.IW = UW, c.IC = d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW, c.OH = d->OH, c.OW = d->OW;
+    c.pad[0] = d->KH - 1 + d->out_pad[0], c.pad[1] = d->KH - 1 + d->out_pad[1];
+    c.pad[2] = d->KW - 1 + d->out_pad[2], c.pad[3] = d->KW - 1 + d->out_pad[3];
+    c.stride[0] = c.stride[1] = 1, c.dilation[0] = c.dilation[1] = 1;
+    c.bias_len = d->bias_len;
+    RescaleParams none{};
+    return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
+                    d->out_dtype, out_dev);
+}
+
+int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
+               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    const char* op = "OpConv3d";
+    if (!d)
+        return fail(ctx, "%s: null descriptor", op);
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+        return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
+    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
+        return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    if (d->N < 0 || d->ID < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KD < 1 || d->KH < 1 ||
+        d->KW < 1)
+        return fail(ctx, "%s: negative tensor dimension", op);
+    // check_conv_attribute with three dimensions (tensor_ops.cpp:120-226)
+    for (int i = 0; i < 6; i++)
+        if (d->pad[i] < 0)
+            return fail(ctx, "%s: At least one pad is smaller than zero", op);
+    for (int i = 0; i < 3; i++)
+        if (d->stride[i] < 1)
+            return fail(ctx, "%s: At least one stride dimension is smaller than one", op);
+    for (int i = 0; i < 3; i++)
+        if (d->dilation[i] < 1)
+            return fail(ctx, "%s: At least one dilation dimension is smaller than one", op);
+    const int64_t full_d = (int64_t)d->ID - 1 + d->pad[0] + d->pad[1] - (int64_t)(d->KD - 1) * d->dilation[0];
+    const int64_t full_h = (int64_t)d->IH - 1 + d->pad[2] + d->pad[3] - (int64_t)(d->KH - 1) * d->dilation[1];
+    const int64_t full_w = (int64_t)d->IW - 1 + d->pad[4] + d->pad[5] - (int64_t)(d->KW - 1) * d->dilation[2];
+    if ((full_d % d->stride[0]) != 0 || (full_h % d->stride[1]) != 0 || (full_w % d->stride[2]) != 0)
+        return fail(ctx, "%s: Parameters must yield exact integer output dimensions", op);
+    if (d->OD != full_d / d->stride[0] + 1 || d->OH != full_h / d->stride[1] + 1 ||
+        d->OW != full_w / d->stride[2] + 1)
+        return fail(ctx, "%s: Mismatch between output shape provided and expected output shape (%lld,%lld,%lld)", op,
+                    (long long)(full_d / d->stride[0] + 1), (long long)(full_h / d->stride[1] + 1),
+                    (long long)(full_w / d->stride[2] + 1));
+    if (d->bias_len != d->OC && d->bias_len != 1)
+        return fail(ctx, "%s: bias channel mismatch %d != %d", op, d->bias_len, d->OC);
+    if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
+        return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    const int64_t total = (int64_t)d->N * d->OD * d->OH * d->OW * d->OC;
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    if (!in_dev || !weight_dev || !bias_dev || !out_dev)
+        return fail(ctx, "%s: null tensor pointer", op);
+    if ((int64_t)d->N * d->OD > INT32_MAX || (int64_t)d->KD * d->IC > INT32_MAX)
+        return fail(ctx, "%s: shape too large", op);
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+
+    const int eb         = dtype_bits(d->in_dtype) / 8;
+    const int row_bytes  = d->IC * eb;
+    const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * row_bytes);
+    const size_t g_bytes = align256((size_t)d->N * d->OD * d->IH * d->IW * d->KD * row_bytes);
+    int rc               = ensure_workspace(ctx, w_bytes + g_bytes);
+    if (rc != TMI_VALID)
+        return rc;
+    uint8_t* w_perm = (uint8_t*)ctx->workspace;
+    uint8_t* gath   = w_perm + w_bytes;
+    if (!launch_permute_w3d(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm))
+        return fail(ctx, "%s: weight re-layout launch failed", op);
+    if (!launch_gather_depth(ctx->stream, row_bytes, d->N, d->ID, d->OD, d->KD, d->IH * d->IW, d->stride[0],
+                             d->dilation[0], d->pad[0], in_zp, in_dev, gath))
+        return fail(ctx, "%s: input re-layout launch failed", op);
+    tmi_conv_desc_t c{};
+    c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
+    c.N = d->N * d->OD, c.IH = d->IH, c.IW = d->IW, c.IC = d->KD * d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW;
+    c.OH = d->OH, c.OW = d->OW;
+    for (int i = 0; i < 4; i++)
+        c.pad[i] = d->pad[2 + i];
+    c.stride[0] = d->stride[1], c.stride[1] = d->stride[2];
+    c.dilation[0] = d->dilation[1], c.dilation[1] = d->dilation[2];
+    c.bias_len = d->bias_len;
+    RescaleParams none{};
+    return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev);
+}
+
 int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
 {

@@ -73,6 +73,16 @@ const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dty
 // elementwise.hip: [N, R, C] -> [N, C, R] for 1- or 2-byte elements (MATMUL's second operand becomes K-contiguous).
 const char* launch_transpose(hipStream_t st, int32_t elem_bytes, int32_t N, int32_t R, int32_t C, const void* in,
                              void* out);
+// relayout.hip: whole-channel-vector copies that turn TRANSPOSE_CONV2D / CONV3D operands into CONV2D operands.
+const char* launch_flip_taps(hipStream_t st, int32_t row_bytes, int32_t OC, int32_t KH, int32_t KW, const void* src,
+                             void* dst);
+const char* launch_upsample(hipStream_t st, int32_t row_bytes, int32_t N, int32_t IH, int32_t IW, int32_t sy,
+                            int32_t sx, int32_t fill, const void* src, void* dst);
+const char* launch_gather_depth(hipStream_t st, int32_t row_bytes, int32_t N, int32_t ID, int32_t OD, int32_t KD,
+                                int32_t HW, int32_t stride_d, int32_t dilation_d, int32_t pad_d0, int32_t fill,
+                                const void* src, void* dst);
+const char* launch_permute_w3d(hipStream_t st, int32_t row_bytes, int32_t OC, int32_t KD, int32_t KHW,
+                               const void* src, void* dst);
 // depthwise.hip: 4 channels per lane, dot4 across taps, fused epilogue; nullptr when not eligible.
 const char* launch_depthwise_vec(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                  const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,

@@ -1,0 +1,113 @@
+"""GPU parity of TRANSPOSE_CONV2D and CONV3D (evaluated as re-laid-out CONV2D problems) against the CPU oracle,
+through the C ABI.  int8 bit for bit; fp16 with the reference's DOT_PRODUCT bound against the fp64 oracle."""
+import numpy as np
+import pytest
+
+import dot_product_check as dp
+import gpu_ops
+import oracle
+from reference_model_amd import Context, TmiError, capi
+from test_oracle_conv3d_tconv import CONV3D_SHAPES, TCONV_SHAPES, ZP_CASES_2X2, ZP_CASES_2X2X2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", params=[capi.KERNEL_AUTO, capi.KERNEL_DIRECT], ids=["auto", "direct"])
+def ctx(request):
+    c = Context(0)
+    c.set_kernel_choice(request.param)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("case", ZP_CASES_2X2)
+def test_transpose_conv2d_reference_zero_point_cases(ctx, case):
+    vals, wts, izp, wzp = case
+    x = np.array(vals, np.int8).reshape(1, 2, 2, 1)
+    w = np.array(wts, np.int8).reshape(1, 2, 2, 1)
+    b = np.zeros(1, np.int32)
+    got, st = gpu_ops.transpose_conv2d(ctx, x, w, b, in_zp=izp, w_zp=wzp)
+    assert st == capi.VALID and np.array_equal(got, oracle.transpose_conv2d("i8", x, w, b, in_zp=izp, w_zp=wzp))
+
+
+@pytest.mark.parametrize("case", ZP_CASES_2X2X2)
+def test_conv3d_reference_zero_point_cases(ctx, case):
+    vals, wts, izp, wzp = case
+    x = np.array(vals, np.int8).reshape(1, 2, 2, 2, 1)
+    w = np.array(wts, np.int8).reshape(1, 2, 2, 2, 1)
+    got, st = gpu_ops.conv3d(ctx, x, w, np.zeros(1, np.int32), in_zp=izp, w_zp=wzp)
+    assert st == capi.VALID and got.reshape(-1).tolist() == [sum((a - izp) * (c - wzp) for a, c in zip(vals, wts))]
+
+
+BIG_TCONV = [
+    (2, 14, 14, 64, 48, 3, 3, (0, 0, 0, 0), (2, 2)),      # a decoder-style 2x upsampling layer
+    (1, 9, 12, 32, 40, 4, 4, (-1, -1, -1, -1), (2, 2)),   # negative out_pad crops the border
+    (1, 20, 20, 16, 16, 5, 1, (2, 0, 0, 3), (1, 3)),
+]
+
+
+@pytest.mark.parametrize("shape", TCONV_SHAPES + BIG_TCONV)
+@pytest.mark.parametrize("zps", [(-3, 9), (0, 0), (-128, 127)])
+def test_transpose_conv2d_i8_bit_exact(ctx, shape, zps):
+    n, ih, iw, ic, oc, kh, kw, out_pad, stride = shape
+    rng = np.random.default_rng(sum(shape[:7]) + zps[0] + 500)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
+    for bias in (rng.integers(-9999, 9999, oc).astype(np.int32), np.array([77], np.int32)):
+        want = oracle.transpose_conv2d("i8", x, w, bias, out_pad, stride, *zps)
+        got, st = gpu_ops.transpose_conv2d(ctx, x, w, bias, out_pad, stride, *zps)
+        assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+
+
+BIG_CONV3D = [
+    (1, 8, 12, 12, 16, 32, 3, 3, 3, (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    (2, 6, 9, 9, 32, 24, 2, 3, 3, (0, 0, 1, 1, 1, 1), (2, 2, 2), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("shape", CONV3D_SHAPES + BIG_CONV3D)
+@pytest.mark.parametrize("zps", [(6, -2), (0, 0)])
+def test_conv3d_i8_bit_exact(ctx, shape, zps):
+    n, idp, ih, iw, ic, oc, kd, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(sum(shape[:9]) + zps[0])
+    x = rng.integers(-128, 128, (n, idp, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kd, kh, kw, ic)).astype(np.int8)
+    for bias in (rng.integers(-9999, 9999, oc).astype(np.int32), np.array([-5], np.int32)):
+        want = oracle.conv3d("i8", x, w, bias, pad, stride, dil, *zps)
+        got, st = gpu_ops.conv3d(ctx, x, w, bias, pad, stride, dil, *zps)
+        assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+
+
+def test_fp16_variants_within_dot_product_bound(ctx):
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, (1, 6, 6, 32)).astype(np.float16)
+    w = rng.normal(0, 0.1, (16, 3, 3, 32)).astype(np.float16)
+    b = rng.normal(0, 0.1, 16).astype(np.float16)
+    got, st = gpu_ops.transpose_conv2d(ctx, x, w, b, (0, 1, 0, 1), (2, 2))
+    ref = oracle.transpose_conv2d("f64", x, w, b, (0, 1, 0, 1), (2, 2))
+    bnd = oracle.transpose_conv2d("f64", x, w, b, (0, 1, 0, 1), (2, 2), abs_mode=True)
+    res = dp.check(got.astype(np.float64), ref, bnd, "fp16", dp.kernel_size_bound(9 * 32, "fp16", has_bias=True))
+    # tolerance: |imp-ref| <= 2*ksb * max(bnd*2^-11, 2^-14) per element and sum err^2 <= 1.6*ksb*T (DOT_PRODUCT)
+    assert st == capi.VALID and res["ok"], res
+    x3 = rng.normal(0, 1, (1, 4, 5, 5, 16)).astype(np.float16)
+    w3 = rng.normal(0, 0.1, (8, 2, 3, 3, 16)).astype(np.float16)
+    b3 = rng.normal(0, 0.1, 8).astype(np.float16)
+    got, st = gpu_ops.conv3d(ctx, x3, w3, b3, (0, 0, 1, 1, 1, 1))
+    ref = oracle.conv3d("f64", x3, w3, b3, (0, 0, 1, 1, 1, 1))
+    bnd = oracle.conv3d("f64", x3, w3, b3, (0, 0, 1, 1, 1, 1), abs_mode=True)
+    res = dp.check(got.astype(np.float64), ref, bnd, "fp16", dp.kernel_size_bound(18 * 16, "fp16", has_bias=True))
+    assert st == capi.VALID and res["ok"], res
+
+
+def test_shape_rules_are_errors(ctx):
+    x, w, b = np.zeros((1, 2, 2, 1), np.int8), np.zeros((1, 3, 3, 1), np.int8), np.zeros(1, np.int32)
+    with pytest.raises(TmiError) as e:
+        gpu_ops.transpose_conv2d(ctx, x, w, b, out_pad=(-3, 0, 0, 0), out_hw=(1, 4))
+    assert e.value.status == capi.ERROR and "out_pad" in e.value.message
+    with pytest.raises(TmiError) as e:
+        gpu_ops.transpose_conv2d(ctx, x, w, b, out_hw=(5, 4))
+    assert "Mismatch between output shape" in e.value.message
+    x3, w3 = np.zeros((1, 4, 4, 4, 1), np.int8), np.zeros((1, 2, 2, 2, 1), np.int8)
+    with pytest.raises(TmiError) as e:
+        gpu_ops.conv3d(ctx, x3, w3, b, stride=(3, 1, 1), out_dhw=(1, 3, 3))
+    assert "exact integer output dimensions" in e.value.message
