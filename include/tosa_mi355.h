@@ -239,6 +239,12 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
  * anything is evaluated.  depthwise != 0 selects the DEPTHWISE_CONV2D rules. */
 int tmi_conv2d_check(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, int32_t depthwise);
 
+/* The checks of OpTransposeConv2d / OpConv3d::checkTensorAttributes and the heads of their eval()
+ * (reference_model/src/ops/tensor_ops.cpp:1982-2056, 2083-2091; 901-933, 963-970), for an adapter's
+ * checkTensorAttributes(). */
+int tmi_transpose_conv2d_check(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d);
+int tmi_conv3d_check(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d);
+
 /* OpRescale::checkTensorAttributes and the zero-point rules at the head of eval()
  * (reference_model/src/ops/type_conversion.cpp:72-154, 242-255). */
 int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int32_t C);

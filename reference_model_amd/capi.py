@@ -30,7 +30,7 @@ EXPORTS = [
     "tmi_last_error", "tmi_last_kernel", "tmi_buf_alloc", "tmi_buf_free", "tmi_upload", "tmi_download",
     "tmi_conv2d", "tmi_depthwise_conv2d", "tmi_matmul", "tmi_rescale", "tmi_clamp", "tmi_conv2d_rescale_clamp",
     "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice", "tmi_conv2d_check", "tmi_rescale_check",
-    "tmi_transpose_conv2d", "tmi_conv3d",
+    "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
 ]
 
 

@@ -5,7 +5,8 @@
 //   TosaBasicBlock  0 name, 1 operators[], 2 tensors[], 3 inputs[str], 4 outputs[str]
 //   TosaTensor      0 name, 1 shape[int32], 2 type(uint32), 3 data[ubyte]
 //   TosaOperator    0 op(uint32), 1 attribute_type(ubyte), 2 attribute(table), 3 inputs[str], 4 outputs[str]
-//   Conv2dAttribute / DepthwiseConv2dAttribute  0 pad, 1 stride, 2 dilation, 3 local_bound, 4 acc_type
+//   Conv2dAttribute / DepthwiseConv2dAttribute / Conv3dAttribute  0 pad, 1 stride, 2 dilation, 3 local_bound, 4 acc_type
+//   TransposeConv2dAttribute  0 out_pad, 1 stride, 2 local_bound, 3 acc_type
 //   RescaleAttribute  0 scale32, 1 rounding_mode, 2 per_channel, 3 input_unsigned, 4 output_unsigned
 //   ClampAttribute    0 min_val[ubyte], 1 max_val[ubyte], 2 nan_mode
 #include <cstdio>
@@ -42,6 +43,10 @@ const char* op_name(uint32_t op)
     {
         case Op_CONV2D:
             return "CONV2D";
+        case Op_CONV3D:
+            return "CONV3D";
+        case Op_TRANSPOSE_CONV2D:
+            return "TRANSPOSE_CONV2D";
         case Op_DEPTHWISE_CONV2D:
             return "DEPTHWISE_CONV2D";
         case Op_MATMUL:
@@ -234,7 +239,16 @@ bool load_tosa_file(const std::string& path, BasicBlock& block, std::string& err
         {
             switch (d.op)
             {
+                case Op_TRANSPOSE_CONV2D:    // out_pad, stride, local_bound, acc_type: the order of the
+                                             // reference's TosaTransposeConv2dAttribute constructor
+                                             // (tensor_ops_tests.cpp:293-296); no example graph confirms it
+                    d.attr.pad         = a.vec<int32_t>(0);
+                    d.attr.stride      = a.vec<int32_t>(1);
+                    d.attr.local_bound = a.scalar<uint8_t>(2, 0) != 0;
+                    d.attr.acc_type    = a.scalar<uint32_t>(3, 0);
+                    break;
                 case Op_CONV2D:
+                case Op_CONV3D:
                 case Op_DEPTHWISE_CONV2D:
                     d.attr.pad         = a.vec<int32_t>(0);
                     d.attr.stride      = a.vec<int32_t>(1);

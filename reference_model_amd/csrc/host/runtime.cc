@@ -391,6 +391,141 @@ public:
     OpDepthwiseConv2d(SubgraphTraverser* sgt, uint64_t id) : ConvBase(sgt, Op_DEPTHWISE_CONV2D, id, true) {}
 };
 
+// TRANSPOSE_CONV2D and CONV3D: operands [input, weight, bias, input_zp, weight_zp] like CONV2D
+// (tensor_ops.cpp:1974, :893); the checks are the C ABI's, run on a dry descriptor in checkTensorAttributes.
+class OpTransposeConv2d : public GraphNode
+{
+public:
+    OpTransposeConv2d(SubgraphTraverser* sgt, uint64_t id) : GraphNode(sgt, Op_TRANSPOSE_CONV2D, id)
+    {
+        requiredInputCount  = 5;
+        requiredOutputCount = 1;
+    }
+    int fill_desc(tmi_tconv_desc_t& d)
+    {
+        const Tensor *in = inputs[0], *w = inputs[1], *bias = inputs[2], *out = outputs[0];
+        if (attribute.pad.size() != 4)
+            return error("illegal size for attribute out_pad");
+        if (attribute.stride.size() != 2)
+            return error("illegal size for attribute stride");
+        memset(&d, 0, sizeof(d));
+        d.in_dtype = tmi_dtype(in->getDtype()), d.out_dtype = tmi_dtype(out->getDtype());
+        d.N = in->shape[0], d.IH = in->shape[1], d.IW = in->shape[2], d.IC = in->shape[3];
+        d.OC = w->shape[0], d.KH = w->shape[1], d.KW = w->shape[2];
+        if (w->shape[3] != d.IC)
+            return error("tensor input channel mismatch %d != %d", w->shape[3], d.IC);
+        if (out->shape[0] != d.N)
+            return error("tensor batch mismatch %d != %d", d.N, out->shape[0]);
+        if (out->shape[3] != d.OC)
+            return error("tensor output channel mismatch %d != %d", d.OC, out->shape[3]);
+        d.OH = out->shape[1], d.OW = out->shape[2];
+        for (int i = 0; i < 4; i++)
+            d.out_pad[i] = attribute.pad[i];
+        d.stride[0] = attribute.stride[0], d.stride[1] = attribute.stride[1];
+        d.bias_len = bias->shape[0];
+        return 0;
+    }
+    int checkTensorAttributes() override
+    {
+        if (validateRequiredOperands())
+            return 1;
+        if (validateRequiredRank(inputs[0], 4, 4) || validateRequiredRank(inputs[1], 4, 4) ||
+            validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
+            validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 4, 4))
+            return 1;
+        if (inputs[1]->getDtype() != inputs[0]->getDtype())
+            return error("weight data type not supported for this configuration of operator");
+        tmi_tconv_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        if (tmi_transpose_conv2d_check(parent_sgt->ctx, &d) != TMI_VALID)
+            return error("%s", tmi_last_error(parent_sgt->ctx));
+        return 0;
+    }
+    int eval() override
+    {
+        tmi_tconv_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        int32_t in_zp = 0, w_zp = 0;
+        if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
+            return error("zero-point operands must be available on the host");
+        SubgraphTraverser* s = parent_sgt;
+        if (call(tmi_transpose_conv2d(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]),
+                                      in_zp, w_zp, s->device_out(outputs[0]))))
+            return 1;
+        return GraphNode::eval();
+    }
+};
+
+class OpConv3d : public GraphNode
+{
+public:
+    OpConv3d(SubgraphTraverser* sgt, uint64_t id) : GraphNode(sgt, Op_CONV3D, id)
+    {
+        requiredInputCount  = 5;
+        requiredOutputCount = 1;
+    }
+    int fill_desc(tmi_conv3d_desc_t& d)
+    {
+        const Tensor *in = inputs[0], *w = inputs[1], *bias = inputs[2], *out = outputs[0];
+        if (attribute.pad.size() != 6)
+            return error("Illegal size for attribute pad");
+        if (attribute.stride.size() != 3)
+            return error("Illegal size for attribute stride");
+        if (attribute.dilation.size() != 3)
+            return error("Illegal size for attribute dilation");
+        memset(&d, 0, sizeof(d));
+        d.in_dtype = tmi_dtype(in->getDtype()), d.out_dtype = tmi_dtype(out->getDtype());
+        d.N = in->shape[0], d.ID = in->shape[1], d.IH = in->shape[2], d.IW = in->shape[3], d.IC = in->shape[4];
+        d.OC = w->shape[0], d.KD = w->shape[1], d.KH = w->shape[2], d.KW = w->shape[3];
+        if (w->shape[4] != d.IC)
+            return error("tensor input channel mismatch %d != %d", w->shape[4], d.IC);
+        if (out->shape[0] != d.N)
+            return error("tensor batch mismatch %d != %d", d.N, out->shape[0]);
+        if (out->shape[4] != d.OC)
+            return error("tensor output channel mismatch %d != %d", d.OC, out->shape[4]);
+        d.OD = out->shape[1], d.OH = out->shape[2], d.OW = out->shape[3];
+        for (int i = 0; i < 6; i++)
+            d.pad[i] = attribute.pad[i];
+        for (int i = 0; i < 3; i++)
+            d.stride[i] = attribute.stride[i], d.dilation[i] = attribute.dilation[i];
+        d.bias_len = bias->shape[0];
+        return 0;
+    }
+    int checkTensorAttributes() override
+    {
+        if (validateRequiredOperands())
+            return 1;
+        if (validateRequiredRank(inputs[0], 5, 5) || validateRequiredRank(inputs[1], 5, 5) ||
+            validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
+            validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 5, 5))
+            return 1;
+        if (inputs[1]->getDtype() != inputs[0]->getDtype())
+            return error("weight data type not supported for this configuration of operator");
+        tmi_conv3d_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        if (tmi_conv3d_check(parent_sgt->ctx, &d) != TMI_VALID)
+            return error("%s", tmi_last_error(parent_sgt->ctx));
+        return 0;
+    }
+    int eval() override
+    {
+        tmi_conv3d_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        int32_t in_zp = 0, w_zp = 0;
+        if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
+            return error("zero-point operands must be available on the host");
+        SubgraphTraverser* s = parent_sgt;
+        if (call(tmi_conv3d(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]), in_zp, w_zp,
+                            s->device_out(outputs[0]))))
+            return 1;
+        return GraphNode::eval();
+    }
+};
+
 // MATMUL: operands [a, b, a_zp, b_zp]
 class OpMatMul : public GraphNode
 {
@@ -530,6 +665,12 @@ int SubgraphTraverser::initializeGraph()
             case Op_DEPTHWISE_CONV2D:
                 n = new OpDepthwiseConv2d(this, id);
                 break;
+            case Op_TRANSPOSE_CONV2D:
+                n = new OpTransposeConv2d(this, id);
+                break;
+            case Op_CONV3D:
+                n = new OpConv3d(this, id);
+                break;
             case Op_MATMUL:
                 n = new OpMatMul(this, id);
                 break;
@@ -541,7 +682,7 @@ int SubgraphTraverser::initializeGraph()
                 break;
             default:
                 last_message = "operator " + std::to_string(o.op) + " is outside the accelerated path "
-                               "(CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP)";
+                               "(CONV2D, CONV3D, DEPTHWISE_CONV2D, TRANSPOSE_CONV2D, MATMUL, RESCALE, CLAMP)";
                 setGraphStatus(GraphStatus::TOSA_ERROR);
                 return 1;
         }

@@ -35,8 +35,10 @@ enum class GraphStatus : int
 enum Op : uint32_t
 {
     Op_CONV2D           = 3,
+    Op_CONV3D           = 4,
     Op_DEPTHWISE_CONV2D = 5,
     Op_MATMUL           = 7,
+    Op_TRANSPOSE_CONV2D = 10,
     Op_CLAMP            = 11,
     Op_RESCALE          = 66,
     Op_CONST            = 67,
@@ -63,7 +65,7 @@ const char* op_name(uint32_t op);
 // ---- serialized graph ------------------------------------------------------------------------------------
 struct Attribute
 {
-    // Conv2dAttribute / DepthwiseConv2dAttribute
+    // Conv2dAttribute / DepthwiseConv2dAttribute / Conv3dAttribute; TransposeConv2dAttribute keeps out_pad in pad
     std::vector<int32_t> pad, stride, dilation;
     bool local_bound  = false;
     uint32_t acc_type = 0;

@@ -517,12 +517,9 @@ static size_t align256(size_t v)
     return (v + 255) & ~(size_t)255;
 }
 
-int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
-                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+// OpTransposeConv2d::checkTensorAttributes and the head of eval() (tensor_ops.cpp:1982-2056, :2083-2091, :2123-2129)
+static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* d, int32_t in_zp, int32_t w_zp)
 {
-    if (!ctx)
-        return TMI_ERROR;
-    const char* op = "OpTransposeConv2d";
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
     if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
@@ -547,6 +544,25 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
         return fail(ctx, "%s: bias channels mismatch %d != %d", op, d->bias_len, d->OC);
     if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
         return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    return TMI_VALID;
+}
+
+int tmi_transpose_conv2d_check(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return validate_tconv(ctx, "OpTransposeConv2d", d, 0, 0);
+}
+
+int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    const char* op = "OpTransposeConv2d";
+    int rc = validate_tconv(ctx, op, d, in_zp, w_zp);
+    if (rc != TMI_VALID)
+        return rc;
     const int64_t total = (int64_t)d->N * d->OH * d->OW * d->OC;
     if (total == 0)
     {
@@ -566,7 +582,7 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
     const int32_t UH     = (d->IH - 1) * d->stride[0] + 1, UW = (d->IW - 1) * d->stride[1] + 1;
     const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * row_bytes);
     const size_t u_bytes = holes ? align256((size_t)d->N * UH * UW * row_bytes) : 0;
-    int rc               = ensure_workspace(ctx, w_bytes + u_bytes);
+    rc                   = ensure_workspace(ctx, w_bytes + u_bytes);
     if (rc != TMI_VALID)
         return rc;
     uint8_t* w_flip = (uint8_t*)ctx->workspace;
@@ -588,12 +604,9 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
                     d->out_dtype, out_dev);
 }
 
-int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
-               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+// OpConv3d::checkTensorAttributes and the head of eval() (tensor_ops.cpp:901-933, :120-226, :963-970, :1024-1033)
+static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t* d, int32_t in_zp, int32_t w_zp)
 {
-    if (!ctx)
-        return TMI_ERROR;
-    const char* op = "OpConv3d";
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
     if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
@@ -627,6 +640,25 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
         return fail(ctx, "%s: bias channel mismatch %d != %d", op, d->bias_len, d->OC);
     if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
         return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    return TMI_VALID;
+}
+
+int tmi_conv3d_check(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return validate_conv3d(ctx, "OpConv3d", d, 0, 0);
+}
+
+int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
+               const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    const char* op = "OpConv3d";
+    int rc = validate_conv3d(ctx, op, d, in_zp, w_zp);
+    if (rc != TMI_VALID)
+        return rc;
     const int64_t total = (int64_t)d->N * d->OD * d->OH * d->OW * d->OC;
     if (total == 0)
     {
@@ -643,7 +675,7 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     const int row_bytes  = d->IC * eb;
     const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * row_bytes);
     const size_t g_bytes = align256((size_t)d->N * d->OD * d->IH * d->IW * d->KD * row_bytes);
-    int rc               = ensure_workspace(ctx, w_bytes + g_bytes);
+    rc                   = ensure_workspace(ctx, w_bytes + g_bytes);
     if (rc != TMI_VALID)
         return rc;
     uint8_t* w_perm = (uint8_t*)ctx->workspace;

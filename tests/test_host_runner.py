@@ -146,6 +146,53 @@ def test_matmul_graph(tmp_path):
 
 
 @pytest.mark.gpu
+def test_transpose_conv2d_and_conv3d_graphs(tmp_path):
+    """TRANSPOSE_CONV2D feeding a RESCALE, and a CONV3D, loaded from flatbuffers and run on the device."""
+    rng = np.random.default_rng(9)
+    x = rng.integers(-128, 128, (1, 6, 7, 16)).astype(np.int8)
+    w = rng.integers(-128, 128, (8, 3, 3, 16)).astype(np.int8)
+    bias = rng.integers(-999, 999, 8).astype(np.int32)
+    out_pad, stride = (0, 1, -1, 0), (2, 2)
+    acc = oracle.transpose_conv2d("i8", x, w, bias, out_pad, stride, in_zp=-4, w_zp=0)
+    mult = rng.integers(1 << 30, 1 << 31, 8).astype(np.int32)
+    shift = np.full(8, 40, np.int8)
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", w.shape, np.int8, w), W.tensor("bias", [8], np.int32, bias),
+          W.tensor("izp", [1], np.int8, [-4]), W.tensor("wzp", [1], np.int8, [0]), W.tensor("acc", acc.shape, np.int32),
+          W.tensor("mult", [8], np.int32, mult), W.tensor("shift", [8], np.int8, shift),
+          W.tensor("rizp", [1], np.int32, [0]), W.tensor("rozp", [1], np.int8, [3]), W.tensor("q", acc.shape, np.int8)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "izp", "wzp", "mult", "shift", "rizp", "rozp")]
+    ops.append(W.operator(10, ["x", "w", "bias", "izp", "wzp"], ["acc"], W.transpose_conv_attr(out_pad, stride)))
+    ops.append(W.operator(R.OP_RESCALE, ["acc", "mult", "shift", "rizp", "rozp"], ["q"], W.rescale_attr()))
+    d1 = tmp_path / "tconv"
+    d1.mkdir()
+    r = _run(_write_case(d1, W.graph(ts, ops, ["x"], ["q"]), {"x": x}, ["q"]))
+    assert r.returncode == 0, r.stderr
+    want, st = oracle.rescale(acc, mult, shift, out_zp=3, out_dtype=np.int8)
+    assert st == oracle.VALID and np.array_equal(np.load(d1 / "q_out.npy"), want)
+
+    x3 = rng.integers(-128, 128, (1, 4, 5, 5, 8)).astype(np.int8)
+    w3 = rng.integers(-128, 128, (4, 2, 3, 3, 8)).astype(np.int8)
+    b3 = np.array([17], np.int32)
+    pad, st3, dil = (1, 0, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)
+    want3 = oracle.conv3d("i8", x3, w3, b3, pad, st3, dil, in_zp=2, w_zp=-1)
+    ts = [W.tensor("x", x3.shape, np.int8), W.tensor("w", w3.shape, np.int8, w3), W.tensor("bias", [1], np.int32, b3),
+          W.tensor("izp", [1], np.int8, [2]), W.tensor("wzp", [1], np.int8, [-1]), W.tensor("o", want3.shape, np.int32)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "izp", "wzp")]
+    ops.append(W.operator(4, ["x", "w", "bias", "izp", "wzp"], ["o"], W.conv_attr(pad, st3, dil)))
+    d2 = tmp_path / "conv3d"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["o"]), {"x": x3}, ["o"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d2 / "o_out.npy"), want3)
+    # a malformed node is rejected when the graph is validated: exit code 2
+    ops[-1] = W.operator(4, ["x", "w", "bias", "izp", "wzp"], ["o"], W.conv_attr((1, 0, 1, 1, 1, 1), (2, 1, 1), dil))
+    d3 = tmp_path / "bad"
+    d3.mkdir()
+    r = _run(_write_case(d3, W.graph(ts, ops, ["x"], ["o"]), {"x": x3}, ["o"]))
+    assert r.returncode == 2 and "exact integer output dimensions" in r.stderr
+
+
+@pytest.mark.gpu
 def test_exit_codes_unpredictable_and_error(tmp_path):
     c = cases.c1()
     # shift 12 admits |acc| < 2^11 only: apply_scale_32's value REQUIRE fires -> exit code 1, output still written

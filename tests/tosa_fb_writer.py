@@ -131,6 +131,11 @@ def conv_attr(pad, stride, dilation, acc_type=5, local_bound=False):
                   (3, "B", int(local_bound)), (4, "I", acc_type)])
 
 
+def transpose_conv_attr(out_pad, stride, acc_type=5, local_bound=False):
+    return table([(0, None, vector("i", out_pad)), (1, None, vector("i", stride)), (2, "B", int(local_bound)),
+                  (3, "I", acc_type)])
+
+
 def rescale_attr(scale32=True, rounding_mode=3, per_channel=True, input_unsigned=False, output_unsigned=False):
     return table([(0, "B", int(scale32)), (1, "I", rounding_mode), (2, "B", int(per_channel)),
                   (3, "B", int(input_unsigned)), (4, "B", int(output_unsigned))])
