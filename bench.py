@@ -44,7 +44,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "copy"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -86,9 +86,33 @@ def main() -> int:
         ctx.close()
         return 0
     W = {}  # workload description filled below
-    if cfg in ("c3", "c4"):
-        c = cases.c3() if cfg == "c3" else cases.c4()
-        depthwise = cfg == "c4"
+    if cfg == "rescale":
+        # stand-alone RESCALE at a size where launch latency no longer matters: the int32 accumulators of eight
+        # batches of the ResNet-style layer, per-channel, double round, to int8
+        import oracle
+        c = cases.c3()
+        rng = np.random.default_rng(cases.SEED ^ 66)
+        acc = rng.integers(-(1 << 23), 1 << 23, (64, 56, 56, 64)).astype(np.int32)
+        tacc, tm, ts = to_dev(acc), to_dev(c["mult"]), to_dev(c["shift"])
+        out = torch.empty(acc.shape, dtype=torch.int8, device=dev)
+        r = ctx.rescale_desc(capi.INT32, capi.INT8, 64, 64, 0, -3, True, capi.ROUND_DOUBLE, True)
+        rows = acc.size // 64
+
+        def step():
+            ctx.rescale(r, 4, rows, 64, tacc, tm, ts, out)
+
+        def cpu_ref():
+            return oracle.rescale(acc[:8], c["mult"], c["shift"], out_zp=-3)[0]
+
+        W = dict(ops=acc.size, bytes=acc.nbytes + acc.size + 64 * 5, exact=True, cpu_ref=cpu_ref, cpu_fraction=1 / 8,
+                 result=lambda: out[:8].cpu().numpy(), dtype="int64",
+                 metric="stand-alone RESCALE int32->int8 GB/s; % HBM peak; bit-exact", unit="GB/s", bound="hbm",
+                 peak=PEAK["hbm"], runit="GB/s",
+                 workload="RESCALE int32 [64,56,56,64] -> int8, per-channel multiplier/shift 38, double_round, "
+                          "output_zp -3 (5 bytes per element)")
+    elif cfg in ("c3", "c4", "c4x8"):
+        c = cases.c3() if cfg == "c3" else (cases.c4() if cfg == "c4" else cases.c4(n=64))
+        depthwise = cfg != "c3"
         n, ih, iw, ic = c["x"].shape
         if depthwise:
             kh, kw, _, m = c["w"].shape
@@ -126,6 +150,8 @@ def main() -> int:
                      unit="GB/s", bound="hbm", peak=PEAK["hbm"], runit="GB/s",
                      workload="configs[3]: INT8 DEPTHWISE_CONV2D [8,112,112,96] 3x3 s2 pad [0,1,0,1] + per-channel "
                               "RESCALE (shift 34..40, double_round), fused")
+            if cfg == "c4x8":    # the same layer at eight times the batch: the kernel's rate without the launch floor
+                W["workload"] = W["workload"].replace("[8,112,112,96]", "[64,112,112,96]") + " (8x the named batch)"
     elif cfg in ("c2", "c5b"):
         c = cases.c2() if cfg == "c2" else cases.c5_matmul()
         n, h, k = c["a"].shape
@@ -212,7 +238,7 @@ def main() -> int:
               "config": {"workload": W["workload"], "kernel": kernel, "ops_per_step": W["ops"],
                          "algorithmic_bytes_per_step": W["bytes"], "graph_status": status},
               "roofline": {"bound": W["bound"], "achieved": round(achieved, 3), "peak": W["peak"], "unit": W["runit"],
-                           "frac": round(achieved / W["peak"], 5), "traffic": MEASURED_TRAFFIC_BYTES[cfg],
+                           "frac": round(achieved / W["peak"], 5), "traffic": MEASURED_TRAFFIC_BYTES.get(cfg),
                            "us_per_launch": round(ev_s_per_launch * 1e6, 3)}}
     if W["bound"] == "hbm" and W["unit"] != "GB/s":
         result["roofline"]["mfma_frac"] = round(W["ops"] / 1e12 / ev_s_per_launch / PEAK["int8_mfma"], 5)

@@ -57,6 +57,104 @@ __global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, co
     raise_flags(flag_word, flags);
 }
 
+// The common RESCALE -- signed INT32 in (no input zero point), 32-bit multipliers, SINGLE or DOUBLE rounding,
+// C a multiple of 4 -- with the per-channel constants in registers: a lane owns 4 consecutive channels and
+// walks down the rows, so multiplier, shift and the 64-bit rounding terms (output zero point folded in) are
+// derived once and an element costs ~9 instructions.  Four rows are in flight per lane.
+typedef int rs_v4i __attribute__((ext_vector_type(4)));
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, const int32_t* __restrict__ in,
+                                                           OutT* __restrict__ out, int64_t rows, int32_t C,
+                                                           int32_t cgs, int32_t rpi, FastDiv div_cgs,
+                                                           uint32_t* flag_word)
+{
+    const int tid  = threadIdx.x;
+    const int slot = fdiv(tid, div_cgs);    // row slot of this lane inside an iteration
+    const bool lane_on = slot < rpi;
+    const int c0   = lane_on ? (tid - slot * cgs) * 4 : 0;
+    uint32_t flags = 0;
+    int32_t mul[4], sh[4];
+    uint32_t lim[4];
+    int64_t rnd_pos[4], rnd_neg[4];
+    bool check = false;
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+    {
+        const int i = p.per_channel ? c0 + c : 0;
+        const ChannelScale cs =
+            make_channel_scale(reinterpret_cast<const int32_t*>(p.multiplier)[i], (int32_t)p.shift[i], p.double_round, flags);
+        const int64_t zp_term = (int64_t)p.out_zp << cs.s;
+        mul[c] = cs.m, sh[c] = cs.s, lim[c] = cs.lim;
+        rnd_pos[c] = cs.rnd_pos + zp_term, rnd_neg[c] = cs.rnd_neg + zp_term;
+        check |= cs.lim != 0x80000000u;
+    }
+    if (!lane_on)
+        flags = 0;
+    constexpr int U = 4;
+    const int64_t step = (int64_t)gridDim.x * rpi;    // rows between two visits of a lane
+    for (int64_t r0 = (int64_t)blockIdx.x * rpi + slot; r0 < rows; r0 += U * step)
+    {
+        rs_v4i v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int64_t r = r0 + u * step;
+            const bool on   = lane_on && r < rows;
+            v[u]            = *reinterpret_cast<const rs_v4i*>(in + (on ? r * C + c0 : 0));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int64_t r = r0 + u * step;
+            const bool on   = lane_on && r < rows;
+            int32_t res[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+            {
+                const int32_t x = v[u][c];
+                if (check && on && (uint32_t)x + lim[c] > 2u * lim[c] - 1u)
+                    flags |= TMI_FLAG_SCALE_VALUE;
+                const int64_t pr = (int64_t)x * (int64_t)mul[c] + (x >= 0 ? rnd_pos[c] : rnd_neg[c]);
+                int32_t o        = (int32_t)(pr >> sh[c]);
+                o                = o < p.lo ? p.lo : o;
+                res[c]           = o > p.hi ? p.hi : o;
+            }
+            if (!on)
+                continue;
+            OutT* q = out + r * C + c0;
+            if constexpr (sizeof(OutT) == 1)
+                *reinterpret_cast<int*>(q) =
+                    (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) | ((res[3] & 0xff) << 24);
+            else if constexpr (sizeof(OutT) == 2)
+            {
+                reinterpret_cast<int*>(q)[0] = (res[0] & 0xffff) | ((res[1] & 0xffff) << 16);
+                reinterpret_cast<int*>(q)[1] = (res[2] & 0xffff) | ((res[3] & 0xffff) << 16);
+            }
+            else
+                *reinterpret_cast<rs_v4i*>(q) = rs_v4i{ res[0], res[1], res[2], res[3] };
+        }
+    }
+    raise_flags(flag_word, flags);
+}
+
+template <typename OutT>
+static const char* launch_rescale_fast(hipStream_t st, const RescaleParams& p, const void* in, void* out, int64_t n,
+                                       int32_t C, uint32_t* flag_word)
+{
+    const int32_t cgs  = C / 4;
+    const int32_t rpi  = 256 / cgs;
+    const int64_t rows = n / C;
+    int64_t blocks     = (rows + (int64_t)rpi * 4 - 1) / ((int64_t)rpi * 4);    // four rows per lane and visit
+    if (blocks > 256 * 8)
+        blocks = 256 * 8;
+    if (blocks < 1)
+        blocks = 1;
+    hipLaunchKernelGGL((rescale_fast_kernel<OutT>), dim3((int)blocks), dim3(256), 0, st, p, (const int32_t*)in,
+                       (OutT*)out, rows, C, cgs, rpi, make_fastdiv(cgs), flag_word);
+    return "rescale_fast";
+}
+
 static int grid_for(int64_t work_items)
 {
     // 256 CUs x 8 blocks of 256 lanes keep every SIMD busy; beyond that the loop strides.
@@ -93,6 +191,16 @@ static const char* launch_rescale_t(hipStream_t st, const RescaleParams& p, cons
 const char* launch_rescale(hipStream_t st, const RescaleParams& p, int32_t in_dtype, int32_t out_dtype,
                            const void* in, void* out, int64_t n, int32_t C, uint32_t* flag_word)
 {
+    if (p.fast && !p.has_clamp && in_dtype == TMI_INT32 && n > 0 && C >= 4 && (C & 3) == 0 && C <= 1024 &&
+        (((uintptr_t)in | (uintptr_t)out) & 15) == 0 && (!p.per_channel || ((uintptr_t)p.multiplier & 3) == 0))
+    {
+        if (out_dtype == TMI_INT8)
+            return launch_rescale_fast<int8_t>(st, p, in, out, n, C, flag_word);
+        if (out_dtype == TMI_INT16)
+            return launch_rescale_fast<int16_t>(st, p, in, out, n, C, flag_word);
+        if (out_dtype == TMI_INT32)
+            return launch_rescale_fast<int32_t>(st, p, in, out, n, C, flag_word);
+    }
 #define TMI_RESCALE_CASE(ID, IT, OD, OT)                                                                            \
     if (in_dtype == ID && out_dtype == OD)                                                                          \
         return launch_rescale_t<IT, OT>(st, p, in, out, n, C, flag_word);
