@@ -122,6 +122,14 @@ struct Mma<bf16_t>
     }
 };
 
+// min(max(v, lo), hi) as one instruction; lo <= hi
+__device__ __forceinline__ int32_t clamp_med3(int32_t v, int32_t lo, int32_t hi)
+{
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+    return r;
+}
+
 __device__ __forceinline__ int dot4_ones(v4i v)
 {
     int s = __builtin_amdgcn_sdot4(v.x, 0x01010101, 0, false);
@@ -228,6 +236,11 @@ static constexpr uint32_t kFill = 0xfffffffeu;
 template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC, bool MULTI>
 __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 {
+    // The kernel arguments span several cache lines; the compiler fetches fields where they are first used,
+    // which serialises one scalar-cache miss per line along the start-up path.  Asking for one field of every
+    // line up front turns that into a single round trip.
+    asm volatile("" ::"s"(a.g.N), "s"(a.g.bias_len), "s"(a.out), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.TH), "s"(a.CH),
+                 "s"(a.n_tiles), "s"(a.rounds), "s"(a.w_batch_stride), "s"(a.div_tw.magic), "s"(a.div_kw.d));
     using M              = Mma<T>;
     using acc_t          = typename M::acc_t;
     using TT             = TileTraits<OCT, PXT, MULTI>;
@@ -354,6 +367,48 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     for (int u = 0; u < PU; u++)
         pacc[u] = 0;
 
+    // Single block, channel vector = block, one round: the (tap, chunk) pairs of a weight row are consecutive
+    // 16-byte chunks in memory and in LDS, so the lane's slots are its first chunk plus compile-time offsets
+    // and need no per-slot arithmetic; only the slot that straddles the end of the row tests its lanes.  Rows
+    // past OC read row 0 of the block (valid memory) and are zeroed when written.
+    const bool w_contig = !MULTI && VEC && a.rounds == 1 && row_bytes == blk_bytes;
+    const int w_full    = n_pairs / LPR;    // slots in which every lane has a chunk
+    const uint8_t* w_lane_src = w_n + (w_oc_ok ? w_src_row : (uint32_t)oc0 * (uint32_t)(taps * row_bytes)) + w_part * 16;
+    const int w_lane_dst      = w_row * a.wstride + w_part * 16;
+    auto issue_weights_contig = [&]() {
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            if (u < w_full)
+                wv[u] = *reinterpret_cast<const v4i*>(w_lane_src + u * LPR * 16);
+            else if (u * LPR < n_pairs)
+                wv[u] = *reinterpret_cast<const v4i*>(w_lane_src + (w_part + u * LPR < n_pairs ? u * LPR * 16 : 0));
+        }
+    };
+    auto commit_weights_contig = [&](uint8_t* wl) {
+        const bool zero_rows = !__all(w_oc_ok);    // wave-uniform
+#pragma unroll
+        for (int u = 0; u < WU; u++)
+        {
+            if (u * LPR >= n_pairs)
+                continue;
+            v4i v = wv[u];
+            if (zero_rows)
+                v = w_oc_ok ? v : v4i{ 0, 0, 0, 0 };
+            uint8_t* dst = wl + w_lane_dst + u * LPR * 16;
+            if (u >= w_full)
+            {
+                const bool ok = w_part + u * LPR < n_pairs;
+                v             = ok ? v : v4i{ 0, 0, 0, 0 };
+                dst           = ok ? dst : dump;
+            }
+            *reinterpret_cast<v4i*>(dst) = v;
+            if constexpr (M::is_int)
+                if (a.za != 0)
+                    wacc += dot4_ones(v);
+        }
+    };
+
     auto describe = [&](int round) {
 #pragma unroll
         for (int u = 0; u < PU; u++)
@@ -369,6 +424,8 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             pdst[u]        = ok ? pix * a.pstride + p_cc16 : -1;
             psrc[u]        = !ok ? kNone : (img ? (uint32_t)(iy * g.IW + ix) * (uint32_t)row_bytes + (uint32_t)p_cc16 : kFill);
         }
+        if (w_contig)
+            return;
 #pragma unroll
         for (int u = 0; u < WU; u++)
         {
@@ -432,6 +489,8 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                     pv[u] = fill_chunk(ic_off + p_cc16, row_bytes, M::is_int ? a.za : 0);
             }
         }
+        if (w_contig)
+            return;    // requested before anything else, see below
 #pragma unroll
         for (int u = 0; u < WU; u++)
         {
@@ -498,6 +557,11 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                     }
                 }
         }
+        if (w_contig)
+        {
+            commit_weights_contig(wl);
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < WU; u++)
         {
@@ -538,6 +602,8 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const bool one_round = a.rounds == 1;
     // a block is whole when it ends inside the channel vector; only the last one in memory order may not be
     auto block_is_whole = [&](int off) { return off + blk_bytes <= row_bytes; };
+    if (w_contig)
+        issue_weights_contig();    // needs no per-slot arithmetic: in flight while the patch slots are worked out
     if (one_round)
     {
         describe(0);
@@ -574,17 +640,20 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     {
         const int oc  = oc0 + tid;
         const bool ok = oc < g.OC && tid < OCB;
+        const int occ = ok ? oc : 0;    // clamped: the loads below are unconditional and issued together
         if constexpr (M::is_int)
         {
+            const int32_t b_raw = reinterpret_cast<const int32_t*>(a.bias)[g.bias_len == 1 ? 0 : occ];
             ChanEntry e;
-            e.bias = ok ? reinterpret_cast<const int32_t*>(a.bias)[g.bias_len == 1 ? 0 : oc] : 0;
             e.m = 0, e.s = 32, e.lim = 0x80000000u, e.rnd_pos = e.rnd_neg = 0;
             if constexpr (EPI == EPI_FAST)
             {
-                // channels past OC get neutral constants (0, 32): every value legal, nothing raised
-                const int32_t m       = ok ? load_multiplier(a.rp, oc) : 0;
-                const int32_t sh      = ok ? load_shift(a.rp, oc) : 32;
-                const ChannelScale cs = make_channel_scale(m, sh, a.rp.double_round, flags);
+                // the fast path has 32-bit multipliers; channels past OC get neutral constants (0, 32): every
+                // value legal, nothing raised
+                const int sc          = a.rp.per_channel ? occ : 0;
+                const int32_t m_raw   = reinterpret_cast<const int32_t*>(a.rp.multiplier)[sc];
+                const int32_t s_raw   = (int32_t)a.rp.shift[sc];
+                const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : 32, a.rp.double_round, flags);
                 // (p + rnd) >> s + zp == (p + rnd + zp * 2^s) >> s: the output zero point rides in the rounding term
                 const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
                 e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos + zp_term, e.rnd_neg = cs.rnd_neg + zp_term;
@@ -594,11 +663,12 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 if (lane == 0)
                     need_check[wave] = any_check;
             }
+            e.bias = ok ? b_raw : 0;
             if (tid < OCB)
                 ctab[tid] = e;
         }
         else if (tid < OCB)
-            ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : oc) : 0.0f;
+            ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : occ) : 0.0f;
     }
 
     const int n_icb = MULTI ? a.n_icb : 1;
@@ -866,8 +936,9 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             {
                 if (fast_i8)
                 {
-                    auto rows = [&](auto checked_tag) {
+                    auto rows = [&](auto checked_tag, auto pcorr_tag) {
                         constexpr bool CHECKED = decltype(checked_tag)::value;
+                        constexpr bool PCORR   = decltype(pcorr_tag)::value;    // weight_zp != 0
 #pragma unroll
                         for (int q = 0; q < 4; q++)
                         {
@@ -882,25 +953,31 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
 #pragma unroll
                                 for (int r = 0; r < 4; r++)
                                 {
-                                    const int32_t v = acc[i][t][4 * q + r] + pcorr[i] + ce[r].bias;
+                                    int32_t v = acc[i][t][4 * q + r] + ce[r].bias;
+                                    if constexpr (PCORR)
+                                        v += pcorr[i];
                                     if constexpr (CHECKED)
                                         if ((uint32_t)v + ce[r].lim > 2u * ce[r].lim - 1u && pix_ok[i])
                                             flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
                                     const int64_t pr =
                                         (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                                    int32_t o = (int32_t)(pr >> ce[r].s);
-                                    o         = o < a.rp.lo ? a.rp.lo : o;
-                                    res[r]    = o > a.rp.hi ? a.rp.hi : o;
+                                    res[r] = clamp_med3((int32_t)(pr >> ce[r].s), a.rp.lo, a.rp.hi);
                                 }
-                                packed[i][q] = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) |
-                                               ((res[3] & 0xff) << 24);
+                                // the low bytes of four clamped values into one word
+                                const int lo2 = __builtin_amdgcn_perm(res[1], res[0], 0x0c0c0400);
+                                const int hi2 = __builtin_amdgcn_perm(res[3], res[2], 0x04000c0c);
+                                packed[i][q]  = lo2 | hi2;
                             }
                         }
                     };
-                    if (check)
-                        rows(std::true_type{});
+                    if (check && a.zw != 0)
+                        rows(std::true_type{}, std::true_type{});
+                    else if (check)
+                        rows(std::true_type{}, std::false_type{});
+                    else if (a.zw != 0)
+                        rows(std::false_type{}, std::true_type{});
                     else
-                        rows(std::false_type{});
+                        rows(std::false_type{}, std::false_type{});
                 }
             }
 
