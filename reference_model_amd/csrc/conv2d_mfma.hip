@@ -268,16 +268,19 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
     const int n_pairs    = taps * a.CH;  // (tap, chunk) pairs per channel block = chunks per weight row
     const int fill_word  = M::is_int ? (a.za & 0xff) * 0x01010101 : 0;    // out-of-image pixels hold input_zp
 
-    // LDS: [channel table][16 zero bytes][check words][1 KB dump area][pair offset table][patch byte sums]
+    // LDS: [channel table][16 zero bytes][check words][(multiplier, bias) table][1 KB dump area][pair offset table][patch byte sums]
     // [buffer 0][buffer 1 when pipelined], a buffer being the weight rows followed by the input patch
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     ChanEntry* ctab        = reinterpret_cast<ChanEntry*>(lds);
     float* ftab            = reinterpret_cast<float*>(lds);    // floating point: bias as float
     constexpr int kCtab    = OCB * (int)sizeof(ChanEntry);
     uint8_t* zero_chunk    = lds + kCtab;
-    int* need_check        = reinterpret_cast<int*>(lds + kCtab + 16);    // two words, one per table wave
-    uint8_t* dump          = lds + kCtab + 32 + lane * 16;    // where staging work items without a destination write
-    constexpr int kFixed   = kCtab + 32 + 1024;
+    int* need_check        = reinterpret_cast<int*>(lds + kCtab + 16);    // per table wave: [0..1] some shift < 32,
+                                                                          // [2..3] the wave's common shift or -1,
+                                                                          // [4..5] output_zp is added after the shift
+    int2* mbtab            = reinterpret_cast<int2*>(lds + kCtab + 48);    // per channel: multiplier, bias
+    uint8_t* dump          = lds + kCtab + 48 + OCB * 8 + lane * 16;    // where staging work items without a destination write
+    constexpr int kFixed   = kCtab + 48 + OCB * 8 + 1024;
     int* pairoff           = reinterpret_cast<int*>(lds + kFixed);
     const int tab_entries  = n_pairs + 32;    // slack: the pipeline reads up to 4G + 1 < 32 entries past the end
     const int tab_bytes    = (tab_entries * 4 + 15) & ~15;
@@ -653,19 +656,37 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 const int sc          = a.rp.per_channel ? occ : 0;
                 const int32_t m_raw   = reinterpret_cast<const int32_t*>(a.rp.multiplier)[sc];
                 const int32_t s_raw   = (int32_t)a.rp.shift[sc];
-                const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : 32, a.rp.double_round, flags);
-                // (p + rnd) >> s + zp == (p + rnd + zp * 2^s) >> s: the output zero point rides in the rounding term
-                const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
+                // channels past OC take the shift of the wave's first channel, so that they do not break a block
+                // whose channels all share one shift
+                const int32_t s_first = __builtin_amdgcn_readfirstlane(ok ? s_raw : 32);
+                const ChannelScale cs =
+                    make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round, flags);
+                // The output zero point rides in the rounding term where that cannot overflow (see
+                // zp_fold_max_shift); if some channel of the wave has too large a shift for it, none of the wave's
+                // channels folds and the epilogue adds output_zp after the shift.
+                const int s_max       = zp_fold_max_shift(a.rp.out_zp);
+                const int nofold      = __any(cs.s > s_max);
+                const int64_t zp_term = nofold ? 0 : ((int64_t)a.rp.out_zp << cs.s);
                 e.m = cs.m, e.s = cs.s, e.lim = cs.lim, e.rnd_pos = cs.rnd_pos + zp_term, e.rnd_neg = cs.rnd_neg + zp_term;
                 // a shift below 32 somewhere: apply_scale_32's value range can be violated and must be checked.
                 // One ballot per table wave; each wave's first lane writes that wave's word.
                 const int any_check = __any(cs.lim != 0x80000000u);
+                // One shift (of at least 32) for the whole wave: the epilogue then keeps the rounding terms in scalar
+                // registers and reads 8 bytes per channel instead of 32.
+                const int uni = __all(cs.s == s_first) && s_first >= 32 && s_first <= s_max;
                 if (lane == 0)
-                    need_check[wave] = any_check;
+                {
+                    need_check[wave]     = any_check;
+                    need_check[2 + wave] = uni ? s_first : -1;
+                    need_check[4 + wave] = nofold;
+                }
             }
             e.bias = ok ? b_raw : 0;
             if (tid < OCB)
-                ctab[tid] = e;
+            {
+                ctab[tid]  = e;
+                mbtab[tid] = int2{ e.m, e.bias };
+            }
         }
         else if (tid < OCB)
             ftab[tid] = ok ? load_as_float<T>(a.bias, g.bias_len == 1 ? 0 : occ) : 0.0f;
@@ -795,7 +816,10 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             for (int m = 1; m < LPR; m <<= 1)
                 sum += __shfl_xor(sum, m);
             if (w_part == 0)
+            {
                 atomicAdd(&ctab[w_ocl].bias, -a.za * sum);
+                atomicAdd(&mbtab[w_ocl].y, -a.za * sum);
+            }
         }
         if (a.zw != 0 && one_round)
         {
@@ -915,8 +939,19 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
             __syncthreads();    // every wave is done reading the operands: LDS becomes the staging area
         int32_t* stage = reinterpret_cast<int32_t*>(lds + kCtab);    // [pixel of the tile][channel of the block]
         bool check     = false;
+        int s_uni      = -1;    // the block's common shift (>= 32), or -1
         if constexpr (EPI == EPI_FAST)
-            check = (need_check[0] | need_check[1]) != 0;
+        {
+            check        = (need_check[0] | need_check[1]) != 0;
+            const int s0 = need_check[2], s1 = need_check[3];
+            s_uni        = __builtin_amdgcn_readfirstlane((s0 >= 0 && (OCB <= 64 || s1 == s0)) ? s0 : -1);
+        }
+        // output_zp where the table wave of this wave's channels did not fold it into the rounding terms
+        auto zp_after_shift = [&](int oclt) {
+            if constexpr (EPI != EPI_FAST)
+                return 0;
+            return __builtin_amdgcn_readfirstlane(need_check[4 + (oclt >= 64 ? 1 : 0)] ? a.rp.out_zp : 0);
+        };
 
 #pragma unroll
         for (int t = 0; t < OCT; t++)
@@ -937,6 +972,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                 if (fast_i8)
                 {
                     auto rows = [&](auto checked_tag, auto pcorr_tag) {
+                        const int zp_post      = zp_after_shift(oclt);
                         constexpr bool CHECKED = decltype(checked_tag)::value;
                         constexpr bool PCORR   = decltype(pcorr_tag)::value;    // weight_zp != 0
 #pragma unroll
@@ -961,7 +997,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                                             flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
                                     const int64_t pr =
                                         (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                                    res[r] = clamp_med3((int32_t)(pr >> ce[r].s), a.rp.lo, a.rp.hi);
+                                    res[r] = clamp_med3((int32_t)(pr >> ce[r].s) + zp_post, a.rp.lo, a.rp.hi);
                                 }
                                 // the low bytes of four clamped values into one word
                                 const int lo2 = __builtin_amdgcn_perm(res[1], res[0], 0x0c0c0400);
@@ -970,7 +1006,45 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                             }
                         }
                     };
-                    if (check && a.zw != 0)
+                    // every channel of the block has the same shift s >= 32: the rounding terms are scalars, the
+                    // result is the high word of the product shifted by s - 32, and no value-range test applies
+                    auto rows_uni = [&](auto pcorr_tag) {
+                        constexpr bool PCORR = decltype(pcorr_tag)::value;
+                        const int64_t dr     = a.rp.double_round ? (int64_t(1) << 30) : 0;
+                        const int64_t rp     = (int64_t(1) << (s_uni - 1)) + dr + ((int64_t)a.rp.out_zp << s_uni);
+                        const int64_t rn     = rp - 2 * dr;
+                        const int sh         = s_uni - 32;
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                        {
+                            int2 mb[4];
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                mb[r] = mbtab[oclt + 4 * q + r];
+#pragma unroll
+                            for (int i = 0; i < PXT; i++)
+                            {
+                                int32_t res[4];
+#pragma unroll
+                                for (int r = 0; r < 4; r++)
+                                {
+                                    int32_t v = acc[i][t][4 * q + r] + mb[r].y;
+                                    if constexpr (PCORR)
+                                        v += pcorr[i];
+                                    const int64_t pr = (int64_t)v * (int64_t)mb[r].x + (v >= 0 ? rp : rn);
+                                    res[r]           = clamp_med3((int32_t)(pr >> 32) >> sh, a.rp.lo, a.rp.hi);
+                                }
+                                const int lo2 = __builtin_amdgcn_perm(res[1], res[0], 0x0c0c0400);
+                                const int hi2 = __builtin_amdgcn_perm(res[3], res[2], 0x04000c0c);
+                                packed[i][q]  = lo2 | hi2;
+                            }
+                        }
+                    };
+                    if (s_uni >= 0 && a.zw != 0)
+                        rows_uni(std::true_type{});
+                    else if (s_uni >= 0)
+                        rows_uni(std::false_type{});
+                    else if (check && a.zw != 0)
                         rows(std::true_type{}, std::true_type{});
                     else if (check)
                         rows(std::true_type{}, std::false_type{});
@@ -1005,7 +1079,7 @@ __global__ __launch_bounds__(512) void conv2d_patch_kernel(PatchArgs a)
                                     flags |= TMI_FLAG_SCALE_VALUE;    // pixels outside the image raise nothing
                                 const int64_t pr =
                                     (int64_t)v * (int64_t)ce[r].m + (v >= 0 ? ce[r].rnd_pos : ce[r].rnd_neg);
-                                v = (int32_t)(pr >> ce[r].s);    // output_zp rides in the rounding term
+                                v = (int32_t)(pr >> ce[r].s) + zp_after_shift(oclt);    // output_zp: in the rounding term, or here
                                 v = v < a.rp.lo ? a.rp.lo : v;
                                 v = v > a.rp.hi ? a.rp.hi : v;
                             }
@@ -1211,8 +1285,9 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
         a.wstride  = (rch + (rch & 1)) * 16 + 16;    // room for a spare zero chunk; = 16 (mod 32)
         a.ksteps   = (rch + 1) / 2;
     };
-    auto fixed_bytes = [&]() {    // channel table, zero chunk, check words, dump area, pair table, patch byte sums
-        return (size_t)OCB * 32 + 32 + 1024 + ((((size_t)taps * a.CH + 32) * 4 + 15) & ~(size_t)15) +
+    auto fixed_bytes = [&]() {    // channel table, zero chunk, check words, (multiplier, bias) table, dump area, pair
+                                  // table, patch byte sums
+        return (size_t)OCB * 32 + 48 + (size_t)OCB * 8 + 1024 + ((((size_t)taps * a.CH + 32) * 4 + 15) & ~(size_t)15) +
                (Mma<T>::is_int ? (((size_t)a.PH * a.PW * 4 + 15) & ~(size_t)15) : 0);
     };
     auto buf_bytes   = [&]() { return (size_t)OCB * a.wstride + (size_t)a.PH * a.PW * a.pstride; };

@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void depthwise_dot4_kernel(DwArgs a)
     }
     uint32_t flags = 0;
     int32_t corr[4];    // bias - za*sum(w) + T*za*zw
-    int32_t mul[4], sh[4];
+    int32_t mul[4], sh[4], zp_post[4] = { 0, 0, 0, 0 };
     uint32_t lim[4];
     int64_t rnd_pos[4], rnd_neg[4];
     bool check = false;    // some channel of this lane has a shift below 32: the value range must be tested
@@ -216,8 +216,10 @@ __global__ __launch_bounds__(256) void depthwise_dot4_kernel(DwArgs a)
         if constexpr (RESCALE)
         {
             const ChannelScale cs = make_channel_scale(mraw[c], sraw[c], a.rp.double_round, flags);
-            // (p + rnd) >> s + zp == (p + rnd + zp * 2^s) >> s: the output zero point rides in the rounding term
-            const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
+            // the output zero point rides in the rounding term where that cannot overflow, else it is added last
+            const bool fold       = cs.s <= zp_fold_max_shift(a.rp.out_zp);
+            const int64_t zp_term = fold ? ((int64_t)a.rp.out_zp << cs.s) : 0;
+            zp_post[c]            = fold ? 0 : a.rp.out_zp;
             mul[c] = cs.m, sh[c] = cs.s, lim[c] = cs.lim;
             rnd_pos[c] = cs.rnd_pos + zp_term, rnd_neg[c] = cs.rnd_neg + zp_term;
             check |= cs.lim != 0x80000000u;
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(256) void depthwise_dot4_kernel(DwArgs a)
                 if (check && on && (uint32_t)v + lim[c] > 2u * lim[c] - 1u)
                     flags |= TMI_FLAG_SCALE_VALUE;
                 const int64_t pr = (int64_t)v * (int64_t)mul[c] + (v >= 0 ? rnd_pos[c] : rnd_neg[c]);
-                v                = (int32_t)(pr >> sh[c]);
+                v                = (int32_t)(pr >> sh[c]) + zp_post[c];
                 v                = v < a.rp.lo ? a.rp.lo : v;
                 v                = v > a.rp.hi ? a.rp.hi : v;
             }

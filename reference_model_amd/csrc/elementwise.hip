@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, cons
     const bool lane_on = slot < rpi;
     const int c0   = lane_on ? (tid - slot * cgs) * 4 : 0;
     uint32_t flags = 0;
-    int32_t mul[4], sh[4];
+    int32_t mul[4], sh[4], zp_post[4];
     uint32_t lim[4];
     int64_t rnd_pos[4], rnd_neg[4];
     bool check = false;
@@ -84,7 +84,9 @@ __global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, cons
         const int i = p.per_channel ? c0 + c : 0;
         const ChannelScale cs =
             make_channel_scale(reinterpret_cast<const int32_t*>(p.multiplier)[i], (int32_t)p.shift[i], p.double_round, flags);
-        const int64_t zp_term = (int64_t)p.out_zp << cs.s;
+        const bool fold       = cs.s <= zp_fold_max_shift(p.out_zp);    // else output_zp is added after the shift
+        const int64_t zp_term = fold ? ((int64_t)p.out_zp << cs.s) : 0;
+        zp_post[c]            = fold ? 0 : p.out_zp;
         mul[c] = cs.m, sh[c] = cs.s, lim[c] = cs.lim;
         rnd_pos[c] = cs.rnd_pos + zp_term, rnd_neg[c] = cs.rnd_neg + zp_term;
         check |= cs.lim != 0x80000000u;
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, cons
                 if (check && on && (uint32_t)x + lim[c] > 2u * lim[c] - 1u)
                     flags |= TMI_FLAG_SCALE_VALUE;
                 const int64_t pr = (int64_t)x * (int64_t)mul[c] + (x >= 0 ? rnd_pos[c] : rnd_neg[c]);
-                int32_t o        = (int32_t)(pr >> sh[c]);
+                int32_t o        = (int32_t)(pr >> sh[c]) + zp_post[c];
                 o                = o < p.lo ? p.lo : o;
                 res[c]           = o > p.hi ? p.hi : o;
             }

@@ -161,6 +161,15 @@ __device__ __forceinline__ ChannelScale make_channel_scale(int32_t m, int32_t s,
     return c;
 }
 
+// (p + rnd) >> s + zp == (p + rnd + zp * 2^s) >> s lets the output zero point ride in the 64-bit rounding term,
+// but only while the sum stays inside int64: |value * multiplier| < 2^62 and rnd <= 2^61 + 2^30 leave room for
+// |zp| * 2^s <= 2^60.  Returns the largest shift for which the fold is safe.
+__device__ __forceinline__ int zp_fold_max_shift(int32_t out_zp)
+{
+    const uint32_t mag = (uint32_t)(out_zp < 0 ? -(int64_t)out_zp : (int64_t)out_zp);
+    return mag == 0 ? 62 : 60 - (32 - __clz((int)mag));
+}
+
 // apply_scale_32 + output_zp + clip (+ CLAMP) for a signed int32 value with zero input_zp.  With a legal
 // value |v| < 2^(s-1) and m < 2^31 the scaled result is below 2^30 in magnitude, so neither of the
 // reference's int32 range checks (quant_util.h:78-82, type_conversion.cpp:352-360) can fire here.

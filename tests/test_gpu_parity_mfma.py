@@ -106,6 +106,45 @@ def test_fused_rescale_output_types_and_ragged_channels(ctx, out_dtype):
     assert st == capi.VALID and np.array_equal(got, _fused_expect(c, out_dtype))
 
 
+@pytest.mark.parametrize("shift", [32, 33, 38, 62])
+@pytest.mark.parametrize("zw", [0, 5])
+def test_fused_rescale_one_shift_for_all_channels(ctx, shift, zw):
+    """All channels share one shift of at least 32: the epilogue variant with scalar rounding terms.  Ragged
+    channel counts (37 of 64, 130 of 192) bring channels past OC into the tables."""
+    for oc, out_zp in ((37, -6), (130, 9)):
+        rng = np.random.default_rng(shift * 7 + oc)
+        c = dict(x=rng.integers(-128, 128, (2, 9, 11, 32)).astype(np.int8),
+                 w=rng.integers(-127, 128, (oc, 3, 3, 32)).astype(np.int8),
+                 bias=rng.integers(-5000, 5000, oc).astype(np.int32), in_zp=-11, w_zp=zw, pad=(1, 1, 1, 1),
+                 stride=(1, 1), dilation=(1, 1), mult=rng.integers(1 << 30, 1 << 31, oc).astype(np.int32),
+                 shift=np.full(oc, shift, np.int8), out_zp=out_zp, clamp=(-100, 90))
+        got, st = _fused_run(ctx, c)
+        assert st == capi.VALID and np.array_equal(got, _fused_expect(c)), (oc, shift)
+
+
+def test_large_shifts_with_output_zero_point_do_not_overflow(ctx):
+    """output_zp * 2^shift does not fit 64 bits next to the product for shifts near 62: the kernels that fold the
+    zero point into the rounding term must stop doing so there (stand-alone RESCALE, depthwise, CONV2D with
+    mixed shifts)."""
+    rng = np.random.default_rng(62)
+    x = rng.integers(-(1 << 31), 1 << 31, (50, 8), dtype=np.int64).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, 8).astype(np.int32)
+    shift = np.array([62, 61, 55, 53, 52, 51, 40, 33], np.int8)
+    for out_zp, od, unsigned in ((-128, np.int8, False), (127, np.int8, False)):
+        want, wst = oracle.rescale(x, mult, shift, out_zp=out_zp, out_dtype=od, output_unsigned=unsigned)
+        got, st = gpu_ops.rescale(ctx, x, mult, shift, out_zp=out_zp, out_dtype=od, output_unsigned=unsigned)
+        assert ctx.last_kernel == "rescale_fast" and st == wst == capi.VALID and np.array_equal(got, want)
+    c = cases.c4(n=1, hw=12, c=8)
+    c["shift"], c["out_zp"] = shift, -128
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"],
+                             c["w_zp"], depthwise=True, rescale=dict(mult=c["mult"], shift=shift, out_zp=-128))
+    assert st == capi.VALID and np.array_equal(got, _dw_expect(c))
+    c = cases.c1()
+    c["shift"], c["out_zp"] = np.resize(shift, 16), 127
+    got, st = _fused_run(ctx, c)
+    assert st == capi.VALID and np.array_equal(got, _fused_expect(c))
+
+
 def test_fused_rescale_require_condition_is_reported(ctx):
     c = cases.c1()
     c["shift"] = np.full(16, 12, np.int8)  # |acc| exceeds 2^11: apply_scale_32's value range (quant_util.h:59-67)
