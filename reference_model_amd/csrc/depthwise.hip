@@ -58,6 +58,10 @@ __device__ __forceinline__ void transpose4x4(const int (&d)[4], int (&e)[4])
 template <int NG, bool K33, bool ZW, bool RESCALE>
 __global__ __launch_bounds__(256) void depthwise_dot4_kernel(DwArgs a)
 {
+    // one field of every cache line of the kernel arguments up front: a single scalar-cache round trip instead
+    // of one per line along the start-up path
+    asm volatile("" ::"s"(a.g.N), "s"(a.g.bias_len), "s"(a.out), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.za), "s"(a.blocks),
+                 "s"(a.div_oh.d));
     const ConvGeom& g = a.g;
     const int tid     = threadIdx.x;
     const int slot    = fdiv(tid, a.div_cgs);    // pixel slot of this lane inside an iteration
@@ -350,7 +354,7 @@ const char* launch_depthwise_vec(hipStream_t st, int32_t in_dtype, int32_t out_d
     a.total_px = (int)total_px;
     // enough workgroups to give every CU several, few enough that a lane's constants serve a few pixels
     const int64_t px_iters = (total_px + a.ppi - 1) / a.ppi;
-    a.iters                = px_iters >= 256 * 16 ? 4 : (px_iters >= 256 * 8 ? 2 : 1);
+    a.iters                = px_iters >= 256 * 64 ? 8 : (px_iters >= 256 * 16 ? 4 : (px_iters >= 256 * 8 ? 2 : 1));
     a.blocks               = (int)((px_iters + a.iters - 1) / a.iters);
     a.div_cgs              = make_fastdiv(a.cgs);
     a.div_ow               = make_fastdiv(g.OW);
