@@ -4,8 +4,8 @@
 // One workgroup (8 waves) computes a TH x TW tile of output pixels of one image for a block of OCB =
 // 32*OCT*WOC output channels.  The waves form a WOC x (8/WOC) grid; each owns OCT channel tiles and PXT pixel
 // tiles of 32, i.e. OCT*PXT accumulator tiles.  The small instantiations (one or two accumulator tiles per
-// wave) are for layers too small to fill the chip otherwise, the 2x2 one for GEMM-sized work, where it
-// halves the LDS traffic per MFMA.  Per block of CH*16 bytes of input channels the workgroup stages in LDS
+// wave) are for layers too small to fill the chip otherwise, the 2x2 and 2x4 ones for GEMM-sized work, where
+// fewer operand bytes pass through L1 and LDS per MFMA.  Per block of CH*16 bytes of input channels the workgroup stages in LDS
 //   - the input patch that the tile needs (PH x PW pixels, out-of-image pixels filled with input_zp, so the
 //     zero-point identity below holds with the full K): one row of CH 16-byte chunks per pixel, and
 //   - the weight slab: one row per output channel holding its KH*KW*CH chunks in (tap, chunk) order, which
@@ -221,10 +221,11 @@ struct alignas(16) ChanEntry
 template <int OCT, int PXT, bool MULTI>
 struct TileTraits
 {
-    static constexpr bool big = OCT * PXT >= 4;
-    static constexpr int WU   = 5;
-    static constexpr int PU   = big ? 8 : (MULTI ? 4 : 2);
-    static constexpr int G    = big ? 1 : 3;
+    static constexpr bool big  = OCT * PXT >= 4;
+    static constexpr bool huge = OCT * PXT >= 8;    // 128 accumulator registers: the staging budget shrinks
+    static constexpr int WU    = huge ? 2 : 5;
+    static constexpr int PU    = huge ? 4 : (big ? 8 : (MULTI ? 4 : 2));
+    static constexpr int G     = big ? 1 : 3;
 };
 
 // Source descriptors of the staging: a byte offset below kFill is loaded, kFill is an out-of-image pixel
@@ -1241,9 +1242,9 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     int OCT = 1, PXT = 1;
     if (vec)
     {
-        static const int cand[3][2] = { { 1, 1 }, { 1, 2 }, { 2, 2 } };
+        static const int cand[4][2] = { { 1, 1 }, { 1, 2 }, { 2, 2 }, { 2, 4 } };
         double best = 0;
-        for (int c = 0; c < 3; c++)
+        for (int c = 0; c < 4; c++)
         {
             const int oct = cand[c][0], pxt = cand[c][1];
             if (oct == 2 && g.OC <= 64)
@@ -1264,8 +1265,8 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     const int OCB           = 32 * OCT * WOC;
     const int64_t oc_blocks = (g.OC + OCB - 1) / OCB;
     const int max_px        = 32 * (8 / WOC) * PXT;
-    const int WU = 5;                                   // the values of TileTraits<OCT, PXT, n_icb > 1>
-    auto PU_for  = [&](int n_icb) { return (OCT * PXT >= 4) ? 8 : (n_icb > 1 ? 4 : 2); };
+    const int WU = OCT * PXT >= 8 ? 2 : 5;              // the values of TileTraits<OCT, PXT, n_icb > 1>
+    auto PU_for  = [&](int n_icb) { return OCT * PXT >= 8 ? 4 : ((OCT * PXT >= 4) ? 8 : (n_icb > 1 ? 4 : 2)); };
     const int LPR = 512 / OCB;
     int TH, TW;
     tile_for(max_px, TH, TW);
@@ -1388,7 +1389,8 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
     TMI_PATCH_CASE(1, 1, 2, E)                                                                                       \
     TMI_PATCH_CASE(2, 1, 1, E)                                                                                       \
     TMI_PATCH_CASE(2, 1, 2, E)                                                                                       \
-    TMI_PATCH_CASE(2, 2, 2, E)
+    TMI_PATCH_CASE(2, 2, 2, E)                                                                                       \
+    TMI_PATCH_CASE(2, 2, 4, E)
     if (vec)
     {
         TMI_PATCH_SHAPES(EPI_PLAIN)

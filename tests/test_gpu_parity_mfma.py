@@ -282,6 +282,20 @@ def test_matmul_i8_mfma_bit_exact(ctx, shape, zps):
     assert st == capi.VALID and np.array_equal(got, oracle.matmul("i8", a, b, *zps))
 
 
+@pytest.mark.parametrize("k", [128, 320])
+def test_matmul_i8_largest_tile_bit_exact(ctx, k):
+    """[4,2048,k] x [4,k,2048]: GEMM-sized enough for the 128-channel x 512-pixel workgroup shape (one channel block
+    for k = 128, five pipelined 64-byte blocks for k = 320).  Expected values from a float64 BLAS product (exact)."""
+    rng = np.random.default_rng(k)
+    a = rng.integers(-128, 128, (4, 2048, k)).astype(np.int8)
+    b = rng.integers(-128, 128, (4, k, 2048)).astype(np.int8)
+    got, st = gpu_ops.matmul(ctx, a, b, 7, -9)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_mfma_i8"
+    want = np.matmul(a.astype(np.float64) - 7, b.astype(np.float64) + 9)
+    assert np.array_equal(got, want.astype(np.int64).astype(np.int32))
+    assert np.array_equal(got[3, :40], oracle.matmul("i8", a[3:4, :40], b[3:4], 7, -9)[0])
+
+
 def test_config2_matmul_full_size(ctx):
     """[8,1024,1024] x [8,1024,1024] -> int32, a_zp -5, b_zp 3: every element against a float64 BLAS product
     (exact: |sum| < 2^53), one batch against the scalar oracle, plus the transposition property
