@@ -44,7 +44,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "copy"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,6 +110,55 @@ def main() -> int:
                  peak=PEAK["hbm"], runit="GB/s",
                  workload="RESCALE int32 [64,56,56,64] -> int8, per-channel multiplier/shift 38, double_round, "
                           "output_zp -3 (5 bytes per element)")
+    elif cfg in ("tconv", "conv3d"):
+        # the two neighbouring operators, at shapes of the same family as the named CONV2D configuration (no
+        # configuration of theirs is named): the timed step includes the operand re-layout kernels
+        import gpu_ops  # noqa: F401  (TconvDesc / Conv3dDesc helpers live in capi)
+        import oracle
+        rng = np.random.default_rng(cases.SEED ^ (10 if cfg == "tconv" else 4))
+        if cfg == "tconv":
+            x = rng.integers(-128, 128, (8, 28, 28, 128)).astype(np.int8)
+            w = np.clip(np.rint(rng.normal(0, 30, (64, 3, 3, 128))), -127, 127).astype(np.int8)
+            bias = np.rint(rng.normal(0, 2 ** 14, 64)).astype(np.int32)
+            out_pad, stride = (0, 1, 0, 1), (2, 2)
+            oh = ow = (28 - 1) * 2 + 1 + 3
+            d = capi.TconvDesc()
+            d.in_dtype, d.out_dtype = capi.INT8, capi.INT32
+            d.N, d.IH, d.IW, d.IC, d.OC, d.KH, d.KW, d.OH, d.OW = 8, 28, 28, 128, 64, 3, 3, oh, ow
+            d.out_pad[:], d.stride[:], d.bias_len = list(out_pad), list(stride), 64
+            out = torch.empty((8, oh, ow, 64), dtype=torch.int32, device=dev)
+            macs = 8 * oh * ow * 64 * 9 * 128    # dense count over the zero-inserted input, as for CONV2D
+            fn, name = ctx.transpose_conv2d, "TRANSPOSE_CONV2D [8,28,28,128]x[64,3,3,128] s2 out_pad [0,1,0,1] -> [8,56,56,64] int32"
+
+            def cpu_ref():
+                return oracle.transpose_conv2d("i8", x[:1], w, bias, out_pad, stride, -7, 0)
+            frac = 1 / 8
+        else:
+            x = rng.integers(-128, 128, (2, 16, 28, 28, 32)).astype(np.int8)
+            w = np.clip(np.rint(rng.normal(0, 30, (64, 3, 3, 3, 32))), -127, 127).astype(np.int8)
+            bias = np.rint(rng.normal(0, 2 ** 14, 64)).astype(np.int32)
+            pad, st3, dil = (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)
+            d = capi.Conv3dDesc()
+            d.in_dtype, d.out_dtype = capi.INT8, capi.INT32
+            d.N, d.ID, d.IH, d.IW, d.IC, d.OC, d.KD, d.KH, d.KW = 2, 16, 28, 28, 32, 64, 3, 3, 3
+            d.OD, d.OH, d.OW = 16, 28, 28
+            d.pad[:], d.stride[:], d.dilation[:], d.bias_len = list(pad), list(st3), list(dil), 64
+            out = torch.empty((2, 16, 28, 28, 64), dtype=torch.int32, device=dev)
+            macs = 2 * 16 * 28 * 28 * 64 * 27 * 32
+            fn, name = ctx.conv3d, "CONV3D [2,16,28,28,32]x[64,3,3,3,32] s1 p1 -> [2,16,28,28,64] int32"
+
+            def cpu_ref():
+                return oracle.conv3d("i8", x[:1], w, bias, pad, st3, dil, -7, 0)
+            frac = 1 / 2
+        tx, tw, tb = to_dev(x), to_dev(w), to_dev(bias)
+
+        def step():
+            fn(d, tx, tw, tb, -7, 0, out)
+
+        W = dict(ops=2 * macs, bytes=x.nbytes + w.nbytes + bias.nbytes + out.numel() * 4, exact=True, cpu_ref=cpu_ref,
+                 cpu_fraction=frac, result=lambda: out[:1].cpu().numpy(), dtype="int8",
+                 metric="int8 %s TOPS; %% int8 MFMA peak; bit-exact" % cfg.upper(), unit="TOPS", bound="mfma",
+                 peak=PEAK["int8_mfma"], runit="TOP/s", workload="INT8 " + name)
     elif cfg in ("c3", "c4", "c4x8"):
         c = cases.c3() if cfg == "c3" else (cases.c4() if cfg == "c4" else cases.c4(n=64))
         depthwise = cfg != "c3"
