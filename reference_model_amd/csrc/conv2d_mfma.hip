@@ -46,17 +46,10 @@
 // LDS table; every lane then spends about ten instructions per output element.
 #include <type_traits>
 
-#include "tmi_kernels.h"
+#include "tmi_mfma.h"
 
 namespace tmi
 {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-typedef __bf16 v8b __attribute__((ext_vector_type(8)));
 
 struct PatchArgs
 {
@@ -86,56 +79,12 @@ struct PatchArgs
     FastDiv div_tw, div_pw, div_tiles_x, div_tiles_y, div_group, div_kw;
 };
 
-template <typename T>
-struct Mma;
-
-template <>
-struct Mma<int8_t>
-{
-    using acc_t                  = v16i;
-    static constexpr bool is_int = true;
-    __device__ static v16i mma(v4i a, v4i b, v16i c)
-    {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-    }
-};
-template <>
-struct Mma<_Float16>
-{
-    using acc_t                  = v16f;
-    static constexpr bool is_int = false;
-    __device__ static v16f mma(v4i a, v4i b, v16f c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0,
-                                                      0, 0);
-    }
-};
-template <>
-struct Mma<bf16_t>
-{
-    using acc_t                  = v16f;
-    static constexpr bool is_int = false;
-    __device__ static v16f mma(v4i a, v4i b, v16f c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b, a), __builtin_bit_cast(v8b, b), c, 0,
-                                                       0, 0);
-    }
-};
-
 // min(max(v, lo), hi) as one instruction; lo <= hi
 __device__ __forceinline__ int32_t clamp_med3(int32_t v, int32_t lo, int32_t hi)
 {
     int32_t r;
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
     return r;
-}
-
-__device__ __forceinline__ int dot4_ones(v4i v)
-{
-    int s = __builtin_amdgcn_sdot4(v.x, 0x01010101, 0, false);
-    s     = __builtin_amdgcn_sdot4(v.y, 0x01010101, s, false);
-    s     = __builtin_amdgcn_sdot4(v.z, 0x01010101, s, false);
-    return __builtin_amdgcn_sdot4(v.w, 0x01010101, s, false);
 }
 
 // Byte-wise version of a chunk load for channel vectors whose length is not a multiple of 16 bytes
@@ -172,35 +121,6 @@ __device__ __forceinline__ v4i fill_chunk(int off, int row_bytes, int fill_byte)
     }
     return r;
 }
-
-template <typename T>
-__device__ __forceinline__ float load_as_float(const void* p, int i);
-template <>
-__device__ __forceinline__ float load_as_float<_Float16>(const void* p, int i)
-{
-    return (float)reinterpret_cast<const _Float16*>(p)[i];
-}
-template <>
-__device__ __forceinline__ float load_as_float<bf16_t>(const void* p, int i)
-{
-    return bf16_to_float(reinterpret_cast<const bf16_t*>(p)[i]);
-}
-template <>
-__device__ __forceinline__ float load_as_float<int8_t>(const void*, int)
-{
-    return 0.0f;
-}
-
-__device__ __forceinline__ void store_from_float(_Float16* p, float v)
-{
-    *p = (_Float16)v;
-}
-__device__ __forceinline__ void store_from_float(bf16_t* p, float v)
-{
-    *p = float_to_bf16(v);
-}
-__device__ __forceinline__ void store_from_float(int8_t*, float)
-{}
 
 enum
 {

@@ -1,0 +1,505 @@
+// GEMM-shaped CONV2D (1x1 taps, stride 1, no padding) and MATMUL on the matrix cores, for work large enough
+// that operand delivery, not set-up, decides the time.
+//
+//   out[b][p][oc] = sum_k (a[b][p][k] - za) * (w[b][oc][k] - zw) + bias[oc]
+//
+// (tensor_ops.cpp:843-882 with one tap; tensor_ops.cpp:1463-1500 for MATMUL, whose second operand arrives
+// with K contiguous.)  Both operands are rows of kb = K * sizeof(element) bytes, kb a multiple of 64.
+//
+// A workgroup of 8 waves (2 along the output channels x 4 along the pixels) owns a tile of 64*OCT channels x
+// 128*PXT pixels; a wave owns OCT x PXT accumulator tiles of 32x32.  K is walked in blocks of 64 bytes per
+// row.  The operands of a block go from global memory straight into LDS (global_load_lds_dwordx4: no
+// staging registers, no LDS store instructions), into one of three or four stage buffers, so the loads of the
+// next blocks are in flight while one is multiplied; one barrier per block both publishes a stage and frees
+// the one the next loads will overwrite.
+//
+// LDS layout of a stage: row r (weight rows first, then pixel rows) occupies bytes [64r, 64r + 64); its four
+// 16-byte chunks are stored permuted, chunk c at position c ^ swz(r), so that the 16 lanes the LDS serves in
+// one cycle, which read the same chunk of 16 different rows, hit 16 different bank groups.  A direct load writes
+// LDS at base + 16 * lane, so lane l of a load serves row l / 4 of a 16-row group and position l % 4, and
+// fetches chunk (l % 4) ^ swz(row) from global memory: the permutation costs nothing.
+//
+// Accumulator rows are assigned to channels as in the patch kernel: row 8q + 4h' + j of a channel tile is
+// channel 16h' + 4q + j, which makes every lane own 16 consecutive channels of one pixel.
+//
+// Zero points (int8): sum(a*w) - zw*sum(a) - za*sum(w) + K*za*zw.  The sums are taken with v_dot4 from the
+// fragments as they pass through registers on their way to the matrix core (only in the ZP instantiation).
+#include "tmi_mfma.h"
+
+namespace tmi
+{
+
+struct GemmArgs
+{
+    const uint8_t* a;    // pixel operand, rows of kb bytes
+    const uint8_t* w;    // weight operand, rows of kb bytes
+    const void* bias;
+    void* out;
+    int64_t a_batch, w_batch, o_batch;    // bytes between batches
+    int32_t M, N;                         // pixel rows per batch, weight rows
+    int32_t kb;                           // bytes per row
+    int32_t n_blocks;                     // kb / 64
+    int32_t tiles_n, tiles_per_batch, tiles_total, per_xcd;
+    int32_t bias_len, za, zw, K;
+    int32_t out_is_wide;    // floating point: 1 = fp32 output, 0 = output of the input type
+    FastDiv div_batch, div_tn;
+};
+
+
+// Bank-group permutation of a stage row.  A ds_read_b128 is served 16 lanes a cycle, and the 16 are not
+// consecutive: within each half wave the quads (4 lanes) {0,3,5,6} go together and the quads {1,2,4,7}
+// (measured with two active lanes reading one bank group at different addresses).  Lane rho of a half reads
+// row rho (pixels) or channel_of_row(rho) (weights) of a 32-row tile, so the four rows of a quad already
+// differ in row % 4, i.e. in which 64 of the 256 bank bytes they use; (row / 8) % 4 separates the four quads
+// of either set for both row assignments.
+__device__ __forceinline__ int swz(int r)
+{
+    return (r >> 3) & 3;
+}
+
+// accumulator row -> channel of its tile
+__device__ __forceinline__ int channel_of_row(int rho)
+{
+    return 16 * ((rho >> 2) & 1) + 4 * (rho >> 3) + (rho & 3);
+}
+
+// Stage buffers of a workgroup: four 64-byte blocks per row.  The 256x256 shape fills the LDS with them; two
+// workgroups of a smaller shape with three stages each were measured and are slower (the operand traffic per
+// matrix instruction, not the barrier, is what the smaller shapes wait for).
+static constexpr int kStages = 4;
+
+template <typename T, int OCT, int PXT, bool ZP>
+__global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
+{
+    using M                = Mma<T>;
+    using acc_t            = typename M::acc_t;
+    constexpr int WROWS    = 64 * OCT;
+    constexpr int PROWS    = 128 * PXT;
+    constexpr int ROWS     = WROWS + PROWS;
+    constexpr int STAGE    = ROWS * 64;
+    constexpr int LOADS    = ROWS / 128;    // direct loads per wave and block (16 rows each)
+    static_assert(ROWS % 128 == 0, "a block must split evenly over the 8 waves");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rho  = lane & 31;
+    const int h    = lane >> 5;
+    const int wo   = wave & 1;
+    const int wp   = wave >> 1;
+
+    // Workgroups are dealt round-robin to the 8 XCDs; each XCD takes a contiguous range of the tile list
+    // (tiles with the same pixel rows are neighbours) so that its L2 sees every operand row few times.
+    const int xcd  = blockIdx.x & 7;
+    const int slot = blockIdx.x >> 3;
+    const int L    = xcd * a.per_xcd + slot;
+    if (L >= a.tiles_total)
+        return;
+    const int batch = (int)fdiv((uint32_t)L, a.div_batch);
+    const int rem   = L - batch * a.tiles_per_batch;
+    const int tm    = (int)fdiv((uint32_t)rem, a.div_tn);
+    const int tn    = rem - tm * a.tiles_n;
+    const int p0    = tm * PROWS;
+    const int oc0   = tn * WROWS;
+
+    const uint8_t* a_base = a.a + batch * a.a_batch;
+    const uint8_t* w_base = a.w + batch * a.w_batch;
+
+    // ---- direct loads: per lane one byte offset per load, constant over the blocks ------------------------
+    uint32_t voff[LOADS];
+    const uint8_t* gbase[LOADS];
+    uint32_t ldst[LOADS];
+#pragma unroll
+    for (int j = 0; j < LOADS; j++)
+    {
+        const int grp   = j * 8 + wave;    // 16-row group of the stage
+        const int r     = grp * 16 + (lane >> 2);
+        const bool is_w = grp * 16 < WROWS;
+        int row         = is_w ? oc0 + r : p0 + r - WROWS;
+        const int last  = (is_w ? a.N : a.M) - 1;
+        row             = row < last ? row : last;    // rows past the end repeat the last one; never stored
+        voff[j]         = (uint32_t)row * (uint32_t)a.kb + (uint32_t)(((lane & 3) ^ swz(r)) * 16);
+        gbase[j]        = is_w ? w_base : a_base;
+        ldst[j]         = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + grp * 1024;
+    }
+    const int nb = a.n_blocks;
+    // Every block period issues one block's loads, also past the end (the last block again, into a stage nobody
+    // reads any more): the count of loads in flight is then the same in every iteration and the wait for a
+    // block is one instruction with an immediate.
+    auto issue_one = [&](int block, int stage, int j) {
+        const int blk      = block < nb ? block : nb - 1;
+        const uint8_t* src = gbase[j] + (size_t)blk * 64;
+        const uint32_t dst = ldst[j] + stage * STAGE;
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(voff[j]), "s"(src), "s"(dst)
+                     : "memory");
+    };
+#pragma unroll
+    for (int s = 0; s < kStages - 1; s++)
+#pragma unroll
+        for (int j = 0; j < LOADS; j++)
+            issue_one(s, s, j);
+
+    // ---- tables: bias per channel of the tile (in the shadow of the first loads) ---------------------------
+    int* tab_bias = reinterpret_cast<int*>(lds + kStages * STAGE);    // WROWS words
+    if (tid < WROWS)
+    {
+        const int oc = oc0 + tid;
+        int v        = 0;
+        if (oc < a.N)
+        {
+            if constexpr (M::is_int)
+                v = reinterpret_cast<const int32_t*>(a.bias)[a.bias_len == 1 ? 0 : oc];
+            else
+                v = __float_as_int(load_as_float<T>(a.bias, a.bias_len == 1 ? 0 : oc));
+        }
+        tab_bias[tid] = v;
+    }
+
+    // ---- fragment addresses -----------------------------------------------------------------------------
+    const int wrow = wo * 32 * OCT + channel_of_row(rho);
+    const int prow = WROWS + wp * 32 * PXT + rho;
+    uint32_t aw[2], ap[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++)
+    {
+        aw[s] = wrow * 64 + (((2 * s + h) ^ swz(wrow)) * 16);
+        ap[s] = prow * 64 + (((2 * s + h) ^ swz(prow)) * 16);
+    }
+
+    acc_t acc[PXT][OCT];
+#pragma unroll
+    for (int i = 0; i < PXT; i++)
+#pragma unroll
+        for (int t = 0; t < OCT; t++)
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                acc[i][t][e] = 0;
+    int wsum[OCT], psum[PXT];
+#pragma unroll
+    for (int t = 0; t < OCT; t++)
+        wsum[t] = 0;
+#pragma unroll
+    for (int i = 0; i < PXT; i++)
+        psum[i] = 0;
+
+    // ---- main loop ----------------------------------------------------------------------------------------
+    // A block is two K-steps.  The fragments of a step are requested one step ahead of their matrix
+    // instructions: step 1 of block n is read while step 0 multiplies, and step 0 of block n+1 while step 1
+    // multiplies.  The barrier that publishes block n+1 therefore sits between the two steps of block n; past
+    // it every wave has consumed block n-1, whose stage the loads of block n+3 may now overwrite.
+    //
+    // Every LDS read and every direct load is placed behind a matrix instruction (and kept there with
+    // scheduling barriers), so that the time those instructions spend waiting for a slot in the LDS and
+    // address queues - all eight waves come out of the barrier together - passes while the matrix core works.
+    constexpr int NM = OCT * PXT;    // matrix instructions per step
+    constexpr int NR = OCT + PXT;    // fragment reads per step
+    v4i fa[2][OCT], fb[2][PXT];
+    // reads in the order the matrix instructions want them: pixel tile 0, the channel tiles, the other pixel tiles
+    auto read_one = [&](const uint8_t* sb, int s, int j) {
+        if (j == 0)
+            fb[s][0] = *reinterpret_cast<const v4i*>(sb + ap[s]);
+        else if (j <= OCT)
+            fa[s][j - 1] = *reinterpret_cast<const v4i*>(sb + aw[s] + (j - 1) * 2048);
+        else
+            fb[s][j - OCT] = *reinterpret_cast<const v4i*>(sb + ap[s] + (j - OCT) * 2048);
+    };
+    auto sums = [&](int s) {
+        if constexpr (ZP)
+        {
+#pragma unroll
+            for (int t = 0; t < OCT; t++)
+                wsum[t] += dot4_ones(fa[s][t]);
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+                psum[i] += dot4_ones(fb[s][i]);
+        }
+    };
+    auto mma_one = [&](int s, int k) {
+        const int i = k / OCT, t = k % OCT;
+        acc[i][t]   = M::mma(fa[s][t], fb[s][i], acc[i][t]);
+    };
+    // A bare s_barrier: __syncthreads() would also drain this wave's LDS reads (the fragments of the step
+    // about to be multiplied), which nothing here needs.  What the barrier orders is the direct loads (waited
+    // for by hand just before it) against the reads that follow it, and the reads of two steps ago against the
+    // loads that follow it; the fragments of block n-1 were consumed before this wave got here.
+    auto publish = [&]() {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((kStages - 3) * LOADS) : "memory");
+    };
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * LOADS) : "memory");
+    __syncthreads();    // block 0 and the bias table are in LDS for every wave
+#pragma unroll
+    for (int j = 0; j < NR; j++)
+        read_one(lds, 0, j);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll 1
+    for (int n = 0; n < nb; n++)
+    {
+        const uint8_t* cur  = lds + (n % kStages) * STAGE;
+        const uint8_t* next = lds + ((n + 1) % kStages) * STAGE;
+        // two requests behind each of the first matrix instructions, so that the last ones of a step cover the
+        // latency of the fragments the next step starts with
+        constexpr int PA = NR > 2 * NM ? (NR + NM - 1) / NM : 2;
+        sums(0);
+#pragma unroll
+        for (int k = 0; k < NM; k++)
+        {
+            mma_one(0, k);
+#pragma unroll
+            for (int j = k * PA; j < (k + 1) * PA && j < NR; j++)
+                read_one(cur, 1, j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        publish();    // block n+1 (after the last block: its repeat) is in LDS for every wave
+        sums(1);
+        constexpr int NO = LOADS + NR;    // direct loads first, they have the longest way to go
+        constexpr int PB = NO > 2 * NM ? (NO + NM - 1) / NM : 2;
+#pragma unroll
+        for (int k = 0; k < NM; k++)
+        {
+            mma_one(1, k);
+#pragma unroll
+            for (int q = k * PB; q < (k + 1) * PB && q < NO; q++)
+            {
+                if (q < LOADS)
+                    issue_one(n + kStages - 1, (n + kStages - 1) % kStages, q);
+                else
+                    read_one(next, 0, q - LOADS);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- epilogue -----------------------------------------------------------------------------------------
+    // The loads issued past the last block are still on their way into LDS: let them land before a stage is
+    // given another use.  The stage buffers are then free: the channel sums go through the first one.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int* tab_wsum = reinterpret_cast<int*>(lds);    // WROWS words
+    if constexpr (ZP)
+    {
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < OCT; t++)
+        {
+            const int sum = wsum[t] + __shfl_xor(wsum[t], 32);
+            if (wp == 0 && h == 0)
+                tab_wsum[wo * 32 * OCT + t * 32 + channel_of_row(rho)] = sum;
+        }
+#pragma unroll
+        for (int i = 0; i < PXT; i++)
+            psum[i] += __shfl_xor(psum[i], 32);
+        __syncthreads();
+    }
+
+    const bool rows16 = (a.N & 15) == 0;    // every lane's 16 channels are inside the tensor or all outside
+    uint8_t* out_b    = reinterpret_cast<uint8_t*>(a.out) + batch * a.o_batch;
+#pragma unroll
+    for (int t = 0; t < OCT; t++)
+    {
+        const int ocl = wo * 32 * OCT + t * 32 + 16 * h;    // first of this lane's 16 channels in the tile
+        const int oc  = oc0 + ocl;
+        int cb[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+        {
+            const v4i b = *reinterpret_cast<const v4i*>(tab_bias + ocl + 4 * q);
+            cb[4 * q] = b.x, cb[4 * q + 1] = b.y, cb[4 * q + 2] = b.z, cb[4 * q + 3] = b.w;
+        }
+        if constexpr (ZP)
+        {
+            const int kzz = a.K * a.za * a.zw;
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+            {
+                const v4i sw = *reinterpret_cast<const v4i*>(tab_wsum + ocl + 4 * q);
+                cb[4 * q] += kzz - a.za * sw.x, cb[4 * q + 1] += kzz - a.za * sw.y;
+                cb[4 * q + 2] += kzz - a.za * sw.z, cb[4 * q + 3] += kzz - a.za * sw.w;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < PXT; i++)
+        {
+            const int p = p0 + wp * 32 * PXT + i * 32 + rho;
+            if (p >= a.M || oc >= a.N)
+                continue;
+            if constexpr (M::is_int)
+            {
+                int32_t* dst    = reinterpret_cast<int32_t*>(out_b) + (size_t)p * a.N + oc;
+                const int pcorr = ZP ? a.zw * psum[i] : 0;
+                int v[16];
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    v[e] = acc[i][t][e] + cb[e] - pcorr;
+                if (rows16)
+                {
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        reinterpret_cast<v4i*>(dst)[q] = v4i{ v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3] };
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        if (oc + e < a.N)
+                            dst[e] = v[e];
+                }
+            }
+            else
+            {
+                float v[16];
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    v[e] = acc[i][t][e] + __int_as_float(cb[e]);
+                if (a.out_is_wide)
+                {
+                    float* dst = reinterpret_cast<float*>(out_b) + (size_t)p * a.N + oc;
+                    if (rows16)
+                    {
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                            reinterpret_cast<v4f*>(dst)[q] = v4f{ v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3] };
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            if (oc + e < a.N)
+                                dst[e] = v[e];
+                    }
+                }
+                else
+                {
+                    T* dst = reinterpret_cast<T*>(out_b) + (size_t)p * a.N + oc;
+                    if (rows16)
+                    {
+                        alignas(16) T packed[16];
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            store_from_float(packed + e, v[e]);
+                        reinterpret_cast<v4i*>(dst)[0] = reinterpret_cast<const v4i*>(packed)[0];
+                        reinterpret_cast<v4i*>(dst)[1] = reinterpret_cast<const v4i*>(packed)[1];
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int e = 0; e < 16; e++)
+                            if (oc + e < a.N)
+                                store_from_float(dst + e, v[e]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int OCT, int PXT, bool ZP>
+static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
+{
+    constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4;
+    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP>;
+    static bool configured     = false;
+    if (!configured)
+    {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes) != hipSuccess)
+            return false;
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
+    return true;
+}
+
+template <typename T>
+static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const char* label)
+{
+    // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
+    // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
+    // to the patch kernel.
+    static const int shapes[3][2] = { { 4, 2 }, { 2, 2 }, { 2, 1 } };
+    int best = -1;
+    double best_cost = 0;
+    for (int c = 0; c < 3; c++)
+    {
+        const int64_t tn = (a.N + 64 * shapes[c][0] - 1) / (64 * shapes[c][0]);
+        const int64_t tm = (a.M + 128 * shapes[c][1] - 1) / (128 * shapes[c][1]);
+        const int64_t tiles = tn * tm * batches;
+        if (tiles > (1 << 22))
+            continue;
+        const double passes = (double)((tiles + 255) / 256);
+        const double cost   = passes * shapes[c][0] * shapes[c][1];
+        if (best < 0 || cost < best_cost * 0.999)
+            best = c, best_cost = cost;
+    }
+    if (best < 0)
+        return nullptr;
+    const int OCT = shapes[best][0], PXT = shapes[best][1];
+    a.tiles_n         = (a.N + 64 * OCT - 1) / (64 * OCT);
+    const int tiles_m = (a.M + 128 * PXT - 1) / (128 * PXT);
+    a.tiles_per_batch = a.tiles_n * tiles_m;
+    a.tiles_total     = a.tiles_per_batch * batches;
+    a.per_xcd         = (a.tiles_total + 7) / 8;
+    a.div_batch       = make_fastdiv((uint32_t)a.tiles_per_batch);
+    a.div_tn          = make_fastdiv((uint32_t)a.tiles_n);
+    const int blocks  = a.per_xcd * 8;
+    const bool zp     = Mma<T>::is_int && (a.za != 0 || a.zw != 0);
+    bool ok           = false;
+#define TMI_GEMM_SHAPE(O, P)                                                                                           \
+    if (OCT == O && PXT == P)                                                                                          \
+    ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int>(st, a, blocks) : launch_gemm_shape<T, O, P, false>(st, a, blocks)
+    TMI_GEMM_SHAPE(4, 2);
+    TMI_GEMM_SHAPE(2, 2);
+    TMI_GEMM_SHAPE(2, 1);
+#undef TMI_GEMM_SHAPE
+    return ok ? label : nullptr;
+}
+
+// nullptr when the operation is not a GEMM this kernel takes; the caller then goes to the patch kernel.
+const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                             const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                             void* out, int64_t w_batch_stride)
+{
+    if (rp.enabled || g.KH != 1 || g.KW != 1 || g.stride_y != 1 || g.stride_x != 1 || g.pad_top != 0 ||
+        g.pad_left != 0 || g.OH != g.IH || g.OW != g.IW)
+        return nullptr;
+    const int eb = in_dtype == TMI_INT8 ? 1 : 2;
+    if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
+        return nullptr;
+    const bool wide = in_dtype == TMI_INT8 ? out_dtype == TMI_INT32 : out_dtype == TMI_FP32;
+    if (!wide && (in_dtype == TMI_INT8 || out_dtype != in_dtype))
+        return nullptr;
+    const int64_t kb = (int64_t)g.IC * eb;
+    if (kb % 64 != 0 || kb < 256)
+        return nullptr;
+    // MATMUL: one GEMM per image with its own weights; CONV2D: all images are rows of one GEMM
+    const bool per_image  = w_batch_stride != 0;
+    const int batches     = per_image ? g.N : 1;
+    const int64_t M       = (int64_t)g.IH * g.IW * (per_image ? 1 : g.N);
+    const int64_t out_eb  = wide ? 4 : eb;
+    if (M < 128 || g.OC < 64 || M * kb >= (int64_t(1) << 32) || (int64_t)g.OC * kb >= (int64_t(1) << 32))
+        return nullptr;
+    // rows are multiples of 64 bytes, so 16-byte aligned bases keep every operand chunk aligned; the 16-byte
+    // stores are only used when OC is a multiple of 16, which keeps every output row and batch aligned too
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out) & 15) || (w_batch_stride & 15))
+        return nullptr;
+    // enough work to fill the CUs with the smallest tile shape
+    if (((M + 127) / 128) * ((g.OC + 127) / 128) * batches < 128)
+        return nullptr;
+
+    GemmArgs a{};
+    a.a = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = bias, a.out = out;
+    a.a_batch = per_image ? M * kb : 0, a.w_batch = per_image ? w_batch_stride : 0;
+    a.o_batch = per_image ? M * g.OC * out_eb : 0;
+    a.M = (int32_t)M, a.N = g.OC, a.kb = (int32_t)kb, a.n_blocks = (int32_t)(kb / 64);
+    a.bias_len = g.bias_len, a.za = in_zp, a.zw = w_zp, a.K = g.IC;
+    a.out_is_wide = wide ? 1 : 0;
+    switch (in_dtype)
+    {
+        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, "gemm_mfma_i8");
+        case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, "gemm_mfma_f16");
+        default: return launch_gemm_t<bf16_t>(st, a, batches, "gemm_mfma_bf16");
+    }
+}
+
+}    // namespace tmi

@@ -313,9 +313,14 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
     if (!depthwise && ctx->kernel_choice != 1)
-        name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
-                                  ctx->flags_dev);
-    if (!name && ctx->kernel_choice == 2)
+    {
+        if (ctx->kernel_choice != 2)
+            name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0);
+        if (!name && ctx->kernel_choice != 3)
+            name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                      ctx->flags_dev);
+    }
+    if (!name && ctx->kernel_choice >= 2)
         return fail(ctx, "%s: no MFMA / vector kernel is eligible for this shape", op);
     if (!name && depthwise)
         name = launch_depthwise_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
@@ -431,7 +436,7 @@ const char* tmi_last_kernel(const tmi_ctx_t* ctx)
 
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
-    if (!ctx || choice < 0 || choice > 2)
+    if (!ctx || choice < 0 || choice > 3)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;
@@ -787,13 +792,22 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
         RescaleParams none{};
         if (!launch_transpose(ctx->stream, eb, N, C, W, b_dev, ctx->workspace))
             return fail(ctx, "OpMatMul: transpose launch failed");
-        name = launch_conv2d_mfma(ctx->stream, in_dtype, in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32, g, a_dev,
-                                  ctx->workspace, ctx->flags_dev + 16, a_zp, b_zp, none, out_dev, ctx->flags_dev,
-                                  (int64_t)W * C * eb);
+        const int32_t out_dtype = in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32;
+        if (ctx->kernel_choice != 2)
+            name = launch_gemm_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, ctx->workspace, ctx->flags_dev + 16,
+                                    a_zp, b_zp, none, out_dev, (int64_t)W * C * eb);
         if (name)
-            name = in_dtype == TMI_INT8 ? "matmul_mfma_i8" : (in_dtype == TMI_FP16 ? "matmul_mfma_f16" : "matmul_mfma_bf16");
+            name = in_dtype == TMI_INT8 ? "matmul_gemm_i8" : (in_dtype == TMI_FP16 ? "matmul_gemm_f16" : "matmul_gemm_bf16");
+        else if (ctx->kernel_choice != 3)
+        {
+            name = launch_conv2d_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, ctx->workspace, ctx->flags_dev + 16,
+                                      a_zp, b_zp, none, out_dev, ctx->flags_dev, (int64_t)W * C * eb);
+            if (name)
+                name = in_dtype == TMI_INT8 ? "matmul_mfma_i8"
+                                            : (in_dtype == TMI_FP16 ? "matmul_mfma_f16" : "matmul_mfma_bf16");
+        }
     }
-    if (!name && ctx->kernel_choice == 2)
+    if (!name && ctx->kernel_choice >= 2)
         return fail(ctx, "OpMatMul: no MFMA kernel is eligible for this shape");
     if (!name)
         name = launch_matmul_direct(ctx->stream, in_dtype, N, H, C, W, a_dev, b_dev, a_zp, b_zp, out_dev);

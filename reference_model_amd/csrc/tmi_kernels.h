@@ -66,6 +66,12 @@ const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_d
 const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                     const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                     const RescaleParams& rp, void* out, uint32_t* flag_word);
+// gemm_mfma.hip: 1x1 / stride 1 / unpadded CONV2D and MATMUL (w_batch_stride != 0: per-image weights) with
+// operands loaded straight into LDS; nullptr when the operation is not such a GEMM or too small to gain.
+const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                             const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                             void* out, int64_t w_batch_stride);
+
 // conv2d_mfma.hip: implicit GEMM on the matrix cores with the fused epilogue; nullptr when not eligible.
 const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,

@@ -1,0 +1,149 @@
+"""GPU parity of the MFMA GEMM kernel (1x1 CONV2D and MATMUL with operands loaded straight into LDS) against
+the CPU oracle and exact float64 BLAS products, through the C ABI.  int8 results are compared bit for bit;
+fp16 / bf16 results with the reference's DOT_PRODUCT bound against fp64 (tolerance stated at the assert)."""
+import numpy as np
+import pytest
+
+import cases
+import dot_product_check as dp
+import gpu_ops
+import oracle
+from reference_model_amd import Context, TmiError, capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = Context(0)
+    c.set_kernel_choice(capi.KERNEL_GEMM)
+    yield c
+    c.close()
+
+
+def exact_matmul_i8(a, b, a_zp, b_zp):
+    """float64 BLAS product: exact, every partial sum is an integer below 2^53"""
+    want = np.matmul(a.astype(np.float64) - a_zp, b.astype(np.float64) - b_zp)
+    return want.astype(np.int64).astype(np.int32)
+
+
+# n, h, c, w: the three workgroup shapes (256x256, 128x256, 128x128 channels x pixels), ragged edges in both
+# directions, channel counts that are not a multiple of 16, one and many 64-byte K blocks
+GEMM_SHAPES = [
+    (4, 2048, 320, 2048),     # 256 tiles of 256x256
+    (8, 1024, 256, 1024),     # 128x256 tiles
+    (2, 1024, 1024, 1024),    # 128x128 tiles
+    (3, 1000, 448, 1100),     # ragged rows and columns, columns a multiple of 4 only
+    (1, 4099, 256, 515),      # odd column count: element-wise stores
+    (32, 300, 64 * 5, 200),
+    (1, 128, 256, 16384),
+    (1, 16384, 256, 64),
+]
+
+
+@pytest.mark.parametrize("shape", GEMM_SHAPES)
+@pytest.mark.parametrize("zps", [(0, 0), (7, -9), (-128, 0), (0, 127)])
+def test_matmul_i8_gemm_bit_exact(ctx, shape, zps):
+    n, h, c, w = shape
+    rng = np.random.default_rng(n * 1000 + h + c + w)
+    a = rng.integers(-128, 128, (n, h, c)).astype(np.int8)
+    b = rng.integers(-128, 128, (n, c, w)).astype(np.int8)
+    got, st = gpu_ops.matmul(ctx, a, b, *zps)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_i8"
+    assert np.array_equal(got, exact_matmul_i8(a, b, *zps))
+    # a corner of the last batch against the scalar oracle (the BLAS product is a second, independent witness)
+    assert np.array_equal(got[-1, -24:], oracle.matmul("i8", a[-1:, -24:], b[-1:], *zps)[0])
+
+
+def test_matmul_i8_gemm_extreme_values(ctx):
+    """all operands at -128 with zero points at +127: the largest products the operator can form"""
+    n, h, c, w = 8, 512, 4096, 512
+    a = np.full((n, h, c), -128, np.int8)
+    b = np.full((n, c, w), -128, np.int8)
+    got, st = gpu_ops.matmul(ctx, a, b, 127, 127)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_i8"
+    assert np.all(got == 255 * 255 * c)
+
+
+def test_gemm_kernel_refuses_what_it_cannot_take(ctx):
+    rng = np.random.default_rng(1)
+    a = rng.integers(-128, 128, (1, 512, 100)).astype(np.int8)     # K bytes not a multiple of 64
+    b = rng.integers(-128, 128, (1, 100, 512)).astype(np.int8)
+    with pytest.raises(TmiError):
+        gpu_ops.matmul(ctx, a, b)
+    a = rng.integers(-128, 128, (1, 64, 256)).astype(np.int8)      # too little work
+    b = rng.integers(-128, 128, (1, 256, 64)).astype(np.int8)
+    with pytest.raises(TmiError):
+        gpu_ops.matmul(ctx, a, b)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (1, 4099, 128, 515)])
+def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
+    n, h, c, w = shape
+    rng = np.random.default_rng(8 + h)
+    a = rng.normal(0, 1 / 8, (n, h, c)).astype(np.float32)
+    b = rng.normal(0, 1 / 8, (n, c, w)).astype(np.float32)
+    if kind == "fp16":
+        a_s, b_s, dtype = a.astype(np.float16), b.astype(np.float16), capi.FP16
+        af, bf = a_s.astype(np.float64), b_s.astype(np.float64)
+    else:
+        a_s, b_s, dtype = cases.float_to_bf16_bits(a), cases.float_to_bf16_bits(b), capi.BF16
+        af, bf = cases.bf16_bits_to_float(a_s).astype(np.float64), cases.bf16_bits_to_float(b_s).astype(np.float64)
+    got, st = gpu_ops.matmul(ctx, a_s, b_s, dtype=dtype)
+    assert st == capi.VALID and got.dtype == np.float32
+    assert ctx.last_kernel == ("matmul_gemm_f16" if kind == "fp16" else "matmul_gemm_bf16")
+    ref, bnd = np.matmul(af, bf), np.matmul(np.abs(af), np.abs(bf))
+    res = dp.check(got, ref, bnd, "fp32", dp.kernel_size_bound(c, "fp32", has_bias=False))
+    # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
+    assert res["ok"], res
+
+
+# ---- 1x1 CONV2D: all images are rows of one GEMM, bias per channel ---------------------------------------------
+@pytest.mark.parametrize("shape", [  # n, ih, iw, ic, oc
+    (8, 56, 56, 256, 64),
+    (4, 28, 28, 512, 648),
+    (1, 97, 131, 256, 130),
+])
+@pytest.mark.parametrize("zps", [(0, 0), (-6, 11)])
+def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
+    n, ih, iw, ic, oc = shape
+    rng = np.random.default_rng(ih * iw + oc)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 1, 1, ic)).astype(np.int8)
+    bias = rng.integers(-(1 << 20), 1 << 20, oc).astype(np.int32)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, in_zp=zps[0], w_zp=zps[1])
+    assert st == capi.VALID and ctx.last_kernel == "gemm_mfma_i8"
+    want = exact_matmul_i8(x.reshape(1, -1, ic), w.reshape(1, oc, ic).transpose(0, 2, 1), *zps)[0] + bias
+    assert np.array_equal(got.reshape(-1, oc), want)
+    sub = oracle.conv2d("i8", x[-1:, -2:], w, bias, in_zp=zps[0], w_zp=zps[1])
+    assert np.array_equal(got[-1:, -2:], sub)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203)])
+def test_conv2d_1x1_fp_gemm_within_dot_product_bound(ctx, kind, shape):
+    n, ih, iw, ic, oc = shape
+    rng = np.random.default_rng(ic + oc)
+    x = rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float32)
+    w = rng.normal(0, 1 / np.sqrt(ic), (oc, 1, 1, ic)).astype(np.float32)
+    b = rng.normal(0, 0.1, oc).astype(np.float32)
+    if kind == "fp16":
+        xs, ws, bs = x.astype(np.float16), w.astype(np.float16), b.astype(np.float16)
+        xf, wf, bf = (v.astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.FP16
+    else:
+        xs, ws, bs = (cases.float_to_bf16_bits(v) for v in (x, w, b))
+        xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.BF16
+    got, st = gpu_ops.conv2d(ctx, xs, ws, bs, dtype=dtype)
+    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16")
+    imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
+    ref = np.matmul(xf.reshape(-1, ic), wf.reshape(oc, ic).T) + bf
+    bnd = np.matmul(np.abs(xf.reshape(-1, ic)), np.abs(wf.reshape(oc, ic).T)) + np.abs(bf)
+    res = dp.check(imp.reshape(-1, oc), ref, bnd, kind, dp.kernel_size_bound(ic, kind))
+    # tolerance: |imp-ref| <= 2*ksb * max(bnd*2^-(1+frac), normal_min) per element, sum err^2 <= 1.6*ksb*T
+    assert res["ok"], res
+    # a corner against the oracle's own loop nest
+    sub = oracle.conv2d("f64", xf[-1:, -2:], wf, bf, (0, 0, 0, 0), (1, 1), (1, 1))
+    assert np.allclose(imp[-1:, -2:], sub, rtol=2.0 ** -7, atol=2.0 ** -10)
