@@ -42,6 +42,7 @@ struct GemmArgs
     int32_t tiles_n, tiles_per_batch, tiles_total, per_xcd;
     int32_t bias_len, za, zw, K;
     int32_t out_is_wide;    // floating point: 1 = fp32 output, 0 = output of the input type
+    int32_t ldw;            // K-major weights: bytes between consecutive K rows (rows of N elements)
     FastDiv div_batch, div_tn;
 };
 
@@ -68,10 +69,35 @@ __device__ __forceinline__ int channel_of_row(int rho)
 // matrix instruction, not the barrier, is what the smaller shapes wait for).
 static constexpr int kStages = 4;
 
-template <typename T, int OCT, int PXT, bool ZP>
+// K-major weights (KM): the weight operand lies in memory as [K][N] (MATMUL's second operand as the operator
+// defines it).  Its part of a stage is then 64 / sizeof(T) rows of K with the tile's 64*OCT channels side by
+// side, loaded as it lies (whole 16-byte pieces of a K row per lane), and the fragments come out of LDS through
+// the transposing reads ds_read_b64_tr_b16 / _b8: a block of 16 lanes hands in 16 addresses of 8 bytes and
+// gets back, per lane, the elements of one column - 4 consecutive K of one channel (2-byte types) or 8 (int8) -
+// so two reads make the 16 bytes of K a lane feeds the matrix instruction.  A transposing read serves 32
+// lanes a cycle; their addresses are 4 (8) consecutive K rows x 64 (32) bytes, which the row stride alone
+// would put on the same banks, so the 64-byte (32-byte) segments of a row are permuted by the row number.
+// With int8 the 8 lanes that share a source address get 8 consecutive channels, so the accumulator rows of
+// the int8 K-major variant are assigned to channels in order (row r is channel r) and a lane stores four
+// groups of 4 channels instead of 16 consecutive ones.
+template <typename T, int OCT, int PXT, bool ZP, bool KM>
 __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 {
     using M                = Mma<T>;
+    constexpr int EB       = (int)sizeof(T);
+    constexpr bool IDENT   = KM && EB == 1;    // accumulator row r of a channel tile is channel r
+    constexpr int RB       = 64 * OCT * EB;    // KM: bytes of a K row in LDS
+    constexpr int KSTEP    = 32 / EB;          // K rows per matrix instruction
+    // KM: units of 16 bytes a row's pieces are moved by, as a function of the K row
+    auto km_swizzle = [](int k) {
+        if constexpr (EB == 2)
+            return (k & 3) << 2;
+        else if constexpr (RB >= 256)
+            return (k & 7) << 1;
+        else
+            return ((k >> 1) & 3) << 1;
+    };
+    auto row_channel = [](int r) { return IDENT ? r : channel_of_row(r); };
     using acc_t            = typename M::acc_t;
     constexpr int WROWS    = 64 * OCT;
     constexpr int PROWS    = 128 * PXT;
@@ -110,6 +136,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     uint32_t voff[LOADS];
     const uint8_t* gbase[LOADS];
     uint32_t ldst[LOADS];
+    uint32_t gstep[LOADS];    // bytes a load's source advances per block
 #pragma unroll
     for (int j = 0; j < LOADS; j++)
     {
@@ -121,6 +148,18 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         row             = row < last ? row : last;    // rows past the end repeat the last one; never stored
         voff[j]         = (uint32_t)row * (uint32_t)a.kb + (uint32_t)(((lane & 3) ^ swz(r)) * 16);
         gbase[j]        = is_w ? w_base : a_base;
+        gstep[j]        = 64;
+        if (KM && is_w)
+        {
+            // 16-byte unit of the weight part -> K row of the block and piece of that row
+            const int unit = grp * 64 + lane;
+            const int k    = unit / (RB / 16);
+            const int pc   = (unit % (RB / 16)) ^ km_swizzle(k);
+            int col        = oc0 * EB + pc * 16;
+            col            = col < a.N * EB - 16 ? col : a.N * EB - 16;    // pieces past the row end: never used
+            voff[j]        = (uint32_t)k * (uint32_t)a.ldw + (uint32_t)col;
+            gstep[j]       = (uint32_t)(64 / EB) * (uint32_t)a.ldw;
+        }
         ldst[j]         = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + grp * 1024;
     }
     const int nb = a.n_blocks;
@@ -129,7 +168,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     // block is one instruction with an immediate.
     auto issue_one = [&](int block, int stage, int j) {
         const int blk      = block < nb ? block : nb - 1;
-        const uint8_t* src = gbase[j] + (size_t)blk * 64;
+        const uint8_t* src = gbase[j] + (size_t)blk * gstep[j];
         const uint32_t dst = ldst[j] + stage * STAGE;
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
@@ -159,7 +198,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     }
 
     // ---- fragment addresses -----------------------------------------------------------------------------
-    const int wrow = wo * 32 * OCT + channel_of_row(rho);
+    const int wrow = wo * 32 * OCT + row_channel(rho);
     const int prow = WROWS + wp * 32 * PXT + rho;
     uint32_t aw[2], ap[2];
 #pragma unroll
@@ -167,6 +206,34 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     {
         aw[s] = wrow * 64 + (((2 * s + h) ^ swz(wrow)) * 16);
         ap[s] = prow * 64 + (((2 * s + h) ^ swz(prow)) * 16);
+    }
+
+    // KM: per channel tile, the address this lane hands to the transposing reads of K-step 0, first read
+    uint32_t akm[OCT];
+    if constexpr (KM)
+    {
+        const int sl   = lane & 15;           // position in the 16-lane block of a transposing read
+        const int brho = (lane >> 4) & 1;     // which 16 accumulator rows of the tile the block serves
+#pragma unroll
+        for (int t = 0; t < OCT; t++)
+        {
+            const int tile = wo * OCT + t;
+            if constexpr (EB == 2)
+            {
+                // source lane sl: K row sl / 4 of the four, channels cb .. cb+3 (lanes 4a .. 4a+3 receive them)
+                const int m  = sl >> 2;
+                const int a4 = sl & 3;
+                const int cb = 16 * (a4 & 1) + 4 * (2 * brho + (a4 >> 1));
+                akm[t]       = (8 * h + m) * RB + ((((tile ^ m) << 2) + (cb >> 3)) << 4) + ((cb * 2) & 15);
+            }
+            else
+            {
+                // source lane sl: K row sl / 2 of the eight, channels 16*brho + 8*(sl % 2) .. +7
+                const int m8 = sl >> 1;
+                const int m  = RB >= 256 ? m8 : (m8 >> 1);
+                akm[t]       = (16 * h + m8) * RB + ((((tile ^ m) << 1) + brho) << 4) + 8 * (sl & 1);
+            }
+        }
     }
 
     acc_t acc[PXT][OCT];
@@ -195,16 +262,33 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     // scheduling barriers), so that the time those instructions spend waiting for a slot in the LDS and
     // address queues - all eight waves come out of the barrier together - passes while the matrix core works.
     constexpr int NM = OCT * PXT;    // matrix instructions per step
-    constexpr int NR = OCT + PXT;    // fragment reads per step
+    constexpr int NW = KM ? 2 * OCT : OCT;    // weight fragment reads per step
+    constexpr int NR = NW + PXT;              // fragment reads per step
     v4i fa[2][OCT], fb[2][PXT];
     // reads in the order the matrix instructions want them: pixel tile 0, the channel tiles, the other pixel tiles
     auto read_one = [&](const uint8_t* sb, int s, int j) {
         if (j == 0)
             fb[s][0] = *reinterpret_cast<const v4i*>(sb + ap[s]);
-        else if (j <= OCT)
-            fa[s][j - 1] = *reinterpret_cast<const v4i*>(sb + aw[s] + (j - 1) * 2048);
+        else if (j <= NW)
+        {
+            if constexpr (KM)
+            {
+                const int t = (j - 1) >> 1, r = (j - 1) & 1;
+                const uint8_t* src = sb + akm[t] + (KSTEP * s + (KSTEP / 4) * r) * RB;
+                v2i half;
+                if constexpr (EB == 2)
+                    half = __builtin_bit_cast(v2i, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                                       (__attribute__((address_space(3))) v4s*)src));
+                else
+                    half = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i*)src);
+                fa[s][t][2 * r]     = half.x;
+                fa[s][t][2 * r + 1] = half.y;
+            }
+            else
+                fa[s][j - 1] = *reinterpret_cast<const v4i*>(sb + aw[s] + (j - 1) * 2048);
+        }
         else
-            fb[s][j - OCT] = *reinterpret_cast<const v4i*>(sb + ap[s] + (j - OCT) * 2048);
+            fb[s][j - NW] = *reinterpret_cast<const v4i*>(sb + ap[s] + (j - NW) * 2048);
     };
     auto sums = [&](int s) {
         if constexpr (ZP)
@@ -285,7 +369,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         {
             const int sum = wsum[t] + __shfl_xor(wsum[t], 32);
             if (wp == 0 && h == 0)
-                tab_wsum[wo * 32 * OCT + t * 32 + channel_of_row(rho)] = sum;
+                tab_wsum[wo * 32 * OCT + t * 32 + row_channel(rho)] = sum;
         }
 #pragma unroll
         for (int i = 0; i < PXT; i++)
@@ -293,18 +377,21 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         __syncthreads();
     }
 
+    // A lane's 16 accumulator registers of a tile are four groups of 4 consecutive channels: group q starts at
+    // channel 16h + 4q (all 16 consecutive), or 8q + 4h with the in-order row assignment.
+    auto group_channel = [&](int q) { return IDENT ? 8 * q + 4 * h : 16 * h + 4 * q; };
     const bool rows16 = (a.N & 15) == 0;    // every lane's 16 channels are inside the tensor or all outside
+    const bool rows4  = (a.N & 3) == 0;     // the same for a group of 4
     uint8_t* out_b    = reinterpret_cast<uint8_t*>(a.out) + batch * a.o_batch;
 #pragma unroll
     for (int t = 0; t < OCT; t++)
     {
-        const int ocl = wo * 32 * OCT + t * 32 + 16 * h;    // first of this lane's 16 channels in the tile
-        const int oc  = oc0 + ocl;
+        const int tl = wo * 32 * OCT + t * 32;    // first channel of the tile within the workgroup's channels
         int cb[16];
 #pragma unroll
         for (int q = 0; q < 4; q++)
         {
-            const v4i b = *reinterpret_cast<const v4i*>(tab_bias + ocl + 4 * q);
+            const v4i b = *reinterpret_cast<const v4i*>(tab_bias + tl + group_channel(q));
             cb[4 * q] = b.x, cb[4 * q + 1] = b.y, cb[4 * q + 2] = b.z, cb[4 * q + 3] = b.w;
         }
         if constexpr (ZP)
@@ -313,7 +400,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 #pragma unroll
             for (int q = 0; q < 4; q++)
             {
-                const v4i sw = *reinterpret_cast<const v4i*>(tab_wsum + ocl + 4 * q);
+                const v4i sw = *reinterpret_cast<const v4i*>(tab_wsum + tl + group_channel(q));
                 cb[4 * q] += kzz - a.za * sw.x, cb[4 * q + 1] += kzz - a.za * sw.y;
                 cb[4 * q + 2] += kzz - a.za * sw.z, cb[4 * q + 3] += kzz - a.za * sw.w;
             }
@@ -322,32 +409,39 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         for (int i = 0; i < PXT; i++)
         {
             const int p = p0 + wp * 32 * PXT + i * 32 + rho;
-            if (p >= a.M || oc >= a.N)
+            if (p >= a.M || oc0 + tl >= a.N)
                 continue;
             if constexpr (M::is_int)
             {
-                int32_t* dst    = reinterpret_cast<int32_t*>(out_b) + (size_t)p * a.N + oc;
+                int32_t* row    = reinterpret_cast<int32_t*>(out_b) + (size_t)p * a.N;
                 const int pcorr = ZP ? a.zw * psum[i] : 0;
-                int v[16];
 #pragma unroll
-                for (int e = 0; e < 16; e++)
-                    v[e] = acc[i][t][e] + cb[e] - pcorr;
-                if (rows16)
+                for (int q = 0; q < 4; q++)
                 {
+                    const int oc = oc0 + tl + group_channel(q);
+                    int v[4];
 #pragma unroll
-                    for (int q = 0; q < 4; q++)
-                        reinterpret_cast<v4i*>(dst)[q] = v4i{ v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3] };
-                }
-                else
-                {
+                    for (int e = 0; e < 4; e++)
+                        v[e] = acc[i][t][4 * q + e] + cb[4 * q + e] - pcorr;
+                    if (rows4)
+                    {
+                        if (oc < a.N)
+                            *reinterpret_cast<v4i*>(row + oc) = v4i{ v[0], v[1], v[2], v[3] };
+                    }
+                    else
+                    {
 #pragma unroll
-                    for (int e = 0; e < 16; e++)
-                        if (oc + e < a.N)
-                            dst[e] = v[e];
+                        for (int e = 0; e < 4; e++)
+                            if (oc + e < a.N)
+                                row[oc + e] = v[e];
+                    }
                 }
             }
             else
             {
+                const int oc = oc0 + tl + 16 * h;    // floating point: always 16 consecutive channels
+                if (oc >= a.N)
+                    continue;
                 float v[16];
 #pragma unroll
                 for (int e = 0; e < 16; e++)
@@ -394,11 +488,11 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     }
 }
 
-template <typename T, int OCT, int PXT, bool ZP>
+template <typename T, int OCT, int PXT, bool ZP, bool KM>
 static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
 {
     constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4;
-    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP>;
+    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, KM>;
     static bool configured     = false;
     if (!configured)
     {
@@ -447,7 +541,14 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const
     bool ok           = false;
 #define TMI_GEMM_SHAPE(O, P)                                                                                           \
     if (OCT == O && PXT == P)                                                                                          \
-    ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int>(st, a, blocks) : launch_gemm_shape<T, O, P, false>(st, a, blocks)
+    {                                                                                                                  \
+        if (a.ldw)                                                                                                     \
+            ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int, true>(st, a, blocks)                                  \
+                    : launch_gemm_shape<T, O, P, false, true>(st, a, blocks);                                          \
+        else                                                                                                           \
+            ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int, false>(st, a, blocks)                                 \
+                    : launch_gemm_shape<T, O, P, false, false>(st, a, blocks);                                         \
+    }
     TMI_GEMM_SHAPE(4, 2);
     TMI_GEMM_SHAPE(2, 2);
     TMI_GEMM_SHAPE(2, 1);
@@ -458,7 +559,7 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const
 // nullptr when the operation is not a GEMM this kernel takes; the caller then goes to the patch kernel.
 const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                              const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                             void* out, int64_t w_batch_stride)
+                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride)
 {
     if (rp.enabled || g.KH != 1 || g.KW != 1 || g.stride_y != 1 || g.stride_x != 1 || g.pad_top != 0 ||
         g.pad_left != 0 || g.OH != g.IH || g.OW != g.IW)
@@ -479,6 +580,9 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     const int64_t out_eb  = wide ? 4 : eb;
     if (M < 128 || g.OC < 64 || M * kb >= (int64_t(1) << 32) || (int64_t)g.OC * kb >= (int64_t(1) << 32))
         return nullptr;
+    // K-major weights: whole 16-byte pieces per K row
+    if (w_kmajor_stride && ((w_kmajor_stride & 15) || w_kmajor_stride != (int64_t)g.OC * eb))
+        return nullptr;
     // rows are multiples of 64 bytes, so 16-byte aligned bases keep every operand chunk aligned; the 16-byte
     // stores are only used when OC is a multiple of 16, which keeps every output row and batch aligned too
     if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out) & 15) || (w_batch_stride & 15))
@@ -494,6 +598,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     a.M = (int32_t)M, a.N = g.OC, a.kb = (int32_t)kb, a.n_blocks = (int32_t)(kb / 64);
     a.bias_len = g.bias_len, a.za = in_zp, a.zw = w_zp, a.K = g.IC;
     a.out_is_wide = wide ? 1 : 0;
+    a.ldw         = (int32_t)w_kmajor_stride;
     switch (in_dtype)
     {
         case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, "gemm_mfma_i8");

@@ -777,27 +777,40 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
     const char* name = nullptr;
     if (ctx->kernel_choice != 1 && C > 0)
     {
-        // MFMA path: make B K-contiguous ([N,C,W] -> [N,W,C]) in the context's scratch buffer, then run the
-        // implicit-GEMM kernel with one "image" per batch: pixels = rows of A, output channels = columns of
-        // B, 1x1 taps, per-image weights.  The bias operand is the permanently zero word kept after the flags.
-        const int eb       = in_dtype == TMI_INT8 ? 1 : 2;
-        const size_t bytes = (size_t)N * C * W * eb;
-        int rc             = ensure_workspace(ctx, bytes);
-        if (rc != TMI_VALID)
-            return rc;
+        // MFMA paths: one "image" per batch, pixels = rows of A, output channels = columns of B, 1x1 taps,
+        // per-image weights.  The bias operand is the permanently zero word kept after the flags.  The GEMM
+        // kernel takes B as it lies in memory ([C][W], transposed on its way out of LDS); what it does not
+        // take that way (rows of B that are not whole 16-byte pieces) is first made K-contiguous ([N,C,W] ->
+        // [N,W,C]) in the context's scratch buffer and offered to the GEMM kernel again, then to the
+        // implicit-GEMM kernel.
+        const int eb = in_dtype == TMI_INT8 ? 1 : 2;
         ConvGeom g{};
         g.N = N, g.IH = H, g.IW = 1, g.IC = C, g.OC = W, g.KH = 1, g.KW = 1, g.OH = H, g.OW = 1;
         g.stride_y = g.stride_x = g.dil_y = g.dil_x = 1;
         g.bias_len = 1, g.M = 1;
         RescaleParams none{};
-        if (!launch_transpose(ctx->stream, eb, N, C, W, b_dev, ctx->workspace))
-            return fail(ctx, "OpMatMul: transpose launch failed");
         const int32_t out_dtype = in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32;
         if (ctx->kernel_choice != 2)
-            name = launch_gemm_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, ctx->workspace, ctx->flags_dev + 16,
-                                    a_zp, b_zp, none, out_dev, (int64_t)W * C * eb);
-        if (name)
+            name = launch_gemm_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, b_dev, ctx->flags_dev + 16, a_zp, b_zp,
+                                    none, out_dev, (int64_t)W * C * eb, (int64_t)W * eb);
+        const bool direct = name != nullptr;    // B read as it lies, no transposed copy
+        if (!name)
+        {
+            const size_t bytes = (size_t)N * C * W * eb;
+            int rc             = ensure_workspace(ctx, bytes);
+            if (rc != TMI_VALID)
+                return rc;
+            if (!launch_transpose(ctx->stream, eb, N, C, W, b_dev, ctx->workspace))
+                return fail(ctx, "OpMatMul: transpose launch failed");
+            if (ctx->kernel_choice != 2)
+                name = launch_gemm_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, ctx->workspace, ctx->flags_dev + 16,
+                                        a_zp, b_zp, none, out_dev, (int64_t)W * C * eb);
+        }
+        if (name && direct)
             name = in_dtype == TMI_INT8 ? "matmul_gemm_i8" : (in_dtype == TMI_FP16 ? "matmul_gemm_f16" : "matmul_gemm_bf16");
+        else if (name)
+            name = in_dtype == TMI_INT8 ? "matmul_tgemm_i8"
+                                        : (in_dtype == TMI_FP16 ? "matmul_tgemm_f16" : "matmul_tgemm_bf16");
         else if (ctx->kernel_choice != 3)
         {
             name = launch_conv2d_mfma(ctx->stream, in_dtype, out_dtype, g, a_dev, ctx->workspace, ctx->flags_dev + 16,

@@ -68,9 +68,11 @@ const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t ou
                                     const RescaleParams& rp, void* out, uint32_t* flag_word);
 // gemm_mfma.hip: 1x1 / stride 1 / unpadded CONV2D and MATMUL (w_batch_stride != 0: per-image weights) with
 // operands loaded straight into LDS; nullptr when the operation is not such a GEMM or too small to gain.
+// w_kmajor_stride != 0: the weights are [K][OC] with that many bytes per K row (MATMUL's second operand as it
+// lies in memory) instead of [OC][K].
 const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                              const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                             void* out, int64_t w_batch_stride);
+                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride = 0);
 
 // conv2d_mfma.hip: implicit GEMM on the matrix cores with the fused epilogue; nullptr when not eligible.
 const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,

@@ -6,6 +6,8 @@
 namespace tmi
 {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));

@@ -34,6 +34,8 @@ GEMM_SHAPES = [
     (8, 1024, 256, 1024),     # 128x256 tiles
     (2, 1024, 1024, 1024),    # 128x128 tiles
     (3, 1000, 448, 1100),     # ragged rows and columns, columns a multiple of 4 only
+    (3, 1000, 448, 1104),     # ragged, whole 16-byte pieces per row of B
+    (5, 520, 192 * 3, 784),
     (1, 4099, 256, 515),      # odd column count: element-wise stores
     (32, 300, 64 * 5, 200),
     (1, 128, 256, 16384),
@@ -49,7 +51,8 @@ def test_matmul_i8_gemm_bit_exact(ctx, shape, zps):
     a = rng.integers(-128, 128, (n, h, c)).astype(np.int8)
     b = rng.integers(-128, 128, (n, c, w)).astype(np.int8)
     got, st = gpu_ops.matmul(ctx, a, b, *zps)
-    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_i8"
+    # B is read as it lies when its rows are whole 16-byte pieces, else from a transposed copy
+    assert st == capi.VALID and ctx.last_kernel == ("matmul_gemm_i8" if w % 16 == 0 else "matmul_tgemm_i8")
     assert np.array_equal(got, exact_matmul_i8(a, b, *zps))
     # a corner of the last batch against the scalar oracle (the BLAS product is a second, independent witness)
     assert np.array_equal(got[-1, -24:], oracle.matmul("i8", a[-1:, -24:], b[-1:], *zps)[0])
@@ -78,7 +81,8 @@ def test_gemm_kernel_refuses_what_it_cannot_take(ctx):
 
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (1, 4099, 128, 515)])
+@pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (3, 1000, 448, 1104),
+                                   (1, 4099, 128, 515), (5, 520, 96 * 3, 784)])
 def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, h, c, w = shape
     rng = np.random.default_rng(8 + h)
@@ -92,7 +96,7 @@ def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
         af, bf = cases.bf16_bits_to_float(a_s).astype(np.float64), cases.bf16_bits_to_float(b_s).astype(np.float64)
     got, st = gpu_ops.matmul(ctx, a_s, b_s, dtype=dtype)
     assert st == capi.VALID and got.dtype == np.float32
-    assert ctx.last_kernel == ("matmul_gemm_f16" if kind == "fp16" else "matmul_gemm_bf16")
+    assert ctx.last_kernel == ("matmul_" + ("gemm" if w % 8 == 0 else "tgemm") + ("_f16" if kind == "fp16" else "_bf16"))
     ref, bnd = np.matmul(af, bf), np.matmul(np.abs(af), np.abs(bf))
     res = dp.check(got, ref, bnd, "fp32", dp.kernel_size_bound(c, "fp32", has_bias=False))
     # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
@@ -147,3 +151,38 @@ def test_conv2d_1x1_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     # a corner against the oracle's own loop nest
     sub = oracle.conv2d("f64", xf[-1:, -2:], wf, bf, (0, 0, 0, 0), (1, 1), (1, 1))
     assert np.allclose(imp[-1:, -2:], sub, rtol=2.0 ** -7, atol=2.0 ** -10)
+
+
+# ---- the benchmark configurations at full size ----------------------------------------------------------------
+def test_config2_matmul_full_size_gemm(ctx):
+    """[8,1024,1024] x [8,1024,1024] -> int32, a_zp -5, b_zp 3: every element against a float64 BLAS product
+    (exact: |sum| < 2^53), one batch corner against the scalar oracle, plus the transposition property
+    (A.B)^T = B^T.A^T computed by the same kernel."""
+    c = cases.c2()
+    got, st = gpu_ops.matmul(ctx, c["a"], c["b"], c["a_zp"], c["b_zp"])
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_i8"
+    assert np.array_equal(got, exact_matmul_i8(c["a"], c["b"], c["a_zp"], c["b_zp"]))
+    assert np.array_equal(got[5, :16], oracle.matmul("i8", c["a"][5:6, :16], c["b"][5:6], c["a_zp"], c["b_zp"])[0])
+    at = np.ascontiguousarray(c["a"].transpose(0, 2, 1))
+    bt = np.ascontiguousarray(c["b"].transpose(0, 2, 1))
+    got_t, _ = gpu_ops.matmul(ctx, bt, at, c["b_zp"], c["a_zp"])
+    assert np.array_equal(got_t, got.transpose(0, 2, 1))
+
+
+def test_config5_bf16_matmul_full_size_gemm(ctx):
+    """[4,2048,4096] x [4,4096,2048] bf16 -> fp32.  256 rows of every batch against fp64 with the DOT_PRODUCT
+    bound; the whole result through a property that needs no reference: scaling A by 2 (exact in bf16) must
+    scale every fp32 partial sum, hence every result, by exactly 2."""
+    c = cases.c5_matmul()
+    got, st = gpu_ops.matmul(ctx, c["a"], c["b"], dtype=capi.BF16)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_bf16"
+    rows = slice(1000, 1256)
+    af = cases.bf16_bits_to_float(c["a"][:, rows]).astype(np.float64)
+    bf = cases.bf16_bits_to_float(c["b"]).astype(np.float64)
+    ref, bnd = np.matmul(af, bf), np.matmul(np.abs(af), np.abs(bf))
+    res = dp.check(got[:, rows], ref, bnd, "fp32", dp.kernel_size_bound(c["a"].shape[2], "fp32", has_bias=False))
+    # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
+    assert res["ok"], res
+    a2 = cases.float_to_bf16_bits(cases.bf16_bits_to_float(c["a"]) * 2.0)
+    got2, _ = gpu_ops.matmul(ctx, a2, c["b"], dtype=capi.BF16)
+    assert np.array_equal(got2, got * np.float32(2.0))
