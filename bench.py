@@ -44,7 +44,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "copy"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,6 +110,32 @@ def main() -> int:
                  peak=PEAK["hbm"], runit="GB/s",
                  workload="RESCALE int32 [64,56,56,64] -> int8, per-channel multiplier/shift 38, double_round, "
                           "output_zp -3 (5 bytes per element)")
+    elif cfg in ("maxpool", "avgpool"):
+        # the pooling neighbours at sizes where launch latency no longer dominates: the 3x3 stride-2 max pooling
+        # behind a ResNet stem for 32 images, and a 2x2 stride-2 average pooling of the same tensor
+        import oracle
+        rng = np.random.default_rng(cases.SEED ^ (8 if cfg == "maxpool" else 2))
+        x = rng.integers(-128, 128, (32, 112, 112, 64)).astype(np.int8)
+        pk, ps, pp = ((3, 3), (2, 2), (0, 1, 0, 1)) if cfg == "maxpool" else ((2, 2), (2, 2), (0, 0, 0, 0))
+        d = capi.PoolDesc()
+        d.dtype, d.acc_dtype = capi.INT8, capi.INT32
+        d.N, d.IH, d.IW, d.C, d.OH, d.OW = 32, 112, 112, 64, 56, 56
+        d.kernel[:], d.stride[:], d.pad[:], d.nan_mode = list(pk), list(ps), list(pp), 1
+        tx = to_dev(x)
+        out = torch.empty((32, 56, 56, 64), dtype=torch.int8, device=dev)
+        if cfg == "maxpool":
+            step = lambda: ctx.max_pool2d(d, tx, out)
+            cpu_ref = lambda: oracle.max_pool2d(x[:4], pk, ps, pp)
+        else:
+            step = lambda: ctx.avg_pool2d(d, tx, -3, 4, out)
+            cpu_ref = lambda: oracle.avg_pool2d(x[:4], pk, ps, pp, -3, 4)
+        W = dict(ops=out.numel() * pk[0] * pk[1], bytes=x.nbytes + out.numel(), exact=True, cpu_ref=cpu_ref,
+                 cpu_fraction=1 / 8, result=lambda: out[:4].cpu().numpy(), dtype="int8" if cfg == "maxpool" else "int32",
+                 metric="int8 %s GB/s; %% HBM peak; bit-exact" % ("MAX_POOL2D" if cfg == "maxpool" else "AVG_POOL2D"),
+                 unit="GB/s", bound="hbm", peak=PEAK["hbm"], runit="GB/s",
+                 workload="%s int8 [32,112,112,64] -> [32,56,56,64], kernel %s stride %s pad %s%s"
+                          % ("MAX_POOL2D" if cfg == "maxpool" else "AVG_POOL2D", list(pk), list(ps), list(pp),
+                             "" if cfg == "maxpool" else ", input_zp -3, output_zp 4"))
     elif cfg in ("tconv", "conv3d"):
         # the two neighbouring operators, at shapes of the same family as the named CONV2D configuration (no
         # configuration of theirs is named): the timed step includes the operand re-layout kernels

@@ -158,6 +158,20 @@ typedef struct
     int32_t bias_len;
 } tmi_conv3d_desc_t;
 
+/* AvgPool2dAttribute / MaxPool2dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:29-117
+ * check_pool2d_attribute, :472-537, :1508-1543).  input [N,IH,IW,C], output [N,OH,OW,C] of the same type. */
+typedef struct
+{
+    int32_t dtype;       /* TMI_INT8 / TMI_INT16 / TMI_FP16 / TMI_BF16 / TMI_FP32 */
+    int32_t acc_dtype;   /* AVG_POOL2D: TMI_INT32 for integers, TMI_FP32 for floating point; ignored by MAX_POOL2D */
+    int32_t N, IH, IW, C;
+    int32_t OH, OW;
+    int32_t kernel[2];   /* y, x */
+    int32_t stride[2];   /* y, x */
+    int32_t pad[4];      /* top, bottom, left, right; each < kernel size */
+    int32_t nan_mode;    /* MAX_POOL2D on floating point: 1 = PROPAGATE, 2 = IGNORE */
+} tmi_pool_desc_t;
+
 /* RescaleAttribute plus the operand facts OpRescale::checkTensorAttributes / eval read
  * (reference_model/src/ops/type_conversion.cpp:111-151, 226-255). */
 typedef struct
@@ -230,6 +244,16 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
 int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
+/* OpAvgPool2d<Dtype,AccDtype>::eval, reference_model/src/ops/tensor_ops.cpp:542-660: the sum over the taps
+ * inside the image, divided by their number (integers: reciprocal_scale + apply_scale_32 with a single rounding,
+ * quant_util.h:32-84, then output_zp and the clip to the type).  Zero points must be 0 unless dtype is INT8. */
+int tmi_avg_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev, int32_t in_zp, int32_t out_zp,
+                   void* out_dev);
+
+/* OpMaxPool2d<Dtype>::eval, reference_model/src/ops/tensor_ops.cpp:1546-1640 (applyMax with the attribute's NaN
+ * mode, reference_model/src/arith_util.h:341-373). */
+int tmi_max_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev, void* out_dev);
+
 /* ---- validation only (no launch) ---------------------------------------------------------------- */
 
 /* The checks OpConv2d / OpDepthwiseConv2d::checkTensorAttributes and the head of eval() perform
@@ -244,6 +268,10 @@ int tmi_conv2d_check(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, int32_t depthwise
  * checkTensorAttributes(). */
 int tmi_transpose_conv2d_check(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d);
 int tmi_conv3d_check(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d);
+
+/* check_pool2d_attribute and the type rules of OpAvgPool2d / OpMaxPool2d::checkTensorAttributes
+ * (reference_model/src/ops/tensor_ops.cpp:29-117, 484-537, 1514-1543); avg != 0 selects AVG_POOL2D. */
+int tmi_pool2d_check(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, int32_t avg);
 
 /* OpRescale::checkTensorAttributes and the zero-point rules at the head of eval()
  * (reference_model/src/ops/type_conversion.cpp:72-154, 242-255). */

@@ -325,3 +325,66 @@ def clamp(inp, lo, hi, nan_mode=1):
                              ctypes.c_int(nan_mode), _ptr(out))
     _check(rc)
     return out.astype(inp.dtype)
+
+
+class PoolShape(ctypes.Structure):
+    _fields_ = [
+        ("N", ctypes.c_int32), ("IH", ctypes.c_int32), ("IW", ctypes.c_int32), ("C", ctypes.c_int32),
+        ("OH", ctypes.c_int32), ("OW", ctypes.c_int32),
+        ("kernel", ctypes.c_int32 * 2), ("stride", ctypes.c_int32 * 2), ("pad", ctypes.c_int32 * 4),
+    ]
+
+
+def pool_out_hw(ih, iw, kernel, stride, pad):
+    """Output size the attribute check accepts (tensor_ops.cpp:100-113), or None when there is none."""
+    fh, fw = ih + pad[0] + pad[1] - kernel[0], iw + pad[2] + pad[3] - kernel[1]
+    if fh < 0 or fw < 0 or fh % stride[0] or fw % stride[1]:
+        return None
+    return fh // stride[0] + 1, fw // stride[1] + 1
+
+
+def _pool_shape(inp, kernel, stride, pad, out_hw):
+    n, ih, iw, c = inp.shape
+    if out_hw is None:
+        out_hw = pool_out_hw(ih, iw, kernel, stride, pad) or (0, 0)
+    return PoolShape(n, ih, iw, c, out_hw[0], out_hw[1], (ctypes.c_int32 * 2)(*kernel), (ctypes.c_int32 * 2)(*stride),
+                     (ctypes.c_int32 * 4)(*pad))
+
+
+def reciprocal_scale(count):
+    m, s = ctypes.c_int32(), ctypes.c_int32()
+    lib().orc_reciprocal_scale(ctypes.c_int32(count), ctypes.byref(m), ctypes.byref(s))
+    return m.value, s.value
+
+
+def avg_pool2d(inp, kernel, stride=(1, 1), pad=(0, 0, 0, 0), in_zp=0, out_zp=0, out_hw=None):
+    """AVG_POOL2D.  int8 / int16 input: int32 accumulator, result of the input type.  float32 input (holding
+    fp16 / bf16 / fp32 values): fp32 accumulator, fp32 result for the caller to narrow."""
+    inp = np.asarray(inp)
+    s = _pool_shape(inp, kernel, stride, pad, out_hw)
+    shape = (s.N, max(s.OH, 0), max(s.OW, 0), s.C)
+    if inp.dtype.kind == "i":
+        info = np.iinfo(inp.dtype)
+        x, out = _c(inp, np.int32), np.zeros(shape, np.int32)
+        rc = lib().orc_avg_pool2d_i32(ctypes.byref(s), _ptr(x), ctypes.c_int32(in_zp), ctypes.c_int32(out_zp),
+                                      ctypes.c_int32(int(info.min)), ctypes.c_int32(int(info.max)), _ptr(out))
+        _check(rc)
+        return out.astype(inp.dtype)
+    x, out = _c(inp, np.float32), np.zeros(shape, np.float32)
+    _check(lib().orc_avg_pool2d_f32(ctypes.byref(s), _ptr(x), _ptr(out)))
+    return out
+
+
+def max_pool2d(inp, kernel, stride=(1, 1), pad=(0, 0, 0, 0), nan_mode=1, out_hw=None):
+    """MAX_POOL2D on int8 / int16 (padding = lowest value of the type) or float32 storage (nan_mode 1 = PROPAGATE,
+    2 = IGNORE)."""
+    inp = np.asarray(inp)
+    s = _pool_shape(inp, kernel, stride, pad, out_hw)
+    shape = (s.N, max(s.OH, 0), max(s.OW, 0), s.C)
+    if inp.dtype.kind == "i":
+        x, out = _c(inp, np.int32), np.zeros(shape, np.int32)
+        _check(lib().orc_max_pool2d_i32(ctypes.byref(s), _ptr(x), ctypes.c_int32(int(np.iinfo(inp.dtype).min)), _ptr(out)))
+        return out.astype(inp.dtype)
+    x, out = _c(inp, np.float32), np.zeros(shape, np.float32)
+    _check(lib().orc_max_pool2d_f32(ctypes.byref(s), _ptr(x), ctypes.c_int(nan_mode), _ptr(out)))
+    return out

@@ -688,6 +688,173 @@ int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int3
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * AVG_POOL2D / MAX_POOL2D.  check_pool2d_attribute (reference_model/src/ops/tensor_ops.cpp:29-117).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_pool_check(const orc_pool_shape_t* s)
+{
+    for (int i = 0; i < 4; i++)
+        if (s->pad[i] < 0)
+            return ORC_ERROR;
+    if (s->kernel[0] < 1 || s->kernel[1] < 1 || s->stride[0] < 1 || s->stride[1] < 1)
+        return ORC_ERROR;
+    if (s->pad[0] >= s->kernel[0] || s->pad[1] >= s->kernel[0] || s->pad[2] >= s->kernel[1] ||
+        s->pad[3] >= s->kernel[1])
+        return ORC_ERROR;
+    const int32_t full_h = s->IH + s->pad[0] + s->pad[1] - s->kernel[0];
+    const int32_t full_w = s->IW + s->pad[2] + s->pad[3] - s->kernel[1];
+    if (full_h % s->stride[0] != 0 || full_w % s->stride[1] != 0)
+        return ORC_ERROR;
+    if (s->OH != full_h / s->stride[0] + 1 || s->OW != full_w / s->stride[1] + 1)
+        return ORC_ERROR;
+    return ORC_VALID;
+}
+
+/* reference_model/src/quant_util.h:32-43 */
+void orc_reciprocal_scale(int32_t count, int32_t* multiplier, int32_t* shift)
+{
+    const uint32_t v = (uint32_t)count - 1u;
+    int32_t lz       = 32;
+    for (int b = 31; b >= 0; b--)
+        if (v >> b)
+        {
+            lz = 31 - b;
+            break;
+        }
+    const int32_t k         = 32 - lz; /* (1<<k)/2 < count <= (1<<k) */
+    const int64_t numerator = ((INT64_C(1) << 30) + 1) << k;
+    *multiplier             = (int32_t)(numerator / count);
+    *shift                  = 30 + k;
+}
+
+/* OpAvgPool2d::eval, integer branch (tensor_ops.cpp:603-650): sum of (in - in_zp) over the taps inside the
+ * image, scaled by the reciprocal of their count with a single rounding, plus out_zp, clipped. */
+int orc_avg_pool2d_i32(const orc_pool_shape_t* s, const int32_t* in, int32_t in_zp, int32_t out_zp, int32_t qmin,
+                       int32_t qmax, int32_t* out)
+{
+    if (orc_pool_check(s) != ORC_VALID)
+        return ORC_ERROR;
+    int status = ORC_VALID;
+    for (int32_t n = 0; n < s->N; n++)
+        for (int32_t oh = 0; oh < s->OH; oh++)
+            for (int32_t ow = 0; ow < s->OW; ow++)
+                for (int32_t c = 0; c < s->C; c++)
+                {
+                    int32_t acc = 0, count = 0;
+                    const int32_t iy = oh * s->stride[0] - s->pad[0];
+                    const int32_t ix = ow * s->stride[1] - s->pad[2];
+                    for (int32_t ky = 0; ky < s->kernel[0]; ky++)
+                        for (int32_t kx = 0; kx < s->kernel[1]; kx++)
+                        {
+                            const int32_t y = iy + ky, x = ix + kx;
+                            if (y >= 0 && y < s->IH && x >= 0 && x < s->IW)
+                            {
+                                acc += in[(((int64_t)n * s->IH + y) * s->IW + x) * s->C + c] - in_zp;
+                                count++;
+                            }
+                        }
+                    int32_t m, sh;
+                    int st = ORC_VALID;
+                    orc_reciprocal_scale(count, &m, &sh);
+                    int32_t v = orc_apply_scale_32(acc, m, sh, 0, &st) + out_zp;
+                    if (st != ORC_VALID)
+                        status = ORC_UNPREDICTABLE;
+                    v = v > qmin ? v : qmin;
+                    v = v < qmax ? v : qmax;
+                    out[(((int64_t)n * s->OH + oh) * s->OW + ow) * s->C + c] = v;
+                }
+    return status;
+}
+
+/* floating-point branch (tensor_ops.cpp:652-657): fp32 accumulator, taps in (ky, kx) order, one division */
+int orc_avg_pool2d_f32(const orc_pool_shape_t* s, const float* in, float* out)
+{
+    if (orc_pool_check(s) != ORC_VALID)
+        return ORC_ERROR;
+    for (int32_t n = 0; n < s->N; n++)
+        for (int32_t oh = 0; oh < s->OH; oh++)
+            for (int32_t ow = 0; ow < s->OW; ow++)
+                for (int32_t c = 0; c < s->C; c++)
+                {
+                    volatile float acc = 0.0f; /* one rounding per addition, no contraction */
+                    int32_t count      = 0;
+                    const int32_t iy   = oh * s->stride[0] - s->pad[0];
+                    const int32_t ix   = ow * s->stride[1] - s->pad[2];
+                    for (int32_t ky = 0; ky < s->kernel[0]; ky++)
+                        for (int32_t kx = 0; kx < s->kernel[1]; kx++)
+                        {
+                            const int32_t y = iy + ky, x = ix + kx;
+                            if (y >= 0 && y < s->IH && x >= 0 && x < s->IW)
+                            {
+                                acc = acc + in[(((int64_t)n * s->IH + y) * s->IW + x) * s->C + c];
+                                count++;
+                            }
+                        }
+                    out[(((int64_t)n * s->OH + oh) * s->OW + ow) * s->C + c] = acc / (float)count;
+                }
+    return ORC_VALID;
+}
+
+/* OpMaxPool2d::eval (tensor_ops.cpp:1546-1640): padding is the lowest value of the type */
+int orc_max_pool2d_i32(const orc_pool_shape_t* s, const int32_t* in, int32_t lowest, int32_t* out)
+{
+    if (orc_pool_check(s) != ORC_VALID)
+        return ORC_ERROR;
+    for (int32_t n = 0; n < s->N; n++)
+        for (int32_t oh = 0; oh < s->OH; oh++)
+            for (int32_t ow = 0; ow < s->OW; ow++)
+                for (int32_t c = 0; c < s->C; c++)
+                {
+                    int32_t best     = lowest;
+                    const int32_t iy = oh * s->stride[0] - s->pad[0];
+                    const int32_t ix = ow * s->stride[1] - s->pad[2];
+                    for (int32_t ky = 0; ky < s->kernel[0]; ky++)
+                        for (int32_t kx = 0; kx < s->kernel[1]; kx++)
+                        {
+                            const int32_t y = iy + ky, x = ix + kx;
+                            if (y >= 0 && y < s->IH && x >= 0 && x < s->IW)
+                            {
+                                const int32_t v = in[(((int64_t)n * s->IH + y) * s->IW + x) * s->C + c];
+                                best            = best >= v ? best : v;
+                            }
+                        }
+                    out[(((int64_t)n * s->OH + oh) * s->OW + ow) * s->C + c] = best;
+                }
+    return ORC_VALID;
+}
+
+/* floating point: applyMax / compareNan (reference_model/src/arith_util.h:341-373); the padding value is
+ * -infinity in PROPAGATE mode (low_extreme, reference_model/src/dtype_limits.h:53) and NaN in IGNORE mode
+ * (arith_util.h:423-432), i.e. padding never changes the result. */
+int orc_max_pool2d_f32(const orc_pool_shape_t* s, const float* in, int nan_mode, float* out)
+{
+    if (orc_pool_check(s) != ORC_VALID || (nan_mode != 1 && nan_mode != 2))
+        return ORC_ERROR;
+    for (int32_t n = 0; n < s->N; n++)
+        for (int32_t oh = 0; oh < s->OH; oh++)
+            for (int32_t ow = 0; ow < s->OW; ow++)
+                for (int32_t c = 0; c < s->C; c++)
+                {
+                    float best       = nan_mode == 2 ? NAN : -INFINITY;
+                    const int32_t iy = oh * s->stride[0] - s->pad[0];
+                    const int32_t ix = ow * s->stride[1] - s->pad[2];
+                    for (int32_t ky = 0; ky < s->kernel[0]; ky++)
+                        for (int32_t kx = 0; kx < s->kernel[1]; kx++)
+                        {
+                            const int32_t y = iy + ky, x = ix + kx;
+                            if (y < 0 || y >= s->IH || x < 0 || x >= s->IW)
+                                continue;
+                            const float v = in[(((int64_t)n * s->IH + y) * s->IW + x) * s->C + c];
+                            if (isnan(best) || isnan(v))
+                                best = nan_mode == 1 ? NAN : (isnan(best) ? v : best);
+                            else
+                                best = best >= v ? best : v;
+                        }
+                    out[(((int64_t)n * s->OH + oh) * s->OW + ow) * s->C + c] = best;
+                }
+    return ORC_VALID;
+}
+
+/* ------------------------------------------------------------------------------------------------
  * OpClamp (reference_model/src/ops/activation_funcs.cpp:27-125) through applyClip
  * (reference_model/src/arith_util.h:389-413).
  * ---------------------------------------------------------------------------------------------- */

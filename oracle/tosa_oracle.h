@@ -1,6 +1,6 @@
 /*
  * CPU oracle for the TOSA tensor-op hot path (CONV2D, DEPTHWISE_CONV2D, MATMUL, RESCALE, CLAMP) and its
- * neighbours CONV3D and TRANSPOSE_CONV2D.
+ * neighbours CONV3D, TRANSPOSE_CONV2D, AVG_POOL2D and MAX_POOL2D.
  *
  * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the arithmetic of the TOSA reference
  * model, used as the checker in the parity tests, in the smoke test and as the timed CPU baseline.
@@ -19,6 +19,11 @@
  *   - conv3d / transpose_conv2d: the literal vectors of tensor_ops_tests.cpp:268-446,622-766 (zero points,
  *     bias broadcast) and an independent numpy restatement (correlation of the zero-upsampled input with the
  *     flipped kernel for TRANSPOSE_CONV2D; per-depth-tap sums of 2-D convolutions for CONV3D).
+ *   - avg_pool2d / max_pool2d: the two literal cases of tensor_ops_tests.cpp:508-575,800-823 (zero point
+ *     subtracted in full precision), reciprocal_scale against exact rational arithmetic for every count up to
+ *     4096 (multiplier = floor(((2^30+1) << k) / count)), and an independent numpy restatement over padded
+ *     windows for general shapes.  Floating-point AVG_POOL2D sums in tap order in fp32 like the reference's
+ *     loop nest (tensor_ops.cpp:613-634), so it is compared bit for bit.
  *   - large shapes: independent numpy int64 einsum / float64 convolution.
  *   - fp accumulate order of MATMUL (Eigen contraction order): parity unpinned (tolerance covered).
  */
@@ -162,6 +167,28 @@ int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int3
                 const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out);
 
 /* CLAMP for the integer instantiations: min(max(x, lo), hi); ORC_ERROR when hi < lo. */
+/* AVG_POOL2D / MAX_POOL2D (reference_model/src/ops/tensor_ops.cpp:29-117 check_pool2d_attribute, :472-660
+ * OpAvgPool2d, :1508-1640 OpMaxPool2d).  Input and output NHWC with the same N and C. */
+typedef struct
+{
+    int32_t N, IH, IW, C;
+    int32_t OH, OW;
+    int32_t kernel[2]; /* y, x */
+    int32_t stride[2]; /* y, x */
+    int32_t pad[4];    /* top, bottom, left, right */
+} orc_pool_shape_t;
+int orc_pool_check(const orc_pool_shape_t* s);
+/* QuantUtil::reciprocal_scale (reference_model/src/quant_util.h:32-43) */
+void orc_reciprocal_scale(int32_t count, int32_t* multiplier, int32_t* shift);
+/* integer AVG_POOL2D: values widened to int32 by the caller, qmin/qmax = limits of the in/out type */
+int orc_avg_pool2d_i32(const orc_pool_shape_t* s, const int32_t* in, int32_t in_zp, int32_t out_zp, int32_t qmin,
+                       int32_t qmax, int32_t* out);
+/* floating-point AVG_POOL2D with an fp32 accumulator; the caller narrows the result to the output type */
+int orc_avg_pool2d_f32(const orc_pool_shape_t* s, const float* in, float* out);
+int orc_max_pool2d_i32(const orc_pool_shape_t* s, const int32_t* in, int32_t lowest, int32_t* out);
+/* nan_mode: 1 = PROPAGATE, 2 = IGNORE */
+int orc_max_pool2d_f32(const orc_pool_shape_t* s, const float* in, int nan_mode, float* out);
+
 int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out);
 /* CLAMP for float storage; nan_mode 1 = PROPAGATE, 2 = IGNORE. */
 int orc_clamp_f32(int64_t n, const float* in, float lo, float hi, int nan_mode, float* out);

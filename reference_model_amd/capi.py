@@ -31,6 +31,7 @@ EXPORTS = [
     "tmi_conv2d", "tmi_depthwise_conv2d", "tmi_matmul", "tmi_rescale", "tmi_clamp", "tmi_conv2d_rescale_clamp",
     "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice", "tmi_conv2d_check", "tmi_rescale_check",
     "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
+    "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
 ]
 
 
@@ -56,6 +57,12 @@ class Conv3dDesc(ctypes.Structure):
                                               "KW", "OD", "OH", "OW")] + [
         ("pad", ctypes.c_int32 * 6), ("stride", ctypes.c_int32 * 3), ("dilation", ctypes.c_int32 * 3),
         ("bias_len", ctypes.c_int32)]
+
+
+class PoolDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("dtype", "acc_dtype", "N", "IH", "IW", "C", "OH", "OW")] + [
+        ("kernel", ctypes.c_int32 * 2), ("stride", ctypes.c_int32 * 2), ("pad", ctypes.c_int32 * 4),
+        ("nan_mode", ctypes.c_int32)]
 
 
 class RescaleDesc(ctypes.Structure):
@@ -110,6 +117,9 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_matmul.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, i32, vp]
     lib.tmi_rescale.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i64, i32, vp, vp, vp, vp]
     lib.tmi_clamp.argtypes = [vp, i32, i64, vp, i32, i32, vp]
+    lib.tmi_avg_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, i32, i32, vp]
+    lib.tmi_max_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, vp]
+    lib.tmi_pool2d_check.argtypes = [vp, ctypes.POINTER(PoolDesc), i32]
     lib.tmi_conv2d_check.argtypes = [vp, ctypes.POINTER(ConvDesc), i32]
     lib.tmi_rescale_check.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i32]
     for name in EXPORTS:
@@ -260,6 +270,12 @@ class Context:
     def transpose_conv2d(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_transpose_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
                                                          _ptr(bias), in_zp, w_zp, _ptr(out)))
+
+    def avg_pool2d(self, d: PoolDesc, inp, in_zp, out_zp, out) -> int:
+        return self._check(self.lib.tmi_avg_pool2d(self.handle, ctypes.byref(d), _ptr(inp), in_zp, out_zp, _ptr(out)))
+
+    def max_pool2d(self, d: PoolDesc, inp, out) -> int:
+        return self._check(self.lib.tmi_max_pool2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(out)))
 
     def conv3d(self, d: Conv3dDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_conv3d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias),

@@ -7,6 +7,8 @@
 //   TosaOperator    0 op(uint32), 1 attribute_type(ubyte), 2 attribute(table), 3 inputs[str], 4 outputs[str]
 //   Conv2dAttribute / DepthwiseConv2dAttribute / Conv3dAttribute  0 pad, 1 stride, 2 dilation, 3 local_bound, 4 acc_type
 //   TransposeConv2dAttribute  0 out_pad, 1 stride, 2 local_bound, 3 acc_type
+//   AvgPool2dAttribute        0 kernel, 1 stride, 2 pad, 3 acc_type
+//   MaxPool2dAttribute        0 kernel, 1 stride, 2 pad, 3 nan_mode
 //   RescaleAttribute  0 scale32, 1 rounding_mode, 2 per_channel, 3 input_unsigned, 4 output_unsigned
 //   ClampAttribute    0 min_val[ubyte], 1 max_val[ubyte], 2 nan_mode
 #include <cstdio>
@@ -47,6 +49,10 @@ const char* op_name(uint32_t op)
             return "CONV3D";
         case Op_TRANSPOSE_CONV2D:
             return "TRANSPOSE_CONV2D";
+        case Op_AVG_POOL2D:
+            return "AVG_POOL2D";
+        case Op_MAX_POOL2D:
+            return "MAX_POOL2D";
         case Op_DEPTHWISE_CONV2D:
             return "DEPTHWISE_CONV2D";
         case Op_MATMUL:
@@ -246,6 +252,17 @@ bool load_tosa_file(const std::string& path, BasicBlock& block, std::string& err
                     d.attr.stride      = a.vec<int32_t>(1);
                     d.attr.local_bound = a.scalar<uint8_t>(2, 0) != 0;
                     d.attr.acc_type    = a.scalar<uint32_t>(3, 0);
+                    break;
+                case Op_AVG_POOL2D:    // kernel, stride, pad, acc_type / nan_mode: the order of the reference's
+                case Op_MAX_POOL2D:    // TosaAvgPool2dAttribute constructor (tensor_ops_tests.cpp:539-540); no
+                                       // example graph confirms it
+                    d.attr.kernel = a.vec<int32_t>(0);
+                    d.attr.stride = a.vec<int32_t>(1);
+                    d.attr.pad    = a.vec<int32_t>(2);
+                    if (d.op == Op_AVG_POOL2D)
+                        d.attr.acc_type = a.scalar<uint32_t>(3, 0);
+                    else
+                        d.attr.nan_mode = a.scalar<uint32_t>(3, 0);
                     break;
                 case Op_CONV2D:
                 case Op_CONV3D:

@@ -458,6 +458,78 @@ public:
     }
 };
 
+// AVG_POOL2D: operands [input, input_zp, output_zp] (tensor_ops.cpp:476); MAX_POOL2D: [input] (:1497).
+class OpPool2d : public GraphNode
+{
+public:
+    OpPool2d(SubgraphTraverser* sgt, Op op, uint64_t id) : GraphNode(sgt, op, id), avg(op == Op_AVG_POOL2D)
+    {
+        requiredInputCount  = avg ? 3 : 1;
+        requiredOutputCount = 1;
+    }
+    const bool avg;
+    int fill_desc(tmi_pool_desc_t& d)
+    {
+        const Tensor *in = inputs[0], *out = outputs[0];
+        if (attribute.pad.size() != 4)
+            return error("illegal size for attribute padding");
+        if (attribute.kernel.size() != 2)
+            return error("illegal size for attribute kernel");
+        if (attribute.stride.size() != 2)
+            return error("illegal size for attribute stride");
+        memset(&d, 0, sizeof(d));
+        d.dtype     = tmi_dtype(in->getDtype());
+        d.acc_dtype = tmi_dtype((DType)attribute.acc_type);
+        d.N = in->shape[0], d.IH = in->shape[1], d.IW = in->shape[2], d.C = in->shape[3];
+        if (out->shape[0] != d.N)
+            return error("tensor batch mismatch %d != %d", d.N, out->shape[0]);
+        if (out->shape[3] != d.C)
+            return error("tensor channel mismatch %d != %d", d.C, out->shape[3]);
+        d.OH = out->shape[1], d.OW = out->shape[2];
+        for (int i = 0; i < 2; i++)
+            d.kernel[i] = attribute.kernel[i], d.stride[i] = attribute.stride[i];
+        for (int i = 0; i < 4; i++)
+            d.pad[i] = attribute.pad[i];
+        d.nan_mode = attribute.nan_mode ? (int32_t)attribute.nan_mode : 1;    // unset = PROPAGATE
+        return 0;
+    }
+    int checkTensorAttributes() override
+    {
+        if (validateRequiredOperands())
+            return 1;
+        if (validateRequiredRank(inputs[0], 4, 4) || validateRequiredRank(outputs[0], 4, 4))
+            return 1;
+        if (avg && (validateRequiredRank(inputs[1], 1, 1) || validateRequiredRank(inputs[2], 1, 1)))
+            return error("input and output zero point must be rank 1");
+        if (inputs[0]->getDtype() != outputs[0]->getDtype())
+            return error("input and output tensor type mismatch");
+        tmi_pool_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        if (tmi_pool2d_check(parent_sgt->ctx, &d, avg ? 1 : 0) != TMI_VALID)
+            return error("%s", tmi_last_error(parent_sgt->ctx));
+        return 0;
+    }
+    int eval() override
+    {
+        tmi_pool_desc_t d;
+        if (fill_desc(d))
+            return 1;
+        SubgraphTraverser* s = parent_sgt;
+        if (avg)
+        {
+            int32_t in_zp = 0, out_zp = 0;
+            if (!inputs[1]->scalar_value(in_zp) || !inputs[2]->scalar_value(out_zp))
+                return error("zero-point operands must be available on the host");
+            if (call(tmi_avg_pool2d(s->ctx, &d, s->device(inputs[0]), in_zp, out_zp, s->device_out(outputs[0]))))
+                return 1;
+        }
+        else if (call(tmi_max_pool2d(s->ctx, &d, s->device(inputs[0]), s->device_out(outputs[0]))))
+            return 1;
+        return GraphNode::eval();
+    }
+};
+
 class OpConv3d : public GraphNode
 {
 public:
@@ -665,6 +737,10 @@ int SubgraphTraverser::initializeGraph()
             case Op_DEPTHWISE_CONV2D:
                 n = new OpDepthwiseConv2d(this, id);
                 break;
+            case Op_AVG_POOL2D:
+            case Op_MAX_POOL2D:
+                n = new OpPool2d(this, (Op)o.op, id);
+                break;
             case Op_TRANSPOSE_CONV2D:
                 n = new OpTransposeConv2d(this, id);
                 break;
@@ -682,7 +758,7 @@ int SubgraphTraverser::initializeGraph()
                 break;
             default:
                 last_message = "operator " + std::to_string(o.op) + " is outside the accelerated path "
-                               "(CONV2D, CONV3D, DEPTHWISE_CONV2D, TRANSPOSE_CONV2D, MATMUL, RESCALE, CLAMP)";
+                               "(CONV2D, CONV3D, DEPTHWISE_CONV2D, TRANSPOSE_CONV2D, MATMUL, RESCALE, CLAMP, AVG_POOL2D, MAX_POOL2D)";
                 setGraphStatus(GraphStatus::TOSA_ERROR);
                 return 1;
         }

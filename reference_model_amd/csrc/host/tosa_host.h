@@ -34,10 +34,12 @@ enum class GraphStatus : int
 // and FP32 are confirmed by the reference's example graphs).
 enum Op : uint32_t
 {
+    Op_AVG_POOL2D       = 2,
     Op_CONV2D           = 3,
     Op_CONV3D           = 4,
     Op_DEPTHWISE_CONV2D = 5,
     Op_MATMUL           = 7,
+    Op_MAX_POOL2D       = 8,
     Op_TRANSPOSE_CONV2D = 10,
     Op_CLAMP            = 11,
     Op_RESCALE          = 66,
@@ -67,6 +69,8 @@ struct Attribute
 {
     // Conv2dAttribute / DepthwiseConv2dAttribute / Conv3dAttribute; TransposeConv2dAttribute keeps out_pad in pad
     std::vector<int32_t> pad, stride, dilation;
+    // AvgPool2dAttribute / MaxPool2dAttribute: kernel (+ stride, pad above; acc_type or nan_mode below)
+    std::vector<int32_t> kernel;
     bool local_bound  = false;
     uint32_t acc_type = 0;
     // RescaleAttribute

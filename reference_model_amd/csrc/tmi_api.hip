@@ -827,6 +827,93 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
     return after_launch(ctx, name);
 }
 
+// check_pool2d_attribute (tensor_ops.cpp:29-117) with the reference's messages, plus the type rules.
+static int validate_pool(tmi_ctx* ctx, const char* op, const tmi_pool_desc_t* d, bool avg, int32_t in_zp,
+                         int32_t out_zp)
+{
+    if (!d)
+        return fail(ctx, "%s: null descriptor", op);
+    const bool is_int = d->dtype == TMI_INT8 || d->dtype == TMI_INT16;
+    const bool is_fp  = d->dtype == TMI_FP16 || d->dtype == TMI_BF16 || d->dtype == TMI_FP32;
+    if (!is_int && !is_fp)
+        return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
+    if (avg && d->acc_dtype != (is_int ? TMI_INT32 : TMI_FP32))
+        return fail(ctx, "%s: accumulator type not supported for this configuration of operator", op);
+    if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->C < 0)
+        return fail(ctx, "%s: negative tensor dimension", op);
+    for (int i = 0; i < 4; i++)
+        if (d->pad[i] < 0)
+            return fail(ctx, "%s: At least one pad is smaller than zero", op);
+    for (int i = 0; i < 2; i++)
+        if (d->kernel[i] < 1)
+            return fail(ctx, "%s: At least one kernel dimension is smaller than one", op);
+    for (int i = 0; i < 2; i++)
+        if (d->stride[i] < 1)
+            return fail(ctx, "%s: At least one stride dimension is smaller than one", op);
+    if (d->pad[0] >= d->kernel[0] || d->pad[1] >= d->kernel[0] || d->pad[2] >= d->kernel[1] ||
+        d->pad[3] >= d->kernel[1])
+        return fail(ctx, "%s: At least one pad is >= kernel dimension", op);
+    const int32_t full_h = d->IH + d->pad[0] + d->pad[1] - d->kernel[0];
+    const int32_t full_w = d->IW + d->pad[2] + d->pad[3] - d->kernel[1];
+    if (full_h % d->stride[0] != 0 || full_w % d->stride[1] != 0)
+        return fail(ctx, "%s: Parameters must yield exact integer output dimensions", op);
+    if (d->OH != full_h / d->stride[0] + 1 || d->OW != full_w / d->stride[1] + 1)
+        return fail(ctx, "%s: Mismatch between output shape provided and expected output shape (%d,%d)", op,
+                    full_h / d->stride[0] + 1, full_w / d->stride[1] + 1);
+    if (avg && d->dtype != TMI_INT8 && in_zp != 0)
+        return fail(ctx, "%s: Input zeropoint must be zero for non int8_t data", op);
+    if (avg && d->dtype != TMI_INT8 && out_zp != 0)
+        return fail(ctx, "%s: Output zeropoint must be zero for non int8_t data", op);
+    if (!avg && is_fp && d->nan_mode != 1 && d->nan_mode != 2)
+        return fail(ctx, "%s: invalid NaN propagation mode", op);
+    return TMI_VALID;
+}
+
+int tmi_pool2d_check(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, int32_t avg)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return validate_pool(ctx, avg ? "OpAvgPool2d" : "OpMaxPool2d", d, avg != 0, 0, 0);
+}
+
+static int run_pool(tmi_ctx* ctx, const char* op, bool avg, const tmi_pool_desc_t* d, const void* in_dev, int32_t in_zp,
+                    int32_t out_zp, void* out_dev)
+{
+    int rc = validate_pool(ctx, op, d, avg, in_zp, out_zp);
+    if (rc != TMI_VALID)
+        return rc;
+    const int64_t total = (int64_t)d->N * d->OH * d->OW * d->C;
+    if (total > 0 && (!in_dev || !out_dev))
+        return fail(ctx, "%s: null tensor pointer", op);
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    const char* name = launch_pool(ctx->stream, avg, d->dtype, d->N, d->IH, d->IW, d->C, d->OH, d->OW, d->kernel[0],
+                                   d->kernel[1], d->stride[0], d->stride[1], d->pad[0], d->pad[2], in_zp, out_zp,
+                                   d->nan_mode, in_dev, out_dev, ctx->flags_dev);
+    if (!name)
+        return fail(ctx, "%s: tensor too large for the pooling kernel", op);
+    return after_launch(ctx, name);
+}
+
+int tmi_avg_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev, int32_t in_zp, int32_t out_zp,
+                   void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_pool(ctx, "OpAvgPool2d", true, d, in_dev, in_zp, out_zp, out_dev);
+}
+
+int tmi_max_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_pool(ctx, "OpMaxPool2d", false, d, in_dev, 0, 0, out_dev);
+}
+
 int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64_t rows, int32_t C,
                 const void* in_dev, const void* multiplier_dev, const void* shift_dev, void* out_dev)
 {

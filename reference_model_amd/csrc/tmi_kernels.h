@@ -66,6 +66,12 @@ const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_d
 const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                     const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                     const RescaleParams& rp, void* out, uint32_t* flag_word);
+// pool.hip: AVG_POOL2D (avg) / MAX_POOL2D; nullptr for a dtype without a kernel or 2^32 work items or more.
+const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int32_t IH, int32_t IW, int32_t C,
+                        int32_t OH, int32_t OW, int32_t kernel_y, int32_t kernel_x, int32_t stride_y, int32_t stride_x,
+                        int32_t pad_top, int32_t pad_left, int32_t in_zp, int32_t out_zp, int32_t nan_mode,
+                        const void* in, void* out, uint32_t* flag_word);
+
 // gemm_mfma.hip: 1x1 / stride 1 / unpadded CONV2D and MATMUL (w_batch_stride != 0: per-image weights) with
 // operands loaded straight into LDS; nullptr when the operation is not such a GEMM or too small to gain.
 // w_kmajor_stride != 0: the weights are [K][OC] with that many bytes per K row (MATMUL's second operand as it

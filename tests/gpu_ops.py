@@ -159,3 +159,33 @@ def conv3d(ctx, x, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), 
     finally:
         for t in list(ctx._owned):
             ctx._free(t)
+
+
+def pool2d(ctx, x, kernel, stride=(1, 1), pad=(0, 0, 0, 0), avg=True, in_zp=0, out_zp=0, nan_mode=1, dtype=None,
+           out_hw=None, acc_dtype=None):
+    """AVG_POOL2D / MAX_POOL2D through the C ABI; returns (out, status).  bf16 travels as uint16 bit patterns."""
+    np_to_tmi = {np.dtype(np.int8): capi.INT8, np.dtype(np.int16): capi.INT16, np.dtype(np.float16): capi.FP16,
+                 np.dtype(np.float32): capi.FP32}
+    tmi_dtype = dtype or np_to_tmi[x.dtype]
+    n, ih, iw, c = x.shape
+    if out_hw is None:
+        out_hw = oracle.pool_out_hw(ih, iw, kernel, stride, pad) or (0, 0)
+    d = capi.PoolDesc()
+    d.dtype = tmi_dtype
+    d.acc_dtype = acc_dtype if acc_dtype is not None else (capi.INT32 if tmi_dtype in (capi.INT8, capi.INT16) else capi.FP32)
+    d.N, d.IH, d.IW, d.C = n, ih, iw, c
+    d.OH, d.OW = out_hw
+    d.kernel[:], d.stride[:], d.pad[:] = list(kernel), list(stride), list(pad)
+    d.nan_mode = nan_mode
+    tx = ctx.upload(x, tmi_dtype)
+    try:
+        to = ctx.empty((n, max(out_hw[0], 0), max(out_hw[1], 0), c), tmi_dtype, x.dtype)
+        if avg:
+            ctx.avg_pool2d(d, tx, in_zp, out_zp, to)
+        else:
+            ctx.max_pool2d(d, tx, to)
+        st = ctx.sync()
+        return to.numpy(), st
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)

@@ -226,3 +226,42 @@ def test_exit_codes_unpredictable_and_error(tmp_path):
     r = _run(_write_case(d3, W.graph(ts, [W.operator(15, ["x", "x"], ["y"])], ["x"], ["y"]),
                          {"x": np.arange(4, dtype=np.int32)}, ["y"]))
     assert r.returncode == 2 and "outside the accelerated path" in r.stderr
+
+
+@pytest.mark.gpu
+def test_pooling_graph(tmp_path):
+    """CONV2D -> RESCALE -> MAX_POOL2D -> AVG_POOL2D: the int8 tail of a classifier block, loaded from a flatbuffer
+    and run on the device; every intermediate stays there."""
+    rng = np.random.default_rng(21)
+    x = rng.integers(-128, 128, (2, 12, 12, 16)).astype(np.int8)
+    w = rng.integers(-128, 128, (32, 3, 3, 16)).astype(np.int8)
+    bias = rng.integers(-999, 999, 32).astype(np.int32)
+    acc = oracle.conv2d("i8", x, w, bias, (1, 1, 1, 1), (1, 1), (1, 1), in_zp=3, w_zp=0)
+    mult = rng.integers(1 << 30, 1 << 31, 32).astype(np.int32)
+    shift = np.full(32, 41, np.int8)
+    q, st = oracle.rescale(acc, mult, shift, out_zp=-2, out_dtype=np.int8)
+    mp = oracle.max_pool2d(q, (2, 2), (2, 2))
+    ap = oracle.avg_pool2d(mp, (3, 3), (3, 3), in_zp=-2, out_zp=5)
+    assert st == oracle.VALID
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", w.shape, np.int8, w), W.tensor("bias", [32], np.int32, bias),
+          W.tensor("izp", [1], np.int8, [3]), W.tensor("wzp", [1], np.int8, [0]), W.tensor("acc", acc.shape, np.int32),
+          W.tensor("mult", [32], np.int32, mult), W.tensor("shift", [32], np.int8, shift),
+          W.tensor("rizp", [1], np.int32, [0]), W.tensor("rozp", [1], np.int8, [-2]), W.tensor("q", q.shape, np.int8),
+          W.tensor("mp", mp.shape, np.int8), W.tensor("aizp", [1], np.int8, [-2]), W.tensor("aozp", [1], np.int8, [5]),
+          W.tensor("ap", ap.shape, np.int8)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "izp", "wzp", "mult", "shift", "rizp", "rozp", "aizp", "aozp")]
+    ops.append(W.operator(3, ["x", "w", "bias", "izp", "wzp"], ["acc"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1))))
+    ops.append(W.operator(R.OP_RESCALE, ["acc", "mult", "shift", "rizp", "rozp"], ["q"], W.rescale_attr()))
+    ops.append(W.operator(8, ["q"], ["mp"], W.pool_attr((2, 2), (2, 2), (0, 0, 0, 0), 1)))
+    ops.append(W.operator(2, ["mp", "aizp", "aozp"], ["ap"], W.pool_attr((3, 3), (3, 3), (0, 0, 0, 0), 5)))
+    d1 = tmp_path / "pool"
+    d1.mkdir()
+    r = _run(_write_case(d1, W.graph(ts, ops, ["x"], ["ap", "mp"]), {"x": x}, ["ap", "mp"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d1 / "mp_out.npy"), mp) and np.array_equal(np.load(d1 / "ap_out.npy"), ap)
+    # a window that does not tile the input is rejected when the graph is validated
+    ops[-1] = W.operator(2, ["mp", "aizp", "aozp"], ["ap"], W.pool_attr((4, 4), (3, 3), (0, 0, 0, 0), 5))
+    d2 = tmp_path / "bad"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["ap"]), {"x": x}, ["ap"]))
+    assert r.returncode == 2 and "exact integer output dimensions" in r.stderr

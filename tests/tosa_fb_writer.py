@@ -136,6 +136,12 @@ def transpose_conv_attr(out_pad, stride, acc_type=5, local_bound=False):
                   (3, "I", acc_type)])
 
 
+def pool_attr(kernel, stride, pad, last):
+    """AvgPool2dAttribute (last = acc_type) / MaxPool2dAttribute (last = nan_mode)"""
+    return table([(0, None, vector("i", kernel)), (1, None, vector("i", stride)), (2, None, vector("i", pad)),
+                  (3, "I", last)])
+
+
 def rescale_attr(scale32=True, rounding_mode=3, per_channel=True, input_unsigned=False, output_unsigned=False):
     return table([(0, "B", int(scale32)), (1, "I", rounding_mode), (2, "B", int(per_channel)),
                   (3, "B", int(input_unsigned)), (4, "B", int(output_unsigned))])
