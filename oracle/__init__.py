@@ -388,3 +388,22 @@ def max_pool2d(inp, kernel, stride=(1, 1), pad=(0, 0, 0, 0), nan_mode=1, out_hw=
     x, out = _c(inp, np.float32), np.zeros(shape, np.float32)
     _check(lib().orc_max_pool2d_f32(ctypes.byref(s), _ptr(x), ctypes.c_int(nan_mode), _ptr(out)))
     return out
+
+
+_DP_OPS = {"matmul": 0, "conv2d": 1, "depthwise": 2}
+_DP_KINDS = {"fp16": 16, "bf16": 17, "fp32": 32}
+
+
+def dot_product_data(op, data_set, param, ks, shape, kind="fp32", kernel=None, acc16=False):
+    """The DOT_PRODUCT test data set `data_set` (0..5) for operand `param` of `op` ("matmul", "conv2d",
+    "depthwise"), as float32 values; kind selects the bound parameter B of the operand type."""
+    L = lib()
+    L.orc_dp_bound_parameter.restype = ctypes.c_float
+    B = L.orc_dp_bound_parameter(ctypes.c_int(_DP_KINDS[kind]), ctypes.c_int(int(acc16)))
+    out = np.zeros(shape, np.float32)
+    shp = (ctypes.c_int32 * len(shape))(*shape)
+    ker = (ctypes.c_int32 * 2)(*kernel) if kernel is not None else None
+    rc = L.orc_dp_generate(ctypes.c_int(_DP_OPS[op]), ctypes.c_int(data_set), ctypes.c_int(param), ctypes.c_uint32(ks),
+                           ctypes.c_float(B), shp, ctypes.c_int(len(shape)), ker, _ptr(out))
+    _check(rc)
+    return out

@@ -888,3 +888,175 @@ int orc_clamp_f32(int64_t n, const float* in, float lo, float hi, int nan_mode, 
     }
     return ORC_VALID;
 }
+
+/* ------------------------------------------------------------------------------------------------
+ * DOT_PRODUCT test data (TOSA specification tosa_mi_data; reference_model/src/generate/
+ * generate_dot_product_states.cpp).  A primitive generator is the sequence r <- r*m + 1 (mod 2^32) with
+ * m = (8*S + 1) * 0x705A5E75, mapped to (-1, 1) by sign bit and the low 31 bits; each set draws from
+ * generators 3*set + {0, 1, 2}.  The arithmetic types below are the reference's: float unless a double
+ * square root enters the expression.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct
+{
+    uint32_t m, r;
+} dp_prim_t;
+
+static void dp_prim_init(dp_prim_t* g, uint32_t S)
+{
+    g->m = (8u * S + 1u) * 0x705A5E75u;
+    g->r = g->m + 1u;
+}
+
+static float dp_prim_next(dp_prim_t* g)
+{
+    const float sign   = (g->r >> 31) == 0 ? 1.0f : -1.0f;
+    const float pseudo = sign * (float)(g->r & 0x7FFFFFFFu) / (float)0x7FFFFFFF;
+    g->r               = g->r * g->m + 1u;
+    return pseudo;
+}
+
+float orc_dp_bound_parameter(int data_kind, int acc16)
+{
+    switch (data_kind)
+    {
+        case 16: return acc16 ? 255.875f : 65504.0f;    /* (1<<8) - 1/8 ; (1<<16) - (1<<5) */
+        case 17: return 18374686479671623680.0f;        /* (1<<64) - (1<<56) */
+        case 32: return 18446742974197923840.0f;        /* (1<<64) - (1<<40) */
+        default: return 0.0f;
+    }
+}
+
+typedef struct
+{
+    int set, p;
+    uint32_t ks;
+    float B;
+    dp_prim_t g0, g1;
+} dp_gen_t;
+
+static void dp_gen_init(dp_gen_t* g, int set, int p, uint32_t ks, float B)
+{
+    g->set = set, g->p = p, g->ks = ks, g->B = B;
+    if (set == 0 || set == 4)
+    {
+        dp_prim_init(&g->g0, 3u * (uint32_t)set);
+        dp_prim_init(&g->g1, 3u * (uint32_t)set + 1u);
+    }
+    else
+        dp_prim_init(&g->g0, 3u * (uint32_t)set + (uint32_t)p);
+}
+
+static float dp_gen_next(dp_gen_t* g, uint32_t k)
+{
+    const int p = g->p;
+    switch (g->set)
+    {
+        case 0: { /* sums of products with zero give zero */
+            const float s0 = dp_prim_next(&g->g0), s1 = dp_prim_next(&g->g1);
+            if (p == 0)
+                return s0 < 0.0f ? 0.0f : s1;
+            if (p == 1)
+                return s0 < 0.0f ? s1 : 0.0f;
+            return 0.0f;
+        }
+        case 1: { /* large exponents */
+            const float s0 = dp_prim_next(&g->g0), s1 = dp_prim_next(&g->g0);
+            float v        = s0 < 0 ? -0.75f : 0.75f;
+            v += 0.25f * s1;
+            if (p != 2)
+                return (float)(((double)g->B / sqrt((double)(g->ks + 1u))) * (double)v);
+            return (g->B * g->B / (float)(g->ks + 1u)) * v;
+        }
+        case 2: { /* small values of similar magnitude onto a large one */
+            const float s = dp_prim_next(&g->g0);
+            if (p != 2)
+                return k == 0 ? 1.0f : (float)((double)s / sqrt((double)g->ks));
+            return 0.0f;
+        }
+        case 3: { /* small values of varying magnitude onto a large one */
+            const float s0 = dp_prim_next(&g->g0), s1 = dp_prim_next(&g->g0);
+            if (p != 2)
+                return k == 0 ? (s0 < 0 ? -16.0f : 16.0f) : expf(2 * s0) * s1;
+            return 0.0f;
+        }
+        case 4: { /* a mixture of zero and non-zero products */
+            const float s0 = dp_prim_next(&g->g0), s1 = dp_prim_next(&g->g1);
+            const float big = (float)(((double)g->B / sqrt((double)g->ks)) * (double)s1);
+            if (p == 0)
+                return k == g->ks / 2 ? (s0 < 0 ? -0.5f : 0.5f) : (s0 < 0 ? 0.0f : big);
+            if (p == 1)
+                return k == g->ks / 2 ? (s0 < 0 ? 0.5f : -0.5f) : (s0 < 0 ? big : 0.0f);
+            return 0.0f;
+        }
+        default: { /* 5: signed inputs of large range */
+            const float s = dp_prim_next(&g->g0);
+            if (p != 2)
+                return (float)(((double)g->B / sqrt((double)(g->ks + 1u))) * (double)s);
+            return 0.0f;
+        }
+    }
+}
+
+int orc_dp_generate(int op, int set, int param, uint32_t ks, float B, const int32_t* shape, int rank,
+                    const int32_t* kernel, float* out)
+{
+    if (set < 0 || set > 5 || param < 0 || param > 2 || !(B > 0.0f) || ks == 0)
+        return ORC_ERROR;
+    dp_gen_t g;
+    dp_gen_init(&g, set, param, ks, B);
+    uint64_t T = 1;
+    for (int i = 0; i < rank; i++)
+        T *= (uint64_t)shape[i];
+    if (param == 2) /* bias: every element is generator(2) */
+    {
+        if (op == ORC_DP_MATMUL || rank != 1)
+            return ORC_ERROR;
+        for (uint64_t t = 0; t < T; t++)
+            out[t] = dp_gen_next(&g, 2);
+        return ORC_VALID;
+    }
+    if (op == ORC_DP_MATMUL)
+    {
+        if (rank != 3)
+            return ORC_ERROR;
+        const uint32_t C = (uint32_t)(param == 0 ? shape[2] : shape[1]);
+        const uint32_t W = (uint32_t)shape[2];
+        for (uint64_t t = 0; t < T; t++)
+            out[t] = dp_gen_next(&g, param == 0 ? (uint32_t)(t % C) : (uint32_t)((t / W) % C));
+        return ORC_VALID;
+    }
+    if (rank != 4)
+        return ORC_ERROR;
+    if (param == 0)
+    {
+        if (!kernel || kernel[0] <= 0 || kernel[1] <= 0)
+            return ORC_ERROR;
+        const uint32_t IH = (uint32_t)shape[1], IW = (uint32_t)shape[2], IC = (uint32_t)shape[3];
+        const uint32_t KH = (uint32_t)kernel[0], KW = (uint32_t)kernel[1];
+        for (uint64_t t = 0; t < T; t++)
+        {
+            const uint32_t ic = (uint32_t)(t % IC), ix = (uint32_t)((t / IC) % IW), iy = (uint32_t)(((t / IC) / IW) % IH);
+            const uint32_t tap = (iy % KH) * KW + (ix % KW);
+            out[t]             = dp_gen_next(&g, op == ORC_DP_CONV2D ? tap * IC + ic : tap);
+        }
+        return ORC_VALID;
+    }
+    if (op == ORC_DP_CONV2D) /* weight [OC, KH, KW, IC] */
+    {
+        const uint32_t KH = (uint32_t)shape[1], KW = (uint32_t)shape[2], IC = (uint32_t)shape[3];
+        for (uint64_t t = 0; t < T; t++)
+        {
+            const uint32_t ic = (uint32_t)(t % IC), kx = (uint32_t)((t / IC) % KW), ky = (uint32_t)(((t / IC) / KW) % KH);
+            out[t]            = dp_gen_next(&g, (ky * KW + kx) * IC + ic);
+        }
+        return ORC_VALID;
+    }
+    /* depthwise weight [KH, KW, C, M] */
+    const uint32_t KH = (uint32_t)shape[0], KW = (uint32_t)shape[1], C = (uint32_t)shape[2], M = (uint32_t)shape[3];
+    for (uint64_t t = 0; t < T; t++)
+    {
+        const uint32_t kx = (uint32_t)(((t / M) / C) % KW), ky = (uint32_t)((((t / M) / C) / KW) % KH);
+        out[t]            = dp_gen_next(&g, ky * KW + kx);
+    }
+    return ORC_VALID;
+}

@@ -24,6 +24,9 @@
  *     4096 (multiplier = floor(((2^30+1) << k) / count)), and an independent numpy restatement over padded
  *     windows for general shapes.  Floating-point AVG_POOL2D sums in tap order in fp32 like the reference's
  *     loop nest (tensor_ops.cpp:613-634), so it is compared bit for bit.
+ *   - DOT_PRODUCT data sets S0..S5: the generator's own goldens, reference_model/test/generate_tests.cpp:315-372
+ *     (MATMUL fp32, first three values of both operands, all six sets), :444-535 (CONV2D fp32, last three values
+ *     of input / weight / bias, all six sets) and :1194-1222 (DEPTHWISE_CONV2D fp16, sets 0 and 1), bit for bit.
  *   - large shapes: independent numpy int64 einsum / float64 convolution.
  *   - fp accumulate order of MATMUL (Eigen contraction order): parity unpinned (tolerance covered).
  */
@@ -188,6 +191,23 @@ int orc_avg_pool2d_f32(const orc_pool_shape_t* s, const float* in, float* out);
 int orc_max_pool2d_i32(const orc_pool_shape_t* s, const int32_t* in, int32_t lowest, int32_t* out);
 /* nan_mode: 1 = PROPAGATE, 2 = IGNORE */
 int orc_max_pool2d_f32(const orc_pool_shape_t* s, const float* in, int nan_mode, float* out);
+
+/* DOT_PRODUCT test data sets S0..S5 of the TOSA specification (tosa_mi_data), as the reference's data generator
+ * produces them (reference_model/src/generate/generate_dot_product_states.cpp:39-300 generators and bound
+ * parameter B, generate_dot_product.cpp:23-50 MATMUL, :113-196 CONV2D, :455-538 DEPTHWISE_CONV2D index maps).
+ * op: 0 MATMUL, 1 CONV2D, 2 DEPTHWISE_CONV2D; param: operand position (0 input / A, 1 weight / B, 2 bias);
+ * shape: the operand's shape; kernel: {KH, KW}, read for the input operand of the convolutions.
+ * Values are produced in fp32; the caller narrows them to the operand's type. */
+enum
+{
+    ORC_DP_MATMUL    = 0,
+    ORC_DP_CONV2D    = 1,
+    ORC_DP_DEPTHWISE = 2
+};
+/* bound parameter B for (data type bits 16 = fp16, 17 = bf16, 32 = fp32; accumulator fp32 unless acc16) */
+float orc_dp_bound_parameter(int data_kind, int acc16);
+int orc_dp_generate(int op, int set, int param, uint32_t ks, float B, const int32_t* shape, int rank,
+                    const int32_t* kernel, float* out);
 
 int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out);
 /* CLAMP for float storage; nan_mode 1 = PROPAGATE, 2 = IGNORE. */
