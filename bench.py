@@ -44,7 +44,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "copy"])
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,6 +110,26 @@ def main() -> int:
                  peak=PEAK["hbm"], runit="GB/s",
                  workload="RESCALE int32 [64,56,56,64] -> int8, per-channel multiplier/shift 38, double_round, "
                           "output_zp -3 (5 bytes per element)")
+    elif cfg == "precise":
+        # the fp64 precise-mode pass of the compliance flow at the shape of the named fp16 CONV2D configuration
+        import oracle
+        c = cases.c5_conv()
+        n, ih, iw, ic = c["x"].shape
+        oc, kh, kw, _ = c["w"].shape
+        tx, tw, tb = to_dev(c["x"]), to_dev(c["w"]), to_dev(c["bias"])
+        out = torch.empty((n, ih, iw, oc), dtype=torch.float64, device=dev)
+        d = ctx.conv_desc(capi.FP16, capi.FP16, (n, ih, iw, ic), oc, kh, kw, (ih, iw), c["pad"], c["stride"],
+                          c["dilation"], oc)
+        step = lambda: ctx.conv2d_precise(d, tx, tw, tb, False, out)
+        x64, w64, b64 = (c[k].astype(np.float64) for k in ("x", "w", "bias"))
+        cpu_ref = lambda: oracle.conv2d("f64", x64[:1], w64, b64, c["pad"], c["stride"], c["dilation"])
+        W = dict(ops=2 * n * ih * iw * oc * kh * kw * ic, bytes=c["x"].nbytes + c["w"].nbytes + c["bias"].nbytes +
+                 out.numel() * 8, exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0 / n,
+                 result=lambda: out[:1].cpu().numpy(), dtype="f64",
+                 metric="fp64 precise-mode CONV2D TFLOPS 3x3 [16,28,28,256]x[256,3,3,256]; bit-exact vs the fp64 oracle",
+                 unit="TFLOPS", bound="mfma", peak=78.6, runit="TFLOP/s",
+                 workload="precise-mode (fp64) pass of configs[4a]: CONV2D 3x3 [16,28,28,256]x[256,3,3,256] s1 p1, "
+                          "fp16 operands, fp64 products and sums in the reference's loop order")
     elif cfg in ("maxpool", "avgpool"):
         # the pooling neighbours at sizes where launch latency no longer dominates: the 3x3 stride-2 max pooling
         # behind a ResNet stem for 32 images, and a 2x2 stride-2 average pooling of the same tensor
@@ -282,7 +302,7 @@ def main() -> int:
                  bound="mfma", peak=PEAK["f16_mfma"], runit="TFLOP/s",
                  workload="configs[4a]: FP16 CONV2D 3x3 [16,28,28,256]x[256,3,3,256] s1 p1, fp32 accumulate")
 
-    big = cfg in ("c5b",)
+    big = cfg in ("c5b", "precise")
     steps = args.steps if args.steps is not None else (200 if big else 2000)
     warmup = args.warmup if args.warmup is not None else (20 if big else 200)
 

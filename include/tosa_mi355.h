@@ -254,6 +254,42 @@ int tmi_avg_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev,
  * mode, reference_model/src/arith_util.h:341-373). */
 int tmi_max_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev, void* out_dev);
 
+/* ---- floating-point compliance passes -------------------------------------------------------------- */
+
+/* The reference evaluates a floating-point graph twice more to judge an implementation: in precise mode
+ * (--precise_mode: all floating-point tensors in fp64, reference_model/src/main.cpp and the FP64 instantiations
+ * of op_factory.cpp) and in bounds mode (the same sums over absolute values, tensor_ops.cpp:757-765,
+ * 1213-1221, 1436-1443).  These entries compute either pass on the device: operands in their storage type
+ * (TMI_FP16 / TMI_BF16), fp64 products and sums in the reference's loop order, fp64 output of the operator's
+ * output shape.  bounds_mode != 0 selects the sums of absolute values. */
+int tmi_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                       const void* bias_dev, int32_t bounds_mode, double* out_dev);
+int tmi_depthwise_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev,
+                                 const void* weight_dev, const void* bias_dev, int32_t bounds_mode, double* out_dev);
+int tmi_matmul_precise(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
+                       const void* a_dev, const void* b_dev, int32_t bounds_mode, double* out_dev);
+
+/* What validateDataDP reports (reference_model/src/verify/verify_dot_product.cpp:89-139). */
+typedef struct
+{
+    double err_sum;          /* sum over the elements of (imp - ref) / max(bnd * 2^-(1+frac), normal_min) */
+    double err_sumsq;        /* sum of their squares */
+    double max_abs_err;      /* largest magnitude among them */
+    int64_t failed_elements; /* elements outside abs_bound, or breaking the zero-bound / NaN rules */
+    int64_t elements;
+    int32_t abs_bound;       /* 2 * ksb */
+    double variance_bound;   /* 1.6 * ksb */
+    int32_t compliant;       /* 1 when every rule of validateDataDP holds */
+} tmi_dp_result_t;
+
+/* The DOT_PRODUCT compliance check (verify_dot_product.cpp:30-139) of n device-resident results imp_dev of
+ * type out_dtype (TMI_FP16 / TMI_BF16 / TMI_FP32) against the precise-mode results ref_dev and the bounds-mode
+ * results bnd_dev.  ksb is the kernel size bound, set_number the test data set (the error-sum rule applies to
+ * sets 3..5; pass -1 for data that is not one of the sets).  Synchronises the context's stream.  Returns
+ * TMI_VALID with result->compliant 0 or 1; TMI_ERROR only for bad arguments. */
+int tmi_dot_product_check(tmi_ctx_t* ctx, int32_t out_dtype, int64_t n, const void* imp_dev, const double* ref_dev,
+                          const double* bnd_dev, int32_t ksb, int32_t set_number, tmi_dp_result_t* result);
+
 /* ---- validation only (no launch) ---------------------------------------------------------------- */
 
 /* The checks OpConv2d / OpDepthwiseConv2d::checkTensorAttributes and the head of eval() perform

@@ -20,7 +20,8 @@ ROUND_SINGLE, ROUND_INEXACT, ROUND_DOUBLE = 1, 2, 3
 FLAG_SCALE_MULTIPLIER, FLAG_SCALE_SHIFT, FLAG_SCALE_VALUE, FLAG_SCALE_RESULT, FLAG_ZP_RESULT = 1, 2, 4, 8, 16
 KERNEL_AUTO, KERNEL_DIRECT, KERNEL_MFMA, KERNEL_GEMM = 0, 1, 2, 3
 
-DTYPE_SIZE = {INT8: 1, INT16: 2, INT32: 4, FP32: 4, FP16: 2, BF16: 2}
+F64 = -64  # host-side tag of the fp64 buffers of the precise / bounds passes (not a TOSA element type)
+DTYPE_SIZE = {INT8: 1, INT16: 2, INT32: 4, FP32: 4, FP16: 2, BF16: 2, F64: 8}
 _NP_TO_TMI = {np.dtype(np.int8): INT8, np.dtype(np.uint8): INT8, np.dtype(np.int16): INT16,
               np.dtype(np.uint16): INT16, np.dtype(np.int32): INT32, np.dtype(np.float32): FP32,
               np.dtype(np.float16): FP16}
@@ -32,6 +33,7 @@ EXPORTS = [
     "tmi_depthwise_conv2d_rescale_clamp", "tmi_ctx_set_kernel_choice", "tmi_conv2d_check", "tmi_rescale_check",
     "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
+    "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
 ]
 
 
@@ -63,6 +65,12 @@ class PoolDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("dtype", "acc_dtype", "N", "IH", "IW", "C", "OH", "OW")] + [
         ("kernel", ctypes.c_int32 * 2), ("stride", ctypes.c_int32 * 2), ("pad", ctypes.c_int32 * 4),
         ("nan_mode", ctypes.c_int32)]
+
+
+class DpResult(ctypes.Structure):
+    _fields_ = [("err_sum", ctypes.c_double), ("err_sumsq", ctypes.c_double), ("max_abs_err", ctypes.c_double),
+                ("failed_elements", ctypes.c_int64), ("elements", ctypes.c_int64), ("abs_bound", ctypes.c_int32),
+                ("variance_bound", ctypes.c_double), ("compliant", ctypes.c_int32)]
 
 
 class RescaleDesc(ctypes.Structure):
@@ -120,6 +128,10 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_avg_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, i32, i32, vp]
     lib.tmi_max_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, vp]
     lib.tmi_pool2d_check.argtypes = [vp, ctypes.POINTER(PoolDesc), i32]
+    lib.tmi_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, vp]
+    lib.tmi_depthwise_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, vp]
+    lib.tmi_matmul_precise.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, vp]
+    lib.tmi_dot_product_check.argtypes = [vp, i32, i64, vp, vp, vp, i32, i32, ctypes.POINTER(DpResult)]
     lib.tmi_conv2d_check.argtypes = [vp, ctypes.POINTER(ConvDesc), i32]
     lib.tmi_rescale_check.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i32]
     for name in EXPORTS:
@@ -155,7 +167,7 @@ class DeviceTensor:
 
     def numpy(self) -> np.ndarray:
         dt = self.np_dtype or {INT8: np.int8, INT16: np.int16, INT32: np.int32, FP32: np.float32,
-                               FP16: np.float16, BF16: np.uint16}[self.dtype]
+                               FP16: np.float16, BF16: np.uint16, F64: np.float64}[self.dtype]
         out = np.empty(self.shape, dtype=dt)
         self.ctx._check(self.ctx.lib.tmi_download(self.ctx.handle, out.ctypes.data_as(ctypes.c_void_p),
                                                   ctypes.c_void_p(self.ptr), self.nbytes))
@@ -270,6 +282,20 @@ class Context:
     def transpose_conv2d(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_transpose_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
                                                          _ptr(bias), in_zp, w_zp, _ptr(out)))
+
+    def conv2d_precise(self, d: ConvDesc, inp, w, bias, bounds_mode, out, depthwise=False) -> int:
+        fn = self.lib.tmi_depthwise_conv2d_precise if depthwise else self.lib.tmi_conv2d_precise
+        return self._check(fn(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias), int(bounds_mode), _ptr(out)))
+
+    def matmul_precise(self, in_dtype, n, h, c, w, a, b, bounds_mode, out) -> int:
+        return self._check(self.lib.tmi_matmul_precise(self.handle, in_dtype, n, h, c, w, _ptr(a), _ptr(b),
+                                                       int(bounds_mode), _ptr(out)))
+
+    def dot_product_check(self, out_dtype, n, imp, ref, bnd, ksb, set_number=-1) -> DpResult:
+        r = DpResult()
+        self._check(self.lib.tmi_dot_product_check(self.handle, out_dtype, n, _ptr(imp), _ptr(ref), _ptr(bnd), ksb,
+                                                   set_number, ctypes.byref(r)))
+        return r
 
     def avg_pool2d(self, d: PoolDesc, inp, in_zp, out_zp, out) -> int:
         return self._check(self.lib.tmi_avg_pool2d(self.handle, ctypes.byref(d), _ptr(inp), in_zp, out_zp, _ptr(out)))

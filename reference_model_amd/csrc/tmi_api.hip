@@ -827,6 +827,107 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
     return after_launch(ctx, name);
 }
 
+// ---- floating-point compliance passes (precise.hip) -------------------------------------------------------
+static int run_conv_precise(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in,
+                            const void* w, const void* bias, int32_t bounds_mode, double* out)
+{
+    ConvGeom g;
+    int rc = validate_conv(ctx, op, d, depthwise, 0, 0, g);
+    if (rc != TMI_VALID)
+        return rc;
+    if (d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+        return fail(ctx, "%s: the precise / bounds passes take floating-point operands", op);
+    const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
+    if (total > 0 && (!in || !w || !bias || !out))
+        return fail(ctx, "%s: null tensor pointer", op);
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    const char* name = launch_conv_precise(ctx->stream, d->in_dtype, depthwise, g, in, w, bias, bounds_mode, out);
+    if (!name)
+        return fail(ctx, "%s: operand type without a precise-mode kernel", op);
+    return after_launch(ctx, name);
+}
+
+int tmi_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                       const void* bias_dev, int32_t bounds_mode, double* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_conv_precise(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, bounds_mode, out_dev);
+}
+
+int tmi_depthwise_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
+                                 const void* bias_dev, int32_t bounds_mode, double* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_conv_precise(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, bounds_mode, out_dev);
+}
+
+int tmi_matmul_precise(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
+                       const void* b_dev, int32_t bounds_mode, double* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
+        return fail(ctx, "OpMatMul: the precise / bounds passes take floating-point operands");
+    if (N < 0 || H < 0 || C < 0 || W < 0)
+        return fail(ctx, "OpMatMul: negative tensor dimension");
+    const int64_t total = (int64_t)N * H * W;
+    if (total > 0 && (!out_dev || (C > 0 && (!a_dev || !b_dev))))
+        return fail(ctx, "OpMatMul: null tensor pointer");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    if (total == 0)
+    {
+        ctx->last_kernel = "empty";
+        return TMI_VALID;
+    }
+    const char* name = launch_matmul_precise(ctx->stream, in_dtype, N, H, C, W, a_dev, b_dev, bounds_mode, out_dev);
+    if (!name)
+        return fail(ctx, "OpMatMul: operand type without a precise-mode kernel");
+    return after_launch(ctx, name);
+}
+
+int tmi_dot_product_check(tmi_ctx_t* ctx, int32_t out_dtype, int64_t n, const void* imp_dev, const double* ref_dev,
+                          const double* bnd_dev, int32_t ksb, int32_t set_number, tmi_dp_result_t* result)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (!result || n <= 0 || !imp_dev || !ref_dev || !bnd_dev || ksb <= 0)
+        return fail(ctx, "dot product check: bad argument");
+    if (out_dtype != TMI_FP16 && out_dtype != TMI_BF16 && out_dtype != TMI_FP32)
+        return fail(ctx, "dot product check: result type must be FP16, BF16 or FP32");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    // accumulators: 3 doubles + 1 word in the upper half of the context's 256-byte flag block
+    uint8_t* acc = reinterpret_cast<uint8_t*>(ctx->flags_dev) + 128;
+    TMI_HIP(ctx, hipMemsetAsync(acc, 0, 32, ctx->stream));
+    const int32_t abs_bound = 2 * ksb;
+    if (!launch_dp_check(ctx->stream, out_dtype, n, imp_dev, ref_dev, bnd_dev, abs_bound,
+                         reinterpret_cast<double*>(acc), reinterpret_cast<unsigned long long*>(acc + 24)))
+        return fail(ctx, "dot product check: launch failed");
+    ctx->last_kernel = "dot_product_check";
+    struct
+    {
+        double v[3];
+        unsigned long long bad;
+    } host;
+    TMI_HIP(ctx, hipMemcpyAsync(&host, acc, 32, hipMemcpyDeviceToHost, ctx->stream));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    result->err_sum = host.v[0], result->err_sumsq = host.v[1], result->max_abs_err = host.v[2];
+    result->failed_elements = (int64_t)host.bad, result->elements = n;
+    result->abs_bound = abs_bound, result->variance_bound = 4.0 * 0.4 * ksb;
+    // validateDataDP: every element within its bound; for sets 3..5 |sum| <= sqrt(10 * var * T); sumsq <= var * T
+    bool ok = host.bad == 0 && result->err_sumsq <= result->variance_bound * (double)n;
+    if (set_number >= 3 && set_number <= 5)
+        ok = ok && fabs(result->err_sum) <= sqrt(10.0 * result->variance_bound * (double)n);
+    result->compliant = ok ? 1 : 0;
+    return TMI_VALID;
+}
+
 // check_pool2d_attribute (tensor_ops.cpp:29-117) with the reference's messages, plus the type rules.
 static int validate_pool(tmi_ctx* ctx, const char* op, const tmi_pool_desc_t* d, bool avg, int32_t in_zp,
                          int32_t out_zp)

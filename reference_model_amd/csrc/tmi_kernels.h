@@ -66,6 +66,16 @@ const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_d
 const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                     const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                     const RescaleParams& rp, void* out, uint32_t* flag_word);
+// precise.hip: fp64 precise-mode / bounds-mode passes (abs_mode != 0: sums over absolute values) of CONV2D,
+// DEPTHWISE_CONV2D and MATMUL on fp16 / bf16 / fp32 operands, and the DOT_PRODUCT check as a reduction
+// (results: 3 doubles, counts: 1 word, both zero before the launch).  nullptr for another operand type.
+const char* launch_conv_precise(hipStream_t st, int32_t in_dtype, bool depthwise, const ConvGeom& g, const void* in,
+                                const void* w, const void* bias, int32_t abs_mode, double* out);
+const char* launch_matmul_precise(hipStream_t st, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
+                                  const void* a, const void* b, int32_t abs_mode, double* out);
+const char* launch_dp_check(hipStream_t st, int32_t out_dtype, int64_t n, const void* imp, const double* ref,
+                            const double* bnd, int32_t abs_bound, double* results, unsigned long long* counts);
+
 // pool.hip: AVG_POOL2D (avg) / MAX_POOL2D; nullptr for a dtype without a kernel or 2^32 work items or more.
 const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int32_t IH, int32_t IW, int32_t C,
                         int32_t OH, int32_t OW, int32_t kernel_y, int32_t kernel_x, int32_t stride_y, int32_t stride_x,

@@ -1,0 +1,165 @@
+"""The floating-point compliance passes on the device: precise mode (fp64) and bounds mode (sums of absolute
+values) of CONV2D / DEPTHWISE_CONV2D / MATMUL against the fp64 oracle, the DOT_PRODUCT check as a device
+reduction against its numpy restatement, and the whole flow - fast kernel, precise pass, bounds pass, check -
+at the full size of the fp16 / bf16 benchmark configurations on the specification's data sets S0..S5."""
+import numpy as np
+import pytest
+
+import cases
+import dot_product_check as dp
+import oracle
+from reference_model_amd import Context, capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = Context(0)
+    yield c
+    c.close()
+
+
+def narrow(values, kind):
+    """float32 values -> (array as it travels to the device, the same values in fp64, TMI dtype)"""
+    if kind == "fp16":
+        with np.errstate(over="ignore"):     # set 1 puts a bias beyond the fp16 range: it becomes infinity, as
+            h = values.astype(np.float16)    # in the reference's generator, and the check's overflow rule applies
+        return h, h.astype(np.float64), capi.FP16
+    b = cases.float_to_bf16_bits(values)
+    return b, cases.bf16_bits_to_float(b).astype(np.float64), capi.BF16
+
+
+def as_f64(t, kind):
+    a = t.numpy()
+    return a.astype(np.float64) if kind in ("fp16", "fp32") else cases.bf16_bits_to_float(a).astype(np.float64)
+
+
+CONV_CASES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
+    (2, 9, 8, 16, 24, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 12, 11, 8, 5, 3, 2, (2, 1, 0, 1), (2, 1), (1, 2)),
+    (3, 5, 5, 40, 16, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("shape", CONV_CASES)
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("bounds", [False, True])
+def test_conv2d_precise_and_bounds_match_the_fp64_oracle(ctx, shape, kind, bounds):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(ih * iw + oc)
+    xs, xf, dtype = narrow(rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float32), kind)
+    ws, wf, _ = narrow(rng.normal(0, 1, (oc, kh, kw, ic)).astype(np.float32), kind)
+    bs, bf, _ = narrow(rng.normal(0, 1, oc).astype(np.float32), kind)
+    oh, ow = oracle.conv_out_hw(ih, iw, kh, kw, pad, stride, dil)
+    d = ctx.conv_desc(dtype, dtype, xs.shape, oc, kh, kw, (oh, ow), pad, stride, dil, oc)
+    out = ctx.empty((n, oh, ow, oc), capi.F64)
+    ctx.conv2d_precise(d, ctx.upload(xs, dtype), ctx.upload(ws, dtype), ctx.upload(bs, dtype), bounds, out)
+    assert ctx.sync() == capi.VALID
+    want = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=bounds)
+    # same products, same order of fp64 additions, bias last: the same fp64 numbers
+    assert np.array_equal(out.numpy(), want)
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("bounds", [False, True])
+def test_depthwise_and_matmul_precise_match_the_fp64_oracle(ctx, kind, bounds):
+    rng = np.random.default_rng(17)
+    n, ih, iw, c, m, kh, kw = 2, 9, 7, 12, 2, 3, 3
+    xs, xf, dtype = narrow(rng.normal(0, 1, (n, ih, iw, c)).astype(np.float32), kind)
+    ws, wf, _ = narrow(rng.normal(0, 1, (kh, kw, c, m)).astype(np.float32), kind)
+    bs, bf, _ = narrow(rng.normal(0, 1, c * m).astype(np.float32), kind)
+    pad, stride, dil = (1, 1, 1, 1), (2, 2), (1, 1)
+    oh, ow = oracle.conv_out_hw(ih, iw, kh, kw, pad, stride, dil)
+    d = ctx.conv_desc(dtype, dtype, xs.shape, c * m, kh, kw, (oh, ow), pad, stride, dil, c * m)
+    out = ctx.empty((n, oh, ow, c * m), capi.F64)
+    ctx.conv2d_precise(d, ctx.upload(xs, dtype), ctx.upload(ws, dtype), ctx.upload(bs, dtype), bounds, out, depthwise=True)
+    assert ctx.sync() == capi.VALID
+    assert np.array_equal(out.numpy(), oracle.depthwise_conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=bounds))
+
+    a_s, af, _ = narrow(rng.normal(0, 1, (3, 17, 96)).astype(np.float32), kind)
+    b_s, bf2, _ = narrow(rng.normal(0, 1, (3, 96, 29)).astype(np.float32), kind)
+    out = ctx.empty((3, 17, 29), capi.F64)
+    ctx.matmul_precise(dtype, 3, 17, 96, 29, ctx.upload(a_s, dtype), ctx.upload(b_s, dtype), bounds, out)
+    assert ctx.sync() == capi.VALID
+    assert np.array_equal(out.numpy(), oracle.matmul("f64", af, bf2, abs_mode=bounds))
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "fp32"])
+def test_device_dot_product_check_matches_its_numpy_restatement(ctx, kind):
+    rng = np.random.default_rng(5)
+    n, ksb = 100_000, 9
+    ref = rng.normal(0, 3, n)
+    bnd = np.abs(ref) + np.abs(rng.normal(0, 3, n))
+    frac = dp.NORMAL_FRAC[kind]
+    noise = rng.normal(0, 0.7, n) * bnd * 2.0 ** (-1 - frac)
+    imp64 = ref + noise
+    bnd[:50], ref[:50], imp64[:50] = 0.0, 0.0, 0.0            # all-zero products
+    if kind == "fp16":
+        imp = imp64.astype(np.float16)
+    elif kind == "bf16":
+        imp = cases.float_to_bf16_bits(imp64.astype(np.float32))
+    else:
+        imp = imp64.astype(np.float32)
+    dtype = {"fp16": capi.FP16, "bf16": capi.BF16, "fp32": capi.FP32}[kind]
+    impf = imp.astype(np.float64) if kind != "bf16" else cases.bf16_bits_to_float(imp).astype(np.float64)
+    want = dp.check(impf, ref, bnd, kind, ksb)
+    r = ctx.dot_product_check(dtype, n, ctx.upload(imp, dtype), ctx.upload(ref, capi.F64), ctx.upload(bnd, capi.F64), ksb)
+    assert r.elements == n and r.abs_bound == 2 * ksb and r.variance_bound == pytest.approx(1.6 * ksb)
+    assert r.max_abs_err == pytest.approx(want["max_err"], rel=1e-12)
+    assert r.err_sumsq == pytest.approx(want["err_sumsq"], rel=1e-9)
+    assert bool(r.compliant) == want["ok"] and r.failed_elements == 0
+    # an element far outside its bound, a non-zero result under a zero bound, a missed NaN
+    bad = impf.copy()
+    bad[1000] += 1000 * bnd[1000]
+    bad[10] = 1.0
+    ref2 = ref.copy()
+    ref2[2000] = np.nan
+    bad_dev = bad.astype(np.float16) if kind == "fp16" else (cases.float_to_bf16_bits(bad.astype(np.float32)) if kind == "bf16"
+                                                                else bad.astype(np.float32))
+    r = ctx.dot_product_check(dtype, n, ctx.upload(bad_dev, dtype), ctx.upload(ref2, capi.F64), ctx.upload(bnd, capi.F64), ksb)
+    assert r.failed_elements == 3 and not r.compliant
+
+
+@pytest.mark.parametrize("data_set", range(6))
+def test_config5_bf16_matmul_compliance_on_the_device(ctx, data_set):
+    """[4,2048,4096] x [4,4096,2048] bf16 -> fp32 on the specification's data set, every pass on the GPU:
+    the GEMM kernel, the fp64 precise pass, the bounds pass and the DOT_PRODUCT check with ksb = C."""
+    n, h, c, w = 4, 2048, 4096, 2048
+    a_s, _, dtype = narrow(oracle.dot_product_data("matmul", data_set, 0, c, (n, h, c), kind="bf16"), "bf16")
+    b_s, _, _ = narrow(oracle.dot_product_data("matmul", data_set, 1, c, (n, c, w), kind="bf16"), "bf16")
+    ta, tb = ctx.upload(a_s, dtype), ctx.upload(b_s, dtype)
+    imp, ref, bnd = ctx.empty((n, h, w), capi.FP32), ctx.empty((n, h, w), capi.F64), ctx.empty((n, h, w), capi.F64)
+    try:
+        ctx.matmul(dtype, n, h, c, w, ta, tb, 0, 0, imp)
+        assert ctx.last_kernel == "matmul_gemm_bf16"
+        ctx.matmul_precise(dtype, n, h, c, w, ta, tb, False, ref)
+        ctx.matmul_precise(dtype, n, h, c, w, ta, tb, True, bnd)
+        r = ctx.dot_product_check(capi.FP32, n * h * w, imp, ref, bnd, dp.kernel_size_bound(c, "fp32", has_bias=False), data_set)
+        assert r.compliant and r.failed_elements == 0, (r.max_abs_err, r.err_sum, r.err_sumsq)
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+
+@pytest.mark.parametrize("data_set", range(6))
+def test_config5_fp16_conv_compliance_on_the_device(ctx, data_set):
+    """fp16 CONV2D 3x3 [16,28,28,256] -> 256 (fp32 accumulate, fp16 result) on the specification's data set."""
+    n, hw, ic, oc = 16, 28, 256, 256
+    ks = 9 * ic
+    xs, _, dtype = narrow(oracle.dot_product_data("conv2d", data_set, 0, ks, (n, hw, hw, ic), kind="fp16", kernel=(3, 3)), "fp16")
+    ws, _, _ = narrow(oracle.dot_product_data("conv2d", data_set, 1, ks, (oc, 3, 3, ic), kind="fp16"), "fp16")
+    bs, _, _ = narrow(oracle.dot_product_data("conv2d", data_set, 2, ks, (oc,), kind="fp16"), "fp16")
+    d = ctx.conv_desc(dtype, dtype, xs.shape, oc, 3, 3, (hw, hw), (1, 1, 1, 1), (1, 1), (1, 1), oc)
+    tx, tw, tb = ctx.upload(xs, dtype), ctx.upload(ws, dtype), ctx.upload(bs, dtype)
+    shape = (n, hw, hw, oc)
+    imp, ref, bnd = ctx.empty(shape, capi.FP16), ctx.empty(shape, capi.F64), ctx.empty(shape, capi.F64)
+    try:
+        ctx.conv2d(d, tx, tw, tb, 0, 0, imp)
+        ctx.conv2d_precise(d, tx, tw, tb, False, ref)
+        ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
+        r = ctx.dot_product_check(capi.FP16, int(np.prod(shape)), imp, ref, bnd, dp.kernel_size_bound(ks, "fp16"), data_set)
+        assert r.compliant and r.failed_elements == 0, (r.max_abs_err, r.err_sum, r.err_sumsq)
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
