@@ -1,5 +1,5 @@
-// GEMM-shaped CONV2D (1x1 taps, stride 1, no padding) and MATMUL on the matrix cores, for work large enough
-// that operand delivery, not set-up, decides the time.
+// CONV2D as a GEMM over (ky, kx, ic) and MATMUL on the matrix cores, for work large enough that operand
+// delivery, not set-up, decides the time.
 //
 //   out[b][p][oc] = sum_k (a[b][p][k] - za) * (w[b][oc][k] - zw) + bias[oc]
 //
@@ -43,6 +43,13 @@ struct GemmArgs
     int32_t bias_len, za, zw, K;
     int32_t out_is_wide;    // floating point: 1 = fp32 output, 0 = output of the input type
     int32_t ldw;            // K-major weights: bytes between consecutive K rows (rows of N elements)
+    // implicit GEMM of a KH x KW convolution: the K axis is (ky, kx, ic), a 64-byte block lies inside one tap
+    const uint8_t* zero_page;    // 64 zero bytes: what a tap outside the image reads
+    int32_t IH, IW, OH, OW, KW, taps;
+    int32_t icb;                 // bytes of one input pixel (IC * sizeof(element)), a multiple of 64
+    int32_t bpt;                 // blocks per tap = icb / 64
+    int32_t sy, sx, dy, dx, pad_top, pad_left;
+    FastDiv div_bpt, div_kw;
     FastDiv div_batch, div_tn;
 };
 
@@ -80,9 +87,23 @@ static constexpr int kStages = 4;
 // With int8 the 8 lanes that share a source address get 8 consecutive channels, so the accumulator rows of
 // the int8 K-major variant are assigned to channels in order (row r is channel r) and a lane stores four
 // groups of 4 channels instead of 16 consecutive ones.
-template <typename T, int OCT, int PXT, bool ZP, bool KM>
+//
+// Convolutions with taps (MODE 2): the pixel operand's row p of K block b is the 64-byte piece b % bpt of input
+// pixel (oy*sy - pad + ky*dy, ox*sx - pad + kx*dx) for tap (ky, kx) = b / bpt of output pixel p: the same
+// direct load with a per-lane pixel offset worked out once, a per-block tap offset in scalar registers, and
+// the 64-byte zero page as the source where the tap falls outside the image (a bit per tap and lane).
+enum
+{
+    GEMM_KCONTIG = 0,
+    GEMM_KMAJOR  = 1,
+    GEMM_TAPS    = 2
+};
+
+template <typename T, int OCT, int PXT, bool ZP, int MODE>
 __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 {
+    constexpr bool KM      = MODE == GEMM_KMAJOR;
+    constexpr bool TAPS    = MODE == GEMM_TAPS;
     using M                = Mma<T>;
     constexpr int EB       = (int)sizeof(T);
     constexpr bool IDENT   = KM && EB == 1;    // accumulator row r of a channel tile is channel r
@@ -162,14 +183,54 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         }
         ldst[j]         = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + grp * 1024;
     }
+    // TAPS: byte offset of the window's first tap of the lane's pixel (may lie before the tensor) and the taps
+    // of the window that fall inside the image.  Loads j < OCT / 2 carry weight rows, the others pixel rows.
+    int32_t coff[LOADS];
+    uint32_t cmask[LOADS];
+    if constexpr (TAPS)
+    {
+#pragma unroll
+        for (int j = OCT / 2; j < LOADS; j++)
+        {
+            const int r = (j * 8 + wave) * 16 + (lane >> 2);
+            int p       = p0 + r - WROWS;
+            p           = p < a.M - 1 ? p : a.M - 1;
+            const int ox = p % a.OW, t2 = p / a.OW;
+            const int oy = t2 % a.OH, n = t2 / a.OH;
+            const int iy0 = oy * a.sy - a.pad_top, ix0 = ox * a.sx - a.pad_left;
+            coff[j]       = ((n * a.IH + iy0) * a.IW + ix0) * a.icb + (((lane & 3) ^ swz(r)) * 16);
+            uint32_t m    = 0;
+            for (int t = 0; t < a.taps; t++)
+            {
+                const int ky = t / a.KW, kx = t - ky * a.KW;
+                const int y = iy0 + ky * a.dy, x = ix0 + kx * a.dx;
+                m |= (y >= 0 && y < a.IH && x >= 0 && x < a.IW ? 1u : 0u) << t;
+            }
+            cmask[j] = m;
+        }
+    }
     const int nb = a.n_blocks;
     // Every block period issues one block's loads, also past the end (the last block again, into a stage nobody
     // reads any more): the count of loads in flight is then the same in every iteration and the wait for a
     // block is one instruction with an immediate.
     auto issue_one = [&](int block, int stage, int j) {
         const int blk      = block < nb ? block : nb - 1;
-        const uint8_t* src = gbase[j] + (size_t)blk * gstep[j];
         const uint32_t dst = ldst[j] + stage * STAGE;
+        if (TAPS && j >= OCT / 2)
+        {
+            // tap of the block (scalar), then per lane: the pixel under that tap, or the zero page
+            const int t       = (int)fdiv((uint32_t)blk, a.div_bpt);
+            const int piece   = blk - t * a.bpt;
+            const int ky      = (int)fdiv((uint32_t)t, a.div_kw);
+            const int kx      = t - ky * a.KW;
+            const int tap_off = (ky * a.dy * a.IW + kx * a.dx) * a.icb + piece * 64;
+            const bool inside = (cmask[j] >> t) & 1u;
+            const uint8_t* src =
+                inside ? a_base + (ptrdiff_t)(coff[j] + tap_off) : a.zero_page + (lane & 3) * 16;
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
+            return;
+        }
+        const uint8_t* src = gbase[j] + (size_t)blk * gstep[j];
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
                      : "v"(voff[j]), "s"(src), "s"(dst)
@@ -488,11 +549,11 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     }
 }
 
-template <typename T, int OCT, int PXT, bool ZP, bool KM>
+template <typename T, int OCT, int PXT, bool ZP, int MODE>
 static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
 {
     constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4;
-    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, KM>;
+    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE>;
     static bool configured     = false;
     if (!configured)
     {
@@ -506,7 +567,7 @@ static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
 }
 
 template <typename T>
-static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const char* label)
+static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool tapped, const char* label)
 {
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
     // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
@@ -539,19 +600,23 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const
     const int blocks  = a.per_xcd * 8;
     const bool zp     = Mma<T>::is_int && (a.za != 0 || a.zw != 0);
     bool ok           = false;
+#define TMI_GEMM_MODE(O, P, MODE)                                                                                      \
+    ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int, MODE>(st, a, blocks)                                          \
+            : launch_gemm_shape<T, O, P, false, MODE>(st, a, blocks)
 #define TMI_GEMM_SHAPE(O, P)                                                                                           \
     if (OCT == O && PXT == P)                                                                                          \
     {                                                                                                                  \
         if (a.ldw)                                                                                                     \
-            ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int, true>(st, a, blocks)                                  \
-                    : launch_gemm_shape<T, O, P, false, true>(st, a, blocks);                                          \
+            TMI_GEMM_MODE(O, P, GEMM_KMAJOR);                                                                          \
+        else if (tapped)                                                                                               \
+            TMI_GEMM_MODE(O, P, GEMM_TAPS);                                                                            \
         else                                                                                                           \
-            ok = zp ? launch_gemm_shape<T, O, P, Mma<T>::is_int, false>(st, a, blocks)                                 \
-                    : launch_gemm_shape<T, O, P, false, false>(st, a, blocks);                                         \
+            TMI_GEMM_MODE(O, P, GEMM_KCONTIG);                                                                         \
     }
     TMI_GEMM_SHAPE(4, 2);
     TMI_GEMM_SHAPE(2, 2);
     TMI_GEMM_SHAPE(2, 1);
+#undef TMI_GEMM_MODE
 #undef TMI_GEMM_SHAPE
     return ok ? label : nullptr;
 }
@@ -559,24 +624,36 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, const
 // nullptr when the operation is not a GEMM this kernel takes; the caller then goes to the patch kernel.
 const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                              const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride)
+                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride, const void* zero_page)
 {
-    if (rp.enabled || g.KH != 1 || g.KW != 1 || g.stride_y != 1 || g.stride_x != 1 || g.pad_top != 0 ||
-        g.pad_left != 0 || g.OH != g.IH || g.OW != g.IW)
+    if (rp.enabled)
         return nullptr;
-    const int eb = in_dtype == TMI_INT8 ? 1 : 2;
+    const int taps    = g.KH * g.KW;
+    const bool plain  = taps == 1 && g.stride_y == 1 && g.stride_x == 1 && g.pad_top == 0 && g.pad_left == 0 &&
+                       g.OH == g.IH && g.OW == g.IW;
     if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
         return nullptr;
+    const int eb = in_dtype == TMI_INT8 ? 1 : 2;
+    if (!plain)
+    {
+        // a convolution with taps, strides or padding: per-image weights and K-major weights are MATMUL's; a tap
+        // outside the image reads zeros, which stands for input_zp only when that is 0
+        if (w_batch_stride || w_kmajor_stride || !zero_page || taps > 32 || in_zp != 0)
+            return nullptr;
+        if ((int64_t)g.N * g.IH * g.IW * g.IC * eb >= (int64_t(1) << 31))
+            return nullptr;
+    }
     const bool wide = in_dtype == TMI_INT8 ? out_dtype == TMI_INT32 : out_dtype == TMI_FP32;
     if (!wide && (in_dtype == TMI_INT8 || out_dtype != in_dtype))
         return nullptr;
-    const int64_t kb = (int64_t)g.IC * eb;
-    if (kb % 64 != 0 || kb < 256)
+    const int64_t icb = (int64_t)g.IC * eb;
+    const int64_t kb  = icb * taps;
+    if (icb % 64 != 0 || kb < 256)
         return nullptr;
     // MATMUL: one GEMM per image with its own weights; CONV2D: all images are rows of one GEMM
     const bool per_image  = w_batch_stride != 0;
     const int batches     = per_image ? g.N : 1;
-    const int64_t M       = (int64_t)g.IH * g.IW * (per_image ? 1 : g.N);
+    const int64_t M       = (int64_t)g.OH * g.OW * (per_image ? 1 : g.N);
     const int64_t out_eb  = wide ? 4 : eb;
     if (M < 128 || g.OC < 64 || M * kb >= (int64_t(1) << 32) || (int64_t)g.OC * kb >= (int64_t(1) << 32))
         return nullptr;
@@ -585,7 +662,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
         return nullptr;
     // rows are multiples of 64 bytes, so 16-byte aligned bases keep every operand chunk aligned; the 16-byte
     // stores are only used when OC is a multiple of 16, which keeps every output row and batch aligned too
-    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out) & 15) || (w_batch_stride & 15))
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)zero_page) & 15) || (w_batch_stride & 15))
         return nullptr;
     // enough work to fill the CUs with the smallest tile shape
     if (((M + 127) / 128) * ((g.OC + 127) / 128) * batches < 128)
@@ -596,14 +673,26 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     a.a_batch = per_image ? M * kb : 0, a.w_batch = per_image ? w_batch_stride : 0;
     a.o_batch = per_image ? M * g.OC * out_eb : 0;
     a.M = (int32_t)M, a.N = g.OC, a.kb = (int32_t)kb, a.n_blocks = (int32_t)(kb / 64);
-    a.bias_len = g.bias_len, a.za = in_zp, a.zw = w_zp, a.K = g.IC;
+    a.bias_len = g.bias_len, a.za = in_zp, a.zw = w_zp, a.K = g.IC * taps;
     a.out_is_wide = wide ? 1 : 0;
     a.ldw         = (int32_t)w_kmajor_stride;
+    a.taps        = 1;
+    if (!plain)
+    {
+        a.taps      = taps;
+        a.zero_page = (const uint8_t*)zero_page;
+        a.IH = g.IH, a.IW = g.IW, a.OH = g.OH, a.OW = g.OW, a.KW = g.KW;
+        a.icb = (int32_t)icb, a.bpt = (int32_t)(icb / 64);
+        a.sy = g.stride_y, a.sx = g.stride_x, a.dy = g.dil_y, a.dx = g.dil_x;
+        a.pad_top = g.pad_top, a.pad_left = g.pad_left;
+        a.div_bpt = make_fastdiv((uint32_t)a.bpt), a.div_kw = make_fastdiv((uint32_t)a.KW);
+    }
+    const bool tapped = !plain;
     switch (in_dtype)
     {
-        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, "gemm_mfma_i8");
-        case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, "gemm_mfma_f16");
-        default: return launch_gemm_t<bf16_t>(st, a, batches, "gemm_mfma_bf16");
+        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, tapped, "gemm_mfma_i8");
+        case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, tapped, "gemm_mfma_f16");
+        default: return launch_gemm_t<bf16_t>(st, a, batches, tapped, "gemm_mfma_bf16");
     }
 }
 

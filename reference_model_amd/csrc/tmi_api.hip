@@ -315,7 +315,8 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     if (!depthwise && ctx->kernel_choice != 1)
     {
         if (ctx->kernel_choice != 2)
-            name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0);
+            name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
+                                    ctx->flags_dev + 48);    // bytes 192..255 of the flag block stay zero
         if (!name && ctx->kernel_choice != 3)
             name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                       ctx->flags_dev);

@@ -186,3 +186,78 @@ def test_config5_bf16_matmul_full_size_gemm(ctx):
     a2 = cases.float_to_bf16_bits(cases.bf16_bits_to_float(c["a"]) * 2.0)
     got2, _ = gpu_ops.matmul(ctx, a2, c["b"], dtype=capi.BF16)
     assert np.array_equal(got2, got * np.float32(2.0))
+
+
+# ---- convolutions with taps through the GEMM kernel (K axis = (ky, kx, ic), taps outside the image read zeros) ----
+TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
+    (16, 28, 28, 256, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # the named fp16 configuration
+    (40, 31, 29, 64, 136, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),      # stride 2, ragged tiles
+    (6, 40, 40, 128, 200, 5, 3, (2, 2, 1, 1), (1, 1), (1, 1)),      # 15 taps
+    (32, 24, 24, 64, 64, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),       # dilation 2
+    (16, 64, 64, 192, 96, 2, 2, (0, 0, 0, 0), (2, 2), (1, 1)),      # no padding
+    (2, 130, 100, 64, 72, 1, 7, (0, 0, 3, 3), (1, 1), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("shape", TAP_SHAPES)
+@pytest.mark.parametrize("w_zp", [0, -11])
+def test_conv2d_taps_i8_gemm_bit_exact(ctx, shape, w_zp):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(ih * iw + oc + kh)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
+    bias = rng.integers(-(1 << 20), 1 << 20, oc).astype(np.int32)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=0, w_zp=w_zp)
+    assert st == capi.VALID and ctx.last_kernel == "gemm_mfma_i8"
+    assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, 0, w_zp))
+    sub = oracle.conv2d("i8", x[-1:], w[:3], bias[:3], pad, stride, dil, in_zp=0, w_zp=w_zp)
+    assert np.array_equal(got[-1:, :, :, :3], sub)
+
+
+def test_conv2d_taps_with_input_zero_point_is_left_to_the_patch_kernel(ctx):
+    rng = np.random.default_rng(2)
+    x = rng.integers(-128, 128, (8, 28, 28, 64)).astype(np.int8)
+    w = rng.integers(-128, 128, (64, 3, 3, 64)).astype(np.int8)
+    with pytest.raises(TmiError):     # padding would have to read input_zp, the zero page holds zeros
+        gpu_ops.conv2d(ctx, x, w, np.zeros(64, np.int32), (1, 1, 1, 1), in_zp=5)
+
+
+@pytest.mark.parametrize("shape", TAP_SHAPES)
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+def test_conv2d_taps_fp_gemm_within_dot_product_bound(ctx, shape, kind):
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(31 + ic + kh)
+    x = rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float32)
+    w = rng.normal(0, 1 / np.sqrt(kh * kw * ic), (oc, kh, kw, ic)).astype(np.float32)
+    b = rng.normal(0, 0.1, oc).astype(np.float32)
+    if kind == "fp16":
+        xs, ws, bs = x.astype(np.float16), w.astype(np.float16), b.astype(np.float16)
+        xf, wf, bf = (v.astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.FP16
+    else:
+        xs, ws, bs = (cases.float_to_bf16_bits(v) for v in (x, w, b))
+        xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.BF16
+    got, st = gpu_ops.conv2d(ctx, xs, ws, bs, pad, stride, dil, dtype=dtype)
+    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16")
+    imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
+    # reference and bound from the device's fp64 precise / bounds passes, which the fp64 oracle pins bit for bit
+    oh, ow = got.shape[1], got.shape[2]
+    d = ctx.conv_desc(dtype, dtype, xs.shape, oc, kh, kw, (oh, ow), pad, stride, dil, oc)
+    tx, tw, tb = ctx.upload(xs, dtype), ctx.upload(ws, dtype), ctx.upload(bs, dtype)
+    ref, bnd = ctx.empty(got.shape, capi.F64), ctx.empty(got.shape, capi.F64)
+    try:
+        ctx.conv2d_precise(d, tx, tw, tb, False, ref)
+        ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
+        assert ctx.sync() == capi.VALID
+        ref_h, bnd_h = ref.numpy(), bnd.numpy()
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+    res = dp.check(imp, ref_h, bnd_h, kind, dp.kernel_size_bound(kh * kw * ic, kind))
+    # tolerance: |imp-ref| <= 2*ksb * max(bnd*2^-(1+frac), normal_min) per element, sum err^2 <= 1.6*ksb*T
+    assert res["ok"], res
+    sub = oracle.conv2d("f64", xf[-1:, -6:], wf[:2], bf[:2], (0, pad[1], pad[2], pad[3]), stride, dil) if stride == (1, 1) and dil == (1, 1) and kh <= 6 else None
+    if sub is not None:     # the bottom rows of the last image against the oracle's own loop nest
+        rows = sub.shape[1]
+        assert np.allclose(imp[-1:, -rows:, :, :2], sub, rtol=2.0 ** -6, atol=2.0 ** -8)
