@@ -42,9 +42,12 @@ struct GemmArgs
     int32_t tiles_n, tiles_per_batch, tiles_total, per_xcd;
     int32_t bias_len, za, zw, K;
     int32_t out_is_wide;    // floating point: 1 = fp32 output, 0 = output of the input type
+    RescaleParams rp;       // int8: the fused RESCALE (+ CLAMP) when enabled, through fast_rescale()
+    uint32_t* flag_word;    // where its REQUIRE conditions are latched
+    int32_t out_bytes;      // fused RESCALE: 1 (int8 results) or 2 (int16)
     int32_t ldw;            // K-major weights: bytes between consecutive K rows (rows of N elements)
     // implicit GEMM of a KH x KW convolution: the K axis is (ky, kx, ic), a 64-byte block lies inside one tap
-    const uint8_t* zero_page;    // 64 zero bytes: what a tap outside the image reads
+    const uint8_t* pad_page;    // 64 bytes of input_zp (zeros for floating point): what a tap outside the image reads
     int32_t IH, IW, OH, OW, KW, taps;
     int32_t icb;                 // bytes of one input pixel (IC * sizeof(element)), a multiple of 64
     int32_t bpt;                 // blocks per tap = icb / 64
@@ -226,7 +229,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             const int tap_off = (ky * a.dy * a.IW + kx * a.dx) * a.icb + piece * 64;
             const bool inside = (cmask[j] >> t) & 1u;
             const uint8_t* src =
-                inside ? a_base + (ptrdiff_t)(coff[j] + tap_off) : a.zero_page + (lane & 3) * 16;
+                inside ? a_base + (ptrdiff_t)(coff[j] + tap_off) : a.pad_page + (lane & 3) * 16;
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
             return;
         }
@@ -256,6 +259,21 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 v = __float_as_int(load_as_float<T>(a.bias, a.bias_len == 1 ? 0 : oc));
         }
         tab_bias[tid] = v;
+    }
+
+    // per-channel constants of the fused RESCALE, derived once per workgroup (WROWS entries of 32 bytes)
+    ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(lds + kStages * STAGE + WROWS * 4);
+    uint32_t flags       = 0;
+    if constexpr (M::is_int)
+    {
+        if (a.rp.enabled && tid < WROWS)
+        {
+            const int oc  = oc0 + tid;
+            const bool ok = oc < a.N;    // channels past the end get neutral constants: nothing raised
+            const int occ = ok ? oc : 0;
+            const int32_t m_raw = load_multiplier(a.rp, occ), s_raw = load_shift(a.rp, occ);
+            tab_cs[tid] = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : 32, a.rp.double_round != 0, flags);
+        }
     }
 
     // ---- fragment addresses -----------------------------------------------------------------------------
@@ -474,8 +492,66 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 continue;
             if constexpr (M::is_int)
             {
-                int32_t* row    = reinterpret_cast<int32_t*>(out_b) + (size_t)p * a.N;
                 const int pcorr = ZP ? a.zw * psum[i] : 0;
+                if (a.rp.enabled)
+                {
+                    // fused RESCALE (+ CLAMP): the lane's 16 consecutive channels leave as 16 (32) bytes
+                    const int ocl = tl + 16 * h;
+                    const int oc  = oc0 + ocl;
+                    if (oc >= a.N)
+                        continue;
+                    int r[16];
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                    {
+                        const ChannelScale cs = tab_cs[ocl + e];
+                        r[e] = fast_rescale(acc[i][t][e] + cb[e] - pcorr, cs, a.rp.out_zp, a.rp.lo, a.rp.hi, flags);
+                    }
+                    uint8_t* dst = out_b + ((size_t)p * a.N + oc) * a.out_bytes;
+                    if (a.out_bytes == 1)
+                    {
+                        if (rows16)
+                        {
+                            v4i packed;
+#pragma unroll
+                            for (int q = 0; q < 4; q++)
+                                packed[q] = (r[4 * q] & 0xff) | ((r[4 * q + 1] & 0xff) << 8) |
+                                            ((r[4 * q + 2] & 0xff) << 16) | ((r[4 * q + 3] & 0xff) << 24);
+                            *reinterpret_cast<v4i*>(dst) = packed;
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 16; e++)
+                                if (oc + e < a.N)
+                                    dst[e] = (uint8_t)r[e];
+                        }
+                    }
+                    else
+                    {
+                        if (rows16)
+                        {
+#pragma unroll
+                            for (int hq = 0; hq < 2; hq++)
+                            {
+                                v4i packed;
+#pragma unroll
+                                for (int q = 0; q < 4; q++)
+                                    packed[q] = (r[8 * hq + 2 * q] & 0xffff) | ((r[8 * hq + 2 * q + 1] & 0xffff) << 16);
+                                reinterpret_cast<v4i*>(dst)[hq] = packed;
+                            }
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 16; e++)
+                                if (oc + e < a.N)
+                                    reinterpret_cast<int16_t*>(dst)[e] = (int16_t)r[e];
+                        }
+                    }
+                    continue;
+                }
+                int32_t* row    = reinterpret_cast<int32_t*>(out_b) + (size_t)p * a.N;
 #pragma unroll
                 for (int q = 0; q < 4; q++)
                 {
@@ -547,12 +623,16 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             }
         }
     }
+    if constexpr (M::is_int)
+        if (a.rp.enabled)
+            raise_flags(a.flag_word, flags);
 }
 
 template <typename T, int OCT, int PXT, bool ZP, int MODE>
 static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
 {
-    constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4;
+    // stages, bias table, per-channel RESCALE constants
+    constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
     auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE>;
     static bool configured     = false;
     if (!configured)
@@ -621,12 +701,29 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
     return ok ? label : nullptr;
 }
 
+// Which of the two MFMA kernels a CONV2D tries first when the caller leaves the choice open.  The patch kernel
+// stages an input patch with its halo once and serves every tap from LDS; this kernel reads each tap's operand
+// block through L2 again, and wins where that does not matter or K is deep.  Measured on MI355X over ResNet-like
+// layers (us, patch kernel / this kernel): pointwise layers int8 8.6 / 7.1, 21.3 / 14.8, 28.4 / 26.4 and
+// fp16 7.5 / 5.3, 26.4 / 11.8, 21.7 / 15.8; 3x3 layers fp16 with IC 256 and 512: 31.7 / 28.2, 56.8 / 50.4,
+// IC 128: 17.9 / 17.4, IC 64: 7.8 / 10.4; 3x3 layers int8: 7.5 / 11.0 (IC 64), 15.7 / 18.1 (IC 128),
+// 23.7 / 25.9 (IC 256), 36.4 / 39.8 (IC 512).
+bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
+{
+    if (g.KH * g.KW == 1)
+        return true;
+    return in_dtype != TMI_INT8 && g.IC >= 128;
+}
+
 // nullptr when the operation is not a GEMM this kernel takes; the caller then goes to the patch kernel.
 const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                              const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride, const void* zero_page)
+                             void* out, int64_t w_batch_stride, int64_t w_kmajor_stride, const void* pad_page,
+                             uint32_t* flag_word)
 {
-    if (rp.enabled)
+    // a fused RESCALE: the fast form only (32-bit scale, SINGLE / DOUBLE rounding), on int8 convolutions
+    if (rp.enabled && (!rp.fast || in_dtype != TMI_INT8 || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16) ||
+                       w_batch_stride || w_kmajor_stride || !flag_word))
         return nullptr;
     const int taps    = g.KH * g.KW;
     const bool plain  = taps == 1 && g.stride_y == 1 && g.stride_x == 1 && g.pad_top == 0 && g.pad_left == 0 &&
@@ -637,14 +734,16 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     if (!plain)
     {
         // a convolution with taps, strides or padding: per-image weights and K-major weights are MATMUL's; a tap
-        // outside the image reads zeros, which stands for input_zp only when that is 0
-        if (w_batch_stride || w_kmajor_stride || !zero_page || taps > 32 || in_zp != 0)
+        // outside the image reads the page of input_zp bytes
+        if (w_batch_stride || w_kmajor_stride || !pad_page || taps > 32)
             return nullptr;
         if ((int64_t)g.N * g.IH * g.IW * g.IC * eb >= (int64_t(1) << 31))
             return nullptr;
     }
     const bool wide = in_dtype == TMI_INT8 ? out_dtype == TMI_INT32 : out_dtype == TMI_FP32;
-    if (!wide && (in_dtype == TMI_INT8 || out_dtype != in_dtype))
+    if (!wide && !rp.enabled && (in_dtype == TMI_INT8 || out_dtype != in_dtype))
+        return nullptr;
+    if (rp.enabled && wide)
         return nullptr;
     const int64_t icb = (int64_t)g.IC * eb;
     const int64_t kb  = icb * taps;
@@ -654,7 +753,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     const bool per_image  = w_batch_stride != 0;
     const int batches     = per_image ? g.N : 1;
     const int64_t M       = (int64_t)g.OH * g.OW * (per_image ? 1 : g.N);
-    const int64_t out_eb  = wide ? 4 : eb;
+    const int64_t out_eb  = rp.enabled ? (out_dtype == TMI_INT8 ? 1 : 2) : (wide ? 4 : eb);
     if (M < 128 || g.OC < 64 || M * kb >= (int64_t(1) << 32) || (int64_t)g.OC * kb >= (int64_t(1) << 32))
         return nullptr;
     // K-major weights: whole 16-byte pieces per K row
@@ -662,7 +761,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
         return nullptr;
     // rows are multiples of 64 bytes, so 16-byte aligned bases keep every operand chunk aligned; the 16-byte
     // stores are only used when OC is a multiple of 16, which keeps every output row and batch aligned too
-    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)zero_page) & 15) || (w_batch_stride & 15))
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || (w_batch_stride & 15))
         return nullptr;
     // enough work to fill the CUs with the smallest tile shape
     if (((M + 127) / 128) * ((g.OC + 127) / 128) * batches < 128)
@@ -675,12 +774,13 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     a.M = (int32_t)M, a.N = g.OC, a.kb = (int32_t)kb, a.n_blocks = (int32_t)(kb / 64);
     a.bias_len = g.bias_len, a.za = in_zp, a.zw = w_zp, a.K = g.IC * taps;
     a.out_is_wide = wide ? 1 : 0;
+    a.rp = rp, a.flag_word = flag_word, a.out_bytes = (int32_t)out_eb;
     a.ldw         = (int32_t)w_kmajor_stride;
     a.taps        = 1;
     if (!plain)
     {
         a.taps      = taps;
-        a.zero_page = (const uint8_t*)zero_page;
+        a.pad_page = (const uint8_t*)pad_page;
         a.IH = g.IH, a.IW = g.IW, a.OH = g.OH, a.OW = g.OW, a.KW = g.KW;
         a.icb = (int32_t)icb, a.bpt = (int32_t)(icb / 64);
         a.sy = g.stride_y, a.sx = g.stride_x, a.dy = g.dil_y, a.dx = g.dil_x;
@@ -690,7 +790,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     const bool tapped = !plain;
     switch (in_dtype)
     {
-        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, tapped, "gemm_mfma_i8");
+        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, tapped, rp.enabled ? "gemm_mfma_i8_rescale" : "gemm_mfma_i8");
         case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, tapped, "gemm_mfma_f16");
         default: return launch_gemm_t<bf16_t>(st, a, batches, tapped, "gemm_mfma_bf16");
     }

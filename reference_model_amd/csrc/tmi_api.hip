@@ -14,6 +14,7 @@ struct tmi_ctx
     hipStream_t stream    = nullptr;
     bool owns_stream      = false;
     uint32_t* flags_dev   = nullptr;    // latched REQUIRE conditions
+    uint8_t* pages_dev    = nullptr;    // 256 pages of 64 bytes, page v filled with byte v: what padding reads
     uint32_t* flags_host  = nullptr;    // pinned staging word
     void* workspace       = nullptr;    // scratch for operand re-layout (MATMUL's transposed B)
     size_t workspace_size = 0;
@@ -314,12 +315,20 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
                                     ctx->flags_dev);
     if (!depthwise && ctx->kernel_choice != 1)
     {
-        if (ctx->kernel_choice != 2)
+        // kernel choice 2 / 3 name one kernel; left open, the likely faster one is tried first
+        const void* pad_page = ctx->pages_dev + (d->in_dtype == TMI_INT8 ? (in_zp & 255) * 64 : 0);
+        const bool gemm_ok   = ctx->kernel_choice != 2;
+        const bool patch_ok  = ctx->kernel_choice != 3;
+        const bool gemm_1st  = gemm_ok && (!patch_ok || gemm_mfma_preferred(d->in_dtype, g));
+        if (gemm_1st)
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
-                                    ctx->flags_dev + 48);    // bytes 192..255 of the flag block stay zero
-        if (!name && ctx->kernel_choice != 3)
+                                    pad_page, ctx->flags_dev);
+        if (!name && patch_ok)
             name = launch_conv2d_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                       ctx->flags_dev);
+        if (!name && gemm_ok && !gemm_1st)
+            name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
+                                    pad_page, ctx->flags_dev);
     }
     if (!name && ctx->kernel_choice >= 2)
         return fail(ctx, "%s: no MFMA / vector kernel is eligible for this shape", op);
@@ -365,7 +374,18 @@ int tmi_ctx_create(tmi_ctx_t** out_ctx, int device)
         return TMI_ERROR;
     }
     *ctx->flags_host = 0;
-    *out_ctx         = ctx;
+    {
+        std::string pages(256 * 64, '\0');
+        for (int v = 0; v < 256; v++)
+            memset(&pages[(size_t)v * 64], v, 64);
+        if (hipMalloc((void**)&ctx->pages_dev, pages.size()) != hipSuccess ||
+            hipMemcpy(ctx->pages_dev, pages.data(), pages.size(), hipMemcpyHostToDevice) != hipSuccess)
+        {
+            tmi_ctx_destroy(ctx);
+            return TMI_ERROR;
+        }
+    }
+    *out_ctx = ctx;
     return TMI_VALID;
 }
 
@@ -380,6 +400,8 @@ int tmi_ctx_destroy(tmi_ctx_t* ctx)
         (void)hipFree(ctx->workspace);
     if (ctx->flags_dev)
         (void)hipFree(ctx->flags_dev);
+    if (ctx->pages_dev)
+        (void)hipFree(ctx->pages_dev);
     if (ctx->flags_host)
         (void)hipHostFree(ctx->flags_host);
     if (ctx->owns_stream && ctx->stream)

@@ -82,15 +82,19 @@ const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int3
                         int32_t pad_top, int32_t pad_left, int32_t in_zp, int32_t out_zp, int32_t nan_mode,
                         const void* in, void* out, uint32_t* flag_word);
 
-// gemm_mfma.hip: CONV2D as a GEMM over (ky, kx, ic) and MATMUL (w_batch_stride != 0: per-image weights) with
-// operands loaded straight into LDS; nullptr when the operation is not such a GEMM or too small to gain.
-// w_kmajor_stride != 0: the weights are [K][OC] with that many bytes per K row (MATMUL's second operand as it
-// lies in memory) instead of [OC][K].  zero_page: 64 zero bytes in device memory, read where a tap falls outside
-// the image; without it only 1x1 / stride 1 / unpadded convolutions are taken.
+// gemm_mfma.hip: whether a CONV2D left to automatic choice tries the GEMM kernel before the patch kernel.
+bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g);
+
+// gemm_mfma.hip: CONV2D as a GEMM over (ky, kx, ic), with a fused RESCALE (+ CLAMP) when rp is enabled and of the
+// fast form, and MATMUL (w_batch_stride != 0: per-image weights), with operands loaded straight into LDS; nullptr
+// when the operation is not such a GEMM or too small to gain.  w_kmajor_stride != 0: the weights are [K][OC] with
+// that many bytes per K row (MATMUL's second operand as it lies in memory) instead of [OC][K].  pad_page: 64
+// bytes of input_zp (zeros for floating point) in device memory, read where a tap falls outside the image;
+// without it only 1x1 / stride 1 / unpadded convolutions are taken.  flag_word: needed for a fused RESCALE.
 const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                              const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                              void* out, int64_t w_batch_stride, int64_t w_kmajor_stride = 0,
-                             const void* zero_page = nullptr);
+                             const void* pad_page = nullptr, uint32_t* flag_word = nullptr);
 
 // conv2d_mfma.hip: implicit GEMM on the matrix cores with the fused epilogue; nullptr when not eligible.
 const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,

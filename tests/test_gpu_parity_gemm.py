@@ -214,12 +214,16 @@ def test_conv2d_taps_i8_gemm_bit_exact(ctx, shape, w_zp):
     assert np.array_equal(got[-1:, :, :, :3], sub)
 
 
-def test_conv2d_taps_with_input_zero_point_is_left_to_the_patch_kernel(ctx):
-    rng = np.random.default_rng(2)
-    x = rng.integers(-128, 128, (8, 28, 28, 64)).astype(np.int8)
-    w = rng.integers(-128, 128, (64, 3, 3, 64)).astype(np.int8)
-    with pytest.raises(TmiError):     # padding would have to read input_zp, the zero page holds zeros
-        gpu_ops.conv2d(ctx, x, w, np.zeros(64, np.int32), (1, 1, 1, 1), in_zp=5)
+@pytest.mark.parametrize("in_zp", [5, -128, 127])
+def test_conv2d_taps_i8_gemm_pads_with_the_input_zero_point(ctx, in_zp):
+    """taps outside the image read a page of input_zp bytes, so they contribute (zp - zp) * (w - w_zp) = 0"""
+    rng = np.random.default_rng(in_zp + 500)
+    x = rng.integers(-128, 128, (32, 28, 28, 64)).astype(np.int8)
+    w = rng.integers(-128, 128, (72, 3, 3, 64)).astype(np.int8)
+    bias = rng.integers(-999, 999, 72).astype(np.int32)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, (1, 1, 1, 1), in_zp=in_zp, w_zp=-4)
+    assert st == capi.VALID and ctx.last_kernel == "gemm_mfma_i8"
+    assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, (1, 1, 1, 1), (1, 1), (1, 1), in_zp, -4))
 
 
 @pytest.mark.parametrize("shape", TAP_SHAPES)
@@ -261,3 +265,96 @@ def test_conv2d_taps_fp_gemm_within_dot_product_bound(ctx, shape, kind):
     if sub is not None:     # the bottom rows of the last image against the oracle's own loop nest
         rows = sub.shape[1]
         assert np.allclose(imp[-1:, -rows:, :, :2], sub, rtol=2.0 ** -6, atol=2.0 ** -8)
+
+
+# ---- int8 convolutions with a fused RESCALE (+ CLAMP) and a non-zero input zero point through the GEMM kernel ----
+def _fused(ctx, c, out_dtype=np.int8):
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"],
+                             rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype),
+                             clamp=c["clamp"])
+    acc = cases.conv2d_exact_blas(c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
+    want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype)
+    if c["clamp"] is not None:
+        want = oracle.clamp(want, *c["clamp"])
+    return got, st, want, wst
+
+
+FUSED_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride
+    (8, 56, 56, 64, 64, 3, 3, (1, 1, 1, 1), (1, 1)),        # the headline layer's geometry
+    (16, 28, 28, 256, 256, 3, 3, (1, 1, 1, 1), (1, 1)),
+    (16, 28, 28, 256, 520, 1, 1, (0, 0, 0, 0), (1, 1)),     # pointwise, ragged channel tiles
+    (40, 31, 29, 64, 136, 3, 3, (1, 1, 1, 1), (2, 2)),
+]
+
+
+@pytest.mark.parametrize("shape", FUSED_SHAPES)
+@pytest.mark.parametrize("zps", [(4, 0, -3), (-128, 7, 100), (0, 0, 0)])
+@pytest.mark.parametrize("out_dtype", [np.int8, np.int16])
+def test_conv2d_fused_rescale_gemm_bit_exact(ctx, shape, zps, out_dtype):
+    n, ih, iw, ic, oc, kh, kw, pad, stride = shape
+    rng = np.random.default_rng(ih + oc + kh)
+    c = dict(x=rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8),
+             w=np.clip(np.rint(rng.normal(0, 40, (oc, kh, kw, ic))), -127, 127).astype(np.int8),
+             bias=rng.integers(-(1 << 16), 1 << 16, oc).astype(np.int32), in_zp=zps[0], w_zp=zps[1],
+             pad=pad, stride=stride, dilation=(1, 1), mult=rng.integers(1 << 30, 1 << 31, oc).astype(np.int32),
+             shift=rng.integers(36, 44, oc).astype(np.int8), out_zp=zps[2] if out_dtype == np.int8 else 0,
+             clamp=(-100, 110) if out_dtype == np.int8 else None)
+    got, st, want, wst = _fused(ctx, c, out_dtype)
+    assert ctx.last_kernel == "gemm_mfma_i8_rescale"
+    assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(got)) > 50     # the scale keeps the results inside the output range
+
+
+def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
+    """a shift below 32 makes apply_scale_32 check the value range (quant_util.h:59-67): UNPREDICTABLE, as the
+    oracle says for the same operands"""
+    n, ih, iw, ic, oc = 16, 28, 28, 256, 256
+    rng = np.random.default_rng(3)
+    c = dict(x=rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8),
+             w=rng.integers(-127, 128, (oc, 3, 3, ic)).astype(np.int8), bias=np.zeros(oc, np.int32), in_zp=3, w_zp=0,
+             pad=(1, 1, 1, 1), stride=(1, 1), dilation=(1, 1), mult=np.full(oc, 1 << 30, np.int32),
+             shift=np.full(oc, 12, np.int8), out_zp=0, clamp=None)
+    got, st, want, wst = _fused(ctx, c)
+    assert ctx.last_kernel == "gemm_mfma_i8_rescale"
+    assert st == wst == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
+
+
+# ---- which MFMA kernel a convolution gets when the choice is left open ----
+@pytest.mark.parametrize("dtype, shape, kernel", [
+    # n, ih, iw, ic, oc, k, pad
+    (capi.INT8, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_i8"),          # 3x3 int8: the patch kernel
+    (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "conv2d_mfma_i8"),
+    (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
+    (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16"),        # 3x3 fp16, deep K
+    (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
+    (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "conv2d_mfma_f16"),        # pointwise the GEMM kernel refuses (K < 256 bytes)
+])
+def test_automatic_kernel_choice(dtype, shape, kernel):
+    n, ih, iw, ic, oc, k, pad = shape
+    rng = np.random.default_rng(ic + oc + k)
+    if dtype == capi.INT8:
+        x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+        w = rng.integers(-128, 128, (oc, k, k, ic)).astype(np.int8)
+        b = rng.integers(-999, 999, oc).astype(np.int32)
+    else:
+        x = rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float16)
+        w = rng.normal(0, 0.05, (oc, k, k, ic)).astype(np.float16)
+        b = rng.normal(0, 1, oc).astype(np.float16)
+    c = Context(0)
+    try:
+        got, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
+        assert st == capi.VALID and c.last_kernel == kernel
+        # the kernel not chosen, where it takes the shape at all
+        c.set_kernel_choice(capi.KERNEL_GEMM if kernel.startswith("conv2d") else capi.KERNEL_MFMA)
+        try:
+            other, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
+        except TmiError:
+            assert kernel.startswith("conv2d") and ic * 2 < 256
+            return
+        assert st == capi.VALID and c.last_kernel != kernel
+    finally:
+        c.close()
+    if dtype == capi.INT8:      # both kernels give the one exact result
+        assert np.array_equal(got, other)
+    else:                       # the same products in fp32, summed in a different order
+        assert np.allclose(got.astype(np.float32), other.astype(np.float32), rtol=2.0 ** -8, atol=2.0 ** -6)
