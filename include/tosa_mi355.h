@@ -52,6 +52,7 @@ enum
     TMI_INT8  = 3,
     TMI_INT16 = 4,
     TMI_INT32 = 5,
+    TMI_INT48 = 6, /* RESCALE input only; one int64 per element, as the reference stores it */
     TMI_FP32  = 7,
     TMI_FP16  = 8,
     TMI_BF16  = 9
@@ -208,7 +209,8 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
 
 /* OpRescale::eval, reference_model/src/ops/type_conversion.cpp:224-421, on a tensor of `rank` dimensions
  * viewed as [rows, C] (C = last dimension, or 1 for rank 0).  multiplier_dev holds INT32 (scale32) or
- * INT16 values, shift_dev INT8 values. */
+ * INT16 values, shift_dev INT8 values.  Input INT8 / INT16 / INT32 / INT48 (the instantiations at :874-903;
+ * INT48 needs scale32 = 0, :122), output INT8 / INT16 / INT32. */
 int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64_t rows, int32_t C,
                 const void* in_dev, const void* multiplier_dev, const void* shift_dev, void* out_dev);
 

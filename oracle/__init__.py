@@ -273,7 +273,7 @@ def apply_scale_16(value, multiplier, shift):
 
 
 _BITS = {np.dtype(np.int8): 8, np.dtype(np.uint8): 8, np.dtype(np.int16): 16, np.dtype(np.uint16): 16,
-         np.dtype(np.int32): 32}
+         np.dtype(np.int32): 32, np.dtype(np.int64): 48}     # int64 is the storage of INT48
 
 
 def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale32=True,
@@ -291,13 +291,14 @@ def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale3
     rank = inp.ndim
     C = inp.shape[-1] if rank > 0 else 1
     rows = int(np.prod(inp.shape[:-1], dtype=np.int64)) if rank > 0 else 1
-    stored = _c(inp.view(_signed(inp.dtype)) if inp.dtype.kind == "u" else inp, np.int32)
+    i48 = a.in_bits == 48
+    stored = _c(inp.view(_signed(inp.dtype)) if inp.dtype.kind == "u" else inp, np.int64 if i48 else np.int32)
     mult = _c(np.atleast_1d(multiplier), np.int32)
     sh = _c(np.atleast_1d(shift), np.int32)
     out = np.zeros(inp.shape, dtype=np.int32)
-    rc = lib().orc_rescale(ctypes.byref(a), ctypes.c_int64(rows), ctypes.c_int32(C), _ptr(stored), _ptr(mult),
-                           _ptr(sh), ctypes.c_int32(mult.size), ctypes.c_int32(sh.size), ctypes.c_int32(rank),
-                           _ptr(out))
+    fn = lib().orc_rescale_i48 if i48 else lib().orc_rescale
+    rc = fn(ctypes.byref(a), ctypes.c_int64(rows), ctypes.c_int32(C), _ptr(stored), _ptr(mult),
+            _ptr(sh), ctypes.c_int32(mult.size), ctypes.c_int32(sh.size), ctypes.c_int32(rank), _ptr(out))
     # narrow to the output dtype keeping the low bits (uint16 32832 is stored as such)
     narrowed = out.astype(np.int64).astype(_signed(out_dtype), casting="unsafe") if out_dtype.kind != "u" else \
         (out.astype(np.int64) & ((1 << (8 * out_dtype.itemsize)) - 1)).astype(out_dtype)
@@ -306,7 +307,7 @@ def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale3
 
 def _signed(dt):
     dt = np.dtype(dt)
-    return {1: np.int8, 2: np.int16, 4: np.int32}[dt.itemsize]
+    return {1: np.int8, 2: np.int16, 4: np.int32, 8: np.int64}[dt.itemsize]
 
 
 def clamp(inp, lo, hi, nan_mode=1):

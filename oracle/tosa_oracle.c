@@ -570,30 +570,36 @@ int32_t orc_apply_scale_16(int64_t value, int16_t multiplier, int32_t shift, int
 }
 
 /* value_extend64_impl (reference_model/src/ops/type_conversion.cpp:183-221) for 8/16/32-bit types. */
-static int64_t value_extend64(int32_t val, int bits, int is_unsigned)
+static int64_t value_extend64(int64_t val, int bits, int is_unsigned)
 {
     switch (bits)
     {
+        case 48: /* int64 storage; bit 47 set: bits 48..63 are set too (:200-215) */
+            if (is_unsigned)
+                return val & INT64_C(0x0000FFFFFFFFFFFF);
+            return (val & INT64_C(0x800000000000)) ? (int64_t)((uint64_t)val | UINT64_C(0xFFFF000000000000)) : val;
         case 8:
             return is_unsigned ? (int64_t)(uint8_t)(int8_t)val : (int64_t)(int8_t)(uint8_t)(val & 0xFF);
         case 16:
             return is_unsigned ? (int64_t)(uint16_t)(int16_t)val : (int64_t)(int16_t)(uint16_t)(val & 0xFFFF);
         case 32:
-            return is_unsigned ? (int64_t)(uint32_t)val : (int64_t)val;
+            return is_unsigned ? (int64_t)(uint32_t)(int32_t)val : (int64_t)(int32_t)val;
         default:
-            return (int64_t)val;
+            return val;
     }
 }
 
 /* ------------------------------------------------------------------------------------------------
  * OpRescale::checkTensorAttributes + eval (type_conversion.cpp:72-154, 224-421).
  * ---------------------------------------------------------------------------------------------- */
-int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
-                const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out)
+/* in32: the int32 storage of INT8 / INT16 / INT32 tensors; in64: the int64 storage of an INT48 tensor */
+static int rescale_impl(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in32, const int64_t* in64,
+                        const int32_t* multiplier, const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank,
+                        int32_t* out)
 {
-    const int i8in = a->in_bits == 8, i16in = a->in_bits == 16, i32in = a->in_bits == 32;
+    const int i8in = a->in_bits == 8, i16in = a->in_bits == 16, i32in = a->in_bits == 32, i48in = a->in_bits == 48;
     const int i8out = a->out_bits == 8, i16out = a->out_bits == 16, i32out = a->out_bits == 32;
-    if (!(i8in || i16in || i32in) || !(i8out || i16out || i32out))
+    if (!(i8in || i16in || i32in || i48in) || !(i8out || i16out || i32out) || (i48in ? !in64 : !in32))
         return ORC_ERROR;
 
     /* checkTensorAttributes :118-151 */
@@ -611,6 +617,9 @@ int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int3
     if (i32in && a->input_unsigned)
         return ORC_ERROR;
     if (i32out && a->output_unsigned)
+        return ORC_ERROR;
+    /* :122, :129, :132 */
+    if (i48in && (a->scale32 || a->output_unsigned || a->input_unsigned))
         return ORC_ERROR;
     if (a->per_channel)
     {
@@ -656,7 +665,8 @@ int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int3
         {
             const int32_t m  = a->per_channel ? multiplier[c] : multiplier[0];
             const int32_t sh = a->per_channel ? shift[c] : shift[0];
-            const int64_t v  = value_extend64(in[r * C + c], a->in_bits, a->input_unsigned) - in_zp_ext;
+            const int64_t st = i48in ? in64[r * C + c] : (int64_t)in32[r * C + c];
+            const int64_t v  = value_extend64(st, a->in_bits, a->input_unsigned) - in_zp_ext;
             int32_t scaled;
             if (!inexact)
             {
@@ -685,6 +695,22 @@ int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int3
             out[r * C + c]  = (int32_t)clipped;
         }
     return status;
+}
+
+int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
+                const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out)
+{
+    if (a->in_bits == 48)
+        return ORC_ERROR;
+    return rescale_impl(a, rows, C, in, NULL, multiplier, shift, n_mult, n_shift, rank, out);
+}
+
+int orc_rescale_i48(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int64_t* in, const int32_t* multiplier,
+                    const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out)
+{
+    if (a->in_bits != 48)
+        return ORC_ERROR;
+    return rescale_impl(a, rows, C, NULL, in, multiplier, shift, n_mult, n_shift, rank, out);
 }
 
 /* ------------------------------------------------------------------------------------------------

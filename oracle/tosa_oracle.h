@@ -151,7 +151,7 @@ int32_t orc_apply_scale_16(int64_t value, int16_t multiplier, int32_t shift, int
 
 typedef struct
 {
-    int32_t in_bits;  /* 8, 16 or 32: nominal width of the input dtype  */
+    int32_t in_bits;  /* 8, 16, 32 or 48: nominal width of the input dtype  */
     int32_t out_bits; /* 8, 16 or 32: nominal width of the output dtype */
     int32_t scale32;
     int32_t rounding_mode;
@@ -168,6 +168,11 @@ typedef struct
  * ORC_UNPREDICTABLE when a REQUIRE fires (output contents then unspecified), else ORC_VALID. */
 int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
                 const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out);
+/* The same for an INT48 input (in_bits = 48), whose storage type is int64 (template_types.h:67-163); a stored
+ * value with bit 47 set gets bits 48..63 set (value_extend64_impl, type_conversion.cpp:200-215), which changes
+ * nothing for values inside the 48-bit range.  Needs scale32 = 0, hence apply_scale_16 (:122). */
+int orc_rescale_i48(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int64_t* in, const int32_t* multiplier,
+                    const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out);
 
 /* CLAMP for the integer instantiations: min(max(x, lo), hi); ORC_ERROR when hi < lo. */
 /* AVG_POOL2D / MAX_POOL2D (reference_model/src/ops/tensor_ops.cpp:29-117 check_pool2d_attribute, :472-660

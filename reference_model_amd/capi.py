@@ -15,15 +15,16 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libtosa_mi355.so")
 
 VALID, UNPREDICTABLE, ERROR = 0, 1, 2
-INT8, INT16, INT32, FP32, FP16, BF16 = 3, 4, 5, 7, 8, 9
+INT8, INT16, INT32, INT48, FP32, FP16, BF16 = 3, 4, 5, 6, 7, 8, 9
 ROUND_SINGLE, ROUND_INEXACT, ROUND_DOUBLE = 1, 2, 3
 FLAG_SCALE_MULTIPLIER, FLAG_SCALE_SHIFT, FLAG_SCALE_VALUE, FLAG_SCALE_RESULT, FLAG_ZP_RESULT = 1, 2, 4, 8, 16
 KERNEL_AUTO, KERNEL_DIRECT, KERNEL_MFMA, KERNEL_GEMM = 0, 1, 2, 3
 
 F64 = -64  # host-side tag of the fp64 buffers of the precise / bounds passes (not a TOSA element type)
-DTYPE_SIZE = {INT8: 1, INT16: 2, INT32: 4, FP32: 4, FP16: 2, BF16: 2, F64: 8}
+DTYPE_SIZE = {INT8: 1, INT16: 2, INT32: 4, INT48: 8, FP32: 4, FP16: 2, BF16: 2, F64: 8}
 _NP_TO_TMI = {np.dtype(np.int8): INT8, np.dtype(np.uint8): INT8, np.dtype(np.int16): INT16,
-              np.dtype(np.uint16): INT16, np.dtype(np.int32): INT32, np.dtype(np.float32): FP32,
+              np.dtype(np.uint16): INT16, np.dtype(np.int32): INT32, np.dtype(np.int64): INT48,
+              np.dtype(np.float32): FP32,
               np.dtype(np.float16): FP16}
 
 EXPORTS = [

@@ -1,6 +1,6 @@
 // RESCALE and CLAMP as stand-alone bandwidth kernels.
 //
-// RESCALE reads 1/2/4 bytes and writes 1/2/4 bytes per element and does ~20 integer instructions per
+// RESCALE reads 1/2/4/8 bytes and writes 1/2/4 bytes per element and does ~20 integer instructions per
 // element, so it is bound by HBM.  Each lane handles VEC consecutive elements of one row with a single
 // vector load and a single vector store; the per-channel constants come from the L1/L2-resident
 // multiplier and shift arrays.
@@ -33,7 +33,7 @@ __global__ __launch_bounds__(256) void rescale_vec_kernel(RescaleParams p, const
         {
             const int32_t m = load_multiplier(p, c0 + j);
             const int32_t s = load_shift(p, c0 + j);
-            r.v[j]          = (OutT)rescale_value(p, (int32_t)a.v[j], m, s, flags);
+            r.v[j]          = (OutT)rescale_value(p, a.v[j], m, s, flags);
         }
         reinterpret_cast<Pack<OutT, VEC>*>(out)[i] = r;
     }
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, co
         const int c     = (int)(i % C);
         const int32_t m = load_multiplier(p, c);
         const int32_t s = load_shift(p, c);
-        out[i]          = (OutT)rescale_value(p, (int32_t)in[i], m, s, flags);
+        out[i]          = (OutT)rescale_value(p, in[i], m, s, flags);
     }
     raise_flags(flag_word, flags);
 }
@@ -215,6 +215,9 @@ const char* launch_rescale(hipStream_t st, const RescaleParams& p, int32_t in_dt
     TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT8, int8_t)
     TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT16, int16_t)
     TMI_RESCALE_CASE(TMI_INT32, int32_t, TMI_INT32, int32_t)
+    TMI_RESCALE_CASE(TMI_INT48, int64_t, TMI_INT8, int8_t)
+    TMI_RESCALE_CASE(TMI_INT48, int64_t, TMI_INT16, int16_t)
+    TMI_RESCALE_CASE(TMI_INT48, int64_t, TMI_INT32, int32_t)
 #undef TMI_RESCALE_CASE
     return nullptr;
 }

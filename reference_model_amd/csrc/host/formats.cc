@@ -34,6 +34,8 @@ size_t dtype_size(DType t)
         case DType_INT32:
         case DType_FP32:
             return 4;
+        case DType_INT48:
+            return 8;    // one int64 per element in memory and in .npy files; 6 bytes in a .tosa payload
         default:
             return 0;
     }
@@ -314,6 +316,8 @@ const char* npy_descr_for(DType t)
             return "<i2";
         case DType_INT32:
             return "<i4";
+        case DType_INT48:
+            return "<i8";
         case DType_FP16:
             return "<f2";
         case DType_FP32:

@@ -5,7 +5,14 @@
 // interprets (verif/runner/tosa_refmodel_sut_run.py:12-18,59-68).
 //
 //   tosa_mi355_run --test_desc=<dir>/desc.json [--ofm_file=<name>] [--flatbuffer_dir=<dir>] [--no_fusion]
+//                  [--precise_mode=1]
+//
+// --precise_mode=1 (reference_model/src/command_line_utils.h:65): floating-point CONV2D / DEPTHWISE_CONV2D /
+// MATMUL results are computed and written in fp64; when the descriptor says
+// test_requirements.bounds_file_required, the graph is evaluated a second time in bounds mode and those results
+// go to "bounds_" + ofm_file (reference_model/src/main.cpp:109-121, :246-251, :404-407).
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <sstream>
@@ -22,6 +29,7 @@ struct Desc
 {
     std::string tosa_file;
     std::vector<std::string> ifm_name, ifm_file, ofm_name, ofm_file;
+    bool bounds_file_required = false;    // test_requirements.bounds_file_required
 };
 
 bool parse_string(const std::string& s, size_t& i, std::string& out)
@@ -92,9 +100,16 @@ bool parse_desc(const std::string& text, Desc& d)
                 return false;
             values.push_back(v);
         }
+        else if (i < text.size() && text[i] == '{')
+            continue;    // a nested object: its keys are read like top-level ones
         else
+        {
+            const size_t v0 = i;
             while (i < text.size() && text[i] != ',' && text[i] != '}')
                 i++;
+            if (key == "bounds_file_required")
+                d.bounds_file_required = text.compare(v0, 4, "true") == 0;
+        }
         if (key == "tosa_file" && !values.empty())
             d.tosa_file = values[0];
         else if (key == "ifm_name")
@@ -126,7 +141,7 @@ int fail(const char* what, const std::string& msg)
 int main(int argc, char** argv)
 {
     std::string test_desc, ofm_override, fb_dir;
-    bool fusion = true;
+    bool fusion = true, precise = false;
     for (int a = 1; a < argc; a++)
     {
         const std::string s = argv[a];
@@ -142,6 +157,8 @@ int main(int argc, char** argv)
             fb_dir = v;
         else if (s == "--no_fusion")
             fusion = false;
+        else if (const char* v = val("--precise_mode="))
+            precise = atoi(v) != 0;
         else
             return fail("unknown argument", s);
     }
@@ -165,51 +182,69 @@ int main(int argc, char** argv)
     if (!load_tosa_file(fb_dir + "/" + desc.tosa_file, block, err))
         return fail("graph", err);
 
-    ModelRunner runner(0);
-    if (!fusion)
-        runner.disableFusion();
-    GraphStatus st = runner.initialize(block);
-    if (st != GraphStatus::TOSA_VALID)
+    // at most two runs; the second one only in precise mode, for the bounds results (reference: main.cpp:123-254)
+    GraphStatus st = GraphStatus::TOSA_VALID;
+    int kernels = 0, folded = 0;
+    std::string message;
+    for (int run = 0; run < (precise && desc.bounds_file_required ? 2 : 1); run++)
     {
-        fprintf(stderr, "Graph result: ERROR (%s)\n", runner.traverser() ? runner.traverser()->last_message.c_str() : "");
-        return (int)st;
-    }
-    for (size_t i = 0; i < desc.ifm_name.size(); i++)
-    {
-        NpyArray arr;
-        if (!read_npy(fb_dir + "/" + desc.ifm_file[i], arr, err))
-            return fail("input", err);
-        Tensor* t = runner.traverser()->findTensorByName(desc.ifm_name[i]);
-        if (!t)
-            return fail("input", "no tensor named " + desc.ifm_name[i]);
-        if (arr.descr != npy_descr_for(t->getDtype()) && !(arr.descr == "<i1" && t->getDtype() == DType_INT8))
-            return fail("input", desc.ifm_file[i] + ": descr " + arr.descr + " does not match the tensor type");
-        if (arr.shape != t->getShape() || arr.data.size() < t->bytes())
-            return fail("input", desc.ifm_file[i] + ": shape does not match tensor " + desc.ifm_name[i]);
-        if (runner.setInput(desc.ifm_name[i], arr.data.data(), t->bytes()))
-            return fail("input", "setInput failed for " + desc.ifm_name[i]);
-    }
-    st = runner.run();
-    SubgraphTraverser* sgt = runner.traverser();
-    if (st == GraphStatus::TOSA_ERROR)
-    {
-        fprintf(stderr, "Graph result: ERROR (%s)\n", sgt->last_message.c_str());
-        return (int)st;
-    }
-    for (size_t i = 0; i < desc.ofm_name.size(); i++)
-    {
-        Tensor* t = sgt->findTensorByName(desc.ofm_name[i]);
-        if (!t || !t->host_valid)
-            return fail("output", "no result for " + desc.ofm_name[i]);
-        std::string name = (i == 0 && !ofm_override.empty()) ? ofm_override : desc.ofm_file[i];
-        if (name.empty() || name[0] != '/')
-            name = fb_dir + "/" + name;
-        if (!write_npy(name, npy_descr_for(t->getDtype()), t->getShape(), t->host.data(), t->bytes(), err))
-            return fail("output", err);
+        ModelRunner runner(0);
+        if (!fusion)
+            runner.disableFusion();
+        runner.setPreciseMode(precise, run == 1);
+        st = runner.initialize(block);
+        if (st != GraphStatus::TOSA_VALID)
+        {
+            fprintf(stderr, "Graph result: ERROR (%s)\n", runner.traverser() ? runner.traverser()->last_message.c_str() : "");
+            return (int)st;
+        }
+        for (size_t i = 0; i < desc.ifm_name.size(); i++)
+        {
+            NpyArray arr;
+            if (!read_npy(fb_dir + "/" + desc.ifm_file[i], arr, err))
+                return fail("input", err);
+            Tensor* t = runner.traverser()->findTensorByName(desc.ifm_name[i]);
+            if (!t)
+                return fail("input", "no tensor named " + desc.ifm_name[i]);
+            if (arr.descr != npy_descr_for(t->getDtype()) && !(arr.descr == "<i1" && t->getDtype() == DType_INT8))
+                return fail("input", desc.ifm_file[i] + ": descr " + arr.descr + " does not match the tensor type");
+            if (arr.shape != t->getShape() || arr.data.size() < t->bytes())
+                return fail("input", desc.ifm_file[i] + ": shape does not match tensor " + desc.ifm_name[i]);
+            if (runner.setInput(desc.ifm_name[i], arr.data.data(), t->bytes()))
+                return fail("input", "setInput failed for " + desc.ifm_name[i]);
+        }
+        st = runner.run();
+        SubgraphTraverser* sgt = runner.traverser();
+        if (st == GraphStatus::TOSA_ERROR)
+        {
+            fprintf(stderr, "Graph result: ERROR (%s)\n", sgt->last_message.c_str());
+            return (int)st;
+        }
+        for (size_t i = 0; i < desc.ofm_name.size(); i++)
+        {
+            Tensor* t = sgt->findTensorByName(desc.ofm_name[i]);
+            if (!t || !t->host_valid)
+                return fail("output", "no result for " + desc.ofm_name[i]);
+            std::string name = (i == 0 && !ofm_override.empty()) ? ofm_override : desc.ofm_file[i];
+            if (run == 1)
+            {
+                const size_t k = name.find_last_of('/');
+                name.insert(k == std::string::npos ? 0 : k + 1, "bounds_");
+            }
+            if (name.empty() || name[0] != '/')
+                name = fb_dir + "/" + name;
+            if (!write_npy(name, t->precise ? "<f8" : npy_descr_for(t->getDtype()), t->getShape(), t->host.data(),
+                           t->bytes(), err))
+                return fail("output", err);
+        }
+        kernels += sgt->kernels_launched, folded += sgt->nodes_folded;
+        message = sgt->last_message;
+        if (st != GraphStatus::TOSA_VALID)
+            break;    // the bounds run only follows a valid first run
     }
     fprintf(stderr, "Graph result: %s (kernels launched: %d, nodes folded into a producer: %d)\n",
-            st == GraphStatus::TOSA_VALID ? "VALID" : "UNPREDICTABLE", sgt->kernels_launched, sgt->nodes_folded);
+            st == GraphStatus::TOSA_VALID ? "VALID" : "UNPREDICTABLE", kernels, folded);
     if (st != GraphStatus::TOSA_VALID)
-        fprintf(stderr, "%s\n", sgt->last_message.c_str());
+        fprintf(stderr, "%s\n", message.c_str());
     return (int)st;
 }

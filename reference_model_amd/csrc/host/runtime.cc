@@ -38,6 +38,13 @@ bool Tensor::scalar_value(int32_t& v) const
         case DType_INT32:
             memcpy(&v, host.data(), 4);
             return true;
+        case DType_INT48:
+        {
+            int64_t t;
+            memcpy(&t, host.data(), 8);
+            v = t < INT32_MIN ? INT32_MIN : (t > INT32_MAX ? INT32_MAX : (int32_t)t);    // only 0 is a legal INT48 zero point
+            return true;
+        }
         case DType_FP16:
         case DType_BF16:
         {
@@ -120,6 +127,8 @@ int32_t tmi_dtype(DType t)
             return TMI_INT16;
         case DType_INT32:
             return TMI_INT32;
+        case DType_INT48:
+            return TMI_INT48;
         case DType_FP32:
             return TMI_FP32;
         case DType_FP16:
@@ -352,6 +361,16 @@ int ConvBase::eval()
     if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
         return error("zero-point operands must be available on the host");
     SubgraphTraverser* s = parent_sgt;
+    if (s->precise_mode && inputs[0]->getDtype() != DType_INT8)
+    {
+        // precise mode (tensor_ops.cpp:790-802, :1245-1257): fp64 accumulation, fp64 result
+        outputs[0]->precise = true;
+        auto fn             = depthwise ? tmi_depthwise_conv2d_precise : tmi_conv2d_precise;
+        if (call(fn(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]), s->bounds_mode ? 1 : 0,
+                    static_cast<double*>(s->device_out(outputs[0])))))
+            return 1;
+        return GraphNode::eval();
+    }
     if (!fused_rescale)
     {
         auto fn = depthwise ? tmi_depthwise_conv2d : tmi_conv2d;
@@ -642,6 +661,16 @@ public:
             return error("zero-point operands must be available on the host");
         const Tensor *a = inputs[0], *b = inputs[1];
         SubgraphTraverser* s = parent_sgt;
+        if (s->precise_mode && a->getDtype() != DType_INT8)
+        {
+            // precise mode (tensor_ops.cpp:1436-1443)
+            outputs[0]->precise = true;
+            if (call(tmi_matmul_precise(s->ctx, tmi_dtype(a->getDtype()), a->shape[0], a->shape[1], a->shape[2],
+                                        b->shape[2], s->device(inputs[0]), s->device(inputs[1]), s->bounds_mode ? 1 : 0,
+                                        static_cast<double*>(s->device_out(outputs[0])))))
+                return 1;
+            return GraphNode::eval();
+        }
         if (call(tmi_matmul(s->ctx, tmi_dtype(a->getDtype()), a->shape[0], a->shape[1], a->shape[2], b->shape[2],
                             s->device(inputs[0]), s->device(inputs[1]), a_zp, b_zp, s->device_out(outputs[0]))))
             return 1;
@@ -711,13 +740,31 @@ int SubgraphTraverser::initializeGraph()
         by_name[d.name] = t;
         if (!d.data.empty())
         {
-            if (d.data.size() < t->bytes())
+            // an INT48 element takes 6 bytes in the serialized payload and one int64 in memory
+            // (reference: subgraph_traverser.cpp:652-656, ConvertU8toI48)
+            const bool i48      = d.dtype == DType_INT48;
+            const size_t stored = i48 ? (size_t)t->getElementCount() * 6 : t->bytes();
+            if (d.data.size() < stored)
             {
                 last_message = "tensor " + d.name + ": constant payload shorter than the tensor";
                 setGraphStatus(GraphStatus::TOSA_ERROR);
                 return 1;
             }
-            t->host.assign(d.data.begin(), d.data.begin() + (std::ptrdiff_t)t->bytes());
+            if (i48)
+            {
+                t->host.resize(t->bytes());
+                for (size_t e = 0; e < (size_t)t->getElementCount(); e++)
+                {
+                    uint64_t v = 0;
+                    for (int b = 0; b < 6; b++)
+                        v |= (uint64_t)d.data[e * 6 + b] << (8 * b);
+                    if (v & 0x800000000000ull)
+                        v |= 0xFFFF000000000000ull;
+                    memcpy(t->host.data() + e * 8, &v, 8);
+                }
+            }
+            else
+                t->host.assign(d.data.begin(), d.data.begin() + (std::ptrdiff_t)t->bytes());
             t->host_valid = true;
             t->is_const   = true;
         }
@@ -939,6 +986,16 @@ int SubgraphTraverser::evaluateAll()
             }
             if (!ready)
                 continue;
+            // the fp64 passes take operands in their storage type: a chain of floating-point operators in
+            // precise mode is outside this path
+            for (Tensor* t : n->inputs)
+                if (t->precise)
+                {
+                    last_message = std::string(op_name(n->nodeType)) + ": operand " + t->name +
+                                   " is an fp64 precise-mode result; only graph inputs and constants are taken";
+                    setGraphStatus(GraphStatus::TOSA_ERROR);
+                    return 1;
+                }
             if (n->eval())
                 return 1;
             done[i]  = true;
@@ -994,6 +1051,8 @@ GraphStatus ModelRunner::initialize(const BasicBlock& block)
 {
     sgt.reset(new SubgraphTraverser(block, device_id));
     sgt->enable_fusion = fusion;
+    sgt->precise_mode  = precise_mode;
+    sgt->bounds_mode   = bounds_mode;
     if (sgt->initializeGraph() || sgt->linkTensorsAndNodes() || sgt->validateGraph())
         return sgt->getGraphStatus() == GraphStatus::TOSA_VALID ? GraphStatus::TOSA_ERROR : sgt->getGraphStatus();
     return sgt->getGraphStatus();

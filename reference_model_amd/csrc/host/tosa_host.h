@@ -135,7 +135,8 @@ public:
     int getRank() const { return (int)shape.size(); }
     DType getDtype() const { return dtype; }
     int64_t getElementCount() const;
-    size_t bytes() const { return (size_t)getElementCount() * dtype_size(dtype); }
+    // a precise-mode result is held as fp64 whatever the serialized element type says
+    size_t bytes() const { return (size_t)getElementCount() * (precise ? 8 : dtype_size(dtype)); }
 
     std::string name;
     std::vector<int32_t> shape;
@@ -146,6 +147,7 @@ public:
     bool dev_valid     = false;
     bool is_const      = false;
     bool is_graph_io   = false;
+    bool precise       = false;    // written by the fp64 precise / bounds pass of a floating-point operator
     GraphNode* producer = nullptr;
     std::vector<GraphNode*> consumers;
 
@@ -200,6 +202,9 @@ public:
     int download(Tensor* t);         // device -> host bytes
     std::string last_message;
     bool enable_fusion = true;
+    // g_func_config.precise_mode / bounds_mode of the reference (include/func_config.h:60-61): floating-point
+    // CONV2D / DEPTHWISE_CONV2D / MATMUL accumulate in fp64 (bounds mode: over absolute values) and write fp64
+    bool precise_mode = false, bounds_mode = false;
     int kernels_launched = 0, nodes_folded = 0;
 
 private:
@@ -222,10 +227,11 @@ public:
     int getOutput(const std::string& name, uint8_t* raw, size_t size);
     SubgraphTraverser* traverser() { return sgt.get(); }
     void disableFusion() { fusion = false; }
+    void setPreciseMode(bool precise, bool bounds) { precise_mode = precise, bounds_mode = bounds; }
 
 private:
     int device_id;
-    bool fusion = true;
+    bool fusion = true, precise_mode = false, bounds_mode = false;
     std::unique_ptr<SubgraphTraverser> sgt;
 };
 

@@ -93,6 +93,8 @@ int dtype_bits(int32_t dt)
         case TMI_INT32:
         case TMI_FP32:
             return 32;
+        case TMI_INT48:
+            return 48;
         default:
             return 0;
     }
@@ -194,7 +196,8 @@ int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, in
 {
     if (!r)
         return fail(ctx, "OpRescale: null descriptor");
-    if (!is_int_dtype(r->in_dtype) || !is_int_dtype(r->out_dtype))
+    const bool i48in = r->in_dtype == TMI_INT48;
+    if ((!is_int_dtype(r->in_dtype) && !i48in) || !is_int_dtype(r->out_dtype))
         return fail(ctx, "OpRescale: unsupported data type");
     const bool i32in = r->in_dtype == TMI_INT32, i32out = r->out_dtype == TMI_INT32;
     const bool i8in = r->in_dtype == TMI_INT8, i8out = r->out_dtype == TMI_INT8;
@@ -216,6 +219,12 @@ int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, in
         return fail(ctx, "OpRescale: Input unsigned int32");
     if (i32out && out_u)
         return fail(ctx, "OpRescale: Output unsigned int32");
+    if (r->scale32 && i48in)
+        return fail(ctx, "OpRescale: Scale set to true but input type is INT48");
+    if (i48in && out_u)
+        return fail(ctx, "OpRescale: Input signed int48 and output_unsigned set to true");
+    if (i48in && in_u)
+        return fail(ctx, "OpRescale: Input unsigned int48");
     if (r->per_channel)
     {
         if (rank < 1)

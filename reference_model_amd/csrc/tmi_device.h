@@ -56,14 +56,17 @@ struct ChannelScale
     uint32_t lim, lim2;          // value v is legal iff (uint32)(v + lim) <= lim2
 };
 
-// value_extend64_impl of the reference (type_conversion.cpp:183-221) for 8/16/32-bit storage.
-__device__ __forceinline__ int64_t value_extend(int32_t v, int bits, bool is_unsigned)
+// value_extend64_impl of the reference (type_conversion.cpp:183-221); INT48 is stored as int64 and never
+// unsigned here (the host rejects it, :132).
+__device__ __forceinline__ int64_t value_extend(int64_t v, int bits, bool is_unsigned)
 {
+    if (bits == 48)
+        return (v & 0x800000000000ll) ? (int64_t)((uint64_t)v | 0xFFFF000000000000ull) : v;
     if (bits == 8)
         return is_unsigned ? (int64_t)(uint8_t)v : (int64_t)(int8_t)v;
     if (bits == 16)
         return is_unsigned ? (int64_t)(uint16_t)v : (int64_t)(int16_t)v;
-    return is_unsigned ? (int64_t)(uint32_t)v : (int64_t)v;
+    return is_unsigned ? (int64_t)(uint32_t)v : (int64_t)(int32_t)v;
 }
 
 // QuantUtil::apply_scale_32 (quant_util.h:45-84).  Violated preconditions set bits in `flags`.
@@ -112,7 +115,7 @@ __device__ __forceinline__ int32_t apply_scale_16(int64_t value, int32_t multipl
 
 // The rescale_func lambda of OpRescale::eval (type_conversion.cpp:305-370) followed by the optional
 // CLAMP (arith_util.h:389-413).  `stored` is the raw stored input value, `m`/`s` the channel's constants.
-__device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int32_t stored, int32_t m, int32_t s,
+__device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t stored, int32_t m, int32_t s,
                                                  uint32_t& flags)
 {
     const int64_t v = value_extend(stored, p.in_bits, p.in_unsigned) - (int64_t)p.in_zp;

@@ -122,6 +122,43 @@ def test_rescale_require_conditions_raise_unpredictable(ctx):
         assert (st, wst) == (capi.UNPREDICTABLE, oracle.UNPREDICTABLE) and ctx.flags & flag, (mult, shift)
 
 
+@pytest.mark.parametrize("out_dt", [np.int8, np.int16, np.int32])
+@pytest.mark.parametrize("shape", [(7, 9, 12), (5, 13), (1 << 16, 8)])      # vector path, scalar path, a larger tensor
+@pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_INEXACT])
+def test_rescale_int48_input(ctx, out_dt, shape, mode):
+    """INT48 (int64 storage), 16-bit multipliers: apply_scale_16 on the 64-bit value (type_conversion.cpp:122,
+    :200-215, quant_util.h:86-108)"""
+    rng = np.random.default_rng(shape[-1] + 48)
+    C = shape[-1]
+    x = rng.integers(-(1 << 47), 1 << 47, shape).astype(np.int64)
+    x.ravel()[:5] = [(1 << 47) - 1, -(1 << 47), 0, -1, 1]
+    mult = rng.integers(1, 1 << 15, C)
+    shift = rng.integers(40, 63, C)
+    if mode == capi.ROUND_INEXACT:      # fp32 arithmetic: keep the scaled values where the cast to int32 is defined
+        shift = rng.integers(50, 63, C)
+    kw = dict(out_dtype=out_dt, scale32=False, rounding_mode=mode)
+    want, wst = oracle.rescale(x, mult, shift, **kw)
+    got, st = gpu_ops.rescale(ctx, x, mult, shift, **kw)
+    assert st == wst == capi.VALID, ctx.flags
+    assert np.array_equal(got, want) and len(np.unique(got)) > 10
+
+
+def test_rescale_int48_checks(ctx):
+    x = np.array([1, 2, (1 << 47) - 1], np.int64)
+    kw = dict(per_channel=False, rounding_mode=capi.ROUND_SINGLE, out_dtype=np.int16)
+    for bad in (dict(scale32=True), dict(scale32=False, input_unsigned=True), dict(scale32=False, in_zp=3)):
+        with pytest.raises(TmiError) as e:
+            gpu_ops.rescale(ctx, x, [1 << 14], [40], **{**kw, **bad})
+        assert e.value.status == capi.ERROR and "OpRescale" in e.value.message
+    with pytest.raises(TmiError):
+        gpu_ops.rescale(ctx, x, [1 << 14], [40], scale32=False, output_unsigned=True, per_channel=False,
+                        rounding_mode=capi.ROUND_SINGLE, out_dtype=np.uint16)
+    # a scaled value beyond int32 is a REQUIRE failure (quant_util.h:102-106)
+    _, st = gpu_ops.rescale(ctx, x, [(1 << 15) - 1], [20], scale32=False, **{**kw, "out_dtype": np.int32})
+    _, wst = oracle.rescale(x, [(1 << 15) - 1], [20], scale32=False, **{**kw, "out_dtype": np.int32})
+    assert (st, wst) == (capi.UNPREDICTABLE, oracle.UNPREDICTABLE) and ctx.flags & capi.FLAG_SCALE_RESULT
+
+
 def test_clamp(ctx):
     x = np.arange(-128, 128).astype(np.int8)
     got, st = gpu_ops.clamp(ctx, np.tile(x, 33)[:8000], 0, 127)

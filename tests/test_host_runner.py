@@ -265,3 +265,93 @@ def test_pooling_graph(tmp_path):
     d2.mkdir()
     r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["ap"]), {"x": x}, ["ap"]))
     assert r.returncode == 2 and "exact integer output dimensions" in r.stderr
+
+
+@pytest.mark.gpu
+def test_int48_rescale_graph(tmp_path):
+    """RESCALE of an INT48 tensor (the accumulator type of 16-bit convolutions): the graph input arrives as an
+    int64 .npy file, a constant INT48 operand as 6 bytes per element (reference: subgraph_traverser.cpp:652-656)"""
+    rng = np.random.default_rng(6)
+    x = rng.integers(-(1 << 47), 1 << 47, (3, 5, 8)).astype(np.int64)
+    k = rng.integers(-(1 << 47), 1 << 47, (3, 5, 8)).astype(np.int64)
+    k.ravel()[:3] = [-(1 << 47), (1 << 47) - 1, -1]
+    mult = rng.integers(1, 1 << 15, 8).astype(np.int16)
+    shift = rng.integers(40, 63, 8).astype(np.int8)
+    kw = dict(out_dtype=np.int16, scale32=False, rounding_mode=oracle.ROUND_SINGLE)
+    (want_x, st1), (want_k, st2) = oracle.rescale(x, mult, shift, **kw), oracle.rescale(k, mult, shift, **kw)
+    assert st1 == st2 == oracle.VALID
+    ts = [W.tensor("x", x.shape, np.int64), W.tensor("k", k.shape, np.int64, k), W.tensor("mult", [8], np.int16, mult),
+          W.tensor("shift", [8], np.int8, shift), W.tensor("izp", [1], np.int64, [0]), W.tensor("ozp", [1], np.int16, [0]),
+          W.tensor("yx", x.shape, np.int16), W.tensor("yk", k.shape, np.int16)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("k", "mult", "shift", "izp", "ozp")]
+    attr = dict(scale32=False, rounding_mode=1)
+    ops.append(W.operator(R.OP_RESCALE, ["x", "mult", "shift", "izp", "ozp"], ["yx"], W.rescale_attr(**attr)))
+    ops.append(W.operator(R.OP_RESCALE, ["k", "mult", "shift", "izp", "ozp"], ["yk"], W.rescale_attr(**attr)))
+    r = _run(_write_case(tmp_path, W.graph(ts, ops, ["x"], ["yx", "yk"]), {"x": x}, ["yx", "yk"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(tmp_path / "yx_out.npy"), want_x)
+    assert np.array_equal(np.load(tmp_path / "yk_out.npy"), want_k)
+    # scale32 with an INT48 input is rejected when the graph is validated (type_conversion.cpp:122)
+    ts[2] = W.tensor("mult", [8], np.int32, mult.astype(np.int32))
+    ops[-2] = W.operator(R.OP_RESCALE, ["x", "mult", "shift", "izp", "ozp"], ["yx"], W.rescale_attr(scale32=True, rounding_mode=1))
+    d2 = tmp_path / "bad"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops[:-1], ["x"], ["yx"]), {"x": x}, ["yx"]))
+    assert r.returncode == 2 and "INT48" in r.stderr
+
+
+@pytest.mark.gpu
+def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
+    """--precise_mode=1 on a compliance-style descriptor (test_requirements.bounds_file_required): the fp16 CONV2D is
+    evaluated in fp64, then once more over absolute values into bounds_<ofm_file> (reference: main.cpp:109-121,
+    :246-251, :404-407); both files equal the fp64 oracle bit for bit.  MATMUL likewise."""
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 1, (2, 9, 8, 24)).astype(np.float16)
+    w = rng.normal(0, 0.2, (10, 3, 3, 24)).astype(np.float16)
+    b = rng.normal(0, 1, 10).astype(np.float16)
+    pad, stride, dil = (1, 1, 1, 1), (1, 1), (1, 1)
+    xf, wf, bf = (v.astype(np.float64) for v in (x, w, b))
+    ref = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil)
+    bnd = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True)
+    ts = [W.tensor("x", x.shape, np.float16), W.tensor("w", w.shape, np.float16, w), W.tensor("b", [10], np.float16, b),
+          W.tensor("z", [1], np.float16, [0]), W.tensor("y", ref.shape, np.float16)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "b", "z")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "b", "z", "z"], ["y"], W.conv_attr(pad, stride, dil, acc_type=7)))
+    d1 = tmp_path / "conv"
+    d1.mkdir()
+    desc = _write_case(d1, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"])
+    meta = json.loads(open(desc).read())
+    meta["test_requirements"] = {"bounds_file_required": True}
+    open(desc, "w").write(json.dumps(meta))
+    r = _run(desc, "--precise_mode=1")
+    assert r.returncode == 0, r.stderr
+    got, got_bnd = np.load(d1 / "y_out.npy"), np.load(d1 / "bounds_y_out.npy")
+    assert got.dtype == got_bnd.dtype == np.float64
+    assert np.array_equal(got, ref) and np.array_equal(got_bnd, bnd)
+    # without the option the result has the graph's element type and no bounds file appears
+    d2 = tmp_path / "plain"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"]))
+    assert r.returncode == 0 and np.load(d2 / "y_out.npy").dtype == np.float16 and not (d2 / "bounds_y_out.npy").exists()
+    # precise mode without the requirement: one run
+    d3 = tmp_path / "nobounds"
+    d3.mkdir()
+    r = _run(_write_case(d3, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"]), "--precise_mode=1")
+    assert r.returncode == 0 and np.array_equal(np.load(d3 / "y_out.npy"), ref) and not (d3 / "bounds_y_out.npy").exists()
+
+    a = rng.normal(0, 1, (2, 5, 40)).astype(np.float16)
+    bb = rng.normal(0, 1, (2, 40, 7)).astype(np.float16)
+    ts = [W.tensor("a", a.shape, np.float16), W.tensor("b", bb.shape, np.float16), W.tensor("z", [1], np.float16, [0]),
+          W.tensor("o", [2, 5, 7], np.float32)]
+    ops = [W.operator(R.OP_CONST, [], ["z"]), W.operator(R.OP_MATMUL, ["a", "b", "z", "z"], ["o"])]
+    d4 = tmp_path / "matmul"
+    d4.mkdir()
+    desc = _write_case(d4, W.graph(ts, ops, ["a", "b"], ["o"]), {"a": a, "b": bb}, ["o"])
+    meta = json.loads(open(desc).read())
+    meta["test_requirements"] = {"bounds_file_required": True}
+    open(desc, "w").write(json.dumps(meta))
+    r = _run(desc, "--precise_mode=1")
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d4 / "o_out.npy"), oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64)))
+    assert np.array_equal(np.load(d4 / "bounds_o_out.npy"),
+                          oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64), abs_mode=True))

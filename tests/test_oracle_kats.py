@@ -228,6 +228,53 @@ def test_rescale_unsigned_input_and_rank0():
     assert st == oracle.VALID and out.shape == () and int(out) == 72
 
 
+def test_rescale_int48_vs_bigint():
+    """INT48 input: int64 storage, 16-bit multipliers, apply_scale_16 (quant_util.h:86-108): with Python's
+    unbounded integers ((v * m + 2^(s-1)) >> s), results beyond int32 being REQUIRE failures"""
+    rng = np.random.default_rng(48)
+    C = 5
+    x = rng.integers(-(1 << 47), 1 << 47, (4, 6, C)).astype(np.int64)
+    x[0, 0, :] = [(1 << 47) - 1, -(1 << 47), 0, -1, 1]                 # the extremes of the type
+    mult = rng.integers(1, 1 << 15, C)
+    shift = rng.integers(40, 63, C)
+    for out_dtype, lo, hi in ((np.int8, -128, 127), (np.int16, -32768, 32767), (np.int32, -(1 << 31), (1 << 31) - 1)):
+        out, st = oracle.rescale(x, mult, shift, out_dtype=out_dtype, scale32=False, rounding_mode=oracle.ROUND_SINGLE)
+        want = np.empty(x.shape, np.int64)
+        for idx in np.ndindex(x.shape):
+            c = idx[-1]
+            r = (int(x[idx]) * int(mult[c]) + (1 << (int(shift[c]) - 1))) >> int(shift[c])
+            assert -(1 << 31) <= r < (1 << 31)
+            want[idx] = min(hi, max(lo, r))
+        assert st == oracle.VALID and np.array_equal(out, want.astype(out_dtype))
+    assert len(np.unique(out)) > 40
+
+
+def test_rescale_int48_boundary_operands():
+    """rescaleTestVals (generate_int_special.cpp:119-131) for INT48: value x multiplier x shift extremes"""
+    lowest, top, mmax = -(1 << 47), (1 << 47) - 1, (1 << 15) - 1
+    for v, m, s in [(-2, 0, 2), (-2, mmax, 2), (1, 0, 2), (1, mmax, 2), (lowest, 0, 62), (lowest, mmax, 62),
+                    (top, 0, 62), (top, mmax, 62)]:
+        out, st = oracle.rescale(np.array([v], np.int64), [m], [s], out_dtype=np.int32, scale32=False,
+                                 rounding_mode=oracle.ROUND_SINGLE, per_channel=False)
+        assert st == oracle.VALID and int(out[0]) == (v * m + (1 << (s - 1))) >> s, (v, m, s)
+    # a result beyond int32 is a REQUIRE failure (quant_util.h:102-106)
+    _, st = oracle.rescale(np.array([top], np.int64), [mmax], [20], out_dtype=np.int32, scale32=False,
+                           rounding_mode=oracle.ROUND_SINGLE, per_channel=False)
+    assert st == oracle.UNPREDICTABLE
+
+
+def test_rescale_int48_attribute_negatives():
+    """type_conversion.cpp:122 (scale32), :129 (output_unsigned), :132 (input_unsigned), :242 (input_zp)"""
+    x = np.array([1, 2], np.int64)
+    kw = dict(per_channel=False, rounding_mode=oracle.ROUND_SINGLE, out_dtype=np.int16)
+    assert oracle.rescale(x, [1 << 14], [20], scale32=False, **kw)[1] == oracle.VALID
+    assert oracle.rescale(x, [1 << 30], [40], scale32=True, **kw)[1] == oracle.ERROR
+    assert oracle.rescale(x, [1 << 14], [20], scale32=False, input_unsigned=True, **kw)[1] == oracle.ERROR
+    assert oracle.rescale(x, [1 << 14], [20], scale32=False, in_zp=3, **kw)[1] == oracle.ERROR
+    kw["out_dtype"] = np.uint16
+    assert oracle.rescale(x, [1 << 14], [20], scale32=False, output_unsigned=True, **kw)[1] == oracle.ERROR
+
+
 def test_clamp_int8():
     x = np.arange(-128, 128).astype(np.int8)
     assert np.array_equal(oracle.clamp(x, 0, 127), np.clip(x, 0, 127))

@@ -8,7 +8,8 @@ import struct
 
 import numpy as np
 
-DTYPE_CODE = {np.dtype(np.int8): 3, np.dtype(np.int16): 4, np.dtype(np.int32): 5, np.dtype(np.float32): 7,
+DTYPE_CODE = {np.dtype(np.int8): 3, np.dtype(np.int16): 4, np.dtype(np.int32): 5, np.dtype(np.int64): 6,
+              np.dtype(np.float32): 7,
               np.dtype(np.float16): 8}
 
 
@@ -113,7 +114,9 @@ class Writer:
 def tensor(name, shape, dtype, data=None):
     f = [(0, None, string(name)), (1, None, vector("i", shape)), (2, "I", DTYPE_CODE[np.dtype(dtype)])]
     if data is not None:
-        raw = np.ascontiguousarray(data, dtype=dtype).tobytes()
+        arr = np.ascontiguousarray(data, dtype=dtype)
+        # INT48 (int64 here) is serialized as the low 6 bytes of every element
+        raw = arr.view(np.uint8).reshape(-1, 8)[:, :6].tobytes() if arr.dtype == np.int64 else arr.tobytes()
         raw += b"\0" * (-len(raw) % 8)
         f.append((3, None, vector("B", raw)))
     return table(f)
