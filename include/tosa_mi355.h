@@ -319,8 +319,9 @@ int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank,
 
 /* Forces a kernel family for the following operator calls: 0 = automatic choice, 1 = direct (one output
  * element per lane, any shape), 2 = MFMA implicit-GEMM ("patch") kernel, 3 = MFMA GEMM kernel with direct
- * loads into LDS (1x1 CONV2D and MATMUL only); 2 and 3 return TMI_ERROR if the shape is not eligible.  Used by
- * the parity tests to check every kernel on the same operands. */
+ * loads into LDS (CONV2D and MATMUL), 4 = the slab kernel for int8 3x3 CONV2D with 64 input channels; 2, 3
+ * and 4 return TMI_ERROR if the shape is not eligible.  Used by the parity tests to check every kernel on the
+ * same operands. */
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
 
 /* Library build identification, e.g. "tosa_mi355 gfx950". */

@@ -79,14 +79,6 @@ struct PatchArgs
     FastDiv div_tw, div_pw, div_tiles_x, div_tiles_y, div_group, div_kw;
 };
 
-// min(max(v, lo), hi) as one instruction; lo <= hi
-__device__ __forceinline__ int32_t clamp_med3(int32_t v, int32_t lo, int32_t hi)
-{
-    int32_t r;
-    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
-    return r;
-}
-
 // Byte-wise version of a chunk load for channel vectors whose length is not a multiple of 16 bytes
 // (rows are then unaligned): bytes past the row end read as 0.  The rare path.
 __device__ __forceinline__ v4i load_chunk_bytes(const uint8_t* row, int off, int row_bytes)

@@ -1,0 +1,444 @@
+// CONV2D for layers whose channel vector is exactly 64 bytes (int8 with IC = 64), 3x3 taps: the small, latency-bound
+// layers of a ResNet stem, where a launch does well under a microsecond of matrix work and everything else is
+// overhead.  The kernel is the shortest path from memory to the matrix cores this chip offers:
+//
+//   - A workgroup (8 waves) owns a TH x TW tile of output pixels of one image and a block of 64 output channels.
+//     It needs the weight slab of the block (64 rows x taps x 64 bytes) and the input patch of the tile with its
+//     halo (PH x PW pixels x 64 bytes).  Both go from global memory straight into LDS with
+//     global_load_lds_dwordx4 (64 lanes x 16 bytes to 1 KB of LDS per instruction): no staging registers, no LDS
+//     stores, and only address arithmetic on the vector ALU.  Seven waves issue about seven loads each.
+//   - An LDS destination is fixed (M0 + 16 * lane) but every lane names its own source, so the layout is chosen
+//     by the mapping slot -> source: weight rows take taps*4 + 1 chunks and patch pixels 5, the odd chunk being
+//     padding.  Both strides are then congruent to 16 modulo 32 bytes, the layout on which a 32-row ds_read_b128
+//     fragment load runs at the full LDS rate.
+//   - A pixel outside the image reads a 64-byte page of input_zp bytes, so it contributes
+//     (zp - zp) * w = 0 like the reference's skipped tap (tensor_ops.cpp:845-852), and the zero-point identity
+//     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  sum(w) per channel is taken with v_dot4
+//     from the weight fragments on their way to the MFMA (in the shadow of the matrix instruction) and handed
+//     from row order to channel order through a wave-private LDS area: no second workgroup barrier.
+//   - While the loads are in flight the eighth wave, which issues none, turns bias / multiplier / shift into
+//     the per-channel constants of the RESCALE in LDS.
+//   - One barrier, then 18 MFMA steps per wave (one 32-channel x 32-pixel accumulator tile), then the fused
+//     RESCALE (+ CLAMP) epilogue of the patch kernel: a lane owns 16 consecutive channels of a pixel and stores
+//     them as 16 bytes (int8), 32 (int16) or 64 (int32).
+//
+// weight_zp must be 0 (the usual case for int8 weights); the patch kernel takes everything else.
+#include <cstring>
+
+#include "tmi_mfma.h"
+
+namespace tmi
+{
+
+struct SlabArgs
+{
+    const uint8_t* in;
+    const uint8_t* w;
+    const int32_t* bias;
+    const uint8_t* pad_page;    // 64 bytes of input_zp
+    void* out;
+    uint32_t* flag_word;
+    RescaleParams rp;
+    int32_t N, IH, IW, OC, OH, OW;
+    int32_t sy, sx, dy, dx, pad_top, pad_left;
+    int32_t TH, TW, PH, PW, tiles_x, tiles_y;
+    int32_t bias_len, za;
+    int32_t n_ocb;
+    int32_t out_kind;    // 0: int32 accumulators, 1: int8 through the RESCALE, 2: int16 through the RESCALE
+    int32_t xcd_remap;
+    int32_t step_py, step_px;    // 89 = step_py * PW + step_px: how far 7 loads (448 slots = 89 pixels + 3 chunks) move
+    FastDiv div_tw, div_pw, div_tiles_x, div_tiles_y, div_ocb;
+};
+
+__device__ __forceinline__ void slab_load(const void* src, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_addr) : "memory");
+}
+
+// the same with a 64-bit scalar base and a 32-bit per-lane byte offset: no 64-bit vector arithmetic per load
+__device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds_addr)
+                 : "memory");
+}
+
+template <int KH, int KW, bool ZA, bool FUSED>
+__global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
+{
+    // one field of every cache line of the arguments up front: a single scalar-cache round trip
+    asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len), "s"(a.div_ocb.d));
+    constexpr int TAPS   = KH * KW;
+    constexpr int RW     = TAPS * 4 + 1;    // chunks per weight row in LDS
+    constexpr int WSLOTS = 64 * RW;
+    constexpr int WLOADS = (WSLOTS + 63) / 64;
+    constexpr int RP     = 5;               // chunks per patch pixel in LDS
+    constexpr int LWAVES = 7;               // waves that issue loads; the eighth builds the tables
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // LDS: [weight rows][patch][64 x ChannelScale][64 x (multiplier, bias)][the block's common shift][per wave: 32 words]
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li     = lane & 31;
+    const int lh     = lane >> 5;
+    const int p_slots = a.PH * a.PW * RP;
+    const int p_loads = (p_slots + 63) >> 6;
+    uint8_t* wl       = lds;
+    uint8_t* pl       = lds + WLOADS * 1024;
+    uint8_t* tabs     = pl + p_loads * 1024;
+    ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tabs);
+    int2* tab_mb         = reinterpret_cast<int2*>(tabs + 64 * sizeof(ChannelScale));    // multiplier, bias
+    int32_t* uni_shift   = reinterpret_cast<int32_t*>(tab_mb + 64);                      // 4 words, one used
+    int32_t* wave_area   = uni_shift + 4 + wave * 32;
+
+    uint32_t bid = blockIdx.x;
+    if (a.xcd_remap)
+    {
+        // consecutive workgroups go to the 8 XCDs in turn: give each XCD a contiguous run of tiles, whose halos
+        // then meet in one L2
+        const uint32_t per = gridDim.x >> 3;
+        bid                = (bid & 7) * per + (bid >> 3);
+    }
+    const uint32_t tile = fdiv(bid, a.div_ocb);
+    const int ocb       = bid - tile * a.n_ocb;
+    const uint32_t trow = fdiv(tile, a.div_tiles_x);
+    const int txi       = tile - trow * a.tiles_x;
+    const int n         = fdiv(trow, a.div_tiles_y);
+    const int tyi       = trow - n * a.tiles_y;
+    const int oy0 = tyi * a.TH, ox0 = txi * a.TW;
+    const int oc0 = ocb * 64;
+    const int y0 = oy0 * a.sy - a.pad_top, x0 = ox0 * a.sx - a.pad_left;
+
+    uint32_t flags = 0;
+    if (wave < LWAVES)
+    {
+        // Load l fills LDS bytes [1024 l, 1024 l + 1024); wave v issues l = v, v + 7, ...  The per-lane source is
+        // worked out once with divisions and then walked: 7 loads on are 448 slots, i.e. 12 weight rows and 4 chunks,
+        // or 89 patch pixels and 3 chunks.  (Integer multiplies and divides run at a quarter of the vector rate;
+        // with them in the loop, issuing the loads took three times as long as the loads themselves.)
+        const uint32_t lbase = (uint32_t)(uintptr_t)lds;
+        {
+            const int s0 = wave * 64 + lane;
+            int row      = s0 / RW;
+            int ch       = s0 - row * RW;
+            uint32_t dst = lbase + wave * 1024;
+            for (int l = wave; l < WLOADS; l += LWAVES)
+            {
+                // row r of a 32-row MFMA operand tile holds channel 16*((r>>2)&1) + 4*(r>>3) + (r&3) of the tile,
+                // which makes a lane's 16 accumulators 16 consecutive channels; rows of channels past OC read
+                // channel 0 of the block (valid memory, results never stored)
+                const int r   = row < 64 ? row : 63;
+                const int chn = (r & 32) + 4 * (r & 4) + ((r >> 1) & 12) + (r & 3);
+                const int c   = oc0 + (oc0 + chn < a.OC ? chn : 0);
+                slab_load_off(__umul24(c, TAPS * 64) + (ch < RW - 1 ? ch : 0) * 16, a.w, dst);
+                dst += LWAVES * 1024;
+                row += (LWAVES * 64) / RW;
+                ch += (LWAVES * 64) % RW;
+                if (ch >= RW)
+                    ch -= RW, row++;
+            }
+        }
+        {
+            const uint8_t* in_n = a.in + (size_t)n * a.IH * a.IW * 64;
+            const int n_pix     = a.PH * a.PW;
+            int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
+            const int s0        = lp * 64 + lane;
+            int pix             = (int)(((uint32_t)s0 * 52429u) >> 18);    // s0 / 5 for s0 < 2^16
+            int ch              = s0 - pix * RP;
+            int py              = fdiv(pix, a.div_pw);
+            int px              = pix - py * a.PW;
+            uint32_t dst        = lbase + (WLOADS + lp) * 1024;
+            for (; lp < p_loads; lp += LWAVES)
+            {
+                const int iy = y0 + py, ix = x0 + px;
+                const bool img = pix < n_pix && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+                const int c16  = (ch < 4 ? ch : 0) * 16;
+                const uint8_t* src = img ? in_n + (uint32_t)((__umul24(iy, a.IW) + ix) * 64 + c16) : a.pad_page + c16;
+                slab_load(src, dst);
+                dst += LWAVES * 1024;
+                ch += (LWAVES * 64) % RP;
+                pix += (LWAVES * 64) / RP;
+                px += a.step_px, py += a.step_py;
+                if (ch >= RP)
+                    ch -= RP, pix++, px++;
+                if (px >= a.PW)
+                    px -= a.PW, py++;
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    else
+    {
+        // the table wave: bias and the per-channel RESCALE constants, one channel per lane
+        const int oc    = oc0 + lane;
+        const bool ok   = oc < a.OC;
+        const int occ   = ok ? oc : 0;
+        const int32_t b = a.bias[a.bias_len == 1 ? 0 : occ];
+        int32_t m       = 0;
+        if constexpr (FUSED)
+        {
+            const int32_t m_raw   = load_multiplier(a.rp, occ);
+            const int32_t s_raw   = load_shift(a.rp, occ);
+            // channels past OC take the first channel's shift, so that they do not break a block whose channels
+            // all share one
+            const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
+            const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
+            tab_cs[lane]          = cs;
+            m                     = cs.m;
+            // One shift of at least 32 for the whole block, small enough for output_zp to ride in the rounding
+            // term: the epilogue keeps the rounding terms in scalar registers and reads 8 bytes per channel.
+            const int uni = __all(cs.s == s_first) && s_first >= 32 && s_first <= zp_fold_max_shift(a.rp.out_zp);
+            if (lane == 0)
+                *uni_shift = uni ? s_first : -1;
+        }
+        tab_mb[lane] = int2{ m, ok ? b : 0 };
+    }
+    __syncthreads();
+
+    // ---- MFMA: wave = (channel tile, pixel tile) ---------------------------------------------------------------
+    const int oct = wave >> 2, pxt = wave & 3;
+    const int P   = a.TH * a.TW;
+    int p         = pxt * 32 + li;
+    const bool p_in_tile = p < P;
+    p             = p_in_tile ? p : 0;
+    const int ty  = fdiv(p, a.div_tw);
+    const int tx  = p - ty * a.TW;
+    v16i acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        acc[r] = 0;
+    int wsum = 0;
+    if (pxt * 32 < P)    // wave-uniform
+    {
+        const uint8_t* wrow = wl + ((oct * 32 + li) * RW) * 16 + lh * 16;
+        const uint8_t* prow = pl + ((ty * a.sy * a.PW + tx * a.sx) * RP) * 16 + lh * 16;
+        const int row_step  = a.dy * a.PW * RP * 16;
+        const int col_step  = a.dx * RP * 16;
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++)
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                {
+                    const v4i fa = *reinterpret_cast<const v4i*>(wrow + ((ky * KW + kx) * 2 + h) * 32);
+                    const v4i fb = *reinterpret_cast<const v4i*>(prow + ky * row_step + kx * col_step + h * 32);
+                    acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
+                    if constexpr (ZA)
+                        wsum += dot4_ones(fa);
+                }
+    }
+
+    // ---- epilogue ----------------------------------------------------------------------------------------------
+    // (lane, register 4q + j) = D[row 8q + 4 lh + j][pixel li] = channel 32 oct + 16 lh + 4q + j
+    const int ocl = oct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
+    int32_t cm[16], cb[16];                // multiplier and bias of the lane's channels
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+    {
+        const v4i mb = *reinterpret_cast<const v4i*>(tab_mb + ocl + 2 * q);
+        cm[2 * q] = mb[0], cb[2 * q] = mb[1], cm[2 * q + 1] = mb[2], cb[2 * q + 1] = mb[3];
+    }
+    if constexpr (ZA)
+    {
+        // the lane's sum covers its K half of row li; the other half sits 32 lanes away.  Row li is channel
+        // 16*((li>>2)&1) + 4*(li>>3) + (li&3) of the tile.
+        wsum += __shfl_xor(wsum, 32);
+        if (lh == 0)
+            wave_area[4 * (li & 4) + ((li >> 1) & 12) + (li & 3)] = wsum;
+        // same wave: the LDS unit works in order, no barrier needed
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+        {
+            const v4i sw = *reinterpret_cast<const v4i*>(wave_area + 16 * lh + 4 * q);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                cb[4 * q + j] -= a.za * sw[j];
+        }
+    }
+    const int oy = oy0 + ty, ox = ox0 + tx;
+    const bool pix_ok  = p_in_tile && pxt * 32 < P && oy < a.OH && ox < a.OW;
+    const bool chan_ok = oc0 + ocl < a.OC;    // OC is a multiple of 16: a lane's 16 channels are in or out together
+    const size_t obase = (((size_t)n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl;
+    if constexpr (!FUSED)
+    {
+        if (pix_ok && chan_ok)
+        {
+            int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase;
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acc[4 * q] + cb[4 * q], acc[4 * q + 1] + cb[4 * q + 1],
+                                                          acc[4 * q + 2] + cb[4 * q + 2], acc[4 * q + 3] + cb[4 * q + 3] };
+        }
+    }
+    else
+    {
+        int32_t r[16];
+        const int s_uni = __builtin_amdgcn_readfirstlane(*uni_shift);
+        if (s_uni >= 0)
+        {
+            // One shift s >= 32 for every channel: (v * m + round) >> s is the high word of the sum shifted by
+            // s - 32; the rounding terms (double rounding and output_zp * 2^s folded in) are two scalars, and
+            // apply_scale_32's value-range test cannot fire (it only exists for shifts below 32).
+            const int64_t dr     = a.rp.double_round ? (int64_t(1) << 30) : 0;
+            const int64_t rnd_p  = (int64_t(1) << (s_uni - 1)) + dr + ((int64_t)a.rp.out_zp << s_uni);
+            const int64_t rnd_n  = rnd_p - 2 * dr;
+            const int sh         = s_uni - 32;
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+            {
+                const int32_t v  = acc[e] + cb[e];
+                const int64_t pr = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? rnd_p : rnd_n);
+                r[e]             = clamp_med3((int32_t)(pr >> 32) >> sh, a.rp.lo, a.rp.hi);
+            }
+        }
+        else
+        {
+            uint32_t eflags = 0;
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+            {
+                const ChannelScale cs = tab_cs[ocl + e];
+                r[e]                  = fast_rescale(acc[e] + cb[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
+            }
+            if (pix_ok && chan_ok)
+                flags |= eflags;    // pixels and channels outside the tensor raise nothing
+        }
+        if (pix_ok && chan_ok)
+        {
+            if (a.out_kind == 1)
+            {
+                v4i pk;
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                {
+                    // the low bytes of four clamped values into one word
+                    const int lo2 = __builtin_amdgcn_perm(r[4 * q + 1], r[4 * q], 0x0c0c0400);
+                    const int hi2 = __builtin_amdgcn_perm(r[4 * q + 3], r[4 * q + 2], 0x04000c0c);
+                    pk[q]         = lo2 | hi2;
+                }
+                *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + obase) = pk;
+            }
+            else
+            {
+                int16_t* o = reinterpret_cast<int16_t*>(a.out) + obase;
+#pragma unroll
+                for (int half = 0; half < 2; half++)
+                {
+                    v4i pk;
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        pk[q] = (r[8 * half + 2 * q] & 0xffff) | ((r[8 * half + 2 * q + 1] & 0xffff) << 16);
+                    *reinterpret_cast<v4i*>(o + 8 * half) = pk;
+                }
+            }
+        }
+    }
+    raise_flags(a.flag_word, flags);
+}
+
+template <int KH, int KW, bool ZA, bool FUSED>
+static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
+{
+    auto kern              = conv2d_slab_kernel<KH, KW, ZA, FUSED>;
+    static bool configured = false;
+    if (!configured)
+    {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024) != hipSuccess)
+            return false;
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, st, a);
+    return true;
+}
+
+template <int KH, int KW>
+static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, bool fused)
+{
+    if (a.za != 0)
+        return fused ? launch_slab_kernel<KH, KW, true, true>(st, a, grid, lds_bytes)
+                     : launch_slab_kernel<KH, KW, true, false>(st, a, grid, lds_bytes);
+    return fused ? launch_slab_kernel<KH, KW, false, true>(st, a, grid, lds_bytes)
+                 : launch_slab_kernel<KH, KW, false, false>(st, a, grid, lds_bytes);
+}
+
+// nullptr when the layer is not one this kernel takes; the caller then goes to the patch kernel.
+const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                               const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                               void* out, const void* pad_page, uint32_t* flag_word)
+{
+    if (in_dtype != TMI_INT8 || g.IC != 64 || g.KH != 3 || g.KW != 3 || w_zp != 0 || !pad_page || !flag_word)
+        return nullptr;
+    if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
+        return nullptr;
+    if (g.OC < 48 || g.OC > 65536 || (g.OC & 15) || g.N < 1 || g.OH < 1 || g.OW < 1)
+        return nullptr;
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || ((uintptr_t)bias & 3))
+        return nullptr;
+    if ((int64_t)g.N * g.IH * g.IW * 64 >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
+        return nullptr;
+
+    // The tile: at most 128 pixels (four 32-pixel tiles, one per wave and channel tile).  A workgroup moves the
+    // weight slab (taps * 64 rows of 64 bytes) plus PH * PW patch rows; whole rounds of 256 workgroups count.
+    // The search depends on the geometry only; a caller repeats the same layer, so the last answer is kept.
+    const int n_ocb = (g.OC + 63) / 64;
+    struct TileChoice
+    {
+        int32_t key[8];
+        int th, tw;
+    };
+    static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0 };
+    const int32_t key[8] = { g.N, g.OH, g.OW, n_ocb, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
+    int best_th = 0, best_tw = 0;
+    if (memcmp(key, last.key, sizeof(key)) == 0)
+        best_th = last.th, best_tw = last.tw;
+    else
+    {
+        int64_t best_cost = 0;
+        for (int th = 1; th <= g.OH && th <= 128; th++)
+            for (int tw = 1; tw <= g.OW && th * tw <= 128; tw++)
+            {
+                const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+                const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
+                if (ph * pw * 5 >= (1 << 16) || ph * pw * 80 > 96 * 1024)
+                    continue;
+                const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
+                const int64_t rounds = (tiles + 255) / 256;
+                // a round costs its loads plus the four 32-pixel MFMA tiles whether they are full or not
+                const int64_t cost = rounds * (9 * 64 + ph * pw + 600);
+                if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
+                    best_th = th, best_tw = tw, best_cost = cost;
+            }
+        memcpy(last.key, key, sizeof(key));
+        last.th = best_th, last.tw = best_tw;
+    }
+    if (!best_th)
+        return nullptr;
+
+    SlabArgs a{};
+    a.in = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = (const int32_t*)bias, a.out = out;
+    a.pad_page = (const uint8_t*)pad_page, a.flag_word = flag_word, a.rp = rp;
+    a.N = g.N, a.IH = g.IH, a.IW = g.IW, a.OC = g.OC, a.OH = g.OH, a.OW = g.OW;
+    a.sy = g.stride_y, a.sx = g.stride_x, a.dy = g.dil_y, a.dx = g.dil_x, a.pad_top = g.pad_top, a.pad_left = g.pad_left;
+    a.TH = best_th, a.TW = best_tw;
+    a.PH = (best_th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+    a.PW = (best_tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
+    a.tiles_y = (g.OH + best_th - 1) / best_th, a.tiles_x = (g.OW + best_tw - 1) / best_tw;
+    a.bias_len = g.bias_len, a.za = in_zp, a.n_ocb = n_ocb;
+    a.out_kind = !rp.enabled ? 0 : (out_dtype == TMI_INT8 ? 1 : 2);
+    const int64_t grid = (int64_t)g.N * a.tiles_y * a.tiles_x * n_ocb;
+    if (grid >= (int64_t(1) << 31))
+        return nullptr;
+    a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? 1 : 0;
+    a.step_py = 89 / a.PW, a.step_px = 89 % a.PW;
+    a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pw = make_fastdiv((uint32_t)a.PW);
+    a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
+    a.div_ocb = make_fastdiv((uint32_t)n_ocb);
+    const int w_loads = (64 * (9 * 4 + 1) + 63) / 64, p_loads = (a.PH * a.PW * 5 + 63) / 64;
+    const int lds_bytes = (w_loads + p_loads) * 1024 + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16 + 8 * 32 * 4;
+    if (!launch_slab_taps<3, 3>(st, a, (int)grid, lds_bytes, rp.enabled != 0))
+        return nullptr;
+    return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";
+}
+
+}    // namespace tmi

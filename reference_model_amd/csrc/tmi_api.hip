@@ -326,10 +326,13 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     {
         // kernel choice 2 / 3 name one kernel; left open, the likely faster one is tried first
         const void* pad_page = ctx->pages_dev + (d->in_dtype == TMI_INT8 ? (in_zp & 255) * 64 : 0);
-        const bool gemm_ok   = ctx->kernel_choice != 2;
-        const bool patch_ok  = ctx->kernel_choice != 3;
+        const bool gemm_ok   = ctx->kernel_choice == 0 || ctx->kernel_choice == 3;
+        const bool patch_ok  = ctx->kernel_choice == 0 || ctx->kernel_choice == 2;
         const bool gemm_1st  = gemm_ok && (!patch_ok || gemm_mfma_preferred(d->in_dtype, g));
-        if (gemm_1st)
+        if (ctx->kernel_choice == 0 || ctx->kernel_choice == 4)
+            name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
+                                      ctx->flags_dev);
+        if (!name && gemm_1st)
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
                                     pad_page, ctx->flags_dev);
         if (!name && patch_ok)
@@ -468,7 +471,7 @@ const char* tmi_last_kernel(const tmi_ctx_t* ctx)
 
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
-    if (!ctx || choice < 0 || choice > 3)
+    if (!ctx || choice < 0 || choice > 4)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;

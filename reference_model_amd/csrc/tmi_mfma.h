@@ -53,6 +53,14 @@ struct Mma<bf16_t>
     }
 };
 
+// min(max(v, lo), hi) as one instruction; lo <= hi
+__device__ __forceinline__ int32_t clamp_med3(int32_t v, int32_t lo, int32_t hi)
+{
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+    return r;
+}
+
 __device__ __forceinline__ int dot4_ones(v4i v)
 {
     int s = __builtin_amdgcn_sdot4(v.x, 0x01010101, 0, false);

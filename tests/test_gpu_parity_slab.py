@@ -1,0 +1,172 @@
+"""GPU parity of the slab kernel (int8 3x3 CONV2D with 64 input channels: weight slab and input patch loaded
+straight into LDS, optional fused RESCALE / CLAMP) against exact float64 BLAS products and the CPU oracle, through
+the C ABI.  Everything here is integer work: results are compared bit for bit."""
+import numpy as np
+import pytest
+
+import cases
+import gpu_ops
+import oracle
+from reference_model_amd import Context, TmiError, capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = Context(0)
+    c.set_kernel_choice(capi.KERNEL_SLAB)
+    yield c
+    c.close()
+
+
+SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation
+    (8, 56, 56, 64, (1, 1, 1, 1), (1, 1), (1, 1)),      # the headline layer
+    (3, 30, 29, 64, (1, 1, 1, 1), (1, 1), (1, 1)),      # ragged tiles in both directions
+    (1, 5, 5, 64, (1, 1, 1, 1), (1, 1), (1, 1)),        # one small tile
+    (2, 17, 23, 48, (0, 0, 0, 0), (1, 1), (1, 1)),      # no padding, 48 channels (the second channel tile half empty)
+    (2, 20, 20, 128, (1, 1, 1, 1), (1, 1), (1, 1)),     # two channel blocks
+    (2, 20, 20, 80, (2, 1, 0, 1), (1, 1), (1, 1)),      # a ragged second block, uneven padding
+    (4, 57, 57, 64, (1, 1, 1, 1), (2, 2), (1, 1)),      # stride 2
+    (2, 34, 31, 64, (0, 1, 1, 0), (2, 1), (1, 1)),      # stride 2 x 1
+    (2, 24, 24, 64, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilation 2
+    (33, 14, 14, 64, (1, 1, 1, 1), (1, 1), (1, 1)),     # more workgroups than compute units, odd count
+]
+
+
+def _operands(shape, seed):
+    n, ih, iw, oc, pad, stride, dil = shape
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 128, (n, ih, iw, 64)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 3, 3, 64)).astype(np.int8)
+    bias = rng.integers(-(1 << 18), 1 << 18, oc).astype(np.int32)
+    return x, w, bias
+
+
+@pytest.mark.parametrize("shape", SLAB_SHAPES)
+@pytest.mark.parametrize("in_zp", [0, -7, 127, -128])
+def test_slab_conv_int32_bit_exact(ctx, shape, in_zp):
+    n, ih, iw, oc, pad, stride, dil = shape
+    x, w, bias = _operands(shape, ih * iw + oc)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
+    assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
+    assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, in_zp, 0))
+    # the last image's first channels against the oracle's own loop nest
+    sub = oracle.conv2d("i8", x[-1:], w[:5], bias[:5], pad, stride, dil, in_zp=in_zp, w_zp=0)
+    assert np.array_equal(got[-1:, :, :, :5], sub)
+
+
+def test_slab_conv_bias_broadcast_and_extremes(ctx):
+    """a bias of length 1 goes to every channel (tensor_ops.cpp:747, :816-823); all-extreme operands reach the
+    largest accumulators the type allows: 576 * 128 * 255 < 2^31"""
+    x = np.full((2, 9, 9, 64), -128, np.int8)
+    w = np.full((64, 3, 3, 64), -128, np.int8)
+    w[1::2] = 127
+    bias = np.array([-12345], np.int32)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, (1, 1, 1, 1), in_zp=127, w_zp=0)
+    assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
+    assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, (1, 1, 1, 1), (1, 1), (1, 1), 127, 0))
+    assert got.max() == 576 * 255 * 128 - 12345 and got.min() == -576 * 255 * 127 - 12345
+
+
+def _fused(ctx, c, out_dtype):
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], 0,
+                             rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype,
+                                          rounding_mode=c.get("mode", capi.ROUND_DOUBLE),
+                                          per_channel=c.get("per_channel", True)),
+                             clamp=c["clamp"])
+    acc = cases.conv2d_exact_blas(c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], 0)
+    want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"], out_dtype=out_dtype,
+                               rounding_mode=c.get("mode", oracle.ROUND_DOUBLE), per_channel=c.get("per_channel", True))
+    if c["clamp"] is not None:
+        want = oracle.clamp(want, *c["clamp"])
+    return got, st, want, wst
+
+
+@pytest.mark.parametrize("shape", SLAB_SHAPES)
+@pytest.mark.parametrize("zps", [(-7, 0), (4, -3), (-128, 100)])
+@pytest.mark.parametrize("out_dtype", [np.int8, np.int16])
+def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
+    n, ih, iw, oc, pad, stride, dil = shape
+    x, _, _ = _operands(shape, ih + iw + oc)
+    rng = np.random.default_rng(oc + ih)
+    c = dict(x=x, w=np.clip(np.rint(rng.normal(0, 30, (oc, 3, 3, 64))), -127, 127).astype(np.int8),
+             bias=np.rint(rng.normal(0, 1 << 14, oc)).astype(np.int32), in_zp=zps[0], pad=pad, stride=stride,
+             dilation=dil, mult=rng.integers(1 << 30, 1 << 31, oc).astype(np.int32),
+             shift=rng.integers(36, 42, oc).astype(np.int8), out_zp=zps[1] if out_dtype == np.int8 else 0,
+             clamp=(-100, 110) if out_dtype == np.int8 else None)
+    got, st, want, wst = _fused(ctx, c, out_dtype)
+    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(got)) > 50
+
+
+def test_slab_config3_full_size(ctx):
+    """the named configuration with its own operands: shift 38 for every channel, DOUBLE rounding, CLAMP [0, 127]"""
+    c = cases.c3()
+    got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"],
+                             rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"]), clamp=c["clamp"])
+    assert ctx.last_kernel == "conv2d_slab_i8_rescale" and st == capi.VALID
+    acc = cases.conv2d_exact_blas(c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
+    want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
+    assert wst == oracle.VALID and np.array_equal(got, oracle.clamp(want, *c["clamp"]))
+
+
+@pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
+def test_slab_fused_rescale_per_tensor_scale_and_rounding_modes(ctx, mode):
+    shape = (2, 20, 20, 64, (1, 1, 1, 1), (1, 1), (1, 1))
+    x, w, bias = _operands(shape, 77)
+    c = dict(x=x, w=w, bias=bias, in_zp=3, pad=shape[4], stride=shape[5], dilation=shape[6],
+             mult=np.array([1518500250], np.int32), shift=np.array([44], np.int8), out_zp=-5, clamp=None, mode=mode,
+             per_channel=False)
+    got, st, want, wst = _fused(ctx, c, np.int8)
+    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert st == wst == capi.VALID and np.array_equal(got, want)
+
+
+def test_slab_fused_rescale_reports_require_conditions(ctx):
+    """a shift below 32 makes apply_scale_32 check the value range (quant_util.h:59-67): UNPREDICTABLE, as the
+    oracle says for the same operands; pixels and channels outside the tensor raise nothing"""
+    shape = (1, 9, 9, 48, (1, 1, 1, 1), (1, 1), (1, 1))
+    x, w, bias = _operands(shape, 5)
+    c = dict(x=x, w=w, bias=np.zeros(48, np.int32), in_zp=3, pad=shape[4], stride=shape[5], dilation=shape[6],
+             mult=np.full(48, 1 << 30, np.int32), shift=np.full(48, 12, np.int8), out_zp=0, clamp=None)
+    got, st, want, wst = _fused(ctx, c, np.int8)
+    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert st == wst == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
+    # all-zero operands: every value is legal, also in the lanes that hold no pixel or channel of the tensor
+    c["x"], c["w"], c["in_zp"] = np.zeros_like(x), np.zeros_like(w), 0
+    got, st, want, wst = _fused(ctx, c, np.int8)
+    assert st == wst == capi.VALID and ctx.flags == 0 and np.array_equal(got, want)
+
+
+def test_slab_kernel_refuses_what_it_cannot_take(ctx):
+    rng = np.random.default_rng(1)
+    bias = np.zeros(64, np.int32)
+    x = rng.integers(-128, 128, (1, 8, 8, 64)).astype(np.int8)
+    w = rng.integers(-128, 128, (64, 3, 3, 64)).astype(np.int8)
+    with pytest.raises(TmiError):      # a weight zero point
+        gpu_ops.conv2d(ctx, x, w, bias, (1, 1, 1, 1), in_zp=0, w_zp=3)
+    with pytest.raises(TmiError):      # 32 input channels
+        gpu_ops.conv2d(ctx, x[..., :32], w[..., :32], bias, (1, 1, 1, 1))
+    with pytest.raises(TmiError):      # 5x5 taps
+        gpu_ops.conv2d(ctx, x, rng.integers(-128, 128, (64, 5, 5, 64)).astype(np.int8), bias, (2, 2, 2, 2))
+    with pytest.raises(TmiError):      # 40 output channels
+        gpu_ops.conv2d(ctx, x, w[:40], bias[:40], (1, 1, 1, 1))
+
+
+def test_automatic_choice_takes_the_slab_kernel_for_its_layers():
+    c = Context(0)
+    try:
+        shape = (2, 28, 28, 64, (1, 1, 1, 1), (1, 1), (1, 1))
+        x, w, bias = _operands(shape, 3)
+        got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], in_zp=-7)
+        assert st == capi.VALID and c.last_kernel == "conv2d_slab_i8"
+        c.set_kernel_choice(capi.KERNEL_MFMA)
+        other, st = gpu_ops.conv2d(c, x, w, bias, shape[4], in_zp=-7)
+        assert st == capi.VALID and c.last_kernel == "conv2d_mfma_i8" and np.array_equal(got, other)
+        c.set_kernel_choice(capi.KERNEL_AUTO)
+        got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], in_zp=-7, w_zp=2)     # weight zero point: the patch kernel
+        assert st == capi.VALID and c.last_kernel == "conv2d_mfma_i8"
+    finally:
+        c.close()
