@@ -1095,14 +1095,9 @@ template <typename T, int WOC, int OCT, int PXT, int EPI, bool VEC, bool MULTI>
 static bool launch_patch(hipStream_t st, PatchArgs& a, size_t lds_bytes, int blocks)
 {
     auto kern                = conv2d_patch_kernel<T, WOC, OCT, PXT, EPI, VEC, MULTI>;
-    static size_t configured = 0;    // largest dynamic LDS size this instantiation was configured for
-    if (lds_bytes > configured)
-    {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes) != hipSuccess)
-            return false;
-        configured = lds_bytes;
-    }
+    static LdsLimit granted{};
+    if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, granted))
+        return false;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
     return true;
 }

@@ -13,12 +13,12 @@
 //     fragment load runs at the full LDS rate.
 //   - A pixel outside the image reads a 64-byte page of input_zp bytes, so it contributes
 //     (zp - zp) * w = 0 like the reference's skipped tap (tensor_ops.cpp:845-852), and the zero-point identity
-//     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  sum(w) per channel is taken with v_dot4
-//     from the weight fragments on their way to the MFMA (in the shadow of the matrix instruction) and handed
-//     from row order to channel order through a wave-private LDS area: no second workgroup barrier.
+//     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  sum(w) per channel costs nothing: a wave's
+//     32 MFMA columns are 31 pixels and one "pixel of ones" (bytes 0x01 in LDS wherever a tap can read), whose
+//     accumulators are the sums, already in the register order of the lanes that need them.
 //   - While the loads are in flight the eighth wave, which issues none, turns bias / multiplier / shift into
 //     the per-channel constants of the RESCALE in LDS.
-//   - One barrier, then 18 MFMA steps per wave (one 32-channel x 32-pixel accumulator tile), then the fused
+//   - One barrier, then 18 MFMA steps per wave (one accumulator tile of 32 channels x 32 columns), then the fused
 //     RESCALE (+ CLAMP) epilogue of the patch kernel: a lane owns 16 consecutive channels of a pixel and stores
 //     them as 16 bytes (int8), 32 (int16) or 64 (int32).
 //
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     constexpr int RP     = 5;               // chunks per patch pixel in LDS
     constexpr int LWAVES = 7;               // waves that issue loads; the eighth builds the tables
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    // LDS: [weight rows][patch][64 x ChannelScale][64 x (multiplier, bias)][the block's common shift][per wave: 32 words]
+    // LDS: [weight rows][patch][pixel of ones][64 x ChannelScale][64 x (multiplier, bias)][the block's common shift]
     const int tid    = threadIdx.x;
     const int lane   = tid & 63;
     const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -84,11 +84,15 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     const int p_loads = (p_slots + 63) >> 6;
     uint8_t* wl       = lds;
     uint8_t* pl       = lds + WLOADS * 1024;
-    uint8_t* tabs     = pl + p_loads * 1024;
+    // fragment offsets of the taps inside the patch, and the "pixel of ones": bytes 0x01 wherever a tap can read
+    const int row_step   = a.dy * a.PW * RP * 16;
+    const int col_step   = a.dx * RP * 16;
+    const int ones_bytes = ZA ? ((KH - 1) * row_step + (KW - 1) * col_step + 64) : 0;
+    uint8_t* ones        = pl + p_loads * 1024;
+    uint8_t* tabs        = ones + ones_bytes;
     ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tabs);
     int2* tab_mb         = reinterpret_cast<int2*>(tabs + 64 * sizeof(ChannelScale));    // multiplier, bias
     int32_t* uni_shift   = reinterpret_cast<int32_t*>(tab_mb + 64);                      // 4 words, one used
-    int32_t* wave_area   = uni_shift + 4 + wave * 32;
 
     uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
@@ -191,28 +195,34 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 *uni_shift = uni ? s_first : -1;
         }
         tab_mb[lane] = int2{ m, ok ? b : 0 };
+        for (int i = lane * 16; i < ones_bytes; i += 1024)
+            *reinterpret_cast<v4i*>(ones + i) = v4i{ 0x01010101, 0x01010101, 0x01010101, 0x01010101 };
     }
     __syncthreads();
 
     // ---- MFMA: wave = (channel tile, pixel tile) ---------------------------------------------------------------
     const int oct = wave >> 2, pxt = wave & 3;
-    const int P   = a.TH * a.TW;
-    int p         = pxt * 32 + li;
-    const bool p_in_tile = p < P;
-    p             = p_in_tile ? p : 0;
+    // A wave's 32 MFMA columns are 31 pixels and, in column 31, the pixel of ones: its accumulators are sum(w) of
+    // the wave's 32 channels, which the zero-point term needs, for the price of nothing (the column would be
+    // computed anyway).
+    constexpr int PXW = 31;
+    const int P       = a.TH * a.TW;
+    int p             = pxt * PXW + li;
+    const bool p_in_tile = li < PXW && p < P;
+    p                 = p_in_tile ? p : 0;
     const int ty  = fdiv(p, a.div_tw);
     const int tx  = p - ty * a.TW;
     v16i acc;
 #pragma unroll
     for (int r = 0; r < 16; r++)
         acc[r] = 0;
-    int wsum = 0;
-    if (pxt * 32 < P)    // wave-uniform
+    const bool wave_active = pxt * PXW < P;    // wave-uniform
+    if (wave_active)
     {
         const uint8_t* wrow = wl + ((oct * 32 + li) * RW) * 16 + lh * 16;
         const uint8_t* prow = pl + ((ty * a.sy * a.PW + tx * a.sx) * RP) * 16 + lh * 16;
-        const int row_step  = a.dy * a.PW * RP * 16;
-        const int col_step  = a.dx * RP * 16;
+        if (ZA && li == PXW)
+            prow = ones + lh * 16;
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
 #pragma unroll
@@ -223,8 +233,6 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                     const v4i fa = *reinterpret_cast<const v4i*>(wrow + ((ky * KW + kx) * 2 + h) * 32);
                     const v4i fb = *reinterpret_cast<const v4i*>(prow + ky * row_step + kx * col_step + h * 32);
                     acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
-                    if constexpr (ZA)
-                        wsum += dot4_ones(fa);
                 }
     }
 
@@ -240,23 +248,15 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     }
     if constexpr (ZA)
     {
-        // the lane's sum covers its K half of row li; the other half sits 32 lanes away.  Row li is channel
-        // 16*((li>>2)&1) + 4*(li>>3) + (li&3) of the tile.
-        wsum += __shfl_xor(wsum, 32);
-        if (lh == 0)
-            wave_area[4 * (li & 4) + ((li >> 1) & 12) + (li & 3)] = wsum;
-        // same wave: the LDS unit works in order, no barrier needed
+        // Lane 31 + 32 lh holds in register e the column of ones for channel 16 lh + e: sum(w) of exactly the
+        // channel this lane has in register e.  |sum(w)| <= taps * 64 * 128 < 2^23 and |za| <= 128: a 24-bit multiply.
+        const int src = (PXW + 32 * lh) * 4;
 #pragma unroll
-        for (int q = 0; q < 4; q++)
-        {
-            const v4i sw = *reinterpret_cast<const v4i*>(wave_area + 16 * lh + 4 * q);
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                cb[4 * q + j] -= a.za * sw[j];
-        }
+        for (int e = 0; e < 16; e++)
+            cb[e] -= __mul24(a.za, __builtin_amdgcn_ds_bpermute(src, acc[e]));
     }
     const int oy = oy0 + ty, ox = ox0 + tx;
-    const bool pix_ok  = p_in_tile && pxt * 32 < P && oy < a.OH && ox < a.OW;
+    const bool pix_ok  = p_in_tile && wave_active && oy < a.OH && ox < a.OW;
     const bool chan_ok = oc0 + ocl < a.OC;    // OC is a multiple of 16: a lane's 16 channels are in or out together
     const size_t obase = (((size_t)n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl;
     if constexpr (!FUSED)
@@ -340,14 +340,9 @@ template <int KH, int KW, bool ZA, bool FUSED>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
     auto kern              = conv2d_slab_kernel<KH, KW, ZA, FUSED>;
-    static bool configured = false;
-    if (!configured)
-    {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                160 * 1024) != hipSuccess)
-            return false;
-        configured = true;
-    }
+    static LdsLimit granted{};
+    if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
+        return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, st, a);
     return true;
 }
@@ -378,7 +373,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     if ((int64_t)g.N * g.IH * g.IW * 64 >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
         return nullptr;
 
-    // The tile: at most 128 pixels (four 32-pixel tiles, one per wave and channel tile).  A workgroup moves the
+    // The tile: at most 124 pixels (four tiles of 31 pixels, one per wave and channel tile).  A workgroup moves the
     // weight slab (taps * 64 rows of 64 bytes) plus PH * PW patch rows; whole rounds of 256 workgroups count.
     // The search depends on the geometry only; a caller repeats the same layer, so the last answer is kept.
     const int n_ocb = (g.OC + 63) / 64;
@@ -395,8 +390,8 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     else
     {
         int64_t best_cost = 0;
-        for (int th = 1; th <= g.OH && th <= 128; th++)
-            for (int tw = 1; tw <= g.OW && th * tw <= 128; tw++)
+        for (int th = 1; th <= g.OH && th <= 124; th++)
+            for (int tw = 1; tw <= g.OW && th * tw <= 124; tw++)
             {
                 const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
                 const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
@@ -435,7 +430,8 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
     const int w_loads = (64 * (9 * 4 + 1) + 63) / 64, p_loads = (a.PH * a.PW * 5 + 63) / 64;
-    const int lds_bytes = (w_loads + p_loads) * 1024 + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16 + 8 * 32 * 4;
+    const int ones_bytes = 2 * (g.dil_y * a.PW + g.dil_x) * 80 + 64;
+    const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
     if (!launch_slab_taps<3, 3>(st, a, (int)grid, lds_bytes, rp.enabled != 0))
         return nullptr;
     return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";

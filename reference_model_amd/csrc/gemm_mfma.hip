@@ -634,14 +634,9 @@ static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
     // stages, bias table, per-channel RESCALE constants
     constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
     auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE>;
-    static bool configured     = false;
-    if (!configured)
-    {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes) != hipSuccess)
-            return false;
-        configured = true;
-    }
+    static LdsLimit granted{};
+    if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, granted))
+        return false;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
     return true;
 }

@@ -5,10 +5,33 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "tmi_device.h"
 
 namespace tmi
 {
+
+// A kernel's dynamic LDS limit is a per-device attribute of the function.  `done` holds, per device, the largest
+// size already granted to one kernel instantiation; the attribute is set again only when a launch needs more.
+// Safe for contexts used from different host threads.
+constexpr int kMaxDevices = 16;
+struct LdsLimit
+{
+    std::atomic<size_t> done[kMaxDevices];
+};
+inline bool ensure_dynamic_lds(const void* kernel, size_t bytes, LdsLimit& lim)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return false;
+    if (bytes <= lim.done[dev].load(std::memory_order_acquire))
+        return true;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+        return false;
+    lim.done[dev].store(bytes, std::memory_order_release);
+    return true;
+}
 
 // Validated geometry of a CONV2D / DEPTHWISE_CONV2D call.
 struct ConvGeom
