@@ -121,24 +121,26 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         // with them in the loop, issuing the loads took three times as long as the loads themselves.)
         const uint32_t lbase = (uint32_t)(uintptr_t)lds;
         {
-            const int s0 = wave * 64 + lane;
-            int row      = s0 / RW;
-            int ch       = s0 - row * RW;
-            uint32_t dst = lbase + wave * 1024;
+            // Weights: LDS row r is channel r of the block, so slot s = (row, chunk) reads byte 16 (s - row) of the
+            // block's weights and the walk is two additions; the spare chunk of a row reads the next row's first
+            // chunk, and whatever lies past the block's last channel (a ragged last block, the last spare chunk)
+            // is clamped to its last chunk: valid memory whose results are never stored.
+            const int s0         = wave * 64 + lane;
+            const int row0       = s0 / RW;
+            int ch               = s0 - row0 * RW;
+            uint32_t off         = 16u * (uint32_t)(s0 - row0);
+            const int rows       = a.OC - oc0 < 64 ? a.OC - oc0 : 64;
+            const uint32_t limit = (uint32_t)rows * (TAPS * 64) - 16u;
+            const uint8_t* wb    = a.w + (size_t)oc0 * (TAPS * 64);
+            uint32_t dst         = lbase + wave * 1024;
             for (int l = wave; l < WLOADS; l += LWAVES)
             {
-                // row r of a 32-row MFMA operand tile holds channel 16*((r>>2)&1) + 4*(r>>3) + (r&3) of the tile,
-                // which makes a lane's 16 accumulators 16 consecutive channels; rows of channels past OC read
-                // channel 0 of the block (valid memory, results never stored)
-                const int r   = row < 64 ? row : 63;
-                const int chn = (r & 32) + 4 * (r & 4) + ((r >> 1) & 12) + (r & 3);
-                const int c   = oc0 + (oc0 + chn < a.OC ? chn : 0);
-                slab_load_off(__umul24(c, TAPS * 64) + (ch < RW - 1 ? ch : 0) * 16, a.w, dst);
+                slab_load_off(off < limit ? off : limit, wb, dst);
                 dst += LWAVES * 1024;
-                row += (LWAVES * 64) / RW;
+                off += 16u * (LWAVES * 64 - (LWAVES * 64) / RW);
                 ch += (LWAVES * 64) % RW;
                 if (ch >= RW)
-                    ch -= RW, row++;
+                    ch -= RW, off -= 16u;
             }
         }
         {
@@ -219,7 +221,11 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     const bool wave_active = pxt * PXW < P;    // wave-uniform
     if (wave_active)
     {
-        const uint8_t* wrow = wl + ((oct * 32 + li) * RW) * 16 + lh * 16;
+        // MFMA operand row li holds channel 16*((li>>2)&1) + 4*(li>>3) + (li&3) of the wave's 32: a lane's 16
+        // accumulators are then 16 consecutive channels.  (The 16 lanes a ds_read_b128 serves together still read
+        // rows that differ modulo 16, which the odd row stride turns into 16 different bank groups.)
+        const int wr        = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
+        const uint8_t* wrow = wl + ((oct * 32 + wr) * RW) * 16 + lh * 16;
         const uint8_t* prow = pl + ((ty * a.sy * a.PW + tx * a.sx) * RP) * 16 + lh * 16;
         if (ZA && li == PXW)
             prow = ones + lh * 16;
