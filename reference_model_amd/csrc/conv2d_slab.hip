@@ -9,8 +9,8 @@
 //     stores, and only address arithmetic on the vector ALU.  Seven waves issue about seven loads each.
 //   - An LDS destination is fixed (M0 + 16 * lane) but every lane names its own source, so the layout is chosen
 //     by the mapping slot -> source: weight rows take taps*4 + 1 chunks and patch pixels 5, the odd chunk being
-//     padding.  Both strides are then congruent to 16 modulo 32 bytes, the layout on which a 32-row ds_read_b128
-//     fragment load runs at the full LDS rate.
+//     padding, and a patch row gets up to 15 more chunks of padding.  The 16 lanes that a ds_read_b128 serves
+//     together then read 16 different bank groups, for the weight fragments and (odd strides) the pixel fragments.
 //   - A pixel outside the image reads a 64-byte page of input_zp bytes, so it contributes
 //     (zp - zp) * w = 0 like the reference's skipped tap (tensor_ops.cpp:845-852), and the zero-point identity
 //     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  sum(w) per channel costs nothing: a wave's
@@ -46,8 +46,9 @@ struct SlabArgs
     int32_t n_ocb;
     int32_t out_kind;    // 0: int32 accumulators, 1: int8 through the RESCALE, 2: int16 through the RESCALE
     int32_t xcd_remap;
-    int32_t step_py, step_px;    // 89 = step_py * PW + step_px: how far 7 loads (448 slots = 89 pixels + 3 chunks) move
-    FastDiv div_tw, div_pw, div_tiles_x, div_tiles_y, div_ocb;
+    int32_t pitch;               // 16-byte chunks per patch row in LDS: 5 per pixel plus the padding that spreads the banks
+    int32_t step_row, step_chunk;    // 448 = step_row * pitch + step_chunk: how far 7 loads (448 slots) move
+    FastDiv div_tw, div_pitch, div_tiles_x, div_tiles_y, div_ocb;
 };
 
 __device__ __forceinline__ void slab_load(const void* src, uint32_t lds_addr)
@@ -80,12 +81,12 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li     = lane & 31;
     const int lh     = lane >> 5;
-    const int p_slots = a.PH * a.PW * RP;
+    const int p_slots = a.PH * a.pitch;
     const int p_loads = (p_slots + 63) >> 6;
     uint8_t* wl       = lds;
     uint8_t* pl       = lds + WLOADS * 1024;
     // fragment offsets of the taps inside the patch, and the "pixel of ones": bytes 0x01 wherever a tap can read
-    const int row_step   = a.dy * a.PW * RP * 16;
+    const int row_step   = a.dy * a.pitch * 16;
     const int col_step   = a.dx * RP * 16;
     const int ones_bytes = ZA ? ((KH - 1) * row_step + (KW - 1) * col_step + 64) : 0;
     uint8_t* ones        = pl + p_loads * 1024;
@@ -117,8 +118,8 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     {
         // Load l fills LDS bytes [1024 l, 1024 l + 1024); wave v issues l = v, v + 7, ...  The per-lane source is
         // worked out once with divisions and then walked: 7 loads on are 448 slots, i.e. 12 weight rows and 4 chunks,
-        // or 89 patch pixels and 3 chunks.  (Integer multiplies and divides run at a quarter of the vector rate;
-        // with them in the loop, issuing the loads took three times as long as the loads themselves.)
+        // or step_row patch rows and step_chunk chunks.  (Integer multiplies and divides run at a quarter of the
+        // vector rate; with them in the loop, issuing the loads took three times as long as the loads themselves.)
         const uint32_t lbase = (uint32_t)(uintptr_t)lds;
         {
             // Weights: LDS row r is channel r of the block, so slot s = (row, chunk) reads byte 16 (s - row) of the
@@ -145,29 +146,24 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         }
         {
             const uint8_t* in_n = a.in + (size_t)n * a.IH * a.IW * 64;
-            const int n_pix     = a.PH * a.PW;
             int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
             const int s0        = lp * 64 + lane;
-            int pix             = (int)(((uint32_t)s0 * 52429u) >> 18);    // s0 / 5 for s0 < 2^16
-            int ch              = s0 - pix * RP;
-            int py              = fdiv(pix, a.div_pw);
-            int px              = pix - py * a.PW;
+            int py              = fdiv(s0, a.div_pitch);    // patch row and chunk inside the row
+            int r               = s0 - py * a.pitch;
             uint32_t dst        = lbase + (WLOADS + lp) * 1024;
             for (; lp < p_loads; lp += LWAVES)
             {
+                const int px   = (int)(((uint32_t)r * 52429u) >> 18);    // r / 5 for r < 2^16
+                const int ch   = r - px * RP;
                 const int iy = y0 + py, ix = x0 + px;
-                const bool img = pix < n_pix && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+                const bool img = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
                 const int c16  = (ch < 4 ? ch : 0) * 16;
                 const uint8_t* src = img ? in_n + (uint32_t)((__umul24(iy, a.IW) + ix) * 64 + c16) : a.pad_page + c16;
                 slab_load(src, dst);
                 dst += LWAVES * 1024;
-                ch += (LWAVES * 64) % RP;
-                pix += (LWAVES * 64) / RP;
-                px += a.step_px, py += a.step_py;
-                if (ch >= RP)
-                    ch -= RP, pix++, px++;
-                if (px >= a.PW)
-                    px -= a.PW, py++;
+                r += a.step_chunk, py += a.step_row;
+                if (r >= a.pitch)
+                    r -= a.pitch, py++;
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -226,7 +222,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         // rows that differ modulo 16, which the odd row stride turns into 16 different bank groups.)
         const int wr        = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
         const uint8_t* wrow = wl + ((oct * 32 + wr) * RW) * 16 + lh * 16;
-        const uint8_t* prow = pl + ((ty * a.sy * a.PW + tx * a.sx) * RP) * 16 + lh * 16;
+        const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * RP) * 16 + lh * 16;
         if (ZA && li == PXW)
             prow = ones + lh * 16;
 #pragma unroll
@@ -401,7 +397,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
             {
                 const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
                 const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
-                if (ph * pw * 5 >= (1 << 16) || ph * pw * 80 > 96 * 1024)
+                if (ph * (pw * 5 + 15) >= (1 << 16) || ph * (pw * 5 + 15) * 16 > 96 * 1024)
                     continue;
                 const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
                 const int64_t rounds = (tiles + 255) / 256;
@@ -431,12 +427,24 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     if (grid >= (int64_t(1) << 31))
         return nullptr;
     a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? 1 : 0;
-    a.step_py = 89 / a.PW, a.step_px = 89 % a.PW;
-    a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pw = make_fastdiv((uint32_t)a.PW);
+    // A patch pixel is 5 chunks; the chunk of output pixel (ty, tx) under tap (0, 0) is ty * sy * pitch + 5 * sx * tx.
+    // A ds_read_b128 serves 16 lanes together, whose chunks must differ modulo 16.  The lanes of a wave are consecutive
+    // tile pixels p = ty * TW + tx, and any 16 lanes served together differ modulo 16, so the reads are free of bank
+    // conflicts when the chunk is an odd multiple of p plus a constant (modulo 16): 5 * sx odd and
+    // sy * pitch = 5 * sx * TW (mod 16).  Up to 15 chunks of padding per patch row arrange that for odd strides;
+    // even strides keep pitch = 5 * PW and their conflicts.
+    int pad = 0;
+    if ((g.stride_x & 1) && (g.stride_y & 1))
+        for (pad = 0; pad < 16; pad++)
+            if (((g.stride_y * (a.PW * 5 + pad) - 5 * g.stride_x * a.TW) & 15) == 0)
+                break;
+    a.pitch     = a.PW * 5 + (pad & 15);
+    a.step_row  = 448 / a.pitch, a.step_chunk = 448 % a.pitch;
+    a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pitch = make_fastdiv((uint32_t)a.pitch);
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
-    const int w_loads = (64 * (9 * 4 + 1) + 63) / 64, p_loads = (a.PH * a.PW * 5 + 63) / 64;
-    const int ones_bytes = 2 * (g.dil_y * a.PW + g.dil_x) * 80 + 64;
+    const int w_loads = (64 * (9 * 4 + 1) + 63) / 64, p_loads = (a.PH * a.pitch + 63) / 64;
+    const int ones_bytes = 2 * (g.dil_y * a.pitch * 16 + g.dil_x * 80) + 64;
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
     if (!launch_slab_taps<3, 3>(st, a, (int)grid, lds_bytes, rp.enabled != 0))
         return nullptr;
