@@ -119,8 +119,8 @@ int tmi_download(tmi_ctx_t* ctx, void* dst_host, const void* src_dev, size_t byt
  * OpConv2d::eval / OpDepthwiseConv2d::eval (reference_model/src/ops/tensor_ops.cpp:725-758, 1174-1207). */
 typedef struct
 {
-    int32_t in_dtype;    /* TMI_INT8, TMI_FP16 or TMI_BF16 (weight has the same type)               */
-    int32_t out_dtype;   /* TMI_INT32 for INT8 input; TMI_FP16 / TMI_BF16 (same as input) otherwise  */
+    int32_t in_dtype;    /* TMI_INT8, TMI_FP16, TMI_BF16 or TMI_FP32 (weight has the same type)     */
+    int32_t out_dtype;   /* TMI_INT32 for INT8 input; the input type otherwise                       */
     int32_t N, IH, IW, IC;
     int32_t OC;          /* CONV2D: weight dim 0.  DEPTHWISE: IC * M (output channels)               */
     int32_t KH, KW;
@@ -193,8 +193,9 @@ typedef struct
 /* ---- operators --------------------------------------------------------------------------------- */
 
 /* OpConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:723-882 (checks :120-226, :690-720).
- * INT8 x INT8 -> INT32 with int32 accumulation, or FP16 / BF16 with fp32 accumulation and an output of
- * the input type.  in_zp / w_zp are the values of operands 3 and 4 (must be 0 for non-INT8). */
+ * INT8 x INT8 -> INT32 with int32 accumulation, or FP16 / BF16 / FP32 with fp32 accumulation and an output
+ * of the input type (the instantiations at :2220-2229; FP32 runs on the one-element-per-lane kernels, in the
+ * reference's summation order).  in_zp / w_zp are the values of operands 3 and 4 (must be 0 for non-INT8). */
 int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
@@ -203,7 +204,7 @@ int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* i
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
 /* OpMatMul::eval, reference_model/src/ops/tensor_ops.cpp:1423-1492 (checks :1347-1420).
- * in_dtype TMI_INT8 -> INT32 output; TMI_FP16 / TMI_BF16 -> FP32 output (fp32 accumulation). */
+ * in_dtype TMI_INT8 -> INT32 output; TMI_FP16 / TMI_BF16 / TMI_FP32 -> FP32 output (fp32 accumulation). */
 int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
                const void* b_dev, int32_t a_zp, int32_t b_zp, void* out_dev);
 

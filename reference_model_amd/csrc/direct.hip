@@ -32,6 +32,15 @@ struct Elem<_Float16>
     }
 };
 template <>
+struct Elem<float>
+{
+    using acc_t = float;
+    __device__ static acc_t load(const float* p, int64_t i)
+    {
+        return p[i];
+    }
+};
+template <>
 struct Elem<bf16_t>
 {
     using acc_t = float;
@@ -227,6 +236,11 @@ static int grid_for(int64_t work_items)
             TMI_LAUNCH_CONV(KERNEL, bf16_t, bf16_t);                                                                \
             return LABEL "_bf16";                                                                                   \
         }                                                                                                           \
+        if (in_dtype == TMI_FP32 && out_dtype == TMI_FP32)                                                          \
+        {                                                                                                           \
+            TMI_LAUNCH_CONV(KERNEL, float, float);                                                                  \
+            return LABEL "_f32";                                                                                    \
+        }                                                                                                           \
         return nullptr;                                                                                             \
     }
 
@@ -256,6 +270,12 @@ const char* launch_matmul_direct(hipStream_t st, int32_t in_dtype, int32_t N, in
         hipLaunchKernelGGL((matmul_direct_kernel<bf16_t, float>), dim3(grid_for(total)), dim3(256), 0, st, N, H, C,
                            W, (const bf16_t*)a, (const bf16_t*)b, 0, 0, (float*)out);
         return "matmul_direct_bf16";
+    }
+    if (in_dtype == TMI_FP32)
+    {
+        hipLaunchKernelGGL((matmul_direct_kernel<float, float>), dim3(grid_for(total)), dim3(256), 0, st, N, H, C, W,
+                           (const float*)a, (const float*)b, 0, 0, (float*)out);
+        return "matmul_direct_f32";
     }
     return nullptr;
 }

@@ -53,6 +53,13 @@ bool Tensor::scalar_value(int32_t& v) const
             v = (t & 0x7fff) ? 1 : 0;    // any non-zero floating-point zero point is illegal anyway
             return true;
         }
+        case DType_FP32:
+        {
+            uint32_t t;
+            memcpy(&t, host.data(), 4);
+            v = (t & 0x7fffffffu) ? 1 : 0;
+            return true;
+        }
         default:
             return false;
     }
@@ -648,7 +655,7 @@ public:
         if (inputs[3]->shape[0] != 1)
             return error("OpMatMul: 'b_zp' zero point shape should be [1]");
         const DType in = a->getDtype();
-        if (b->getDtype() != in || !(in == DType_INT8 || in == DType_FP16 || in == DType_BF16))
+        if (b->getDtype() != in || !(in == DType_INT8 || in == DType_FP16 || in == DType_BF16 || in == DType_FP32))
             return error("OpMatMul: input data type not supported for this configuration of operator");
         if (o->getDtype() != (in == DType_INT8 ? DType_INT32 : DType_FP32))
             return error("OpMatMul: Output data type not supported for this configuration of operator");

@@ -112,7 +112,7 @@ int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool d
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 && d->in_dtype != TMI_FP32)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     const int32_t want_out = d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype;
     if (d->out_dtype != want_out)
@@ -789,7 +789,7 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
 {
     if (!ctx)
         return TMI_ERROR;
-    if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
+    if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16 && in_dtype != TMI_FP32)
         return fail(ctx, "OpMatMul: input data type not supported for this configuration of operator");
     if (N < 0 || H < 0 || C < 0 || W < 0)
         return fail(ctx, "OpMatMul: negative tensor dimension");
@@ -810,7 +810,7 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
         return TMI_VALID;
     }
     const char* name = nullptr;
-    if (ctx->kernel_choice != 1 && C > 0)
+    if (ctx->kernel_choice != 1 && C > 0 && in_dtype != TMI_FP32)
     {
         // MFMA paths: one "image" per batch, pixels = rows of A, output channels = columns of B, 1x1 taps,
         // per-image weights.  The bias operand is the permanently zero word kept after the flags.  The GEMM

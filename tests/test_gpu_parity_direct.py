@@ -305,3 +305,43 @@ def test_bf16_direct_matmul(ctx):
     want = oracle.matmul("f32", cases.bf16_bits_to_float(a), cases.bf16_bits_to_float(b))
     got, st = gpu_ops.matmul(ctx, a, b, dtype=capi.BF16)
     assert st == capi.VALID and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ---- FP32 CONV2D / DEPTHWISE_CONV2D / MATMUL (OpConv2d<FP32,FP32,FP32,FP32> etc., tensor_ops.cpp:2220-2270) ----
+@pytest.mark.parametrize("shape", [
+    # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
+    (1, 32, 32, 8, 16, 1, 1, (0, 0, 0, 0), (1, 1), (1, 1)),      # the reference's FP32 example geometry
+    (2, 9, 11, 5, 7, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),
+    (1, 12, 10, 6, 4, 3, 2, (0, 1, 1, 0), (2, 1), (1, 2)),
+])
+def test_conv2d_fp32_reproduces_the_reference_summation_order(ctx, shape):
+    """the one-element-per-lane kernel adds the products in the reference's ky -> kx -> ic order with separate
+    multiplies and adds, like the oracle's loop nest: equal bit for bit"""
+    n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
+    rng = np.random.default_rng(ic * oc + kh)
+    x = rng.normal(0, 1, (n, ih, iw, ic)).astype(np.float32)
+    w = rng.normal(0, 0.3, (oc, kh, kw, ic)).astype(np.float32)
+    b = rng.normal(0, 1, oc).astype(np.float32)
+    got, st = gpu_ops.conv2d(ctx, x, w, b, pad, stride, dil, dtype=capi.FP32)
+    assert st == capi.VALID and ctx.last_kernel == "conv2d_direct_f32" and got.dtype == np.float32
+    assert np.array_equal(got, oracle.conv2d("f32", x, w, b, pad, stride, dil))
+    # and within a few fp32 roundings of the fp64 result
+    ref = oracle.conv2d("f64", x.astype(np.float64), w.astype(np.float64), b.astype(np.float64), pad, stride, dil)
+    assert np.allclose(got, ref, rtol=1e-5, atol=1e-5)
+
+
+def test_depthwise_and_matmul_fp32(ctx):
+    rng = np.random.default_rng(32)
+    x = rng.normal(0, 1, (2, 9, 8, 6)).astype(np.float32)
+    w = rng.normal(0, 0.5, (3, 3, 6, 2)).astype(np.float32)
+    b = rng.normal(0, 1, 12).astype(np.float32)
+    got, st = gpu_ops.conv2d(ctx, x, w, b, (1, 1, 1, 1), depthwise=True, dtype=capi.FP32)
+    assert st == capi.VALID and ctx.last_kernel == "depthwise_direct_f32"
+    assert np.array_equal(got, oracle.depthwise_conv2d("f32", x, w, b, (1, 1, 1, 1)))
+    a = rng.normal(0, 1, (3, 7, 20)).astype(np.float32)
+    bm = rng.normal(0, 1, (3, 20, 5)).astype(np.float32)
+    got, st = gpu_ops.matmul(ctx, a, bm, dtype=capi.FP32)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_direct_f32"
+    assert np.array_equal(got, oracle.matmul("f32", a, bm))
+    with pytest.raises(TmiError):      # zero points are for INT8 only (tensor_ops.cpp:1433-1434)
+        gpu_ops.matmul(ctx, a, bm, a_zp=1, dtype=capi.FP32)

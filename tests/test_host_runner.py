@@ -117,6 +117,21 @@ def test_reference_qi8_example_directory(golden_dir, tmp_path, fusion):
 
 
 @pytest.mark.gpu
+def test_reference_f32_example_directory(golden_dir, tmp_path):
+    """the graph of the reference's conv2d_f32_test (test/model_runner_tests.cpp:85-125), compared the way that test
+    compares: doctest::Approx with its default epsilon (100 float epsilons relative to 1 + |value|)"""
+    out = str(tmp_path / "out.npy")
+    r = _run(os.path.join(golden_dir, "f32_conv2d_1x1", "desc.json"), f"--ofm_file={out}")
+    assert r.returncode == 0, r.stderr
+    want = np.load(os.path.join(golden_dir, "f32_conv2d_1x1", "tflite_result.npy")).astype(np.float64)
+    got = np.load(out)
+    assert got.dtype == np.float32 and got.shape == want.shape
+    eps = float(np.finfo(np.float32).eps) * 100
+    assert (np.abs(got - want) < eps * (1.0 + np.maximum(np.abs(got), np.abs(want)))).all()
+    assert np.array_equal(got, want.astype(np.float32))    # the same eight products in the same order: bit for bit
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("which", ["conv_rescale_clamp", "depthwise_rescale"])
 def test_synthetic_graphs_match_oracle(tmp_path, which):
     depthwise = which == "depthwise_rescale"
