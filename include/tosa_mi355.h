@@ -263,7 +263,7 @@ int tmi_max_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev,
  * (--precise_mode: all floating-point tensors in fp64, reference_model/src/main.cpp and the FP64 instantiations
  * of op_factory.cpp) and in bounds mode (the same sums over absolute values, tensor_ops.cpp:757-765,
  * 1213-1221, 1436-1443).  These entries compute either pass on the device: operands in their storage type
- * (TMI_FP16 / TMI_BF16), fp64 products and sums in the reference's loop order, fp64 output of the operator's
+ * (TMI_FP16 / TMI_BF16 / TMI_FP32), fp64 products and sums in the reference's loop order, fp64 output of the operator's
  * output shape.  bounds_mode != 0 selects the sums of absolute values. */
 int tmi_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                        const void* bias_dev, int32_t bounds_mode, double* out_dev);

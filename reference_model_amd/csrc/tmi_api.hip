@@ -870,7 +870,7 @@ static int run_conv_precise(tmi_ctx* ctx, const char* op, bool depthwise, const 
     int rc = validate_conv(ctx, op, d, depthwise, 0, 0, g);
     if (rc != TMI_VALID)
         return rc;
-    if (d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    if (d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 && d->in_dtype != TMI_FP32)
         return fail(ctx, "%s: the precise / bounds passes take floating-point operands", op);
     const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
     if (total > 0 && (!in || !w || !bias || !out))
@@ -908,7 +908,7 @@ int tmi_matmul_precise(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, i
 {
     if (!ctx)
         return TMI_ERROR;
-    if (in_dtype != TMI_FP16 && in_dtype != TMI_BF16)
+    if (in_dtype != TMI_FP16 && in_dtype != TMI_BF16 && in_dtype != TMI_FP32)
         return fail(ctx, "OpMatMul: the precise / bounds passes take floating-point operands");
     if (N < 0 || H < 0 || C < 0 || W < 0)
         return fail(ctx, "OpMatMul: negative tensor dimension");

@@ -26,6 +26,8 @@ def narrow(values, kind):
         with np.errstate(over="ignore"):     # set 1 puts a bias beyond the fp16 range: it becomes infinity, as
             h = values.astype(np.float16)    # in the reference's generator, and the check's overflow rule applies
         return h, h.astype(np.float64), capi.FP16
+    if kind == "fp32":
+        return values, values.astype(np.float64), capi.FP32
     b = cases.float_to_bf16_bits(values)
     return b, cases.bf16_bits_to_float(b).astype(np.float64), capi.BF16
 
@@ -43,7 +45,7 @@ CONV_CASES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
 
 
 @pytest.mark.parametrize("shape", CONV_CASES)
-@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "fp32"])
 @pytest.mark.parametrize("bounds", [False, True])
 def test_conv2d_precise_and_bounds_match_the_fp64_oracle(ctx, shape, kind, bounds):
     n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
@@ -61,7 +63,7 @@ def test_conv2d_precise_and_bounds_match_the_fp64_oracle(ctx, shape, kind, bound
     assert np.array_equal(out.numpy(), want)
 
 
-@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "fp32"])
 @pytest.mark.parametrize("bounds", [False, True])
 def test_depthwise_and_matmul_precise_match_the_fp64_oracle(ctx, kind, bounds):
     rng = np.random.default_rng(17)
@@ -159,6 +161,45 @@ def test_config5_fp16_conv_compliance_on_the_device(ctx, data_set):
         ctx.conv2d_precise(d, tx, tw, tb, False, ref)
         ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
         r = ctx.dot_product_check(capi.FP16, int(np.prod(shape)), imp, ref, bnd, dp.kernel_size_bound(ks, "fp16"), data_set)
+        assert r.compliant and r.failed_elements == 0, (r.max_abs_err, r.err_sum, r.err_sumsq)
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+
+@pytest.mark.parametrize("data_set", range(6))
+def test_fp32_conv_and_matmul_compliance_on_the_device(ctx, data_set):
+    """FP32 operators (fp32 accumulation in the reference's order) on the specification's data sets, whose fp32
+    generator output is pinned bit for bit by the reference's goldens: implementation, fp64 precise pass, bounds
+    pass and DOT_PRODUCT check (ksb = KS + 1 with a bias, fp32 accumulator and result) on the GPU."""
+    n, hw, ic, oc = 2, 14, 48, 24
+    ks = 9 * ic
+    xs = oracle.dot_product_data("conv2d", data_set, 0, ks, (n, hw, hw, ic), kind="fp32", kernel=(3, 3))
+    ws = oracle.dot_product_data("conv2d", data_set, 1, ks, (oc, 3, 3, ic), kind="fp32")
+    bs = oracle.dot_product_data("conv2d", data_set, 2, ks, (oc,), kind="fp32")
+    d = ctx.conv_desc(capi.FP32, capi.FP32, xs.shape, oc, 3, 3, (hw, hw), (1, 1, 1, 1), (1, 1), (1, 1), oc)
+    shape = (n, hw, hw, oc)
+    try:
+        tx, tw, tb = ctx.upload(xs, capi.FP32), ctx.upload(ws, capi.FP32), ctx.upload(bs, capi.FP32)
+        imp, ref, bnd = ctx.empty(shape, capi.FP32), ctx.empty(shape, capi.F64), ctx.empty(shape, capi.F64)
+        ctx.conv2d(d, tx, tw, tb, 0, 0, imp)
+        assert ctx.last_kernel == "conv2d_direct_f32"
+        ctx.conv2d_precise(d, tx, tw, tb, False, ref)
+        ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
+        r = ctx.dot_product_check(capi.FP32, int(np.prod(shape)), imp, ref, bnd, dp.kernel_size_bound(ks, "fp32"), data_set)
+        assert r.compliant and r.failed_elements == 0, (r.max_abs_err, r.err_sum, r.err_sumsq)
+        assert np.array_equal(ref.numpy(), oracle.conv2d("f64", xs.astype(np.float64), ws.astype(np.float64),
+                                                         bs.astype(np.float64), (1, 1, 1, 1), (1, 1), (1, 1)))
+        nb, h, c, w = 2, 24, 200, 16
+        a_s = oracle.dot_product_data("matmul", data_set, 0, c, (nb, h, c), kind="fp32")
+        b_s = oracle.dot_product_data("matmul", data_set, 1, c, (nb, c, w), kind="fp32")
+        ta, tb2 = ctx.upload(a_s, capi.FP32), ctx.upload(b_s, capi.FP32)
+        imp, ref, bnd = ctx.empty((nb, h, w), capi.FP32), ctx.empty((nb, h, w), capi.F64), ctx.empty((nb, h, w), capi.F64)
+        ctx.matmul(capi.FP32, nb, h, c, w, ta, tb2, 0, 0, imp)
+        assert ctx.last_kernel == "matmul_direct_f32"
+        ctx.matmul_precise(capi.FP32, nb, h, c, w, ta, tb2, False, ref)
+        ctx.matmul_precise(capi.FP32, nb, h, c, w, ta, tb2, True, bnd)
+        r = ctx.dot_product_check(capi.FP32, nb * h * w, imp, ref, bnd, dp.kernel_size_bound(c, "fp32", has_bias=False), data_set)
         assert r.compliant and r.failed_elements == 0, (r.max_abs_err, r.err_sum, r.err_sumsq)
     finally:
         for t in list(ctx._owned):
