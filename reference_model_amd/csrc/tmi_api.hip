@@ -319,7 +319,10 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         ctx->last_kernel = "empty";
         return TMI_VALID;
     }
-    if (depthwise && ctx->kernel_choice != 1)
+    if (depthwise && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
+        name = launch_depthwise_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                     ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);
+    if (depthwise && !name && ctx->kernel_choice != 1 && ctx->kernel_choice != 4)
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
     if (!depthwise && ctx->kernel_choice != 1)

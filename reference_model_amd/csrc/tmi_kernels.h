@@ -112,6 +112,12 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                void* out, const void* pad_page, uint32_t* flag_word);
 
+// depthwise_slab.hip: int8 DEPTHWISE_CONV2D with multiplier 1, 3x3 taps, weight_zp = 0 and 32..512 channels in
+// multiples of 16 on the matrix cores (one MFMA per tap against a diagonal weight tile); nullptr for anything else.
+const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                                  const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                                  void* out, const void* pad_page, uint32_t* flag_word);
+
 // gemm_mfma.hip: whether a CONV2D left to automatic choice tries the GEMM kernel before the patch kernel.
 bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g);
 
