@@ -184,13 +184,24 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             // all share one
             const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
             const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
-            tab_cs[lane]          = cs;
             m                     = cs.m;
-            // One shift of at least 32 for the whole block, small enough for output_zp to ride in the rounding
-            // term: the epilogue keeps the rounding terms in scalar registers and reads 8 bytes per channel.
-            const int uni = __all(cs.s == s_first) && s_first >= 32 && s_first <= zp_fold_max_shift(a.rp.out_zp);
+            // The epilogue has three forms:
+            //   every shift >= 32 and small enough for output_zp * 2^shift to ride in the 64-bit rounding term: the
+            //   result is the high word of the sum shifted by shift - 32, no value-range test (-2);
+            //   the same with one shift for the whole block: the rounding terms are scalars and a channel needs 8
+            //   bytes of constants (the shift itself);
+            //   anything else: fast_rescale() with its range test and a 64-bit shift (-1).
+            const int folds = __all(cs.s >= 32 && cs.s <= zp_fold_max_shift(a.rp.out_zp));
+            const int uni   = folds && __all(cs.s == s_first);
+            ChannelScale e  = cs;
+            if (folds)
+            {
+                const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
+                e.rnd_pos += zp_term, e.rnd_neg += zp_term;
+            }
+            tab_cs[lane] = e;
             if (lane == 0)
-                *uni_shift = uni ? s_first : -1;
+                *uni_shift = uni ? s_first : (folds ? -2 : -1);
         }
         tab_mb[lane] = int2{ m, ok ? b : 0 };
         for (int i = lane * 16; i < ones_bytes; i += 1024)
@@ -291,6 +302,17 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 const int32_t v  = acc[e] + cb[e];
                 const int64_t pr = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? rnd_p : rnd_n);
                 r[e]             = clamp_med3((int32_t)(pr >> 32) >> sh, a.rp.lo, a.rp.hi);
+            }
+        }
+        else if (s_uni == -2)
+        {
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+            {
+                const ChannelScale cs = tab_cs[ocl + e];
+                const int32_t v       = acc[e] + cb[e];
+                const int64_t pr      = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? cs.rnd_pos : cs.rnd_neg);
+                r[e]                  = clamp_med3((int32_t)(pr >> 32) >> (cs.s - 32), a.rp.lo, a.rp.hi);
             }
         }
         else
