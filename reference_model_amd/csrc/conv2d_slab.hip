@@ -1,5 +1,5 @@
-// CONV2D for layers whose channel vector is exactly 64 bytes (int8 with IC = 64), 3x3 taps: the small, latency-bound
-// layers of a ResNet stem, where a launch does well under a microsecond of matrix work and everything else is
+// CONV2D for layers whose channel vector is 64 or 128 bytes (int8 with IC = 64 or 128), 3x3 taps: the small,
+// latency-bound layers of a ResNet stem, where a launch does well under a microsecond of matrix work and everything else is
 // overhead.  The kernel is the shortest path from memory to the matrix cores this chip offers:
 //
 //   - A workgroup (8 waves) owns a TH x TW tile of output pixels of one image and a block of 64 output channels.
@@ -8,7 +8,7 @@
 //     global_load_lds_dwordx4 (64 lanes x 16 bytes to 1 KB of LDS per instruction): no staging registers, no LDS
 //     stores, and only address arithmetic on the vector ALU.  Seven waves issue about seven loads each.
 //   - An LDS destination is fixed (M0 + 16 * lane) but every lane names its own source, so the layout is chosen
-//     by the mapping slot -> source: weight rows take taps*4 + 1 chunks and patch pixels 5, the odd chunk being
+//     by the mapping slot -> source: weight rows take taps*CH + 1 chunks and patch pixels CH + 1, the odd chunk being
 //     padding, and a patch row gets up to 15 more chunks of padding.  The 16 lanes that a ds_read_b128 serves
 //     together then read 16 different bank groups, for the weight fragments and (odd strides) the pixel fragments.
 //   - A pixel outside the image reads a 64-byte page of input_zp bytes, so it contributes
@@ -63,16 +63,18 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
                  : "memory");
 }
 
-template <int KH, int KW, bool ZA, bool FUSED>
+// CH: 16-byte chunks of a channel vector (4: 64 input channels, 8: 128)
+template <int KH, int KW, int CH, bool ZA, bool FUSED>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
     asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len), "s"(a.div_ocb.d));
     constexpr int TAPS   = KH * KW;
-    constexpr int RW     = TAPS * 4 + 1;    // chunks per weight row in LDS
+    constexpr int RW     = TAPS * CH + 1;    // chunks per weight row in LDS (odd)
+    constexpr int KB     = CH * 16;          // bytes of a channel vector
     constexpr int WSLOTS = 64 * RW;
     constexpr int WLOADS = (WSLOTS + 63) / 64;
-    constexpr int RP     = 5;               // chunks per patch pixel in LDS
+    constexpr int RP     = CH + 1;          // chunks per patch pixel in LDS (odd)
     constexpr int LWAVES = 7;               // waves that issue loads; the eighth builds the tables
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // LDS: [weight rows][patch][pixel of ones][64 x ChannelScale][64 x (multiplier, bias)][the block's common shift]
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     // fragment offsets of the taps inside the patch, and the "pixel of ones": bytes 0x01 wherever a tap can read
     const int row_step   = a.dy * a.pitch * 16;
     const int col_step   = a.dx * RP * 16;
-    const int ones_bytes = ZA ? ((KH - 1) * row_step + (KW - 1) * col_step + 64) : 0;
+    const int ones_bytes = ZA ? ((KH - 1) * row_step + (KW - 1) * col_step + KB) : 0;
     uint8_t* ones        = pl + p_loads * 1024;
     uint8_t* tabs        = ones + ones_bytes;
     ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tabs);
@@ -131,8 +133,8 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             int ch               = s0 - row0 * RW;
             uint32_t off         = 16u * (uint32_t)(s0 - row0);
             const int rows       = a.OC - oc0 < 64 ? a.OC - oc0 : 64;
-            const uint32_t limit = (uint32_t)rows * (TAPS * 64) - 16u;
-            const uint8_t* wb    = a.w + (size_t)oc0 * (TAPS * 64);
+            const uint32_t limit = (uint32_t)rows * (TAPS * KB) - 16u;
+            const uint8_t* wb    = a.w + (size_t)oc0 * (TAPS * KB);
             uint32_t dst         = lbase + wave * 1024;
             for (int l = wave; l < WLOADS; l += LWAVES)
             {
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             }
         }
         {
-            const uint8_t* in_n = a.in + (size_t)n * a.IH * a.IW * 64;
+            const uint8_t* in_n = a.in + (size_t)n * a.IH * a.IW * KB;
             int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
             const int s0        = lp * 64 + lane;
             int py              = fdiv(s0, a.div_pitch);    // patch row and chunk inside the row
@@ -153,12 +155,12 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             uint32_t dst        = lbase + (WLOADS + lp) * 1024;
             for (; lp < p_loads; lp += LWAVES)
             {
-                const int px   = (int)(((uint32_t)r * 52429u) >> 18);    // r / 5 for r < 2^16
+                const int px   = (int)((uint32_t)r / (uint32_t)RP);
                 const int ch   = r - px * RP;
                 const int iy = y0 + py, ix = x0 + px;
                 const bool img = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
-                const int c16  = (ch < 4 ? ch : 0) * 16;
-                const uint8_t* src = img ? in_n + (uint32_t)((__umul24(iy, a.IW) + ix) * 64 + c16) : a.pad_page + c16;
+                const int c16  = (ch < CH ? ch : 0) * 16;
+                const uint8_t* src = img ? in_n + (uint32_t)((__umul24(iy, a.IW) + ix) * KB + c16) : a.pad_page + (c16 & 48);
                 slab_load(src, dst);
                 dst += LWAVES * 1024;
                 r += a.step_chunk, py += a.step_row;
@@ -241,9 +243,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 #pragma unroll
             for (int kx = 0; kx < KW; kx++)
 #pragma unroll
-                for (int h = 0; h < 2; h++)
+                for (int h = 0; h < CH / 2; h++)
                 {
-                    const v4i fa = *reinterpret_cast<const v4i*>(wrow + ((ky * KW + kx) * 2 + h) * 32);
+                    const v4i fa = *reinterpret_cast<const v4i*>(wrow + ((ky * KW + kx) * (CH / 2) + h) * 32);
                     const v4i fb = *reinterpret_cast<const v4i*>(prow + ky * row_step + kx * col_step + h * 32);
                     acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
                 }
@@ -360,10 +362,10 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     raise_flags(a.flag_word, flags);
 }
 
-template <int KH, int KW, bool ZA, bool FUSED>
+template <int KH, int KW, int CH, bool ZA, bool FUSED>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
-    auto kern              = conv2d_slab_kernel<KH, KW, ZA, FUSED>;
+    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
@@ -371,14 +373,14 @@ static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int 
     return true;
 }
 
-template <int KH, int KW>
+template <int KH, int KW, int CH>
 static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, bool fused)
 {
     if (a.za != 0)
-        return fused ? launch_slab_kernel<KH, KW, true, true>(st, a, grid, lds_bytes)
-                     : launch_slab_kernel<KH, KW, true, false>(st, a, grid, lds_bytes);
-    return fused ? launch_slab_kernel<KH, KW, false, true>(st, a, grid, lds_bytes)
-                 : launch_slab_kernel<KH, KW, false, false>(st, a, grid, lds_bytes);
+        return fused ? launch_slab_kernel<KH, KW, CH, true, true>(st, a, grid, lds_bytes)
+                     : launch_slab_kernel<KH, KW, CH, true, false>(st, a, grid, lds_bytes);
+    return fused ? launch_slab_kernel<KH, KW, CH, false, true>(st, a, grid, lds_bytes)
+                 : launch_slab_kernel<KH, KW, CH, false, false>(st, a, grid, lds_bytes);
 }
 
 // nullptr when the layer is not one this kernel takes; the caller then goes to the patch kernel.
@@ -386,7 +388,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                void* out, const void* pad_page, uint32_t* flag_word)
 {
-    if (in_dtype != TMI_INT8 || g.IC != 64 || g.KH != 3 || g.KW != 3 || w_zp != 0 || !pad_page || !flag_word)
+    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 128) || g.KH != 3 || g.KW != 3 || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
         return nullptr;
@@ -394,20 +396,21 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
         return nullptr;
     if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || ((uintptr_t)bias & 3))
         return nullptr;
-    if ((int64_t)g.N * g.IH * g.IW * 64 >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
+    if ((int64_t)g.N * g.IH * g.IW * g.IC >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
         return nullptr;
 
     // The tile: at most 124 pixels (four tiles of 31 pixels, one per wave and channel tile).  A workgroup moves the
     // weight slab (taps * 64 rows of 64 bytes) plus PH * PW patch rows; whole rounds of 256 workgroups count.
     // The search depends on the geometry only; a caller repeats the same layer, so the last answer is kept.
     const int n_ocb = (g.OC + 63) / 64;
+    const int ch = g.IC / 16, rp_chunks = ch + 1;    // chunks of a channel vector; chunks per patch pixel in LDS
     struct TileChoice
     {
         int32_t key[8];
         int th, tw;
     };
     static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0 };
-    const int32_t key[8] = { g.N, g.OH, g.OW, n_ocb, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
+    const int32_t key[8] = { g.N, g.OH, g.OW, n_ocb * 256 + ch, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
     int best_th = 0, best_tw = 0;
     if (memcmp(key, last.key, sizeof(key)) == 0)
         best_th = last.th, best_tw = last.tw;
@@ -419,12 +422,12 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
             {
                 const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
                 const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
-                if (ph * (pw * 5 + 15) >= (1 << 16) || ph * (pw * 5 + 15) * 16 > 96 * 1024)
+                if (ph * (pw * rp_chunks + 15) >= (1 << 16) || ph * (pw * rp_chunks + 15) * 16 > 64 * 1024)
                     continue;
                 const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
                 const int64_t rounds = (tiles + 255) / 256;
                 // a round costs its loads plus the four 32-pixel MFMA tiles whether they are full or not
-                const int64_t cost = rounds * (9 * 64 + ph * pw + 600);
+                const int64_t cost = rounds * ((9 * 64 + ph * pw) * (ch / 4) + 600);
                 if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
                     best_th = th, best_tw = tw, best_cost = cost;
             }
@@ -449,26 +452,27 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     if (grid >= (int64_t(1) << 31))
         return nullptr;
     a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? 1 : 0;
-    // A patch pixel is 5 chunks; the chunk of output pixel (ty, tx) under tap (0, 0) is ty * sy * pitch + 5 * sx * tx.
+    // A patch pixel is R = CH + 1 chunks; the chunk of output pixel (ty, tx) under tap (0, 0) is ty * sy * pitch + R * sx * tx.
     // A ds_read_b128 serves 16 lanes together, whose chunks must differ modulo 16.  The lanes of a wave are consecutive
     // tile pixels p = ty * TW + tx, and any 16 lanes served together differ modulo 16, so the reads are free of bank
-    // conflicts when the chunk is an odd multiple of p plus a constant (modulo 16): 5 * sx odd and
-    // sy * pitch = 5 * sx * TW (mod 16).  Up to 15 chunks of padding per patch row arrange that for odd strides;
+    // conflicts when the chunk is an odd multiple of p plus a constant (modulo 16): R * sx odd and
+    // sy * pitch = R * sx * TW (mod 16).  Up to 15 chunks of padding per patch row arrange that for odd strides;
     // even strides keep pitch = 5 * PW and their conflicts.
     int pad = 0;
     if ((g.stride_x & 1) && (g.stride_y & 1))
         for (pad = 0; pad < 16; pad++)
-            if (((g.stride_y * (a.PW * 5 + pad) - 5 * g.stride_x * a.TW) & 15) == 0)
+            if (((g.stride_y * (a.PW * rp_chunks + pad) - rp_chunks * g.stride_x * a.TW) & 15) == 0)
                 break;
-    a.pitch     = a.PW * 5 + (pad & 15);
+    a.pitch     = a.PW * rp_chunks + (pad & 15);
     a.step_row  = 448 / a.pitch, a.step_chunk = 448 % a.pitch;
     a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pitch = make_fastdiv((uint32_t)a.pitch);
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
-    const int w_loads = (64 * (9 * 4 + 1) + 63) / 64, p_loads = (a.PH * a.pitch + 63) / 64;
-    const int ones_bytes = 2 * (g.dil_y * a.pitch * 16 + g.dil_x * 80) + 64;
+    const int w_loads = 9 * ch + 1, p_loads = (a.PH * a.pitch + 63) / 64;
+    const int ones_bytes = 2 * (g.dil_y * a.pitch * 16 + g.dil_x * rp_chunks * 16) + g.IC;
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
-    if (!launch_slab_taps<3, 3>(st, a, (int)grid, lds_bytes, rp.enabled != 0))
+    if (!(ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, rp.enabled != 0)
+                  : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, rp.enabled != 0)))
         return nullptr;
     return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";
 }

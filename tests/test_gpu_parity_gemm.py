@@ -322,7 +322,7 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
 # ---- which MFMA kernel a convolution gets when the choice is left open ----
 @pytest.mark.parametrize("dtype, shape, kernel", [
     # n, ih, iw, ic, oc, k, pad
-    (capi.INT8, (8, 56, 56, 128, 64, 3, 1), "conv2d_mfma_i8"),         # 3x3 int8: the patch kernel
+    (capi.INT8, (8, 56, 56, 192, 64, 3, 1), "conv2d_mfma_i8"),         # 3x3 int8: the patch kernel
     (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "conv2d_mfma_i8"),
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
     (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16"),        # 3x3 fp16, deep K

@@ -20,7 +20,7 @@ def ctx():
     c.close()
 
 
-SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation
+SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation[, ic: 64 unless given]
     (8, 56, 56, 64, (1, 1, 1, 1), (1, 1), (1, 1)),      # the headline layer
     (3, 30, 29, 64, (1, 1, 1, 1), (1, 1), (1, 1)),      # ragged tiles in both directions
     (1, 5, 5, 64, (1, 1, 1, 1), (1, 1), (1, 1)),        # one small tile
@@ -31,14 +31,18 @@ SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation
     (2, 34, 31, 64, (0, 1, 1, 0), (2, 1), (1, 1)),      # stride 2 x 1
     (2, 24, 24, 64, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilation 2
     (33, 14, 14, 64, (1, 1, 1, 1), (1, 1), (1, 1)),     # more workgroups than compute units, odd count
+    (4, 28, 28, 128, (1, 1, 1, 1), (1, 1), (1, 1), 128),    # 128 input channels: four MFMA steps per tap
+    (2, 19, 17, 80, (1, 0, 2, 1), (1, 1), (1, 1), 128),     # ragged tiles and channel block
+    (2, 29, 29, 64, (1, 1, 1, 1), (2, 2), (1, 1), 128),     # stride 2
 ]
 
 
 def _operands(shape, seed):
-    n, ih, iw, oc, pad, stride, dil = shape
+    n, ih, iw, oc, pad, stride, dil = shape[:7]
+    ic = shape[7] if len(shape) > 7 else 64
     rng = np.random.default_rng(seed)
-    x = rng.integers(-128, 128, (n, ih, iw, 64)).astype(np.int8)
-    w = rng.integers(-128, 128, (oc, 3, 3, 64)).astype(np.int8)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 3, 3, ic)).astype(np.int8)
     bias = rng.integers(-(1 << 18), 1 << 18, oc).astype(np.int32)
     return x, w, bias
 
@@ -46,7 +50,7 @@ def _operands(shape, seed):
 @pytest.mark.parametrize("shape", SLAB_SHAPES)
 @pytest.mark.parametrize("in_zp", [0, -7, 127, -128])
 def test_slab_conv_int32_bit_exact(ctx, shape, in_zp):
-    n, ih, iw, oc, pad, stride, dil = shape
+    n, ih, iw, oc, pad, stride, dil = shape[:7]
     x, w, bias = _operands(shape, ih * iw + oc)
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
     assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
@@ -87,10 +91,10 @@ def _fused(ctx, c, out_dtype):
 @pytest.mark.parametrize("zps", [(-7, 0), (4, -3), (-128, 100)])
 @pytest.mark.parametrize("out_dtype", [np.int8, np.int16])
 def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
-    n, ih, iw, oc, pad, stride, dil = shape
+    n, ih, iw, oc, pad, stride, dil = shape[:7]
     x, _, _ = _operands(shape, ih + iw + oc)
     rng = np.random.default_rng(oc + ih)
-    c = dict(x=x, w=np.clip(np.rint(rng.normal(0, 30, (oc, 3, 3, 64))), -127, 127).astype(np.int8),
+    c = dict(x=x, w=np.clip(np.rint(rng.normal(0, 30, (oc, 3, 3, x.shape[3]))), -127, 127).astype(np.int8),
              bias=np.rint(rng.normal(0, 1 << 14, oc)).astype(np.int32), in_zp=zps[0], pad=pad, stride=stride,
              dilation=dil, mult=rng.integers(1 << 30, 1 << 31, oc).astype(np.int32),
              shift=rng.integers(36, 42, oc).astype(np.int8), out_zp=zps[1] if out_dtype == np.int8 else 0,
