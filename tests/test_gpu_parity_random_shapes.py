@@ -1,0 +1,80 @@
+"""Seeded random geometries through the two kernels that load their operands straight into LDS (the CONV2D slab
+kernel and the matrix-core DEPTHWISE_CONV2D kernel): the tile search, the padded LDS pitches and the incremental
+source walks depend on the geometry in ways a hand-picked list does not exhaust.  Integer work: bit for bit against
+the CPU oracle."""
+import numpy as np
+import pytest
+
+import gpu_ops
+import oracle
+from reference_model_amd import Context, capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = Context(0)
+    c.set_kernel_choice(capi.KERNEL_SLAB)
+    yield c
+    c.close()
+
+
+def _geometry(rng):
+    """a legal (ih, iw, pad, stride, dilation) for 3x3 taps: (ih - 1 + pad - 2 * dilation) % stride == 0"""
+    while True:
+        stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dil = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        pad = tuple(int(v) for v in rng.integers(0, 3, 4))
+        oh, ow = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        ih = (oh - 1) * stride[0] + 2 * dil[0] + 1 - pad[0] - pad[1]
+        iw = (ow - 1) * stride[1] + 2 * dil[1] + 1 - pad[2] - pad[3]
+        if ih >= 1 and iw >= 1:
+            return ih, iw, pad, stride, dil
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_conv2d_slab_random_geometry(ctx, seed):
+    rng = np.random.default_rng(1000 + seed)
+    ih, iw, pad, stride, dil = _geometry(rng)
+    n, ic = int(rng.integers(1, 5)), int(rng.choice([64, 128]))
+    oc = 16 * int(rng.integers(3, 11))
+    in_zp = int(rng.integers(-128, 128))
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 3, 3, ic)).astype(np.int8)
+    bias = rng.integers(-(1 << 18), 1 << 18, oc).astype(np.int32)
+    acc = oracle.conv2d("i8", x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
+    assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
+    assert np.array_equal(got, acc), (ih, iw, ic, oc, pad, stride, dil)
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    shift = rng.integers(37, 45, oc).astype(np.int8) if seed % 3 else np.full(oc, 41, np.int8)
+    out_zp = int(rng.integers(-20, 20))
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0,
+                             rescale=dict(mult=mult, shift=shift, out_zp=out_zp), clamp=(-120, 120))
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp)
+    assert st == wst == capi.VALID and ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert np.array_equal(got, oracle.clamp(want, -120, 120)), (ih, iw, ic, oc, pad, stride, dil)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_depthwise_mfma_random_geometry(ctx, seed):
+    rng = np.random.default_rng(2000 + seed)
+    ih, iw, pad, stride, dil = _geometry(rng)
+    n, c = int(rng.integers(1, 5)), 16 * int(rng.integers(2, 21))
+    in_zp = int(rng.integers(-128, 128))
+    x = rng.integers(-128, 128, (n, ih, iw, c)).astype(np.int8)
+    w = rng.integers(-128, 128, (3, 3, c, 1)).astype(np.int8)
+    bias = rng.integers(-(1 << 16), 1 << 16, c).astype(np.int32)
+    acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True)
+    assert st == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8"
+    assert np.array_equal(got, acc), (ih, iw, c, pad, stride, dil)
+    mult = rng.integers(1 << 30, 1 << 31, c).astype(np.int32)
+    shift = rng.integers(33, 40, c).astype(np.int8) if seed % 3 else np.full(c, 35, np.int8)
+    out_zp = int(rng.integers(-20, 20))
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True,
+                             rescale=dict(mult=mult, shift=shift, out_zp=out_zp))
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp)
+    assert st == wst == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8_rescale"
+    assert np.array_equal(got, want), (ih, iw, c, pad, stride, dil)
