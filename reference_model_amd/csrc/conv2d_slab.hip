@@ -1,4 +1,4 @@
-// CONV2D for layers whose channel vector is 64 or 128 bytes (int8 with IC = 64 or 128), 3x3 taps: the small,
+// CONV2D for layers whose channel vector is 64 or 128 bytes (int8 with IC = 64 or 128), 3x3 or 1x1 taps: the small,
 // latency-bound layers of a ResNet stem, where a launch does well under a microsecond of matrix work and everything else is
 // overhead.  The kernel is the shortest path from memory to the matrix cores this chip offers:
 //
@@ -388,8 +388,10 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                void* out, const void* pad_page, uint32_t* flag_word)
 {
-    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 128) || g.KH != 3 || g.KW != 3 || w_zp != 0 || !pad_page || !flag_word)
+    const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
+    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
+    const int taps = g.KH * g.KW;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
         return nullptr;
     if (g.OC < 48 || g.OC > 65536 || (g.OC & 15) || g.N < 1 || g.OH < 1 || g.OW < 1)
@@ -410,7 +412,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
         int th, tw;
     };
     static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0 };
-    const int32_t key[8] = { g.N, g.OH, g.OW, n_ocb * 256 + ch, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
+    const int32_t key[8] = { g.N, g.OH, g.OW, (n_ocb * 256 + ch) * 4 + g.KH, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
     int best_th = 0, best_tw = 0;
     if (memcmp(key, last.key, sizeof(key)) == 0)
         best_th = last.th, best_tw = last.tw;
@@ -427,7 +429,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                 const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
                 const int64_t rounds = (tiles + 255) / 256;
                 // a round costs its loads plus the four 32-pixel MFMA tiles whether they are full or not
-                const int64_t cost = rounds * ((9 * 64 + ph * pw) * (ch / 4) + 600);
+                const int64_t cost = rounds * ((taps * 64 + ph * pw) * (ch / 4) + 600);
                 if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
                     best_th = th, best_tw = tw, best_cost = cost;
             }
@@ -468,11 +470,15 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pitch = make_fastdiv((uint32_t)a.pitch);
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
-    const int w_loads = 9 * ch + 1, p_loads = (a.PH * a.pitch + 63) / 64;
-    const int ones_bytes = 2 * (g.dil_y * a.pitch * 16 + g.dil_x * rp_chunks * 16) + g.IC;
+    const int w_loads = taps * ch + 1, p_loads = (a.PH * a.pitch + 63) / 64;
+    const int ones_bytes = (g.KH - 1) * g.dil_y * a.pitch * 16 + (g.KW - 1) * g.dil_x * rp_chunks * 16 + g.IC;
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
-    if (!(ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, rp.enabled != 0)
-                  : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, rp.enabled != 0)))
+    const bool fused = rp.enabled != 0;
+    const bool ok    = k33 ? (ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused)
+                                      : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused))
+                           : (ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused)
+                                      : launch_slab_taps<1, 1, 8>(st, a, (int)grid, lds_bytes, fused));
+    if (!ok)
         return nullptr;
     return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";
 }

@@ -105,6 +105,34 @@ def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
     assert len(np.unique(got)) > 50
 
 
+@pytest.mark.parametrize("shape", [  # n, ih, iw, ic, oc, pad, stride
+    (8, 56, 56, 64, 256, (0, 0, 0, 0), (1, 1)),         # a bottleneck block's expanding 1x1 layer
+    (4, 28, 28, 128, 512, (0, 0, 0, 0), (1, 1)),
+    (4, 29, 29, 128, 64, (0, 0, 0, 0), (2, 2)),         # a down-sampling shortcut
+    (3, 17, 13, 64, 80, (1, 0, 0, 2), (1, 1)),          # padding on a pointwise layer: the border is bias only
+])
+@pytest.mark.parametrize("in_zp", [0, -7])
+def test_slab_pointwise_layers_bit_exact(ctx, shape, in_zp):
+    """1x1 taps with 64 or 128 input channels: too little K for the GEMM kernel, one or two MFMA steps here"""
+    n, ih, iw, ic, oc, pad, stride = shape
+    rng = np.random.default_rng(ih * oc + ic)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 1, 1, ic)).astype(np.int8)
+    bias = rng.integers(-(1 << 18), 1 << 18, oc).astype(np.int32)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, in_zp=in_zp, w_zp=0)
+    assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
+    acc = cases.conv2d_exact_blas(x, w, bias, pad, stride, (1, 1), in_zp, 0)
+    assert np.array_equal(got, acc)
+    assert np.array_equal(got[:1, :, :, :3], oracle.conv2d("i8", x[:1], w[:3], bias[:3], pad, stride, in_zp=in_zp, w_zp=0))
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    shift = rng.integers(35, 41, oc).astype(np.int8)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, in_zp=in_zp, w_zp=0,
+                             rescale=dict(mult=mult, shift=shift, out_zp=3), clamp=(-128, 100))
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=3)
+    assert st == wst == capi.VALID and ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert np.array_equal(got, oracle.clamp(want, -128, 100))
+
+
 def test_slab_config3_full_size(ctx):
     """the named configuration with its own operands: shift 38 for every channel, DOUBLE rounding, CLAMP [0, 127]"""
     c = cases.c3()
