@@ -1,4 +1,4 @@
-// CONV2D for layers whose channel vector is 64 or 128 bytes (int8 with IC = 64 or 128), 3x3 or 1x1 taps: the small,
+// CONV2D for layers whose channel vector is 64, 96 or 128 bytes (int8 with IC = 64, 96 or 128), 3x3 or 1x1 taps: the small,
 // latency-bound layers of a ResNet stem, where a launch does well under a microsecond of matrix work and everything else is
 // overhead.  The kernel is the shortest path from memory to the matrix cores this chip offers:
 //
@@ -63,7 +63,7 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
                  : "memory");
 }
 
-// CH: 16-byte chunks of a channel vector (4: 64 input channels, 8: 128)
+// CH: 16-byte chunks of a channel vector (4, 6, 8: 64, 96, 128 input channels)
 template <int KH, int KW, int CH, bool ZA, bool FUSED>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
@@ -389,7 +389,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                void* out, const void* pad_page, uint32_t* flag_word)
 {
     const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
-    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
+    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 96 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
     const int taps = g.KH * g.KW;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
@@ -429,7 +429,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                 const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
                 const int64_t rounds = (tiles + 255) / 256;
                 // a round costs its loads plus the four 32-pixel MFMA tiles whether they are full or not
-                const int64_t cost = rounds * ((taps * 64 + ph * pw) * (ch / 4) + 600);
+                const int64_t cost = rounds * ((taps * 64 + ph * pw) * ch / 4 + 600);
                 if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
                     best_th = th, best_tw = tw, best_cost = cost;
             }
@@ -474,10 +474,15 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     const int ones_bytes = (g.KH - 1) * g.dil_y * a.pitch * 16 + (g.KW - 1) * g.dil_x * rp_chunks * 16 + g.IC;
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
     const bool fused = rp.enabled != 0;
-    const bool ok    = k33 ? (ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused)
-                                      : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused))
-                           : (ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused)
-                                      : launch_slab_taps<1, 1, 8>(st, a, (int)grid, lds_bytes, fused));
+    bool ok;
+    if (k33)
+        ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused)
+                     : (ch == 6 ? launch_slab_taps<3, 3, 6>(st, a, (int)grid, lds_bytes, fused)
+                                : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused));
+    else
+        ok = ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused)
+                     : (ch == 6 ? launch_slab_taps<1, 1, 6>(st, a, (int)grid, lds_bytes, fused)
+                                : launch_slab_taps<1, 1, 8>(st, a, (int)grid, lds_bytes, fused));
     if (!ok)
         return nullptr;
     return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";

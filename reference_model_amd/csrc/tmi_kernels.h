@@ -105,7 +105,7 @@ const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int3
                         int32_t pad_top, int32_t pad_left, int32_t in_zp, int32_t out_zp, int32_t nan_mode,
                         const void* in, void* out, uint32_t* flag_word);
 
-// conv2d_slab.hip: int8 CONV2D with IC = 64 or 128, 3x3 or 1x1 taps and weight_zp = 0 (int32 result, or the fast form of a fused
+// conv2d_slab.hip: int8 CONV2D with IC = 64, 96 or 128, 3x3 or 1x1 taps and weight_zp = 0 (int32 result, or the fast form of a fused
 // RESCALE to int8 / int16): weight slab and input patch loaded straight into LDS; nullptr for anything else.
 // pad_page: 64 bytes of input_zp in device memory.
 const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,

@@ -37,7 +37,7 @@ def _geometry(rng):
 def test_conv2d_slab_random_geometry(ctx, seed):
     rng = np.random.default_rng(1000 + seed)
     ih, iw, pad, stride, dil = _geometry(rng)
-    n, ic = int(rng.integers(1, 5)), int(rng.choice([64, 128]))
+    n, ic = int(rng.integers(1, 5)), int(rng.choice([64, 96, 128]))
     oc = 16 * int(rng.integers(3, 11))
     in_zp = int(rng.integers(-128, 128))
     x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)

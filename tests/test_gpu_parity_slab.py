@@ -34,6 +34,7 @@ SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation[, ic: 64 unless given]
     (4, 28, 28, 128, (1, 1, 1, 1), (1, 1), (1, 1), 128),    # 128 input channels: four MFMA steps per tap
     (2, 19, 17, 80, (1, 0, 2, 1), (1, 1), (1, 1), 128),     # ragged tiles and channel block
     (2, 29, 29, 64, (1, 1, 1, 1), (2, 2), (1, 1), 128),     # stride 2
+    (3, 21, 22, 64, (1, 1, 1, 1), (1, 1), (1, 1), 96),      # 96 input channels: three MFMA steps per tap
 ]
 
 
@@ -109,6 +110,7 @@ def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
     (8, 56, 56, 64, 256, (0, 0, 0, 0), (1, 1)),         # a bottleneck block's expanding 1x1 layer
     (4, 28, 28, 128, 512, (0, 0, 0, 0), (1, 1)),
     (4, 29, 29, 128, 64, (0, 0, 0, 0), (2, 2)),         # a down-sampling shortcut
+    (4, 28, 28, 96, 64, (0, 0, 0, 0), (1, 1)),          # a MobileNet projection layer
     (3, 17, 13, 64, 80, (1, 0, 0, 2), (1, 1)),          # padding on a pointwise layer: the border is bias only
 ])
 @pytest.mark.parametrize("in_zp", [0, -7])
