@@ -2,13 +2,12 @@
 """Benchmark of the hot path on one MI355X.
 
 A step is one pass of one operator (one C-ABI call) over one batch of seeded synthetic operands that are
-resident in HBM before the timed region starts.  The default workload is the one BASELINE.json's metric is
-quoted on:
+resident in HBM before the timed region starts.  The default workload is the headline configuration:
 
   c3   INT8 CONV2D 3x3 [8,56,56,64]x[64,3,3,64] s1 p1 + per-channel RESCALE (shift 38, double_round) +
        CLAMP [0,127], fused (default; unit TOPS, MFMA roofline)
 
-and --config selects the other BASELINE configurations, each reported against the roofline that bounds it:
+and --config selects the other benchmark configurations, each reported against the roofline that bounds it:
 
   c2   INT8 MATMUL [8,1024,1024]x[8,1024,1024] -> int32            (TOPS; HBM roofline, int32 result)
   c4   INT8 DEPTHWISE_CONV2D [8,112,112,96] s2 + RESCALE, fused     (GB/s; HBM roofline)

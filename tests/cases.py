@@ -1,4 +1,4 @@
-"""Seeded synthetic operands for the BASELINE configurations and for small parity cases.
+"""Seeded synthetic operands for the benchmark configurations and for small parity cases.
 
 Values are produced on the host by numpy's PCG64 seeded per configuration, so the oracle and the GPU see
 identical bytes.

@@ -370,3 +370,44 @@ def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
     assert np.array_equal(np.load(d4 / "o_out.npy"), oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64)))
     assert np.array_equal(np.load(d4 / "bounds_o_out.npy"),
                           oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64), abs_mode=True))
+
+
+# ---- system-under-test module for the reference's conformance runner ----------------------------------------
+class _RunnerArgs:
+    verbose = False
+    precise_mode = False
+
+
+def _copy_example(golden_dir, tmp_path, name):
+    import shutil
+    dst = tmp_path / name
+    shutil.copytree(os.path.join(golden_dir, name), dst)
+    return dst
+
+
+def test_sut_module_command_line_and_status_without_a_gpu(golden_dir, tmp_path):
+    from reference_model_amd import sut_run
+    d = _copy_example(golden_dir, tmp_path, "qi8_conv2d_1x1")
+    assert sut_run.parse_runner_args(["precise_mode", "runner=/x/y", "timeout=5"]) == {
+        "precise_mode": True, "runner": "/x/y", "timeout": "5"}
+    sut = sut_run.TosaSUTRunner(_RunnerArgs(), ["no_fusion"], d)
+    assert sut.command() == [RUN, f"--test_desc={d / 'desc.json'}", "--no_fusion"]
+    sut = sut_run.TosaSUTRunner(_RunnerArgs(), ["precise_mode"], d)
+    assert sut.command()[-1] == "--precise_mode=1"
+    missing = sut_run.TosaSUTRunner(_RunnerArgs(), ["runner=/nonexistent/tosa_mi355_run"], d)
+    result, message = missing.runTestGraph()
+    assert result == sut_run.TosaTestRunner.TosaGraphResult.OTHER_ERROR and "nonexistent" in message
+    import torch
+    if not torch.cuda.is_available():
+        result, message = sut_run.TosaSUTRunner(_RunnerArgs(), [], d).runTestGraph()
+        assert result == sut_run.TosaTestRunner.TosaGraphResult.TOSA_ERROR and "no CPU fall-back" in message
+        assert not (d / "ref_model_output_0.npy").exists()
+
+
+@pytest.mark.gpu
+def test_sut_module_runs_the_reference_example_directory(golden_dir, tmp_path):
+    from reference_model_amd import sut_run
+    d = _copy_example(golden_dir, tmp_path, "qi8_conv2d_1x1")
+    result, message = sut_run.TosaSUTRunner(_RunnerArgs(), [], d).runTestGraph()
+    assert result == sut_run.TosaTestRunner.TosaGraphResult.TOSA_VALID and message is None
+    assert np.array_equal(np.load(d / "ref_model_output_0.npy"), np.load(d / "tflite_result.npy"))
