@@ -13,9 +13,10 @@
 //     together then read 16 different bank groups, for the weight fragments and (odd strides) the pixel fragments.
 //   - A pixel outside the image reads a 64-byte page of input_zp bytes, so it contributes
 //     (zp - zp) * w = 0 like the reference's skipped tap (tensor_ops.cpp:845-852), and the zero-point identity
-//     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  sum(w) per channel costs nothing: a wave's
-//     32 MFMA columns are 31 pixels and one "pixel of ones" (bytes 0x01 in LDS wherever a tap can read), whose
-//     accumulators are the sums, already in the register order of the lanes that need them.
+//     sum((a - za) w) = sum(a w) - za * sum(w) holds with the full K.  za * sum(w) per channel costs nothing: a
+//     wave's 32 MFMA columns are 31 pixels and one "zero-point pixel" (input_zp bytes in LDS wherever a tap can
+//     read), whose accumulators are those terms, already in the register order of the lanes that need them.
+//     The accumulators of the 31 pixels start at the bias, those of the zero-point column at zero.
 //   - While the loads are in flight the eighth wave, which issues none, turns bias / multiplier / shift into
 //     the per-channel constants of the RESCALE in LDS.
 //   - One barrier, then 18 MFMA steps per wave (one accumulator tile of 32 channels x 32 columns), then the fused
@@ -77,7 +78,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     constexpr int RP     = CH + 1;          // chunks per patch pixel in LDS (odd)
     constexpr int LWAVES = 7;               // waves that issue loads; the eighth builds the tables
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    // LDS: [weight rows][patch][pixel of ones][64 x ChannelScale][64 x (multiplier, bias)][the block's common shift]
+    // LDS: [weight rows][patch][zero-point pixel][64 x ChannelScale][64 x HighWordScale][64 multipliers][64 biases, 16 zeros][the block's common shift]
     const int tid    = threadIdx.x;
     const int lane   = tid & 63;
     const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -87,15 +88,17 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     const int p_loads = (p_slots + 63) >> 6;
     uint8_t* wl       = lds;
     uint8_t* pl       = lds + WLOADS * 1024;
-    // fragment offsets of the taps inside the patch, and the "pixel of ones": bytes 0x01 wherever a tap can read
+    // fragment offsets of the taps inside the patch, and the zero-point pixel: input_zp bytes wherever a tap can read
     const int row_step   = a.dy * a.pitch * 16;
     const int col_step   = a.dx * RP * 16;
     const int ones_bytes = ZA ? ((KH - 1) * row_step + (KW - 1) * col_step + KB) : 0;
     uint8_t* ones        = pl + p_loads * 1024;
     uint8_t* tabs        = ones + ones_bytes;
     ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tabs);
-    int2* tab_mb         = reinterpret_cast<int2*>(tabs + 64 * sizeof(ChannelScale));    // multiplier, bias
-    int32_t* uni_shift   = reinterpret_cast<int32_t*>(tab_mb + 64);                      // 4 words, one used
+    HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(tabs + 64 * sizeof(ChannelScale));
+    int32_t* tab_m       = reinterpret_cast<int32_t*>(tab_hw + 64);                         // multipliers
+    int32_t* tab_b       = tab_m + 64;                                                      // biases, then 16 zeros
+    int32_t* uni_shift   = tab_b + 80;                                                      // 4 words, one used
 
     uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
@@ -188,34 +191,33 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
             m                     = cs.m;
             // The epilogue has three forms:
-            //   every shift >= 32 and small enough for output_zp * 2^shift to ride in the 64-bit rounding term: the
-            //   result is the high word of the sum shifted by shift - 32, no value-range test (-2);
-            //   the same with one shift for the whole block: the rounding terms are scalars and a channel needs 8
-            //   bytes of constants (the shift itself);
+            //   every shift large enough for the high-word form (tmi_device.h) and small enough for output_zp * 2^shift
+            //   to ride in the 64-bit rounding term: 16 bytes of constants per channel, no value-range test (-2);
+            //   the same with one shift for the whole block: the rounding term and the shift are scalars and a channel
+            //   needs its multiplier only (the shift itself);
             //   anything else: fast_rescale() with its range test and a 64-bit shift (-1).
-            const int folds = __all(cs.s >= 32 && cs.s <= zp_fold_max_shift(a.rp.out_zp));
+            const int s_min = a.rp.double_round ? 33 : 32;
+            const int folds = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp));
             const int uni   = folds && __all(cs.s == s_first);
-            ChannelScale e  = cs;
-            if (folds)
-            {
-                const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
-                e.rnd_pos += zp_term, e.rnd_neg += zp_term;
-            }
-            tab_cs[lane] = e;
+            tab_cs[lane]    = cs;
+            tab_hw[lane]    = make_high_word_scale(cs, a.rp.out_zp);
             if (lane == 0)
                 *uni_shift = uni ? s_first : (folds ? -2 : -1);
         }
-        tab_mb[lane] = int2{ m, ok ? b : 0 };
+        tab_m[lane] = m;
+        tab_b[lane] = ok ? b : 0;
+        if (lane < 16)
+            tab_b[64 + lane] = 0;
+        const int za4 = (a.za & 0xff) * 0x01010101;
         for (int i = lane * 16; i < ones_bytes; i += 1024)
-            *reinterpret_cast<v4i*>(ones + i) = v4i{ 0x01010101, 0x01010101, 0x01010101, 0x01010101 };
+            *reinterpret_cast<v4i*>(ones + i) = v4i{ za4, za4, za4, za4 };
     }
     __syncthreads();
 
     // ---- MFMA: wave = (channel tile, pixel tile) ---------------------------------------------------------------
     const int oct = wave >> 2, pxt = wave & 3;
-    // A wave's 32 MFMA columns are 31 pixels and, in column 31, the pixel of ones: its accumulators are sum(w) of
-    // the wave's 32 channels, which the zero-point term needs, for the price of nothing (the column would be
-    // computed anyway).
+    // A wave's 32 MFMA columns are 31 pixels and, in column 31, the zero-point pixel: its accumulators are
+    // input_zp * sum(w) of the wave's 32 channels, for the price of nothing (the column would be computed anyway).
     constexpr int PXW = 31;
     const int P       = a.TH * a.TW;
     int p             = pxt * PXW + li;
@@ -223,10 +225,18 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     p                 = p_in_tile ? p : 0;
     const int ty  = fdiv(p, a.div_tw);
     const int tx  = p - ty * a.TW;
+    // The accumulators start at the bias of the lane's 16 channels (the zero-point column at zero).
+    const int ocl = oct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
     v16i acc;
+    {
+        const int32_t* b16 = tab_b + ((ZA && li == PXW) ? 64 : ocl);
 #pragma unroll
-    for (int r = 0; r < 16; r++)
-        acc[r] = 0;
+        for (int q = 0; q < 4; q++)
+        {
+            const v4i b4 = *reinterpret_cast<const v4i*>(b16 + 4 * q);
+            acc[4 * q] = b4[0], acc[4 * q + 1] = b4[1], acc[4 * q + 2] = b4[2], acc[4 * q + 3] = b4[3];
+        }
+    }
     const bool wave_active = pxt * PXW < P;    // wave-uniform
     if (wave_active)
     {
@@ -253,22 +263,14 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 
     // ---- epilogue ----------------------------------------------------------------------------------------------
     // (lane, register 4q + j) = D[row 8q + 4 lh + j][pixel li] = channel 32 oct + 16 lh + 4q + j
-    const int ocl = oct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
-    int32_t cm[16], cb[16];                // multiplier and bias of the lane's channels
-#pragma unroll
-    for (int q = 0; q < 8; q++)
-    {
-        const v4i mb = *reinterpret_cast<const v4i*>(tab_mb + ocl + 2 * q);
-        cm[2 * q] = mb[0], cb[2 * q] = mb[1], cm[2 * q + 1] = mb[2], cb[2 * q + 1] = mb[3];
-    }
     if constexpr (ZA)
     {
-        // Lane 31 + 32 lh holds in register e the column of ones for channel 16 lh + e: sum(w) of exactly the
-        // channel this lane has in register e.  |sum(w)| <= taps * 64 * 128 < 2^23 and |za| <= 128: a 24-bit multiply.
+        // Lane 31 + 32 lh holds in register e the zero-point column for channel 16 lh + e: input_zp * sum(w) of
+        // exactly the channel this lane has in register e.
         const int src = (PXW + 32 * lh) * 4;
 #pragma unroll
         for (int e = 0; e < 16; e++)
-            cb[e] -= __mul24(a.za, __builtin_amdgcn_ds_bpermute(src, acc[e]));
+            acc[e] -= __builtin_amdgcn_ds_bpermute(src, acc[e]);
     }
     const int oy = oy0 + ty, ox = ox0 + tx;
     const bool pix_ok  = p_in_tile && wave_active && oy < a.OH && ox < a.OW;
@@ -281,8 +283,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase;
 #pragma unroll
             for (int q = 0; q < 4; q++)
-                *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acc[4 * q] + cb[4 * q], acc[4 * q + 1] + cb[4 * q + 1],
-                                                          acc[4 * q + 2] + cb[4 * q + 2], acc[4 * q + 3] + cb[4 * q + 3] };
+                *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3] };
         }
     }
     else
@@ -291,30 +292,51 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         const int s_uni = __builtin_amdgcn_readfirstlane(*uni_shift);
         if (s_uni >= 0)
         {
-            // One shift s >= 32 for every channel: (v * m + round) >> s is the high word of the sum shifted by
-            // s - 32; the rounding terms (double rounding and output_zp * 2^s folded in) are two scalars, and
-            // apply_scale_32's value-range test cannot fire (it only exists for shifts below 32).
-            const int64_t dr     = a.rp.double_round ? (int64_t(1) << 30) : 0;
-            const int64_t rnd_p  = (int64_t(1) << (s_uni - 1)) + dr + ((int64_t)a.rp.out_zp << s_uni);
-            const int64_t rnd_n  = rnd_p - 2 * dr;
-            const int sh         = s_uni - 32;
+            // one shift for every channel: the high-word form with its constants in scalar registers
+            const int64_t rnd = (int64_t(1) << (s_uni - 1)) + (a.rp.double_round ? (int64_t(1) << 30) : 0) +
+                                ((int64_t)a.rp.out_zp << s_uni);
+            const int32_t hi_p  = (int32_t)(rnd >> 32);
+            const uint32_t lo_p = (uint32_t)rnd;
+            const int sh        = s_uni - 32;
+            int32_t cm[16];    // multipliers of the lane's channels
 #pragma unroll
-            for (int e = 0; e < 16; e++)
+            for (int q = 0; q < 4; q++)
             {
-                const int32_t v  = acc[e] + cb[e];
-                const int64_t pr = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? rnd_p : rnd_n);
-                r[e]             = clamp_med3((int32_t)(pr >> 32) >> sh, a.rp.lo, a.rp.hi);
+                const v4i m4 = *reinterpret_cast<const v4i*>(tab_m + ocl + 4 * q);
+                cm[4 * q] = m4[0], cm[4 * q + 1] = m4[1], cm[4 * q + 2] = m4[2], cm[4 * q + 3] = m4[3];
+            }
+            if (a.rp.double_round)
+            {
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    r[e] = clamp_med3(high_word_rescale<true>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+            }
+            else
+            {
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    r[e] = clamp_med3(high_word_rescale<false>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
             }
         }
         else if (s_uni == -2)
         {
-#pragma unroll
-            for (int e = 0; e < 16; e++)
+            if (a.rp.double_round)
             {
-                const ChannelScale cs = tab_cs[ocl + e];
-                const int32_t v       = acc[e] + cb[e];
-                const int64_t pr      = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? cs.rnd_pos : cs.rnd_neg);
-                r[e]                  = clamp_med3((int32_t)(pr >> 32) >> (cs.s - 32), a.rp.lo, a.rp.hi);
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                {
+                    const HighWordScale c = tab_hw[ocl + e];
+                    r[e] = clamp_med3(high_word_rescale<true>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                {
+                    const HighWordScale c = tab_hw[ocl + e];
+                    r[e] = clamp_med3(high_word_rescale<false>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                }
             }
         }
         else
@@ -324,7 +346,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             for (int e = 0; e < 16; e++)
             {
                 const ChannelScale cs = tab_cs[ocl + e];
-                r[e]                  = fast_rescale(acc[e] + cb[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
+                r[e]                  = fast_rescale(acc[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
             }
             if (pix_ok && chan_ok)
                 flags |= eflags;    // pixels and channels outside the tensor raise nothing
@@ -472,7 +494,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
     const int w_loads = taps * ch + 1, p_loads = (a.PH * a.pitch + 63) / 64;
     const int ones_bytes = (g.KH - 1) * g.dil_y * a.pitch * 16 + (g.KW - 1) * g.dil_x * rp_chunks * 16 + g.IC;
-    const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)sizeof(ChannelScale) + 64 * 8 + 16;
+    const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 80 * 4 + 16;
     const bool fused = rp.enabled != 0;
     bool ok;
     if (k33)

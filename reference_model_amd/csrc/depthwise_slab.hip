@@ -60,7 +60,7 @@ __device__ __forceinline__ void dwslab_load(const void* src, uint32_t lds_addr)
 }
 
 template <bool ZA, bool FUSED>
-__global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
+__global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
 {
     asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len), "s"(a.n_units),
                  "s"(a.div_cblk.d));
@@ -75,13 +75,15 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
     const int C       = a.C;
     const int p_slots = a.PH * a.pitch;
     const int p_loads = (p_slots + 63) >> 6;
-    // LDS: [patch][weights: 9 x C bytes][C x ChannelScale][C x (multiplier, bias - za * sum(w))][common shift per table wave]
+    // LDS: [patch][weights: 9 x C bytes][C x ChannelScale][C x HighWordScale][C multipliers][C x (bias - za * sum(w))][common shift per table wave]
     uint8_t* pl          = lds;
     int32_t* wtab        = reinterpret_cast<int32_t*>(lds + p_loads * 1024);    // the weight byte in all four bytes of a word
     const int wtab_bytes = TAPS * C * 4;
     ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(lds + p_loads * 1024 + wtab_bytes);
-    int2* tab_mb         = reinterpret_cast<int2*>(tab_cs + C);
-    int32_t* uni_shift   = reinterpret_cast<int32_t*>(tab_mb + C);    // 8 words
+    HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(tab_cs + C);
+    int32_t* tab_m       = reinterpret_cast<int32_t*>(tab_hw + C);
+    int32_t* tab_b       = tab_m + C;
+    int32_t* uni_shift   = tab_b + C;    // 8 words
 
     uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
@@ -164,26 +166,25 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
                 make_channel_scale(tab_lane ? t_mult : 0, tab_lane ? t_shift : s_first, a.rp.double_round != 0, flags);
             m             = cs.m;
             // The epilogue has three forms, chosen per group of 64 channels (one table wave):
-            //   every shift >= 32 and small enough for output_zp * 2^shift to ride in the 64-bit rounding term: the
-            //   result is the high word of the sum shifted by shift - 32, no value-range test (-2);
-            //   the same with one shift for all 64 channels: rounding terms and shift are scalars (the shift itself);
+            //   every shift large enough for the high-word form (tmi_device.h) and small enough for output_zp * 2^shift
+            //   to ride in the 64-bit rounding term: 16 bytes of constants per channel, no value-range test (-2);
+            //   the same with one shift for all 64 channels: rounding term and shift are scalars (the shift itself);
             //   anything else: fast_rescale() with its range test and a 64-bit shift (-1).
-            const int folds = __all(cs.s >= 32 && cs.s <= zp_fold_max_shift(a.rp.out_zp));
+            const int s_min = a.rp.double_round ? 33 : 32;
+            const int folds = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp));
             const int uni   = folds && __all(cs.s == s_first);
-            ChannelScale e  = cs;
-            if (folds)
-            {
-                const int64_t zp_term = (int64_t)a.rp.out_zp << cs.s;
-                e.rnd_pos += zp_term, e.rnd_neg += zp_term;
-            }
             if (tab_lane)
-                tab_cs[tid] = e;
+            {
+                tab_cs[tid] = cs;
+                tab_hw[tid] = make_high_word_scale(cs, a.rp.out_zp);
+            }
             if (lane == 0)
                 uni_shift[wave] = uni ? s_first : (folds ? -2 : -1);
         }
         if (tab_lane)
         {
-            tab_mb[tid] = int2{ m, t_bias - (ZA ? a.za * wsum : 0) };
+            tab_m[tid] = m;
+            tab_b[tid] = t_bias - (ZA ? a.za * wsum : 0);
 #pragma unroll
             for (int t = 0; t < TAPS; t++)
                 wtab[t * C + tid] = ((int)t_w[t] & 0xff) * 0x01010101;
@@ -227,10 +228,16 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
                 fa[t]        = v4i{ wv & wmask[0], wv & wmask[1], wv & wmask[2], wv & wmask[3] };
             }
         }
+        // (lane, register e) = channel c0 + 16 lh + e of pixel li; the accumulators start at the channel's bias term
+        const int cl  = c0 + 16 * lh;
+        const int clc = cl < C ? cl : 0;    // C is a multiple of 16
         v16i acc;
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[r] = 0;
+        for (int q = 0; q < 4; q++)
+        {
+            const v4i b4 = *reinterpret_cast<const v4i*>(tab_b + clc + 4 * q);
+            acc[4 * q] = b4[0], acc[4 * q + 1] = b4[1], acc[4 * q + 2] = b4[2], acc[4 * q + 3] = b4[3];
+        }
         const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * a.ppitch) * 16 + c0 + lh * 16;
 #pragma unroll
         for (int ky = 0; ky < 3; ky++)
@@ -241,18 +248,9 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
                 acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ky * 3 + kx], fb, acc, 0, 0, 0);
             }
 
-        // ---- epilogue: (lane, register e) = channel c0 + 16 lh + e of pixel li --------------------------------------
-        const int cl = c0 + 16 * lh;
+        // ---- epilogue ------------------------------------------------------------------------------------------------
         const int oy = oy0 + ty, ox = ox0 + tx;
-        const bool ok = p_in_tile && oy < a.OH && ox < a.OW && cl < C;    // C is a multiple of 16
-        const int clc = cl < C ? cl : 0;
-        int32_t cm[16], cbias[16];
-#pragma unroll
-        for (int q = 0; q < 8; q++)
-        {
-            const v4i mb = *reinterpret_cast<const v4i*>(tab_mb + clc + 2 * q);
-            cm[2 * q] = mb[0], cbias[2 * q] = mb[1], cm[2 * q + 1] = mb[2], cbias[2 * q + 1] = mb[3];
-        }
+        const bool ok = p_in_tile && oy < a.OH && ox < a.OW && cl < C;
         const size_t obase = (((size_t)n * a.OH + oy) * a.OW + ox) * C + cl;
         if constexpr (!FUSED)
         {
@@ -261,9 +259,7 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
                 int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase;
 #pragma unroll
                 for (int q = 0; q < 4; q++)
-                    *reinterpret_cast<v4i*>(o + 4 * q) =
-                        v4i{ acc[4 * q] + cbias[4 * q], acc[4 * q + 1] + cbias[4 * q + 1], acc[4 * q + 2] + cbias[4 * q + 2],
-                             acc[4 * q + 3] + cbias[4 * q + 3] };
+                    *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3] };
             }
         }
         else
@@ -272,29 +268,51 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
             const int s_uni = __builtin_amdgcn_readfirstlane(uni_shift[c0 >> 6]);    // the form of this block's group
             if (s_uni >= 0)
             {
-                // one shift s >= 32 for every channel: the rounding terms (double rounding and output_zp * 2^s folded
-                // in) are two scalars and apply_scale_32's value-range test cannot fire
-                const int64_t dr    = a.rp.double_round ? (int64_t(1) << 30) : 0;
-                const int64_t rnd_p = (int64_t(1) << (s_uni - 1)) + dr + ((int64_t)a.rp.out_zp << s_uni);
-                const int64_t rnd_n = rnd_p - 2 * dr;
+                // one shift for all 64 channels: the high-word form with its constants in scalar registers
+                const int64_t rnd = (int64_t(1) << (s_uni - 1)) + (a.rp.double_round ? (int64_t(1) << 30) : 0) +
+                                    ((int64_t)a.rp.out_zp << s_uni);
+                const int32_t hi_p  = (int32_t)(rnd >> 32);
+                const uint32_t lo_p = (uint32_t)rnd;
                 const int sh        = s_uni - 32;
+                int32_t cm[16];
 #pragma unroll
-                for (int e = 0; e < 16; e++)
+                for (int q = 0; q < 4; q++)
                 {
-                    const int32_t v  = acc[e] + cbias[e];
-                    const int64_t pr = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? rnd_p : rnd_n);
-                    r[e]             = clamp_med3((int32_t)(pr >> 32) >> sh, a.rp.lo, a.rp.hi);
+                    const v4i m4 = *reinterpret_cast<const v4i*>(tab_m + clc + 4 * q);
+                    cm[4 * q] = m4[0], cm[4 * q + 1] = m4[1], cm[4 * q + 2] = m4[2], cm[4 * q + 3] = m4[3];
+                }
+                if (a.rp.double_round)
+                {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        r[e] = clamp_med3(high_word_rescale<true>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        r[e] = clamp_med3(high_word_rescale<false>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
                 }
             }
             else if (s_uni == -2)
             {
-#pragma unroll
-                for (int e = 0; e < 16; e++)
+                if (a.rp.double_round)
                 {
-                    const ChannelScale cs = tab_cs[clc + e];
-                    const int32_t v       = acc[e] + cbias[e];
-                    const int64_t pr      = (int64_t)v * (int64_t)cm[e] + (v >= 0 ? cs.rnd_pos : cs.rnd_neg);
-                    r[e]                  = clamp_med3((int32_t)(pr >> 32) >> (cs.s - 32), a.rp.lo, a.rp.hi);
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                    {
+                        const HighWordScale c = tab_hw[clc + e];
+                        r[e] = clamp_med3(high_word_rescale<true>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                    {
+                        const HighWordScale c = tab_hw[clc + e];
+                        r[e] = clamp_med3(high_word_rescale<false>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                    }
                 }
             }
             else
@@ -304,7 +322,7 @@ __global__ __launch_bounds__(512) void depthwise_slab_kernel(DwSlabArgs a)
                 for (int e = 0; e < 16; e++)
                 {
                     const ChannelScale cs = tab_cs[clc + e];
-                    r[e]                  = fast_rescale(acc[e] + cbias[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
+                    r[e]                  = fast_rescale(acc[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
                 }
                 if (ok)
                     flags |= eflags;    // pixels and channels outside the tensor raise nothing
@@ -399,7 +417,9 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
                 const int units        = ((th * tw + 31) / 32) * n_cblk;
                 const int64_t tiles    = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw);
                 const int64_t rounds   = (tiles + 255) / 256;
-                for (int nw = 4; nw <= 8; nw += 2)
+                // A single round of workgroups (one per CU) is as fast as its slowest wave: up to 16 waves, so that a
+                // wave has one unit.  With more rounds two workgroups of at most 8 waves share a CU and overlap.
+                for (int nw = 4; nw <= (rounds == 1 ? 16 : 8); nw += 2)
                 {
                     if (nw * 64 < C)    // the first C lanes build the per-channel tables
                         continue;
@@ -452,7 +472,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_cblk = make_fastdiv((uint32_t)n_cblk);
     const int p_loads   = (a.PH * a.pitch + 63) / 64;
-    const int lds_bytes = p_loads * 1024 + 9 * C * 4 + C * (int)sizeof(ChannelScale) + C * 8 + 32;
+    const int lds_bytes = p_loads * 1024 + 9 * C * 4 + C * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + C * 8 + 32;
     bool ok;
     if (in_zp != 0)
         ok = rp.enabled ? launch_dwslab_kernel<true, true>(st, a, (int)grid, per_round, lds_bytes)

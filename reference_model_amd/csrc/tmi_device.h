@@ -173,6 +173,38 @@ __device__ __forceinline__ int zp_fold_max_shift(int32_t out_zp)
     return mag == 0 ? 62 : 60 - (32 - __clz((int)mag));
 }
 
+// High-word form of apply_scale_32 + output_zp for a channel whose shift s is at least 32 (33 with double rounding)
+// and at most zp_fold_max_shift(): (v * m + rnd(v)) >> s == ((v * m + rnd(v)) >> 32) >> (s - 32), and the value-range
+// test of apply_scale_32 cannot fire.  rnd(v) = R for v >= 0 and R - 2^31 for v < 0 when double rounding, with
+// R = 2^(s-1) + 2^30 + output_zp * 2^s: the low word of R is 2^30, so the low word of rnd(v) is R.lo | (sign << 31)
+// and its high word R.hi + (v >> 31).  Without double rounding rnd(v) = R = 2^(s-1) + output_zp * 2^s.
+struct HighWordScale
+{
+    int32_t m;      // multiplier
+    int32_t hi;     // R >> 32
+    int32_t sh;     // s - 32
+    uint32_t lo;    // low word of R
+};
+
+__device__ __forceinline__ HighWordScale make_high_word_scale(const ChannelScale& c, int32_t out_zp)
+{
+    const int64_t r = c.rnd_pos + ((int64_t)out_zp << c.s);
+    return HighWordScale{ c.m, (int32_t)(r >> 32), c.s - 32, (uint32_t)r };
+}
+
+template <bool DOUBLE_ROUND>
+__device__ __forceinline__ int32_t high_word_rescale(int32_t v, int32_t m, int32_t hi, uint32_t lo, int32_t sh)
+{
+    if (DOUBLE_ROUND)
+    {
+        const int32_t t = v >> 31;
+        lo |= (uint32_t)t << 31;
+        hi += t;
+    }
+    const int64_t pr = (int64_t)v * (int64_t)m + (int64_t)(((uint64_t)(uint32_t)hi << 32) | lo);
+    return (int32_t)(pr >> 32) >> sh;
+}
+
 // apply_scale_32 + output_zp + clip (+ CLAMP) for a signed int32 value with zero input_zp.  With a legal
 // value |v| < 2^(s-1) and m < 2^31 the scaled result is below 2^30 in magnitude, so neither of the
 // reference's int32 range checks (quant_util.h:78-82, type_conversion.cpp:352-360) can fire here.
