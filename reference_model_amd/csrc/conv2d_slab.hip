@@ -248,17 +248,29 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * RP) * 16 + lh * 16;
         if (ZA && li == PXW)
             prow = ones + lh * 16;
+        // K step s = (tap s / (CH/2), half s % (CH/2)).  The fragments of step s + DEPTH are requested before the
+        // MFMA of step s and the order is pinned: an LDS read takes several MFMA times to come back with eight waves
+        // asking, and left alone the scheduler requests a step's fragments only one MFMA ahead.
+        constexpr int STEPS = TAPS * (CH / 2);
+        constexpr int DEPTH = STEPS < 8 ? STEPS : 8;
+        v4i fa[STEPS], fb[STEPS];
+        auto request = [&](int s) {
+            const int tap = s / (CH / 2), h = s % (CH / 2);
+            fa[s] = *reinterpret_cast<const v4i*>(wrow + s * 32);
+            fb[s] = *reinterpret_cast<const v4i*>(prow + (tap / KW) * row_step + (tap % KW) * col_step + h * 32);
+        };
 #pragma unroll
-        for (int ky = 0; ky < KH; ky++)
+        for (int s = 0; s < DEPTH; s++)
+            request(s);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kx = 0; kx < KW; kx++)
-#pragma unroll
-                for (int h = 0; h < CH / 2; h++)
-                {
-                    const v4i fa = *reinterpret_cast<const v4i*>(wrow + ((ky * KW + kx) * (CH / 2) + h) * 32);
-                    const v4i fb = *reinterpret_cast<const v4i*>(prow + ky * row_step + kx * col_step + h * 32);
-                    acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
-                }
+        for (int s = 0; s < STEPS; s++)
+        {
+            if (s + DEPTH < STEPS)
+                request(s + DEPTH);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     // ---- epilogue ----------------------------------------------------------------------------------------------
