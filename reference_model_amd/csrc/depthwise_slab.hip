@@ -217,17 +217,13 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
         p             = p_in_tile ? p : 0;
         const int ty  = fdiv(p, a.div_tw);
         const int tx  = p - ty * a.TW;
-        // the diagonal operands of this channel block (channels past C: zero rows)
-        v4i fa[TAPS];
-        {
-            const int c = c0 + wr;
-#pragma unroll
-            for (int t = 0; t < TAPS; t++)
-            {
-                const int wv = c < C ? wtab[t * C + c] : 0;
-                fa[t]        = v4i{ wv & wmask[0], wv & wmask[1], wv & wmask[2], wv & wmask[3] };
-            }
-        }
+        // Everything the nine MFMAs need is requested up front, in a pinned order: left alone, the compiler requests a
+        // tap's pixel fragment right before its MFMA and a wave waits out the LDS latency nine times in a row.
+        // The diagonal operands of this channel block are built from the replicated weight bytes (channels past C:
+        // zero rows).
+        const int c          = c0 + wr;
+        const int32_t* wcol  = wtab + (c < C ? c : 0);
+        const uint8_t* prow  = pl + (ty * a.sy * a.pitch + tx * a.sx * a.ppitch) * 16 + c0 + lh * 16;
         // (lane, register e) = channel c0 + 16 lh + e of pixel li; the accumulators start at the channel's bias term
         const int cl  = c0 + 16 * lh;
         const int clc = cl < C ? cl : 0;    // C is a multiple of 16
@@ -238,15 +234,25 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
             const v4i b4 = *reinterpret_cast<const v4i*>(tab_b + clc + 4 * q);
             acc[4 * q] = b4[0], acc[4 * q + 1] = b4[1], acc[4 * q + 2] = b4[2], acc[4 * q + 3] = b4[3];
         }
-        const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * a.ppitch) * 16 + c0 + lh * 16;
+        int wv[TAPS];
+        v4i fb[TAPS];
 #pragma unroll
-        for (int ky = 0; ky < 3; ky++)
+        for (int t = 0; t < TAPS; t++)
+            wv[t] = wcol[t * C];
 #pragma unroll
-            for (int kx = 0; kx < 3; kx++)
-            {
-                const v4i fb = *reinterpret_cast<const v4i*>(prow + ky * row_step + kx * col_step);
-                acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ky * 3 + kx], fb, acc, 0, 0, 0);
-            }
+        for (int t = 0; t < TAPS; t++)
+            fb[t] = *reinterpret_cast<const v4i*>(prow + (t / 3) * row_step + (t % 3) * col_step);
+        __builtin_amdgcn_sched_barrier(0);
+        int wm[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            wm[k] = c < C ? wmask[k] : 0;
+#pragma unroll
+        for (int t = 0; t < TAPS; t++)
+        {
+            const v4i fa = v4i{ wv[t] & wm[0], wv[t] & wm[1], wv[t] & wm[2], wv[t] & wm[3] };
+            acc          = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb[t], acc, 0, 0, 0);
+        }
 
         // ---- epilogue ------------------------------------------------------------------------------------------------
         const int oy = oy0 + ty, ox = ox0 + tx;
