@@ -150,3 +150,37 @@ def test_automatic_choice_takes_the_matrix_core_kernel_for_its_layers():
         assert st == capi.VALID and c.last_kernel == "depthwise_dot4_i8"    # weight zero point: the vector kernel
     finally:
         c.close()
+
+
+# shifts at the borders between the epilogue's forms (chosen per 64 channels): 32 with double rounding takes the
+# general form, 33 the high-word form; single rounding takes the high-word form from 32 on; mixtures; shifts too large
+# for output_zp * 2^shift to ride in the rounding term; multipliers at their extremes
+_FORM_CASES = [
+    ("uniform 32", lambda rng, c: np.full(c, 32)), ("uniform 33", lambda rng, c: np.full(c, 33)),
+    ("32..34", lambda rng, c: rng.integers(32, 35, c)), ("33..36", lambda rng, c: rng.integers(33, 37, c)),
+    ("30..34", lambda rng, c: rng.integers(30, 35, c)), ("52..62", lambda rng, c: rng.integers(52, 63, c)),
+    ("64 x 33, then 33..36", lambda rng, c: np.concatenate([np.full(64, 33), rng.integers(33, 37, c - 64)])),
+]
+
+
+@pytest.mark.parametrize("name,shifts", _FORM_CASES, ids=[c[0] for c in _FORM_CASES])
+@pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
+@pytest.mark.parametrize("out_dtype,out_zp", [(np.int8, -128), (np.int8, 127), (np.int16, 0)])
+def test_depthwise_mfma_epilogue_form_borders(ctx, name, shifts, mode, out_dtype, out_zp):
+    n, ih, iw, c, pad = 2, 13, 11, 160, (1, 1, 1, 1)
+    rng = np.random.default_rng(len(name) + mode)
+    shift = shifts(rng, c).astype(np.int8)
+    small = int(shift.max()) < 40
+    x = rng.integers(-128, 128, (n, ih, iw, c)).astype(np.int8)
+    w = rng.integers(-128, 128, (3, 3, c, 1)).astype(np.int8)
+    bias = rng.integers(-300, 300, c).astype(np.int32) if small else rng.integers(-(1 << 28), 1 << 28, c).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, c).astype(np.int32)
+    mult[:4] = [(1 << 31) - 1, 1 << 30, 0, 1]
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, in_zp=-3, w_zp=0, depthwise=True,
+                             rescale=dict(mult=mult, shift=shift, out_zp=out_zp, out_dtype=out_dtype, rounding_mode=mode))
+    assert ctx.last_kernel == "depthwise_mfma_i8_rescale"
+    acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, in_zp=-3, w_zp=0)
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp, out_dtype=out_dtype, rounding_mode=mode)
+    assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))
+    if small and out_dtype == np.int16:
+        assert len(np.unique(got)) > 50

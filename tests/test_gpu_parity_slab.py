@@ -204,3 +204,39 @@ def test_automatic_choice_takes_the_slab_kernel_for_its_layers():
         assert st == capi.VALID and c.last_kernel == "conv2d_mfma_i8"
     finally:
         c.close()
+
+
+# shifts at the borders between the epilogue's forms: 32 with double rounding takes the general form, 33 the
+# high-word form; single rounding takes the high-word form from 32 on; a mixture of both; shifts too large for
+# output_zp * 2^shift to ride in the rounding term; every multiplier at its extremes
+_FORM_CASES = [
+    ("uniform 32", lambda rng, oc: np.full(oc, 32)), ("uniform 33", lambda rng, oc: np.full(oc, 33)),
+    ("32..34", lambda rng, oc: rng.integers(32, 35, oc)), ("33..36", lambda rng, oc: rng.integers(33, 37, oc)),
+    ("30..34", lambda rng, oc: rng.integers(30, 35, oc)), ("uniform 58", lambda rng, oc: np.full(oc, 58)),
+    ("52..62", lambda rng, oc: rng.integers(52, 63, oc)),
+]
+
+
+@pytest.mark.parametrize("name,shifts", _FORM_CASES, ids=[c[0] for c in _FORM_CASES])
+@pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
+@pytest.mark.parametrize("out_dtype,out_zp", [(np.int8, -128), (np.int8, 127), (np.int16, 0)])
+def test_slab_fused_rescale_epilogue_form_borders(ctx, name, shifts, mode, out_dtype, out_zp):
+    shape = (2, 13, 11, 80, (1, 1, 1, 1), (1, 1), (1, 1))
+    x, _, _ = _operands(shape, 5)
+    rng = np.random.default_rng(len(name) + mode)
+    oc = shape[3]
+    shift = shifts(rng, oc).astype(np.int8)
+    # accumulators of a few thousand, so that a shift of 30..36 leaves values inside the output range; the large
+    # shifts get accumulators near 2^24 and multipliers near 2^31
+    small = int(shift.max()) < 40
+    w = rng.integers(-2, 3, (oc, 3, 3, 64)).astype(np.int8) if small else rng.integers(-127, 128, (oc, 3, 3, 64)).astype(np.int8)
+    bias = rng.integers(-300, 300, oc).astype(np.int32) if small else rng.integers(-(1 << 24), 1 << 24, oc).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    mult[:4] = [(1 << 31) - 1, 1 << 30, 0, 1]
+    c = dict(x=x, w=w, bias=bias, in_zp=-3, pad=shape[4], stride=shape[5], dilation=shape[6], mult=mult, shift=shift,
+             out_zp=out_zp, clamp=None, mode=mode)
+    got, st, want, wst = _fused(ctx, c, out_dtype)
+    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))
+    if small and out_dtype == np.int16:
+        assert len(np.unique(got)) > 50
