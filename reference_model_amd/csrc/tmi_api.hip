@@ -630,11 +630,10 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
         return rc;
     uint8_t* w_flip = (uint8_t*)ctx->workspace;
     uint8_t* u      = w_flip + w_bytes;
-    if (!launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip))
-        return fail(ctx, "%s: weight re-layout launch failed", op);
-    if (holes && !launch_upsample(ctx->stream, row_bytes, d->N, d->IH, d->IW, d->stride[0], d->stride[1], in_zp,
-                                  in_dev, u))
-        return fail(ctx, "%s: input re-layout launch failed", op);
+    if (!(holes ? launch_tconv_operands(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip, d->N, d->IH, d->IW,
+                                        d->stride[0], d->stride[1], in_zp, in_dev, u)
+                : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
+        return fail(ctx, "%s: operand re-layout launch failed", op);
     tmi_conv_desc_t c{};
     c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
     c.N = d->N, c.IH = UH, c.IW = UW, c.IC = d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW, c.OH = d->OH, c.OW = d->OW;
@@ -723,11 +722,9 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
         return rc;
     uint8_t* w_perm = (uint8_t*)ctx->workspace;
     uint8_t* gath   = w_perm + w_bytes;
-    if (!launch_permute_w3d(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm))
-        return fail(ctx, "%s: weight re-layout launch failed", op);
-    if (!launch_gather_depth(ctx->stream, row_bytes, d->N, d->ID, d->OD, d->KD, d->IH * d->IW, d->stride[0],
-                             d->dilation[0], d->pad[0], in_zp, in_dev, gath))
-        return fail(ctx, "%s: input re-layout launch failed", op);
+    if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
+                                d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
+        return fail(ctx, "%s: operand re-layout launch failed", op);
     tmi_conv_desc_t c{};
     c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
     c.N = d->N * d->OD, c.IH = d->IH, c.IW = d->IW, c.IC = d->KD * d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW;

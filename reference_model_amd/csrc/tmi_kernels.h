@@ -149,6 +149,12 @@ const char* launch_gather_depth(hipStream_t st, int32_t row_bytes, int32_t N, in
                                 const void* src, void* dst);
 const char* launch_permute_w3d(hipStream_t st, int32_t row_bytes, int32_t OC, int32_t KD, int32_t KHW,
                                const void* src, void* dst);
+const char* launch_tconv_operands(hipStream_t st, int32_t row_bytes, int32_t OC, int32_t KH, int32_t KW, const void* w_src,
+                                  void* w_dst, int32_t N, int32_t IH, int32_t IW, int32_t sy, int32_t sx, int32_t fill,
+                                  const void* in_src, void* in_dst);
+const char* launch_conv3d_operands(hipStream_t st, int32_t row_bytes, int32_t OC, int32_t KD, int32_t KHW, const void* w_src,
+                                   void* w_dst, int32_t N, int32_t ID, int32_t OD, int32_t HW, int32_t stride_d,
+                                   int32_t dilation_d, int32_t pad_d0, int32_t fill, const void* in_src, void* in_dst);
 // depthwise.hip: 4 channels per lane, dot4 across taps, fused epilogue; nullptr when not eligible.
 const char* launch_depthwise_vec(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                  const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
