@@ -237,8 +237,9 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
                                        int32_t clamp_max, void* out_dev);
 
 /* OpTransposeConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:2058-2197 (checks :1982-2056).
- * Evaluated as a stride-1 CONV2D with flipped taps over the input with stride-1 holes filled with input_zp;
- * the re-laid-out operands live in the context's scratch buffer. */
+ * Evaluated as a stride-1 CONV2D with flipped taps over the input with stride-1 holes filled with input_zp.
+ * INT8 with 3x3 taps, 64 / 96 / 128 input channels and w_zp 0 reads both operands in place (holes and flip are
+ * part of the kernel's addressing); otherwise the re-laid-out operands live in the context's scratch buffer. */
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 

@@ -50,6 +50,10 @@ struct SlabArgs
     int32_t pitch;               // 16-byte chunks per patch row in LDS: 5 per pixel plus the padding that spreads the banks
     int32_t step_row, step_chunk;    // 448 = step_row * pitch + step_chunk: how far 7 loads (448 slots) move
     FastDiv div_tw, div_pitch, div_tiles_x, div_tiles_y, div_ocb;
+    // TRANSPOSE_CONV2D: IH x IW above are those of the input with up_y - 1 (up_x - 1) holes between its rows (columns),
+    // which is never materialised; the tensor in memory is IHr x IWr
+    int32_t up_y, up_x, IHr, IWr;
+    FastDiv div_up_y, div_up_x;
 };
 
 __device__ __forceinline__ void slab_load(const void* src, uint32_t lds_addr)
@@ -65,7 +69,11 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
 }
 
 // CH: 16-byte chunks of a channel vector (4, 6, 8: 64, 96, 128 input channels)
-template <int KH, int KW, int CH, bool ZA, bool FUSED>
+// TC: TRANSPOSE_CONV2D (tensor_ops.cpp:2138-2187) as the stride-1 CONV2D with flipped taps over the input with holes:
+// a hole reads the page of input_zp bytes like a pixel outside the image (it contributes (zp - zp) * w = 0, as the
+// reference's skipped tap does), and the flip is applied where a K step picks its place in the patch, so neither
+// operand is copied.
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
@@ -150,7 +158,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             }
         }
         {
-            const uint8_t* in_n = a.in + (size_t)n * a.IH * a.IW * KB;
+            const uint8_t* in_n = a.in + (size_t)n * (TC ? a.IHr * a.IWr : a.IH * a.IW) * KB;
             int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
             const int s0        = lp * 64 + lane;
             int py              = fdiv(s0, a.div_pitch);    // patch row and chunk inside the row
@@ -161,9 +169,16 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 const int px   = (int)((uint32_t)r / (uint32_t)RP);
                 const int ch   = r - px * RP;
                 const int iy = y0 + py, ix = x0 + px;
-                const bool img = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+                bool img       = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
                 const int c16  = (ch < CH ? ch : 0) * 16;
-                const uint8_t* src = img ? in_n + (uint32_t)((__umul24(iy, a.IW) + ix) * KB + c16) : a.pad_page + (c16 & 48);
+                uint32_t pixel = __umul24(iy, a.IW) + ix;
+                if constexpr (TC)
+                {
+                    const int ry = fdiv(img ? iy : 0, a.div_up_y), rx = fdiv(img ? ix : 0, a.div_up_x);
+                    img          = img && ry * a.up_y == iy && rx * a.up_x == ix;
+                    pixel        = __umul24(ry, a.IWr) + rx;
+                }
+                const uint8_t* src = img ? in_n + (uint32_t)(pixel * KB + c16) : a.pad_page + (c16 & 48);
                 slab_load(src, dst);
                 dst += LWAVES * 1024;
                 r += a.step_chunk, py += a.step_row;
@@ -256,8 +271,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         v4i fa[STEPS], fb[STEPS];
         auto request = [&](int s) {
             const int tap = s / (CH / 2), h = s % (CH / 2);
+            const int at  = TC ? TAPS - 1 - tap : tap;    // flipped taps: weight tap (ky, kx) meets patch tap (KH-1-ky, KW-1-kx)
             fa[s] = *reinterpret_cast<const v4i*>(wrow + s * 32);
-            fb[s] = *reinterpret_cast<const v4i*>(prow + (tap / KW) * row_step + (tap % KW) * col_step + h * 32);
+            fb[s] = *reinterpret_cast<const v4i*>(prow + (at / KW) * row_step + (at % KW) * col_step + h * 32);
         };
 #pragma unroll
         for (int s = 0; s < DEPTH; s++)
@@ -396,10 +412,10 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     raise_flags(a.flag_word, flags);
 }
 
-template <int KH, int KW, int CH, bool ZA, bool FUSED>
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
-    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED>;
+    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
@@ -420,10 +436,12 @@ static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int ld
 // nullptr when the layer is not one this kernel takes; the caller then goes to the patch kernel.
 const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                               void* out, const void* pad_page, uint32_t* flag_word)
+                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc)
 {
     const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
     if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 96 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
+        return nullptr;
+    if (tc && (!k33 || rp.enabled || tc->up_y < 1 || tc->up_x < 1 || g.stride_y != 1 || g.stride_x != 1))
         return nullptr;
     const int taps = g.KH * g.KW;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
@@ -509,6 +527,20 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 80 * 4 + 16;
     const bool fused = rp.enabled != 0;
     bool ok;
+    if (tc)
+    {
+        a.up_y = tc->up_y, a.up_x = tc->up_x, a.IHr = tc->IH, a.IWr = tc->IW;
+        a.div_up_y = make_fastdiv((uint32_t)tc->up_y), a.div_up_x = make_fastdiv((uint32_t)tc->up_x);
+        if (a.za != 0)
+            ok = ch == 4 ? launch_slab_kernel<3, 3, 4, true, false, true>(st, a, (int)grid, lds_bytes)
+                         : (ch == 6 ? launch_slab_kernel<3, 3, 6, true, false, true>(st, a, (int)grid, lds_bytes)
+                                    : launch_slab_kernel<3, 3, 8, true, false, true>(st, a, (int)grid, lds_bytes));
+        else
+            ok = ch == 4 ? launch_slab_kernel<3, 3, 4, false, false, true>(st, a, (int)grid, lds_bytes)
+                         : (ch == 6 ? launch_slab_kernel<3, 3, 6, false, false, true>(st, a, (int)grid, lds_bytes)
+                                    : launch_slab_kernel<3, 3, 8, false, false, true>(st, a, (int)grid, lds_bytes));
+        return ok ? "transpose_conv2d_slab_i8" : nullptr;
+    }
     if (k33)
         ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused)
                      : (ch == 6 ? launch_slab_taps<3, 3, 6>(st, a, (int)grid, lds_bytes, fused)

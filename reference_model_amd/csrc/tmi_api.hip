@@ -623,6 +623,27 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
     const int row_bytes  = d->IC * eb;
     const bool holes     = d->stride[0] > 1 || d->stride[1] > 1;
     const int32_t UH     = (d->IH - 1) * d->stride[0] + 1, UW = (d->IW - 1) * d->stride[1] + 1;
+    tmi_conv_desc_t c{};
+    c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
+    c.N = d->N, c.IH = UH, c.IW = UW, c.IC = d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW, c.OH = d->OH, c.OW = d->OW;
+    c.pad[0] = d->KH - 1 + d->out_pad[0], c.pad[1] = d->KH - 1 + d->out_pad[1];
+    c.pad[2] = d->KW - 1 + d->out_pad[2], c.pad[3] = d->KW - 1 + d->out_pad[3];
+    c.stride[0] = c.stride[1] = 1, c.dilation[0] = c.dilation[1] = 1;
+    c.bias_len = d->bias_len;
+    RescaleParams none{};
+    // the slab kernel reads both operands where they lie (holes and flip are part of its addressing)
+    if ((ctx->kernel_choice == 0 || ctx->kernel_choice == 4) && d->in_dtype == TMI_INT8)
+    {
+        ConvGeom g;
+        rc = validate_conv(ctx, op, &c, false, in_zp, w_zp, g);
+        if (rc != TMI_VALID)
+            return rc;
+        const SlabHoles h{ d->stride[0], d->stride[1], d->IH, d->IW };
+        const char* name = launch_conv2d_slab(ctx->stream, d->in_dtype, d->out_dtype, g, in_dev, weight_dev, bias_dev, in_zp,
+                                              w_zp, none, out_dev, ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev, &h);
+        if (name)
+            return after_launch(ctx, name);
+    }
     const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * row_bytes);
     const size_t u_bytes = holes ? align256((size_t)d->N * UH * UW * row_bytes) : 0;
     rc                   = ensure_workspace(ctx, w_bytes + u_bytes);
@@ -634,14 +655,6 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
                                         d->stride[0], d->stride[1], in_zp, in_dev, u)
                 : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
         return fail(ctx, "%s: operand re-layout launch failed", op);
-    tmi_conv_desc_t c{};
-    c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
-    c.N = d->N, c.IH = UH, c.IW = UW, c.IC = d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW, c.OH = d->OH, c.OW = d->OW;
-    c.pad[0] = d->KH - 1 + d->out_pad[0], c.pad[1] = d->KH - 1 + d->out_pad[1];
-    c.pad[2] = d->KW - 1 + d->out_pad[2], c.pad[3] = d->KW - 1 + d->out_pad[3];
-    c.stride[0] = c.stride[1] = 1, c.dilation[0] = c.dilation[1] = 1;
-    c.bias_len = d->bias_len;
-    RescaleParams none{};
     return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
                     d->out_dtype, out_dev);
 }

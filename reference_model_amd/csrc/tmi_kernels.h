@@ -108,9 +108,16 @@ const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int3
 // conv2d_slab.hip: int8 CONV2D with IC = 64, 96 or 128, 3x3 or 1x1 taps and weight_zp = 0 (int32 result, or the fast form of a fused
 // RESCALE to int8 / int16): weight slab and input patch loaded straight into LDS; nullptr for anything else.
 // pad_page: 64 bytes of input_zp in device memory.
+// TRANSPOSE_CONV2D through the slab kernel: the CONV2D geometry handed over describes the stride-1 convolution over the
+// input with up_y - 1 (up_x - 1) holes between its rows (columns); IH x IW are those of the tensor in memory, and
+// the weights are in TRANSPOSE_CONV2D's own tap order.
+struct SlabHoles
+{
+    int32_t up_y, up_x, IH, IW;
+};
 const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                               void* out, const void* pad_page, uint32_t* flag_word);
+                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc = nullptr);
 
 // depthwise_slab.hip: int8 DEPTHWISE_CONV2D with multiplier 1, 3x3 taps, weight_zp = 0 and 32..512 channels in
 // multiples of 16 on the matrix cores (one MFMA per tap against a diagonal weight tile); nullptr for anything else.

@@ -59,6 +59,45 @@ def test_transpose_conv2d_i8_bit_exact(ctx, shape, zps):
         assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
 
 
+SLAB_TCONV = [  # 3x3 taps, 64 / 96 / 128 input channels, zero weight_zp: both operands are read where they lie
+    (2, 14, 14, 64, 48, (0, 0, 0, 0), (2, 2)),        # a decoder-style 2x upsampling layer
+    (4, 28, 28, 128, 64, (0, -1, 0, -1), (2, 2)),     # cropped to exactly twice the input
+    (3, 9, 11, 96, 80, (1, 0, 0, 2), (1, 1)),         # no holes: the flip alone
+    (2, 7, 10, 64, 64, (-1, -2, 0, -1), (2, 3)),      # different strides, cropping on three sides
+    (1, 6, 5, 128, 112, (0, 0, -2, 0), (3, 1)),
+]
+
+
+@pytest.fixture(scope="module")
+def auto_ctx():
+    c = Context(0)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("shape", SLAB_TCONV)
+@pytest.mark.parametrize("in_zp", [0, -7, 127])
+def test_transpose_conv2d_slab_reads_operands_in_place(auto_ctx, shape, in_zp):
+    ctx = auto_ctx
+    n, ih, iw, ic, oc, out_pad, stride = shape
+    rng = np.random.default_rng(ih * iw + ic + oc)
+    x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, 3, 3, ic)).astype(np.int8)
+    for bias in (rng.integers(-9999, 9999, oc).astype(np.int32), np.array([-77], np.int32)):
+        want = oracle.transpose_conv2d("i8", x, w, bias, out_pad, stride, in_zp, 0)
+        got, st = gpu_ops.transpose_conv2d(ctx, x, w, bias, out_pad, stride, in_zp, 0)
+        assert ctx.last_kernel == "transpose_conv2d_slab_i8"
+        assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(got)) > 50
+    # a weight zero point, or any other kernel choice, goes through the re-laid-out operands: same result
+    ctx.set_kernel_choice(capi.KERNEL_MFMA)
+    try:
+        got2, st = gpu_ops.transpose_conv2d(ctx, x, w, bias, out_pad, stride, in_zp, 0)
+        assert ctx.last_kernel != "transpose_conv2d_slab_i8" and st == capi.VALID and np.array_equal(got2, want)
+    finally:
+        ctx.set_kernel_choice(capi.KERNEL_AUTO)
+
+
 BIG_CONV3D = [
     (1, 8, 12, 12, 16, 32, 3, 3, 3, (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)),
     (2, 6, 9, 9, 32, 24, 2, 3, 3, (0, 0, 1, 1, 1, 1), (2, 2, 2), (1, 1, 1)),
