@@ -244,7 +244,9 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
 /* OpConv3d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:935-1120 (checks :901-933, :120-226).
- * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side. */
+ * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side.  INT8 with 3x3 taps in
+ * the plane, KD*IC = 64 / 96 / 128 (IC 32 or 64) and w_zp 0 reads both operands in place; otherwise the gathered
+ * input and the permuted weights live in the context's scratch buffer. */
 int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 

@@ -54,6 +54,10 @@ struct SlabArgs
     // which is never materialised; the tensor in memory is IHr x IWr
     int32_t up_y, up_x, IHr, IWr;
     FastDiv div_up_y, div_up_x;
+    // CONV3D: image n above is output slice (n / OD, n % OD); chunk group kd of a pixel comes from input slice
+    // od * sd + kd * dd - pd0 of a volume of ID slices
+    int32_t ID, OD, sd, dd, pd0;
+    FastDiv div_od;
 };
 
 __device__ __forceinline__ void slab_load(const void* src, uint32_t lds_addr)
@@ -73,7 +77,11 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
 // a hole reads the page of input_zp bytes like a pixel outside the image (it contributes (zp - zp) * w = 0, as the
 // reference's skipped tap does), and the flip is applied where a K step picks its place in the patch, so neither
 // operand is copied.
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false>
+// KD > 1: CONV3D (tensor_ops.cpp:1058-1108) with the KD depth taps as channel groups of a CONV2D over the output
+// slices: the patch loader takes chunk group kd of a pixel from input slice od * sd + kd * dd - pd0 (a slice outside
+// the volume reads the input_zp page), and the weights stay in their own [OC][KD][KH][KW][IC] order, a K step
+// (tap, kd, half) finding its place in the row at compile time.  Neither operand is copied.
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
@@ -159,6 +167,10 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         }
         {
             const uint8_t* in_n = a.in + (size_t)n * (TC ? a.IHr * a.IWr : a.IH * a.IW) * KB;
+            constexpr int ICC   = CH / KD;    // chunks of a channel vector in memory
+            const int nb        = KD > 1 ? (int)fdiv(n, a.div_od) : 0;
+            const int slice0    = nb * a.ID;                              // first slice of the volume
+            const int z0        = (n - nb * a.OD) * a.sd - a.pd0;         // slice under depth tap 0
             int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
             const int s0        = lp * 64 + lane;
             int py              = fdiv(s0, a.div_pitch);    // patch row and chunk inside the row
@@ -179,6 +191,15 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                     pixel        = __umul24(ry, a.IWr) + rx;
                 }
                 const uint8_t* src = img ? in_n + (uint32_t)(pixel * KB + c16) : a.pad_page + (c16 & 48);
+                if constexpr (KD > 1)
+                {
+                    const int chc = ch < CH ? ch : 0;
+                    const int kd  = chc / ICC, cc = chc - kd * ICC;
+                    const int z   = z0 + kd * a.dd;
+                    img           = img && (unsigned)z < (unsigned)a.ID;
+                    src           = img ? a.in + (((uint32_t)(slice0 + z) * (uint32_t)(a.IH * a.IW) + pixel) * (ICC * 16) + cc * 16)
+                                        : a.pad_page + (c16 & 48);
+                }
                 slab_load(src, dst);
                 dst += LWAVES * 1024;
                 r += a.step_chunk, py += a.step_row;
@@ -272,7 +293,13 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         auto request = [&](int s) {
             const int tap = s / (CH / 2), h = s % (CH / 2);
             const int at  = TC ? TAPS - 1 - tap : tap;    // flipped taps: weight tap (ky, kx) meets patch tap (KH-1-ky, KW-1-kx)
-            fa[s] = *reinterpret_cast<const v4i*>(wrow + s * 32);
+            int aoff      = s * 32;
+            if constexpr (KD > 1)
+            {
+                constexpr int ICH = CH / KD / 2;    // 32-byte pieces of a channel vector in memory
+                aoff              = (((h / ICH) * TAPS + tap) * ICH + h % ICH) * 32;
+            }
+            fa[s] = *reinterpret_cast<const v4i*>(wrow + aoff);
             fb[s] = *reinterpret_cast<const v4i*>(prow + (at / KW) * row_step + (at % KW) * col_step + h * 32);
         };
 #pragma unroll
@@ -412,10 +439,10 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     raise_flags(a.flag_word, flags);
 }
 
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false>
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
-    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC>;
+    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC, KD>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
@@ -436,13 +463,21 @@ static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int ld
 // nullptr when the layer is not one this kernel takes; the caller then goes to the patch kernel.
 const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc)
+                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc,
+                               const SlabDepth* c3d)
 {
     const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
     if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 96 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
     if (tc && (!k33 || rp.enabled || tc->up_y < 1 || tc->up_x < 1 || g.stride_y != 1 || g.stride_x != 1))
         return nullptr;
+    if (c3d)
+    {
+        const int icr = c3d->KD > 0 ? g.IC / c3d->KD : 0;    // channels of the tensor in memory
+        const bool kd_ok = (icr == 32 && c3d->KD >= 2 && c3d->KD <= 4) || (icr == 64 && c3d->KD == 2);
+        if (tc || !k33 || rp.enabled || !kd_ok || icr * c3d->KD != g.IC || c3d->OD < 1 || g.N % c3d->OD != 0)
+            return nullptr;
+    }
     const int taps = g.KH * g.KW;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
         return nullptr;
@@ -527,6 +562,25 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 80 * 4 + 16;
     const bool fused = rp.enabled != 0;
     bool ok;
+    if (c3d)
+    {
+        a.ID = c3d->ID, a.OD = c3d->OD, a.sd = c3d->stride_d, a.dd = c3d->dilation_d, a.pd0 = c3d->pad_d0;
+        a.div_od = make_fastdiv((uint32_t)c3d->OD);
+        const bool za = a.za != 0;
+        if (ch == 4)
+            ok = za ? launch_slab_kernel<3, 3, 4, true, false, false, 2>(st, a, (int)grid, lds_bytes)
+                    : launch_slab_kernel<3, 3, 4, false, false, false, 2>(st, a, (int)grid, lds_bytes);
+        else if (ch == 6)
+            ok = za ? launch_slab_kernel<3, 3, 6, true, false, false, 3>(st, a, (int)grid, lds_bytes)
+                    : launch_slab_kernel<3, 3, 6, false, false, false, 3>(st, a, (int)grid, lds_bytes);
+        else if (c3d->KD == 4)
+            ok = za ? launch_slab_kernel<3, 3, 8, true, false, false, 4>(st, a, (int)grid, lds_bytes)
+                    : launch_slab_kernel<3, 3, 8, false, false, false, 4>(st, a, (int)grid, lds_bytes);
+        else
+            ok = za ? launch_slab_kernel<3, 3, 8, true, false, false, 2>(st, a, (int)grid, lds_bytes)
+                    : launch_slab_kernel<3, 3, 8, false, false, false, 2>(st, a, (int)grid, lds_bytes);
+        return ok ? "conv3d_slab_i8" : nullptr;
+    }
     if (tc)
     {
         a.up_y = tc->up_y, a.up_x = tc->up_x, a.IHr = tc->IH, a.IWr = tc->IW;

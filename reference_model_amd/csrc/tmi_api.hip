@@ -728,16 +728,6 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
 
     const int eb         = dtype_bits(d->in_dtype) / 8;
     const int row_bytes  = d->IC * eb;
-    const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * row_bytes);
-    const size_t g_bytes = align256((size_t)d->N * d->OD * d->IH * d->IW * d->KD * row_bytes);
-    rc                   = ensure_workspace(ctx, w_bytes + g_bytes);
-    if (rc != TMI_VALID)
-        return rc;
-    uint8_t* w_perm = (uint8_t*)ctx->workspace;
-    uint8_t* gath   = w_perm + w_bytes;
-    if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
-                                d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
-        return fail(ctx, "%s: operand re-layout launch failed", op);
     tmi_conv_desc_t c{};
     c.in_dtype = d->in_dtype, c.out_dtype = d->out_dtype;
     c.N = d->N * d->OD, c.IH = d->IH, c.IW = d->IW, c.IC = d->KD * d->IC, c.OC = d->OC, c.KH = d->KH, c.KW = d->KW;
@@ -748,6 +738,30 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     c.dilation[0] = d->dilation[1], c.dilation[1] = d->dilation[2];
     c.bias_len = d->bias_len;
     RescaleParams none{};
+    // the slab kernel reads both operands where they lie (the depth taps are part of its addressing)
+    if ((ctx->kernel_choice == 0 || ctx->kernel_choice == 4) && d->in_dtype == TMI_INT8 && d->KD > 1)
+    {
+        ConvGeom g;
+        rc = validate_conv(ctx, op, &c, false, in_zp, w_zp, g);
+        if (rc != TMI_VALID)
+            return rc;
+        const SlabDepth dep{ d->KD, d->ID, d->OD, d->stride[0], d->dilation[0], d->pad[0] };
+        const char* name = launch_conv2d_slab(ctx->stream, d->in_dtype, d->out_dtype, g, in_dev, weight_dev, bias_dev, in_zp,
+                                              w_zp, none, out_dev, ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev,
+                                              nullptr, &dep);
+        if (name)
+            return after_launch(ctx, name);
+    }
+    const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * row_bytes);
+    const size_t g_bytes = align256((size_t)d->N * d->OD * d->IH * d->IW * d->KD * row_bytes);
+    rc                   = ensure_workspace(ctx, w_bytes + g_bytes);
+    if (rc != TMI_VALID)
+        return rc;
+    uint8_t* w_perm = (uint8_t*)ctx->workspace;
+    uint8_t* gath   = w_perm + w_bytes;
+    if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
+                                d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
+        return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev);
 }
 

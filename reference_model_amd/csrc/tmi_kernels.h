@@ -115,9 +115,16 @@ struct SlabHoles
 {
     int32_t up_y, up_x, IH, IW;
 };
+// CONV3D through the slab kernel: the CONV2D geometry handed over has N * OD images and KD * IC channels; the input
+// tensor [N, ID, IH, IW, IC] and the weights [OC, KD, KH, KW, IC] are read where they lie.
+struct SlabDepth
+{
+    int32_t KD, ID, OD, stride_d, dilation_d, pad_d0;
+};
 const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc = nullptr);
+                               void* out, const void* pad_page, uint32_t* flag_word, const SlabHoles* tc = nullptr,
+                               const SlabDepth* c3d = nullptr);
 
 // depthwise_slab.hip: int8 DEPTHWISE_CONV2D with multiplier 1, 3x3 taps, weight_zp = 0 and 32..512 channels in
 // multiples of 16 on the matrix cores (one MFMA per tap against a diagonal weight tile); nullptr for anything else.

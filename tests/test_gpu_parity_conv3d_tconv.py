@@ -117,6 +117,39 @@ def test_conv3d_i8_bit_exact(ctx, shape, zps):
         assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
 
 
+SLAB_CONV3D = [  # 3x3 taps in the plane, KD x IC = 64 / 96 / 128 bytes per pixel, zero weight_zp: operands read in place
+    (2, 8, 14, 14, 32, 64, 3, (1, 1, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)),    # the bench configuration's geometry, small
+    (1, 6, 9, 11, 32, 48, 2, (0, 1, 1, 0, 2, 1), (1, 1, 1), (1, 1, 1)),     # two depth taps, uneven padding
+    (2, 9, 10, 10, 32, 80, 4, (2, 1, 1, 1, 1, 1), (2, 1, 1), (1, 1, 1)),    # four depth taps, depth stride 2
+    (1, 7, 8, 8, 64, 64, 2, (1, 1, 1, 1, 1, 1), (1, 1, 1), (2, 1, 1)),      # 64 channels, depth dilation 2
+    (1, 7, 13, 9, 32, 64, 3, (1, 1, 0, 0, 1, 1), (1, 2, 1), (1, 1, 1)),     # stride 2 along the height
+    (3, 5, 6, 6, 32, 112, 3, (3, 3, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)),     # depth padding larger than the taps reach
+]
+
+
+@pytest.mark.parametrize("shape", SLAB_CONV3D)
+@pytest.mark.parametrize("in_zp", [0, 6, -128])
+def test_conv3d_slab_reads_operands_in_place(auto_ctx, shape, in_zp):
+    ctx = auto_ctx
+    n, idp, ih, iw, ic, oc, kd, pad, stride, dil = shape
+    rng = np.random.default_rng(idp * ih + iw + ic + oc + kd)
+    x = rng.integers(-128, 128, (n, idp, ih, iw, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kd, 3, 3, ic)).astype(np.int8)
+    for bias in (rng.integers(-9999, 9999, oc).astype(np.int32), np.array([-5], np.int32)):
+        want = oracle.conv3d("i8", x, w, bias, pad, stride, dil, in_zp, 0)
+        got, st = gpu_ops.conv3d(ctx, x, w, bias, pad, stride, dil, in_zp, 0)
+        assert ctx.last_kernel == "conv3d_slab_i8"
+        assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(got)) > 50
+    # any other kernel choice goes through the re-laid-out operands: same result
+    ctx.set_kernel_choice(capi.KERNEL_MFMA)
+    try:
+        got2, st = gpu_ops.conv3d(ctx, x, w, bias, pad, stride, dil, in_zp, 0)
+        assert ctx.last_kernel != "conv3d_slab_i8" and st == capi.VALID and np.array_equal(got2, want)
+    finally:
+        ctx.set_kernel_choice(capi.KERNEL_AUTO)
+
+
 def test_fp16_variants_within_dot_product_bound(ctx):
     rng = np.random.default_rng(12)
     x = rng.normal(0, 1, (1, 6, 6, 32)).astype(np.float16)
