@@ -38,7 +38,7 @@ PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/
 # the same counters read for a plain copy of known size (the committed rocprofv3 summaries hold the raw
 # figures).
 MEASURED_TRAFFIC_BYTES = {"c3": 3639807, "c2": 51169875, "c4": 12201793, "c5a": 22848575, "c5b": 269061469,
-                          "maxpool": 43565388, "avgpool": 32175434, "tconv": 8340286, "conv3d": 8037071,
+                          "maxpool": 32144806, "avgpool": 32183530, "tconv": 8340286, "conv3d": 8037071,
                           "rescale": 64289281, "c4x8": 96473119}
 
 

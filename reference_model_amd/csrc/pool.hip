@@ -30,6 +30,8 @@ struct PoolArgs
     int32_t in_zp, out_zp, qmin, qmax;
     int32_t nan_mode;    // MAX_POOL2D, floating point: 1 = PROPAGATE, 2 = IGNORE
     int32_t groups;      // channel groups of VEC elements per pixel
+    int32_t full_mult, full_k;    // AVG_POOL2D: reciprocal_scale of a whole window (ky * kx taps), worked out on the host
+    int32_t xcd_remap;            // the grid is a multiple of 8 workgroups: give each XCD a contiguous range of pixels
 };
 
 template <typename T>
@@ -89,10 +91,17 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a)
     using P                  = PoolType<T>;
     using acc_t              = typename P::acc_t;
     constexpr int kVecBytes  = VEC * (int)sizeof(T);
-    const int64_t stride     = (int64_t)gridDim.x * blockDim.x;
     uint32_t flags           = 0;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total; i += stride)
+    // Consecutive workgroups go to the 8 XCDs in turn, each with its own L2.  Windows that overlap (stride < kernel)
+    // share input rows with the next output row: XCD x takes workgroups [x * per, x * per + per) of the pixel order, so
+    // that neighbouring output rows meet in one L2 instead of fetching the shared rows from HBM twice.
+    uint32_t bid = blockIdx.x;
+    if (a.xcd_remap)
+        bid = (bid & 7) * (gridDim.x >> 3) + (bid >> 3);
     {
+        const int64_t i = (int64_t)bid * blockDim.x + threadIdx.x;
+        if (i >= a.total)
+            return;
         // (pixel, channel group); totals below 2^32 are checked on the host
         const uint32_t pix = (uint32_t)i / (uint32_t)a.groups;
         const int grp      = (int)((uint32_t)i - pix * (uint32_t)a.groups);
@@ -145,15 +154,38 @@ __global__ __launch_bounds__(256) void pool_kernel(PoolArgs a)
         if constexpr (AVG && P::is_int)
         {
             // QuantUtil::reciprocal_scale: (1 << k) / 2 < count <= (1 << k)
-            const int count    = (y1 - y0) * (x1 - x0);
-            const int k        = 32 - __clz(count - 1);    // __clz(0) = 32
-            const int32_t mult = (int32_t)((((uint64_t(1) << 30) + 1) << k) / (uint32_t)count);
-#pragma unroll
-            for (int e = 0; e < VEC; e++)
+            const int count = (y1 - y0) * (x1 - x0);
+            int k           = a.full_k;
+            int32_t mult    = a.full_mult;
+            if (count != a.ky * a.kx)    // a window cut by the border: the 64-bit division is worth avoiding elsewhere
             {
-                int32_t v = apply_scale_32(acc[e], mult, 30 + k, false, flags) + a.out_zp;
-                v         = v > a.qmin ? v : a.qmin;
-                r[e]      = P::narrow(v < a.qmax ? v : a.qmax);
+                k    = 32 - __clz(count - 1);    // __clz(0) = 32
+                mult = (int32_t)((((uint64_t(1) << 30) + 1) << k) / (uint32_t)count);
+            }
+            if (a.ky * a.kx <= 8192)
+            {
+                // |acc| <= taps * 2^16 <= 2^(k + 16) stays below 2^(29 + k), the range apply_scale_32 asks of a value for
+                // the shift 30 + k (quant_util.h:59-67), and the scaled value stays below 2^30: neither REQUIRE can
+                // fire, so the plain formula is the whole function
+                const int shift   = 30 + k;
+                const int64_t rnd = int64_t(1) << (shift - 1);
+#pragma unroll
+                for (int e = 0; e < VEC; e++)
+                {
+                    int32_t v = (int32_t)(((int64_t)acc[e] * mult + rnd) >> shift) + a.out_zp;
+                    v         = v > a.qmin ? v : a.qmin;
+                    r[e]      = P::narrow(v < a.qmax ? v : a.qmax);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int e = 0; e < VEC; e++)
+                {
+                    int32_t v = apply_scale_32(acc[e], mult, 30 + k, false, flags) + a.out_zp;
+                    v         = v > a.qmin ? v : a.qmin;
+                    r[e]      = P::narrow(v < a.qmax ? v : a.qmax);
+                }
             }
         }
         else if constexpr (AVG)
@@ -188,9 +220,8 @@ static const char* launch_pool_t(hipStream_t st, PoolArgs& a, int32_t N, const c
     a.total           = (int64_t)N * a.OH * a.OW * a.groups;
     if (a.total >= (int64_t(1) << 32))
         return nullptr;
-    int64_t blocks = (a.total + 255) / 256;
-    if (blocks > 256 * 32)
-        blocks = 256 * 32;
+    const int64_t blocks = ((a.total + 255) / 256 + 7) & ~int64_t(7);    // whole groups of 8 for the XCD order
+    a.xcd_remap          = 1;
     if (vec)
         hipLaunchKernelGGL((pool_kernel<T, AVG, VEC>), dim3((int)blocks), dim3(256), 0, st, a);
     else
@@ -209,6 +240,15 @@ const char* launch_pool(hipStream_t st, bool avg, int32_t dtype, int32_t N, int3
     a.IH = IH, a.IW = IW, a.C = C, a.OH = OH, a.OW = OW;
     a.ky = kernel_y, a.kx = kernel_x, a.sy = stride_y, a.sx = stride_x, a.pad_top = pad_top, a.pad_left = pad_left;
     a.in_zp = in_zp, a.out_zp = out_zp, a.nan_mode = nan_mode;
+    {
+        // QuantUtil::reciprocal_scale (quant_util.h:32-43) for a window that lies inside the image
+        const uint32_t count = (uint32_t)kernel_y * (uint32_t)kernel_x;
+        int k                = 0;
+        while (k < 32 && (uint64_t(1) << k) < count)
+            k++;
+        a.full_k    = k;
+        a.full_mult = count ? (int32_t)((((uint64_t(1) << 30) + 1) << k) / count) : 0;
+    }
     switch (dtype)
     {
         case TMI_INT8:
