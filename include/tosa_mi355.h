@@ -106,6 +106,14 @@ const char* tmi_last_error(const tmi_ctx_t* ctx);
 /* Name of the kernel variant chosen by the most recent operator call (for tests and profiling). */
 const char* tmi_last_kernel(const tmi_ctx_t* ctx);
 
+/* Grows the context's scratch buffer (the re-laid-out operands of TRANSPOSE_CONV2D / CONV3D layers that are not
+ * read in place, MATMUL's transposed second operand) to at least `bytes`.  Lifetime rule of that buffer: an operator
+ * call that needs more than the buffer holds allocates a larger block and keeps the old one until
+ * tmi_ctx_destroy(), so launches already enqueued and HIP graphs captured earlier stay valid; while the context's
+ * stream is being captured such a call returns TMI_ERROR instead of allocating -- size the buffer beforehand with
+ * this function or with one eager call of the same operator.  Has no counterpart in the reference. */
+int tmi_ctx_reserve_workspace(tmi_ctx_t* ctx, size_t bytes);
+
 /* ---- device memory (replaces Tensor::allocate / deallocate and the element-wise host copies of
  *      reference_model/src/tensor.cpp:993-1015, 4722-4736) -------------------------------------------- */
 int tmi_buf_alloc(tmi_ctx_t* ctx, size_t bytes, void** out_dev);

@@ -35,7 +35,9 @@ EXPORTS = [
     "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
     "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
+    "tmi_ctx_reserve_workspace",
 ]
+
 
 
 class ConvDesc(ctypes.Structure):
@@ -113,6 +115,7 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_last_kernel.argtypes = [vp]
     lib.tmi_last_kernel.restype = ctypes.c_char_p
     lib.tmi_ctx_set_kernel_choice.argtypes = [vp, i32]
+    lib.tmi_ctx_reserve_workspace.argtypes = [vp, ctypes.c_size_t]
     lib.tmi_buf_alloc.argtypes = [vp, ctypes.c_size_t, ctypes.POINTER(vp)]
     lib.tmi_buf_free.argtypes = [vp, vp]
     lib.tmi_upload.argtypes = [vp, vp, vp, ctypes.c_size_t]
@@ -123,6 +126,9 @@ def load_library() -> ctypes.CDLL:
     fused = conv_args + [ctypes.POINTER(RescaleDesc), vp, vp, i32, i32, i32, vp]
     lib.tmi_conv2d_rescale_clamp.argtypes = fused
     lib.tmi_depthwise_conv2d_rescale_clamp.argtypes = fused
+    tconv_args = [vp, ctypes.POINTER(TconvDesc), vp, vp, vp, i32, i32, vp]
+    lib.tmi_transpose_conv2d.argtypes = tconv_args
+    lib.tmi_conv3d.argtypes = [vp, ctypes.POINTER(Conv3dDesc), vp, vp, vp, i32, i32, vp]
     lib.tmi_matmul.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, i32, vp]
     lib.tmi_rescale.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i64, i32, vp, vp, vp, vp]
     lib.tmi_clamp.argtypes = [vp, i32, i64, vp, i32, i32, vp]
@@ -283,6 +289,9 @@ class Context:
     def transpose_conv2d(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_transpose_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
                                                          _ptr(bias), in_zp, w_zp, _ptr(out)))
+
+    def reserve_workspace(self, nbytes: int) -> int:
+        return self._check(self.lib.tmi_ctx_reserve_workspace(self.handle, nbytes))
 
     def conv2d_precise(self, d: ConvDesc, inp, w, bias, bounds_mode, out, depthwise=False) -> int:
         fn = self.lib.tmi_depthwise_conv2d_precise if depthwise else self.lib.tmi_conv2d_precise

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <vector>
 
 #include "tmi_kernels.h"
 
@@ -18,6 +19,7 @@ struct tmi_ctx
     uint32_t* flags_host  = nullptr;    // pinned staging word
     void* workspace       = nullptr;    // scratch for operand re-layout (MATMUL's transposed B)
     size_t workspace_size = 0;
+    std::vector<void*> retired;         // outgrown scratch blocks: captured graphs may still name them
     uint32_t last_flags   = 0;
     int32_t kernel_choice = 0;
     std::string last_error;
@@ -65,17 +67,23 @@ int after_launch(tmi_ctx* ctx, const char* kernel_name)
     return TMI_VALID;
 }
 
-// Grows the context's scratch buffer; the old one is released only after the stream has drained.
+// Grows the context's scratch buffer.  An outgrown block is kept until tmi_ctx_destroy: launches already
+// enqueued, and HIP graphs captured from earlier calls, still name it.  Growing is refused while the stream is
+// being captured (an allocation cannot be part of a graph): the caller sizes the buffer with an eager call of
+// the same operator first, or uses tmi_ctx_reserve_workspace().
 int ensure_workspace(tmi_ctx* ctx, size_t bytes)
 {
     if (bytes <= ctx->workspace_size)
         return TMI_VALID;
-    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+        return fail(ctx, "the context's scratch buffer would have to grow to %zu bytes during stream capture: "
+                         "call tmi_ctx_reserve_workspace first", bytes);
+    void* block = nullptr;
+    TMI_HIP(ctx, hipMalloc(&block, bytes));
     if (ctx->workspace)
-        TMI_HIP(ctx, hipFree(ctx->workspace));
-    ctx->workspace      = nullptr;
-    ctx->workspace_size = 0;
-    TMI_HIP(ctx, hipMalloc(&ctx->workspace, bytes));
+        ctx->retired.push_back(ctx->workspace);
+    ctx->workspace      = block;
     ctx->workspace_size = bytes;
     return TMI_VALID;
 }
@@ -413,6 +421,8 @@ int tmi_ctx_destroy(tmi_ctx_t* ctx)
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->workspace)
         (void)hipFree(ctx->workspace);
+    for (void* block : ctx->retired)
+        (void)hipFree(block);
     if (ctx->flags_dev)
         (void)hipFree(ctx->flags_dev);
     if (ctx->pages_dev)
@@ -478,6 +488,14 @@ int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;
+}
+
+int tmi_ctx_reserve_workspace(tmi_ctx_t* ctx, size_t bytes)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    return ensure_workspace(ctx, bytes);
 }
 
 int tmi_buf_alloc(tmi_ctx_t* ctx, size_t bytes, void** out_dev)
