@@ -251,6 +251,21 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
+/* Size of the scratch array behind tmi_transpose_conv2d_noalloc: 16 MiB of device memory per GPU the library is
+ * used on, part of the library's device image and held until the process ends. */
+#define TMI_NOALLOC_SCRATCH_BYTES (16u << 20)
+
+/* tmi_transpose_conv2d for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same operands, results and
+ * status as tmi_transpose_conv2d, but the re-laid-out operands (flipped weights: OC*KH*KW*IC elements; the input
+ * with its stride holes: N*((IH-1)*sy+1)*((IW-1)*sx+1)*IC elements, each rounded up to 256 bytes) go to a static
+ * device array of TMI_NOALLOC_SCRATCH_BYTES instead of the context's growable buffer: the call performs no
+ * hipMalloc / hipFree and returns TMI_ERROR, launching nothing, when the operands need more than that.  All
+ * contexts on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ * contexts) race; calls on one stream are ordered and each call rewrites every byte it later reads. */
+int tmi_transpose_conv2d_noalloc(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                                 const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
+
 /* OpConv3d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:935-1120 (checks :901-933, :120-226).
  * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side.  INT8 with 3x3 taps in
  * the plane, KD*IC = 64 / 96 / 128 (IC 32 or 64) and w_zp 0 reads both operands in place; otherwise the gathered

@@ -35,9 +35,10 @@ EXPORTS = [
     "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
     "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
-    "tmi_ctx_reserve_workspace",
+    "tmi_ctx_reserve_workspace", "tmi_transpose_conv2d_noalloc",
 ]
 
+NOALLOC_SCRATCH_BYTES = 16 << 20  # TMI_NOALLOC_SCRATCH_BYTES
 
 
 class ConvDesc(ctypes.Structure):
@@ -128,6 +129,7 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_depthwise_conv2d_rescale_clamp.argtypes = fused
     tconv_args = [vp, ctypes.POINTER(TconvDesc), vp, vp, vp, i32, i32, vp]
     lib.tmi_transpose_conv2d.argtypes = tconv_args
+    lib.tmi_transpose_conv2d_noalloc.argtypes = tconv_args
     lib.tmi_conv3d.argtypes = [vp, ctypes.POINTER(Conv3dDesc), vp, vp, vp, i32, i32, vp]
     lib.tmi_matmul.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, i32, vp]
     lib.tmi_rescale.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i64, i32, vp, vp, vp, vp]
@@ -289,6 +291,10 @@ class Context:
     def transpose_conv2d(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
         return self._check(self.lib.tmi_transpose_conv2d(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
                                                          _ptr(bias), in_zp, w_zp, _ptr(out)))
+
+    def transpose_conv2d_noalloc(self, d: TconvDesc, inp, w, bias, in_zp, w_zp, out) -> int:
+        return self._check(self.lib.tmi_transpose_conv2d_noalloc(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
+                                                                 _ptr(bias), in_zp, w_zp, _ptr(out)))
 
     def reserve_workspace(self, nbytes: int) -> int:
         return self._check(self.lib.tmi_ctx_reserve_workspace(self.handle, nbytes))

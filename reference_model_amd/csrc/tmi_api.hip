@@ -4,10 +4,43 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
 #include "tmi_kernels.h"
+
+// Scratch memory of tmi_transpose_conv2d_noalloc, the one entry point that may not allocate: it lives in the
+// library's device image, so every GPU the library runs on holds its own copy (at its own address) from the
+// moment the code object is loaded until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the per-device address obtained from it at context creation is what kernels receive.
+static __device__ __align__(256) unsigned char scratch[TMI_NOALLOC_SCRATCH_BYTES];
+
+namespace
+{
+using tmi::kMaxDevices;
+std::mutex g_scratch_mutex;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};    // device address of `scratch` on each device, once known
+
+// Looks up this device's copy of `scratch` (the device must be current).  No allocation happens here: the
+// array is part of the loaded code object.
+hipError_t scratch_address(int device, unsigned char** out)
+{
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device])
+    {
+        unsigned char* p = nullptr;
+        hipError_t e     = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess)
+            return e;
+        if (!p)
+            return hipErrorInvalidSymbol;
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return hipSuccess;
+}
+}    // namespace
 
 struct tmi_ctx
 {
@@ -20,6 +53,7 @@ struct tmi_ctx
     void* workspace       = nullptr;    // scratch for operand re-layout (MATMUL's transposed B)
     size_t workspace_size = 0;
     std::vector<void*> retired;         // outgrown scratch blocks: captured graphs may still name them
+    unsigned char* static_scratch = nullptr;    // this device's copy of the library's static scratch array
     uint32_t last_flags   = 0;
     int32_t kernel_choice = 0;
     std::string last_error;
@@ -379,7 +413,7 @@ int tmi_ctx_create(tmi_ctx_t** out_ctx, int device)
         return TMI_ERROR;
     *out_ctx = nullptr;
     int count = 0;
-    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count)
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count || device >= kMaxDevices)
         return TMI_ERROR;
     tmi_ctx* ctx = new tmi_ctx();
     ctx->device  = device;
@@ -389,6 +423,11 @@ int tmi_ctx_create(tmi_ctx_t** out_ctx, int device)
         return TMI_ERROR;
     }
     ctx->owns_stream = true;
+    if (scratch_address(device, &ctx->static_scratch) != hipSuccess)
+    {
+        tmi_ctx_destroy(ctx);
+        return TMI_ERROR;
+    }
     if (hipMalloc((void**)&ctx->flags_dev, 256) != hipSuccess ||
         hipHostMalloc((void**)&ctx->flags_host, 256, hipHostMallocDefault) != hipSuccess ||
         hipMemset(ctx->flags_dev, 0, 256) != hipSuccess)
@@ -615,11 +654,11 @@ int tmi_transpose_conv2d_check(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d)
     return validate_tconv(ctx, "OpTransposeConv2d", d, 0, 0);
 }
 
-int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
-                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+// TRANSPOSE_CONV2D on either scratch memory: the context's buffer, grown on demand (static_only = false), or the
+// library's static array, which is never grown (static_only = true: nothing on this path allocates or frees).
+static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_desc_t* d, const void* in_dev,
+                                const void* weight_dev, const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
 {
-    if (!ctx)
-        return TMI_ERROR;
     const char* op = "OpTransposeConv2d";
     int rc = validate_tconv(ctx, op, d, in_zp, w_zp);
     if (rc != TMI_VALID)
@@ -664,10 +703,22 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
     }
     const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * row_bytes);
     const size_t u_bytes = holes ? align256((size_t)d->N * UH * UW * row_bytes) : 0;
-    rc                   = ensure_workspace(ctx, w_bytes + u_bytes);
-    if (rc != TMI_VALID)
-        return rc;
-    uint8_t* w_flip = (uint8_t*)ctx->workspace;
+    uint8_t* w_flip = nullptr;
+    if (static_only)
+    {
+        if (w_bytes + u_bytes > (size_t)TMI_NOALLOC_SCRATCH_BYTES)
+            return fail(ctx, "%s: the re-laid-out operands need %zu bytes of scratch memory, more than the %zu bytes "
+                             "of the static scratch array (TMI_NOALLOC_SCRATCH_BYTES)", op, w_bytes + u_bytes,
+                        (size_t)TMI_NOALLOC_SCRATCH_BYTES);
+        w_flip = ctx->static_scratch;
+    }
+    else
+    {
+        rc = ensure_workspace(ctx, w_bytes + u_bytes);
+        if (rc != TMI_VALID)
+            return rc;
+        w_flip = (uint8_t*)ctx->workspace;
+    }
     uint8_t* u      = w_flip + w_bytes;
     if (!(holes ? launch_tconv_operands(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip, d->N, d->IH, d->IW,
                                         d->stride[0], d->stride[1], in_zp, in_dev, u)
@@ -675,6 +726,22 @@ int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* 
         return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
                     d->out_dtype, out_dev);
+}
+
+int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                         const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_transpose_conv2d(ctx, false, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, out_dev);
+}
+
+int tmi_transpose_conv2d_noalloc(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
+                                 const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    return run_transpose_conv2d(ctx, true, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, out_dev);
 }
 
 // OpConv3d::checkTensorAttributes and the head of eval() (tensor_ops.cpp:901-933, :120-226, :963-970, :1024-1033)
