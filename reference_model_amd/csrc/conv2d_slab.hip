@@ -237,8 +237,12 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             const int uni   = folds && __all(cs.s == s_first);
             tab_cs[lane]    = cs;
             tab_hw[lane]    = make_high_word_scale(cs, a.rp.out_zp);
+            // With double rounding, a value below zero takes a rounding term 2^31 smaller; when the result is clamped at
+            // or above output_zp anyway, a negative value ends at the lower limit with either term (the scaled value is at
+            // most 0 for a multiplier >= 0), so that form skips the sign test (bit 8).
+            const int relu = a.rp.double_round && a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
             if (lane == 0)
-                *uni_shift = uni ? s_first : (folds ? -2 : -1);
+                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? -2 : -1);
         }
         tab_m[lane] = m;
         tab_b[lane] = ok ? b : 0;
@@ -344,7 +348,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     else
     {
         int32_t r[16];
-        const int s_uni = __builtin_amdgcn_readfirstlane(*uni_shift);
+        const int form  = __builtin_amdgcn_readfirstlane(*uni_shift);
+        const int s_uni = form >= 0 ? (form & 255) : form;
+        const int relu  = form >= 0 ? (form >> 8) : 0;
         if (s_uni >= 0)
         {
             // one shift for every channel: the high-word form with its constants in scalar registers
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 const v4i m4 = *reinterpret_cast<const v4i*>(tab_m + ocl + 4 * q);
                 cm[4 * q] = m4[0], cm[4 * q + 1] = m4[1], cm[4 * q + 2] = m4[2], cm[4 * q + 3] = m4[3];
             }
-            if (a.rp.double_round)
+            if (a.rp.double_round && !relu)
             {
 #pragma unroll
                 for (int e = 0; e < 16; e++)
