@@ -73,8 +73,16 @@ enum
     TMI_FLAG_SCALE_SHIFT      = 1u << 1, /* shift outside [2,62]                quant_util.h:53-58  */
     TMI_FLAG_SCALE_VALUE      = 1u << 2, /* value outside [-2^(s-1), 2^(s-1))   quant_util.h:59-67  */
     TMI_FLAG_SCALE_RESULT     = 1u << 3, /* scaled result exceeds int32         quant_util.h:78-82  */
-    TMI_FLAG_ZP_RESULT        = 1u << 4  /* result + output_zp exceeds int32    type_conversion.cpp:352-360 */
+    TMI_FLAG_ZP_RESULT        = 1u << 4, /* result + output_zp exceeds int32    type_conversion.cpp:352-360 */
+    TMI_FLAG_LEVEL            = 1u << 5  /* a LEVEL_CHECK of the configured level failed (found on the host)  */
 };
+
+/* tosa_level_t of the reference (reference_model/include/func_config.h:23-36); all zero = no level
+ * (func_config_t::NONE), { 6, 8192, 8192, 256, 64 } = EIGHTK (:65). */
+typedef struct
+{
+    int32_t max_rank, max_kernel, max_stride, max_scale, max_tensor_list_size;
+} tmi_level_t;
 
 typedef struct tmi_ctx tmi_ctx_t;
 
@@ -95,6 +103,15 @@ int tmi_ctx_set_stream(tmi_ctx_t* ctx, void* hip_stream);
  * Counterpart of reading SubgraphTraverser::getGraphStatus() after evaluateAll()
  * (reference_model/src/model_runner_impl.cpp:56-126). */
 int tmi_ctx_sync(tmi_ctx_t* ctx);
+
+/* g_func_config.tosa_level (--tosa_level, reference_model/src/command_line_utils.h:62).  With a level set, every
+ * operator call evaluates the reference's LEVEL_CHECKs for it (e.g. reference_model/src/ops/tensor_ops.cpp:761-771 for
+ * CONV2D: dilation * kernel and pads against MAX_KERNEL, strides against MAX_STRIDE; RESCALE: rank against MAX_RANK).
+ * As in the reference (include/func_debug.h:132-141) a violated limit does not stop evaluation: the operator runs,
+ * TMI_FLAG_LEVEL is latched, the next tmi_ctx_sync() returns TMI_UNPREDICTABLE and tmi_last_error() names the limit.
+ * NULL or an all-zero level switches the checks off.  tmi_clamp takes no rank, so CLAMP's rank check
+ * (activation_funcs.cpp:32) stays with the caller. */
+int tmi_ctx_set_level(tmi_ctx_t* ctx, const tmi_level_t* level);
 
 /* Flag bits (TMI_FLAG_*) seen by the most recent tmi_ctx_sync(). */
 uint32_t tmi_ctx_flags(const tmi_ctx_t* ctx);
@@ -137,6 +154,9 @@ typedef struct
     int32_t stride[2];   /* y, x */
     int32_t dilation[2]; /* y, x */
     int32_t bias_len;    /* 1 (broadcast) or OC */
+    int32_t acc_dtype;   /* the attribute's acc_type: TMI_INT32 for INT8 operands, TMI_FP32 for floating point (the
+                            reference also instantiates FP16 accumulation of FP16 operands, op_factory.h:97-118, which
+                            is not built: TMI_ERROR) */
 } tmi_conv_desc_t;
 
 /* TransposeConv2dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:1982-2056).
@@ -151,6 +171,7 @@ typedef struct
     int32_t out_pad[4];  /* top, bottom, left, right; each > -kernel size */
     int32_t stride[2];   /* y, x */
     int32_t bias_len;    /* 1 (broadcast) or OC */
+    int32_t acc_dtype;   /* as in tmi_conv_desc_t */
 } tmi_tconv_desc_t;
 
 /* Conv3dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:901-933, check :120-226).
@@ -165,6 +186,7 @@ typedef struct
     int32_t stride[3];   /* d, y, x */
     int32_t dilation[3]; /* d, y, x */
     int32_t bias_len;
+    int32_t acc_dtype;   /* as in tmi_conv_desc_t */
 } tmi_conv3d_desc_t;
 
 /* AvgPool2dAttribute / MaxPool2dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:29-117
@@ -228,6 +250,12 @@ int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64
 int tmi_clamp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, int32_t min_val, int32_t max_val,
               void* out_dev);
 
+/* OpClamp::eval for FP16 / BF16 / FP32 (reference_model/src/ops/activation_funcs.cpp:97-106): applyClip with the
+ * attribute's nan_mode (1 = PROPAGATE, 2 = IGNORE; reference_model/src/arith_util.h:341-413), then the rounding to the
+ * stored type.  TMI_ERROR when max_val < min_val or either is NaN. */
+int tmi_clamp_fp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, float min_val, float max_val,
+                 int32_t nan_mode, void* out_dev);
+
 /* CONV2D -> RESCALE (-> CLAMP) evaluated as one kernel: the int32 convolution result never reaches HBM.
  * Same results as tmi_conv2d + tmi_rescale (+ tmi_clamp) on the same operands.  The rescale input is the
  * INT32 convolution output (r->in_dtype must be TMI_INT32, r->in_zp 0); per-channel constants have OC
@@ -290,11 +318,16 @@ int tmi_max_pool2d(tmi_ctx_t* ctx, const tmi_pool_desc_t* d, const void* in_dev,
  * of op_factory.cpp) and in bounds mode (the same sums over absolute values, tensor_ops.cpp:757-765,
  * 1213-1221, 1436-1443).  These entries compute either pass on the device: operands in their storage type
  * (TMI_FP16 / TMI_BF16 / TMI_FP32), fp64 products and sums in the reference's loop order, fp64 output of the operator's
- * output shape.  bounds_mode != 0 selects the sums of absolute values. */
+ * output shape.  bounds_mode != 0 selects the sums of absolute values.  local_bound is the operator's attribute of
+ * that name (Conv2dAttribute / DepthwiseConv2dAttribute): when it is 0, the bounds pass replaces every input element
+ * by the largest magnitude of the whole input tensor (reference_model/src/ops/tensor_ops.cpp:797-801, 1252-1256), which
+ * is the flatbuffer default; it has no effect on the precise pass.  MATMUL has no such attribute
+ * (tensor_ops.cpp:1436-1441 takes absolute values only). */
 int tmi_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
-                       const void* bias_dev, int32_t bounds_mode, double* out_dev);
+                       const void* bias_dev, int32_t bounds_mode, int32_t local_bound, double* out_dev);
 int tmi_depthwise_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev,
-                                 const void* weight_dev, const void* bias_dev, int32_t bounds_mode, double* out_dev);
+                                 const void* weight_dev, const void* bias_dev, int32_t bounds_mode, int32_t local_bound,
+                                 double* out_dev);
 int tmi_matmul_precise(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
                        const void* a_dev, const void* b_dev, int32_t bounds_mode, double* out_dev);
 
@@ -351,6 +384,19 @@ int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank,
  * and 4 return TMI_ERROR if the shape is not eligible.  Used by the parity tests to check every kernel on the
  * same operands. */
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
+
+/* Launches a kernel that does nothing - grid workgroups of block threads with lds_bytes of dynamic LDS - on
+ * the context's stream: what one launch of that shape costs before any work.  No counterpart in the
+ * reference; used by the benchmark's launch-floor configuration. */
+int tmi_debug_launch_empty(tmi_ctx_t* ctx, int32_t grid, int32_t block, int32_t lds_bytes);
+
+/* Host arithmetic only, no GPU call.  The tiled kernels split a block index into (channel block, tile column,
+ * tile row, image) with multiply-high divisions that are exact while dividend * divisor < 2^32; a launcher
+ * whose layer is outside that leaves the layer to another kernel.  Returns 1 if a grid of `grid` blocks with
+ * these divisors passes that guard, else 0, and writes the decode of `block` by the same arithmetic to out4
+ * (if not NULL).  Used by the unit tests of the guard. */
+int tmi_debug_tile_decode(int64_t grid, uint32_t n_ocb, uint32_t tiles_x, uint32_t tiles_y, uint32_t block,
+                          int32_t* out4);
 
 /* Library build identification, e.g. "tosa_mi355 gfx950". */
 const char* tmi_version(void);

@@ -15,6 +15,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libtosa_oracle.so")
+_LIB_OMP_PATH = os.path.join(_HERE, "libtosa_oracle_omp.so")   # the same source built with -fopenmp (all host cores)
 
 VALID, UNPREDICTABLE, ERROR = 0, 1, 2
 ROUND_SINGLE, ROUND_INEXACT, ROUND_DOUBLE = 1, 2, 3
@@ -44,22 +45,31 @@ class RescaleAttr(ctypes.Structure):
         "input_unsigned", "output_unsigned", "in_zp", "out_zp")]
 
 
-_lib = None
+_libs = {}
+_parallel = False
+
+
+def set_parallel(on: bool) -> None:
+    """Selects the OpenMP build (CONV2D / DEPTHWISE_CONV2D / MATMUL loops over all host cores) for the calls that
+    follow; the scalar build, which is the reference-equivalent single-threaded path, is the default."""
+    global _parallel
+    _parallel = bool(on)
 
 
 def lib() -> ctypes.CDLL:
-    global _lib
-    if _lib is None:
-        if not os.path.exists(_LIB_PATH):
+    path = _LIB_OMP_PATH if _parallel else _LIB_PATH
+    if path not in _libs:
+        if not os.path.exists(path):
             build()
-        _lib = ctypes.CDLL(_LIB_PATH)
-        _lib.orc_apply_scale_32.restype = ctypes.c_int32
-        _lib.orc_apply_scale_32.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int,
-                                            ctypes.POINTER(ctypes.c_int)]
-        _lib.orc_apply_scale_16.restype = ctypes.c_int32
-        _lib.orc_apply_scale_16.argtypes = [ctypes.c_int64, ctypes.c_int16, ctypes.c_int32,
-                                            ctypes.POINTER(ctypes.c_int)]
-    return _lib
+        L = ctypes.CDLL(path)
+        L.orc_apply_scale_32.restype = ctypes.c_int32
+        L.orc_apply_scale_32.argtypes = [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int,
+                                         ctypes.POINTER(ctypes.c_int)]
+        L.orc_apply_scale_16.restype = ctypes.c_int32
+        L.orc_apply_scale_16.argtypes = [ctypes.c_int64, ctypes.c_int16, ctypes.c_int32,
+                                         ctypes.POINTER(ctypes.c_int)]
+        _libs[path] = L
+    return _libs[path]
 
 
 def _ptr(a: np.ndarray):
@@ -114,8 +124,14 @@ _KINDS = {
 }
 
 
+def _abs_code(abs_mode, local_bound):
+    """0: ordinary pass; 1: bounds pass (absolute values); 2: bounds pass of an operator whose local_bound attribute
+    is false: the input is replaced by its largest magnitude (tensor_ops.cpp:797-801, 1252-1256)."""
+    return 0 if not abs_mode else (1 if local_bound else 2)
+
+
 def conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0,
-           abs_mode=False, out_hw=None):
+           abs_mode=False, out_hw=None, local_bound=True):
     """CONV2D.  inp NHWC, w OHWI, bias [1] or [OC].  kind in i8/i32/f32/f64."""
     et, bt, ot = _KINDS[kind]
     inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
@@ -132,14 +148,14 @@ def conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1),
     elif kind == "f32":
         rc = L.orc_conv2d_f32(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), _ptr(out))
     else:
-        rc = L.orc_conv2d_f64(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int(int(abs_mode)),
-                              _ptr(out))
+        rc = L.orc_conv2d_f64(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias),
+                              ctypes.c_int(_abs_code(abs_mode, local_bound)), _ptr(out))
     _check(rc)
     return out
 
 
 def depthwise_conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0,
-                     abs_mode=False, out_hw=None):
+                     abs_mode=False, out_hw=None, local_bound=True):
     """DEPTHWISE_CONV2D.  inp NHWC, w [KH,KW,C,M], bias [1] or [C*M]."""
     et, bt, ot = _KINDS[kind]
     inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
@@ -157,7 +173,7 @@ def depthwise_conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilati
         rc = L.orc_depthwise_f32(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias), _ptr(out))
     else:
         rc = L.orc_depthwise_f64(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias),
-                                 ctypes.c_int(int(abs_mode)), _ptr(out))
+                                 ctypes.c_int(_abs_code(abs_mode, local_bound)), _ptr(out))
     _check(rc)
     return out
 

@@ -51,6 +51,8 @@ int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m)
     static int NAME(const orc_conv_shape_t* s, const T* in, const T* w, const T* bias, T in_zp, T w_zp,          \
                     int abs_mode, T* out)                                                                          \
     {                                                                                                              \
+        /* abs_mode 1: bounds mode; 2: bounds mode of an operator without local_bound, whose input is replaced by   \
+           its largest magnitude (tensor_ops.cpp:797-801) */                                                       \
         if (orc_conv_check(s, 0) != ORC_VALID)                                                                     \
             return ORC_ERROR;                                                                                      \
         const int N = s->N, IH = s->IH, IW = s->IW, IC = s->IC, OC = s->OC, KH = s->KH, KW = s->KW;                \
@@ -69,6 +71,11 @@ int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m)
         }                                                                                                          \
         for (size_t i = 0; i < n_w; i++)                                                                           \
             wv[i] = abs_mode ? ABS_EXPR(w[i]) : w[i];                                                              \
+        T in_abs_max = 0;                                                                                          \
+        if (abs_mode == 2)                                                                                         \
+            for (size_t i = 0; i < (size_t)N * IH * IW * IC; i++)                                                  \
+                if (ABS_EXPR(in[i]) > in_abs_max)                                                                  \
+                    in_abs_max = ABS_EXPR(in[i]);                                                                  \
         for (int n = 0; n < N; n++)                                                                                \
             for (int y = 0; y < PH; y++)                                                                           \
                 for (int x = 0; x < PW; x++)                                                                       \
@@ -80,10 +87,11 @@ int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m)
                         {                                                                                          \
                             v = in[(((size_t)n * IH + iy) * IW + ix) * IC + c];                                    \
                             if (abs_mode)                                                                          \
-                                v = ABS_EXPR(v);                                                                   \
+                                v = abs_mode == 2 ? in_abs_max : ABS_EXPR(v);                                      \
                         }                                                                                          \
                         padded[(((size_t)n * PH + y) * PW + x) * IC + c] = v;                                      \
                     }                                                                                              \
+        _Pragma("omp parallel for collapse(2) schedule(static)")                                                   \
         for (int ob = 0; ob < N; ob++)                                                                             \
             for (int oy = 0; oy < OH; oy++)                                                                        \
                 for (int ox = 0; ox < OW; ox++)                                                                    \
@@ -376,6 +384,13 @@ int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const 
         const int OH = s->OH, OW = s->OW;                                                                          \
         const int pt = s->pad[0], pl = s->pad[2];                                                                  \
         const int sy = s->stride[0], sx = s->stride[1], dy = s->dilation[0], dx = s->dilation[1];                  \
+        /* abs_mode 2: bounds mode without local_bound (tensor_ops.cpp:1252-1256) */                               \
+        T in_abs_max = 0;                                                                                          \
+        if (abs_mode == 2)                                                                                         \
+            for (size_t i = 0; i < (size_t)N * IH * IW * IC; i++)                                                  \
+                if (ABS_EXPR(in[i]) > in_abs_max)                                                                  \
+                    in_abs_max = ABS_EXPR(in[i]);                                                                  \
+        _Pragma("omp parallel for collapse(2) schedule(static)")                                                   \
         for (int ob = 0; ob < N; ob++)                                                                             \
             for (int oy = 0; oy < OH; oy++)                                                                        \
                 for (int ox = 0; ox < OW; ox++)                                                                    \
@@ -395,7 +410,7 @@ int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const 
                                     T b = w[(((size_t)ky * KW + kx) * IC + ic) * M + km];                          \
                                     if (abs_mode)                                                                  \
                                     {                                                                              \
-                                        a = ABS_EXPR(a);                                                           \
+                                        a = abs_mode == 2 ? in_abs_max : ABS_EXPR(a);                              \
                                         b = ABS_EXPR(b);                                                           \
                                     }                                                                              \
                                     acc += (a - in_zp) * (b - w_zp);                                               \
@@ -455,12 +470,18 @@ int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, co
     {                                                                                                              \
         if (N < 0 || H < 0 || C < 0 || W < 0)                                                                      \
             return ORC_ERROR;                                                                                      \
+        int failed = 0;                                                                                            \
+        _Pragma("omp parallel")                                                                                    \
+        {                                                                                                          \
         T* row = (T*)malloc(sizeof(T) * (size_t)(W > 0 ? W : 1));                                                  \
         if (!row)                                                                                                  \
-            return ORC_ERROR;                                                                                      \
+            failed = 1;                                                                                            \
+        _Pragma("omp for collapse(2) schedule(static)")                                                            \
         for (int n = 0; n < N; n++)                                                                                \
             for (int h = 0; h < H; h++)                                                                            \
             {                                                                                                      \
+                if (!row)                                                                                          \
+                    continue;                                                                                      \
                 for (int x = 0; x < W; x++)                                                                        \
                     row[x] = 0;                                                                                    \
                 for (int c = 0; c < C; c++)                                                                        \
@@ -481,7 +502,8 @@ int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, co
                 memcpy(out + ((size_t)n * H + h) * W, row, sizeof(T) * (size_t)W);                                 \
             }                                                                                                      \
         free(row);                                                                                                 \
-        return ORC_VALID;                                                                                          \
+        }                                                                                                          \
+        return failed ? ORC_ERROR : ORC_VALID;                                                                     \
     }
 
 ORC_DEFINE_MATMUL(matmul_i32_impl, int32_t, ORC_ABS_I32)

@@ -35,7 +35,8 @@ EXPORTS = [
     "tmi_transpose_conv2d", "tmi_conv3d", "tmi_transpose_conv2d_check", "tmi_conv3d_check",
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
     "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
-    "tmi_ctx_reserve_workspace", "tmi_transpose_conv2d_noalloc",
+    "tmi_ctx_reserve_workspace", "tmi_transpose_conv2d_noalloc", "tmi_ctx_set_level", "tmi_clamp_fp",
+    "tmi_debug_launch_empty", "tmi_debug_tile_decode",
 ]
 
 NOALLOC_SCRATCH_BYTES = 16 << 20  # TMI_NOALLOC_SCRATCH_BYTES
@@ -48,27 +49,49 @@ class ConvDesc(ctypes.Structure):
         ("OC", ctypes.c_int32), ("KH", ctypes.c_int32), ("KW", ctypes.c_int32),
         ("OH", ctypes.c_int32), ("OW", ctypes.c_int32),
         ("pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("dilation", ctypes.c_int32 * 2),
-        ("bias_len", ctypes.c_int32),
+        ("bias_len", ctypes.c_int32), ("acc_dtype", ctypes.c_int32),
     ]
 
 
 class TconvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("in_dtype", "out_dtype", "N", "IH", "IW", "IC", "OC", "KH", "KW", "OH",
                                               "OW")] + [
-        ("out_pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("bias_len", ctypes.c_int32)]
+        ("out_pad", ctypes.c_int32 * 4), ("stride", ctypes.c_int32 * 2), ("bias_len", ctypes.c_int32),
+        ("acc_dtype", ctypes.c_int32)]
+
+    def __setattr__(self, name, value):
+        # the accumulator type follows the operand type unless it is set explicitly afterwards
+        super().__setattr__(name, value)
+        if name == "in_dtype":
+            super().__setattr__("acc_dtype", INT32 if value == INT8 else FP32)
 
 
 class Conv3dDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("in_dtype", "out_dtype", "N", "ID", "IH", "IW", "IC", "OC", "KD", "KH",
                                               "KW", "OD", "OH", "OW")] + [
         ("pad", ctypes.c_int32 * 6), ("stride", ctypes.c_int32 * 3), ("dilation", ctypes.c_int32 * 3),
-        ("bias_len", ctypes.c_int32)]
+        ("bias_len", ctypes.c_int32), ("acc_dtype", ctypes.c_int32)]
+
+    def __setattr__(self, name, value):
+        super().__setattr__(name, value)
+        if name == "in_dtype":
+            super().__setattr__("acc_dtype", INT32 if value == INT8 else FP32)
 
 
 class PoolDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("dtype", "acc_dtype", "N", "IH", "IW", "C", "OH", "OW")] + [
         ("kernel", ctypes.c_int32 * 2), ("stride", ctypes.c_int32 * 2), ("pad", ctypes.c_int32 * 4),
         ("nan_mode", ctypes.c_int32)]
+
+
+class Level(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("max_rank", "max_kernel", "max_stride", "max_scale",
+                                              "max_tensor_list_size")]
+
+
+LEVEL_NONE = (0, 0, 0, 0, 0)
+LEVEL_EIGHTK = (6, 8192, 8192, 256, 64)
+FLAG_LEVEL = 32
 
 
 class DpResult(ctypes.Structure):
@@ -134,11 +157,16 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_matmul.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, i32, vp]
     lib.tmi_rescale.argtypes = [vp, ctypes.POINTER(RescaleDesc), i32, i64, i32, vp, vp, vp, vp]
     lib.tmi_clamp.argtypes = [vp, i32, i64, vp, i32, i32, vp]
+    lib.tmi_clamp_fp.argtypes = [vp, i32, i64, vp, ctypes.c_float, ctypes.c_float, i32, vp]
+    lib.tmi_ctx_set_level.argtypes = [vp, ctypes.POINTER(Level)]
+    lib.tmi_debug_launch_empty.argtypes = [vp, i32, i32, i32]
+    lib.tmi_debug_tile_decode.argtypes = [i64, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+                                          ctypes.POINTER(ctypes.c_int32)]
     lib.tmi_avg_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, i32, i32, vp]
     lib.tmi_max_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, vp]
     lib.tmi_pool2d_check.argtypes = [vp, ctypes.POINTER(PoolDesc), i32]
-    lib.tmi_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, vp]
-    lib.tmi_depthwise_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, vp]
+    lib.tmi_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, i32, vp]
+    lib.tmi_depthwise_conv2d_precise.argtypes = [vp, ctypes.POINTER(ConvDesc), vp, vp, vp, i32, i32, vp]
     lib.tmi_matmul_precise.argtypes = [vp, i32, i32, i32, i32, i32, vp, vp, i32, vp]
     lib.tmi_dot_product_check.argtypes = [vp, i32, i64, vp, vp, vp, i32, i32, ctypes.POINTER(DpResult)]
     lib.tmi_conv2d_check.argtypes = [vp, ctypes.POINTER(ConvDesc), i32]
@@ -259,8 +287,10 @@ class Context:
 
     # -- descriptors ---------------------------------------------------------------------------
     @staticmethod
-    def conv_desc(in_dtype, out_dtype, in_shape, oc, kh, kw, out_hw, pad, stride, dilation, bias_len) -> ConvDesc:
+    def conv_desc(in_dtype, out_dtype, in_shape, oc, kh, kw, out_hw, pad, stride, dilation, bias_len,
+                  acc_dtype=None) -> ConvDesc:
         d = ConvDesc()
+        d.acc_dtype = acc_dtype if acc_dtype is not None else (INT32 if in_dtype == INT8 else FP32)
         d.in_dtype, d.out_dtype = in_dtype, out_dtype
         d.N, d.IH, d.IW, d.IC = in_shape
         d.OC, d.KH, d.KW = oc, kh, kw
@@ -299,9 +329,10 @@ class Context:
     def reserve_workspace(self, nbytes: int) -> int:
         return self._check(self.lib.tmi_ctx_reserve_workspace(self.handle, nbytes))
 
-    def conv2d_precise(self, d: ConvDesc, inp, w, bias, bounds_mode, out, depthwise=False) -> int:
+    def conv2d_precise(self, d: ConvDesc, inp, w, bias, bounds_mode, out, depthwise=False, local_bound=True) -> int:
         fn = self.lib.tmi_depthwise_conv2d_precise if depthwise else self.lib.tmi_conv2d_precise
-        return self._check(fn(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias), int(bounds_mode), _ptr(out)))
+        return self._check(fn(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w), _ptr(bias), int(bounds_mode),
+                              int(local_bound), _ptr(out)))
 
     def matmul_precise(self, in_dtype, n, h, c, w, a, b, bounds_mode, out) -> int:
         return self._check(self.lib.tmi_matmul_precise(self.handle, in_dtype, n, h, c, w, _ptr(a), _ptr(b),
@@ -351,6 +382,17 @@ class Context:
 
     def clamp(self, dtype, n, inp, lo, hi, out) -> int:
         return self._check(self.lib.tmi_clamp(self.handle, dtype, n, _ptr(inp), lo, hi, _ptr(out)))
+
+    def clamp_fp(self, dtype, n, inp, lo, hi, nan_mode, out) -> int:
+        return self._check(self.lib.tmi_clamp_fp(self.handle, dtype, n, _ptr(inp), float(lo), float(hi), int(nan_mode),
+                                                 _ptr(out)))
+
+    def launch_empty(self, grid, block, lds_bytes) -> int:
+        return self._check(self.lib.tmi_debug_launch_empty(self.handle, grid, block, lds_bytes))
+
+    def set_level(self, level=LEVEL_NONE):
+        lv = Level(*level)
+        self._check(self.lib.tmi_ctx_set_level(self.handle, ctypes.byref(lv)))
 
 
 def _stored(zp: int, dtype: int) -> int:

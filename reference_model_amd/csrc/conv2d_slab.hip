@@ -544,7 +544,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     a.bias_len = g.bias_len, a.za = in_zp, a.n_ocb = n_ocb;
     a.out_kind = !rp.enabled ? 0 : (out_dtype == TMI_INT8 ? 1 : 2);
     const int64_t grid = (int64_t)g.N * a.tiles_y * a.tiles_x * n_ocb;
-    if (grid >= (int64_t(1) << 31))
+    if (!tile_decode_is_exact(grid, (uint32_t)n_ocb, (uint32_t)a.tiles_x, (uint32_t)a.tiles_y))
         return nullptr;
     a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? 1 : 0;
     // A patch pixel is R = CH + 1 chunks; the chunk of output pixel (ty, tx) under tap (0, 0) is ty * sy * pitch + R * sx * tx.
@@ -572,6 +572,8 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     {
         a.ID = c3d->ID, a.OD = c3d->OD, a.sd = c3d->stride_d, a.dd = c3d->dilation_d, a.pd0 = c3d->pad_d0;
         a.div_od = make_fastdiv((uint32_t)c3d->OD);
+        if (!fastdiv_exact_up_to((uint64_t)g.N - 1, (uint32_t)c3d->OD))    // image index = volume * OD + output slice
+            return nullptr;
         const bool za = a.za != 0;
         if (ch == 4)
             ok = za ? launch_slab_kernel<3, 3, 4, true, false, false, 2>(st, a, (int)grid, lds_bytes)
@@ -591,6 +593,9 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     {
         a.up_y = tc->up_y, a.up_x = tc->up_x, a.IHr = tc->IH, a.IWr = tc->IW;
         a.div_up_y = make_fastdiv((uint32_t)tc->up_y), a.div_up_x = make_fastdiv((uint32_t)tc->up_x);
+        // the divided coordinates are rows and columns of the input with its holes (g.IH x g.IW)
+        if (!fastdiv_exact_up_to((uint64_t)g.IH, (uint32_t)tc->up_y) || !fastdiv_exact_up_to((uint64_t)g.IW, (uint32_t)tc->up_x))
+            return nullptr;
         if (a.za != 0)
             ok = ch == 4 ? launch_slab_kernel<3, 3, 4, true, false, true>(st, a, (int)grid, lds_bytes)
                          : (ch == 6 ? launch_slab_kernel<3, 3, 6, true, false, true>(st, a, (int)grid, lds_bytes)

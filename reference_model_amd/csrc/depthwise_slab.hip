@@ -474,7 +474,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     a.step_row = per_round / a.pitch;
     a.step_px = (per_round % a.pitch) / ppitch, a.step_ch = (per_round % a.pitch) % ppitch;
     const int64_t grid = (int64_t)g.N * a.tiles_y * a.tiles_x;
-    if (grid >= (int64_t(1) << 31))
+    if (!tile_decode_is_exact(grid, 1u, (uint32_t)a.tiles_x, (uint32_t)a.tiles_y))
         return nullptr;
     a.xcd_remap = grid % 8 == 0 ? 1 : 0;
     a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pitch = make_fastdiv((uint32_t)a.pitch);

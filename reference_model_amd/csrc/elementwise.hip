@@ -272,6 +272,99 @@ const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* ou
 }
 
 // ------------------------------------------------------------------------------------------------
+// CLAMP on FP16 / BF16 / FP32 (activation_funcs.cpp:97-106): applyMax(x, min) then applyMin(., max) of
+// arith_util.h:341-413 with the attribute's NaN mode (1 = PROPAGATE: a NaN stays a NaN; 2 = IGNORE: the NaN operand is
+// dropped, so a NaN input ends at min), evaluated in float and rounded back to the stored type (fpTrunc).
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float clampf_load(const T* p, int64_t i);
+template <>
+__device__ __forceinline__ float clampf_load<float>(const float* p, int64_t i)
+{
+    return p[i];
+}
+template <>
+__device__ __forceinline__ float clampf_load<_Float16>(const _Float16* p, int64_t i)
+{
+    return (float)p[i];
+}
+template <>
+__device__ __forceinline__ float clampf_load<bf16_t>(const bf16_t* p, int64_t i)
+{
+    return bf16_to_float(p[i]);
+}
+__device__ __forceinline__ void clampf_store(float* p, int64_t i, float v)
+{
+    p[i] = v;
+}
+__device__ __forceinline__ void clampf_store(_Float16* p, int64_t i, float v)
+{
+    p[i] = (_Float16)v;
+}
+__device__ __forceinline__ void clampf_store(bf16_t* p, int64_t i, float v)
+{
+    p[i] = float_to_bf16(v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void clamp_fp_kernel(const T* __restrict__ in, T* __restrict__ out, int64_t n, float lo,
+                                                       float hi, int nan_mode)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    {
+        float v = clampf_load<T>(in, i);
+        if (v != v)
+            v = nan_mode == 1 ? v : lo;
+        else
+        {
+            v = v >= lo ? v : lo;
+            v = v < hi ? v : hi;
+        }
+        clampf_store(out, i, v);
+    }
+}
+
+const char* launch_clamp_fp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, float lo, float hi,
+                            int32_t nan_mode)
+{
+    if (n == 0)
+        return "clamp_empty";
+    const dim3 grid(grid_for(n)), block(256);
+    if (dtype == TMI_FP32)
+        hipLaunchKernelGGL(clamp_fp_kernel<float>, grid, block, 0, st, (const float*)in, (float*)out, n, lo, hi, nan_mode);
+    else if (dtype == TMI_FP16)
+        hipLaunchKernelGGL(clamp_fp_kernel<_Float16>, grid, block, 0, st, (const _Float16*)in, (_Float16*)out, n, lo, hi,
+                           nan_mode);
+    else if (dtype == TMI_BF16)
+        hipLaunchKernelGGL(clamp_fp_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)in, (bf16_t*)out, n, lo, hi, nan_mode);
+    else
+        return nullptr;
+    return "clamp_fp";
+}
+
+// ------------------------------------------------------------------------------------------------
+// A kernel that does nothing, for measuring what one launch of a given grid, block and LDS size costs.
+// ------------------------------------------------------------------------------------------------
+__global__ void empty_kernel(int32_t touch)
+{
+    extern __shared__ unsigned char empty_lds[];
+    if (touch)    // never set: keeps the dynamic LDS allocation part of the kernel
+        empty_lds[threadIdx.x] = 0;
+}
+
+const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t lds_bytes)
+{
+    if (grid < 1 || block < 1 || block > 1024 || lds_bytes < 0 || lds_bytes > 160 * 1024)
+        return nullptr;
+    if (lds_bytes > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)empty_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+        return nullptr;
+    hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), lds_bytes, st, 0);
+    return "empty_kernel";
+}
+
+// ------------------------------------------------------------------------------------------------
 // Batched transpose [N, R, C] -> [N, C, R] through a padded 64x64 LDS tile: rows are read and written as
 // contiguous runs along the fastest dimension of their side.
 // ------------------------------------------------------------------------------------------------

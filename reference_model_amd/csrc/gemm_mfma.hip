@@ -655,7 +655,9 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
         const int64_t tn = (a.N + 64 * shapes[c][0] - 1) / (64 * shapes[c][0]);
         const int64_t tm = (a.M + 128 * shapes[c][1] - 1) / (128 * shapes[c][1]);
         const int64_t tiles = tn * tm * batches;
-        if (tiles > (1 << 22))
+        // the tile index is split by two FastDiv divisions, exact while dividend * divisor < 2^32
+        if (tiles > (1 << 22) || !fastdiv_exact_up_to((uint64_t)tiles - 1, (uint32_t)(tn * tm)) ||
+            !fastdiv_exact_up_to((uint64_t)(tn * tm) - 1, (uint32_t)tn))
             continue;
         const double passes = (double)((tiles + 255) / 256);
         const double cost   = passes * shapes[c][0] * shapes[c][1];

@@ -5,7 +5,7 @@
 // interprets (verif/runner/tosa_refmodel_sut_run.py:12-18,59-68).
 //
 //   tosa_mi355_run --test_desc=<dir>/desc.json [--ofm_file=<name>] [--flatbuffer_dir=<dir>] [--no_fusion]
-//                  [--precise_mode=1]
+//                  [--precise_mode=1] [--tosa_level=NONE|EIGHTK]
 //
 // --precise_mode=1 (reference_model/src/command_line_utils.h:65): floating-point CONV2D / DEPTHWISE_CONV2D /
 // MATMUL results are computed and written in fp64; when the descriptor says
@@ -142,6 +142,7 @@ int main(int argc, char** argv)
 {
     std::string test_desc, ofm_override, fb_dir;
     bool fusion = true, precise = false;
+    tmi_level_t level = { 0, 0, 0, 0, 0 };
     for (int a = 1; a < argc; a++)
     {
         const std::string s = argv[a];
@@ -159,6 +160,16 @@ int main(int argc, char** argv)
             fusion = false;
         else if (const char* v = val("--precise_mode="))
             precise = atoi(v) != 0;
+        else if (const char* v = val("--tosa_level="))
+        {
+            // command_line_utils.h:62, main.cpp: NONE or EIGHTK (func_config.h:65)
+            if (std::string(v) == "EIGHTK")
+                level = tmi_level_t{ 6, 8192, 8192, 256, 64 };
+            else if (std::string(v) == "NONE")
+                level = tmi_level_t{ 0, 0, 0, 0, 0 };
+            else
+                return fail("unknown TOSA level", v);
+        }
         else
             return fail("unknown argument", s);
     }
@@ -192,6 +203,7 @@ int main(int argc, char** argv)
         if (!fusion)
             runner.disableFusion();
         runner.setPreciseMode(precise, run == 1);
+        runner.setLevel(level);
         st = runner.initialize(block);
         if (st != GraphStatus::TOSA_VALID)
         {

@@ -208,7 +208,8 @@ public:
             d.pad[i] = attribute.pad[i];
         for (int i = 0; i < 2; i++)
             d.stride[i] = attribute.stride[i], d.dilation[i] = attribute.dilation[i];
-        d.bias_len = bias->shape[0];
+        d.bias_len  = bias->shape[0];
+        d.acc_dtype = tmi_dtype((DType)attribute.acc_type);
         return 0;
     }
 
@@ -222,10 +223,6 @@ public:
             return 1;
         if (inputs[1]->getDtype() != inputs[0]->getDtype())
             return error("weight data type not supported for this configuration of operator");
-        const DType in = inputs[0]->getDtype();
-        const uint32_t want_acc = in == DType_INT8 ? DType_INT32 : DType_FP32;
-        if (attribute.acc_type != want_acc)
-            return error("accumulator type %u not supported for this configuration of operator", attribute.acc_type);
         tmi_conv_desc_t d;
         if (fill_desc(d))
             return 1;
@@ -342,10 +339,78 @@ public:
             return error("OpClamp: input and output must have the same shape and type");
         return 0;
     }
+    // min_val / max_val of a floating-point CLAMP: bytes of the tensor's own type (activation_funcs.cpp:36-89)
+    int decode_fp(float& lo, float& hi)
+    {
+        const DType t   = inputs[0]->getDtype();
+        const size_t es = dtype_size(t);
+        if (attribute.min_val.size() < es || attribute.max_val.size() < es)
+            return error("OpClamp: malformed min/max attribute");
+        auto one = [&](const std::vector<uint8_t>& b) -> float {
+            if (t == DType_FP32)
+            {
+                float f;
+                memcpy(&f, b.data(), 4);
+                return f;
+            }
+            uint16_t h;
+            memcpy(&h, b.data(), 2);
+            if (t == DType_BF16)
+            {
+                const uint32_t u = (uint32_t)h << 16;
+                float f;
+                memcpy(&f, &u, 4);
+                return f;
+            }
+            // IEEE half -> float
+            const uint32_t sign = (uint32_t)(h & 0x8000) << 16;
+            uint32_t exp = (h >> 10) & 31, man = h & 1023, u;
+            if (exp == 0)
+            {
+                if (man == 0)
+                    u = sign;
+                else
+                {
+                    int e = -1;
+                    do
+                    {
+                        man <<= 1;
+                        e++;
+                    } while (!(man & 1024));
+                    u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 1023) << 13);
+                }
+            }
+            else if (exp == 31)
+                u = sign | 0x7f800000u | (man << 13);
+            else
+                u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+            float f;
+            memcpy(&f, &u, 4);
+            return f;
+        };
+        lo = one(attribute.min_val), hi = one(attribute.max_val);
+        return 0;
+    }
     int eval() override
     {
         if (folded)
             return GraphNode::eval();
+        const DType t = inputs[0]->getDtype();
+        if (t == DType_FP16 || t == DType_BF16 || t == DType_FP32)
+        {
+            if (parent_sgt->precise_mode)
+                return error("CLAMP has no precise-mode (fp64) evaluation in this library");
+            float lo = 0.0f, hi = 0.0f;
+            if (decode_fp(lo, hi))
+                return 1;
+            SubgraphTraverser* s = parent_sgt;
+            // NanPropagationMode: 1 = PROPAGATE (also the default of an absent field), 2 = IGNORE
+            const int32_t nan_mode = attribute.nan_mode == 2 ? 2 : 1;
+            if (call(tmi_clamp_fp(s->ctx, tmi_dtype(t), inputs[0]->getElementCount(), s->device(inputs[0]), lo, hi, nan_mode,
+                                  s->device_out(outputs[0]))))
+                return 1;
+            return GraphNode::eval();
+        }
         int32_t lo = 0, hi = 0;
         if (decode(lo, hi))
             return 1;
@@ -374,7 +439,7 @@ int ConvBase::eval()
         outputs[0]->precise = true;
         auto fn             = depthwise ? tmi_depthwise_conv2d_precise : tmi_conv2d_precise;
         if (call(fn(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]), s->bounds_mode ? 1 : 0,
-                    static_cast<double*>(s->device_out(outputs[0])))))
+                    attribute.local_bound ? 1 : 0, static_cast<double*>(s->device_out(outputs[0])))))
             return 1;
         return GraphNode::eval();
     }
@@ -448,7 +513,8 @@ public:
         for (int i = 0; i < 4; i++)
             d.out_pad[i] = attribute.pad[i];
         d.stride[0] = attribute.stride[0], d.stride[1] = attribute.stride[1];
-        d.bias_len = bias->shape[0];
+        d.bias_len  = bias->shape[0];
+        d.acc_dtype = tmi_dtype((DType)attribute.acc_type);
         return 0;
     }
     int checkTensorAttributes() override
@@ -470,6 +536,10 @@ public:
     }
     int eval() override
     {
+        // precise / bounds mode (the reference evaluates this operator in fp64 and on absolute values then,
+        // e.g. tensor_ops.cpp:601-605): no such pass exists here, and the ordinary result must not stand in for it
+        if (parent_sgt->precise_mode && inputs[0]->getDtype() != DType_INT8 && inputs[0]->getDtype() != DType_INT16)
+            return error("%s has no precise-mode (fp64) evaluation in this library", "TRANSPOSE_CONV2D");
         tmi_tconv_desc_t d;
         if (fill_desc(d))
             return 1;
@@ -538,6 +608,10 @@ public:
     }
     int eval() override
     {
+        // precise / bounds mode (the reference evaluates this operator in fp64 and on absolute values then,
+        // e.g. tensor_ops.cpp:601-605): no such pass exists here, and the ordinary result must not stand in for it
+        if (parent_sgt->precise_mode && inputs[0]->getDtype() != DType_INT8 && inputs[0]->getDtype() != DType_INT16)
+            return error("%s has no precise-mode (fp64) evaluation in this library", "AVG_POOL2D / MAX_POOL2D");
         tmi_pool_desc_t d;
         if (fill_desc(d))
             return 1;
@@ -588,7 +662,8 @@ public:
             d.pad[i] = attribute.pad[i];
         for (int i = 0; i < 3; i++)
             d.stride[i] = attribute.stride[i], d.dilation[i] = attribute.dilation[i];
-        d.bias_len = bias->shape[0];
+        d.bias_len  = bias->shape[0];
+        d.acc_dtype = tmi_dtype((DType)attribute.acc_type);
         return 0;
     }
     int checkTensorAttributes() override
@@ -610,6 +685,10 @@ public:
     }
     int eval() override
     {
+        // precise / bounds mode (the reference evaluates this operator in fp64 and on absolute values then,
+        // e.g. tensor_ops.cpp:601-605): no such pass exists here, and the ordinary result must not stand in for it
+        if (parent_sgt->precise_mode && inputs[0]->getDtype() != DType_INT8 && inputs[0]->getDtype() != DType_INT16)
+            return error("%s has no precise-mode (fp64) evaluation in this library", "CONV3D");
         tmi_conv3d_desc_t d;
         if (fill_desc(d))
             return 1;
@@ -883,6 +962,14 @@ int SubgraphTraverser::linkTensorsAndNodes()
             GraphNode* rs = acc->consumers[0];
             if (rs->inputs.size() != 5 || rs->inputs[0] != acc || rs->outputs.size() != 1)
                 continue;
+            // the fused kernel reads the RESCALE's multiplier / shift / zero points when the convolution runs: they must
+            // hold their values by then (constants or graph inputs), which the ready list only guarantees for the
+            // convolution's own operands
+            bool settled = true;
+            for (int i = 1; i < 5; i++)
+                settled = settled && (rs->inputs[i]->is_const || rs->inputs[i]->producer == nullptr);
+            if (!settled)
+                continue;
             ConvBase* conv      = static_cast<ConvBase*>(n.get());
             conv->fused_rescale = rs;
             rs->folded          = true;
@@ -923,9 +1010,16 @@ void* SubgraphTraverser::device(Tensor* t)
 {
     if (t->dev_valid && t->dev)
         return t->dev;
+    if (!t->host_valid)
+    {
+        // neither copy holds the tensor's value: an operand that no node has produced yet
+        last_message = "tensor " + t->getName() + " is read before it has a value";
+        setGraphStatus(GraphStatus::TOSA_ERROR);
+        return nullptr;
+    }
     if (!t->dev && tmi_buf_alloc(ctx, t->bytes(), &t->dev) != TMI_VALID)
         return nullptr;
-    if (t->host_valid && t->bytes())
+    if (t->bytes())
         if (tmi_upload(ctx, t->dev, t->host.data(), t->bytes()) != TMI_VALID)
             return nullptr;
     t->dev_valid = true;
@@ -1040,8 +1134,11 @@ int SubgraphTraverser::evaluateAll()
     const int rc = tmi_ctx_sync(ctx);
     if (rc == TMI_UNPREDICTABLE)
     {
-        last_message = "OpRescale failure: a REQUIRE condition of apply_scale fired (flags " +
-                       std::to_string(tmi_ctx_flags(ctx)) + ")";
+        const uint32_t flags = tmi_ctx_flags(ctx);
+        if (flags & TMI_FLAG_LEVEL)
+            last_message = std::string("LEVEL_CHECK() fails: ") + tmi_last_error(ctx);
+        else
+            last_message = "OpRescale failure: a REQUIRE condition of apply_scale fired (flags " + std::to_string(flags) + ")";
         setGraphStatus(GraphStatus::TOSA_UNPREDICTABLE);
     }
     else if (rc == TMI_ERROR)
@@ -1060,6 +1157,8 @@ GraphStatus ModelRunner::initialize(const BasicBlock& block)
     sgt->enable_fusion = fusion;
     sgt->precise_mode  = precise_mode;
     sgt->bounds_mode   = bounds_mode;
+    if (sgt->ctx)
+        tmi_ctx_set_level(sgt->ctx, &level);
     if (sgt->initializeGraph() || sgt->linkTensorsAndNodes() || sgt->validateGraph())
         return sgt->getGraphStatus() == GraphStatus::TOSA_VALID ? GraphStatus::TOSA_ERROR : sgt->getGraphStatus();
     return sgt->getGraphStatus();

@@ -228,10 +228,13 @@ public:
     SubgraphTraverser* traverser() { return sgt.get(); }
     void disableFusion() { fusion = false; }
     void setPreciseMode(bool precise, bool bounds) { precise_mode = precise, bounds_mode = bounds; }
+    // g_func_config.tosa_level (func_config.h:63-66); all zero = NONE
+    void setLevel(const tmi_level_t& l) { level = l; }
 
 private:
     int device_id;
     bool fusion = true, precise_mode = false, bounds_mode = false;
+    tmi_level_t level = { 0, 0, 0, 0, 0 };
     std::unique_ptr<SubgraphTraverser> sgt;
 };
 

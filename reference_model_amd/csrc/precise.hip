@@ -47,13 +47,44 @@ struct PreciseConvArgs
     int32_t abs_mode;
     int32_t depthwise;
     int32_t vec;    // channel vectors are whole, aligned 16-byte pieces
+    // bounds mode without local_bound (tensor_ops.cpp:797-801, 1252-1256): every input element is replaced by the
+    // largest magnitude of the input tensor, found by absmax_kernel; nullptr otherwise
+    const double* input_abs_max;
 };
+
+// The largest |x| of a tensor into *out (zero before the launch; non-negative doubles order like their bit patterns).
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_kernel(const void* x, int64_t n, double* out)
+{
+    __shared__ double red[256];
+    double m             = 0.0;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        m = fmax(m, fabs(widen<T>(x, (size_t)i)));
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1)
+    {
+        if ((int)threadIdx.x < s)
+            red[threadIdx.x] = fmax(red[threadIdx.x], red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0)
+        atomicMax(reinterpret_cast<unsigned long long*>(out), (unsigned long long)__double_as_longlong(red[0]));
+}
+
+__global__ void store_zero_kernel(double* p)
+{
+    *p = 0.0;
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void precise_conv_kernel(PreciseConvArgs a)
 {
     const ConvGeom& g    = a.g;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const bool flat      = a.input_abs_max != nullptr;    // the input is one constant
+    const double gmax    = flat ? *a.input_abs_max : 0.0;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.total; i += stride)
     {
         const int oc      = (int)(i % g.OC);
@@ -80,7 +111,7 @@ __global__ __launch_bounds__(256) void precise_conv_kernel(PreciseConvArgs a)
                     double u = widen<T>(a.in, in_base + c);
                     double v = widen<T>(a.w, (((size_t)ky * g.KW + kx) * g.IC + c) * g.M + m);
                     if (a.abs_mode)
-                        u = fabs(u), v = fabs(v);
+                        u = flat ? gmax : fabs(u), v = fabs(v);
                     acc = acc + u * v;
                 }
                 else
@@ -103,7 +134,7 @@ __global__ __launch_bounds__(256) void precise_conv_kernel(PreciseConvArgs a)
                             {
                                 double u = widen<T>(xu, e), v = widen<T>(xw, e);
                                 if (a.abs_mode)
-                                    u = fabs(u), v = fabs(v);
+                                    u = flat ? gmax : fabs(u), v = fabs(v);
                                 acc = acc + u * v;
                             }
                         }
@@ -113,7 +144,7 @@ __global__ __launch_bounds__(256) void precise_conv_kernel(PreciseConvArgs a)
                         double u = widen<T>(a.in, in_base + ic);
                         double v = widen<T>(a.w, w_base + ic);
                         if (a.abs_mode)
-                            u = fabs(u), v = fabs(v);
+                            u = flat ? gmax : fabs(u), v = fabs(v);
                         acc = acc + u * v;
                     }
                 }
@@ -177,13 +208,28 @@ static int grid_for(int64_t total)
 }
 
 const char* launch_conv_precise(hipStream_t st, int32_t in_dtype, bool depthwise, const ConvGeom& g, const void* in,
-                                const void* w, const void* bias, int32_t abs_mode, double* out)
+                                const void* w, const void* bias, int32_t abs_mode, double* abs_max_slot, double* out)
 {
     PreciseConvArgs a{};
     a.g = g, a.in = in, a.w = w, a.bias = bias, a.out = out, a.abs_mode = abs_mode, a.depthwise = depthwise ? 1 : 0;
     a.total = (int64_t)g.N * g.OH * g.OW * g.OC;
     const int eb = in_dtype == TMI_FP32 ? 4 : 2;
     a.vec        = ((int64_t)g.IC * eb) % 16 == 0 && (((uintptr_t)in | (uintptr_t)w) & 15) == 0;
+    if (abs_mode && abs_max_slot)
+    {
+        // the bounds pass of an operator without local_bound: the input tensor's largest magnitude first
+        const int64_t n_in = (int64_t)g.N * g.IH * g.IW * g.IC;
+        const dim3 rgrid(grid_for(n_in)), rblock(256);
+        hipLaunchKernelGGL(store_zero_kernel, dim3(1), dim3(1), 0, st, abs_max_slot);
+        switch (in_dtype)
+        {
+            case TMI_FP16: hipLaunchKernelGGL(absmax_kernel<_Float16>, rgrid, rblock, 0, st, in, n_in, abs_max_slot); break;
+            case TMI_BF16: hipLaunchKernelGGL(absmax_kernel<bf16_t>, rgrid, rblock, 0, st, in, n_in, abs_max_slot); break;
+            case TMI_FP32: hipLaunchKernelGGL(absmax_kernel<float>, rgrid, rblock, 0, st, in, n_in, abs_max_slot); break;
+            default: return nullptr;
+        }
+        a.input_abs_max = abs_max_slot;
+    }
     switch (in_dtype)
     {
         case TMI_FP16: hipLaunchKernelGGL(precise_conv_kernel<_Float16>, dim3(grid_for(a.total)), dim3(256), 0, st, a); break;

@@ -55,6 +55,8 @@ struct tmi_ctx
     std::vector<void*> retired;         // outgrown scratch blocks: captured graphs may still name them
     unsigned char* static_scratch = nullptr;    // this device's copy of the library's static scratch array
     uint32_t last_flags   = 0;
+    uint32_t host_flags   = 0;          // conditions found on the host since the last sync (TMI_FLAG_LEVEL)
+    tmi_level_t level     = { 0, 0, 0, 0, 0 };    // all zero: no level configured (func_config_t::NONE)
     int32_t kernel_choice = 0;
     std::string last_error;
     const char* last_kernel = "";
@@ -80,6 +82,40 @@ int fail(tmi_ctx* ctx, const char* fmt, ...)
 int hip_fail(tmi_ctx* ctx, hipError_t e, const char* what)
 {
     return fail(ctx, "%s: %s", what, hipGetErrorString(e));
+}
+
+// LEVEL_CHECK (func_debug.h:132-141): with a level configured, a violated limit makes the graph UNPREDICTABLE and
+// evaluation goes on.  The condition is latched on the host and reported by the next tmi_ctx_sync().
+bool level_on(const tmi_ctx* ctx)
+{
+    const tmi_level_t& l = ctx->level;
+    return l.max_rank || l.max_kernel || l.max_stride || l.max_scale || l.max_tensor_list_size;
+}
+
+void level_check(tmi_ctx* ctx, bool cond, const char* op, const char* what)
+{
+    if (cond || !level_on(ctx))
+        return;
+    ctx->host_flags |= TMI_FLAG_LEVEL;
+    ctx->last_error = std::string(op) + ": LEVEL_CHECK: " + what;
+}
+
+// the LEVEL_CHECKs at the head of OpConv2d / OpDepthwiseConv2d::eval (tensor_ops.cpp:761-771, 1210-1220)
+void level_check_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d)
+{
+    if (!level_on(ctx))
+        return;
+    const tmi_level_t& l = ctx->level;
+    level_check(ctx, (int64_t)d->dilation[0] * d->KH <= l.max_kernel, op, "dilation_y * KH should be smaller than or equal to MAX_KERNEL");
+    level_check(ctx, (int64_t)d->dilation[1] * d->KW <= l.max_kernel, op, "dilation_x * KW should be smaller than or equal to MAX_KERNEL");
+    static const char* const pad_msg[4] = { "pad_top should be smaller than or equal to MAX_KERNEL",
+                                            "pad_bottom should be smaller than or equal to MAX_KERNEL",
+                                            "pad_left should be smaller than or equal to MAX_KERNEL",
+                                            "pad_right should be smaller than or equal to MAX_KERNEL" };
+    for (int i = 0; i < 4; i++)
+        level_check(ctx, d->pad[i] <= l.max_kernel, op, pad_msg[i]);
+    level_check(ctx, d->stride[0] <= l.max_stride, op, "stride_y should be smaller than or equal to MAX_STRIDE");
+    level_check(ctx, d->stride[1] <= l.max_stride, op, "stride_x should be smaller than or equal to MAX_STRIDE");
 }
 
 #define TMI_HIP(ctx, call)                                                                                          \
@@ -159,6 +195,11 @@ int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool d
     const int32_t want_out = d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype;
     if (d->out_dtype != want_out)
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    // the accumulator type is part of the operator's type signature (op_factory.h:97-118, tensor_ops.cpp:2219-2251):
+    // INT32 for INT8 operands, FP32 for floating point; FP16 accumulation of FP16 operands exists in the reference and
+    // is not built here
+    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+        return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1 || d->OH < 0 ||
         d->OW < 0)
         return fail(ctx, "%s: negative tensor dimension", op);
@@ -343,13 +384,17 @@ int validate_fused_rescale(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* 
     return TMI_VALID;
 }
 
+// check_level: false for the CONV2D that TRANSPOSE_CONV2D / CONV3D are evaluated as (their own limits were checked)
 int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in, const void* w,
-             const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, int32_t out_dtype, void* out)
+             const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, int32_t out_dtype, void* out,
+             bool check_level = true)
 {
     ConvGeom g;
     int rc = validate_conv(ctx, op, d, depthwise, in_zp, w_zp, g);
     if (rc != TMI_VALID)
         return rc;
+    if (check_level)
+        level_check_conv(ctx, op, d);
     const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
     if (total > 0 && (!in || !w || !bias || !out))
         return fail(ctx, "%s: null tensor pointer", op);
@@ -495,15 +540,16 @@ int tmi_ctx_sync(tmi_ctx_t* ctx)
     TMI_HIP(ctx, hipMemcpyAsync(ctx->flags_host, ctx->flags_dev, sizeof(uint32_t), hipMemcpyDeviceToHost,
                                 ctx->stream));
     TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
-    ctx->last_flags = *ctx->flags_host;
-    if (ctx->last_flags)
+    const uint32_t dev_flags = *ctx->flags_host;
+    ctx->last_flags          = dev_flags | ctx->host_flags;
+    ctx->host_flags          = 0;
+    if (dev_flags)
     {
         // cleared with a plain stream-ordered memset: nothing captures this path into a graph
         TMI_HIP(ctx, hipMemsetAsync(ctx->flags_dev, 0, sizeof(uint32_t), ctx->stream));
         TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        return TMI_UNPREDICTABLE;
     }
-    return TMI_VALID;
+    return ctx->last_flags ? TMI_UNPREDICTABLE : TMI_VALID;
 }
 
 uint32_t tmi_ctx_flags(const tmi_ctx_t* ctx)
@@ -521,12 +567,46 @@ const char* tmi_last_kernel(const tmi_ctx_t* ctx)
     return ctx ? ctx->last_kernel : "";
 }
 
+int tmi_ctx_set_level(tmi_ctx_t* ctx, const tmi_level_t* level)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    ctx->level = level ? *level : tmi_level_t{ 0, 0, 0, 0, 0 };
+    return TMI_VALID;
+}
+
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
     if (!ctx || choice < 0 || choice > 4)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;
+}
+
+int tmi_debug_launch_empty(tmi_ctx_t* ctx, int32_t grid, int32_t block, int32_t lds_bytes)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    const char* name = launch_empty(ctx->stream, grid, block, lds_bytes);
+    if (!name)
+        return fail(ctx, "tmi_debug_launch_empty: grid %d, block %d, LDS %d bytes cannot be launched", grid, block, lds_bytes);
+    return after_launch(ctx, name);
+}
+
+int tmi_debug_tile_decode(int64_t grid, uint32_t n_ocb, uint32_t tiles_x, uint32_t tiles_y, uint32_t block,
+                          int32_t* out4)
+{
+    const int exact = tile_decode_is_exact(grid, n_ocb, tiles_x, tiles_y) ? 1 : 0;
+    if (out4 && n_ocb && tiles_x && tiles_y)
+    {
+        const uint32_t tile = fdiv_host(block, make_fastdiv(n_ocb));
+        const uint32_t trow = fdiv_host(tile, make_fastdiv(tiles_x));
+        const uint32_t n    = fdiv_host(trow, make_fastdiv(tiles_y));
+        out4[0] = (int32_t)(block - tile * n_ocb), out4[1] = (int32_t)(tile - trow * tiles_x);
+        out4[2] = (int32_t)(trow - n * tiles_y), out4[3] = (int32_t)n;
+    }
+    return exact;
 }
 
 int tmi_ctx_reserve_workspace(tmi_ctx_t* ctx, size_t bytes)
@@ -626,6 +706,8 @@ static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* 
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+        return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1)
         return fail(ctx, "%s: negative tensor dimension", op);
     // checkTensorAttributes (tensor_ops.cpp:2017-2053)
@@ -663,6 +745,17 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
     int rc = validate_tconv(ctx, op, d, in_zp, w_zp);
     if (rc != TMI_VALID)
         return rc;
+    if (level_on(ctx))
+    {
+        // tensor_ops.cpp:2096-2104
+        const tmi_level_t& l = ctx->level;
+        level_check(ctx, d->KH <= l.max_kernel, op, "KH should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, d->KW <= l.max_kernel, op, "KW should be smaller than or equal to MAX_KERNEL");
+        for (int i = 0; i < 4; i++)
+            level_check(ctx, d->out_pad[i] <= l.max_kernel, op, "out_pad should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, d->stride[0] <= l.max_stride, op, "stride_y should be smaller than or equal to MAX_STRIDE");
+        level_check(ctx, d->stride[1] <= l.max_stride, op, "stride_x should be smaller than or equal to MAX_STRIDE");
+    }
     const int64_t total = (int64_t)d->N * d->OH * d->OW * d->OC;
     if (total == 0)
     {
@@ -686,7 +779,7 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
     c.pad[0] = d->KH - 1 + d->out_pad[0], c.pad[1] = d->KH - 1 + d->out_pad[1];
     c.pad[2] = d->KW - 1 + d->out_pad[2], c.pad[3] = d->KW - 1 + d->out_pad[3];
     c.stride[0] = c.stride[1] = 1, c.dilation[0] = c.dilation[1] = 1;
-    c.bias_len = d->bias_len;
+    c.bias_len = d->bias_len, c.acc_dtype = d->acc_dtype;
     RescaleParams none{};
     // the slab kernel reads both operands where they lie (holes and flip are part of its addressing)
     if ((ctx->kernel_choice == 0 || ctx->kernel_choice == 4) && d->in_dtype == TMI_INT8)
@@ -725,7 +818,7 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
                 : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
         return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
-                    d->out_dtype, out_dev);
+                    d->out_dtype, out_dev, false);
 }
 
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
@@ -753,6 +846,8 @@ static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
+    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+        return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->ID < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KD < 1 || d->KH < 1 ||
         d->KW < 1)
         return fail(ctx, "%s: negative tensor dimension", op);
@@ -799,6 +894,18 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     int rc = validate_conv3d(ctx, op, d, in_zp, w_zp);
     if (rc != TMI_VALID)
         return rc;
+    if (level_on(ctx))
+    {
+        // tensor_ops.cpp:981-995
+        const tmi_level_t& l = ctx->level;
+        level_check(ctx, (int64_t)d->dilation[0] * d->KD <= l.max_kernel, op, "dilation_d * KD should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, (int64_t)d->dilation[1] * d->KH <= l.max_kernel, op, "dilation_y * KH should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, (int64_t)d->dilation[2] * d->KW <= l.max_kernel, op, "dilation_x * KW should be smaller than or equal to MAX_KERNEL");
+        for (int i = 0; i < 6; i++)
+            level_check(ctx, d->pad[i] <= l.max_kernel, op, "pad should be smaller than or equal to MAX_KERNEL");
+        for (int i = 0; i < 3; i++)
+            level_check(ctx, d->stride[i] <= l.max_stride, op, "stride should be smaller than or equal to MAX_STRIDE");
+    }
     const int64_t total = (int64_t)d->N * d->OD * d->OH * d->OW * d->OC;
     if (total == 0)
     {
@@ -821,7 +928,7 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
         c.pad[i] = d->pad[2 + i];
     c.stride[0] = d->stride[1], c.stride[1] = d->stride[2];
     c.dilation[0] = d->dilation[1], c.dilation[1] = d->dilation[2];
-    c.bias_len = d->bias_len;
+    c.bias_len = d->bias_len, c.acc_dtype = d->acc_dtype;
     RescaleParams none{};
     // the slab kernel reads both operands where they lie (the depth taps are part of its addressing)
     if ((ctx->kernel_choice == 0 || ctx->kernel_choice == 4) && d->in_dtype == TMI_INT8 && d->KD > 1)
@@ -847,7 +954,7 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
                                 d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
         return fail(ctx, "%s: operand re-layout launch failed", op);
-    return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev);
+    return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev, false);
 }
 
 int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
@@ -976,7 +1083,7 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
 
 // ---- floating-point compliance passes (precise.hip) -------------------------------------------------------
 static int run_conv_precise(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in,
-                            const void* w, const void* bias, int32_t bounds_mode, double* out)
+                            const void* w, const void* bias, int32_t bounds_mode, int32_t local_bound, double* out)
 {
     ConvGeom g;
     int rc = validate_conv(ctx, op, d, depthwise, 0, 0, g);
@@ -993,26 +1100,30 @@ static int run_conv_precise(tmi_ctx* ctx, const char* op, bool depthwise, const 
         ctx->last_kernel = "empty";
         return TMI_VALID;
     }
-    const char* name = launch_conv_precise(ctx->stream, d->in_dtype, depthwise, g, in, w, bias, bounds_mode, out);
+    // one double of the context's 256-byte block (bytes 160..167) holds the input's largest magnitude
+    double* abs_max_slot = (bounds_mode && !local_bound) ? reinterpret_cast<double*>(reinterpret_cast<uint8_t*>(ctx->flags_dev) + 160)
+                                                         : nullptr;
+    const char* name = launch_conv_precise(ctx->stream, d->in_dtype, depthwise, g, in, w, bias, bounds_mode, abs_max_slot, out);
     if (!name)
         return fail(ctx, "%s: operand type without a precise-mode kernel", op);
     return after_launch(ctx, name);
 }
 
 int tmi_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
-                       const void* bias_dev, int32_t bounds_mode, double* out_dev)
+                       const void* bias_dev, int32_t bounds_mode, int32_t local_bound, double* out_dev)
 {
     if (!ctx)
         return TMI_ERROR;
-    return run_conv_precise(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, bounds_mode, out_dev);
+    return run_conv_precise(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, bounds_mode, local_bound, out_dev);
 }
 
 int tmi_depthwise_conv2d_precise(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
-                                 const void* bias_dev, int32_t bounds_mode, double* out_dev)
+                                 const void* bias_dev, int32_t bounds_mode, int32_t local_bound, double* out_dev)
 {
     if (!ctx)
         return TMI_ERROR;
-    return run_conv_precise(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, bounds_mode, out_dev);
+    return run_conv_precise(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, bounds_mode, local_bound,
+                            out_dev);
 }
 
 int tmi_matmul_precise(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
@@ -1130,6 +1241,17 @@ static int run_pool(tmi_ctx* ctx, const char* op, bool avg, const tmi_pool_desc_
     int rc = validate_pool(ctx, op, d, avg, in_zp, out_zp);
     if (rc != TMI_VALID)
         return rc;
+    if (level_on(ctx))
+    {
+        // tensor_ops.cpp:575-582, 1572-1579
+        const tmi_level_t& l = ctx->level;
+        level_check(ctx, d->kernel[0] <= l.max_kernel, op, "kernel_y should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, d->kernel[1] <= l.max_kernel, op, "kernel_x should be smaller than or equal to MAX_KERNEL");
+        level_check(ctx, d->stride[0] <= l.max_stride, op, "stride_y should be smaller than or equal to MAX_STRIDE");
+        level_check(ctx, d->stride[1] <= l.max_stride, op, "stride_x should be smaller than or equal to MAX_STRIDE");
+        for (int i = 0; i < 4; i++)
+            level_check(ctx, d->pad[i] <= l.max_kernel, op, "pad should be smaller than or equal to MAX_KERNEL");
+    }
     const int64_t total = (int64_t)d->N * d->OH * d->OW * d->C;
     if (total > 0 && (!in_dev || !out_dev))
         return fail(ctx, "%s: null tensor pointer", op);
@@ -1175,6 +1297,8 @@ int tmi_rescale(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank, int64
     int rc = validate_rescale(ctx, r, rank, C, multiplier_dev, shift_dev, p);
     if (rc != TMI_VALID)
         return rc;
+    // type_conversion.cpp:76
+    level_check(ctx, rank <= ctx->level.max_rank, "OpRescale", "Rank should be smaller than or equal to MAX_RANK");
     const int64_t n = rows * (int64_t)C;
     if (n > 0 && (!in_dev || !out_dev))
         return fail(ctx, "OpRescale: null tensor pointer");
@@ -1197,6 +1321,25 @@ int tmi_clamp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, int3
         return fail(ctx, "OpClamp: bad tensor");
     TMI_HIP(ctx, hipSetDevice(ctx->device));
     return after_launch(ctx, launch_clamp(ctx->stream, dtype, in_dev, out_dev, n, min_val, max_val));
+}
+
+int tmi_clamp_fp(tmi_ctx_t* ctx, int32_t dtype, int64_t n, const void* in_dev, float min_val, float max_val,
+                 int32_t nan_mode, void* out_dev)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (dtype != TMI_FP16 && dtype != TMI_BF16 && dtype != TMI_FP32)
+        return fail(ctx, "OpClamp: unsupported TOSA_REF_TYPE");
+    if (max_val < min_val)
+        return fail(ctx, "OpClamp: max smaller than min");
+    if (min_val != min_val || max_val != max_val)
+        return fail(ctx, "OpClamp: min/max cannot be NaN");
+    if (nan_mode != 1 && nan_mode != 2)
+        return fail(ctx, "OpClamp: invalid NaN propagation mode");
+    if (n < 0 || (n > 0 && (!in_dev || !out_dev)))
+        return fail(ctx, "OpClamp: bad tensor");
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    return after_launch(ctx, launch_clamp_fp(ctx->stream, dtype, in_dev, out_dev, n, min_val, max_val, nan_mode));
 }
 
 }    // extern "C"

@@ -29,6 +29,30 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f)
     return f.d <= 1 ? n : __umulhi(n, f.magic);
 }
 
+// The same quotient on the host (the multiply-high written out).
+inline uint32_t fdiv_host(uint32_t n, FastDiv f)
+{
+    return f.d <= 1 ? n : (uint32_t)(((uint64_t)n * f.magic) >> 32);
+}
+
+// fdiv(n, make_fastdiv(d)) is exact for every n <= max_n.
+inline bool fastdiv_exact_up_to(uint64_t max_n, uint32_t d)
+{
+    return d <= 1 || max_n * (uint64_t)d < (uint64_t(1) << 32);
+}
+
+// The tiled kernels turn a block index into (channel block, tile column, tile row, image) with three FastDiv
+// divisions: block / n_ocb, then / tiles_x, then / tiles_y.  True when all three are exact for every block of the
+// grid; a launcher whose layer fails this leaves the layer to a kernel with another decomposition.
+inline bool tile_decode_is_exact(int64_t grid, uint32_t n_ocb, uint32_t tiles_x, uint32_t tiles_y)
+{
+    if (grid <= 0 || grid >= (int64_t(1) << 31) || !n_ocb || !tiles_x || !tiles_y)
+        return false;
+    const uint64_t max_bid = (uint64_t)grid - 1, max_tile = max_bid / n_ocb, max_trow = max_tile / tiles_x;
+    return fastdiv_exact_up_to(max_bid, n_ocb) && fastdiv_exact_up_to(max_tile, tiles_x) &&
+           fastdiv_exact_up_to(max_trow, tiles_y);
+}
+
 // Everything a kernel needs to apply RESCALE (and an optional CLAMP) to one value.  Filled on the host
 // after validation, passed by value.
 struct RescaleParams

@@ -80,6 +80,10 @@ const char* launch_rescale(hipStream_t st, const RescaleParams& p, int32_t in_dt
                            const void* in, void* out, int64_t n, int32_t C, uint32_t* flag_word);
 const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, int32_t lo,
                          int32_t hi);
+const char* launch_clamp_fp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, float lo, float hi,
+                            int32_t nan_mode);
+// a kernel without work: the cost of one launch of this grid, block and dynamic LDS size
+const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t lds_bytes);
 
 // direct.hip: one output element per lane, any legal shape.  out_dtype is the stored output type
 // (INT32 without rescale; the rescale output type with it; FP16/BF16/FP32 for floating point).
@@ -92,8 +96,10 @@ const char* launch_depthwise_direct(hipStream_t st, int32_t in_dtype, int32_t ou
 // precise.hip: fp64 precise-mode / bounds-mode passes (abs_mode != 0: sums over absolute values) of CONV2D,
 // DEPTHWISE_CONV2D and MATMUL on fp16 / bf16 / fp32 operands, and the DOT_PRODUCT check as a reduction
 // (results: 3 doubles, counts: 1 word, both zero before the launch).  nullptr for another operand type.
+// abs_max_slot: device scratch of one double; when given together with abs_mode, every input element is replaced by
+// the input tensor's largest magnitude (the bounds pass of an operator whose local_bound attribute is false).
 const char* launch_conv_precise(hipStream_t st, int32_t in_dtype, bool depthwise, const ConvGeom& g, const void* in,
-                                const void* w, const void* bias, int32_t abs_mode, double* out);
+                                const void* w, const void* bias, int32_t abs_mode, double* abs_max_slot, double* out);
 const char* launch_matmul_precise(hipStream_t st, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
                                   const void* a, const void* b, int32_t abs_mode, double* out);
 const char* launch_dp_check(hipStream_t st, int32_t out_dtype, int64_t n, const void* imp, const double* ref,

@@ -34,8 +34,13 @@ def test_library_exports_every_declared_symbol():
 
 def test_structs_match_header_sizes():
     from reference_model_amd import capi
-    assert ctypes.sizeof(capi.ConvDesc) == 4 * 20
+    # the int32 fields of each descriptor in include/tosa_mi355.h
+    assert ctypes.sizeof(capi.ConvDesc) == 4 * 21
+    assert ctypes.sizeof(capi.TconvDesc) == 4 * 19
+    assert ctypes.sizeof(capi.Conv3dDesc) == 4 * 28
+    assert ctypes.sizeof(capi.PoolDesc) == 4 * 17
     assert ctypes.sizeof(capi.RescaleDesc) == 4 * 11
+    assert ctypes.sizeof(capi.Level) == 4 * 5
 
 
 def test_no_cpu_fallback_without_device():

@@ -123,6 +123,56 @@ def test_device_dot_product_check_matches_its_numpy_restatement(ctx, kind):
     assert r.failed_elements == 3 and not r.compliant
 
 
+@pytest.mark.parametrize("kind", ["fp16", "bf16", "fp32"])
+def test_device_dot_product_check_branches(ctx, kind):
+    """every branch of validateElement / validateDataDP (verify_dot_product.cpp:34-87, 127-139): a NaN reference met
+    and missed, a NaN bound, a bound at which the sum may overflow the output type, and the error-sum rule that only
+    the data sets 3..5 carry"""
+    rng = np.random.default_rng(11)
+    n, ksb = 4096, 5
+    frac = dp.NORMAL_FRAC[kind]
+    big = {"fp16": 65000.0, "bf16": 3.3e38, "fp32": 3.3e38}[kind]      # bnd * (1 + abs_bound * 2^-(1+frac)) overflows
+    dtype = {"fp16": capi.FP16, "bf16": capi.BF16, "fp32": capi.FP32}[kind]
+
+    def to_dev(a64):
+        if kind == "fp16":
+            return a64.astype(np.float16)
+        if kind == "bf16":
+            return cases.float_to_bf16_bits(a64.astype(np.float32))
+        return a64.astype(np.float32)
+
+    def back(a):
+        return cases.bf16_bits_to_float(a).astype(np.float64) if kind == "bf16" else a.astype(np.float64)
+
+    ref = rng.normal(0, 2, n)
+    bnd = np.abs(ref) + 1.0
+    imp64 = ref + 0.3 * bnd * 2.0 ** (-1 - frac)          # every error +0.3 units: a bias, well inside abs_bound
+    ref[5], imp64[5] = np.nan, np.nan                     # NaN reference, matched
+    bnd[6] = np.nan                                       # NaN bound: anything goes
+    imp64[6] = 12345.0
+    with np.errstate(over="ignore"):
+        bnd[7] = big                                      # may overflow: anything goes
+        imp64[7] = -1.0
+    imp = to_dev(imp64)
+    for set_number in (-1, 0, 3, 5):
+        want = dp.check(back(imp), ref, bnd, kind, ksb, set_number)
+        r = ctx.dot_product_check(dtype, n, ctx.upload(imp, dtype), ctx.upload(ref, capi.F64), ctx.upload(bnd, capi.F64), ksb,
+                                  set_number)
+        assert r.failed_elements == want["failed_elements"] == 0
+        assert r.err_sum == pytest.approx(want["err_sum"], rel=1e-9)
+        assert r.err_sumsq == pytest.approx(want["err_sumsq"], rel=1e-9)
+        assert bool(r.compliant) == want["ok"]
+        # 4093 errors of about +0.3 (fp16 / bf16 round them to multiples of a unit): the sum is beyond
+        # sqrt(10 * 1.6 ksb * T) = 572, which only sets 3..5 hold against
+        assert want["ok"] == (set_number not in (3, 5)) and abs(want["err_sum"]) > 600
+    # the NaN reference missed
+    imp2 = back(imp).copy()
+    imp2[5] = 0.0
+    want = dp.check(imp2, ref, bnd, kind, ksb)
+    r = ctx.dot_product_check(dtype, n, ctx.upload(to_dev(imp2), dtype), ctx.upload(ref, capi.F64), ctx.upload(bnd, capi.F64), ksb)
+    assert r.failed_elements == want["failed_elements"] == 1 and not r.compliant and not want["ok"]
+
+
 @pytest.mark.parametrize("data_set", range(6))
 def test_config5_bf16_matmul_compliance_on_the_device(ctx, data_set):
     """[4,2048,4096] x [4,4096,2048] bf16 -> fp32 on the specification's data set, every pass on the GPU:

@@ -327,7 +327,9 @@ def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
     pad, stride, dil = (1, 1, 1, 1), (1, 1), (1, 1)
     xf, wf, bf = (v.astype(np.float64) for v in (x, w, b))
     ref = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil)
-    bnd = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True)
+    # the attribute's local_bound is absent = false here: the bounds pass replaces the input by its largest magnitude
+    # (tensor_ops.cpp:797-801)
+    bnd = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True, local_bound=False)
     ts = [W.tensor("x", x.shape, np.float16), W.tensor("w", w.shape, np.float16, w), W.tensor("b", [10], np.float16, b),
           W.tensor("z", [1], np.float16, [0]), W.tensor("y", ref.shape, np.float16)]
     ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "b", "z")]
@@ -343,6 +345,19 @@ def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
     got, got_bnd = np.load(d1 / "y_out.npy"), np.load(d1 / "bounds_y_out.npy")
     assert got.dtype == got_bnd.dtype == np.float64
     assert np.array_equal(got, ref) and np.array_equal(got_bnd, bnd)
+    # local_bound = true: the sums over the absolute values themselves
+    ops_lb = ops[:-1] + [W.operator(R.OP_CONV2D, ["x", "w", "b", "z", "z"], ["y"],
+                                    W.conv_attr(pad, stride, dil, acc_type=7, local_bound=True))]
+    d5 = tmp_path / "conv_local"
+    d5.mkdir()
+    desc5 = _write_case(d5, W.graph(ts, ops_lb, ["x"], ["y"]), {"x": x}, ["y"])
+    meta5 = dict(json.loads(open(desc5).read()), test_requirements={"bounds_file_required": True})
+    open(desc5, "w").write(json.dumps(meta5))
+    r = _run(desc5, "--precise_mode=1")
+    assert r.returncode == 0, r.stderr
+    local = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True)
+    assert np.array_equal(np.load(d5 / "bounds_y_out.npy"), local) and np.array_equal(np.load(d5 / "y_out.npy"), ref)
+    assert np.all(bnd >= local) and not np.array_equal(bnd, local)
     # without the option the result has the graph's element type and no bounds file appears
     d2 = tmp_path / "plain"
     d2.mkdir()
@@ -370,6 +385,64 @@ def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
     assert np.array_equal(np.load(d4 / "o_out.npy"), oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64)))
     assert np.array_equal(np.load(d4 / "bounds_o_out.npy"),
                           oracle.matmul("f64", a.astype(np.float64), bb.astype(np.float64), abs_mode=True))
+
+
+@pytest.mark.gpu
+def test_precise_mode_is_refused_where_no_fp64_pass_exists(tmp_path):
+    """floating-point TRANSPOSE_CONV2D / AVG_POOL2D / CLAMP have no fp64 evaluation here: with --precise_mode=1 the
+    graph ends with status 2 instead of writing the ordinary result under the precise run's name"""
+    rng = np.random.default_rng(13)
+    x = rng.normal(0, 1, (1, 6, 6, 8)).astype(np.float16)
+    ts = [W.tensor("x", x.shape, np.float16), W.tensor("z", [1], np.float16, [0]), W.tensor("y", [1, 3, 3, 8], np.float16)]
+    ops = [W.operator(R.OP_CONST, [], ["z"]),
+           W.operator(R.OP_AVG_POOL2D, ["x", "z", "z"], ["y"], W.pool_attr((2, 2), (2, 2), (0, 0, 0, 0), 7))]
+    desc = _write_case(tmp_path, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"])
+    assert _run(desc).returncode == 0
+    r = _run(desc, "--precise_mode=1")
+    assert r.returncode == 2 and "precise-mode" in r.stderr
+
+
+@pytest.mark.gpu
+def test_fp16_conv2d_then_clamp_runs_on_the_device(tmp_path):
+    """an fp16 CONV2D followed by a floating-point CLAMP (activation_funcs.cpp:97-106) ends with status 0"""
+    rng = np.random.default_rng(14)
+    x = rng.normal(0, 1, (1, 7, 7, 16)).astype(np.float16)
+    w = rng.normal(0, 0.3, (8, 3, 3, 16)).astype(np.float16)
+    b = rng.normal(0, 1, 8).astype(np.float16)
+    ts = [W.tensor("x", x.shape, np.float16), W.tensor("w", w.shape, np.float16, w), W.tensor("b", [8], np.float16, b),
+          W.tensor("z", [1], np.float16, [0]), W.tensor("c", [1, 7, 7, 8], np.float16), W.tensor("y", [1, 7, 7, 8], np.float16)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "b", "z")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "b", "z", "z"], ["c"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1), acc_type=7)))
+    ops.append(W.operator(R.OP_CLAMP, ["c"], ["y"], W.clamp_attr(-0.5, 1.25, np.float16)))
+    r = _run(_write_case(tmp_path, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"]))
+    assert r.returncode == 0, r.stderr
+    got = np.load(tmp_path / "y_out.npy")
+    assert got.dtype == np.float16 and got.min() == np.float16(-0.5) and got.max() == np.float16(1.25)
+    conv = oracle.conv2d("f32", x, w, b, (1, 1, 1, 1)).astype(np.float64)
+    inside = (conv > -0.45) & (conv < 1.2)
+    assert np.allclose(got[inside].astype(np.float64), conv[inside], atol=4e-3)
+
+
+@pytest.mark.gpu
+def test_tosa_level_makes_a_violating_graph_unpredictable(tmp_path):
+    """--tosa_level=EIGHTK: a pad beyond MAX_KERNEL = 8192 fails a LEVEL_CHECK (tensor_ops.cpp:766-769): the graph
+    is evaluated and ends UNPREDICTABLE (func_debug.h:132-141); without a level the same graph is VALID"""
+    x = np.ones((1, 2, 2, 8), np.int8)
+    w = np.ones((8, 1, 1, 8), np.int8)
+    pad = (8193, 0, 0, 0)
+    oh = 2 + 8193
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", w.shape, np.int8, w), W.tensor("b", [8], np.int32, np.zeros(8, np.int32)),
+          W.tensor("z", [1], np.int8, [0]), W.tensor("y", [1, oh, 2, 8], np.int32)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "b", "z")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "b", "z", "z"], ["y"], W.conv_attr(pad, (1, 1), (1, 1))))
+    desc = _write_case(tmp_path, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"])
+    assert _run(desc).returncode == 0
+    want = np.load(tmp_path / "y_out.npy").copy()
+    assert want[0, :8193].max() == 0 and want[0, 8193:].min() == 8
+    r = _run(desc, "--tosa_level=EIGHTK")
+    assert r.returncode == 1 and "MAX_KERNEL" in r.stderr
+    assert np.array_equal(np.load(tmp_path / "y_out.npy"), want)       # evaluated all the same
+    assert _run(desc, "--tosa_level=NONE").returncode == 0
 
 
 # ---- system-under-test module for the reference's conformance runner ----------------------------------------

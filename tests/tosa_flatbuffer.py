@@ -18,6 +18,7 @@ import numpy as np
 # Op / DType numbers of the TOSA 1.0 serialization schema; ops 3, 15, 57, 61, 66, 67, 68, 71 and dtypes
 # 3, 5, 7 are confirmed by the reference's example graphs.
 OP_CONV2D, OP_DEPTHWISE_CONV2D, OP_MATMUL, OP_CLAMP, OP_RESCALE, OP_CONST = 3, 5, 7, 11, 66, 67
+OP_AVG_POOL2D, OP_CONV3D, OP_MAX_POOL2D, OP_TRANSPOSE_CONV2D = 2, 4, 8, 10
 DTYPE_NP = {3: np.int8, 4: np.int16, 5: np.int32, 7: np.float32, 8: np.float16}
 
 
