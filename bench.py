@@ -14,10 +14,14 @@ and --config selects the other benchmark configurations, each reported against t
   c5a  FP16 CONV2D 3x3 [16,28,28,256]x[256,3,3,256], fp32 accumulate (TFLOPS; MFMA roofline)
   c5b  BF16 MATMUL [4,2048,4096]x[4,4096,2048] -> fp32              (TFLOPS; MFMA roofline)
 
-The timed steps are replayed from HIP graphs of up to 100 steps each (--eager: one host launch per step).
-One JSON line is printed: value = whole-job throughput over the timed steps (host clock), roofline.achieved =
-algorithmic work per launch / average launch duration from HIP events recorded on the launch stream, and
-cpu_baseline = the scalar C oracle (1 core) on a bounded sample of the same workload.
+and three configurations that measure the box rather than an operator: launch_floor (a kernel that does nothing,
+with the grid, block and LDS size of the headline kernel) and copy (copy / read-only / write-only streams).
+
+The timed steps are replayed from HIP graphs of up to 100 steps each (--eager: one host launch per step).  The
+region of --steps steps is enqueued --repeats times back to back, each repeat between two HIP events on the launch
+stream; ms_per_step, value and roofline.achieved come from the median repeat, and the host clock around the whole
+region (synchronised on both sides) is reported beside it.  One JSON line is printed.  cpu_baseline = the C oracle
+on a bounded sample of the same workload: on one core (value) and, where its loops are parallel, on all host cores.
 """
 from __future__ import annotations
 
@@ -37,9 +41,9 @@ PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what
 # the same counters read for a plain copy of known size (the committed rocprofv3 summaries hold the raw
 # figures).
-MEASURED_TRAFFIC_BYTES = {"c3": 3639807, "c2": 51169875, "c4": 12201793, "c5a": 22848575, "c5b": 269061469,
-                          "maxpool": 32144806, "avgpool": 32183530, "tconv": 8340286, "conv3d": 8037071,
-                          "rescale": 64289281, "c4x8": 96473119}
+MEASURED_TRAFFIC_BYTES = {"c3": 3610128, "c2": 51125487, "c4": 12201417, "c5a": 22847896, "c5b": 269061069,
+                          "maxpool": 32145619, "avgpool": 32182579, "tconv": 8340031, "conv3d": 8036867,
+                          "rescale": 64287481, "c4x8": 96470586, "c3x4": 13241906}
 
 
 def main() -> int:
@@ -47,7 +51,11 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy"])
+    ap.add_argument("--repeats", type=int, default=None,
+                    help="times the region of --steps steps is run; the median repeat is reported "
+                         "(default: enough repeats for 10000 steps, between 5 and 500)")
+    ap.add_argument("--copy-mib", type=int, default=1024, help="buffer size of --config copy")
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy", "launch_floor"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     ap.add_argument("--eager", action="store_true",
                     help="issue every step from the host instead of replaying HIP graphs of the steps")
@@ -71,30 +79,64 @@ def main() -> int:
     stream = torch.cuda.current_stream()
     ctx.set_stream(stream.cuda_stream)
 
+    def the_oracle():
+        # the CPU oracle is the checker and the CPU baseline: nothing before the timed region touches it
+        import oracle
+        return oracle
+
+    def conv_out_hw(ih, iw, kh, kw, pad, stride, dilation):
+        return ((ih - 1 + pad[0] + pad[1] - (kh - 1) * dilation[0]) // stride[0] + 1,
+                (iw - 1 + pad[2] + pad[3] - (kw - 1) * dilation[1]) // stride[1] + 1)
+
+    def accuracy_figures(imp, ref, bnd, out_type, out_dtype, ks, has_bias):
+        """the result against the library's own fp64 pass over the same operands: the DOT_PRODUCT check (device
+        reduction), and the largest ULP and relative errors (numpy over the downloaded tensors)"""
+        import dot_product_check as dp
+        ksb = dp.kernel_size_bound(ks, out_type, has_bias=has_bias)
+        r = ctx.dot_product_check(out_dtype, imp.numel(), imp, ref, bnd, ksb, -1)
+        ctx.sync()
+        st = dp.check(imp.cpu().numpy(), ref.cpu().numpy(), bnd.cpu().numpy(), out_type, ksb)
+        return {"dot_product_compliant": bool(r.compliant), "max_err_in_bound_units": round(float(r.max_abs_err), 4),
+                "allowed_err_in_bound_units": int(r.abs_bound), "max_ulp": round(st["max_ulp"], 3),
+                "max_rel_err": float("%.4g" % st["max_rel"]),
+                "max_ulp_where_ref_is_at_least_an_eighth_of_the_bound": round(st["max_ulp_conditioned"], 3),
+                "max_err_relative_to_sum_of_abs_products": float("%.4g" % st["max_rel_to_bound"])}
+
     def to_dev(a):
         a = np.ascontiguousarray(a)
         if a.dtype == np.uint16:  # bf16 bit patterns
             return torch.from_numpy(a.view(np.int16)).to(dev)
         return torch.from_numpy(a).to(dev)
 
-    cfg = args.config
+    cfg = "c3" if args.config == "launch_floor" else args.config
     if cfg == "copy":
-        # calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain device copy of known size
-        nbytes = 64 << 20
+        # what the memory system sustains: copy, read-only and write-only passes over one buffer (1 GiB by default,
+        # four times the 256 MiB last-level cache; --copy-mib 64 is the known-size dispatch that calibrates the
+        # FETCH_SIZE / WRITE_SIZE counters)
+        nbytes = args.copy_mib << 20
         src = torch.zeros(nbytes, dtype=torch.int8, device=dev)
         dst = torch.empty_like(src)
-        for _ in range(args.steps or 20):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps({"metric": "copy calibration", "bytes_read_per_launch": nbytes,
-                          "bytes_written_per_launch": nbytes}))
+        out = {"metric": "streaming rates of the box", "unit": "GB/s", "bytes": nbytes}
+        for mode, name, moved in ((0, "copy", 2 * nbytes), (1, "read", nbytes), (2, "write", nbytes)):
+            n_steps = args.steps or 20
+            for _ in range(3):
+                ctx.stream_probe(mode, src, dst, nbytes)
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(n_steps + 1)]
+            for i in range(n_steps):
+                evs[i].record(stream)
+                ctx.stream_probe(mode, src, dst, nbytes)
+            evs[n_steps].record(stream)
+            torch.cuda.synchronize()
+            t = sorted(evs[i].elapsed_time(evs[i + 1]) * 1e-3 for i in range(n_steps))[n_steps // 2]
+            out[name] = {"GB_per_s": round(moved / t / 1e9, 1), "us": round(t * 1e6, 2), "bytes_moved": moved,
+                         "frac_of_8TBps": round(moved / t / 8e12, 4)}
+        print(json.dumps(out))
         ctx.close()
         return 0
     W = {}  # workload description filled below
     if cfg == "rescale":
         # stand-alone RESCALE at a size where launch latency no longer matters: the int32 accumulators of eight
         # batches of the ResNet-style layer, per-channel, double round, to int8
-        import oracle
         c = cases.c3()
         rng = np.random.default_rng(cases.SEED ^ 66)
         acc = rng.integers(-(1 << 23), 1 << 23, (64, 56, 56, 64)).astype(np.int32)
@@ -107,7 +149,7 @@ def main() -> int:
             ctx.rescale(r, 4, rows, 64, tacc, tm, ts, out)
 
         def cpu_ref():
-            return oracle.rescale(acc[:8], c["mult"], c["shift"], out_zp=-3)[0]
+            return the_oracle().rescale(acc[:8], c["mult"], c["shift"], out_zp=-3)[0]
 
         W = dict(ops=acc.size, bytes=acc.nbytes + acc.size + 64 * 5, exact=True, cpu_ref=cpu_ref, cpu_fraction=1 / 8,
                  result=lambda: out[:8].cpu().numpy(), dtype="int64",
@@ -117,7 +159,6 @@ def main() -> int:
                           "output_zp -3 (5 bytes per element)")
     elif cfg == "precise":
         # the fp64 precise-mode pass of the compliance flow at the shape of the named fp16 CONV2D configuration
-        import oracle
         c = cases.c5_conv()
         n, ih, iw, ic = c["x"].shape
         oc, kh, kw, _ = c["w"].shape
@@ -127,9 +168,9 @@ def main() -> int:
                           c["dilation"], oc)
         step = lambda: ctx.conv2d_precise(d, tx, tw, tb, False, out)
         x64, w64, b64 = (c[k].astype(np.float64) for k in ("x", "w", "bias"))
-        cpu_ref = lambda: oracle.conv2d("f64", x64[:1], w64, b64, c["pad"], c["stride"], c["dilation"])
+        cpu_ref = lambda: the_oracle().conv2d("f64", x64[:1], w64, b64, c["pad"], c["stride"], c["dilation"])
         W = dict(ops=2 * n * ih * iw * oc * kh * kw * ic, bytes=c["x"].nbytes + c["w"].nbytes + c["bias"].nbytes +
-                 out.numel() * 8, exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0 / n,
+                 out.numel() * 8, exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0 / n, parallel_oracle=True,
                  result=lambda: out[:1].cpu().numpy(), dtype="f64",
                  metric="fp64 precise-mode CONV2D TFLOPS 3x3 [16,28,28,256]x[256,3,3,256]; bit-exact vs the fp64 oracle",
                  unit="TFLOPS", bound="mfma", peak=78.6, runit="TFLOP/s",
@@ -138,7 +179,6 @@ def main() -> int:
     elif cfg in ("maxpool", "avgpool"):
         # the pooling neighbours at sizes where launch latency no longer dominates: the 3x3 stride-2 max pooling
         # behind a ResNet stem for 32 images, and a 2x2 stride-2 average pooling of the same tensor
-        import oracle
         rng = np.random.default_rng(cases.SEED ^ (8 if cfg == "maxpool" else 2))
         x = rng.integers(-128, 128, (32, 112, 112, 64)).astype(np.int8)
         pk, ps, pp = ((3, 3), (2, 2), (0, 1, 0, 1)) if cfg == "maxpool" else ((2, 2), (2, 2), (0, 0, 0, 0))
@@ -150,10 +190,10 @@ def main() -> int:
         out = torch.empty((32, 56, 56, 64), dtype=torch.int8, device=dev)
         if cfg == "maxpool":
             step = lambda: ctx.max_pool2d(d, tx, out)
-            cpu_ref = lambda: oracle.max_pool2d(x[:4], pk, ps, pp)
+            cpu_ref = lambda: the_oracle().max_pool2d(x[:4], pk, ps, pp)
         else:
             step = lambda: ctx.avg_pool2d(d, tx, -3, 4, out)
-            cpu_ref = lambda: oracle.avg_pool2d(x[:4], pk, ps, pp, -3, 4)
+            cpu_ref = lambda: the_oracle().avg_pool2d(x[:4], pk, ps, pp, -3, 4)
         W = dict(ops=out.numel() * pk[0] * pk[1], bytes=x.nbytes + out.numel(), exact=True, cpu_ref=cpu_ref,
                  cpu_fraction=1 / 8, result=lambda: out[:4].cpu().numpy(), dtype="int8" if cfg == "maxpool" else "int32",
                  metric="int8 %s GB/s; %% HBM peak; bit-exact" % ("MAX_POOL2D" if cfg == "maxpool" else "AVG_POOL2D"),
@@ -164,8 +204,6 @@ def main() -> int:
     elif cfg in ("tconv", "conv3d"):
         # the two neighbouring operators, at shapes of the same family as the named CONV2D configuration (no
         # configuration of theirs is named): the timed step includes the operand re-layout kernels
-        import gpu_ops  # noqa: F401  (TconvDesc / Conv3dDesc helpers live in capi)
-        import oracle
         rng = np.random.default_rng(cases.SEED ^ (10 if cfg == "tconv" else 4))
         if cfg == "tconv":
             x = rng.integers(-128, 128, (8, 28, 28, 128)).astype(np.int8)
@@ -182,7 +220,7 @@ def main() -> int:
             fn, name = ctx.transpose_conv2d, "TRANSPOSE_CONV2D [8,28,28,128]x[64,3,3,128] s2 out_pad [0,1,0,1] -> [8,56,56,64] int32"
 
             def cpu_ref():
-                return oracle.transpose_conv2d("i8", x[:1], w, bias, out_pad, stride, -7, 0)
+                return the_oracle().transpose_conv2d("i8", x[:1], w, bias, out_pad, stride, -7, 0)
             frac = 1 / 8
         else:
             x = rng.integers(-128, 128, (2, 16, 28, 28, 32)).astype(np.int8)
@@ -199,7 +237,7 @@ def main() -> int:
             fn, name = ctx.conv3d, "CONV3D [2,16,28,28,32]x[64,3,3,3,32] s1 p1 -> [2,16,28,28,64] int32"
 
             def cpu_ref():
-                return oracle.conv3d("i8", x[:1], w, bias, pad, st3, dil, -7, 0)
+                return the_oracle().conv3d("i8", x[:1], w, bias, pad, st3, dil, -7, 0)
             frac = 1 / 2
         tx, tw, tb = to_dev(x), to_dev(w), to_dev(bias)
 
@@ -219,8 +257,7 @@ def main() -> int:
             oc = ic * m
         else:
             oc, kh, kw, _ = c["w"].shape
-        import oracle
-        oh, ow = oracle.conv_out_hw(ih, iw, kh, kw, c["pad"], c["stride"], c["dilation"])
+        oh, ow = conv_out_hw(ih, iw, kh, kw, c["pad"], c["stride"], c["dilation"])
         macs = n * oh * ow * oc * kh * kw * (1 if depthwise else ic)
         t = {k: to_dev(c[k]) for k in ("x", "w", "bias", "mult", "shift")}
         out = torch.empty((n, oh, ow, oc), dtype=torch.int8, device=dev)
@@ -233,13 +270,14 @@ def main() -> int:
             fn(d, t["x"], t["w"], t["bias"], c["in_zp"], c["w_zp"], r, t["mult"], t["shift"], out, c["clamp"])
 
         def cpu_ref():
-            f = oracle.depthwise_conv2d if depthwise else oracle.conv2d
+            f = the_oracle().depthwise_conv2d if depthwise else the_oracle().conv2d
             acc = f("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
-            ref, _ = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
-            return ref if c["clamp"] is None else oracle.clamp(ref, *c["clamp"])
+            ref, _ = the_oracle().rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
+            return ref if c["clamp"] is None else the_oracle().clamp(ref, *c["clamp"])
 
         W = dict(ops=2 * macs, bytes=sum(c[k].nbytes for k in ("x", "w", "bias", "mult", "shift")) + out.numel(),
-                 exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0, result=lambda: out.cpu().numpy(), dtype="int8")
+                 exact=True, cpu_ref=cpu_ref, cpu_fraction=1.0, result=lambda: out.cpu().numpy(), dtype="int8",
+                 parallel_oracle=True)
         if cfg in ("c3", "c3x4"):
             W.update(metric="int8 CONV2D+RESCALE TOPS at 3x3 ResNet shape; % int8 MFMA peak; bit-exact", unit="TOPS",
                      bound="mfma", peak=PEAK["int8_mfma"], runit="TOP/s",
@@ -267,17 +305,24 @@ def main() -> int:
         def step():
             ctx.matmul(in_dtype, n, h, k, w, ta, tb, a_zp, b_zp, out)
 
-        import oracle
         rows = 64 if cfg == "c2" else 8  # bounded CPU sample: the first `rows` rows of batch 0
 
         def cpu_ref():
             if cfg == "c2":
-                return oracle.matmul("i8", c["a"][:1, :rows], c["b"][:1], a_zp, b_zp)
-            return oracle.matmul("f32", cases.bf16_bits_to_float(c["a"][:1, :rows]), cases.bf16_bits_to_float(c["b"][:1]))
+                return the_oracle().matmul("i8", c["a"][:1, :rows], c["b"][:1], a_zp, b_zp)
+            return the_oracle().matmul("f32", cases.bf16_bits_to_float(c["a"][:1, :rows]), cases.bf16_bits_to_float(c["b"][:1]))
 
         W = dict(ops=2 * n * h * k * w, bytes=c["a"].nbytes + c["b"].nbytes + out.numel() * 4, exact=cfg == "c2",
                  cpu_ref=cpu_ref, cpu_fraction=rows / (n * h), result=lambda: out[:1, :rows].cpu().numpy(),
-                 dtype="int8" if cfg == "c2" else "bf16")
+                 dtype="int8" if cfg == "c2" else "bf16", parallel_oracle=True)
+        if cfg == "c5b":
+            def accuracy():
+                ref = torch.empty((n, h, w), dtype=torch.float64, device=dev)
+                bnd = torch.empty_like(ref)
+                ctx.matmul_precise(in_dtype, n, h, k, w, ta, tb, False, ref)
+                ctx.matmul_precise(in_dtype, n, h, k, w, ta, tb, True, bnd)
+                return accuracy_figures(out, ref, bnd, "fp32", capi.FP32, k, False)
+            W["accuracy"] = accuracy
         if cfg == "c2":
             W.update(metric="int8 MATMUL TOPS [8,1024,1024]x[8,1024,1024]; bit-exact", unit="TOPS", bound="hbm",
                      peak=PEAK["hbm"], runit="GB/s",
@@ -298,21 +343,46 @@ def main() -> int:
         def step():
             ctx.conv2d(d, tx, tw, tb, 0, 0, out)
 
-        import oracle
 
         def cpu_ref():  # bounded CPU sample: image 0 only
-            return oracle.conv2d("f32", c["x"][:1], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"])
+            return the_oracle().conv2d("f32", c["x"][:1], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"])
 
         W = dict(ops=2 * n * ih * iw * oc * kh * kw * ic, bytes=c["x"].nbytes + c["w"].nbytes + c["bias"].nbytes +
-                 out.numel() * 2, exact=False, cpu_ref=cpu_ref, cpu_fraction=1.0 / n,
+                 out.numel() * 2, exact=False, cpu_ref=cpu_ref, cpu_fraction=1.0 / n, parallel_oracle=True,
                  result=lambda: out[:1].cpu().numpy(), dtype="fp16",
                  metric="fp16 CONV2D TFLOPS 3x3 [16,28,28,256]x[256,3,3,256], fp32 accumulate", unit="TFLOPS",
                  bound="mfma", peak=PEAK["f16_mfma"], runit="TFLOP/s",
                  workload="configs[4a]: FP16 CONV2D 3x3 [16,28,28,256]x[256,3,3,256] s1 p1, fp32 accumulate")
 
+        def accuracy():
+            ref = torch.empty((n, ih, iw, oc), dtype=torch.float64, device=dev)
+            bnd = torch.empty_like(ref)
+            ctx.conv2d_precise(d, tx, tw, tb, False, ref)
+            ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
+            return accuracy_figures(out, ref, bnd, "fp16", capi.FP16, kh * kw * ic, True)
+        W["accuracy"] = accuracy
+
+    if args.config == "launch_floor":
+        # a kernel that does nothing, launched with the grid, block and LDS size the headline kernel has just used
+        step()
+        ctx.sync()
+        grid, block, lds = ctx.last_launch_shape()
+        if not grid:
+            print("bench.py: the headline configuration did not run on the kernel whose launch is measured", file=sys.stderr)
+            return 1
+        step = lambda: ctx.launch_empty(grid, block, lds)
+        W = dict(ops=0, bytes=0, exact=True, cpu_ref=None, cpu_fraction=0.0, result=None, dtype="none",
+                 metric="launch floor: microseconds per launch of a kernel without work", unit="us", bound="hbm",
+                 peak=PEAK["hbm"], runit="GB/s", workload="empty kernel, %d workgroups of %d threads, %d bytes of LDS each "
+                 "(the launch shape of configs[2]'s kernel)" % (grid, block, lds))
+        cfg = "launch_floor"
+
     big = cfg in ("c5b", "precise")
     steps = args.steps if args.steps is not None else (200 if big else 2000)
     warmup = args.warmup if args.warmup is not None else (20 if big else 200)
+    repeats = args.repeats if args.repeats is not None else max(5, min(500, -(-10000 // steps)))
+    if big and args.repeats is None:
+        repeats = 5
 
     for _ in range(warmup):
         step()
@@ -320,8 +390,15 @@ def main() -> int:
     # The steps are recorded into a HIP graph (up to 100 C-ABI calls per graph, nothing but their kernel launches)
     # and the graph is replayed: a launch from the host costs about as much as the small configurations' kernels
     # run, and a serving loop would not pay it per layer either.  --eager times host-issued launches instead.
-    use_graph = not args.eager and cfg not in ("precise", "copy")
-    chunk = math.gcd(steps, 100) if use_graph else 1
+    use_graph = not args.eager and cfg != "precise"
+    # The region of `steps` steps runs `repeats` times back to back; the host clock brackets all of it with a
+    # synchronisation on both sides.  HIP events on the launch stream cut it into timed units: one graph replay
+    # (the graph holds up to 100 steps and may span several short regions, since a replay costs about 10 us by
+    # itself), or one region when every step is launched from the host.  A GPU that has just woken up runs its
+    # first units at ramping clocks: the median unit is the figure reported.
+    total = steps * repeats
+    chunk = math.gcd(total, 100) if use_graph else steps
+    units = total // chunk
     graph = None
     if use_graph:
         graph = torch.cuda.CUDAGraph()
@@ -334,55 +411,84 @@ def main() -> int:
         ctx.set_stream(stream.cuda_stream)
         graph.replay()    # untimed: the first replay uploads the graph
         torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    events = [torch.cuda.Event(enable_timing=True) for _ in range(units + 1)]
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    ev0.record(stream)
-    if use_graph:
-        for _ in range(steps // chunk):
+    for u in range(units):
+        events[u].record(stream)
+        if use_graph:
             graph.replay()
-    else:
-        for _ in range(steps):
-            step()
-    ev1.record(stream)
+        else:
+            for _ in range(chunk):
+                step()
+    events[units].record(stream)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     status = ctx.sync()
     kernel = ctx.last_kernel
-    ms_per_step = (t1 - t0) * 1e3 / steps
-    ev_s_per_launch = ev0.elapsed_time(ev1) * 1e-3 / steps
+    per_unit = sorted(events[i].elapsed_time(events[i + 1]) * 1e-3 / chunk for i in range(units))
+    s_per_step = per_unit[units // 2] if units % 2 else 0.5 * (per_unit[units // 2 - 1] + per_unit[units // 2])
+    ms_per_step = s_per_step * 1e3
+    host_ms_per_step = (t1 - t0) * 1e3 / total
+
+    if cfg == "launch_floor":
+        print(json.dumps({"metric": W["metric"], "value": round(s_per_step * 1e6, 4), "unit": "us", "n_gpus": 1,
+                          "steps": steps, "warmup": warmup, "repeats": repeats, "ms_per_step": round(ms_per_step, 6),
+                          "higher_is_better": False, "data": "synthetic",
+                          "config": {"workload": W["workload"], "kernel": kernel,
+                                     "launch": "%d steps as %d HIP graphs of %d launches; the median graph by HIP "
+                                               "events on the launch stream" % (total, units, chunk) if use_graph
+                                     else "one host launch per step",
+                                     "us_per_launch_fastest_unit": round(per_unit[0] * 1e6, 4),
+                                     "us_per_launch_slowest_unit": round(per_unit[-1] * 1e6, 4),
+                                     "host_clock_us_per_launch": round(host_ms_per_step * 1e3, 4)}}))
+        ctx.close()
+        return 0
 
     work = W["bytes"] / 1e9 if W["unit"] == "GB/s" else W["ops"] / 1e12
-    value = work / (ms_per_step * 1e-3)
+    value = work / s_per_step
     rwork = W["bytes"] / 1e9 if W["bound"] == "hbm" else W["ops"] / 1e12
-    achieved = rwork / ev_s_per_launch
+    achieved = rwork / s_per_step
 
+    launch = "%d repeats of the %d-step region back to back (%d steps), " % (repeats, steps, total)
+    launch += ("replayed as %d HIP graphs of %d steps" % (units, chunk) if use_graph
+               else "one host launch per step, %d units of %d steps" % (units, chunk))
+    launch += "; ms_per_step = the median unit by HIP events on the launch stream"
     result = {"metric": W["metric"], "value": round(value, 3), "unit": W["unit"], "n_gpus": 1, "steps": steps,
-              "warmup": warmup, "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak",
-              "vs_baseline": None, "dtype": W["dtype"], "data": "synthetic",
+              "warmup": warmup, "repeats": repeats, "ms_per_step": round(ms_per_step, 6), "higher_is_better": True,
+              "scaling": "weak", "vs_baseline": None, "dtype": W["dtype"], "data": "synthetic",
               "config": {"workload": W["workload"], "kernel": kernel, "ops_per_step": W["ops"],
-                         "algorithmic_bytes_per_step": W["bytes"], "graph_status": status,
-                         "launch": "HIP graph of %d steps, replayed %d times" % (chunk, steps // chunk) if use_graph
-                         else "one host launch per step"},
+                         "algorithmic_bytes_per_step": W["bytes"], "graph_status": status, "launch": launch,
+                         "ms_per_step_fastest_unit": round(per_unit[0] * 1e3, 6),
+                         "ms_per_step_slowest_unit": round(per_unit[-1] * 1e3, 6),
+                         "host_clock_ms_per_step_whole_region": round(host_ms_per_step, 6)},
               "roofline": {"bound": W["bound"], "achieved": round(achieved, 3), "peak": W["peak"], "unit": W["runit"],
                            "frac": round(achieved / W["peak"], 5), "traffic": MEASURED_TRAFFIC_BYTES.get(cfg),
-                           "us_per_launch": round(ev_s_per_launch * 1e6, 3)}}
+                           "us_per_launch": round(s_per_step * 1e6, 3)}}
     if W["bound"] == "hbm" and W["unit"] != "GB/s":
-        result["roofline"]["mfma_frac"] = round(W["ops"] / 1e12 / ev_s_per_launch / PEAK["int8_mfma"], 5)
+        result["roofline"]["mfma_frac"] = round(W["ops"] / 1e12 / s_per_step / PEAK["int8_mfma"], 5)
 
     rc = 0
     if not args.no_cpu_baseline:
-        # the oracle on one host core: repeated over the sample until about 10 s of CPU work have been timed
-        best, ref, spent, runs = None, None, 0.0, 0
-        while runs < 3 or (spent < 10.0 and runs < 400):
-            c0 = time.perf_counter()
-            ref = W["cpu_ref"]()
-            dt = time.perf_counter() - c0
-            best = dt if best is None else min(best, dt)
-            spent += dt
-            runs += 1
-            if best > 10.0:
-                break
         got = W["result"]()
+
+        def time_oracle(budget):
+            # repeated over the sample until about `budget` seconds of CPU work have been timed
+            best, ref, spent, runs = None, None, 0.0, 0
+            while runs < 3 or (spent < budget and runs < 400):
+                c0 = time.perf_counter()
+                ref = W["cpu_ref"]()
+                dt = time.perf_counter() - c0
+                best = dt if best is None else min(best, dt)
+                spent += dt
+                runs += 1
+                if best > budget:
+                    break
+            return best, ref, spent, runs
+
+        orc = the_oracle()
+        orc.set_parallel(False)
+        best, ref, spent, runs = time_oracle(10.0)
         if W["exact"]:
             ok = bool(np.array_equal(got, ref))
             result["config"]["bit_exact_vs_oracle"] = ok
@@ -390,14 +496,36 @@ def main() -> int:
             g64 = got.astype(np.float64)
             r64 = np.asarray(ref, np.float64)
             err = float(np.max(np.abs(g64 - r64) / np.maximum(np.abs(r64), 1e-3)))
-            ok = err < 2e-2  # sanity only: the DOT_PRODUCT-bound check against fp64 lives in the tests
+            ok = err < 2e-2  # sanity only: the figures against fp64 follow
             result["config"]["max_rel_err_vs_fp32_oracle"] = err
+            if "accuracy" in W:
+                acc = W["accuracy"]()
+                result["config"]["accuracy_vs_fp64"] = acc
+                ok = ok and acc["dot_product_compliant"]
         cpu_work = work * W["cpu_fraction"]
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                cpu_model = next(line.split(":", 1)[1].strip() for line in f if line.startswith("model name"))
+        except (OSError, StopIteration):
+            pass
+        sample = "whole batch" if W["cpu_fraction"] == 1.0 else "leading rows / first image"
         result["cpu_baseline"] = {"value": round(cpu_work / best, 6), "unit": W["unit"], "cores": 1, "kind": "port",
                                   "sample": "%.4g of one step's work (%s), fastest of %d runs of the scalar C oracle "
-                                            "(%.1f s of CPU work in all), %.2f s per run"
-                                            % (W["cpu_fraction"], "whole batch" if W["cpu_fraction"] == 1.0
-                                               else "leading rows / first image", runs, spent, best)}
+                                            "(%.1f s of CPU work in all), %.3f s per run"
+                                            % (W["cpu_fraction"], sample, runs, spent, best),
+                                  "cpu_model": cpu_model, "host_logical_cpus": os.cpu_count()}
+        if W.get("parallel_oracle"):
+            # the same C source built with OpenMP: the operator's outer loops over all the threads the host grants
+            orc.set_parallel(True)
+            threads = orc.threads()
+            pbest, pref, pspent, pruns = time_oracle(5.0)
+            orc.set_parallel(False)
+            same = bool(np.array_equal(np.asarray(pref), np.asarray(ref)))
+            result["cpu_baseline"]["all_cores"] = {
+                "value": round(cpu_work / pbest, 6), "unit": W["unit"], "cores": threads, "kind": "port",
+                "sample": "the same sample with the OpenMP build of the oracle on %d threads, fastest of %d runs, "
+                          "%.3f s per run; results identical to the scalar build: %s" % (threads, pruns, pbest, same)}
         if not ok:
             print("bench.py: GPU result differs from the oracle", file=sys.stderr)
             rc = 1

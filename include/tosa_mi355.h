@@ -390,6 +390,16 @@ int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
  * reference; used by the benchmark's launch-floor configuration. */
 int tmi_debug_launch_empty(tmi_ctx_t* ctx, int32_t grid, int32_t block, int32_t lds_bytes);
 
+/* Streams `bytes` bytes (a positive multiple of 16, buffers 16-byte aligned) on the context's stream: mode 0
+ * copies src to dst, mode 1 only reads src (dst receives nothing unless every word read is 0xFFFFFFFF; it must
+ * still be a valid 16-byte buffer), mode 2 only writes dst.  What the memory system sustains, to quote kernel
+ * rates against.  No counterpart in the reference. */
+int tmi_debug_stream(tmi_ctx_t* ctx, int32_t mode, const void* src_dev, void* dst_dev, int64_t bytes);
+
+/* Grid (workgroups), block (threads) and dynamic LDS bytes of the calling thread's latest launch of the CONV2D
+ * kernel that keeps a layer's operands in LDS; zeros before the first.  Feeds tmi_debug_launch_empty. */
+void tmi_debug_last_launch_shape(int32_t* out3);
+
 /* Host arithmetic only, no GPU call.  The tiled kernels split a block index into (channel block, tile column,
  * tile row, image) with multiply-high divisions that are exact while dividend * divisor < 2^32; a launcher
  * whose layer is outside that leaves the layer to another kernel.  Returns 1 if a grid of `grid` blocks with

@@ -56,6 +56,11 @@ def set_parallel(on: bool) -> None:
     _parallel = bool(on)
 
 
+def threads() -> int:
+    """host threads the selected build runs CONV2D / DEPTHWISE_CONV2D / MATMUL on"""
+    return int(lib().orc_threads())
+
+
 def lib() -> ctypes.CDLL:
     path = _LIB_OMP_PATH if _parallel else _LIB_PATH
     if path not in _libs:

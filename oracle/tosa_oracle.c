@@ -906,6 +906,20 @@ int orc_max_pool2d_f32(const orc_pool_shape_t* s, const float* in, int nan_mode,
  * OpClamp (reference_model/src/ops/activation_funcs.cpp:27-125) through applyClip
  * (reference_model/src/arith_util.h:389-413).
  * ---------------------------------------------------------------------------------------------- */
+/* threads the loops of this build run on: 1 for the scalar build, the OpenMP team size otherwise */
+#ifdef _OPENMP
+#include <omp.h>
+int orc_threads(void)
+{
+    return omp_get_max_threads();
+}
+#else
+int orc_threads(void)
+{
+    return 1;
+}
+#endif
+
 int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out)
 {
     if (hi < lo)

@@ -214,6 +214,7 @@ float orc_dp_bound_parameter(int data_kind, int acc16);
 int orc_dp_generate(int op, int set, int param, uint32_t ks, float B, const int32_t* shape, int rank,
                     const int32_t* kernel, float* out);
 
+int orc_threads(void);
 int orc_clamp_i32(int64_t n, const int32_t* in, int32_t lo, int32_t hi, int32_t* out);
 /* CLAMP for float storage; nan_mode 1 = PROPAGATE, 2 = IGNORE. */
 int orc_clamp_f32(int64_t n, const float* in, float lo, float hi, int nan_mode, float* out);

@@ -36,7 +36,7 @@ EXPORTS = [
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
     "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
     "tmi_ctx_reserve_workspace", "tmi_transpose_conv2d_noalloc", "tmi_ctx_set_level", "tmi_clamp_fp",
-    "tmi_debug_launch_empty", "tmi_debug_tile_decode",
+    "tmi_debug_launch_empty", "tmi_debug_tile_decode", "tmi_debug_last_launch_shape", "tmi_debug_stream",
 ]
 
 NOALLOC_SCRATCH_BYTES = 16 << 20  # TMI_NOALLOC_SCRATCH_BYTES
@@ -160,6 +160,9 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_clamp_fp.argtypes = [vp, i32, i64, vp, ctypes.c_float, ctypes.c_float, i32, vp]
     lib.tmi_ctx_set_level.argtypes = [vp, ctypes.POINTER(Level)]
     lib.tmi_debug_launch_empty.argtypes = [vp, i32, i32, i32]
+    lib.tmi_debug_last_launch_shape.argtypes = [ctypes.POINTER(ctypes.c_int32)]
+    lib.tmi_debug_last_launch_shape.restype = None
+    lib.tmi_debug_stream.argtypes = [vp, i32, vp, vp, i64]
     lib.tmi_debug_tile_decode.argtypes = [i64, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
                                           ctypes.POINTER(ctypes.c_int32)]
     lib.tmi_avg_pool2d.argtypes = [vp, ctypes.POINTER(PoolDesc), vp, i32, i32, vp]
@@ -386,6 +389,14 @@ class Context:
     def clamp_fp(self, dtype, n, inp, lo, hi, nan_mode, out) -> int:
         return self._check(self.lib.tmi_clamp_fp(self.handle, dtype, n, _ptr(inp), float(lo), float(hi), int(nan_mode),
                                                  _ptr(out)))
+
+    def stream_probe(self, mode, src, dst, nbytes) -> int:
+        return self._check(self.lib.tmi_debug_stream(self.handle, mode, _ptr(src), _ptr(dst), nbytes))
+
+    def last_launch_shape(self):
+        out = (ctypes.c_int32 * 3)()
+        self.lib.tmi_debug_last_launch_shape(out)
+        return tuple(out)
 
     def launch_empty(self, grid, block, lds_bytes) -> int:
         return self._check(self.lib.tmi_debug_launch_empty(self.handle, grid, block, lds_bytes))

@@ -445,6 +445,8 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     raise_flags(a.flag_word, flags);
 }
 
+thread_local int32_t last_launch_shape[3] = { 0, 0, 0 };
+
 template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
@@ -453,6 +455,7 @@ static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int 
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, st, a);
+    last_launch_shape[0] = grid, last_launch_shape[1] = 512, last_launch_shape[2] = lds_bytes;
     return true;
 }
 

@@ -365,6 +365,60 @@ const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t ld
 }
 
 // ------------------------------------------------------------------------------------------------
+// Streaming probes: what the memory system sustains for a plain copy, a read-only and a write-only pass over
+// `vecs` 16-byte vectors.  Each workgroup walks the buffer with a grid stride, four vectors per lane and step.
+// MODE 0 = copy, 1 = read only (the lanes fold what they read and store it only if it has a value the fold
+// cannot take, so the loads stay), 2 = write only.
+// ------------------------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_probe_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                           int64_t vecs, uint32_t fill)
+{
+    const int64_t stride = (int64_t)gridDim.x * 256 * 4;
+    uint32_t fold        = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 * 4 + threadIdx.x; i < vecs; i += stride)
+    {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (MODE != 2 && i + u * 256 < vecs)
+                v[u] = __builtin_nontemporal_load(src + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+        {
+            if (i + u * 256 >= vecs)
+                continue;
+            if (MODE == 1)
+                fold |= (v[u].x & v[u].y & v[u].z & v[u].w) >> 31 | (v[u].x ^ v[u].y ^ v[u].z ^ v[u].w) << 1;
+            else
+                __builtin_nontemporal_store(MODE == 0 ? v[u] : u32x4{ fill, fill, fill, fill }, dst + i + u * 256);
+        }
+    }
+    if (MODE == 1 && fold == fill)    // the caller passes a value the fold of its data never takes
+        dst[0] = u32x4{ fold, fold, fold, fold };
+}
+
+const char* launch_stream_probe(hipStream_t st, int32_t mode, const void* src, void* dst, int64_t bytes)
+{
+    if (bytes < 16 || (bytes & 15) || (((uintptr_t)src | (uintptr_t)dst) & 15) || !dst || (mode != 2 && !src))
+        return nullptr;
+    const int64_t vecs = bytes / 16;
+    const int64_t wgs  = (vecs + 1023) / 1024;
+    const int grid     = (int)(wgs < 256 * 16 ? wgs : 256 * 16);
+    if (mode == 0)
+        hipLaunchKernelGGL(stream_probe_kernel<0>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0u);
+    else if (mode == 1)
+        hipLaunchKernelGGL(stream_probe_kernel<1>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0xFFFFFFFFu);
+    else if (mode == 2)
+        hipLaunchKernelGGL(stream_probe_kernel<2>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0x01010101u);
+    else
+        return nullptr;
+    return mode == 0 ? "stream_copy" : (mode == 1 ? "stream_read" : "stream_write");
+}
+
+// ------------------------------------------------------------------------------------------------
 // Batched transpose [N, R, C] -> [N, C, R] through a padded 64x64 LDS tile: rows are read and written as
 // contiguous runs along the fastest dimension of their side.
 // ------------------------------------------------------------------------------------------------

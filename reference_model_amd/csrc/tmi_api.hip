@@ -594,6 +594,24 @@ int tmi_debug_launch_empty(tmi_ctx_t* ctx, int32_t grid, int32_t block, int32_t 
     return after_launch(ctx, name);
 }
 
+int tmi_debug_stream(tmi_ctx_t* ctx, int32_t mode, const void* src_dev, void* dst_dev, int64_t bytes)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    const char* name = launch_stream_probe(ctx->stream, mode, src_dev, dst_dev, bytes);
+    if (!name)
+        return fail(ctx, "tmi_debug_stream: mode %d with %lld bytes: the mode is 0..2, the buffers are 16-byte aligned and "
+                         "the size is a positive multiple of 16", mode, (long long)bytes);
+    return after_launch(ctx, name);
+}
+
+void tmi_debug_last_launch_shape(int32_t* out3)
+{
+    if (out3)
+        out3[0] = last_launch_shape[0], out3[1] = last_launch_shape[1], out3[2] = last_launch_shape[2];
+}
+
 int tmi_debug_tile_decode(int64_t grid, uint32_t n_ocb, uint32_t tiles_x, uint32_t tiles_y, uint32_t block,
                           int32_t* out4)
 {

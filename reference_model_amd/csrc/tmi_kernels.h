@@ -82,6 +82,11 @@ const char* launch_clamp(hipStream_t st, int32_t dtype, const void* in, void* ou
                          int32_t hi);
 const char* launch_clamp_fp(hipStream_t st, int32_t dtype, const void* in, void* out, int64_t n, float lo, float hi,
                             int32_t nan_mode);
+// copy (mode 0), read-only (1) or write-only (2) pass over `bytes` bytes: what the memory system sustains
+const char* launch_stream_probe(hipStream_t st, int32_t mode, const void* src, void* dst, int64_t bytes);
+// grid, block and dynamic LDS bytes of this thread's latest launch of the kernel that loads a CONV2D layer's
+// operands straight into LDS (zeros before the first)
+extern thread_local int32_t last_launch_shape[3];
 // a kernel without work: the cost of one launch of this grid, block and dynamic LDS size
 const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t lds_bytes);
 

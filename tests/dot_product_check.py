@@ -67,13 +67,20 @@ def check(imp: np.ndarray, ref: np.ndarray, bnd: np.ndarray, out_type: str, ksb:
     ok = not bool(failed.any()) and sumsq <= var_bound * T
     if 3 <= set_number <= 5:
         ok = ok and abs(err_sum) <= math.sqrt(10 * var_bound * T)
-    # ULP and relative error as the reference's ULP verifier defines them (verify_ulp.cpp:27-47)
-    fin = np.isfinite(ref) & np.isfinite(imp)
+    # ULP as the reference's ULP verifier defines it (verify_ulp.cpp:27-47: the unit is the last bit at the power of
+    # two of |ref|, not below normal_min; a zero reference has no ULP), the relative error, and the error relative
+    # to the bound tensor (the sum of the absolute products, the scale the DOT_PRODUCT check itself uses)
+    fin = np.isfinite(ref) & np.isfinite(imp) & (ref != 0.0)
     with np.errstate(invalid="ignore", divide="ignore"):
         mag = np.maximum(2.0 ** np.floor(np.log2(np.maximum(np.abs(ref[fin]), 1e-300))), NORMAL_MIN[out_type])
         ulp = np.abs(imp[fin] - ref[fin]) / (mag * 2.0 ** (-frac))
         nz = np.abs(ref[fin]) > 0
         rel = np.abs(imp[fin] - ref[fin])[nz] / np.abs(ref[fin])[nz]
-    return dict(ok=bool(ok), max_err=max_err, abs_bound=abs_bound, err_sum=err_sum, err_sumsq=sumsq,
+        # elements without cancellation worth speaking of: |ref| at least an eighth of the sum of absolute products
+        cond = np.abs(ref[fin]) >= bnd[fin] / 8
+        pos = fin & (bnd > 0)
+        to_bound = np.abs(imp[pos] - ref[pos]) / bnd[pos]
+    return dict(ok=bool(ok), max_rel_to_bound=float(to_bound.max()) if to_bound.size else 0.0, max_err=max_err, abs_bound=abs_bound, err_sum=err_sum, err_sumsq=sumsq,
                 var_limit=var_bound * T, failed_elements=int(failed.sum()),
-                max_ulp=float(ulp.max()) if ulp.size else 0.0, max_rel=float(rel.max()) if rel.size else 0.0)
+                max_ulp=float(ulp.max()) if ulp.size else 0.0,
+                max_ulp_conditioned=float(ulp[cond].max()) if cond.any() else 0.0, max_rel=float(rel.max()) if rel.size else 0.0)

@@ -254,3 +254,59 @@ def test_fp32_conv_and_matmul_compliance_on_the_device(ctx, data_set):
     finally:
         for t in list(ctx._owned):
             ctx._free(t)
+
+
+def test_benchmark_fp16_conv_and_bf16_matmul_errors_at_full_size(ctx):
+    """The two floating-point benchmark configurations on the benchmark's own operands, at full size, against the
+    library's fp64 pass over the same operands (itself bit-equal to the fp64 oracle on the small cases above):
+    the DOT_PRODUCT check, the largest error in ULPs of the output type as the reference's ULP verifier defines
+    the unit (verify_ulp.cpp:27-47), the largest relative error, and the largest error relative to the sum of the
+    absolute products.  Measured on MI355X: fp16 CONV2D 14.7 ULP over all elements, 0.50 ULP where the result is
+    at least an eighth of that sum (the rounding of the fp32 sum to fp16 and nothing else), 7.3e-5 of the sum; bf16
+    MATMUL to fp32 3.8 ULP on those elements and 1.5e-7 of the sum (over all elements 2.3e8 ULP and a relative error of
+    16: results of 1e-7 against a sum of absolute products of 50).  An element whose products
+    cancel has an error of many ULPs of its small result whatever the accumulation order, so the asserted limits
+    are on the well-conditioned elements and on the error relative to the sum, with headroom of about two."""
+    c = cases.c5_conv()
+    n, ih, iw, ic = c["x"].shape
+    oc, kh, kw, _ = c["w"].shape
+    d = ctx.conv_desc(capi.FP16, capi.FP16, c["x"].shape, oc, kh, kw, (ih, iw), c["pad"], c["stride"], c["dilation"], oc)
+    try:
+        tx, tw, tb = ctx.upload(c["x"], capi.FP16), ctx.upload(c["w"], capi.FP16), ctx.upload(c["bias"], capi.FP16)
+        shape = (n, ih, iw, oc)
+        imp, ref, bnd = ctx.empty(shape, capi.FP16), ctx.empty(shape, capi.F64), ctx.empty(shape, capi.F64)
+        ctx.conv2d(d, tx, tw, tb, 0, 0, imp)
+        assert ctx.last_kernel == "gemm_mfma_f16"
+        ctx.conv2d_precise(d, tx, tw, tb, False, ref)
+        ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
+        ksb = dp.kernel_size_bound(kh * kw * ic, "fp16")
+        r = ctx.dot_product_check(capi.FP16, int(np.prod(shape)), imp, ref, bnd, ksb)
+        assert ctx.sync() == capi.VALID and r.compliant
+        st = dp.check(imp.numpy(), ref.numpy(), bnd.numpy(), "fp16", ksb)
+        print("fp16 CONV2D [16,28,28,256]x[256,3,3,256]:", st)
+        assert st["ok"] and st["max_ulp"] <= 32 and st["max_ulp_conditioned"] <= 1.0
+        assert st["max_rel_to_bound"] <= 2.0 ** -12          # half an fp16 ULP of the sum of absolute products
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)
+
+    m = cases.c5_matmul()
+    nb, h, k = m["a"].shape
+    w = m["b"].shape[2]
+    try:
+        ta, tb = ctx.upload(m["a"], capi.BF16), ctx.upload(m["b"], capi.BF16)
+        imp, ref, bnd = ctx.empty((nb, h, w), capi.FP32), ctx.empty((nb, h, w), capi.F64), ctx.empty((nb, h, w), capi.F64)
+        ctx.matmul(capi.BF16, nb, h, k, w, ta, tb, 0, 0, imp)
+        assert ctx.last_kernel == "matmul_gemm_bf16"
+        ctx.matmul_precise(capi.BF16, nb, h, k, w, ta, tb, False, ref)
+        ctx.matmul_precise(capi.BF16, nb, h, k, w, ta, tb, True, bnd)
+        ksb = dp.kernel_size_bound(k, "fp32", has_bias=False)
+        r = ctx.dot_product_check(capi.FP32, nb * h * w, imp, ref, bnd, ksb)
+        assert ctx.sync() == capi.VALID and r.compliant
+        st = dp.check(imp.numpy(), ref.numpy(), bnd.numpy(), "fp32", ksb)
+        print("bf16 MATMUL [4,2048,4096]x[4,4096,2048]:", st)
+        assert st["ok"] and st["max_ulp_conditioned"] <= 8
+        assert st["max_rel_to_bound"] <= 2.0 ** -21           # four fp32 ULPs of the sum of absolute products
+    finally:
+        for t in list(ctx._owned):
+            ctx._free(t)

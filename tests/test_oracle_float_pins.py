@@ -128,3 +128,30 @@ def test_conv2d_f64_bounds_pass_without_local_bound(pad, stride, dilation):
     if pad == (1, 1, 1, 1) and stride == (1, 1):
         patch = np.abs(x[0, 2:5, 3:6, :])
         assert abs(local[0, 3, 4, 1] - (np.einsum("yxc,yxc->", patch, np.abs(w[1])) + abs(bias[1]))) < 1e-12
+
+
+def test_float_clamp_against_numpy_and_the_nan_rules():
+    """activation_funcs.cpp:97-106 over applyClip (arith_util.h:390-413): max with min_val, then min with max_val;
+    a NaN input stays NaN under PROPAGATE (1) and becomes min_val under IGNORE (2): applyMax(NaN, min) = min, and
+    applyMin(min, max) = min"""
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.normal(0, 3, 1000), [np.inf, -np.inf, 0.0, -0.0, 1.0, -1.0]]).astype(np.float32)
+    for lo, hi in ((-1.0, 1.0), (0.0, 6.0), (-np.inf, np.inf), (2.5, 2.5)):
+        for mode in (1, 2):
+            assert np.array_equal(oracle.clamp(x, lo, hi, mode), np.clip(x, np.float32(lo), np.float32(hi)))
+    xn = np.array([np.nan, 0.5, -7.0, np.nan, 9.0], np.float32)
+    got = oracle.clamp(xn, -1.0, 2.0, 1)
+    assert np.isnan(got[[0, 3]]).all() and np.array_equal(got[[1, 2, 4]], np.array([0.5, -1.0, 2.0], np.float32))
+    assert np.array_equal(oracle.clamp(xn, -1.0, 2.0, 2), np.array([-1.0, 0.5, -1.0, -1.0, 2.0], np.float32))
+    # the comparisons are (a >= min) ? a : min and (a < max) ? a : max: an input zero of either sign is kept when it
+    # equals min, and replaced by max's own zero when it equals max
+    z = oracle.clamp(np.array([-0.0, 0.0], np.float32), 0.0, 1.0, 1)
+    assert np.signbit(z[0]) and not np.signbit(z[1])
+    z = oracle.clamp(np.array([-0.0, 0.0], np.float32), -1.0, 0.0, 1)
+    assert not np.signbit(z[0]) and not np.signbit(z[1])
+    # half-precision storage: the result of clamping representable values to representable limits is representable
+    h = rng.normal(0, 3, 500).astype(np.float16)
+    assert np.array_equal(oracle.clamp(h, -1.5, 2.25, 1), np.clip(h, np.float16(-1.5), np.float16(2.25)))
+    for bad in ((1.0, 0.0), (np.nan, 1.0), (0.0, np.nan)):
+        with pytest.raises(oracle.OracleStatus):
+            oracle.clamp(x, bad[0], bad[1], 1)
