@@ -117,7 +117,8 @@ def main() -> int:
         src = torch.zeros(nbytes, dtype=torch.int8, device=dev)
         dst = torch.empty_like(src)
         out = {"metric": "streaming rates of the box", "unit": "GB/s", "bytes": nbytes}
-        for mode, name, moved in ((0, "copy", 2 * nbytes), (1, "read", nbytes), (2, "write", nbytes)):
+        for mode, name, moved in ((0, "copy", 2 * nbytes), (1, "read", nbytes), (2, "write", nbytes),
+                                  (3, "read_into_lds", nbytes)):
             n_steps = args.steps or 20
             for _ in range(3):
                 ctx.stream_probe(mode, src, dst, nbytes)

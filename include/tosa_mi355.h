@@ -392,7 +392,7 @@ int tmi_debug_launch_empty(tmi_ctx_t* ctx, int32_t grid, int32_t block, int32_t 
 
 /* Streams `bytes` bytes (a positive multiple of 16, buffers 16-byte aligned) on the context's stream: mode 0
  * copies src to dst, mode 1 only reads src (dst receives nothing unless every word read is 0xFFFFFFFF; it must
- * still be a valid 16-byte buffer), mode 2 only writes dst.  What the memory system sustains, to quote kernel
+ * still be a valid 16-byte buffer), mode 2 only writes dst, mode 3 reads src with loads that go straight into LDS.  What the memory system sustains, to quote kernel
  * rates against.  No counterpart in the reference. */
 int tmi_debug_stream(tmi_ctx_t* ctx, int32_t mode, const void* src_dev, void* dst_dev, int64_t bytes);
 

@@ -60,8 +60,87 @@ __global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, co
 // The common RESCALE -- signed INT32 in (no input zero point), 32-bit multipliers, SINGLE or DOUBLE rounding,
 // C a multiple of 4 -- with the per-channel constants in registers: a lane owns 4 consecutive channels and
 // walks down the rows, so multiplier, shift and the 64-bit rounding terms (output zero point folded in) are
-// derived once and an element costs ~9 instructions.  Four rows are in flight per lane.
+// derived once.  A workgroup visits `rpi` rows at a time (a unit); its units are blockIdx, blockIdx + grid, ...
+// Four units are in flight per lane: the load of unit k + 4 is issued as soon as unit k has been converted, so
+// the loads of a wave never drain while it computes.
+//
+// HW: every channel of the wave has a shift of at least 32 (33 with double rounding) that also lets the output
+// zero point ride in the rounding term: the result is the high word of value * multiplier + R shifted by
+// shift - 32, with R's sign-dependent part (double rounding) patched into the addend - no 64-bit shift and no
+// range test, which cannot fire for such shifts.
 typedef int rs_v4i __attribute__((ext_vector_type(4)));
+
+struct RescaleLane
+{
+    int32_t mul[4], sh[4], zp_post[4], hw_hi[4];
+    uint32_t lim[4], hw_lo[4];
+    int64_t rnd_pos[4], rnd_neg[4];
+    bool check;
+};
+
+template <typename OutT, bool HW, bool DR>
+__device__ __forceinline__ void rescale_store_row(const RescaleParams& p, const RescaleLane& k, rs_v4i v, OutT* q,
+                                                  uint32_t& flags)
+{
+    int32_t res[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+    {
+        const int32_t x = v[c];
+        int32_t o;
+        if constexpr (HW)
+            o = high_word_rescale<DR>(x, k.mul[c], k.hw_hi[c], k.hw_lo[c], k.sh[c]);
+        else
+        {
+            if (k.check && (uint32_t)x + k.lim[c] > 2u * k.lim[c] - 1u)
+                flags |= TMI_FLAG_SCALE_VALUE;
+            const int64_t pr = (int64_t)x * (int64_t)k.mul[c] + (x >= 0 ? k.rnd_pos[c] : k.rnd_neg[c]);
+            o                = (int32_t)(pr >> k.sh[c]) + k.zp_post[c];
+        }
+        o      = o < p.lo ? p.lo : o;
+        res[c] = o > p.hi ? p.hi : o;
+    }
+    if constexpr (sizeof(OutT) == 1)
+        *reinterpret_cast<int*>(q) = (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) | ((res[3] & 0xff) << 24);
+    else if constexpr (sizeof(OutT) == 2)
+    {
+        reinterpret_cast<int*>(q)[0] = (res[0] & 0xffff) | ((res[1] & 0xffff) << 16);
+        reinterpret_cast<int*>(q)[1] = (res[2] & 0xffff) | ((res[3] & 0xffff) << 16);
+    }
+    else
+        *reinterpret_cast<rs_v4i*>(q) = rs_v4i{ res[0], res[1], res[2], res[3] };
+}
+
+template <typename OutT, bool HW, bool DR>
+__device__ __forceinline__ void rescale_walk(const RescaleParams& p, const RescaleLane& k, const int32_t* __restrict__ in,
+                                             OutT* __restrict__ out, int64_t rows, int32_t C, int32_t rpi, int slot,
+                                             int c0, bool lane_on, uint32_t& flags)
+{
+    constexpr int U    = 4;
+    const int64_t step = (int64_t)gridDim.x * rpi;    // rows between two units of a workgroup
+    int64_t r          = (int64_t)blockIdx.x * rpi + slot;
+    rs_v4i v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+    {
+        const int64_t ru = r + u * step;
+        v[u]             = *reinterpret_cast<const rs_v4i*>(in + ((lane_on && ru < rows) ? ru * C + c0 : 0));
+    }
+    // every lane of the workgroup runs the same number of rounds: the loads of a round are issued by all
+    for (int64_t base = (int64_t)blockIdx.x * rpi; base < rows; base += U * step, r += U * step)
+    {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+        {
+            const int64_t ru  = r + u * step;
+            const rs_v4i cur  = v[u];
+            const int64_t nxt = ru + U * step;
+            v[u]              = *reinterpret_cast<const rs_v4i*>(in + ((lane_on && nxt < rows) ? nxt * C + c0 : 0));
+            if (lane_on && ru < rows)
+                rescale_store_row<OutT, HW, DR>(p, k, cur, out + ru * C + c0, flags);
+        }
+    }
+}
 
 template <typename OutT>
 __global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, const int32_t* __restrict__ in,
@@ -69,74 +148,46 @@ __global__ __launch_bounds__(256) void rescale_fast_kernel(RescaleParams p, cons
                                                            int32_t cgs, int32_t rpi, FastDiv div_cgs,
                                                            uint32_t* flag_word)
 {
-    const int tid  = threadIdx.x;
-    const int slot = fdiv(tid, div_cgs);    // row slot of this lane inside an iteration
+    const int tid      = threadIdx.x;
+    const int slot     = fdiv(tid, div_cgs);    // row slot of this lane inside a unit
     const bool lane_on = slot < rpi;
-    const int c0   = lane_on ? (tid - slot * cgs) * 4 : 0;
-    uint32_t flags = 0;
-    int32_t mul[4], sh[4], zp_post[4];
-    uint32_t lim[4];
-    int64_t rnd_pos[4], rnd_neg[4];
-    bool check = false;
+    const int c0       = lane_on ? (tid - slot * cgs) * 4 : 0;
+    uint32_t flags     = 0;
+    RescaleLane k;
+    k.check    = false;
+    bool hw_ok = true;
+    const int max_fold = zp_fold_max_shift(p.out_zp);
 #pragma unroll
     for (int c = 0; c < 4; c++)
     {
         const int i = p.per_channel ? c0 + c : 0;
         const ChannelScale cs =
             make_channel_scale(reinterpret_cast<const int32_t*>(p.multiplier)[i], (int32_t)p.shift[i], p.double_round, flags);
-        const bool fold       = cs.s <= zp_fold_max_shift(p.out_zp);    // else output_zp is added after the shift
+        const bool fold       = cs.s <= max_fold;    // else output_zp is added after the shift
         const int64_t zp_term = fold ? ((int64_t)p.out_zp << cs.s) : 0;
-        zp_post[c]            = fold ? 0 : p.out_zp;
-        mul[c] = cs.m, sh[c] = cs.s, lim[c] = cs.lim;
-        rnd_pos[c] = cs.rnd_pos + zp_term, rnd_neg[c] = cs.rnd_neg + zp_term;
-        check |= cs.lim != 0x80000000u;
+        k.zp_post[c]          = fold ? 0 : p.out_zp;
+        k.mul[c] = cs.m, k.lim[c] = cs.lim;
+        k.rnd_pos[c] = cs.rnd_pos + zp_term, k.rnd_neg[c] = cs.rnd_neg + zp_term;
+        k.check |= cs.lim != 0x80000000u;
+        hw_ok &= fold && cs.s >= (p.double_round ? 33 : 32) && flags == 0;
+        const HighWordScale h = make_high_word_scale(cs, p.out_zp);
+        k.hw_hi[c] = h.hi, k.hw_lo[c] = h.lo;
+        k.sh[c] = cs.s;
     }
     if (!lane_on)
-        flags = 0;
-    constexpr int U = 4;
-    const int64_t step = (int64_t)gridDim.x * rpi;    // rows between two visits of a lane
-    for (int64_t r0 = (int64_t)blockIdx.x * rpi + slot; r0 < rows; r0 += U * step)
+        flags = 0, hw_ok = true;
+    if (__all(hw_ok))
     {
-        rs_v4i v[U];
 #pragma unroll
-        for (int u = 0; u < U; u++)
-        {
-            const int64_t r = r0 + u * step;
-            const bool on   = lane_on && r < rows;
-            v[u]            = *reinterpret_cast<const rs_v4i*>(in + (on ? r * C + c0 : 0));
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-        {
-            const int64_t r = r0 + u * step;
-            const bool on   = lane_on && r < rows;
-            int32_t res[4];
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-            {
-                const int32_t x = v[u][c];
-                if (check && on && (uint32_t)x + lim[c] > 2u * lim[c] - 1u)
-                    flags |= TMI_FLAG_SCALE_VALUE;
-                const int64_t pr = (int64_t)x * (int64_t)mul[c] + (x >= 0 ? rnd_pos[c] : rnd_neg[c]);
-                int32_t o        = (int32_t)(pr >> sh[c]) + zp_post[c];
-                o                = o < p.lo ? p.lo : o;
-                res[c]           = o > p.hi ? p.hi : o;
-            }
-            if (!on)
-                continue;
-            OutT* q = out + r * C + c0;
-            if constexpr (sizeof(OutT) == 1)
-                *reinterpret_cast<int*>(q) =
-                    (res[0] & 0xff) | ((res[1] & 0xff) << 8) | ((res[2] & 0xff) << 16) | ((res[3] & 0xff) << 24);
-            else if constexpr (sizeof(OutT) == 2)
-            {
-                reinterpret_cast<int*>(q)[0] = (res[0] & 0xffff) | ((res[1] & 0xffff) << 16);
-                reinterpret_cast<int*>(q)[1] = (res[2] & 0xffff) | ((res[3] & 0xffff) << 16);
-            }
-            else
-                *reinterpret_cast<rs_v4i*>(q) = rs_v4i{ res[0], res[1], res[2], res[3] };
-        }
+        for (int c = 0; c < 4; c++)
+            k.sh[c] -= 32;
+        if (p.double_round)
+            rescale_walk<OutT, true, true>(p, k, in, out, rows, C, rpi, slot, c0, lane_on, flags);
+        else
+            rescale_walk<OutT, true, false>(p, k, in, out, rows, C, rpi, slot, c0, lane_on, flags);
     }
+    else
+        rescale_walk<OutT, false, false>(p, k, in, out, rows, C, rpi, slot, c0, lane_on, flags);
     raise_flags(flag_word, flags);
 }
 
@@ -144,12 +195,16 @@ template <typename OutT>
 static const char* launch_rescale_fast(hipStream_t st, const RescaleParams& p, const void* in, void* out, int64_t n,
                                        int32_t C, uint32_t* flag_word)
 {
-    const int32_t cgs  = C / 4;
-    const int32_t rpi  = 256 / cgs;
-    const int64_t rows = n / C;
-    int64_t blocks     = (rows + (int64_t)rpi * 4 - 1) / ((int64_t)rpi * 4);    // four rows per lane and visit
-    if (blocks > 256 * 8)
-        blocks = 256 * 8;
+    const int32_t cgs   = C / 4;
+    const int32_t rpi   = 256 / cgs;
+    const int64_t rows  = n / C;
+    const int64_t units = (rows + rpi - 1) / rpi;
+    // Two workgroups per CU, each with four 16-byte loads in flight per lane, stream faster than more workgroups
+    // do (measured on [64,56,56,64]: 12.0 us with 2 per CU, 13.4 with 4, 14.8 with 8, 16.2 with 16; the arithmetic
+    // is not what limits it: without it the same walk takes 11.5 us); and as many units for one workgroup as for
+    // any other where that is possible
+    const int64_t visits = (units + 256 * 2 - 1) / (256 * 2);
+    int64_t blocks       = (units + visits - 1) / visits;
     if (blocks < 1)
         blocks = 1;
     hipLaunchKernelGGL((rescale_fast_kernel<OutT>), dim3((int)blocks), dim3(256), 0, st, p, (const int32_t*)in,
@@ -400,9 +455,31 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(const u32x4* __restri
         dst[0] = u32x4{ fold, fold, fold, fold };
 }
 
+// MODE 3 of the probe: the same read-only pass with loads that go straight into LDS (global_load_lds_dwordx4), which
+// is how the convolution kernels fetch their patches
+__global__ __launch_bounds__(256) void stream_probe_lds_kernel(const u32x4* __restrict__ src, int64_t vecs)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char probe_lds[];
+    const int wave       = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t lbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)probe_lds) + wave * 8192;
+    const int64_t stride = (int64_t)gridDim.x * 256 * 4;
+    int slot             = 0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 * 4 + threadIdx.x; i + 3 * 256 < vecs; i += stride)
+    {
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+        {
+            const u32x4* p = src + i + u * 256;
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(p), "s"(__builtin_amdgcn_readfirstlane(lbase + slot * 1024)) : "memory");
+            slot = (slot + 1) & 7;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 const char* launch_stream_probe(hipStream_t st, int32_t mode, const void* src, void* dst, int64_t bytes)
 {
-    if (bytes < 16 || (bytes & 15) || (((uintptr_t)src | (uintptr_t)dst) & 15) || !dst || (mode != 2 && !src))
+    if (bytes < 16 || (bytes & 15) || (((uintptr_t)src | (uintptr_t)dst) & 15) || !dst || (mode != 2 && !src) || mode < 0 || mode > 3)
         return nullptr;
     const int64_t vecs = bytes / 16;
     const int64_t wgs  = (vecs + 1023) / 1024;
@@ -411,11 +488,13 @@ const char* launch_stream_probe(hipStream_t st, int32_t mode, const void* src, v
         hipLaunchKernelGGL(stream_probe_kernel<0>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0u);
     else if (mode == 1)
         hipLaunchKernelGGL(stream_probe_kernel<1>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0xFFFFFFFFu);
+    else if (mode == 3)
+        hipLaunchKernelGGL(stream_probe_lds_kernel, dim3(grid), dim3(256), 32768, st, (const u32x4*)src, vecs);
     else if (mode == 2)
         hipLaunchKernelGGL(stream_probe_kernel<2>, dim3(grid), dim3(256), 0, st, (const u32x4*)src, (u32x4*)dst, vecs, 0x01010101u);
     else
         return nullptr;
-    return mode == 0 ? "stream_copy" : (mode == 1 ? "stream_read" : "stream_write");
+    return mode == 0 ? "stream_copy" : (mode == 1 ? "stream_read" : (mode == 2 ? "stream_write" : "stream_read_lds"));
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -601,7 +601,7 @@ int tmi_debug_stream(tmi_ctx_t* ctx, int32_t mode, const void* src_dev, void* ds
     TMI_HIP(ctx, hipSetDevice(ctx->device));
     const char* name = launch_stream_probe(ctx->stream, mode, src_dev, dst_dev, bytes);
     if (!name)
-        return fail(ctx, "tmi_debug_stream: mode %d with %lld bytes: the mode is 0..2, the buffers are 16-byte aligned and "
+        return fail(ctx, "tmi_debug_stream: mode %d with %lld bytes: the mode is 0..3, the buffers are 16-byte aligned and "
                          "the size is a positive multiple of 16", mode, (long long)bytes);
     return after_launch(ctx, name);
 }

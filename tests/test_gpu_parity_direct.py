@@ -40,6 +40,46 @@ def test_rescale_i32_to_i8_per_channel(ctx, shape, mode):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("shape", [(3000, 64), (517, 96), (100003, 8), (33, 1024), (70000, 4), (9, 7, 11, 32)])
+@pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
+@pytest.mark.parametrize("shifts", ["high", "mixed", "edge32", "low"])
+@pytest.mark.parametrize("out_dt,out_zp", [(np.int8, -128), (np.int8, 17), (np.int16, 0), (np.int32, 0)])
+def test_rescale_i32_register_resident_kernel_in_every_form(ctx, shape, mode, shifts, out_dt, out_zp):
+    """signed int32 -> int8 / int16 / int32 with C a multiple of 4 goes through the kernel that keeps the channel
+    constants in registers; it takes the high word of the product when every shift of a wave is at least 32 (33
+    with double rounding) and the 64-bit form otherwise.  Values span the whole int32 range where the shift allows
+    and sit at the rounding boundaries."""
+    rng = np.random.default_rng((hash(shape) ^ len(shifts) ^ mode) & 0xFFFF)
+    C = shape[-1]
+    lo_s, hi_s = {"high": (33, 47), "mixed": (28, 40), "edge32": (32, 34), "low": (20, 31)}[shifts]
+    shift = rng.integers(lo_s, hi_s, C).astype(np.int8)
+    mult = rng.integers(1 << 30, 1 << 31, C).astype(np.int32)
+    mult[rng.integers(0, C)] = 0
+    mag = 31 if lo_s >= 32 else lo_s - 2          # |value| < 2^(shift - 1) keeps the reference's range test quiet
+    x = rng.integers(-(1 << mag), 1 << mag, shape, dtype=np.int64)
+    x.flat[:4] = [-(1 << mag), (1 << mag) - 1, 0, -1]
+    x = x.astype(np.int32)
+    want, wst = oracle.rescale(x, mult, shift, out_zp=out_zp, out_dtype=out_dt, rounding_mode=mode)
+    got, st = gpu_ops.rescale(ctx, x, mult, shift, out_zp=out_zp, out_dtype=out_dt, rounding_mode=mode)
+    assert st == wst == capi.VALID and ctx.last_kernel == "rescale_fast"
+    assert np.array_equal(got, want)
+
+
+def test_rescale_i32_register_resident_kernel_flags_out_of_range_values(ctx):
+    """a value at or beyond 2^(shift - 1) in magnitude fails the reference's REQUIRE (quant_util.h:56-60): the graph
+    result is UNPREDICTABLE, on the 64-bit form of the kernel (shifts below 32)"""
+    rng = np.random.default_rng(8)
+    x = rng.integers(-(1 << 20), 1 << 20, (500, 16)).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, 16).astype(np.int32)
+    shift = np.full(16, 24, np.int8)
+    _, st = gpu_ops.rescale(ctx, x, mult, shift)
+    assert st == capi.VALID
+    x[321, 5] = 1 << 23
+    _, st = gpu_ops.rescale(ctx, x, mult, shift)
+    _, wst = oracle.rescale(x, mult, shift)
+    assert st == wst == capi.UNPREDICTABLE
+
+
 @pytest.mark.parametrize("in_dt,out_dt,in_u,out_u,in_zp,out_zp", [
     (np.int8, np.int8, False, False, -5, 9), (np.int8, np.int16, False, False, 3, 0),
     (np.int8, np.int32, False, False, 0, 0), (np.int16, np.int8, False, False, 0, -128),
