@@ -334,7 +334,8 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     const int oy = oy0 + ty, ox = ox0 + tx;
     const bool pix_ok  = p_in_tile && wave_active && oy < a.OH && ox < a.OW;
     const bool chan_ok = oc0 + ocl < a.OC;    // OC is a multiple of 16: a lane's 16 channels are in or out together
-    const size_t obase = (((size_t)n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl;
+    // the tensor has fewer than 2^31 elements (checked by the launcher): 32-bit arithmetic, scalar where it can be
+    const size_t obase = (uint32_t)(((n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl);
     if constexpr (!FUSED)
     {
         if (pix_ok && chan_ok)

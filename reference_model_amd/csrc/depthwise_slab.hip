@@ -185,9 +185,10 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
         {
             tab_m[tid] = m;
             tab_b[tid] = t_bias - (ZA ? a.za * wsum : 0);
+            int32_t* wp = wtab + tid;
 #pragma unroll
-            for (int t = 0; t < TAPS; t++)
-                wtab[t * C + tid] = ((int)t_w[t] & 0xff) * 0x01010101;
+            for (int t = 0; t < TAPS; t++, wp += C)    // byte 0 in all four bytes: one permute, no multiply
+                *wp = __builtin_amdgcn_perm((int)t_w[t], (int)t_w[t], 0x04040404);
         }
         else
             flags = 0;    // lanes without a channel report nothing
@@ -223,7 +224,11 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
         // zero rows).
         const int c          = c0 + wr;
         const int32_t* wcol  = wtab + (c < C ? c : 0);
-        const uint8_t* prow  = pl + (ty * a.sy * a.pitch + tx * a.sx * a.ppitch) * 16 + c0 + lh * 16;
+        // the nine tap addresses are this one plus scalars; kept opaque so that the products are not redistributed
+        // over the taps (a 32-bit vector multiply runs at a quarter of the rate)
+        uint32_t pbase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)pl +
+                         (uint32_t)((ty * a.sy * a.pitch + tx * a.sx * a.ppitch) * 16 + c0 + lh * 16);
+        asm volatile("" : "+v"(pbase));
         // (lane, register e) = channel c0 + 16 lh + e of pixel li; the accumulators start at the channel's bias term
         const int cl  = c0 + 16 * lh;
         const int clc = cl < C ? cl : 0;    // C is a multiple of 16
@@ -241,7 +246,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
             wv[t] = wcol[t * C];
 #pragma unroll
         for (int t = 0; t < TAPS; t++)
-            fb[t] = *reinterpret_cast<const v4i*>(prow + (t / 3) * row_step + (t % 3) * col_step);
+            fb[t] = *(const __attribute__((address_space(3))) v4i*)(pbase + (uint32_t)((t / 3) * row_step + (t % 3) * col_step));
         __builtin_amdgcn_sched_barrier(0);
         int wm[4];
 #pragma unroll
@@ -257,7 +262,8 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
         // ---- epilogue ------------------------------------------------------------------------------------------------
         const int oy = oy0 + ty, ox = ox0 + tx;
         const bool ok = p_in_tile && oy < a.OH && ox < a.OW && cl < C;
-        const size_t obase = (((size_t)n * a.OH + oy) * a.OW + ox) * C + cl;
+        // the tensor has fewer than 2^31 elements (checked by the launcher): 32-bit arithmetic
+        const size_t obase = (uint32_t)(((n * a.OH + oy) * a.OW + ox) * C + cl);
         if constexpr (!FUSED)
         {
             if (ok)
