@@ -46,7 +46,7 @@ struct SlabArgs
     int32_t bias_len, za;
     int32_t n_ocb;
     int32_t out_kind;    // 0: int32 accumulators, 1: int8 through the RESCALE, 2: int16 through the RESCALE
-    int32_t xcd_remap;
+    int32_t xcd_remap;    // 0, or grid / 8: workgroup b takes tile (b % 8) * (grid / 8) + b / 8
     int32_t pitch;               // 16-byte chunks per patch row in LDS: 5 per pixel plus the padding that spreads the banks
     int32_t step_row, step_chunk;    // 448 = step_row * pitch + step_chunk: how far 7 loads (448 slots) move
     FastDiv div_tw, div_pitch, div_tiles_x, div_tiles_y, div_ocb;
@@ -85,7 +85,11 @@ template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD =
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
-    asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len), "s"(a.div_ocb.d));
+    // every scalar argument the kernel reads, named once so that they are fetched together at the top (fields
+    // first needed later are otherwise loaded one at a time, each with its own wait)
+    asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.out_zp), "s"(*reinterpret_cast<const uint32_t*>(&a.rp.scale32)),
+                 "s"(*reinterpret_cast<const uint32_t*>(&a.rp.in_bits)), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len),
+                 "s"(a.div_ocb.d));
     constexpr int TAPS   = KH * KW;
     constexpr int RW     = TAPS * CH + 1;    // chunks per weight row in LDS (odd)
     constexpr int KB     = CH * 16;          // bytes of a channel vector
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     {
         // consecutive workgroups go to the 8 XCDs in turn: give each XCD a contiguous run of tiles, whose halos
         // then meet in one L2
-        const uint32_t per = gridDim.x >> 3;
+        const uint32_t per = (uint32_t)a.xcd_remap;    // an eighth of the grid: no hidden-argument load for gridDim
         bid                = (bid & 7) * per + (bid >> 3);
     }
     const uint32_t tile = fdiv(bid, a.div_ocb);
@@ -550,7 +554,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     const int64_t grid = (int64_t)g.N * a.tiles_y * a.tiles_x * n_ocb;
     if (!tile_decode_is_exact(grid, (uint32_t)n_ocb, (uint32_t)a.tiles_x, (uint32_t)a.tiles_y))
         return nullptr;
-    a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? 1 : 0;
+    a.xcd_remap = (grid % 8 == 0 && n_ocb == 1) ? (int32_t)(grid / 8) : 0;
     // A patch pixel is R = CH + 1 chunks; the chunk of output pixel (ty, tx) under tap (0, 0) is ty * sy * pitch + R * sx * tx.
     // A ds_read_b128 serves 16 lanes together, whose chunks must differ modulo 16.  The lanes of a wave are consecutive
     // tile pixels p = ty * TW + tx, and any 16 lanes served together differ modulo 16, so the reads are free of bank

@@ -43,7 +43,7 @@ struct DwSlabArgs
     int32_t TH, TW, PH, PW, tiles_x, tiles_y;
     int32_t bias_len, za;
     int32_t out_kind;    // 0: int32 accumulators, 1: int8 through the RESCALE, 2: int16 through the RESCALE
-    int32_t xcd_remap;
+    int32_t xcd_remap;    // 0, or grid / 8: workgroup b takes tile (b % 8) * (grid / 8) + b / 8
     int32_t cpp;         // 16-byte chunks per pixel = C / 16
     int32_t ppitch;      // chunks per patch pixel in LDS (odd)
     int32_t pitch;       // chunks per patch row in LDS
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
     uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
     {
-        const uint32_t per = gridDim.x >> 3;
+        const uint32_t per = (uint32_t)a.xcd_remap;    // an eighth of the grid: no hidden-argument load for gridDim
         bid                = (bid & 7) * per + (bid >> 3);
     }
     const uint32_t trow = fdiv(bid, a.div_tiles_x);
@@ -482,7 +482,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     const int64_t grid = (int64_t)g.N * a.tiles_y * a.tiles_x;
     if (!tile_decode_is_exact(grid, 1u, (uint32_t)a.tiles_x, (uint32_t)a.tiles_y))
         return nullptr;
-    a.xcd_remap = grid % 8 == 0 ? 1 : 0;
+    a.xcd_remap = grid % 8 == 0 ? (int32_t)(grid / 8) : 0;
     a.div_tw = make_fastdiv((uint32_t)a.TW), a.div_pitch = make_fastdiv((uint32_t)a.pitch);
     a.div_ppitch = make_fastdiv((uint32_t)ppitch);
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
