@@ -41,9 +41,9 @@ PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what
 # the same counters read for a plain copy of known size (the committed rocprofv3 summaries hold the raw
 # figures).
-MEASURED_TRAFFIC_BYTES = {"c3": 3610128, "c2": 51125487, "c4": 12201417, "c5a": 22847896, "c5b": 269061069,
-                          "maxpool": 32145619, "avgpool": 32182579, "tconv": 8340031, "conv3d": 8036867,
-                          "rescale": 64287481, "c4x8": 96470586, "c3x4": 13241906}
+MEASURED_TRAFFIC_BYTES = {"c3": 3609285, "c2": 51062425, "c4": 12187176, "c5a": 22849700, "c5b": 269075463,
+                          "maxpool": 32148344, "avgpool": 32185529, "tconv": 8338973, "conv3d": 8034837,
+                          "rescale": 64324084, "c4x8": 96464107, "c3x4": 13241489}
 
 
 def main() -> int:
