@@ -197,3 +197,60 @@ def test_pooling_int8_conformance_target_shapes(ctx, case, avg):
         want = oracle.max_pool2d(x, kernel, stride, pad)
         got, st = gpu_ops.pool2d(ctx, x, kernel, stride, pad, False)
     assert st == capi.VALID and np.array_equal(got, want), ctx.last_kernel
+
+
+# ---- the sizes of the generator's --level-8k-sizes groups: kernels, strides, dilations and pads at MAX_KERNEL =
+# MAX_STRIDE = 8192 (tosa_ext_profile_ops_info.json, third group of each operator), with the level set: the
+# operators stay VALID at the limit
+@pytest.fixture()
+def ctx_8k():
+    c = Context(0)
+    c.set_level(capi.LEVEL_EIGHTK)
+    yield c
+    c.close()
+
+
+CONV_8K = [  # input shape, (OC, KH, KW), stride, dilation, pad
+    ((1, 8193, 2, 2), (3, 8192, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    ((1, 3, 8195, 1), (2, 2, 8192), (1, 3), (1, 1), (0, 0, 0, 0)),
+    ((1, 8193, 3, 3), (2, 1, 2), (8192, 1), (1, 1), (0, 0, 0, 0)),
+    ((1, 4097, 2, 2), (2, 2, 1), (1, 1), (4096, 1), (0, 0, 0, 0)),
+    ((2, 2, 2, 4), (3, 2, 2), (1, 1), (1, 1), (8192, 0, 0, 0)),
+    ((1, 2, 3, 2), (2, 3, 2), (1, 1), (1, 1), (0, 1, 0, 8192)),
+]
+
+
+@pytest.mark.parametrize("case", CONV_8K, ids=lambda c: "x".join(map(str, c[0])) + "_k" + "x".join(map(str, c[1])))
+def test_conv2d_and_depthwise_at_the_8k_level_limits(ctx_8k, case):
+    shape, (oc, kh, kw), stride, dil, pad = case
+    rng = np.random.default_rng(sum(shape) + kh + kw)
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    w = rng.integers(-128, 128, (oc, kh, kw, shape[3])).astype(np.int8)
+    bias = rng.integers(-(1 << 20), 1 << 20, oc).astype(np.int32)
+    want = oracle.conv2d("i8", x, w, bias, pad, stride, dil, in_zp=-3, w_zp=5)
+    got, st = gpu_ops.conv2d(ctx_8k, x, w, bias, pad, stride, dil, in_zp=-3, w_zp=5)
+    assert st == capi.VALID and ctx_8k.flags == 0 and np.array_equal(got, want), ctx_8k.last_kernel
+    wd = rng.integers(-128, 128, (kh, kw, shape[3], 2)).astype(np.int8)
+    bd = rng.integers(-(1 << 16), 1 << 16, shape[3] * 2).astype(np.int32)
+    want = oracle.depthwise_conv2d("i8", x, wd, bd, pad, stride, dil, in_zp=-3, w_zp=5)
+    got, st = gpu_ops.conv2d(ctx_8k, x, wd, bd, pad, stride, dil, in_zp=-3, w_zp=5, depthwise=True)
+    assert st == capi.VALID and np.array_equal(got, want), ctx_8k.last_kernel
+
+
+def test_pooling_and_transpose_conv2d_at_the_8k_level_limits(ctx_8k):
+    rng = np.random.default_rng(8192)
+    x = rng.integers(-128, 128, (1, 8193, 3, 2)).astype(np.int8)
+    got, st = gpu_ops.pool2d(ctx_8k, x, (8192, 1), (1, 1), avg=False)
+    assert st == capi.VALID and np.array_equal(got, oracle.max_pool2d(x, (8192, 1), (1, 1)))
+    got, st = gpu_ops.pool2d(ctx_8k, x, (8192, 2), (1, 1), (0, 0, 0, 0), True, -5, 7)
+    assert st == capi.VALID and np.array_equal(got, oracle.avg_pool2d(x, (8192, 2), (1, 1), (0, 0, 0, 0), -5, 7))
+    got, st = gpu_ops.pool2d(ctx_8k, x, (2, 1), (8191, 2), avg=False)
+    assert st == capi.VALID and np.array_equal(got, oracle.max_pool2d(x, (2, 1), (8191, 2)))
+    xt = rng.integers(-128, 128, (1, 2, 2, 3)).astype(np.int8)
+    wt = rng.integers(-128, 128, (2, 2, 3, 3)).astype(np.int8)
+    bt = rng.integers(-1000, 1000, 2).astype(np.int32)
+    got, st = gpu_ops.transpose_conv2d(ctx_8k, xt, wt, bt, (0, 0, 0, 0), (8192, 1), -4, 0)
+    assert st == capi.VALID and np.array_equal(got, oracle.transpose_conv2d("i8", xt, wt, bt, (0, 0, 0, 0), (8192, 1), -4, 0))
+    wk = rng.integers(-128, 128, (1, 8192, 1, 3)).astype(np.int8)
+    got, st = gpu_ops.transpose_conv2d(ctx_8k, xt, wk, bt[:1], (0, 0, 0, 0), (1, 1), -4, 2)
+    assert st == capi.VALID and np.array_equal(got, oracle.transpose_conv2d("i8", xt, wk, bt[:1], (0, 0, 0, 0), (1, 1), -4, 2))
