@@ -246,7 +246,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
             wv[t] = wcol[t * C];
 #pragma unroll
         for (int t = 0; t < TAPS; t++)
-            fb[t] = *(const __attribute__((address_space(3))) v4i*)(pbase + (uint32_t)((t / 3) * row_step + (t % 3) * col_step));
+            fb[t] = *(const __attribute__((address_space(3))) v4i*)(uintptr_t)(pbase + (uint32_t)((t / 3) * row_step + (t % 3) * col_step));
         __builtin_amdgcn_sched_barrier(0);
         int wm[4];
 #pragma unroll
