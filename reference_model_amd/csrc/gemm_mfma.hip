@@ -9,9 +9,11 @@
 // A workgroup of 8 waves (2 along the output channels x 4 along the pixels) owns a tile of 64*OCT channels x
 // 128*PXT pixels; a wave owns OCT x PXT accumulator tiles of 32x32.  K is walked in blocks of 64 bytes per
 // row.  The operands of a block go from global memory straight into LDS (global_load_lds_dwordx4: no
-// staging registers, no LDS store instructions), into one of three or four stage buffers, so the loads of the
-// next blocks are in flight while one is multiplied; one barrier per block both publishes a stage and frees
-// the one the next loads will overwrite.
+// staging registers, no LDS store instructions), into a ring of stage buffers, so the loads of the next blocks
+// are in flight while one is multiplied; one barrier per block both publishes a stage and frees the one the
+// next loads will overwrite.  Where the ring can be six or eight stages long and K is deep, the blocks are
+// requested two at a time - the two 64-byte halves of a row's 128-byte line back to back, which the L1 merges
+// into one request to L2 - with one barrier per pair.
 //
 // LDS layout of a stage: row r (weight rows first, then pixel rows) occupies bytes [64r, 64r + 64); its four
 // 16-byte chunks are stored permuted, chunk c at position c ^ swz(r), so that the 16 lanes the LDS serves in
@@ -25,6 +27,7 @@
 // Zero points (int8): sum(a*w) - zw*sum(a) - za*sum(w) + K*za*zw.  The sums are taken with v_dot4 from the
 // fragments as they pass through registers on their way to the matrix core (only in the ZP instantiation).
 #include "tmi_mfma.h"
+#include <type_traits>
 
 namespace tmi
 {
@@ -77,7 +80,7 @@ __device__ __forceinline__ int channel_of_row(int rho)
 // Stage buffers of a workgroup: four 64-byte blocks per row.  The 256x256 shape fills the LDS with them; two
 // workgroups of a smaller shape with three stages each were measured and are slower (the operand traffic per
 // matrix instruction, not the barrier, is what the smaller shapes wait for).
-static constexpr int kStages = 4;
+static constexpr int kStagesDefault = 4;
 
 // K-major weights (KM): the weight operand lies in memory as [K][N] (MATMUL's second operand as the operator
 // defines it).  Its part of a stage is then 64 / sizeof(T) rows of K with the tile's 64*OCT channels side by
@@ -102,9 +105,10 @@ enum
     GEMM_TAPS    = 2
 };
 
-template <typename T, int OCT, int PXT, bool ZP, int MODE>
+template <typename T, int OCT, int PXT, bool ZP, int MODE, int kStages, bool PAIR>
 __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 {
+    static_assert(!PAIR || (kStages >= 6 && kStages % 2 == 0), "pairs of blocks need an even ring of six stages or more");
     constexpr bool KM      = MODE == GEMM_KMAJOR;
     constexpr bool TAPS    = MODE == GEMM_TAPS;
     using M                = Mma<T>;
@@ -239,11 +243,27 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                      : "v"(voff[j]), "s"(src), "s"(dst)
                      : "memory");
     };
+    // PAIR: the two 64-byte blocks that share a 128-byte line are requested back to back (the second request
+    // then finds the line on its way into the L1 instead of fetching it from L2 again), a pair every two blocks
+    auto issue_pair = [&](int block, int q) {
+        issue_one(block + (q & 1), block + (q & 1), q >> 1);    // prologue: stage = block
+    };
+    if constexpr (PAIR)
+    {
 #pragma unroll
-    for (int s = 0; s < kStages - 1; s++)
+        for (int s = 0; s < kStages - 2; s += 2)
 #pragma unroll
-        for (int j = 0; j < LOADS; j++)
-            issue_one(s, s, j);
+            for (int q = 0; q < 2 * LOADS; q++)
+                issue_pair(s, q);
+    }
+    else
+    {
+#pragma unroll
+        for (int s = 0; s < kStages - 1; s++)
+#pragma unroll
+            for (int j = 0; j < LOADS; j++)
+                issue_one(s, s, j);
+    }
 
     // ---- tables: bias per channel of the tile (in the shadow of the first loads) ---------------------------
     int* tab_bias = reinterpret_cast<int*>(lds + kStages * STAGE);    // WROWS words
@@ -391,19 +411,24 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     auto publish = [&]() {
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((kStages - 3) * LOADS) : "memory");
     };
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * LOADS) : "memory");
+    // PAIR: a pair lands as a whole (its loads alternate between the two blocks), so one barrier per pair, in
+    // the second block, publishes the next pair; another pair may still be on its way behind it.
+    auto publish_pair = [&]() {
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PAIR ? (kStages / 2 - 3) * 2 * LOADS : 0) : "memory");
+    };
+    if constexpr (PAIR)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PAIR ? (kStages / 2 - 2) * 2 * LOADS : 0) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * LOADS) : "memory");
     __syncthreads();    // block 0 and the bias table are in LDS for every wave
 #pragma unroll
     for (int j = 0; j < NR; j++)
         read_one(lds, 0, j);
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll 1
-    for (int n = 0; n < nb; n++)
-    {
-        const uint8_t* cur  = lds + (n % kStages) * STAGE;
-        const uint8_t* next = lds + ((n + 1) % kStages) * STAGE;
-        // two requests behind each of the first matrix instructions, so that the last ones of a step cover the
-        // latency of the fragments the next step starts with
+    // first K-step of a block: its matrix instructions, and the requests for the fragments of the second step;
+    // two requests behind each of the first matrix instructions, so that the last ones of a step cover the
+    // latency of the fragments the next step starts with
+    auto first_step = [&](const uint8_t* cur) {
         constexpr int PA = NR > 2 * NM ? (NR + NM - 1) / NM : 2;
         sums(0);
 #pragma unroll
@@ -415,10 +440,14 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 read_one(cur, 1, j);
             __builtin_amdgcn_sched_barrier(0);
         }
-        publish();    // block n+1 (after the last block: its repeat) is in LDS for every wave
-        sums(1);
-        constexpr int NO = LOADS + NR;    // direct loads first, they have the longest way to go
+    };
+    // second K-step: its matrix instructions, NL direct loads (they have the longest way to go, so they come
+    // first) and the requests for the first fragments of the next block
+    auto second_step = [&](const uint8_t* next, auto NL_tag, auto&& load) {
+        constexpr int NL = decltype(NL_tag)::value;
+        constexpr int NO = NL + NR;
         constexpr int PB = NO > 2 * NM ? (NO + NM - 1) / NM : 2;
+        sums(1);
 #pragma unroll
         for (int k = 0; k < NM; k++)
         {
@@ -426,12 +455,52 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 #pragma unroll
             for (int q = k * PB; q < (k + 1) * PB && q < NO; q++)
             {
-                if (q < LOADS)
-                    issue_one(n + kStages - 1, (n + kStages - 1) % kStages, q);
+                if (q < NL)
+                    load(q);
                 else
-                    read_one(next, 0, q - LOADS);
+                    read_one(next, 0, q - NL);
             }
             __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if constexpr (PAIR)
+    {
+        int sc = 0;    // stage of the pair's first block
+#pragma unroll 1
+        for (int n = 0; n + 1 < nb; n += 2)
+        {
+            const int sn        = sc + 2 < kStages ? sc + 2 : 0;
+            const int sfree     = sc >= 2 ? sc - 2 : kStages - 2;    // the pair consumed before this one
+            const uint8_t* cur0 = lds + sc * STAGE;
+            first_step(cur0);
+            second_step(cur0 + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+            first_step(cur0 + STAGE);
+            publish_pair();    // the next pair is in LDS for every wave, and every wave is past the pair before
+            second_step(lds + sn * STAGE, std::integral_constant<int, 2 * LOADS>{}, [&](int q) {
+                issue_one(n + kStages - 2 + (q & 1), sfree + (q & 1), q >> 1);
+            });
+            sc = sn;
+        }
+        if (nb & 1)
+        {
+            // the last block of an odd count: the first half of a pair whose second half is a repeat
+            const uint8_t* cur = lds + sc * STAGE;
+            first_step(cur);
+            second_step(cur + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+        }
+    }
+    else
+    {
+#pragma unroll 1
+        for (int n = 0; n < nb; n++)
+        {
+            const uint8_t* cur  = lds + (n % kStages) * STAGE;
+            const uint8_t* next = lds + ((n + 1) % kStages) * STAGE;
+            first_step(cur);
+            publish();    // block n+1 (after the last block: its repeat) is in LDS for every wave
+            second_step(next, std::integral_constant<int, LOADS>{}, [&](int q) {
+                issue_one(n + kStages - 1, (n + kStages - 1) % kStages, q);
+            });
         }
     }
 
@@ -628,17 +697,34 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             raise_flags(a.flag_word, flags);
 }
 
-template <typename T, int OCT, int PXT, bool ZP, int MODE>
-static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
+template <typename T, int OCT, int PXT, bool ZP, int MODE, int STAGES, bool PAIR>
+static bool launch_gemm_pipe(hipStream_t st, const GemmArgs& a, int blocks)
 {
     // stages, bias table, per-channel RESCALE constants
-    constexpr size_t lds_bytes = (size_t)kStages * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
-    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE>;
+    constexpr size_t lds_bytes = (size_t)STAGES * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
+    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE, STAGES, PAIR>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, granted))
         return false;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(512), lds_bytes, st, a);
     return true;
+}
+
+template <typename T, int OCT, int PXT, bool ZP, int MODE>
+static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
+{
+    // The two smaller shapes have LDS to spare for a ring of 8 x 16 KB or 6 x 24 KB, which lets them request
+    // the blocks in pairs (both halves of every 128-byte line together).  Measured on MI355X, us without /
+    // with: 3x3 layers fp16 [16,28,28,256]->256 24.8 / 23.4, [8,28,28,512]->512 51.1 / 48.1, int8 42.1 / 38.9;
+    // with few blocks the longer prologue costs more than the pairs return (pointwise [8,56,56,256]->64 fp16
+    // 5.0 / 5.6, int8 7.1 / 7.5; 32 blocks: 12.1 / 12.4), and the deeper ring without pairs is slower everywhere.
+    if constexpr (OCT * PXT <= 4)
+    {
+        constexpr int DEEP = OCT * PXT == 2 ? 8 : 6;
+        if (a.n_blocks > 32)
+            return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, DEEP, true>(st, a, blocks);
+    }
+    return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, kStagesDefault, false>(st, a, blocks);
 }
 
 template <typename T>

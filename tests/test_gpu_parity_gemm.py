@@ -40,6 +40,9 @@ GEMM_SHAPES = [
     (32, 300, 64 * 5, 200),
     (1, 128, 256, 16384),
     (1, 16384, 256, 64),
+    (2, 1024, 64 * 37, 1024),  # deep K on the small shapes: blocks requested in pairs, an odd number of them
+    (3, 900, 64 * 40, 1104),   # the same with an even number and ragged tiles
+    (8, 1024, 64 * 35, 1024),  # 128x256 tiles, odd
 ]
 
 
@@ -82,7 +85,8 @@ def test_gemm_kernel_refuses_what_it_cannot_take(ctx):
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (3, 1000, 448, 1104),
-                                   (1, 4099, 128, 515), (5, 520, 96 * 3, 784)])
+                                   (1, 4099, 128, 515), (5, 520, 96 * 3, 784),
+                                   (3, 1000, 32 * 37, 1104), (8, 1024, 32 * 42, 1024)])  # deep K: blocks in pairs
 def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, h, c, w = shape
     rng = np.random.default_rng(8 + h)
@@ -196,6 +200,7 @@ TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
     (32, 24, 24, 64, 64, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),       # dilation 2
     (16, 64, 64, 192, 96, 2, 2, (0, 0, 0, 0), (2, 2), (1, 1)),      # no padding
     (2, 130, 100, 64, 72, 1, 7, (0, 0, 3, 3), (1, 1), (1, 1)),
+    (16, 28, 28, 320, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 5 blocks per tap: pairs of blocks straddle taps
 ]
 
 
