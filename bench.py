@@ -41,9 +41,9 @@ PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what
 # the same counters read for a plain copy of known size (the committed rocprofv3 summaries hold the raw
 # figures).
-MEASURED_TRAFFIC_BYTES = {"c3": 3609285, "c2": 51062425, "c4": 12187176, "c5a": 22849700, "c5b": 269075463,
-                          "maxpool": 32148344, "avgpool": 32185529, "tconv": 8338973, "conv3d": 8034837,
-                          "rescale": 64324084, "c4x8": 96464107, "c3x4": 13241489}
+MEASURED_TRAFFIC_BYTES = {"c3": 3609330, "c2": 50853260, "c4": 12187223, "c5a": 22866096, "c5b": 268924401,
+                          "maxpool": 32148819, "avgpool": 32185708, "tconv": 8339131, "conv3d": 8034977,
+                          "rescale": 64324430, "c4x8": 96464556, "c3x4": 13241652}
 
 
 def main() -> int:

@@ -105,10 +105,20 @@ enum
     GEMM_TAPS    = 2
 };
 
-template <typename T, int OCT, int PXT, bool ZP, int MODE, int kStages, bool PAIR>
+enum
+{
+    PIPE_SINGLE     = 0,    // a ring of kStages stages, one 64-byte block requested per block period
+    PIPE_PAIRS      = 1,    // a ring of six or eight stages, two blocks requested every second period
+    PIPE_PIXEL_PAIRS = 2    // K-major weights: four stages of weight rows, three slots of two blocks of pixel rows
+};
+
+template <typename T, int OCT, int PXT, bool ZP, int MODE, int kStages, int PIPE>
 __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 {
+    constexpr bool PAIR    = PIPE == PIPE_PAIRS;
+    constexpr bool APAIR   = PIPE == PIPE_PIXEL_PAIRS;
     static_assert(!PAIR || (kStages >= 6 && kStages % 2 == 0), "pairs of blocks need an even ring of six stages or more");
+    static_assert(!APAIR || (MODE == GEMM_KMAJOR && kStages == 4), "pixel pairs: K-major weights in a ring of four");
     constexpr bool KM      = MODE == GEMM_KMAJOR;
     constexpr bool TAPS    = MODE == GEMM_TAPS;
     using M                = Mma<T>;
@@ -132,6 +142,8 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     constexpr int ROWS     = WROWS + PROWS;
     constexpr int STAGE    = ROWS * 64;
     constexpr int LOADS    = ROWS / 128;    // direct loads per wave and block (16 rows each)
+    constexpr int WLOADS   = WROWS / 128;   // of which carry weight rows
+    constexpr int PLOADS   = LOADS - WLOADS;
     static_assert(ROWS % 128 == 0, "a block must split evenly over the 8 waves");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -197,7 +209,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     if constexpr (TAPS)
     {
 #pragma unroll
-        for (int j = OCT / 2; j < LOADS; j++)
+        for (int j = WLOADS; j < LOADS; j++)
         {
             const int r = (j * 8 + wave) * 16 + (lane >> 2);
             int p       = p0 + r - WROWS;
@@ -220,10 +232,9 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     // Every block period issues one block's loads, also past the end (the last block again, into a stage nobody
     // reads any more): the count of loads in flight is then the same in every iteration and the wait for a
     // block is one instruction with an immediate.
-    auto issue_one = [&](int block, int stage, int j) {
+    auto issue_at = [&](int block, uint32_t dst, int j) {
         const int blk      = block < nb ? block : nb - 1;
-        const uint32_t dst = ldst[j] + stage * STAGE;
-        if (TAPS && j >= OCT / 2)
+        if (TAPS && j >= WLOADS)
         {
             // tap of the block (scalar), then per lane: the pixel under that tap, or the zero page
             const int t       = (int)fdiv((uint32_t)blk, a.div_bpt);
@@ -245,6 +256,17 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     };
     // PAIR: the two 64-byte blocks that share a 128-byte line are requested back to back (the second request
     // then finds the line on its way into the L1 instead of fetching it from L2 again), a pair every two blocks
+    auto issue_one = [&](int block, int stage, int j) { issue_at(block, ldst[j] + stage * STAGE, j); };
+    // PIXEL_PAIRS: the weight rows (whole lines already, K-major) keep a ring of four single blocks at the start
+    // of the LDS; the pixel rows are requested in pairs into three slots of two blocks behind it
+    constexpr int WB    = WROWS * 64;
+    constexpr int PB    = PROWS * 64;
+    constexpr int PBASE = 4 * WB;
+    auto issue_w = [&](int block, int j) { issue_at(block, ldst[j] + (block & 3) * WB, j); };
+    auto issue_p = [&](int block, int slot, int q) {    // q-th load of the pair that starts at the even `block`
+        const int j = WLOADS + (q >> 1);
+        issue_at(block + (q & 1), ldst[j] - WB + PBASE + slot * 2 * PB + (q & 1) * PB, j);
+    };
     auto issue_pair = [&](int block, int q) {
         issue_one(block + (q & 1), block + (q & 1), q >> 1);    // prologue: stage = block
     };
@@ -256,6 +278,22 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             for (int q = 0; q < 2 * LOADS; q++)
                 issue_pair(s, q);
     }
+    else if constexpr (APAIR)
+    {
+        // in the order the loop continues: pixel pair 0, weights 0, weights 1, pixel pair 1, weights 2
+#pragma unroll
+        for (int q = 0; q < 2 * PLOADS; q++)
+            issue_p(0, 0, q);
+#pragma unroll
+        for (int j = 0; j < 2 * WLOADS; j++)
+            issue_w(j / WLOADS, j % WLOADS);
+#pragma unroll
+        for (int q = 0; q < 2 * PLOADS; q++)
+            issue_p(2, 1, q);
+#pragma unroll
+        for (int j = 0; j < WLOADS; j++)
+            issue_w(2, j);
+    }
     else
     {
 #pragma unroll
@@ -266,9 +304,11 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     }
 
     // ---- tables: bias per channel of the tile (in the shadow of the first loads) ---------------------------
-    int* tab_bias = reinterpret_cast<int*>(lds + kStages * STAGE);    // WROWS words
-    if (tid < WROWS)
-    {
+    // (PIXEL_PAIRS fills the LDS with operands: its bias table is written after the loop, into a free stage)
+    int* tab_bias = reinterpret_cast<int*>(APAIR ? lds + 4096 : lds + kStages * STAGE);    // WROWS words
+    auto write_bias_table = [&]() {
+        if (tid >= WROWS)
+            return;
         const int oc = oc0 + tid;
         int v        = 0;
         if (oc < a.N)
@@ -279,12 +319,14 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 v = __float_as_int(load_as_float<T>(a.bias, a.bias_len == 1 ? 0 : oc));
         }
         tab_bias[tid] = v;
-    }
+    };
+    if constexpr (!APAIR)
+        write_bias_table();
 
     // per-channel constants of the fused RESCALE, derived once per workgroup (WROWS entries of 32 bytes)
     ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(lds + kStages * STAGE + WROWS * 4);
     uint32_t flags       = 0;
-    if constexpr (M::is_int)
+    if constexpr (M::is_int && !APAIR)
     {
         if (a.rp.enabled && tid < WROWS)
         {
@@ -365,9 +407,11 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     constexpr int NR = NW + PXT;              // fragment reads per step
     v4i fa[2][OCT], fb[2][PXT];
     // reads in the order the matrix instructions want them: pixel tile 0, the channel tiles, the other pixel tiles
-    auto read_one = [&](const uint8_t* sb, int s, int j) {
+    // wb: the stage's weight rows; pb: its pixel rows minus their offset in a whole stage (ap[] includes it)
+    auto read_one = [&](const uint8_t* wb, const uint8_t* pb, int s, int j) {
+        const uint8_t* sb = wb;
         if (j == 0)
-            fb[s][0] = *reinterpret_cast<const v4i*>(sb + ap[s]);
+            fb[s][0] = *reinterpret_cast<const v4i*>(pb + ap[s]);
         else if (j <= NW)
         {
             if constexpr (KM)
@@ -387,7 +431,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 fa[s][j - 1] = *reinterpret_cast<const v4i*>(sb + aw[s] + (j - 1) * 2048);
         }
         else
-            fb[s][j - NW] = *reinterpret_cast<const v4i*>(sb + ap[s] + (j - NW) * 2048);
+            fb[s][j - NW] = *reinterpret_cast<const v4i*>(pb + ap[s] + (j - NW) * 2048);
     };
     auto sums = [&](int s) {
         if constexpr (ZP)
@@ -418,17 +462,19 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     };
     if constexpr (PAIR)
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PAIR ? (kStages / 2 - 2) * 2 * LOADS : 0) : "memory");
+    else if constexpr (APAIR)
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PLOADS + 2 * WLOADS) : "memory");
     else
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 2) * LOADS) : "memory");
     __syncthreads();    // block 0 and the bias table are in LDS for every wave
 #pragma unroll
     for (int j = 0; j < NR; j++)
-        read_one(lds, 0, j);
+        read_one(lds, APAIR ? lds + PBASE - WB : lds, 0, j);
     __builtin_amdgcn_sched_barrier(0);
     // first K-step of a block: its matrix instructions, and the requests for the fragments of the second step;
     // two requests behind each of the first matrix instructions, so that the last ones of a step cover the
     // latency of the fragments the next step starts with
-    auto first_step = [&](const uint8_t* cur) {
+    auto first_step = [&](const uint8_t* cur, const uint8_t* curp) {
         constexpr int PA = NR > 2 * NM ? (NR + NM - 1) / NM : 2;
         sums(0);
 #pragma unroll
@@ -437,13 +483,13 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             mma_one(0, k);
 #pragma unroll
             for (int j = k * PA; j < (k + 1) * PA && j < NR; j++)
-                read_one(cur, 1, j);
+                read_one(cur, curp, 1, j);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
     // second K-step: its matrix instructions, NL direct loads (they have the longest way to go, so they come
     // first) and the requests for the first fragments of the next block
-    auto second_step = [&](const uint8_t* next, auto NL_tag, auto&& load) {
+    auto second_step = [&](const uint8_t* next, const uint8_t* nextp, auto NL_tag, auto&& load) {
         constexpr int NL = decltype(NL_tag)::value;
         constexpr int NO = NL + NR;
         constexpr int PB = NO > 2 * NM ? (NO + NM - 1) / NM : 2;
@@ -458,7 +504,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 if (q < NL)
                     load(q);
                 else
-                    read_one(next, 0, q - NL);
+                    read_one(next, nextp, 0, q - NL);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -472,11 +518,11 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             const int sn        = sc + 2 < kStages ? sc + 2 : 0;
             const int sfree     = sc >= 2 ? sc - 2 : kStages - 2;    // the pair consumed before this one
             const uint8_t* cur0 = lds + sc * STAGE;
-            first_step(cur0);
-            second_step(cur0 + STAGE, std::integral_constant<int, 0>{}, [](int) {});
-            first_step(cur0 + STAGE);
+            first_step(cur0, cur0);
+            second_step(cur0 + STAGE, cur0 + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+            first_step(cur0 + STAGE, cur0 + STAGE);
             publish_pair();    // the next pair is in LDS for every wave, and every wave is past the pair before
-            second_step(lds + sn * STAGE, std::integral_constant<int, 2 * LOADS>{}, [&](int q) {
+            second_step(lds + sn * STAGE, lds + sn * STAGE, std::integral_constant<int, 2 * LOADS>{}, [&](int q) {
                 issue_one(n + kStages - 2 + (q & 1), sfree + (q & 1), q >> 1);
             });
             sc = sn;
@@ -485,8 +531,46 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         {
             // the last block of an odd count: the first half of a pair whose second half is a repeat
             const uint8_t* cur = lds + sc * STAGE;
-            first_step(cur);
-            second_step(cur + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+            first_step(cur, cur);
+            second_step(cur + STAGE, cur + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+        }
+    }
+    else if constexpr (APAIR)
+    {
+        // Loads are waited for in the order they were issued.  Behind the weights of block n+1 (needed at the
+        // barrier of an even block n) come a pixel pair and a block of weights; behind the pixel pair and the
+        // weights of block n+2 (needed at the barrier of the odd block n+1) a block of weights.
+        int slot = 0;    // pixel slot of the pair (n, n+1)
+#pragma unroll 1
+        for (int n = 0; n + 1 < nb; n += 2)
+        {
+            const int slot_next = slot == 2 ? 0 : slot + 1;
+            const int slot_free = slot == 0 ? 2 : slot - 1;    // held the pair before this one
+            const uint8_t* wb0  = lds + (n & 3) * WB;
+            const uint8_t* wb1  = lds + ((n + 1) & 3) * WB;
+            const uint8_t* wb2  = lds + ((n + 2) & 3) * WB;
+            const uint8_t* pb0  = lds + PBASE - WB + slot * 2 * PB;
+            const uint8_t* pb2  = lds + PBASE - WB + slot_next * 2 * PB;
+            first_step(wb0, pb0);
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * PLOADS + WLOADS) : "memory");
+            second_step(wb1, pb0 + PB, std::integral_constant<int, WLOADS>{}, [&](int q) { issue_w(n + 3, q); });
+            first_step(wb1, pb0 + PB);
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(WLOADS) : "memory");
+            second_step(wb2, pb2, std::integral_constant<int, 2 * PLOADS + WLOADS>{}, [&](int q) {
+                if (q < 2 * PLOADS)
+                    issue_p(n + 4, slot_free, q);
+                else
+                    issue_w(n + 4, q - 2 * PLOADS);
+            });
+            slot = slot_next;
+        }
+        if (nb & 1)
+        {
+            // the last block of an odd count: published by the barrier before it, nothing left to request
+            const uint8_t* wb = lds + ((nb - 1) & 3) * WB;
+            const uint8_t* pb = lds + PBASE - WB + slot * 2 * PB;
+            first_step(wb, pb);
+            second_step(wb, pb, std::integral_constant<int, 0>{}, [](int) {});
         }
     }
     else
@@ -496,9 +580,9 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         {
             const uint8_t* cur  = lds + (n % kStages) * STAGE;
             const uint8_t* next = lds + ((n + 1) % kStages) * STAGE;
-            first_step(cur);
+            first_step(cur, cur);
             publish();    // block n+1 (after the last block: its repeat) is in LDS for every wave
-            second_step(next, std::integral_constant<int, LOADS>{}, [&](int q) {
+            second_step(next, next, std::integral_constant<int, LOADS>{}, [&](int q) {
                 issue_one(n + kStages - 1, (n + kStages - 1) % kStages, q);
             });
         }
@@ -509,19 +593,24 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     // given another use.  The stage buffers are then free: the channel sums go through the first one.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     int* tab_wsum = reinterpret_cast<int*>(lds);    // WROWS words
-    if constexpr (ZP)
+    if constexpr (ZP || APAIR)
     {
-        __syncthreads();
-#pragma unroll
-        for (int t = 0; t < OCT; t++)
+        __syncthreads();    // every wave has read its last fragments and seen its last loads land
+        if constexpr (APAIR)
+            write_bias_table();
+        if constexpr (ZP)
         {
-            const int sum = wsum[t] + __shfl_xor(wsum[t], 32);
-            if (wp == 0 && h == 0)
-                tab_wsum[wo * 32 * OCT + t * 32 + row_channel(rho)] = sum;
-        }
 #pragma unroll
-        for (int i = 0; i < PXT; i++)
-            psum[i] += __shfl_xor(psum[i], 32);
+            for (int t = 0; t < OCT; t++)
+            {
+                const int sum = wsum[t] + __shfl_xor(wsum[t], 32);
+                if (wp == 0 && h == 0)
+                    tab_wsum[wo * 32 * OCT + t * 32 + row_channel(rho)] = sum;
+            }
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+                psum[i] += __shfl_xor(psum[i], 32);
+        }
         __syncthreads();
     }
 
@@ -562,7 +651,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             if constexpr (M::is_int)
             {
                 const int pcorr = ZP ? a.zw * psum[i] : 0;
-                if (a.rp.enabled)
+                if (!APAIR && a.rp.enabled)
                 {
                     // fused RESCALE (+ CLAMP): the lane's 16 consecutive channels leave as 16 (32) bytes
                     const int ocl = tl + 16 * h;
@@ -692,17 +781,20 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             }
         }
     }
-    if constexpr (M::is_int)
+    if constexpr (M::is_int && !APAIR)
         if (a.rp.enabled)
             raise_flags(a.flag_word, flags);
 }
 
-template <typename T, int OCT, int PXT, bool ZP, int MODE, int STAGES, bool PAIR>
+template <typename T, int OCT, int PXT, bool ZP, int MODE, int STAGES, int PIPE>
 static bool launch_gemm_pipe(hipStream_t st, const GemmArgs& a, int blocks)
 {
-    // stages, bias table, per-channel RESCALE constants
-    constexpr size_t lds_bytes = (size_t)STAGES * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
-    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE, STAGES, PAIR>;
+    // stages, bias table, per-channel RESCALE constants; PIXEL_PAIRS: four stages of weight rows and three slots
+    // of two blocks of pixel rows, the bias table goes through a stage after the loop
+    constexpr size_t lds_bytes = PIPE == PIPE_PIXEL_PAIRS
+                                     ? (size_t)4 * 64 * OCT * 64 + (size_t)6 * 128 * PXT * 64
+                                     : (size_t)STAGES * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
+    auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE, STAGES, PIPE>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, granted))
         return false;
@@ -722,9 +814,22 @@ static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
     {
         constexpr int DEEP = OCT * PXT == 2 ? 8 : 6;
         if (a.n_blocks > 32)
-            return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, DEEP, true>(st, a, blocks);
+            return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, DEEP, PIPE_PAIRS>(st, a, blocks);
     }
-    return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, kStagesDefault, false>(st, a, blocks);
+    // MATMUL on the two larger shapes: the second operand lies K-major and is fetched in whole lines already; the
+    // first one's rows are requested in pairs (a third fewer read requests at the L2 for the named bf16 MATMUL,
+    // 8.8 M instead of 12.8 M).  Measured, us without / with: bf16 [4,2048,4096]x[4,4096,2048] 127.3 / 124.7 and
+    // 123.7 / 120.3 on two boxes, [1,4096,2048]x[1,2048,4096] 71.9 / 70.6, int8 [1,4096,4096]x[1,4096,4096]
+    // 65.1 / 64.1; below some 48 blocks of K nothing or the other way (int8 [8,1024,512] 13.8 / 14.0,
+    // [16,1024,768] 23.2 / 23.6).  The layout needs the whole LDS for the 256x256 shape: if the device does not
+    // grant it, the plain ring runs.
+    if constexpr (MODE == GEMM_KMAJOR && OCT * PXT >= 4)
+    {
+        if (a.n_blocks >= 48 && !a.rp.enabled &&
+            launch_gemm_pipe<T, OCT, PXT, ZP, MODE, 4, PIPE_PIXEL_PAIRS>(st, a, blocks))
+            return true;
+    }
+    return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, kStagesDefault, PIPE_SINGLE>(st, a, blocks);
 }
 
 template <typename T>

@@ -43,6 +43,9 @@ GEMM_SHAPES = [
     (2, 1024, 64 * 37, 1024),  # deep K on the small shapes: blocks requested in pairs, an odd number of them
     (3, 900, 64 * 40, 1104),   # the same with an even number and ragged tiles
     (8, 1024, 64 * 35, 1024),  # 128x256 tiles, odd
+    (4, 2048, 64 * 49, 2048),  # K-major operand, 48 blocks or more: the first operand's rows requested in pairs;
+    (8, 1024, 64 * 50, 1024),  # 256x256 and 128x256 tiles, odd and even block counts, ragged edges
+    (3, 1000, 64 * 51, 1104),
 ]
 
 
@@ -86,7 +89,8 @@ def test_gemm_kernel_refuses_what_it_cannot_take(ctx):
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (3, 1000, 448, 1104),
                                    (1, 4099, 128, 515), (5, 520, 96 * 3, 784),
-                                   (3, 1000, 32 * 37, 1104), (8, 1024, 32 * 42, 1024)])  # deep K: blocks in pairs
+                                   (3, 1000, 32 * 37, 1104), (8, 1024, 32 * 42, 1024),   # deep K: blocks in pairs
+                                   (4, 2048, 32 * 49, 2048), (3, 1000, 32 * 52, 1104)])  # ... the first operand's rows
 def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, h, c, w = shape
     rng = np.random.default_rng(8 + h)
