@@ -64,6 +64,50 @@ def test_matmul_i8_gemm_bit_exact(ctx, shape, zps):
     assert np.array_equal(got[-1, -24:], oracle.matmul("i8", a[-1:, -24:], b[-1:], *zps)[0])
 
 
+def random_matmul_shapes(count, seed):
+    """seeded shapes around the block counts where the kernel changes how it requests its operands (32 and 48
+    blocks of 64 bytes), odd and even counts, ragged tiles in both directions"""
+    rng = np.random.default_rng(seed)
+    shapes = []
+    while len(shapes) < count:
+        n = int(rng.integers(1, 5))
+        h = int(rng.integers(128, 1400))
+        w = 16 * int(rng.integers(8, 90))
+        blocks = int(rng.choice([4, 7, 16, 31, 32, 33, 34, 47, 48, 49, 50, 63, 64, 65]))
+        if ((h + 127) // 128) * ((w + 127) // 128) * n >= 128:    # enough work for the kernel to take it
+            shapes.append((n, h, blocks, w))
+    return shapes
+
+
+@pytest.mark.parametrize("shape", random_matmul_shapes(28, 20240607))
+def test_matmul_i8_gemm_random_shapes_bit_exact(ctx, shape):
+    n, h, blocks, w = shape
+    c = 64 * blocks
+    rng = np.random.default_rng(h * 7 + w + blocks)
+    a = rng.integers(-128, 128, (n, h, c)).astype(np.int8)
+    b = rng.integers(-128, 128, (n, c, w)).astype(np.int8)
+    zps = (int(rng.integers(-128, 128)), int(rng.integers(-128, 128))) if blocks % 2 else (0, 0)
+    got, st = gpu_ops.matmul(ctx, a, b, *zps)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_i8"
+    assert np.array_equal(got, exact_matmul_i8(a, b, *zps))
+
+
+@pytest.mark.parametrize("shape", random_matmul_shapes(10, 77))
+def test_matmul_bf16_gemm_random_shapes_within_dot_product_bound(ctx, shape):
+    n, h, blocks, w = shape
+    c = 32 * blocks
+    rng = np.random.default_rng(h + w + blocks)
+    a_s = cases.float_to_bf16_bits(rng.normal(0, 1 / 8, (n, h, c)).astype(np.float32))
+    b_s = cases.float_to_bf16_bits(rng.normal(0, 1 / 8, (n, c, w)).astype(np.float32))
+    af, bf = cases.bf16_bits_to_float(a_s).astype(np.float64), cases.bf16_bits_to_float(b_s).astype(np.float64)
+    got, st = gpu_ops.matmul(ctx, a_s, b_s, dtype=capi.BF16)
+    assert st == capi.VALID and ctx.last_kernel == "matmul_gemm_bf16"
+    ref, bnd = np.matmul(af, bf), np.matmul(np.abs(af), np.abs(bf))
+    # tolerance: |imp-ref| <= 2*C * max(bnd*2^-24, 2^-126) per element and sum err^2 <= 1.6*C*T
+    res = dp.check(got, ref, bnd, "fp32", dp.kernel_size_bound(c, "fp32", has_bias=False))
+    assert res["ok"], res
+
+
 def test_matmul_i8_gemm_extreme_values(ctx):
     """all operands at -128 with zero points at +127: the largest products the operator can form"""
     n, h, c, w = 8, 512, 4096, 512
