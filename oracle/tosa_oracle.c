@@ -284,6 +284,9 @@ int orc_tconv_check(const orc_tconv_shape_t* s)
 {
     if (s->stride[0] < 1 || s->stride[1] < 1)
         return ORC_ERROR;
+    /* a tensor with a negative dimension is never allocated (subgraph_traverser.cpp:583-590): no such call */
+    if (s->OH < 0 || s->OW < 0)
+        return ORC_ERROR;
     if (s->out_pad[0] <= -s->KH || s->out_pad[1] <= -s->KH || s->out_pad[2] <= -s->KW || s->out_pad[3] <= -s->KW)
         return ORC_ERROR;
     if (s->OH != (s->IH - 1) * s->stride[0] + s->out_pad[0] + s->out_pad[1] + s->KH ||

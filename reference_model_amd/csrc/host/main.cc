@@ -207,7 +207,8 @@ int main(int argc, char** argv)
         st = runner.initialize(block);
         if (st != GraphStatus::TOSA_VALID)
         {
-            fprintf(stderr, "Graph result: ERROR (%s)\n", runner.traverser() ? runner.traverser()->last_message.c_str() : "");
+            fprintf(stderr, "Graph result: %s (%s)\n", st == GraphStatus::TOSA_UNPREDICTABLE ? "UNPREDICTABLE" : "ERROR",
+                    runner.traverser() ? runner.traverser()->last_message.c_str() : "");
             return (int)st;
         }
         for (size_t i = 0; i < desc.ifm_name.size(); i++)

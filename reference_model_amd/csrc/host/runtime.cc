@@ -994,6 +994,19 @@ int SubgraphTraverser::validateGraph()
             setGraphStatus(GraphStatus::TOSA_ERROR);
             return 1;
         }
+    // A tensor that an operator names is never allocated with a dimension of zero or less: the graph is
+    // UNPREDICTABLE (reference: subgraph_traverser.cpp:579-590, SubgraphTraverser::allocateTensor).
+    for (auto& n : nodes)
+        for (const std::vector<Tensor*>* list : { &n->inputs, &n->outputs })
+            for (Tensor* t : *list)
+                for (int32_t dim : t->getShape())
+                    if (dim <= 0)
+                    {
+                        last_message = "Failed to allocate tensor " + t->getName() + " with invalid dimension of " +
+                                       std::to_string(dim);
+                        setGraphStatus(GraphStatus::TOSA_UNPREDICTABLE);
+                        return 1;
+                    }
     return 0;
 }
 

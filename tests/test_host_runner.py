@@ -241,6 +241,19 @@ def test_exit_codes_unpredictable_and_error(tmp_path):
     r = _run(_write_case(d3, W.graph(ts, [W.operator(15, ["x", "x"], ["y"])], ["x"], ["y"]),
                          {"x": np.arange(4, dtype=np.int32)}, ["y"]))
     assert r.returncode == 2 and "outside the accelerated path" in r.stderr
+    # a tensor that an operator names with a dimension of zero: the reference never allocates it and calls the graph
+    # UNPREDICTABLE (subgraph_traverser.cpp:579-590) -> exit code 1, nothing written
+    x0 = np.zeros((0, 32, 32, 8), np.int8)
+    ts = [W.tensor("x", x0.shape, np.int8), W.tensor("w", c["w"].shape, np.int8, c["w"]),
+          W.tensor("bias", [16], np.int32, c["bias"]), W.tensor("z", [1], np.int8, [0]),
+          W.tensor("acc", [0, 32, 32, 16], np.int32)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "bias", "z")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "bias", "z", "z"], ["acc"], W.conv_attr([0, 0, 0, 0], [1, 1], [1, 1])))
+    d4 = tmp_path / "z"
+    d4.mkdir()
+    r = _run(_write_case(d4, W.graph(ts, ops, ["x"], ["acc"]), {"x": x0}, ["acc"]))
+    assert r.returncode == 1 and "UNPREDICTABLE" in r.stderr and "invalid dimension of 0" in r.stderr
+    assert not (d4 / "acc_out.npy").exists()
 
 
 @pytest.mark.gpu
