@@ -705,7 +705,10 @@ static int rescale_impl(const orc_rescale_attr_t* a, int64_t rows, int32_t C, co
                 /* INEXACT_ROUND with FP32 maths (:318-324), round to nearest even */
                 volatile float t = (float)v * (float)m;
                 volatile float u = t * exp2f((float)(-sh));
-                scaled           = (int32_t)rintf(u);
+                const float ri   = rintf(u);
+                /* outside the int32 range the reference's cast is undefined; its x86-64 builds return INT32_MIN
+                 * (cvtss2si's "integer indefinite"), stated here instead of left to the compiler */
+                scaled = (ri >= -2147483648.0f && ri < 2147483648.0f) ? (int32_t)ri : INT32_MIN;
             }
             if (status != ORC_VALID)
                 break;

@@ -147,7 +147,11 @@ __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t
     if (p.inexact_round)
     {
         const float t = (float)v * (float)m;
-        scaled        = (int32_t)rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
+        const float u = rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
+        // Outside the int32 range the reference's cast (type_conversion.cpp:323) is undefined; an x86-64 build of it
+        // returns INT32_MIN for every such value (the conversion instruction's "integer indefinite"), and so does
+        // this one, rather than the saturated value the device's own conversion would give.
+        scaled = (u >= -2147483648.0f && u < 2147483648.0f) ? (int32_t)u : INT32_MIN;
     }
     else if (p.scale32)
         scaled = apply_scale_32((int32_t)v, m, s, p.double_round, flags);

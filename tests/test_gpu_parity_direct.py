@@ -111,6 +111,27 @@ def test_rescale_dtype_matrix(ctx, in_dt, out_dt, in_u, out_u, in_zp, out_zp, sc
         assert np.array_equal(got.view(want.dtype), want), mode
 
 
+@pytest.mark.parametrize("in_dt", [np.int8, np.int16, np.int32])
+@pytest.mark.parametrize("out_dt,out_zp", [(np.int8, 60), (np.int16, 0), (np.int32, 0)])
+def test_rescale_inexact_round_with_products_beyond_int32(ctx, in_dt, out_dt, out_zp):
+    """INEXACT_ROUND over the whole input range with shifts small enough for float(value) * float(multiplier) * 2^-shift
+    to leave int32: the reference's cast is undefined there, its x86-64 builds return INT32_MIN, and the device
+    returns the same (not its own saturating conversion), so results and status agree element for element"""
+    rng = np.random.default_rng(np.dtype(in_dt).itemsize * 10 + np.dtype(out_dt).itemsize)
+    info = np.iinfo(in_dt)
+    x = rng.integers(info.min, info.max + 1, (40, 24)).astype(in_dt)
+    x.ravel()[:3] = [info.min, info.max, 0]
+    mult = rng.integers(1 << 30, 1 << 31, 24).astype(np.int32)
+    shift = rng.integers(2, 40, 24).astype(np.int8)
+    kw = dict(out_zp=out_zp, out_dtype=out_dt, rounding_mode=capi.ROUND_INEXACT)
+    want, wst = oracle.rescale(x, mult, shift, **kw)
+    got, st = gpu_ops.rescale(ctx, x, mult, shift, **kw)
+    assert st == wst == capi.VALID
+    assert np.array_equal(got, want)
+    if out_dt == np.int32:
+        assert (want == -(1 << 31)).sum() > 20    # the case is there
+
+
 def test_rescale_reference_literals(ctx):  # type_conversion_tests.cpp:324-335, 385-405
     for mode in (capi.ROUND_SINGLE, capi.ROUND_INEXACT):
         got, st = gpu_ops.rescale(ctx, np.array([65], np.int8), [4], [2], in_zp=1, out_zp=32768, out_dtype=np.uint16,

@@ -171,6 +171,23 @@ def test_rescale_inexact_round_literals():  # type_conversion_tests.cpp:385-405
     assert st == oracle.VALID and out.tolist() == [114]
 
 
+def test_rescale_inexact_round_is_float_arithmetic_and_names_its_overflow_value():
+    """INEXACT_ROUND is float(value) * float(multiplier) * 2^-shift rounded to nearest even (type_conversion.cpp:320-323),
+    checked against numpy float32; a product outside int32 makes the reference's cast undefined, and the value its
+    x86-64 builds return, INT32_MIN, is what the oracle states"""
+    rng = np.random.default_rng(5)
+    x = rng.integers(-(1 << 20), 1 << 20, (50, 8)).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, 8).astype(np.int32)
+    shift = rng.integers(30, 45, 8).astype(np.int32)
+    out, st = oracle.rescale(x, mult, shift, out_dtype=np.int32, rounding_mode=oracle.ROUND_INEXACT)
+    want = np.rint((x.astype(np.float32) * mult.astype(np.float32)) * np.exp2(-shift.astype(np.float32)))
+    assert st == oracle.VALID and np.array_equal(out, want.astype(np.int64))
+    big = np.array([[(1 << 31) - 1, -(1 << 31), 100000, -100000, 8192, 3]], np.int32)
+    out, st = oracle.rescale(big, [1803664250], [12], out_dtype=np.int32, rounding_mode=oracle.ROUND_INEXACT,
+                             per_channel=False)
+    assert st == oracle.VALID and out.tolist() == [[-(1 << 31)] * 5 + [1321043]]
+
+
 @pytest.mark.parametrize("inp,mult,shift,kw", [  # type_conversion_tests.cpp:337-383
     (np.array([20, -5, -16], np.int8), [4, 2], [16, 5, 9], dict(scale32=True, per_channel=True, in_zp=-19,
                                                                   out_dtype=np.int32)),
