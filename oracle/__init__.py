@@ -385,6 +385,8 @@ def avg_pool2d(inp, kernel, stride=(1, 1), pad=(0, 0, 0, 0), in_zp=0, out_zp=0, 
     inp = np.asarray(inp)
     s = _pool_shape(inp, kernel, stride, pad, out_hw)
     shape = (s.N, max(s.OH, 0), max(s.OW, 0), s.C)
+    if inp.dtype != np.int8 and (in_zp != 0 or out_zp != 0):
+        raise OracleStatus(ERROR)    # zero points belong to int8 only (tensor_ops.cpp:568-571)
     if inp.dtype.kind == "i":
         info = np.iinfo(inp.dtype)
         x, out = _c(inp, np.int32), np.zeros(shape, np.int32)

@@ -141,3 +141,13 @@ def test_pool_attribute_errors(kernel, stride, pad, out_hw):
     for fn in (oracle.avg_pool2d, oracle.max_pool2d):
         with pytest.raises(oracle.OracleStatus):
             fn(x, kernel, stride, pad, out_hw=out_hw)
+
+
+def test_avg_pool_zero_points_are_for_int8_only():
+    """OpAvgPool2d::eval, tensor_ops.cpp:568-571: a zero point other than 0 with int16 or floating-point data is an error"""
+    for x in (np.zeros((1, 4, 4, 2), np.int16), np.zeros((1, 4, 4, 2), np.float32)):
+        for zps in ((5, 0), (0, -3)):
+            with pytest.raises(oracle.OracleStatus):
+                oracle.avg_pool2d(x, (2, 2), (2, 2), (0, 0, 0, 0), *zps)
+    assert oracle.avg_pool2d(np.full((1, 4, 4, 2), 7, np.int8), (2, 2), (2, 2), (0, 0, 0, 0), 5, -3).tolist() == \
+        np.full((1, 2, 2, 2), -1, np.int8).tolist()
