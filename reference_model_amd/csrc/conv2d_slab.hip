@@ -81,7 +81,10 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
 // slices: the patch loader takes chunk group kd of a pixel from input slice od * sd + kd * dd - pd0 (a slice outside
 // the volume reads the input_zp page), and the weights stay in their own [OC][KD][KH][KW][IC] order, a K step
 // (tap, kd, half) finding its place in the row at compile time.  Neither operand is copied.
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1>
+// NPT: accumulator tiles (of 32 columns) per wave.  Two of them share every weight fragment, which cuts the LDS
+// traffic of the K loop by a quarter; the workgroup's tile is then up to 252 pixels, which only pays when the layer
+// has more tiles than the chip has CUs.
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
@@ -260,28 +263,39 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 
     // ---- MFMA: wave = (channel tile, pixel tile) ---------------------------------------------------------------
     const int oct = wave >> 2, pxt = wave & 3;
-    // A wave's 32 MFMA columns are 31 pixels and, in column 31, the zero-point pixel: its accumulators are
+    // A wave's first 32 MFMA columns are 31 pixels and, in column 31, the zero-point pixel: its accumulators are
     // input_zp * sum(w) of the wave's 32 channels, for the price of nothing (the column would be computed anyway).
-    constexpr int PXW = 31;
-    const int P       = a.TH * a.TW;
-    int p             = pxt * PXW + li;
-    const bool p_in_tile = li < PXW && p < P;
-    p                 = p_in_tile ? p : 0;
-    const int ty  = fdiv(p, a.div_tw);
-    const int tx  = p - ty * a.TW;
+    // A second accumulator tile (NPT = 2) holds 32 more pixels.
+    constexpr int PXW  = 31;
+    constexpr int WPIX = PXW + 32 * (NPT - 1);    // pixels of a wave
+    const int P        = a.TH * a.TW;
+    bool p_in_tile[NPT];
+    int ty[NPT], tx[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; k++)
+    {
+        int p        = pxt * WPIX + (k ? PXW + 32 * (k - 1) : 0) + li;
+        p_in_tile[k] = (k || li < PXW) && p < P;
+        p            = p_in_tile[k] ? p : 0;
+        ty[k]        = fdiv(p, a.div_tw);
+        tx[k]        = p - ty[k] * a.TW;
+    }
     // The accumulators start at the bias of the lane's 16 channels (the zero-point column at zero).
     const int ocl = oct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
-    v16i acc;
+    v16i acc[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; k++)
     {
-        const int32_t* b16 = tab_b + ((ZA && li == PXW) ? 64 : ocl);
+        const int32_t* b16 = tab_b + ((ZA && k == 0 && li == PXW) ? 64 : ocl);
 #pragma unroll
         for (int q = 0; q < 4; q++)
         {
             const v4i b4 = *reinterpret_cast<const v4i*>(b16 + 4 * q);
-            acc[4 * q] = b4[0], acc[4 * q + 1] = b4[1], acc[4 * q + 2] = b4[2], acc[4 * q + 3] = b4[3];
+            acc[k][4 * q] = b4[0], acc[k][4 * q + 1] = b4[1], acc[k][4 * q + 2] = b4[2], acc[k][4 * q + 3] = b4[3];
         }
     }
-    const bool wave_active = pxt * PXW < P;    // wave-uniform
+    const bool wave_active = pxt * WPIX < P;                     // wave-uniform
+    const bool second_active = NPT > 1 && pxt * WPIX + PXW < P;  // wave-uniform: the second tile has a pixel
     if (wave_active)
     {
         // MFMA operand row li holds channel 16*((li>>2)&1) + 4*(li>>3) + (li&3) of the wave's 32: a lane's 16
@@ -289,15 +303,19 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         // rows that differ modulo 16, which the odd row stride turns into 16 different bank groups.)
         const int wr        = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
         const uint8_t* wrow = wl + ((oct * 32 + wr) * RW) * 16 + lh * 16;
-        const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * RP) * 16 + lh * 16;
+        const uint8_t* prow[NPT];
+#pragma unroll
+        for (int k = 0; k < NPT; k++)
+            prow[k] = pl + (ty[k] * a.sy * a.pitch + tx[k] * a.sx * RP) * 16 + lh * 16;
         if (ZA && li == PXW)
-            prow = ones + lh * 16;
+            prow[0] = ones + lh * 16;
         // K step s = (tap s / (CH/2), half s % (CH/2)).  The fragments of step s + DEPTH are requested before the
         // MFMA of step s and the order is pinned: an LDS read takes several MFMA times to come back with eight waves
         // asking, and left alone the scheduler requests a step's fragments only one MFMA ahead.
         constexpr int STEPS = TAPS * (CH / 2);
-        constexpr int DEPTH = STEPS < 8 ? STEPS : 8;
-        v4i fa[STEPS], fb[STEPS];
+        constexpr int AHEAD = NPT > 1 ? 5 : 8;    // two tiles: fewer steps ahead, to stay within 128 registers
+        constexpr int DEPTH = STEPS < AHEAD ? STEPS : AHEAD;
+        v4i fa[STEPS], fb[NPT][STEPS];
         auto request = [&](int s) {
             const int tap = s / (CH / 2), h = s % (CH / 2);
             const int at  = TC ? TAPS - 1 - tap : tap;    // flipped taps: weight tap (ky, kx) meets patch tap (KH-1-ky, KW-1-kx)
@@ -308,7 +326,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 aoff              = (((h / ICH) * TAPS + tap) * ICH + h % ICH) * 32;
             }
             fa[s] = *reinterpret_cast<const v4i*>(wrow + aoff);
-            fb[s] = *reinterpret_cast<const v4i*>(prow + (at / KW) * row_step + (at % KW) * col_step + h * 32);
+#pragma unroll
+            for (int k = 0; k < NPT; k++)
+                fb[k][s] = *reinterpret_cast<const v4i*>(prow[k] + (at / KW) * row_step + (at % KW) * col_step + h * 32);
         };
 #pragma unroll
         for (int s = 0; s < DEPTH; s++)
@@ -319,7 +339,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         {
             if (s + DEPTH < STEPS)
                 request(s + DEPTH);
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
+#pragma unroll
+            for (int k = 0; k < NPT; k++)
+                acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[k][s], acc[k], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -328,16 +350,27 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     // (lane, register 4q + j) = D[row 8q + 4 lh + j][pixel li] = channel 32 oct + 16 lh + 4q + j
     if constexpr (ZA)
     {
-        // Lane 31 + 32 lh holds in register e the zero-point column for channel 16 lh + e: input_zp * sum(w) of
-        // exactly the channel this lane has in register e.
+        // Lane 31 + 32 lh of the first tile holds in register e the zero-point column for channel 16 lh + e:
+        // input_zp * sum(w) of exactly the channel this lane has in register e (of either tile).
         const int src = (PXW + 32 * lh) * 4;
 #pragma unroll
         for (int e = 0; e < 16; e++)
-            acc[e] -= __builtin_amdgcn_ds_bpermute(src, acc[e]);
+        {
+            const int zsum = __builtin_amdgcn_ds_bpermute(src, acc[0][e]);
+#pragma unroll
+            for (int k = 0; k < NPT; k++)
+                acc[k][e] -= zsum;
+        }
     }
-    const int oy = oy0 + ty, ox = ox0 + tx;
-    const bool pix_ok  = p_in_tile && wave_active && oy < a.OH && ox < a.OW;
     const bool chan_ok = oc0 + ocl < a.OC;    // OC is a multiple of 16: a lane's 16 channels are in or out together
+#pragma unroll
+    for (int k = 0; k < NPT; k++)
+    {
+    if (k > 0 && !second_active)
+        break;
+    const v16i& acck = acc[k];
+    const int oy = oy0 + ty[k], ox = ox0 + tx[k];
+    const bool pix_ok  = p_in_tile[k] && wave_active && oy < a.OH && ox < a.OW;
     // the tensor has fewer than 2^31 elements (checked by the launcher): 32-bit arithmetic, scalar where it can be
     const size_t obase = (uint32_t)(((n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl);
     if constexpr (!FUSED)
@@ -347,7 +380,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             int32_t* o = reinterpret_cast<int32_t*>(a.out) + obase;
 #pragma unroll
             for (int q = 0; q < 4; q++)
-                *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3] };
+                *reinterpret_cast<v4i*>(o + 4 * q) = v4i{ acck[4 * q], acck[4 * q + 1], acck[4 * q + 2], acck[4 * q + 3] };
         }
     }
     else
@@ -375,13 +408,13 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             {
 #pragma unroll
                 for (int e = 0; e < 16; e++)
-                    r[e] = clamp_med3(high_word_rescale<true>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+                    r[e] = clamp_med3(high_word_rescale<true>(acck[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
             }
             else
             {
 #pragma unroll
                 for (int e = 0; e < 16; e++)
-                    r[e] = clamp_med3(high_word_rescale<false>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+                    r[e] = clamp_med3(high_word_rescale<false>(acck[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
             }
         }
         else if (s_uni == -2)
@@ -392,7 +425,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 for (int e = 0; e < 16; e++)
                 {
                     const HighWordScale c = tab_hw[ocl + e];
-                    r[e] = clamp_med3(high_word_rescale<true>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                    r[e] = clamp_med3(high_word_rescale<true>(acck[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
                 }
             }
             else
@@ -401,7 +434,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 for (int e = 0; e < 16; e++)
                 {
                     const HighWordScale c = tab_hw[ocl + e];
-                    r[e] = clamp_med3(high_word_rescale<false>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                    r[e] = clamp_med3(high_word_rescale<false>(acck[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
                 }
             }
         }
@@ -412,7 +445,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             for (int e = 0; e < 16; e++)
             {
                 const ChannelScale cs = tab_cs[ocl + e];
-                r[e]                  = fast_rescale(acc[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
+                r[e]                  = fast_rescale(acck[e], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
             }
             if (pix_ok && chan_ok)
                 flags |= eflags;    // pixels and channels outside the tensor raise nothing
@@ -447,15 +480,16 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             }
         }
     }
+    }
     raise_flags(a.flag_word, flags);
 }
 
 thread_local int32_t last_launch_shape[3] = { 0, 0, 0 };
 
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1>
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
-    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC, KD>;
+    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC, KD, NPT>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
@@ -465,8 +499,16 @@ static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int 
 }
 
 template <int KH, int KW, int CH>
-static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, bool fused)
+static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, bool fused, bool wide)
 {
+    if (wide)
+    {
+        if (a.za != 0)
+            return fused ? launch_slab_kernel<KH, KW, CH, true, true, false, 1, 2>(st, a, grid, lds_bytes)
+                         : launch_slab_kernel<KH, KW, CH, true, false, false, 1, 2>(st, a, grid, lds_bytes);
+        return fused ? launch_slab_kernel<KH, KW, CH, false, true, false, 1, 2>(st, a, grid, lds_bytes)
+                     : launch_slab_kernel<KH, KW, CH, false, false, false, 1, 2>(st, a, grid, lds_bytes);
+    }
     if (a.za != 0)
         return fused ? launch_slab_kernel<KH, KW, CH, true, true>(st, a, grid, lds_bytes)
                      : launch_slab_kernel<KH, KW, CH, true, false>(st, a, grid, lds_bytes);
@@ -505,37 +547,61 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     // The tile: at most 124 pixels (four tiles of 31 pixels, one per wave and channel tile).  A workgroup moves the
     // weight slab (taps * 64 rows of 64 bytes) plus PH * PW patch rows; whole rounds of 256 workgroups count.
     // The search depends on the geometry only; a caller repeats the same layer, so the last answer is kept.
+    //
+    // Layers of unit stride with more such tiles than the chip has CUs run the two-tiles-per-wave form on tiles of
+    // up to 252 pixels instead.  Measured on MI355X, us with one / two tiles per wave (graph replays, fused RESCALE):
+    // 3x3 [32,56,56,64]->64 10.5 / 8.6, [64,..] 17.5 / 15.1, [20,..] 8.2 / 7.7, [16,..] 6.0 / 5.8, [10,..] 5.4 / 5.3,
+    // [8,56,56,128]->128 9.7 / 7.9, [32,28,28,128]->128 9.4 / 7.9, [64,14,14,128]->256 9.6 / 7.6; 1x1
+    // [8,56,56,64]->256 6.6 / 5.9, [32,..] 17.6 / 16.9, [16,28,28,128]->512 6.8 / 6.1, [32,..] 11.8 / 12.1;
+    // a single round of the small tiles is faster with them ([8,56,56,64]->64 4.3 / 5.1, [16,28,28,128]->128 5.5 / 6.4),
+    // and so is stride 2, whose patch grows with the tile ([32,57,57,128]->64 9.5 / 11.7).
     const int n_ocb = (g.OC + 63) / 64;
     const int ch = g.IC / 16, rp_chunks = ch + 1;    // chunks of a channel vector; chunks per patch pixel in LDS
     struct TileChoice
     {
         int32_t key[8];
         int th, tw;
+        bool wide;
     };
-    static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0 };
-    const int32_t key[8] = { g.N, g.OH, g.OW, (n_ocb * 256 + ch) * 4 + g.KH, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
+    static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0, false };
+    const int32_t key[8] = { g.N, g.OH, g.OW, ((n_ocb * 256 + ch) * 4 + g.KH) * 2 + ((tc || c3d) ? 1 : 0), g.stride_y, g.stride_x,
+                             g.dil_y, g.dil_x };
     int best_th = 0, best_tw = 0;
+    bool wide = false;
     if (memcmp(key, last.key, sizeof(key)) == 0)
-        best_th = last.th, best_tw = last.tw;
+        best_th = last.th, best_tw = last.tw, wide = last.wide;
     else
     {
-        int64_t best_cost = 0;
-        for (int th = 1; th <= g.OH && th <= 124; th++)
-            for (int tw = 1; tw <= g.OW && th * tw <= 124; tw++)
-            {
-                const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
-                const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
-                if (ph * (pw * rp_chunks + 15) >= (1 << 16) || ph * (pw * rp_chunks + 15) * 16 > 64 * 1024)
-                    continue;
-                const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
-                const int64_t rounds = (tiles + 255) / 256;
-                // a round costs its loads plus the four 32-pixel MFMA tiles whether they are full or not
-                const int64_t cost = rounds * ((taps * 64 + ph * pw) * ch / 4 + 600);
-                if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
-                    best_th = th, best_tw = tw, best_cost = cost;
-            }
+        int64_t best_rounds = 0;
+        auto search = [&](int max_pix, int64_t fixed) {
+            int64_t best_cost = 0;
+            best_th = best_tw = 0;
+            for (int th = 1; th <= g.OH && th <= max_pix; th++)
+                for (int tw = 1; tw <= g.OW && th * tw <= max_pix; tw++)
+                {
+                    const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+                    const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
+                    if (ph * (pw * rp_chunks + 15) >= (1 << 16) || ph * (pw * rp_chunks + 15) * 16 > 64 * 1024)
+                        continue;
+                    const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
+                    const int64_t rounds = (tiles + 255) / 256;
+                    // a round costs its loads plus its 32-pixel MFMA tiles whether they are full or not
+                    const int64_t cost = rounds * ((taps * 64 + ph * pw) * ch / 4 + fixed);
+                    if (!best_th || cost < best_cost || (cost == best_cost && th * tw > best_th * best_tw))
+                        best_th = th, best_tw = tw, best_cost = cost, best_rounds = rounds;
+                }
+        };
+        search(124, 600);
+        if (best_th && best_rounds > 1 && g.stride_y == 1 && g.stride_x == 1 && !tc && !c3d)
+        {
+            const int th1 = best_th, tw1 = best_tw;
+            search(252, 1100);
+            wide = best_th != 0;
+            if (!wide)
+                best_th = th1, best_tw = tw1;
+        }
         memcpy(last.key, key, sizeof(key));
-        last.th = best_th, last.tw = best_tw;
+        last.th = best_th, last.tw = best_tw, last.wide = wide;
     }
     if (!best_th)
         return nullptr;
@@ -615,13 +681,13 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
         return ok ? "transpose_conv2d_slab_i8" : nullptr;
     }
     if (k33)
-        ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused)
-                     : (ch == 6 ? launch_slab_taps<3, 3, 6>(st, a, (int)grid, lds_bytes, fused)
-                                : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused));
+        ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused, wide)
+                     : (ch == 6 ? launch_slab_taps<3, 3, 6>(st, a, (int)grid, lds_bytes, fused, wide)
+                                : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused, wide));
     else
-        ok = ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused)
-                     : (ch == 6 ? launch_slab_taps<1, 1, 6>(st, a, (int)grid, lds_bytes, fused)
-                                : launch_slab_taps<1, 1, 8>(st, a, (int)grid, lds_bytes, fused));
+        ok = ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused, wide)
+                     : (ch == 6 ? launch_slab_taps<1, 1, 6>(st, a, (int)grid, lds_bytes, fused, wide)
+                                : launch_slab_taps<1, 1, 8>(st, a, (int)grid, lds_bytes, fused, wide));
     if (!ok)
         return nullptr;
     return rp.enabled ? "conv2d_slab_i8_rescale" : "conv2d_slab_i8";

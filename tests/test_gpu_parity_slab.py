@@ -35,6 +35,12 @@ SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation[, ic: 64 unless given]
     (2, 19, 17, 80, (1, 0, 2, 1), (1, 1), (1, 1), 128),     # ragged tiles and channel block
     (2, 29, 29, 64, (1, 1, 1, 1), (2, 2), (1, 1), 128),     # stride 2
     (3, 21, 22, 64, (1, 1, 1, 1), (1, 1), (1, 1), 96),      # 96 input channels: three MFMA steps per tap
+    # unit stride and more 124-pixel tiles than the chip has CUs: two accumulator tiles per wave on tiles of up to 252 pixels
+    (20, 37, 41, 64, (1, 1, 1, 1), (1, 1), (1, 1)),         # ragged tiles
+    (12, 50, 50, 80, (1, 0, 1, 2), (1, 1), (1, 1), 128),    # 128 input channels, a ragged second channel block
+    (70, 14, 14, 128, (1, 1, 1, 1), (1, 1), (1, 1)),        # one tile per image: the last wave's second tile is empty
+    (24, 40, 40, 64, (2, 2, 2, 2), (1, 1), (2, 2)),         # dilation 2
+    (28, 36, 36, 64, (1, 1, 1, 1), (1, 1), (1, 1), 96),     # 96 input channels
 ]
 
 
@@ -112,6 +118,8 @@ def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
     (4, 29, 29, 128, 64, (0, 0, 0, 0), (2, 2)),         # a down-sampling shortcut
     (4, 28, 28, 96, 64, (0, 0, 0, 0), (1, 1)),          # a MobileNet projection layer
     (3, 17, 13, 64, 80, (1, 0, 0, 2), (1, 1)),          # padding on a pointwise layer: the border is bias only
+    (9, 61, 47, 64, 192, (0, 0, 0, 0), (1, 1)),         # two accumulator tiles per wave, ragged tiles
+    (5, 33, 35, 128, 320, (1, 0, 0, 2), (1, 1)),        # the same with padding and five channel blocks
 ])
 @pytest.mark.parametrize("in_zp", [0, -7])
 def test_slab_pointwise_layers_bit_exact(ctx, shape, in_zp):
@@ -144,6 +152,24 @@ def test_slab_config3_full_size(ctx):
     acc = cases.conv2d_exact_blas(c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
     want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
     assert wst == oracle.VALID and np.array_equal(got, oracle.clamp(want, *c["clamp"]))
+
+
+def test_slab_tile_width_follows_the_number_of_tiles(ctx):
+    """a single round of 124-pixel tiles keeps one accumulator tile per wave; more tiles than CUs at unit stride get
+    the two-tile form on tiles of up to 252 pixels (fewer, larger workgroups); stride 2 never does"""
+    rng = np.random.default_rng(3)
+
+    def grid_of(n, hw, stride):
+        x = rng.integers(-128, 128, (n, hw, hw, 64)).astype(np.int8)
+        w = rng.integers(-128, 128, (64, 3, 3, 64)).astype(np.int8)
+        bias = np.zeros(64, np.int32)
+        _, st = gpu_ops.conv2d(ctx, x, w, bias, (1, 1, 1, 1), (stride, stride), in_zp=-7, w_zp=0)
+        assert st == capi.VALID and ctx.last_kernel == "conv2d_slab_i8"
+        return ctx.last_launch_shape()[0]
+
+    assert grid_of(8, 56, 1) == 256          # 7 x 14 tiles, 32 per image
+    assert grid_of(32, 56, 1) == 512         # 14 x 14 tiles, 16 per image, instead of 1024 tiles of 7 x 14
+    assert grid_of(32, 57, 2) > 32 * 29 * 29 // 252 * 2    # stride 2: tiles of at most 124 pixels
 
 
 @pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
