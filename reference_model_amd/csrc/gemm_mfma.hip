@@ -613,6 +613,18 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         }
         __syncthreads();
     }
+    // Four-byte results (int32, fp32) whose rows are whole 128-byte lines per channel tile leave through LDS: a lane
+    // holds 64 bytes of one pixel's row, so a store instruction straight from the accumulators is 64 separate
+    // 16-byte requests to the L2 (4.2 M of them for the named bf16 MATMUL, which kept its 256 workgroups storing
+    // for 22 us at the end); transposed through a per-wave 4.5 KB buffer, an instruction writes 8 whole lines.
+    // (The buffer lies in the stage memory: every wave must be done with its fragments first.)
+    const bool wide_out = M::is_int ? !(!APAIR && a.rp.enabled) : a.out_is_wide != 0;
+    const bool lines    = wide_out && (a.N & 31) == 0;
+    if constexpr (!(ZP || APAIR))
+        if (lines)
+            __syncthreads();
+    constexpr int TPITCH = 144;    // bytes per pixel row in the buffer: 128 + 16, so that rows spread over the banks
+    uint8_t* tbuf        = lds + 8192 + wave * (32 * TPITCH);
 
     // A lane's 16 accumulator registers of a tile are four groups of 4 consecutive channels: group q starts at
     // channel 16h + 4q (all 16 consecutive), or 8q + 4h with the in-order row assignment.
@@ -646,6 +658,39 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         for (int i = 0; i < PXT; i++)
         {
             const int p = p0 + wp * 32 * PXT + i * 32 + rho;
+            if (lines)
+            {
+                const int pt0 = p0 + wp * 32 * PXT + i * 32;    // the tile's first pixel row
+                if (pt0 >= a.M || oc0 + tl >= a.N)
+                    continue;
+                int w4[16];
+                if constexpr (M::is_int)
+                {
+                    const int pcorr = ZP ? a.zw * psum[i] : 0;
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        w4[e] = acc[i][t][e] + cb[e] - pcorr;
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 16; e++)
+                        w4[e] = __float_as_int(acc[i][t][e] + __int_as_float(cb[e]));
+                }
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    *reinterpret_cast<v4i*>(tbuf + rho * TPITCH + group_channel(q) * 4) =
+                        v4i{ w4[4 * q], w4[4 * q + 1], w4[4 * q + 2], w4[4 * q + 3] };
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                {
+                    const int row = (lane >> 3) + 8 * j, piece = lane & 7;
+                    const v4i d   = *reinterpret_cast<const v4i*>(tbuf + row * TPITCH + piece * 16);
+                    if (pt0 + row < a.M)
+                        *reinterpret_cast<v4i*>(out_b + ((size_t)(pt0 + row) * a.N + oc0 + tl) * 4 + piece * 16) = d;
+                }
+                continue;
+            }
             if (p >= a.M || oc0 + tl >= a.N)
                 continue;
             if constexpr (M::is_int)
