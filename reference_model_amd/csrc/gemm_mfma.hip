@@ -620,11 +620,17 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     // (The buffer lies in the stage memory: every wave must be done with its fragments first.)
     const bool wide_out = M::is_int ? !(!APAIR && a.rp.enabled) : a.out_is_wide != 0;
     const bool lines    = wide_out && (a.N & 31) == 0;
+    // Floating-point results of the input type (2 bytes): a pixel's OCT x 32 channels are 128 or 256 bytes, gathered
+    // from all the wave's channel tiles before they leave.
+    constexpr int HROW   = OCT * 64;    // bytes of a pixel's channels held by this wave
+    constexpr int HPITCH = HROW + 16;
+    const bool half_lines = !M::is_int && !wide_out && (a.N & 63) == 0 && oc0 + (wo + 1) * 32 * OCT <= a.N;
+    const bool any_half_lines = !M::is_int && !wide_out && (a.N & 63) == 0;    // the same for every wave
     if constexpr (!(ZP || APAIR))
-        if (lines)
+        if (lines || any_half_lines)
             __syncthreads();
     constexpr int TPITCH = 144;    // bytes per pixel row in the buffer: 128 + 16, so that rows spread over the banks
-    uint8_t* tbuf        = lds + 8192 + wave * (32 * TPITCH);
+    uint8_t* tbuf        = lds + 8192 + wave * (32 * (HPITCH > TPITCH ? HPITCH : TPITCH));
 
     // A lane's 16 accumulator registers of a tile are four groups of 4 consecutive channels: group q starts at
     // channel 16h + 4q (all 16 consecutive), or 8q + 4h with the in-order row assignment.
@@ -632,6 +638,48 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     const bool rows16 = (a.N & 15) == 0;    // every lane's 16 channels are inside the tensor or all outside
     const bool rows4  = (a.N & 3) == 0;     // the same for a group of 4
     uint8_t* out_b    = reinterpret_cast<uint8_t*>(a.out) + batch * a.o_batch;
+    if constexpr (!M::is_int)
+    {
+        if (half_lines)
+        {
+#pragma unroll
+            for (int i = 0; i < PXT; i++)
+            {
+                const int pt0 = p0 + wp * 32 * PXT + i * 32;    // the tile's first pixel row
+                if (pt0 >= a.M)
+                    continue;
+#pragma unroll
+                for (int t = 0; t < OCT; t++)
+                {
+                    const int tl = wo * 32 * OCT + t * 32;
+                    alignas(16) T packed[16];
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                    {
+                        const v4i b = *reinterpret_cast<const v4i*>(tab_bias + tl + 16 * h + 4 * q);
+                        store_from_float(packed + 4 * q, acc[i][t][4 * q] + __int_as_float(b.x));
+                        store_from_float(packed + 4 * q + 1, acc[i][t][4 * q + 1] + __int_as_float(b.y));
+                        store_from_float(packed + 4 * q + 2, acc[i][t][4 * q + 2] + __int_as_float(b.z));
+                        store_from_float(packed + 4 * q + 3, acc[i][t][4 * q + 3] + __int_as_float(b.w));
+                    }
+                    uint8_t* d = tbuf + rho * HPITCH + t * 64 + h * 32;
+                    reinterpret_cast<v4i*>(d)[0] = reinterpret_cast<const v4i*>(packed)[0];
+                    reinterpret_cast<v4i*>(d)[1] = reinterpret_cast<const v4i*>(packed)[1];
+                }
+                constexpr int PIECES = HROW / 16;      // 16-byte pieces per pixel row: 8 or 16
+                constexpr int RPI    = 64 / PIECES;    // rows per store instruction
+#pragma unroll
+                for (int j = 0; j < 32 / RPI; j++)
+                {
+                    const int row = lane / PIECES + RPI * j, piece = lane % PIECES;
+                    const v4i d   = *reinterpret_cast<const v4i*>(tbuf + row * HPITCH + piece * 16);
+                    if (pt0 + row < a.M)
+                        *reinterpret_cast<v4i*>(out_b + ((size_t)(pt0 + row) * a.N + oc0 + wo * 32 * OCT) * 2 + piece * 16) = d;
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int t = 0; t < OCT; t++)
     {
