@@ -57,6 +57,12 @@ struct GemmArgs
     int32_t sy, sx, dy, dx, pad_top, pad_left;
     FastDiv div_bpt, div_kw;
     FastDiv div_batch, div_tn;
+    // patch mode: a tile is rows_per_tile whole output rows of one image; its input patch stays in LDS
+    int32_t rows_per_tile, tiles_per_image;
+    int32_t patch_w, patch_pixels;    // patch width in pixels, pixels of the patch
+    int32_t patch_units;              // 64-byte units of the patch = bpt * patch_pixels
+    int32_t patch_bytes;              // LDS the patch takes
+    FastDiv div_tpi, div_pw, div_ppix, div_ow;
 };
 
 
@@ -102,7 +108,8 @@ enum
 {
     GEMM_KCONTIG = 0,
     GEMM_KMAJOR  = 1,
-    GEMM_TAPS    = 2
+    GEMM_TAPS    = 2,
+    GEMM_PATCH   = 3
 };
 
 enum
@@ -121,6 +128,12 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     static_assert(!APAIR || (MODE == GEMM_KMAJOR && kStages == 4), "pixel pairs: K-major weights in a ring of four");
     constexpr bool KM      = MODE == GEMM_KMAJOR;
     constexpr bool TAPS    = MODE == GEMM_TAPS;
+    // PATCH: a convolution with taps whose tile is whole output rows of one image.  The input patch under the tile
+    // (with its halo; pixels outside the image come from the page of input_zp bytes) is fetched once, as planes of
+    // 64-byte pieces, and stays in LDS behind the ring; the ring holds weight rows only, and the pixel fragments of
+    // block (tap, piece) are read from plane `piece` at the tap's offset.
+    constexpr bool PATCH   = MODE == GEMM_PATCH;
+    static_assert(!PATCH || (PIPE == PIPE_PAIRS && PXT == 1), "the patch form: pairs of weight blocks, 128 pixel rows");
     using M                = Mma<T>;
     constexpr int EB       = (int)sizeof(T);
     constexpr bool IDENT   = KM && EB == 1;    // accumulator row r of a channel tile is channel r
@@ -139,7 +152,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     using acc_t            = typename M::acc_t;
     constexpr int WROWS    = 64 * OCT;
     constexpr int PROWS    = 128 * PXT;
-    constexpr int ROWS     = WROWS + PROWS;
+    constexpr int ROWS     = PATCH ? WROWS : WROWS + PROWS;    // rows of a ring stage
     constexpr int STAGE    = ROWS * 64;
     constexpr int LOADS    = ROWS / 128;    // direct loads per wave and block (16 rows each)
     constexpr int WLOADS   = WROWS / 128;   // of which carry weight rows
@@ -166,7 +179,17 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     const int rem   = L - batch * a.tiles_per_batch;
     const int tm    = (int)fdiv((uint32_t)rem, a.div_tn);
     const int tn    = rem - tm * a.tiles_n;
-    const int p0    = tm * PROWS;
+    int p0          = tm * PROWS;
+    int m_end       = a.M;    // pixel rows of the tile end here
+    int patch_n = 0, patch_oy0 = 0;
+    if constexpr (PATCH)
+    {
+        patch_n             = (int)fdiv((uint32_t)tm, a.div_tpi);
+        patch_oy0           = (tm - patch_n * a.tiles_per_image) * a.rows_per_tile;
+        const int rows_here = a.OH - patch_oy0 < a.rows_per_tile ? a.OH - patch_oy0 : a.rows_per_tile;
+        p0                  = (patch_n * a.OH + patch_oy0) * a.OW;
+        m_end               = p0 + rows_here * a.OW;
+    }
     const int oc0   = tn * WROWS;
 
     const uint8_t* a_base = a.a + batch * a.a_batch;
@@ -270,6 +293,33 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     auto issue_pair = [&](int block, int q) {
         issue_one(block + (q & 1), block + (q & 1), q >> 1);    // prologue: stage = block
     };
+    // PATCH: the patch first (loads complete in the order they were issued, so the wait for the first weight blocks
+    // covers it).  Unit u = plane (u / patch_pixels), pixel (u % patch_pixels); a wave instruction moves 16 units.
+    constexpr int PATCH_OFF = kStages * STAGE;
+    if constexpr (PATCH)
+    {
+        const int iy0 = patch_oy0 * a.sy - a.pad_top;
+        const uint32_t dst0 =
+            (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds + PATCH_OFF + wave * 1024;
+#pragma unroll 1
+        for (int u0 = 0; u0 < a.patch_units; u0 += 128)
+        {
+            const int u       = u0 + wave * 16 + (lane >> 2);
+            const int plane   = (int)fdiv((uint32_t)u, a.div_ppix);
+            const int pix     = u - plane * a.patch_pixels;
+            const int r       = (int)fdiv((uint32_t)pix, a.div_pw);
+            const int c       = pix - r * a.patch_w;
+            const int iy      = iy0 + r, ix = c - a.pad_left;
+            const bool inside = iy >= 0 && iy < a.IH && ix >= 0 && ix < a.IW;
+            const uint8_t* src =
+                inside ? a_base + (ptrdiff_t)(((patch_n * a.IH + iy) * a.IW + ix) * a.icb + plane * 64 +
+                                              (((lane & 3) ^ swz(pix)) * 16))
+                       : a.pad_page + (lane & 3) * 16;
+            const uint32_t dst = dst0 + (uint32_t)u0 * 64;
+            if (u < a.patch_units)    // (lanes past the last unit write nothing)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory");
+        }
+    }
     if constexpr (PAIR)
     {
 #pragma unroll
@@ -305,7 +355,8 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
 
     // ---- tables: bias per channel of the tile (in the shadow of the first loads) ---------------------------
     // (PIXEL_PAIRS fills the LDS with operands: its bias table is written after the loop, into a free stage)
-    int* tab_bias = reinterpret_cast<int*>(APAIR ? lds + 4096 : lds + kStages * STAGE);    // WROWS words
+    uint8_t* tables = lds + kStages * STAGE + (PATCH ? a.patch_bytes : 0);
+    int* tab_bias   = reinterpret_cast<int*>(APAIR ? lds + 4096 : tables);    // WROWS words
     auto write_bias_table = [&]() {
         if (tid >= WROWS)
             return;
@@ -324,7 +375,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         write_bias_table();
 
     // per-channel constants of the fused RESCALE, derived once per workgroup (WROWS entries of 32 bytes)
-    ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(lds + kStages * STAGE + WROWS * 4);
+    ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tables + WROWS * 4);
     uint32_t flags       = 0;
     if constexpr (M::is_int && !APAIR)
     {
@@ -348,6 +399,36 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         aw[s] = wrow * 64 + (((2 * s + h) ^ swz(wrow)) * 16);
         ap[s] = prow * 64 + (((2 * s + h) ^ swz(prow)) * 16);
     }
+
+    // PATCH: the lane's pixel fragments of block (tap, piece) lie in plane `piece` at the patch pixel under that tap
+    int pbase = 0;    // patch pixel under the first tap of the lane's output pixel
+    if constexpr (PATCH)
+    {
+        int r_out = wp * 32 + rho;
+        r_out     = r_out < m_end - p0 ? r_out : 0;    // rows past the tile's end: any pixel, never stored
+        const int py = (int)fdiv((uint32_t)r_out, a.div_ow);
+        pbase        = py * a.sy * a.patch_w + (r_out - py * a.OW) * a.sx;
+    }
+    // Per block: the plane of the piece (a scalar) plus the lane's part, which changes with the tap only.
+    uint32_t patch_lane = 0;
+    auto patch_block = [&](int block) {
+        if constexpr (PATCH)
+        {
+            const int blk   = block < nb ? block : nb - 1;
+            const int t     = (int)fdiv((uint32_t)blk, a.div_bpt);
+            const int piece = blk - t * a.bpt;
+            if (piece == 0 || block == 0)
+            {
+                const int ky = (int)fdiv((uint32_t)t, a.div_kw);
+                const int kx = t - ky * a.KW;
+                const int pp = pbase + ky * a.dy * a.patch_w + kx * a.dx;
+                patch_lane   = (uint32_t)PATCH_OFF + ((uint32_t)pp << 6) + (uint32_t)((h ^ swz(pp)) << 4);
+            }
+            ap[0] = patch_lane + (uint32_t)(piece * a.patch_pixels) * 64u;
+            ap[1] = ap[0] ^ 32u;    // K-step 1: pieces 2 + h of the permuted four
+        }
+    };
+    patch_block(0);
 
     // KM: per channel tile, the address this lane hands to the transposing reads of K-step 0, first read
     uint32_t akm[OCT];
@@ -511,28 +592,123 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     };
     if constexpr (PAIR)
     {
-        int sc = 0;    // stage of the pair's first block
-#pragma unroll 1
-        for (int n = 0; n + 1 < nb; n += 2)
+        // Where every operand row is K-contiguous (no taps to decode per load), a trip round the ring needs no
+        // arithmetic per load: the sources of its blocks are one scalar pointer per load, advanced once per trip, plus
+        // an offset field, and the destination stage is a constant added to the wave's LDS base on its way into M0.
+        // Such a trip only requests blocks that exist; the last trips, whose requests run past the last block and
+        // repeat it, take the general form.
+        constexpr bool FASTABLE = !TAPS && !KM;    // (K-major weight rows advance by their own stride)
+        // (The offset field of a direct load moves the LDS destination as well as the source, so the constant that
+        // goes into M0 takes it off again; offsets are counted from the trip's third request, the one into stage 0,
+        // which keeps every M0 value at or above the wave's LDS base.)
+        const uint8_t* fptr[LOADS];    // per load: source of block n + kStages of the current trip
+#pragma unroll
+        for (int j = 0; j < LOADS; j++)
+            fptr[j] = gbase[j] + (size_t)kStages * gstep[j];
+        auto issue_fast = [&](int rel, int j) {
+#define TMI_FAST_LOAD(R)                                                                                               \
+    case R:                                                                                                            \
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%4"                    \
+                     :                                                                                                 \
+                     : "v"(voff[j]), "s"(fptr[j]), "s"(ldst[j]),                                                       \
+                       "n"(((R + kStages - 2) % kStages) * STAGE - (R - 2) * 64), "n"((R - 2) * 64)                    \
+                     : "memory", "scc");                                                                               \
+        break;
+            switch (rel)
+            {
+                TMI_FAST_LOAD(0)
+                TMI_FAST_LOAD(1)
+                TMI_FAST_LOAD(2)
+                TMI_FAST_LOAD(3)
+                TMI_FAST_LOAD(4)
+                TMI_FAST_LOAD(5)
+                TMI_FAST_LOAD(6)
+                TMI_FAST_LOAD(7)
+            }
+#undef TMI_FAST_LOAD
+        };
+        // PATCH, pieces per tap a multiple of the ring length: the blocks of a trip lie under one tap, in consecutive
+        // planes, so their fragment addresses are the trip's first plus k planes (scalars set up here)
+        uint32_t plane_k[kStages];
+        uint32_t trip_ap = 0;
+        if constexpr (PATCH)
         {
+#pragma unroll
+            for (int k = 0; k < kStages; k++)
+                plane_k[k] = (uint32_t)(k * a.patch_pixels) * 64u;
+        }
+        const bool fast_patch = !PATCH || a.bpt % kStages == 0;
+        // one pair of blocks, n and n + 1, in stages sc and sc + 1
+        auto pair = [&](int n, int sc, auto FAST) {
+            constexpr bool fast = decltype(FAST)::value;
             const int sn        = sc + 2 < kStages ? sc + 2 : 0;
             const int sfree     = sc >= 2 ? sc - 2 : kStages - 2;    // the pair consumed before this one
             const uint8_t* cur0 = lds + sc * STAGE;
-            first_step(cur0, cur0);
-            second_step(cur0 + STAGE, cur0 + STAGE, std::integral_constant<int, 0>{}, [](int) {});
-            first_step(cur0 + STAGE, cur0 + STAGE);
+            // (PATCH: pixel fragments are addressed from the start of the LDS, and the addresses of the next block's
+            // are set before the step that requests its first fragments)
+            auto next_patch = [&](int k) {    // block k of the trip (fast) or block n - sc + k
+                if constexpr (PATCH)
+                {
+                    if (fast && k < kStages)
+                        ap[0] = trip_ap + plane_k[k], ap[1] = ap[0] ^ 32u;
+                    else
+                        patch_block(n - sc + k);
+                }
+            };
+            first_step(cur0, PATCH ? lds : cur0);
+            next_patch(sc + 1);
+            second_step(cur0 + STAGE, PATCH ? lds : cur0 + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+            first_step(cur0 + STAGE, PATCH ? lds : cur0 + STAGE);
             publish_pair();    // the next pair is in LDS for every wave, and every wave is past the pair before
-            second_step(lds + sn * STAGE, lds + sn * STAGE, std::integral_constant<int, 2 * LOADS>{}, [&](int q) {
-                issue_one(n + kStages - 2 + (q & 1), sfree + (q & 1), q >> 1);
-            });
-            sc = sn;
+            next_patch(sc + 2);
+            second_step(lds + sn * STAGE, PATCH ? lds : lds + sn * STAGE, std::integral_constant<int, 2 * LOADS>{},
+                        [&](int q) {
+                            if constexpr (fast)
+                                issue_fast(sc + (q & 1), q >> 1);
+                            else
+                                issue_one(n + kStages - 2 + (q & 1), sfree + (q & 1), q >> 1);
+                        });
+        };
+        // Once round the ring per iteration, so that every stage address is a constant of its instruction (an offset
+        // field instead of an addition per fragment read and per load); the pairs left over follow one by one.
+        int n = 0;
+        if constexpr (FASTABLE)
+        {
+            if (fast_patch)
+            {
+#pragma unroll 1
+                for (; n + 2 * kStages - 2 <= nb; n += kStages)
+                {
+                    trip_ap = ap[0];    // block n: set by the trip before, or by the prologue
+#pragma unroll
+                    for (int sc = 0; sc < kStages; sc += 2)
+                        pair(n + sc, sc, std::true_type{});
+#pragma unroll
+                    for (int j = 0; j < LOADS; j++)
+                        fptr[j] += kStages * 64;
+                }
+            }
+        }
+#pragma unroll 1
+        for (; n + kStages - 1 < nb; n += kStages)
+        {
+#pragma unroll
+            for (int sc = 0; sc < kStages; sc += 2)
+                pair(n + sc, sc, std::false_type{});
+        }
+        int sc = 0;    // stage of the pair's first block
+#pragma unroll 1
+        for (; n + 1 < nb; n += 2)
+        {
+            pair(n, sc, std::false_type{});
+            sc = sc + 2 < kStages ? sc + 2 : 0;
         }
         if (nb & 1)
         {
             // the last block of an odd count: the first half of a pair whose second half is a repeat
             const uint8_t* cur = lds + sc * STAGE;
-            first_step(cur, cur);
-            second_step(cur + STAGE, cur + STAGE, std::integral_constant<int, 0>{}, [](int) {});
+            first_step(cur, PATCH ? lds : cur);
+            second_step(cur + STAGE, PATCH ? lds : cur + STAGE, std::integral_constant<int, 0>{}, [](int) {});
         }
     }
     else if constexpr (APAIR)
@@ -646,7 +822,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             for (int i = 0; i < PXT; i++)
             {
                 const int pt0 = p0 + wp * 32 * PXT + i * 32;    // the tile's first pixel row
-                if (pt0 >= a.M)
+                if (pt0 >= m_end)
                     continue;
 #pragma unroll
                 for (int t = 0; t < OCT; t++)
@@ -673,7 +849,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 {
                     const int row = lane / PIECES + RPI * j, piece = lane % PIECES;
                     const v4i d   = *reinterpret_cast<const v4i*>(tbuf + row * HPITCH + piece * 16);
-                    if (pt0 + row < a.M)
+                    if (pt0 + row < m_end)
                         *reinterpret_cast<v4i*>(out_b + ((size_t)(pt0 + row) * a.N + oc0 + wo * 32 * OCT) * 2 + piece * 16) = d;
                 }
             }
@@ -709,7 +885,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             if (lines)
             {
                 const int pt0 = p0 + wp * 32 * PXT + i * 32;    // the tile's first pixel row
-                if (pt0 >= a.M || oc0 + tl >= a.N)
+                if (pt0 >= m_end || oc0 + tl >= a.N)
                     continue;
                 int w4[16];
                 if constexpr (M::is_int)
@@ -734,12 +910,12 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 {
                     const int row = (lane >> 3) + 8 * j, piece = lane & 7;
                     const v4i d   = *reinterpret_cast<const v4i*>(tbuf + row * TPITCH + piece * 16);
-                    if (pt0 + row < a.M)
+                    if (pt0 + row < m_end)
                         *reinterpret_cast<v4i*>(out_b + ((size_t)(pt0 + row) * a.N + oc0 + tl) * 4 + piece * 16) = d;
                 }
                 continue;
             }
-            if (p >= a.M || oc0 + tl >= a.N)
+            if (p >= m_end || oc0 + tl >= a.N)
                 continue;
             if constexpr (M::is_int)
             {
@@ -884,9 +1060,12 @@ static bool launch_gemm_pipe(hipStream_t st, const GemmArgs& a, int blocks)
 {
     // stages, bias table, per-channel RESCALE constants; PIXEL_PAIRS: four stages of weight rows and three slots
     // of two blocks of pixel rows, the bias table goes through a stage after the loop
-    constexpr size_t lds_bytes = PIPE == PIPE_PIXEL_PAIRS
-                                     ? (size_t)4 * 64 * OCT * 64 + (size_t)6 * 128 * PXT * 64
-                                     : (size_t)STAGES * (64 * OCT + 128 * PXT) * 64 + 64 * OCT * 4 + 64 * OCT * 32;
+    const size_t lds_bytes = PIPE == PIPE_PIXEL_PAIRS
+                                 ? (size_t)4 * 64 * OCT * 64 + (size_t)6 * 128 * PXT * 64
+                                 : (MODE == GEMM_PATCH
+                                        ? (size_t)STAGES * 64 * OCT * 64 + (size_t)a.patch_bytes
+                                        : (size_t)STAGES * (64 * OCT + 128 * PXT) * 64) +
+                                       64 * OCT * 4 + 64 * OCT * 32;
     auto kern                  = gemm_lds_kernel<T, OCT, PXT, ZP, MODE, STAGES, PIPE>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, granted))
@@ -925,9 +1104,70 @@ static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
     return launch_gemm_pipe<T, OCT, PXT, ZP, MODE, kStagesDefault, PIPE_SINGLE>(st, a, blocks);
 }
 
+// The patch form of a convolution with taps (stride 1): tiles of whole output rows, 128 x 128 results, the input patch
+// resident in LDS behind a ring of eight weight stages.  False when the layer does not fit the form.
+template <typename T>
+static bool launch_gemm_patch(hipStream_t st, GemmArgs& a)
+{
+    constexpr int kRing = 8 * 128 * 64, kTables = 128 * 4 + 128 * 32, kLds = 160 * 1024;
+    if (a.sy != 1 || a.sx != 1 || a.OW > 128 || a.N < 128 || a.n_blocks < 8)
+        return false;
+    const int kh          = a.taps / a.KW;
+    const int rows        = 128 / a.OW < a.OH ? 128 / a.OW : a.OH;
+    // the tiles must not leave much of their 128 pixel rows, or of the image's last tile, unused
+    if (rows * a.OW < 96 || (int64_t)a.OH * 4 < (int64_t)((a.OH + rows - 1) / rows) * rows * 3)
+        return false;
+    const int patch_h     = (rows - 1) * a.sy + (kh - 1) * a.dy + 1;
+    const int patch_w     = (a.OW - 1) * a.sx + (a.KW - 1) * a.dx + 1;
+    const int64_t pixels  = (int64_t)patch_h * patch_w;
+    const int64_t units   = pixels * a.bpt;
+    const int64_t bytes   = (units * 64 + 1023) / 1024 * 1024;
+    if (kRing + bytes + kTables > kLds)
+        return false;
+    const int images      = a.M / (a.OH * a.OW);
+    a.rows_per_tile       = rows;
+    a.tiles_per_image     = (a.OH + rows - 1) / rows;
+    a.patch_w             = patch_w;
+    a.patch_pixels        = (int32_t)pixels;
+    a.patch_units         = (int32_t)units;
+    a.patch_bytes         = (int32_t)bytes;
+    a.div_tpi             = make_fastdiv((uint32_t)a.tiles_per_image);
+    a.div_pw              = make_fastdiv((uint32_t)patch_w);
+    a.div_ppix            = make_fastdiv((uint32_t)pixels);
+    a.div_ow              = make_fastdiv((uint32_t)a.OW);
+    a.tiles_n             = (a.N + 127) / 128;
+    const int64_t tiles_m = (int64_t)images * a.tiles_per_image;
+    const int64_t tiles   = tiles_m * a.tiles_n;
+    // the divisions of the tile decode and of the patch loads are exact in these ranges
+    if (tiles > (1 << 22) || !fastdiv_exact_up_to((uint64_t)tiles - 1, (uint32_t)tiles) ||
+        !fastdiv_exact_up_to((uint64_t)tiles - 1, (uint32_t)a.tiles_n) ||
+        !fastdiv_exact_up_to((uint64_t)tiles_m, (uint32_t)a.tiles_per_image) ||
+        !fastdiv_exact_up_to((uint64_t)units + 128, (uint32_t)pixels) ||
+        !fastdiv_exact_up_to((uint64_t)pixels, (uint32_t)patch_w) || !fastdiv_exact_up_to(128, (uint32_t)a.OW))
+        return false;
+    a.tiles_per_batch = (int32_t)tiles;
+    a.tiles_total     = (int32_t)tiles;
+    a.per_xcd         = (a.tiles_total + 7) / 8;
+    a.div_batch       = make_fastdiv((uint32_t)a.tiles_per_batch);
+    a.div_tn          = make_fastdiv((uint32_t)a.tiles_n);
+    const bool zp     = Mma<T>::is_int && (a.za != 0 || a.zw != 0);
+    if (zp)
+        return launch_gemm_pipe<T, 2, 1, Mma<T>::is_int, GEMM_PATCH, 8, PIPE_PAIRS>(st, a, a.per_xcd * 8);
+    return launch_gemm_pipe<T, 2, 1, false, GEMM_PATCH, 8, PIPE_PAIRS>(st, a, a.per_xcd * 8);
+}
+
 template <typename T>
 static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool tapped, const char* label)
 {
+    // Floating-point convolutions with taps whose patch fits the LDS take the patch form.  Measured on MI355X, us
+    // taps form / patch form (host clock, launch included): fp16 3x3 [16,28,28,256]->256 25.0 / 22.0,
+    // [16,28,28,192]->256 20.6 / 18.4, [16,20,20,256]->384 23.2 / 20.5, [16,56,56,128]->128 26.1 / 25.7, dilation 2
+    // [16,28,28,256]->256 25.3 / 25.6.
+    if constexpr (!Mma<T>::is_int)
+    {
+        if (tapped && batches == 1 && launch_gemm_patch<T>(st, a))
+            return label;
+    }
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
     // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
     // to the patch kernel.

@@ -160,6 +160,8 @@ def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     (8, 56, 56, 256, 64),
     (4, 28, 28, 512, 648),
     (1, 97, 131, 256, 130),
+    (8, 32, 33, 2944, 200),    # 46 blocks of K: whole trips round the ring of stages, then the general form
+    (8, 30, 34, 3520, 136),    # 55 blocks: an odd count behind the trips
 ])
 @pytest.mark.parametrize("zps", [(0, 0), (-6, 11)])
 def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
@@ -177,7 +179,7 @@ def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
 
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203)])
+@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203), (8, 32, 33, 1472, 200)])
 def test_conv2d_1x1_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, ih, iw, ic, oc = shape
     rng = np.random.default_rng(ic + oc)
@@ -249,6 +251,11 @@ TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
     (16, 64, 64, 192, 96, 2, 2, (0, 0, 0, 0), (2, 2), (1, 1)),      # no padding
     (2, 130, 100, 64, 72, 1, 7, (0, 0, 3, 3), (1, 1), (1, 1)),
     (16, 28, 28, 320, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 5 blocks per tap: pairs of blocks straddle taps
+    # floating point, stride 1, a patch that fits the LDS: the patch form (tiles of whole output rows)
+    (24, 29, 20, 256, 160, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # last tile of an image and of the channels ragged
+    (20, 30, 30, 128, 128, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),     # dilation 2, 4 blocks per tap
+    (20, 26, 21, 192, 136, 2, 3, (0, 1, 2, 0), (1, 1), (1, 1)),     # uneven padding, 6 blocks per tap
+    (24, 20, 36, 256, 128, 1, 3, (0, 0, 1, 1), (1, 1), (1, 1)),     # one row of taps, tiles of 3 rows
 ]
 
 
