@@ -751,8 +751,74 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
     }
     else
     {
+        int n = 0;
+        // Whole trips round the ring first, as in the pair form: stage addresses are constants, a K-contiguous row's
+        // block is the trip's pointer plus an offset field (taken off the LDS side again in M0, counted from the
+        // request that goes into stage 0), a K-major weight block has one running pointer per stage.  A trip only
+        // requests blocks that exist; the rest of the loop is the general form.
+        if constexpr (!TAPS && kStages == 4)
+        {
+            const uint8_t* fptr[LOADS];            // K-contiguous: source of block n + kStages
+            const uint8_t* kptr[LOADS][kStages];    // K-major: source of block n + kStages - 1 + r
+#pragma unroll
+            for (int j = 0; j < LOADS; j++)
+            {
+                fptr[j] = gbase[j] + (size_t)kStages * gstep[j];
+#pragma unroll
+                for (int r = 0; r < kStages; r++)
+                    kptr[j][r] = gbase[j] + (size_t)(kStages - 1 + r) * gstep[j];
+            }
+            auto issue_trip = [&](int r, int j) {
+                if (KM && j < WLOADS)
+                {
+                    const uint32_t dst = ldst[j] + ((r + kStages - 1) % kStages) * STAGE;
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                                 :
+                                 : "v"(voff[j]), "s"(kptr[j][r]), "s"(dst)
+                                 : "memory");
+                    return;
+                }
+#define TMI_TRIP_LOAD(R)                                                                                               \
+    case R:                                                                                                            \
+        asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%4"                    \
+                     :                                                                                                 \
+                     : "v"(voff[j]), "s"(fptr[j]), "s"(ldst[j]),                                                       \
+                       "n"(((R + kStages - 1) % kStages) * STAGE - (R - 1) * 64), "n"((R - 1) * 64)                    \
+                     : "memory", "scc");                                                                               \
+        break;
+                switch (r)
+                {
+                    TMI_TRIP_LOAD(0)
+                    TMI_TRIP_LOAD(1)
+                    TMI_TRIP_LOAD(2)
+                    TMI_TRIP_LOAD(3)
+                }
+#undef TMI_TRIP_LOAD
+            };
 #pragma unroll 1
-        for (int n = 0; n < nb; n++)
+            for (; n + 2 * kStages - 1 <= nb; n += kStages)
+            {
+#pragma unroll
+                for (int r = 0; r < kStages; r++)
+                {
+                    const uint8_t* cur  = lds + r * STAGE;
+                    const uint8_t* next = lds + ((r + 1) % kStages) * STAGE;
+                    first_step(cur, cur);
+                    publish();
+                    second_step(next, next, std::integral_constant<int, LOADS>{}, [&](int q) { issue_trip(r, q); });
+                }
+#pragma unroll
+                for (int j = 0; j < LOADS; j++)
+                {
+                    fptr[j] += (size_t)kStages * gstep[j];
+#pragma unroll
+                    for (int r = 0; r < kStages; r++)
+                        kptr[j][r] += (size_t)kStages * gstep[j];
+                }
+            }
+        }
+#pragma unroll 1
+        for (; n < nb; n++)
         {
             const uint8_t* cur  = lds + (n % kStages) * STAGE;
             const uint8_t* next = lds + ((n + 1) % kStages) * STAGE;
