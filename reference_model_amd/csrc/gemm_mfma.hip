@@ -1223,7 +1223,8 @@ static bool launch_gemm_patch(hipStream_t st, GemmArgs& a)
 }
 
 template <typename T>
-static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool tapped, const char* label)
+static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool tapped, const char* label,
+                                 const char* patch_label = nullptr)
 {
     // Floating-point convolutions with taps whose patch fits the LDS take the patch form.  Measured on MI355X, us
     // taps form / patch form (host clock, launch included): fp16 3x3 [16,28,28,256]->256 25.0 / 22.0,
@@ -1231,8 +1232,8 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
     // [16,28,28,256]->256 25.3 / 25.6.
     if constexpr (!Mma<T>::is_int)
     {
-        if (tapped && batches == 1 && launch_gemm_patch<T>(st, a))
-            return label;
+        if (tapped && batches == 1 && patch_label && launch_gemm_patch<T>(st, a))
+            return patch_label;
     }
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
     // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
@@ -1378,8 +1379,8 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     switch (in_dtype)
     {
         case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, tapped, rp.enabled ? "gemm_mfma_i8_rescale" : "gemm_mfma_i8");
-        case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, tapped, "gemm_mfma_f16");
-        default: return launch_gemm_t<bf16_t>(st, a, batches, tapped, "gemm_mfma_bf16");
+        case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, tapped, "gemm_mfma_f16", "gemm_mfma_f16_patch");
+        default: return launch_gemm_t<bf16_t>(st, a, batches, tapped, "gemm_mfma_bf16", "gemm_mfma_bf16_patch");
     }
 }
 

@@ -276,7 +276,7 @@ def test_benchmark_fp16_conv_and_bf16_matmul_errors_at_full_size(ctx):
         shape = (n, ih, iw, oc)
         imp, ref, bnd = ctx.empty(shape, capi.FP16), ctx.empty(shape, capi.F64), ctx.empty(shape, capi.F64)
         ctx.conv2d(d, tx, tw, tb, 0, 0, imp)
-        assert ctx.last_kernel == "gemm_mfma_f16"
+        assert ctx.last_kernel == "gemm_mfma_f16_patch"
         ctx.conv2d_precise(d, tx, tw, tb, False, ref)
         ctx.conv2d_precise(d, tx, tw, tb, True, bnd)
         ksb = dp.kernel_size_bound(kh * kw * ic, "fp16")

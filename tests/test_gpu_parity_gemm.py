@@ -303,7 +303,13 @@ def test_conv2d_taps_fp_gemm_within_dot_product_bound(ctx, shape, kind):
         xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
         dtype = capi.BF16
     got, st = gpu_ops.conv2d(ctx, xs, ws, bs, pad, stride, dil, dtype=dtype)
-    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16")
+    # stride 1 and a patch of (rows + (kh-1) dil) x (ow + (kw-1) dil) pixels that fits beside the ring: the patch form
+    oh, ow = got.shape[1], got.shape[2]
+    rows = min(128 // ow, oh) if ow <= 128 else 0
+    patch_bytes = (rows - 1 + (kh - 1) * dil[0] + 1) * (ow - 1 + (kw - 1) * dil[1] + 1) * ic * 2
+    patch = (stride == (1, 1) and rows * ow >= 96 and oc >= 128 and oh * 4 >= -(-oh // rows) * rows * 3
+             and 65536 + 4608 + -(-patch_bytes // 1024) * 1024 <= 160 * 1024)
+    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16") + ("_patch" if patch else "")
     imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
     # reference and bound from the device's fp64 precise / bounds passes, which the fp64 oracle pins bit for bit
     oh, ow = got.shape[1], got.shape[2]
@@ -385,7 +391,8 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.INT8, (8, 56, 56, 192, 64, 3, 1), "conv2d_mfma_i8"),         # 3x3 int8: the patch kernel
     (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "conv2d_mfma_i8"),
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
-    (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16"),        # 3x3 fp16, deep K
+    (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),  # 3x3 fp16, deep K, the patch fits the LDS
+    (capi.FP16, (8, 28, 28, 512, 512, 3, 1), "gemm_mfma_f16"),         # the same with a patch that does not fit
     (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "conv2d_mfma_f16"),        # pointwise the GEMM kernel refuses (K < 256 bytes)
 ])
