@@ -1156,6 +1156,10 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
             const int oct = cand[c][0], pxt = cand[c][1];
             if (oct == 2 && g.OC <= 64)
                 continue;
+            // with the fused fast RESCALE the four- and eight-tile shapes do not fit the register file (320 and 576
+            // bytes of scratch per lane, and a kernel with a scratch segment ran 2.4 times as long as the plain one)
+            if (oct == 2 && rp.enabled && rp.fast)
+                continue;
             const int ocb = 32 * oct * WOC, max_px = 32 * (8 / WOC) * pxt;
             int th, tw;
             tile_for(max_px, th, tw);
@@ -1303,7 +1307,10 @@ static const char* launch_conv2d_mfma_t(hipStream_t st, const ConvGeom& g, int32
         TMI_PATCH_SHAPES(EPI_PLAIN)
         if constexpr (Mma<T>::is_int)
         {
-            TMI_PATCH_SHAPES(EPI_FAST)
+            TMI_PATCH_CASE(1, 1, 1, EPI_FAST)
+            TMI_PATCH_CASE(1, 1, 2, EPI_FAST)
+            TMI_PATCH_CASE(2, 1, 1, EPI_FAST)
+            TMI_PATCH_CASE(2, 1, 2, EPI_FAST)
             TMI_PATCH_SHAPES(EPI_GENERIC)
         }
     }

@@ -1172,24 +1172,32 @@ static bool launch_gemm_shape(hipStream_t st, const GemmArgs& a, int blocks)
 
 // The patch form of a convolution with taps (stride 1): tiles of whole output rows, 128 x 128 results, the input patch
 // resident in LDS behind a ring of eight weight stages.  False when the layer does not fit the form.
+// Geometry of the patch form, or false: output rows per tile, patch height and width in pixels.
+static bool patch_form_geometry(int OH, int OW, int KH, int KW, int sy, int sx, int dy, int dx, int64_t icb, int OC,
+                                int& rows, int& patch_h, int& patch_w)
+{
+    constexpr int kRing = 8 * 128 * 64, kTables = 128 * 4 + 128 * 32, kLds = 160 * 1024;
+    if (sy != 1 || sx != 1 || OW > 128 || OC < 128 || icb % 64 != 0 || (int64_t)KH * KW * icb / 64 < 8)
+        return false;
+    rows = 128 / OW < OH ? 128 / OW : OH;
+    // the tiles must not leave much of their 128 pixel rows, or of the image's last tile, unused
+    if (rows * OW < 96 || (int64_t)OH * 4 < (int64_t)((OH + rows - 1) / rows) * rows * 3)
+        return false;
+    patch_h              = (rows - 1) * sy + (KH - 1) * dy + 1;
+    patch_w              = (OW - 1) * sx + (KW - 1) * dx + 1;
+    const int64_t bytes  = ((int64_t)patch_h * patch_w * icb + 1023) / 1024 * 1024;
+    return kRing + bytes + kTables <= kLds;
+}
+
 template <typename T>
 static bool launch_gemm_patch(hipStream_t st, GemmArgs& a)
 {
-    constexpr int kRing = 8 * 128 * 64, kTables = 128 * 4 + 128 * 32, kLds = 160 * 1024;
-    if (a.sy != 1 || a.sx != 1 || a.OW > 128 || a.N < 128 || a.n_blocks < 8)
+    int rows = 0, patch_h = 0, patch_w = 0;
+    if (!patch_form_geometry(a.OH, a.OW, a.taps / a.KW, a.KW, a.sy, a.sx, a.dy, a.dx, a.icb, a.N, rows, patch_h, patch_w))
         return false;
-    const int kh          = a.taps / a.KW;
-    const int rows        = 128 / a.OW < a.OH ? 128 / a.OW : a.OH;
-    // the tiles must not leave much of their 128 pixel rows, or of the image's last tile, unused
-    if (rows * a.OW < 96 || (int64_t)a.OH * 4 < (int64_t)((a.OH + rows - 1) / rows) * rows * 3)
-        return false;
-    const int patch_h     = (rows - 1) * a.sy + (kh - 1) * a.dy + 1;
-    const int patch_w     = (a.OW - 1) * a.sx + (a.KW - 1) * a.dx + 1;
     const int64_t pixels  = (int64_t)patch_h * patch_w;
     const int64_t units   = pixels * a.bpt;
     const int64_t bytes   = (units * 64 + 1023) / 1024 * 1024;
-    if (kRing + bytes + kTables > kLds)
-        return false;
     const int images      = a.M / (a.OH * a.OW);
     a.rows_per_tile       = rows;
     a.tiles_per_image     = (a.OH + rows - 1) / rows;
@@ -1230,11 +1238,8 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
     // taps form / patch form (host clock, launch included): fp16 3x3 [16,28,28,256]->256 25.0 / 22.0,
     // [16,28,28,192]->256 20.6 / 18.4, [16,20,20,256]->384 23.2 / 20.5, [16,56,56,128]->128 26.1 / 25.7, dilation 2
     // [16,28,28,256]->256 25.3 / 25.6.
-    if constexpr (!Mma<T>::is_int)
-    {
-        if (tapped && batches == 1 && patch_label && launch_gemm_patch<T>(st, a))
-            return patch_label;
-    }
+    if (tapped && batches == 1 && patch_label && launch_gemm_patch<T>(st, a))
+        return patch_label;
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
     // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
     // to the patch kernel.
@@ -1300,7 +1305,15 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
 {
     if (g.KH * g.KW == 1)
         return true;
-    return in_dtype != TMI_INT8 && g.IC >= 128;
+    if (in_dtype != TMI_INT8)
+        return g.IC >= 128;
+    // int8 layers with taps: where this kernel can keep the input patch in LDS it is the faster one.  us patch
+    // kernel / this kernel (host clock): 3x3 [16,28,28,256]->256 25.3 / 19.8, [8,28,28,512]->512 37.3 / 28.4,
+    // [16,56,56,128]->128 29.0 / 22.6, [32,28,28,256]->256 39.8 / 33.6; with the fused RESCALE 19.4 / 18.7,
+    // 31.7 / 28.3, (slab kernel 15.3) / 24.8, 41 / 36.9.
+    int rows, patch_h, patch_w;
+    return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, g.IC, g.OC, rows,
+                               patch_h, patch_w);
 }
 
 // nullptr when the operation is not a GEMM this kernel takes; the caller then goes to the patch kernel.
@@ -1378,7 +1391,9 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     const bool tapped = !plain;
     switch (in_dtype)
     {
-        case TMI_INT8: return launch_gemm_t<int8_t>(st, a, batches, tapped, rp.enabled ? "gemm_mfma_i8_rescale" : "gemm_mfma_i8");
+        case TMI_INT8:
+            return launch_gemm_t<int8_t>(st, a, batches, tapped, rp.enabled ? "gemm_mfma_i8_rescale" : "gemm_mfma_i8",
+                                         rp.enabled ? "gemm_mfma_i8_rescale_patch" : "gemm_mfma_i8_patch");
         case TMI_FP16: return launch_gemm_t<_Float16>(st, a, batches, tapped, "gemm_mfma_f16", "gemm_mfma_f16_patch");
         default: return launch_gemm_t<bf16_t>(st, a, batches, tapped, "gemm_mfma_bf16", "gemm_mfma_bf16_patch");
     }

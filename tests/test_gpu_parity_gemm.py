@@ -243,6 +243,18 @@ def test_config5_bf16_matmul_full_size_gemm(ctx):
 
 
 # ---- convolutions with taps through the GEMM kernel (K axis = (ky, kx, ic), taps outside the image read zeros) ----
+def patch_form(oh, ow, ic_bytes, oc, kh, kw, stride, dil):
+    """"_patch" where the GEMM kernel keeps the input patch of a tile in LDS: stride 1, tiles of whole output rows that
+    use at least 96 of their 128 pixel rows and 3/4 of an image's last tile, and a patch of (rows + (kh-1) dil) x
+    (ow + (kw-1) dil) pixels that fits behind the ring of weight stages (64 KB) and the tables"""
+    if tuple(stride) != (1, 1) or ow > 128 or oc < 128 or kh * kw * ic_bytes // 64 < 8:
+        return ""
+    rows = min(128 // ow, oh)
+    patch_bytes = (rows - 1 + (kh - 1) * dil[0] + 1) * (ow - 1 + (kw - 1) * dil[1] + 1) * ic_bytes
+    fits = 65536 + 4608 + -(-patch_bytes // 1024) * 1024 <= 160 * 1024
+    return "_patch" if rows * ow >= 96 and oh * 4 >= -(-oh // rows) * rows * 3 and fits else ""
+
+
 TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
     (16, 28, 28, 256, 256, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # the named fp16 configuration
     (40, 31, 29, 64, 136, 3, 3, (1, 1, 1, 1), (2, 2), (1, 1)),      # stride 2, ragged tiles
@@ -268,7 +280,8 @@ def test_conv2d_taps_i8_gemm_bit_exact(ctx, shape, w_zp):
     w = rng.integers(-128, 128, (oc, kh, kw, ic)).astype(np.int8)
     bias = rng.integers(-(1 << 20), 1 << 20, oc).astype(np.int32)
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=0, w_zp=w_zp)
-    assert st == capi.VALID and ctx.last_kernel == "gemm_mfma_i8"
+    assert st == capi.VALID
+    assert ctx.last_kernel == "gemm_mfma_i8" + patch_form(got.shape[1], got.shape[2], ic, oc, kh, kw, stride, dil)
     assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, pad, stride, dil, 0, w_zp))
     sub = oracle.conv2d("i8", x[-1:], w[:3], bias[:3], pad, stride, dil, in_zp=0, w_zp=w_zp)
     assert np.array_equal(got[-1:, :, :, :3], sub)
@@ -303,13 +316,9 @@ def test_conv2d_taps_fp_gemm_within_dot_product_bound(ctx, shape, kind):
         xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
         dtype = capi.BF16
     got, st = gpu_ops.conv2d(ctx, xs, ws, bs, pad, stride, dil, dtype=dtype)
-    # stride 1 and a patch of (rows + (kh-1) dil) x (ow + (kw-1) dil) pixels that fits beside the ring: the patch form
     oh, ow = got.shape[1], got.shape[2]
-    rows = min(128 // ow, oh) if ow <= 128 else 0
-    patch_bytes = (rows - 1 + (kh - 1) * dil[0] + 1) * (ow - 1 + (kw - 1) * dil[1] + 1) * ic * 2
-    patch = (stride == (1, 1) and rows * ow >= 96 and oc >= 128 and oh * 4 >= -(-oh // rows) * rows * 3
-             and 65536 + 4608 + -(-patch_bytes // 1024) * 1024 <= 160 * 1024)
-    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16") + ("_patch" if patch else "")
+    assert st == capi.VALID and ctx.last_kernel == ("gemm_mfma_f16" if kind == "fp16" else "gemm_mfma_bf16") + patch_form(
+        oh, ow, ic * 2, oc, kh, kw, stride, dil)
     imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
     # reference and bound from the device's fp64 precise / bounds passes, which the fp64 oracle pins bit for bit
     oh, ow = got.shape[1], got.shape[2]
@@ -366,7 +375,7 @@ def test_conv2d_fused_rescale_gemm_bit_exact(ctx, shape, zps, out_dtype):
              shift=rng.integers(36, 44, oc).astype(np.int8), out_zp=zps[2] if out_dtype == np.int8 else 0,
              clamp=(-100, 110) if out_dtype == np.int8 else None)
     got, st, want, wst = _fused(ctx, c, out_dtype)
-    assert ctx.last_kernel == "gemm_mfma_i8_rescale"
+    assert ctx.last_kernel == "gemm_mfma_i8_rescale" + patch_form(got.shape[1], got.shape[2], ic, oc, kh, kw, stride, (1, 1))
     assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
     assert len(np.unique(got)) > 50     # the scale keeps the results inside the output range
 
@@ -381,7 +390,7 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
              pad=(1, 1, 1, 1), stride=(1, 1), dilation=(1, 1), mult=np.full(oc, 1 << 30, np.int32),
              shift=np.full(oc, 12, np.int8), out_zp=0, clamp=None)
     got, st, want, wst = _fused(ctx, c)
-    assert ctx.last_kernel == "gemm_mfma_i8_rescale"
+    assert ctx.last_kernel == "gemm_mfma_i8_rescale_patch"
     assert st == wst == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
 
 
@@ -389,7 +398,8 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
 @pytest.mark.parametrize("dtype, shape, kernel", [
     # n, ih, iw, ic, oc, k, pad
     (capi.INT8, (8, 56, 56, 192, 64, 3, 1), "conv2d_mfma_i8"),         # 3x3 int8: the patch kernel
-    (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "conv2d_mfma_i8"),
+    (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_i8_patch"),   # 3x3 int8 whose patch the GEMM kernel can keep in LDS
+    (capi.INT8, (16, 28, 28, 1024, 256, 3, 1), "conv2d_mfma_i8"),      # 3x3 int8 whose patch (6 x 30 x 1 KB) does not fit
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
     (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),  # 3x3 fp16, deep K, the patch fits the LDS
     (capi.FP16, (8, 28, 28, 512, 512, 3, 1), "gemm_mfma_f16"),         # the same with a patch that does not fit
