@@ -689,12 +689,16 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                 }
             }
         }
-#pragma unroll 1
-        for (; n + kStages - 1 < nb; n += kStages)
+        // (not with taps: the unrolled trip with the tap decode of every pixel load does not fit the register file)
+        if constexpr (!TAPS)
         {
+#pragma unroll 1
+            for (; n + kStages - 1 < nb; n += kStages)
+            {
 #pragma unroll
-            for (int sc = 0; sc < kStages; sc += 2)
-                pair(n + sc, sc, std::false_type{});
+                for (int sc = 0; sc < kStages; sc += 2)
+                    pair(n + sc, sc, std::false_type{});
+            }
         }
         int sc = 0;    // stage of the pair's first block
 #pragma unroll 1
