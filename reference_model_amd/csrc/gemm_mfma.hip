@@ -637,10 +637,13 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             for (int k = 0; k < kStages; k++)
                 plane_k[k] = (uint32_t)(k * a.patch_pixels) * 64u;
         }
-        const bool fast_patch = !PATCH || a.bpt % kStages == 0;
+        // (FAST: 0 the general form, 1 a trip under one tap, 2 a trip whose halves lie under two taps)
+        const int fast_patch = !PATCH || a.bpt % kStages == 0 ? 1 : (a.bpt * 2 == kStages ? 2 : 0);
+        uint32_t half_ap = 0;    // FAST 2: fragment address of the trip's block kStages / 2
         // one pair of blocks, n and n + 1, in stages sc and sc + 1
         auto pair = [&](int n, int sc, auto FAST) {
-            constexpr bool fast = decltype(FAST)::value;
+            constexpr int fast_form = decltype(FAST)::value;
+            constexpr bool fast     = fast_form != 0;
             const int sn        = sc + 2 < kStages ? sc + 2 : 0;
             const int sfree     = sc >= 2 ? sc - 2 : kStages - 2;    // the pair consumed before this one
             const uint8_t* cur0 = lds + sc * STAGE;
@@ -649,10 +652,16 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             auto next_patch = [&](int k) {    // block k of the trip (fast) or block n - sc + k
                 if constexpr (PATCH)
                 {
-                    if (fast && k < kStages)
+                    if (fast_form == 1 && k < kStages)
                         ap[0] = trip_ap + plane_k[k], ap[1] = ap[0] ^ 32u;
+                    else if (fast_form == 2 && k < kStages && k != kStages / 2)
+                        ap[0] = (k < kStages / 2 ? trip_ap : half_ap) + plane_k[k % (kStages / 2)], ap[1] = ap[0] ^ 32u;
                     else
+                    {
                         patch_block(n - sc + k);
+                        if (fast_form == 2 && k == kStages / 2)
+                            half_ap = ap[0];
+                    }
                 }
             };
             first_step(cur0, PATCH ? lds : cur0);
@@ -674,7 +683,7 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
         int n = 0;
         if constexpr (FASTABLE)
         {
-            if (fast_patch)
+            if (fast_patch == 1)
             {
 #pragma unroll 1
                 for (; n + 2 * kStages - 2 <= nb; n += kStages)
@@ -682,10 +691,27 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
                     trip_ap = ap[0];    // block n: set by the trip before, or by the prologue
 #pragma unroll
                     for (int sc = 0; sc < kStages; sc += 2)
-                        pair(n + sc, sc, std::true_type{});
+                        pair(n + sc, sc, std::integral_constant<int, 1>{});
 #pragma unroll
                     for (int j = 0; j < LOADS; j++)
                         fptr[j] += kStages * 64;
+                }
+            }
+            if constexpr (PATCH)
+            {
+                if (fast_patch == 2)
+                {
+#pragma unroll 1
+                    for (; n + 2 * kStages - 2 <= nb; n += kStages)
+                    {
+                        trip_ap = ap[0];
+#pragma unroll
+                        for (int sc = 0; sc < kStages; sc += 2)
+                            pair(n + sc, sc, std::integral_constant<int, 2>{});
+#pragma unroll
+                        for (int j = 0; j < LOADS; j++)
+                            fptr[j] += kStages * 64;
+                    }
                 }
             }
         }
@@ -697,14 +723,14 @@ __global__ __launch_bounds__(512) void gemm_lds_kernel(GemmArgs a)
             {
 #pragma unroll
                 for (int sc = 0; sc < kStages; sc += 2)
-                    pair(n + sc, sc, std::false_type{});
+                    pair(n + sc, sc, std::integral_constant<int, 0>{});
             }
         }
         int sc = 0;    // stage of the pair's first block
 #pragma unroll 1
         for (; n + 1 < nb; n += 2)
         {
-            pair(n, sc, std::false_type{});
+            pair(n, sc, std::integral_constant<int, 0>{});
             sc = sc + 2 < kStages ? sc + 2 : 0;
         }
         if (nb & 1)
