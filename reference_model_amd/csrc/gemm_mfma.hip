@@ -1242,6 +1242,11 @@ static bool launch_gemm_patch(hipStream_t st, GemmArgs& a)
     a.tiles_n             = (a.N + 127) / 128;
     const int64_t tiles_m = (int64_t)images * a.tiles_per_image;
     const int64_t tiles   = tiles_m * a.tiles_n;
+    // A workgroup has a CU to itself, so the time hardly depends on how many there are; from some 48 tiles on this
+    // form is faster than the patch kernel (us patch kernel / this form, host clock: fp16 3x3 [4,28,28,256]->256
+    // 21.3 / 16.5, [16,14,14,256]->256 21.5 / 16.5, [8,28,28,128]->128 13.0 / 10.5; int8 14.8 / 11.1, 14.6 / 11.1).
+    if (tiles < 48)
+        return false;
     // the divisions of the tile decode and of the patch loads are exact in these ranges
     if (tiles > (1 << 22) || !fastdiv_exact_up_to((uint64_t)tiles - 1, (uint32_t)tiles) ||
         !fastdiv_exact_up_to((uint64_t)tiles - 1, (uint32_t)a.tiles_n) ||
@@ -1270,6 +1275,9 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
     // [16,28,28,256]->256 25.3 / 25.6.
     if (tapped && batches == 1 && patch_label && launch_gemm_patch<T>(st, a))
         return patch_label;
+    // enough work to fill the CUs with the smallest tile shape
+    if ((((int64_t)a.M + 127) / 128) * ((a.N + 127) / 128) * batches < 128)
+        return nullptr;
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256
     // CUs times the matrix work of one tile.  Work too small to fill the CUs with the smallest shape is left
     // to the patch kernel.
@@ -1394,9 +1402,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
     // stores are only used when OC is a multiple of 16, which keeps every output row and batch aligned too
     if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || (w_batch_stride & 15))
         return nullptr;
-    // enough work to fill the CUs with the smallest tile shape
-    if (((M + 127) / 128) * ((g.OC + 127) / 128) * batches < 128)
-        return nullptr;
+    // (enough work to fill the CUs: checked by the launcher of the form that takes the layer)
 
     GemmArgs a{};
     a.a = (const uint8_t*)in, a.w = (const uint8_t*)w, a.bias = bias, a.out = out;

@@ -268,6 +268,7 @@ TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
     (20, 30, 30, 128, 128, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),     # dilation 2, 4 blocks per tap
     (20, 26, 21, 192, 136, 2, 3, (0, 1, 2, 0), (1, 1), (1, 1)),     # uneven padding, 6 blocks per tap
     (24, 20, 36, 256, 128, 1, 3, (0, 0, 1, 1), (1, 1), (1, 1)),     # one row of taps, tiles of 3 rows
+    (3, 30, 26, 128, 200, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # 48 tiles of whole rows where 128-pixel tiles would be 38
 ]
 
 
@@ -403,6 +404,9 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
     (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),  # 3x3 fp16, deep K, the patch fits the LDS
     (capi.FP16, (8, 28, 28, 512, 512, 3, 1), "gemm_mfma_f16"),         # the same with a patch that does not fit
+    (capi.FP16, (4, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),   # 56 tiles of four output rows: enough for the patch form
+    (capi.INT8, (16, 14, 14, 256, 256, 3, 1), "gemm_mfma_i8_patch"),   # 64 tiles of nine and five rows
+    (capi.FP16, (2, 28, 28, 256, 256, 3, 1), "conv2d_mfma_f16"),       # 28 tiles: too few
     (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "conv2d_mfma_f16"),        # pointwise the GEMM kernel refuses (K < 256 bytes)
 ])
@@ -426,7 +430,9 @@ def test_automatic_kernel_choice(dtype, shape, kernel):
         try:
             other, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
         except TmiError:
-            assert kernel.startswith("conv2d") and ic * 2 < 256
+            # the GEMM kernel refuses rows of K below 256 bytes and layers with too few tiles; the patch kernel, which
+            # takes any shape, is then the only one
+            assert kernel.startswith("conv2d") and (ic * 2 < 256 or n * ih * iw < 128 * 48)
             return
         assert st == capi.VALID and c.last_kernel != kernel
     finally:
