@@ -162,6 +162,8 @@ def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     (1, 97, 131, 256, 130),
     (8, 32, 33, 2944, 200),    # 46 blocks of K: whole trips round the ring of stages, then the general form
     (8, 30, 34, 3520, 136),    # 55 blocks: an odd count behind the trips
+    (1, 14, 14, 1024, 200),    # four tiles: a pointwise layer is this kernel's from there on
+    (3, 7, 7, 2048, 520),      # ragged in both directions, 10 tiles
 ])
 @pytest.mark.parametrize("zps", [(0, 0), (-6, 11)])
 def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
@@ -179,7 +181,7 @@ def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
 
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203), (8, 32, 33, 1472, 200)])
+@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203), (8, 32, 33, 1472, 200), (1, 14, 14, 1024, 200)])
 def test_conv2d_1x1_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, ih, iw, ic, oc = shape
     rng = np.random.default_rng(ic + oc)
@@ -407,6 +409,9 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (4, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),   # 56 tiles of four output rows: enough for the patch form
     (capi.INT8, (16, 14, 14, 256, 256, 3, 1), "gemm_mfma_i8_patch"),   # 64 tiles of nine and five rows
     (capi.FP16, (2, 28, 28, 256, 256, 3, 1), "conv2d_mfma_f16"),       # 28 tiles: too few
+    (capi.FP16, (1, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_f16"),       # pointwise with 16 tiles: still the GEMM kernel
+    (capi.FP16, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_f16"),          # 3x3, no patch form (49 pixels a tile), 100 tiles
+    (capi.FP16, (32, 7, 7, 512, 512, 3, 1), "conv2d_mfma_f16"),        # the same with 52 tiles: the patch kernel
     (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "conv2d_mfma_f16"),        # pointwise the GEMM kernel refuses (K < 256 bytes)
 ])
