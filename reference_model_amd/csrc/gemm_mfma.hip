@@ -1275,12 +1275,13 @@ static const char* launch_gemm_t(hipStream_t st, GemmArgs& a, int batches, bool 
     // [16,28,28,256]->256 25.3 / 25.6.
     if (tapped && batches == 1 && patch_label && launch_gemm_patch<T>(st, a))
         return patch_label;
-    // Enough work for this kernel to be the faster one, in tiles of the smallest shape.  MATMUL: enough to fill the
-    // CUs.  A pointwise convolution: almost any (us patch kernel / this kernel, host clock: fp16 [1,14,14,1024]->1024,
+    // Enough work for this kernel to be the faster one, in tiles of the smallest shape.  MATMUL and pointwise
+    // convolutions: almost any (us patch kernel / this kernel, host clock: MATMUL int8 [1,512,512]x[1,512,512], 16
+    // tiles, 10.1 / 5.4; [8,256,256]x[8,256,256] 9.3 / 5.0; bf16 12.6 / 6.3, 10.5 / 5.4; fp16 [1,14,14,1024]->1024,
     // 16 tiles, 15.1 / 7.2; [4,7,7,2048]->512, 8 tiles, 23.4 / 13.4; [2,28,28,512]->128 9.5 / 5.4; int8 11.1 / 6.0,
     // 15.5 / 7.6, 7.9 / 5.0).  A convolution with taps: from some 96 tiles (fp16 3x3 [64,7,7,512]->512, 100 tiles,
     // 64.8 / 40.0; [16,14,14,512]->512 41.4 / 40.0; [32,7,7,512]->512, 52 tiles, 34.5 / 39.7).
-    const int64_t min_tiles = a.taps > 1 ? 96 : (a.ldw == 0 && a.w_batch == 0 ? 4 : 128);
+    const int64_t min_tiles = a.taps > 1 ? 96 : 4;
     if ((((int64_t)a.M + 127) / 128) * ((a.N + 127) / 128) * batches < min_tiles)
         return nullptr;
     // Tile shapes, largest first; the cost of a shape is the number of passes its tiles take over the 256

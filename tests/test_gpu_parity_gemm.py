@@ -46,6 +46,9 @@ GEMM_SHAPES = [
     (4, 2048, 64 * 49, 2048),  # K-major operand, 48 blocks or more: the first operand's rows requested in pairs;
     (8, 1024, 64 * 50, 1024),  # 256x256 and 128x256 tiles, odd and even block counts, ragged edges
     (3, 1000, 64 * 51, 1104),
+    (1, 512, 512, 512),       # 16 tiles: small products are this kernel's too
+    (8, 256, 256, 256),
+    (1, 130, 64 * 5, 200),    # four ragged tiles
 ]
 
 
