@@ -1392,7 +1392,7 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
         return nullptr;
     const int64_t icb = (int64_t)g.IC * eb;
     const int64_t kb  = icb * taps;
-    if (icb % 64 != 0 || kb < 256)
+    if (icb % 64 != 0)
         return nullptr;
     // MATMUL: one GEMM per image with its own weights; CONV2D: all images are rows of one GEMM
     const bool per_image  = w_batch_stride != 0;

@@ -419,7 +419,14 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         const bool gemm_ok   = ctx->kernel_choice == 0 || ctx->kernel_choice == 3;
         const bool patch_ok  = ctx->kernel_choice == 0 || ctx->kernel_choice == 2;
         const bool gemm_1st  = gemm_ok && (!patch_ok || gemm_mfma_preferred(d->in_dtype, g));
-        if (ctx->kernel_choice == 0 || ctx->kernel_choice == 4)
+        // A pointwise layer with int32 results and more than 2 M of them: the GEMM kernel, whose results leave as
+        // whole lines, before the slab kernel (us slab / GEMM, host clock: [8,56,56,64]->256 12.8 / 8.8,
+        // [32,56,56,64]->256 35.9 / 21.6, [8,28,28,128]->512 8.3 / 6.6, [32,28,28,128]->512 24.0 / 14.5; smaller ones
+        // and every layer with the fused RESCALE are the slab kernel's: 5.3 / 5.5, fused 6.9 / 10.1, 19.6 / 28.3).
+        if (ctx->kernel_choice == 0 && !rp.enabled && g.KH * g.KW == 1 && total > (int64_t(1) << 21))
+            name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
+                                    pad_page, ctx->flags_dev);
+        if (!name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
         if (!name && gemm_1st)

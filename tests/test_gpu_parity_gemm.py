@@ -166,6 +166,8 @@ def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     (8, 32, 33, 2944, 200),    # 46 blocks of K: whole trips round the ring of stages, then the general form
     (8, 30, 34, 3520, 136),    # 55 blocks: an odd count behind the trips
     (1, 14, 14, 1024, 200),    # four tiles: a pointwise layer is this kernel's from there on
+    (8, 56, 56, 64, 256),      # one block of K
+    (4, 40, 40, 128, 136),     # two
     (3, 7, 7, 2048, 520),      # ragged in both directions, 10 tiles
 ])
 @pytest.mark.parametrize("zps", [(0, 0), (-6, 11)])
@@ -184,7 +186,8 @@ def test_conv2d_1x1_i8_gemm_bit_exact(ctx, shape, zps):
 
 
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203), (8, 32, 33, 1472, 200), (1, 14, 14, 1024, 200)])
+@pytest.mark.parametrize("shape", [(8, 40, 40, 256, 208), (2, 61, 67, 128, 203), (8, 32, 33, 1472, 200), (1, 14, 14, 1024, 200),
+                                   (8, 56, 56, 64, 256), (4, 40, 40, 32, 136)])
 def test_conv2d_1x1_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, ih, iw, ic, oc = shape
     rng = np.random.default_rng(ic + oc)
@@ -416,7 +419,9 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_f16"),          # 3x3, no patch form (49 pixels a tile), 100 tiles
     (capi.FP16, (32, 7, 7, 512, 512, 3, 1), "conv2d_mfma_f16"),        # the same with 52 tiles: the patch kernel
     (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
-    (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "conv2d_mfma_f16"),        # pointwise the GEMM kernel refuses (K < 256 bytes)
+    (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_f16"),          # pointwise with two blocks of K
+    (capi.INT8, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_i8"),           # int8 pointwise, int32 results, 6.4 M of them: before the slab kernel
+    (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_slab_i8"),          # the same with 1.6 M results: the slab kernel
 ])
 def test_automatic_kernel_choice(dtype, shape, kernel):
     n, ih, iw, ic, oc, k, pad = shape
@@ -438,9 +443,9 @@ def test_automatic_kernel_choice(dtype, shape, kernel):
         try:
             other, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
         except TmiError:
-            # the GEMM kernel refuses rows of K below 256 bytes and layers with too few tiles; the patch kernel, which
-            # takes any shape, is then the only one
-            assert kernel.startswith("conv2d") and (ic * 2 < 256 or n * ih * iw < 128 * 48)
+            # the GEMM kernel refuses layers with too few tiles; the patch kernel, which takes any shape, is then
+            # the only one
+            assert kernel.startswith("conv2d") and n * ih * iw < 128 * 48
             return
         assert st == capi.VALID and c.last_kernel != kernel
     finally:
