@@ -49,6 +49,9 @@ GEMM_SHAPES = [
     (1, 512, 512, 512),       # 16 tiles: small products are this kernel's too
     (8, 256, 256, 256),
     (1, 130, 64 * 5, 200),    # four ragged tiles
+    (8, 1024, 64, 1024),      # one block of K
+    (3, 500, 128, 392),       # two, ragged
+    (1, 4096, 192, 4096),     # three, 256x256 tiles
 ]
 
 
@@ -137,7 +140,8 @@ def test_gemm_kernel_refuses_what_it_cannot_take(ctx):
 @pytest.mark.parametrize("shape", [(2, 2048, 512, 2048), (8, 1024, 256, 1024), (3, 1000, 448, 1100), (3, 1000, 448, 1104),
                                    (1, 4099, 128, 515), (5, 520, 96 * 3, 784),
                                    (3, 1000, 32 * 37, 1104), (8, 1024, 32 * 42, 1024),   # deep K: blocks in pairs
-                                   (4, 2048, 32 * 49, 2048), (3, 1000, 32 * 52, 1104)])  # ... the first operand's rows
+                                   (4, 2048, 32 * 49, 2048), (3, 1000, 32 * 52, 1104),   # ... the first operand's rows
+                                   (8, 1024, 32, 1024), (3, 500, 64, 392), (16, 512, 96, 512)])  # one to three blocks of K
 def test_matmul_fp_gemm_within_dot_product_bound(ctx, kind, shape):
     n, h, c, w = shape
     rng = np.random.default_rng(8 + h)
