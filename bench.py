@@ -41,7 +41,7 @@ PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by what
 # the same counters read for a plain copy of known size (the committed rocprofv3 summaries hold the raw
 # figures).
-MEASURED_TRAFFIC_BYTES = {"c3": 3619281, "c2": 50584017, "c4": 12185797, "c5a": 22432246, "c5b": 268617295,
+MEASURED_TRAFFIC_BYTES = {"c3": 3619281, "c2": 50589106, "c4": 12185797, "c5a": 22443535, "c5b": 268661559,
                           "maxpool": 32143337, "avgpool": 32181860, "tconv": 8354359, "conv3d": 8034721,
                           "rescale": 64316729, "c4x8": 96453041, "c3x4": 13335922}
 
