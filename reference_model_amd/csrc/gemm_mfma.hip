@@ -1349,14 +1349,18 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
 {
     if (g.KH * g.KW == 1)
         return true;
-    if (in_dtype != TMI_INT8)
-        return g.IC >= 128;
+    if (in_dtype != TMI_INT8 && g.IC >= 128)
+        return true;
     // int8 layers with taps: where this kernel can keep the input patch in LDS it is the faster one.  us patch
     // kernel / this kernel (host clock): 3x3 [16,28,28,256]->256 25.3 / 19.8, [8,28,28,512]->512 37.3 / 28.4,
     // [16,56,56,128]->128 29.0 / 22.6, [32,28,28,256]->256 39.8 / 33.6; with the fused RESCALE 19.4 / 18.7,
-    // 31.7 / 28.3, (slab kernel 15.3) / 24.8, 41 / 36.9.
+    // 31.7 / 28.3, (slab kernel 15.3) / 24.8, 41 / 36.9.  The same for fp16 / bf16 layers with fewer than 128
+    // channels, which the form without the patch loses: fp16 3x3 [8,56,56,64]->128 11.0 / 9.3, ->256 20.1 / 16.6,
+    // [16,28,28,64]->256 11.3 / 8.9, [8,56,56,96]->192 26.0 / 20.1, [8,56,56,32]->128 8.3 / 6.6
+    // (without the patch, [32,56,56,64]->64: 20.3 / 30.6).
     int rows, patch_h, patch_w;
-    return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, g.IC, g.OC, rows,
+    const int icb = g.IC * (in_dtype == TMI_INT8 ? 1 : 2);
+    return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, icb, g.OC, rows,
                                patch_h, patch_w);
 }
 

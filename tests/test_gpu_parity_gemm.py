@@ -281,6 +281,11 @@ TAP_SHAPES = [  # n, ih, iw, ic, oc, kh, kw, pad, stride, dilation
     (20, 26, 21, 192, 136, 2, 3, (0, 1, 2, 0), (1, 1), (1, 1)),     # uneven padding, 6 blocks per tap
     (24, 20, 36, 256, 128, 1, 3, (0, 0, 1, 1), (1, 1), (1, 1)),     # one row of taps, tiles of 3 rows
     (3, 30, 26, 128, 200, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # 48 tiles of whole rows where 128-pixel tiles would be 38
+    (12, 30, 28, 64, 136, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # few channels: one (int8) or two (fp) blocks per tap
+]
+FP_TAP_SHAPES = [  # rows of K that are whole 64-byte blocks for two-byte elements only
+    (12, 28, 30, 32, 128, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # one block per tap
+    (10, 33, 25, 96, 160, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),      # three
 ]
 
 
@@ -312,7 +317,7 @@ def test_conv2d_taps_i8_gemm_pads_with_the_input_zero_point(ctx, in_zp):
     assert np.array_equal(got, cases.conv2d_exact_blas(x, w, bias, (1, 1, 1, 1), (1, 1), (1, 1), in_zp, -4))
 
 
-@pytest.mark.parametrize("shape", TAP_SHAPES)
+@pytest.mark.parametrize("shape", TAP_SHAPES + FP_TAP_SHAPES)
 @pytest.mark.parametrize("kind", ["fp16", "bf16"])
 def test_conv2d_taps_fp_gemm_within_dot_product_bound(ctx, shape, kind):
     n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
@@ -422,7 +427,8 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (1, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_f16"),       # pointwise with 16 tiles: still the GEMM kernel
     (capi.FP16, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_f16"),          # 3x3, no patch form (49 pixels a tile), 100 tiles
     (capi.FP16, (32, 7, 7, 512, 512, 3, 1), "conv2d_mfma_f16"),        # the same with 52 tiles: the patch kernel
-    (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64
+    (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64, too few output channels for the patch form
+    (capi.FP16, (8, 56, 56, 64, 128, 3, 1), "gemm_mfma_f16_patch"),    # the same with 128: the GEMM kernel's patch form
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_f16"),          # pointwise with two blocks of K
     (capi.INT8, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_i8"),           # int8 pointwise, int32 results, 6.4 M of them: before the slab kernel
     (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_slab_i8"),          # the same with 1.6 M results: the slab kernel
