@@ -1358,6 +1358,14 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
     // channels, which the form without the patch loses: fp16 3x3 [8,56,56,64]->128 11.0 / 9.3, ->256 20.1 / 16.6,
     // [16,28,28,64]->256 11.3 / 8.9, [8,56,56,96]->192 26.0 / 20.1, [8,56,56,32]->128 8.3 / 6.6
     // (without the patch, [32,56,56,64]->64: 20.3 / 30.6).
+    // int8 layers with taps and a stride: the patch kernel's patch grows with the stride, this kernel's loads do
+    // not.  us patch kernel / this kernel, 3x3 stride 2: [64,28,28,256]->256 (196 tiles) 34.6 / 22.3,
+    // [32,56,56,192]->192 45.2 / 26.8, [128,14,14,512]->512 89.1 / 33.8, [32,28,28,256]->512 34.4 / 21.8; with the
+    // fused RESCALE 30.3 / 22.1, 49.4 / 28.2, 88.2 / 34.4, 29.9 / 22.0.  Around 100 tiles the two tie
+    // ([32,28,28,512]->256 32.4 / 33.1, [32,28,28,192]->256 17.6 / 17.9, fused 15.5 / 19.0), so from 128 on.
+    if (in_dtype == TMI_INT8 && g.stride_y * g.stride_x > 1 &&
+        ((int64_t)g.N * g.OH * g.OW + 127) / 128 * ((g.OC + 127) / 128) >= 128)
+        return true;
     int rows, patch_h, patch_w;
     const int icb = g.IC * (in_dtype == TMI_INT8 ? 1 : 2);
     return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, icb, g.OC, rows,

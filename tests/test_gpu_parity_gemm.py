@@ -414,11 +414,13 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
 
 # ---- which MFMA kernel a convolution gets when the choice is left open ----
 @pytest.mark.parametrize("dtype, shape, kernel", [
-    # n, ih, iw, ic, oc, k, pad
+    # n, ih, iw, ic, oc, k, pad[, stride]
     (capi.INT8, (8, 56, 56, 192, 64, 3, 1), "conv2d_mfma_i8"),         # 3x3 int8: the patch kernel
     (capi.INT8, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_i8_patch"),   # 3x3 int8 whose patch the GEMM kernel can keep in LDS
     (capi.INT8, (16, 28, 28, 1024, 256, 3, 1), "conv2d_mfma_i8"),      # 3x3 int8 whose patch (6 x 30 x 1 KB) does not fit
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
+    (capi.INT8, (64, 28, 28, 256, 256, 3, 1, 2), "gemm_mfma_i8"),      # 3x3 int8 with stride 2 and 200 tiles: the GEMM kernel
+    (capi.INT8, (32, 28, 28, 256, 256, 3, 1, 2), "conv2d_mfma_i8"),    # the same with 100 tiles: the patch kernel
     (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),  # 3x3 fp16, deep K, the patch fits the LDS
     (capi.FP16, (8, 28, 28, 512, 512, 3, 1), "gemm_mfma_f16"),         # the same with a patch that does not fit
     (capi.FP16, (4, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),   # 56 tiles of four output rows: enough for the patch form
@@ -434,7 +436,9 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_slab_i8"),          # the same with 1.6 M results: the slab kernel
 ])
 def test_automatic_kernel_choice(dtype, shape, kernel):
-    n, ih, iw, ic, oc, k, pad = shape
+    n, ih, iw, ic, oc, k, pad = shape[:7]
+    stride = shape[7] if len(shape) > 7 else 1
+    pads = (pad,) * 4 if stride == 1 else (pad, pad - 1, pad, pad - 1)    # 28 + 1 - 3 is a multiple of 2
     rng = np.random.default_rng(ic + oc + k)
     if dtype == capi.INT8:
         x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
@@ -446,12 +450,12 @@ def test_automatic_kernel_choice(dtype, shape, kernel):
         b = rng.normal(0, 1, oc).astype(np.float16)
     c = Context(0)
     try:
-        got, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
+        got, st = gpu_ops.conv2d(c, x, w, b, pads, (stride, stride), dtype=dtype)
         assert st == capi.VALID and c.last_kernel == kernel
         # the kernel not chosen, where it takes the shape at all
         c.set_kernel_choice(capi.KERNEL_GEMM if kernel.startswith("conv2d") else capi.KERNEL_MFMA)
         try:
-            other, st = gpu_ops.conv2d(c, x, w, b, (pad,) * 4, dtype=dtype)
+            other, st = gpu_ops.conv2d(c, x, w, b, pads, (stride, stride), dtype=dtype)
         except TmiError:
             # the GEMM kernel refuses layers with too few tiles; the patch kernel, which takes any shape, is then
             # the only one
