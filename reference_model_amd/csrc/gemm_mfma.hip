@@ -1363,9 +1363,20 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
     // [32,56,56,192]->192 45.2 / 26.8, [128,14,14,512]->512 89.1 / 33.8, [32,28,28,256]->512 34.4 / 21.8; with the
     // fused RESCALE 30.3 / 22.1, 49.4 / 28.2, 88.2 / 34.4, 29.9 / 22.0.  Around 100 tiles the two tie
     // ([32,28,28,512]->256 32.4 / 33.1, [32,28,28,192]->256 17.6 / 17.9, fused 15.5 / 19.0), so from 128 on.
-    if (in_dtype == TMI_INT8 && g.stride_y * g.stride_x > 1 &&
-        ((int64_t)g.N * g.OH * g.OW + 127) / 128 * ((g.OC + 127) / 128) >= 128)
-        return true;
+    // Without a stride the patch kernel is the faster one on the mid-sized layers the rule was first measured on
+    // (100 - 200 tiles: [16,28,28,256]->256 23.7 / 25.9, [16,14,14,512]->512 36.4 / 39.8) and loses beyond: 3x3
+    // [16,28,28,1024]->256 (196 tiles) 63.0 / 60.3, [20,28,28,1024]->256 (246) 101.3 / 64.7, [32,28,28,1024]->256
+    // 109.4 / 93.3, [12,56,56,512]->128 59.3 / 51.2, [16,56,56,512]->128 64.2 / 52.6; with the fused RESCALE 58.9 / 60.5,
+    // 121.3 / 65.3, 113.4 / 94.2, 68.6 / 52.2, 61.4 / 53.2.  On images smaller than a tile it loses from this kernel's
+    // minimum on: [32,7,7,1024]->1024 (104 tiles) 74.0 / 58.8, [64,7,7,512]->512 42.4 / 32.8, [128,7,7,1024]->1024
+    // 288.4 / 93.8.  With 64 output channels half of this kernel's tile is empty and the patch kernel stays ahead
+    // ([32,56,56,256]->64 45.4 / 59.2).
+    if (in_dtype == TMI_INT8 && g.OC >= 96)
+    {
+        const int64_t tiles = ((int64_t)g.N * g.OH * g.OW + 127) / 128 * ((g.OC + 127) / 128);
+        if (tiles >= (g.stride_y * g.stride_x > 1 ? 128 : 200) || (g.OH * g.OW <= 64 && tiles >= 96))
+            return true;
+    }
     int rows, patch_h, patch_w;
     const int icb = g.IC * (in_dtype == TMI_INT8 ? 1 : 2);
     return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, icb, g.OC, rows,

@@ -421,6 +421,8 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.INT8, (16, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_i8"),       # pointwise: the GEMM kernel
     (capi.INT8, (64, 28, 28, 256, 256, 3, 1, 2), "gemm_mfma_i8"),      # 3x3 int8 with stride 2 and 200 tiles: the GEMM kernel
     (capi.INT8, (32, 28, 28, 256, 256, 3, 1, 2), "conv2d_mfma_i8"),    # the same with 100 tiles: the patch kernel
+    (capi.INT8, (20, 28, 28, 1024, 256, 3, 1), "gemm_mfma_i8"),        # 3x3 int8 outside the patch form, 246 tiles: the GEMM kernel
+    (capi.INT8, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_i8"),           # images smaller than a tile, 100 tiles: the GEMM kernel
     (capi.FP16, (16, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),  # 3x3 fp16, deep K, the patch fits the LDS
     (capi.FP16, (8, 28, 28, 512, 512, 3, 1), "gemm_mfma_f16"),         # the same with a patch that does not fit
     (capi.FP16, (4, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),   # 56 tiles of four output rows: enough for the patch form
