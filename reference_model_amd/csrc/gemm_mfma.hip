@@ -1371,12 +1371,19 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
     // minimum on: [32,7,7,1024]->1024 (104 tiles) 74.0 / 58.8, [64,7,7,512]->512 42.4 / 32.8, [128,7,7,1024]->1024
     // 288.4 / 93.8.  With 64 output channels half of this kernel's tile is empty and the patch kernel stays ahead
     // ([32,56,56,256]->64 45.4 / 59.2).
+    const int64_t tiles = ((int64_t)g.N * g.OH * g.OW + 127) / 128 * ((g.OC + 127) / 128);
     if (in_dtype == TMI_INT8 && g.OC >= 96)
     {
-        const int64_t tiles = ((int64_t)g.N * g.OH * g.OW + 127) / 128 * ((g.OC + 127) / 128);
         if (tiles >= (g.stride_y * g.stride_x > 1 ? 128 : 200) || (g.OH * g.OW <= 64 && tiles >= 96))
             return true;
     }
+    // fp16 / bf16 layers with taps and 64 or 96 channels outside the patch form (a stride, rows wider than a tile): what
+    // the patch kernel wins there are the layers with 64 output channels.  fp16 3x3, us patch kernel / this kernel:
+    // stride 2 [32,56,56,64]->128 (196 tiles) 16.6 / 11.5, [64,28,28,96]->192 21.5 / 13.4, [64,56,56,64]->128
+    // 29.9 / 17.5, [32,56,56,64]->256 29.5 / 17.6; stride 1 [2,160,160,64]->128 30.9 / 17.5, [8,160,160,64]->96
+    // 66.2 / 49.5; with 32 channels the two tie ([16,112,112,32]->128 stride 2 13.2 / 13.4).
+    if (in_dtype != TMI_INT8 && g.IC >= 64 && g.OC >= 96 && tiles >= 196)
+        return true;
     int rows, patch_h, patch_w;
     const int icb = g.IC * (in_dtype == TMI_INT8 ? 1 : 2);
     return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, icb, g.OC, rows,
