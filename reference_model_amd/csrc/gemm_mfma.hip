@@ -1349,7 +1349,12 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
 {
     if (g.KH * g.KW == 1)
         return true;
-    if (in_dtype != TMI_INT8 && g.IC >= 128)
+    // fp16 / bf16 layers with taps and 128 channels or more are this kernel's, except those that leave half of its
+    // 128-channel tile empty: 3x3 stride 1, us patch kernel / this kernel: [32,56,56,256]->64 57.7 / 75.2,
+    // [8,112,112,128]->64 33.6 / 45.7, [16,56,56,128]->64 18.1 / 24.8 (a tie from 512 channels on:
+    // [32,28,28,512]->64 40.6 / 40.4; with a stride this kernel again: [32,56,56,256]->64 stride 2 35.5 / 24.4;
+    // and from 80 output channels: [64,28,28,512]->80 93.3 / 79.7, [16,56,56,256]->96 53.4 / 40.3).
+    if (in_dtype != TMI_INT8 && g.IC >= 128 && !(g.OC <= 64 && g.IC < 512 && g.stride_y * g.stride_x == 1))
         return true;
     // int8 layers with taps: where this kernel can keep the input patch in LDS it is the faster one.  us patch
     // kernel / this kernel (host clock): 3x3 [16,28,28,256]->256 25.3 / 19.8, [8,28,28,512]->512 37.3 / 28.4,
