@@ -25,6 +25,7 @@
 //
 // weight_zp must be 0 (the usual case for int8 weights); the patch kernel takes everything else.
 #include <cstring>
+#include <type_traits>
 
 #include "tmi_mfma.h"
 
@@ -70,6 +71,13 @@ __device__ __forceinline__ void slab_load_off(uint32_t off, const void* base, ui
 {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds_addr)
                  : "memory");
+}
+
+// A workgroup barrier that waits for this wave's LDS accesses and nothing else: loads into LDS that are still in flight
+// (counted by vmcnt) stay in flight across it.
+__device__ __forceinline__ void slab_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // CH: 16-byte chunks of a channel vector (4, 6, 8: 64, 96, 128 input channels)
@@ -484,6 +492,449 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     raise_flags(a.flag_word, flags);
 }
 
+// 3x3 layers with 64 input channels, unit stride and a fused RESCALE (the headline layer and its larger batches): tiles of
+// up to several hundred pixels, and the weights in registers.  A wave owns one of the block's two channel tiles of 32
+// for the whole workgroup, so after the barrier it reads its 18 weight fragments (72 registers) from LDS once and then
+// walks the tile's pixel tiles of 32 (wave w: channel tile w % 2, pixel tiles w / 2, w / 2 + 4, ...).  A K step is one
+// fragment read and one matrix instruction (the kernel above reads 2.5 fragments per matrix instruction with one
+// accumulator tile per wave and 1.5 with two) and a workgroup loads the weight slab once for all its pixels.
+// input_zp * sum(w) comes from the weight registers (dot products with a word of ones, once per wave), so all 32
+// columns of a pixel tile are pixels, and a tile starts from bias - input_zp * sum(w) as the third operand of its first
+// matrix instruction.  What bounds a workgroup once its operands have landed is the rate at which a wave issues
+// instructions (two waves per SIMD: about one instruction per eight clocks each), so the loop is written to issue as
+// few as it can: with one shift for all channels the requantisation of a pixel tile is dealt over the K steps of the
+// wave's next one, four instructions per output element, and the fragments of the next tile are requested in the last
+// steps of the current one.
+template <bool ZA>
+__global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
+{
+    constexpr int KH = 3, KW = 3, CH = 4;    // 3x3 taps of 64 input channels: 18 weight fragments, 72 registers
+    constexpr int NW = 8;
+    asm volatile("" ::"s"(a.in), "s"(a.rp.shift), "s"(a.rp.out_zp), "s"(*reinterpret_cast<const uint32_t*>(&a.rp.scale32)),
+                 "s"(*reinterpret_cast<const uint32_t*>(&a.rp.in_bits)), "s"(a.rp.lo), "s"(a.N), "s"(a.TH), "s"(a.bias_len),
+                 "s"(a.div_ocb.d));
+    constexpr int TAPS   = KH * KW;
+    constexpr int RW     = TAPS * CH + 1;    // chunks per weight row in LDS (odd)
+    constexpr int KB     = CH * 16;          // bytes of a channel vector
+    constexpr int WSLOTS = 64 * RW;
+    constexpr int WLOADS = (WSLOTS + 63) / 64;
+    constexpr int RP     = CH + 1;          // chunks per patch pixel in LDS (odd)
+    constexpr int LWAVES = NW - 1;          // waves that issue loads; the eighth builds the tables
+    constexpr int STEPS  = TAPS * (CH / 2);
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // LDS: [weight rows][patch][64 x ChannelScale][64 x HighWordScale][64 multipliers][64 biases][the block's common shift]
+    //      [8 waves x 32 start values]
+    const int tid    = threadIdx.x;
+    const int lane   = tid & 63;
+    const int wave   = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li     = lane & 31;
+    const int lh     = lane >> 5;
+    const int p_slots = a.PH * a.pitch;
+    const int p_loads = (p_slots + 63) >> 6;
+    uint8_t* wl       = lds;
+    uint8_t* pl       = lds + WLOADS * 1024;
+    const int row_step   = a.dy * a.pitch * 16;
+    const int col_step   = a.dx * RP * 16;
+    uint8_t* tabs        = pl + p_loads * 1024;
+    ChannelScale* tab_cs = reinterpret_cast<ChannelScale*>(tabs);
+    HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(tabs + 64 * sizeof(ChannelScale));
+    int32_t* tab_m       = reinterpret_cast<int32_t*>(tab_hw + 64);    // multipliers
+    int32_t* tab_b       = tab_m + 64;                                 // biases
+    int32_t* uni_shift   = tab_b + 64;                                 // 4 words, one used
+    int32_t* wave_start  = uni_shift + 4 + wave * 32;                  // this wave's start values
+
+    uint32_t bid = blockIdx.x;
+    if (a.xcd_remap)
+    {
+        const uint32_t per = (uint32_t)a.xcd_remap;
+        bid                = (bid & 7) * per + (bid >> 3);
+    }
+    const uint32_t tile = fdiv(bid, a.div_ocb);
+    const int ocb       = bid - tile * a.n_ocb;
+    const uint32_t trow = fdiv(tile, a.div_tiles_x);
+    const int txi       = tile - trow * a.tiles_x;
+    const int n         = fdiv(trow, a.div_tiles_y);
+    const int tyi       = trow - n * a.tiles_y;
+    const int oy0 = tyi * a.TH, ox0 = txi * a.TW;
+    const int oc0 = ocb * 64;
+    const int y0 = oy0 * a.sy - a.pad_top, x0 = ox0 * a.sx - a.pad_left;
+
+    uint32_t flags = 0;
+    const int ct = wave & 1, q = wave >> 1;
+    // MFMA operand row li holds channel 16*((li>>2)&1) + 4*(li>>3) + (li&3) of the tile's 32, so that a lane's 16
+    // accumulators are 16 consecutive channels
+    const int wr  = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
+    const int ocl = ct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
+    const bool chan_ok = oc0 + ocl < a.OC;    // OC is a multiple of 16: a lane's 16 channels are in or out together
+    // the bias of the channel whose weight row this lane holds: asked for now, needed after the weights are in registers
+    int32_t bias_row = 0;
+    if constexpr (ZA)
+        bias_row = oc0 + ct * 32 + wr < a.OC ? a.bias[a.bias_len == 1 ? 0 : oc0 + ct * 32 + wr] : 0;
+    const uint32_t lbase = (uint32_t)(uintptr_t)lds;
+    if (wave < LWAVES)
+    {
+        {
+            // Weights: LDS row r is channel r of the block, slot s = (row, chunk) reads byte 16 (s - row) of the block's
+            // weights; seven loads on are 448 slots.  Whatever lies past the block's last channel is clamped to its last chunk.
+            const int rows       = a.OC - oc0 < 64 ? a.OC - oc0 : 64;
+            const uint32_t limit = (uint32_t)rows * (TAPS * KB) - 16u;
+            const uint8_t* wb    = a.w + (size_t)oc0 * (TAPS * KB);
+            for (int l = wave; l < WLOADS; l += LWAVES)
+            {
+                const int s0       = l * 64 + lane;
+                const int row0     = s0 / RW;
+                const uint32_t off = 16u * (uint32_t)(s0 - row0);
+                slab_load_off(off < limit ? off : limit, wb, lbase + l * 1024);
+            }
+        }
+        {
+            const uint8_t* in_n = a.in + (size_t)n * (a.IH * a.IW) * KB;
+            int lp              = wave + ((WLOADS - wave + LWAVES - 1) / LWAVES) * LWAVES - WLOADS;    // first patch load of this wave
+            const int s0        = lp * 64 + lane;
+            int py              = fdiv(s0, a.div_pitch);    // patch row and chunk inside the row
+            int r               = s0 - py * a.pitch;
+            uint32_t dst        = lbase + (WLOADS + lp) * 1024;
+            for (; lp < p_loads; lp += LWAVES)
+            {
+                const int px   = (int)((uint32_t)r / (uint32_t)RP);
+                const int ch   = r - px * RP;
+                const int iy = y0 + py, ix = x0 + px;
+                const bool img = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+                const int c16  = (ch < CH ? ch : 0) * 16;
+                const uint32_t pixel = __umul24(iy, a.IW) + ix;
+                const uint8_t* src = img ? in_n + (uint32_t)(pixel * KB + c16) : a.pad_page + (c16 & 48);
+                slab_load(src, dst);
+                dst += LWAVES * 1024;
+                r += a.step_chunk, py += a.step_row;
+                if (r >= a.pitch)
+                    r -= a.pitch, py++;
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    else
+    {
+        // the table wave: bias and the per-channel RESCALE constants, one channel per lane
+        const int oc    = oc0 + lane;
+        const bool ok   = oc < a.OC;
+        const int occ   = ok ? oc : 0;
+        {
+            const int32_t m_raw   = load_multiplier(a.rp, occ);
+            const int32_t s_raw   = load_shift(a.rp, occ);
+            const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
+            const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
+            // the three forms of the epilogue, chosen as in the kernel above
+            const int s_min = a.rp.double_round ? 33 : 32;
+            const int folds = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp));
+            const int uni   = folds && __all(cs.s == s_first);
+            tab_cs[lane]    = cs;
+            tab_hw[lane]    = make_high_word_scale(cs, a.rp.out_zp);
+            const int relu = a.rp.double_round && a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
+            if (lane == 0)
+                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? -2 : -1);
+            tab_m[lane] = cs.m;
+        }
+        tab_b[lane] = ok ? a.bias[a.bias_len == 1 ? 0 : occ] : 0;
+    }
+    slab_barrier();    // weights, patch and tables are in LDS
+    v4i fa[STEPS];
+    {
+        const uint8_t* wrow = wl + ((ct * 32 + wr) * RW) * 16 + lh * 16;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+            fa[s] = *reinterpret_cast<const v4i*>(wrow + s * 32);
+        if constexpr (ZA)
+        {
+            // sum(w) of the row this lane holds: its own half of K in every step, plus the other half from lane ^ 32;
+            // four partial sums, because one dependent chain of 4 * STEPS dot products would be the longest thing a wave
+            // does here
+            int part[4] = { 0, 0, 0, 0 };
+#pragma unroll
+            for (int s = 0; s < STEPS; s++)
+            {
+                part[0] = __builtin_amdgcn_sdot4(fa[s].x, 0x01010101, part[0], false);
+                part[1] = __builtin_amdgcn_sdot4(fa[s].y, 0x01010101, part[1], false);
+                part[2] = __builtin_amdgcn_sdot4(fa[s].z, 0x01010101, part[2], false);
+                part[3] = __builtin_amdgcn_sdot4(fa[s].w, 0x01010101, part[3], false);
+            }
+            int sum = (part[0] + part[1]) + (part[2] + part[3]);
+            sum += __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, sum);
+            if (lh == 0)
+                wave_start[wr] = (int32_t)((uint32_t)bias_row - (uint32_t)a.za * (uint32_t)sum);
+            __builtin_amdgcn_wave_barrier();    // the wave's own LDS accesses complete in order
+        }
+    }
+    // what a tile starts from (bias - input_zp * sum(w) of the lane's 16 channels): the third operand of its first matrix
+    // instruction
+    v16i start;
+    {
+        const int32_t* b16 = ZA ? wave_start + 16 * lh : tab_b + ocl;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+        {
+            const v4i b4 = *reinterpret_cast<const v4i*>(b16 + 4 * g);
+            start[4 * g] = b4[0], start[4 * g + 1] = b4[1], start[4 * g + 2] = b4[2], start[4 * g + 3] = b4[3];
+        }
+    }
+    const int P        = a.TH * a.TW;
+    const int NT       = (P + 31) >> 5;
+    // the pixel fragments of step s + DEPTH are requested before the matrix instruction of step s, order pinned
+    constexpr int AHEAD = 8;
+    constexpr int DEPTH = STEPS < AHEAD ? STEPS : AHEAD;
+    const int form = __builtin_amdgcn_readfirstlane(*uni_shift);
+    if (form >= 0)
+    {
+        if (q < NT)
+        {
+            // One shift for every channel of the block (the usual case): the requantisation of a pixel tile runs between
+            // the matrix instructions of the wave's next pixel tile, one output element per K step, so that the vector
+            // ALU works while the matrix core does.  (Left to themselves the two waves of a SIMD run their K loops and
+            // their epilogues in step, and matrix core and vector ALU take turns.)
+            const int s_uni   = form & 255;
+            const bool sign   = a.rp.double_round && !(form >> 8);    // the rounding term depends on the value's sign
+            const int64_t rnd = (int64_t(1) << (s_uni - 1)) + (a.rp.double_round ? (int64_t(1) << 30) : 0) +
+                                ((int64_t)a.rp.out_zp << s_uni);
+            const int32_t hi_p  = (int32_t)(rnd >> 32);
+            const uint32_t lo_p = (uint32_t)rnd;
+            const int sh        = s_uni - 32;
+            int32_t cm[16];    // multipliers of the lane's channels
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+            {
+                const v4i m4 = *reinterpret_cast<const v4i*>(tab_m + ocl + 4 * g);
+                cm[4 * g] = m4[0], cm[4 * g + 1] = m4[1], cm[4 * g + 2] = m4[2], cm[4 * g + 3] = m4[3];
+            }
+            const int32_t v_lo = a.rp.lo, v_hi = a.rp.hi;
+            // SIGN: the rounding term depends on the value's sign; WIDE: int16 results (two stores) instead of int8
+            auto pipelined = [&](auto SIGN, auto WIDE) {
+                constexpr bool kSign = decltype(SIGN)::value, kWide = decltype(WIDE)::value;
+                struct Place
+                {
+                    uint32_t prow;    // byte offset of the lane's pixel under tap (0, 0) in the patch
+                    uint32_t base;    // the lane's first output element
+                    uint32_t ok;      // whether the lane stores
+                };
+                auto place = [&](int pt) {
+                    int p              = pt * 32 + li;
+                    const bool in_tile = p < P;
+                    p                  = in_tile ? p : 0;
+                    const int ty       = fdiv(p, a.div_tw);
+                    const int tx       = p - ty * a.TW;
+                    const int oy = oy0 + ty, ox = ox0 + tx;
+                    return Place{ (uint32_t)((ty * a.sy * a.pitch + tx * a.sx * RP) * 16 + lh * 16),
+                                  (uint32_t)(((n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl),
+                                  (uint32_t)(in_tile && oy < a.OH && ox < a.OW && chan_ok) };
+                };
+                v4i fb[STEPS];
+                auto request = [&](const Place& at, int s) {
+                    const int tap = s / (CH / 2), h = s % (CH / 2);
+                    fb[s]         = *reinterpret_cast<const v4i*>(pl + at.prow + (tap / KW) * row_step + (tap % KW) * col_step + h * 32);
+                };
+                int32_t r[4];
+                v4i pk, pk2;
+                // the requantisation of tile `done` (accumulators prv), dealt over the K steps of the tile after it: step 0
+                // nothing (the last matrix instruction of `done` is still running), steps 1..16 one element each, packed
+                // as soon as a word is complete, step 17 stores
+                auto requant_piece = [&](int s, const v16i& prv, const Place& done) {
+                    if (s >= 1 && s <= 16)
+                    {
+                        const int e = s - 1;
+                        r[e & 3]    = kSign ? clamp_med3(high_word_rescale<true>(prv[e], cm[e], hi_p, lo_p, sh), v_lo, v_hi)
+                                          : clamp_med3(high_word_rescale_const(prv[e], cm[e], rnd, sh), v_lo, v_hi);
+                        if constexpr (!kWide)
+                        {
+                            if ((e & 3) == 3)
+                            {
+                                const int lo2 = __builtin_amdgcn_perm(r[1], r[0], 0x0c0c0400);
+                                const int hi2 = __builtin_amdgcn_perm(r[3], r[2], 0x04000c0c);
+                                pk[e >> 2]    = lo2 | hi2;
+                            }
+                        }
+                        else if (e & 1)
+                        {
+                            const int word = (r[(e & 3) - 1] & 0xffff) | ((r[e & 3] & 0xffff) << 16);
+                            if (e < 8)
+                                pk[e >> 1] = word;
+                            else
+                                pk2[(e - 8) >> 1] = word;
+                        }
+                    }
+                    else if (s == 17 && done.ok)
+                    {
+                        if constexpr (!kWide)
+                            *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + done.base) = pk;
+                        else
+                        {
+                            int16_t* o                       = reinterpret_cast<int16_t*>(a.out) + done.base;
+                            *reinterpret_cast<v4i*>(o)     = pk;
+                            *reinterpret_cast<v4i*>(o + 8) = pk2;
+                        }
+                    }
+                };
+                // One tile: its K loop, with the first fragments of the tile after it requested in its last steps (so that
+                // the matrix instructions of consecutive tiles follow each other without a gap) and the requantisation of
+                // the tile before it between its matrix instructions.
+                auto tile = [&](v16i& acc, const v16i& prv, const Place& cur, const Place& next, const Place& done, auto REQUANT) {
+#pragma unroll
+                    for (int s = 0; s < STEPS; s++)
+                    {
+                        if (s + DEPTH < STEPS)
+                            request(cur, s + DEPTH);
+                        else
+                            request(next, s + DEPTH - STEPS);
+                        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], s == 0 ? start : acc, 0, 0, 0);
+                        if constexpr (decltype(REQUANT)::value)
+                            requant_piece(s, prv, done);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                };
+                v16i acc0 = start, acc1 = start;
+                int pt      = q;
+                Place cur   = place(pt), next = pt + (NW / 2) < NT ? place(pt + (NW / 2)) : cur, done = cur;
+#pragma unroll
+                for (int s = 0; s < DEPTH; s++)
+                    request(cur, s);
+                __builtin_amdgcn_sched_barrier(0);
+                tile(acc0, acc1, cur, next, done, std::false_type{});
+                while (true)
+                {
+                    // acc0 holds tile pt; the next one goes into acc1
+                    done = cur, cur = next, pt += (NW / 2);
+                    if (pt >= NT)
+                    {
+#pragma unroll
+                        for (int s = 0; s < 18; s++)
+                            requant_piece(s, acc0, done);
+                        break;
+                    }
+                    next = pt + (NW / 2) < NT ? place(pt + (NW / 2)) : cur;
+                    tile(acc1, acc0, cur, next, done, std::true_type{});
+                    done = cur, cur = next, pt += (NW / 2);
+                    if (pt >= NT)
+                    {
+#pragma unroll
+                        for (int s = 0; s < 18; s++)
+                            requant_piece(s, acc1, done);
+                        break;
+                    }
+                    next = pt + (NW / 2) < NT ? place(pt + (NW / 2)) : cur;
+                    tile(acc0, acc1, cur, next, done, std::true_type{});
+                }
+            };
+            if (a.out_kind == 1)
+                sign ? pipelined(std::true_type{}, std::false_type{}) : pipelined(std::false_type{}, std::false_type{});
+            else
+                sign ? pipelined(std::true_type{}, std::true_type{}) : pipelined(std::false_type{}, std::true_type{});
+        }
+        raise_flags(a.flag_word, flags);
+        return;
+    }
+    // Shifts that differ between the channels (or lie outside the high-word form): tile after tile, K loop and then the
+    // requantisation with per-channel constants from the tables.
+    for (int pt = q; pt < NT; pt += (NW / 2))
+    {
+        int p              = pt * 32 + li;
+        const bool in_tile = p < P;
+        p                  = in_tile ? p : 0;
+        const int ty       = fdiv(p, a.div_tw);
+        const int tx       = p - ty * a.TW;
+        const uint8_t* prow = pl + (ty * a.sy * a.pitch + tx * a.sx * RP) * 16 + lh * 16;
+        v16i acc = start;
+        v4i fb[STEPS];
+        auto request = [&](int s) {
+            const int tap = s / (CH / 2), h = s % (CH / 2);
+            fb[s]         = *reinterpret_cast<const v4i*>(prow + (tap / KW) * row_step + (tap % KW) * col_step + h * 32);
+        };
+#pragma unroll
+        for (int s = 0; s < DEPTH; s++)
+            request(s);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < STEPS; s++)
+        {
+            if (s + DEPTH < STEPS)
+                request(s + DEPTH);
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+
+        // (lane, register 4g + j) = D[row 8g + 4 lh + j][pixel li] = channel 32 ct + 16 lh + 4g + j
+        const int oy = oy0 + ty, ox = ox0 + tx;
+        const bool pix_ok  = in_tile && oy < a.OH && ox < a.OW;
+        const size_t obase = (uint32_t)(((n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl);
+        {
+            // four channels at a time, each group packed as soon as it is done
+            const bool store = pix_ok && chan_ok;
+            v4i pk, pk2;    // int8: pk; int16: pk, pk2
+            uint32_t eflags = 0;
+            auto pack = [&](int g, const int32_t (&r)[4]) {
+                if (a.out_kind == 1)
+                {
+                    const int lo2 = __builtin_amdgcn_perm(r[1], r[0], 0x0c0c0400);
+                    const int hi2 = __builtin_amdgcn_perm(r[3], r[2], 0x04000c0c);
+                    pk[g]         = lo2 | hi2;
+                }
+                else
+                {
+                    const int w0 = (r[0] & 0xffff) | ((r[1] & 0xffff) << 16), w1 = (r[2] & 0xffff) | ((r[3] & 0xffff) << 16);
+                    if (g < 2)
+                        pk[2 * g] = w0, pk[2 * g + 1] = w1;
+                    else
+                        pk2[2 * g - 4] = w0, pk2[2 * g - 3] = w1;
+                }
+            };
+            if (form == -2)
+            {
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                {
+                    int32_t r[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                    {
+                        const HighWordScale c = tab_hw[ocl + 4 * g + j];
+                        r[j] = a.rp.double_round ? clamp_med3(high_word_rescale<true>(acc[4 * g + j], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi)
+                                                 : clamp_med3(high_word_rescale<false>(acc[4 * g + j], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                    }
+                    pack(g, r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                {
+                    int32_t r[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                    {
+                        const ChannelScale cs = tab_cs[ocl + 4 * g + j];
+                        r[j]                  = fast_rescale(acc[4 * g + j], cs, a.rp.out_zp, a.rp.lo, a.rp.hi, eflags);
+                    }
+                    pack(g, r);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (store)
+                    flags |= eflags;    // pixels and channels outside the tensor raise nothing
+            }
+            if (store)
+            {
+                if (a.out_kind == 1)
+                    *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(a.out) + obase) = pk;
+                else
+                {
+                    int16_t* o                       = reinterpret_cast<int16_t*>(a.out) + obase;
+                    *reinterpret_cast<v4i*>(o)     = pk;
+                    *reinterpret_cast<v4i*>(o + 8) = pk2;
+                }
+            }
+        }
+    }
+    raise_flags(a.flag_word, flags);
+}
+
+
 thread_local int32_t last_launch_shape[3] = { 0, 0, 0 };
 
 template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1>
@@ -496,6 +947,19 @@ static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int 
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, st, a);
     last_launch_shape[0] = grid, last_launch_shape[1] = 512, last_launch_shape[2] = lds_bytes;
     return true;
+}
+
+static bool launch_slab_wreg(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
+{
+    auto launch = [&](auto kern) {
+        static LdsLimit granted{};
+        if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
+            return false;
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, st, a);
+        last_launch_shape[0] = grid, last_launch_shape[1] = 512, last_launch_shape[2] = lds_bytes;
+        return true;
+    };
+    return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true>) : launch(conv2d_slab_wreg_kernel<false>);
 }
 
 template <int KH, int KW, int CH>
@@ -560,16 +1024,16 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     struct TileChoice
     {
         int32_t key[8];
-        int th, tw;
-        bool wide;
+        int th, tw, form;
     };
-    static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0, false };
-    const int32_t key[8] = { g.N, g.OH, g.OW, ((n_ocb * 256 + ch) * 4 + g.KH) * 2 + ((tc || c3d) ? 1 : 0), g.stride_y, g.stride_x,
+    // form 0: one accumulator tile per wave, tiles of at most 124 pixels; 1: two accumulator tiles per wave, at most 252
+    // pixels; 2: weights in registers (conv2d_slab_wreg_kernel), tiles as large as the LDS takes
+    static thread_local TileChoice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0, 0 };
+    const int32_t key[8] = { g.N, g.OH, g.OW, (((n_ocb * 256 + ch) * 4 + g.KH) * 2 + ((tc || c3d) ? 1 : 0)) * 2 + (rp.enabled ? 1 : 0), g.stride_y, g.stride_x,
                              g.dil_y, g.dil_x };
-    int best_th = 0, best_tw = 0;
-    bool wide = false;
+    int best_th = 0, best_tw = 0, form = 0;
     if (memcmp(key, last.key, sizeof(key)) == 0)
-        best_th = last.th, best_tw = last.tw, wide = last.wide;
+        best_th = last.th, best_tw = last.tw, form = last.form;
     else
     {
         int64_t best_rounds = 0;
@@ -591,18 +1055,54 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                         best_th = th, best_tw = tw, best_cost = cost, best_rounds = rounds;
                 }
         };
-        search(124, 600);
-        if (best_th && best_rounds > 1 && g.stride_y == 1 && g.stride_x == 1 && !tc && !c3d)
+        // The form with the weights in registers: a workgroup's time is its prologue (arguments, the latency of the
+        // loads, the weight fragments read into registers), its loads (1 KB each) and the matrix instructions of its
+        // busiest SIMD, which holds waves s and s + 4, i.e. the pixel tiles s / 2 + 4 j and s / 2 + 2 + 4 j.
+        auto search_wreg = [&]() {
+            int64_t best_cost = 0;
+            best_th = best_tw = 0;
+            const int steps = taps * ch / 2;
+            for (int th = 1; th <= g.OH; th++)
+                for (int tw = 1; tw <= g.OW; tw++)
+                {
+                    const int ph = (th - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+                    const int pw = (tw - 1) * g.stride_x + (g.KW - 1) * g.dil_x + 1;
+                    const int64_t slots = (int64_t)ph * (pw * rp_chunks + 15);
+                    if (slots >= (1 << 16) || slots * 16 + (taps * ch + 1) * 1024 > 150 * 1024)
+                        break;
+                    const int nt      = (th * tw + 31) / 32;
+                    const int busiest = (nt + 3) / 4 + (nt > 2 ? (nt - 2 + 3) / 4 : 0);
+                    const int64_t tiles  = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw) * n_ocb;
+                    const int64_t rounds = (tiles + 255) / 256;
+                    const int64_t cost   = rounds * (900 + 12 * (taps * ch + 1 + (slots + 63) / 64) + 15 * steps * busiest);
+                    if (!best_th || cost < best_cost || (cost == best_cost && th * tw < best_th * best_tw))
+                        best_th = th, best_tw = tw, best_cost = cost;
+                }
+        };
+        // Measured on MI355X, us per launch (graph replays, fused RESCALE) with one tile per wave / two / the weights in
+        // registers: 3x3 [8,56,56,64]->64 4.18 / 5.04 / 4.09, [10,..] 5.4 / 5.2 / 4.5, [16,..] 5.9 / 5.7 / 5.25, [20,..]
+        // 8.0 / 7.4 / 5.8, [32,..] 10.2 / 8.5 / 7.2, [64,..] 16.6 / 14.9 / 11.8, [8,56,56,64]->128 5.7 / 5.6 / 5.1,
+        // [4,28,28,64]->64 3.6 / 4.2 / 3.3; with 96 or 128 input channels the weights leave no room for the second
+        // accumulator tile and the form loses ([8,56,56,128]->128 9.3 / 7.7 / 8.5), and with int32 results all three tie.
+        const bool plain = !tc && !c3d;
+        if (plain && k33 && ch == 4 && g.stride_y == 1 && g.stride_x == 1 && rp.enabled)
+            search_wreg(), form = 2;
+        else
         {
-            const int th1 = best_th, tw1 = best_tw;
-            search(252, 1100);
-            wide = best_th != 0;
-            if (!wide)
-                best_th = th1, best_tw = tw1;
+            search(124, 600);
+            if (best_th && best_rounds > 1 && g.stride_y == 1 && g.stride_x == 1 && plain)
+            {
+                const int th1 = best_th, tw1 = best_tw;
+                search(252, 1100);
+                form = best_th ? 1 : 0;
+                if (!form)
+                    best_th = th1, best_tw = tw1;
+            }
         }
         memcpy(last.key, key, sizeof(key));
-        last.th = best_th, last.tw = best_tw, last.wide = wide;
+        last.th = best_th, last.tw = best_tw, last.form = form;
     }
+    const bool wide = form == 1;
     if (!best_th)
         return nullptr;
 
@@ -642,6 +1142,11 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 80 * 4 + 16;
     const bool fused = rp.enabled != 0;
     bool ok;
+    if (form == 2)
+    {
+        const int wreg_lds = (w_loads + p_loads) * 1024 + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 64 * 4 + 16 + 8 * 32 * 4;
+        return launch_slab_wreg(st, a, (int)grid, wreg_lds) ? "conv2d_slab_wreg_i8_rescale" : nullptr;
+    }
     if (c3d)
     {
         a.ID = c3d->ID, a.OD = c3d->OD, a.sd = c3d->stride_d, a.dd = c3d->dilation_d, a.pd0 = c3d->pad_d0;

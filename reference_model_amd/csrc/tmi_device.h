@@ -233,6 +233,15 @@ __device__ __forceinline__ int32_t high_word_rescale(int32_t v, int32_t m, int32
     return (int32_t)(pr >> 32) >> sh;
 }
 
+// The same for a rounding term that does not depend on the value's sign (single rounding, or double rounding where a
+// negative value is clamped away anyway): the whole 64-bit term is the addend of the multiply-add, one instruction.
+__device__ __forceinline__ int32_t high_word_rescale_const(int32_t v, int32_t m, int64_t rnd, int32_t sh)
+{
+    int64_t pr;
+    asm("v_mad_i64_i32 %0, vcc, %1, %2, %3" : "=v"(pr) : "v"(v), "v"(m), "s"(rnd) : "vcc");
+    return (int32_t)(pr >> 32) >> sh;
+}
+
 // apply_scale_32 + output_zp + clip (+ CLAMP) for a signed int32 value with zero input_zp.  With a legal
 // value |v| < 2^(s-1) and m < 2^31 the scaled result is below 2^30 in magnitude, so neither of the
 // reference's int32 range checks (quant_util.h:78-82, type_conversion.cpp:352-360) can fire here.

@@ -44,6 +44,11 @@ SLAB_SHAPES = [  # n, ih, iw, oc, pad, stride, dilation[, ic: 64 unless given]
 ]
 
 
+def fused_kernel(ic, stride):
+    """the fused form of a 3x3 layer with 64 input channels and unit stride keeps the weights in registers"""
+    return "conv2d_slab_wreg_i8_rescale" if ic == 64 and tuple(stride) == (1, 1) else "conv2d_slab_i8_rescale"
+
+
 def _operands(shape, seed):
     n, ih, iw, oc, pad, stride, dil = shape[:7]
     ic = shape[7] if len(shape) > 7 else 64
@@ -107,7 +112,7 @@ def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
              shift=rng.integers(36, 42, oc).astype(np.int8), out_zp=zps[1] if out_dtype == np.int8 else 0,
              clamp=(-100, 110) if out_dtype == np.int8 else None)
     got, st, want, wst = _fused(ctx, c, out_dtype)
-    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert ctx.last_kernel == fused_kernel(x.shape[3], stride)
     assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
     assert len(np.unique(got)) > 50
 
@@ -148,7 +153,7 @@ def test_slab_config3_full_size(ctx):
     c = cases.c3()
     got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"],
                              rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"]), clamp=c["clamp"])
-    assert ctx.last_kernel == "conv2d_slab_i8_rescale" and st == capi.VALID
+    assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale" and st == capi.VALID
     acc = cases.conv2d_exact_blas(c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"])
     want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
     assert wst == oracle.VALID and np.array_equal(got, oracle.clamp(want, *c["clamp"]))
@@ -172,6 +177,27 @@ def test_slab_tile_width_follows_the_number_of_tiles(ctx):
     assert grid_of(32, 57, 2) > 32 * 29 * 29 // 252 * 2    # stride 2: tiles of at most 124 pixels
 
 
+@pytest.mark.parametrize("n,hw,shifts", [(8, 56, "uniform"), (32, 56, "uniform"), (32, 56, "mixed"), (5, 50, "uniform"),
+                                         (40, 28, "mixed"), (3, 112, "uniform")])
+def test_slab_weights_in_registers_form_on_large_tiles(ctx, n, hw, shifts):
+    """fused 3x3 layers with 64 input channels: one workgroup per CU walks a tile of several hundred pixels with the
+    weights in registers; with one shift for all channels the requantisation of a pixel tile runs inside the K loop of
+    the next one, otherwise (mixed shifts) after its own"""
+    rng = np.random.default_rng(n * hw)
+    x = rng.integers(-128, 128, (n, hw, hw, 64)).astype(np.int8)
+    w = np.clip(np.rint(rng.normal(0, 30, (64, 3, 3, 64))), -127, 127).astype(np.int8)
+    bias = np.rint(rng.normal(0, 1 << 14, 64)).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, 64).astype(np.int32)
+    shift = np.full(64, 38, np.int8) if shifts == "uniform" else rng.integers(31, 41, 64).astype(np.int8)
+    c = dict(x=x, w=w, bias=bias, in_zp=-7, pad=(1, 1, 1, 1), stride=(1, 1), dilation=(1, 1), mult=mult, shift=shift,
+             out_zp=2, clamp=(0, 127))
+    got, st, want, wst = _fused(ctx, c, np.int8)
+    assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale" and st == wst
+    assert np.array_equal(got, want), int(np.count_nonzero(got != want))
+    if hw == 56 and n in (8, 32):
+        assert ctx.last_launch_shape()[0] == 256    # one round of workgroups: 7 x 14 and 7 x 56 pixels each
+
+
 @pytest.mark.parametrize("mode", [capi.ROUND_SINGLE, capi.ROUND_DOUBLE])
 def test_slab_fused_rescale_per_tensor_scale_and_rounding_modes(ctx, mode):
     shape = (2, 20, 20, 64, (1, 1, 1, 1), (1, 1), (1, 1))
@@ -180,7 +206,7 @@ def test_slab_fused_rescale_per_tensor_scale_and_rounding_modes(ctx, mode):
              mult=np.array([1518500250], np.int32), shift=np.array([44], np.int8), out_zp=-5, clamp=None, mode=mode,
              per_channel=False)
     got, st, want, wst = _fused(ctx, c, np.int8)
-    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale"
     assert st == wst == capi.VALID and np.array_equal(got, want)
 
 
@@ -192,7 +218,7 @@ def test_slab_fused_rescale_reports_require_conditions(ctx):
     c = dict(x=x, w=w, bias=np.zeros(48, np.int32), in_zp=3, pad=shape[4], stride=shape[5], dilation=shape[6],
              mult=np.full(48, 1 << 30, np.int32), shift=np.full(48, 12, np.int8), out_zp=0, clamp=None)
     got, st, want, wst = _fused(ctx, c, np.int8)
-    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale"
     assert st == wst == capi.UNPREDICTABLE and ctx.flags & capi.FLAG_SCALE_VALUE
     # all-zero operands: every value is legal, also in the lanes that hold no pixel or channel of the tensor
     c["x"], c["w"], c["in_zp"] = np.zeros_like(x), np.zeros_like(w), 0
@@ -262,7 +288,7 @@ def test_slab_fused_rescale_epilogue_form_borders(ctx, name, shifts, mode, out_d
     c = dict(x=x, w=w, bias=bias, in_zp=-3, pad=shape[4], stride=shape[5], dilation=shape[6], mult=mult, shift=shift,
              out_zp=out_zp, clamp=None, mode=mode)
     got, st, want, wst = _fused(ctx, c, out_dtype)
-    assert ctx.last_kernel == "conv2d_slab_i8_rescale"
+    assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale"
     assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))
     if small and out_dtype == np.int16:
         assert len(np.unique(got)) > 50
