@@ -113,6 +113,14 @@ int tmi_ctx_sync(tmi_ctx_t* ctx);
  * (activation_funcs.cpp:32) stays with the caller. */
 int tmi_ctx_set_level(tmi_ctx_t* ctx, const tmi_level_t* level);
 
+/* g_func_config.precise_mode / compliance_mode / bounds_mode as far as RESCALE reads them
+ * (reference_model/src/ops/type_conversion.cpp:318-346): with precise_mode an INEXACT_ROUND RESCALE computes the scaled
+ * value in FP64 and truncates it; with compliance_mode as well it first moves the value to the edge of the error bound
+ * the specification grants an FP32 implementation, ceil(x - bound) in the normal pass and floor(x + bound) in the
+ * bounds pass.  All zero (the default): FP32 maths, rounded to nearest.  The floating-point operators take their
+ * precise and bounds passes through the tmi_*_precise entry points and do not read this setting. */
+int tmi_ctx_set_precise_mode(tmi_ctx_t* ctx, int32_t precise_mode, int32_t compliance_mode, int32_t bounds_mode);
+
 /* Flag bits (TMI_FLAG_*) seen by the most recent tmi_ctx_sync(). */
 uint32_t tmi_ctx_flags(const tmi_ctx_t* ctx);
 
@@ -130,6 +138,15 @@ const char* tmi_last_kernel(const tmi_ctx_t* ctx);
  * stream is being captured such a call returns TMI_ERROR instead of allocating -- size the buffer beforehand with
  * this function or with one eager call of the same operator.  Has no counterpart in the reference. */
 int tmi_ctx_reserve_workspace(tmi_ctx_t* ctx, size_t bytes);
+
+/* Size of the scratch buffer in use (`live`) and of the outgrown blocks still held (`retired`); either pointer may be
+ * NULL.  An operator call that outgrows the buffer at least doubles it, so `retired` stays below `live` unless
+ * tmi_ctx_reserve_workspace() was called with sizes of the caller's own choosing.  Has no counterpart in the reference. */
+int tmi_ctx_workspace_bytes(const tmi_ctx_t* ctx, size_t* live, size_t* retired);
+
+/* Frees the outgrown blocks after waiting for the context's stream.  Only for callers that hold no captured HIP graph
+ * from before the last growth: such a graph may still name a block freed here.  Has no counterpart in the reference. */
+int tmi_ctx_trim_workspace(tmi_ctx_t* ctx);
 
 /* ---- device memory (replaces Tensor::allocate / deallocate and the element-wise host copies of
  *      reference_model/src/tensor.cpp:993-1015, 4722-4736) -------------------------------------------- */
@@ -154,9 +171,10 @@ typedef struct
     int32_t stride[2];   /* y, x */
     int32_t dilation[2]; /* y, x */
     int32_t bias_len;    /* 1 (broadcast) or OC */
-    int32_t acc_dtype;   /* the attribute's acc_type: TMI_INT32 for INT8 operands, TMI_FP32 for floating point (the
-                            reference also instantiates FP16 accumulation of FP16 operands, op_factory.h:97-118, which
-                            is not built: TMI_ERROR) */
+    int32_t acc_dtype;   /* the attribute's acc_type: TMI_INT32 for INT8 operands, TMI_FP32 for floating point; 0 (a
+                            descriptor zeroed by a caller that predates the field) means that default.  The reference
+                            also instantiates FP16 accumulation of FP16 operands (op_factory.h:97-118), which is not
+                            built: TMI_ERROR */
 } tmi_conv_desc_t;
 
 /* TransposeConv2dAttribute plus operand shapes (reference_model/src/ops/tensor_ops.cpp:1982-2056).

@@ -298,8 +298,9 @@ _BITS = {np.dtype(np.int8): 8, np.dtype(np.uint8): 8, np.dtype(np.int16): 16, np
 
 
 def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale32=True,
-            rounding_mode=ROUND_DOUBLE, per_channel=True, input_unsigned=False, output_unsigned=False):
-    """RESCALE.  Returns (out, status); out has dtype out_dtype (bit pattern of the stored value)."""
+            rounding_mode=ROUND_DOUBLE, per_channel=True, input_unsigned=False, output_unsigned=False, inexact_mode=0):
+    """RESCALE.  Returns (out, status); out has dtype out_dtype (bit pattern of the stored value).
+    inexact_mode: how INEXACT_ROUND is evaluated (0 FP32; 1 precise mode; 2 / 3 precise + compliance, normal / bounds pass)."""
     inp = np.asarray(inp)
     out_dtype = np.dtype(out_dtype)
     a = RescaleAttr()
@@ -318,8 +319,10 @@ def rescale(inp, multiplier, shift, in_zp=0, out_zp=0, out_dtype=np.int8, scale3
     sh = _c(np.atleast_1d(shift), np.int32)
     out = np.zeros(inp.shape, dtype=np.int32)
     fn = lib().orc_rescale_i48 if i48 else lib().orc_rescale
+    lib().orc_set_inexact_mode(ctypes.c_int(int(inexact_mode)))
     rc = fn(ctypes.byref(a), ctypes.c_int64(rows), ctypes.c_int32(C), _ptr(stored), _ptr(mult),
             _ptr(sh), ctypes.c_int32(mult.size), ctypes.c_int32(sh.size), ctypes.c_int32(rank), _ptr(out))
+    lib().orc_set_inexact_mode(ctypes.c_int(0))
     # narrow to the output dtype keeping the low bits (uint16 32832 is stored as such)
     narrowed = out.astype(np.int64).astype(_signed(out_dtype), casting="unsafe") if out_dtype.kind != "u" else \
         (out.astype(np.int64) & ((1 << (8 * out_dtype.itemsize)) - 1)).astype(out_dtype)

@@ -617,6 +617,14 @@ static int64_t value_extend64(int64_t val, int bits, int is_unsigned)
 /* ------------------------------------------------------------------------------------------------
  * OpRescale::checkTensorAttributes + eval (type_conversion.cpp:72-154, 224-421).
  * ---------------------------------------------------------------------------------------------- */
+/* g_func_config.precise_mode / compliance_mode / bounds_mode as RESCALE's INEXACT_ROUND reads them (:318-346):
+ * 0 FP32 maths; 1 precise mode (FP64, truncated); 2 / 3 precise mode with compliance mode, normal / bounds pass. */
+static int g_inexact_mode = 0;
+void orc_set_inexact_mode(int mode)
+{
+    g_inexact_mode = mode;
+}
+
 /* in32: the int32 storage of INT8 / INT16 / INT32 tensors; in64: the int64 storage of an INT48 tensor */
 static int rescale_impl(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in32, const int64_t* in64,
                         const int32_t* multiplier, const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank,
@@ -699,6 +707,25 @@ static int rescale_impl(const orc_rescale_attr_t* a, int64_t rows, int32_t C, co
                     scaled = orc_apply_scale_32((int32_t)v, m, sh, double_round, &status);
                 else
                     scaled = orc_apply_scale_16(v, (int16_t)m, sh, &status);
+            }
+            else if (g_inexact_mode)
+            {
+                /* INEXACT_ROUND in precise mode: FP64 maths (:326-346) */
+                volatile double t = (double)v * (double)m;
+                volatile double x = t * exp2((double)(-sh));
+                if (g_inexact_mode >= 2)
+                {
+                    const double with_zp  = x + (double)out_zp_ext;
+                    const double half_ulp = exp2(-23 - 1);
+                    volatile double three = 3 * fabs(x);
+                    volatile double sum   = three + fabs(with_zp);
+                    volatile double prod  = sum * half_ulp;
+                    const double err_bnd  = 0.5 + prod;
+                    volatile double moved = g_inexact_mode == 3 ? x + err_bnd : x - err_bnd;
+                    x                     = g_inexact_mode == 3 ? floor(moved) : ceil(moved);
+                }
+                /* the cast of a value outside int32 is undefined in the reference; the convention of the FP32 branch */
+                scaled = (x > -2147483649.0 && x < 2147483648.0) ? (int32_t)x : INT32_MIN;
             }
             else
             {

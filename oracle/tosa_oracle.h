@@ -168,6 +168,10 @@ typedef struct
  * ORC_UNPREDICTABLE when a REQUIRE fires (output contents then unspecified), else ORC_VALID. */
 int orc_rescale(const orc_rescale_attr_t* a, int64_t rows, int32_t C, const int32_t* in, const int32_t* multiplier,
                 const int32_t* shift, int32_t n_mult, int32_t n_shift, int32_t rank, int32_t* out);
+/* How INEXACT_ROUND is evaluated by the calls that follow (g_func_config of the reference, type_conversion.cpp:318-346):
+ * 0 FP32 maths (the default); 1 precise mode: FP64 maths, truncated; 2 / 3 precise mode with compliance mode: the FP64
+ * value moved to the lower / upper edge of the error bound (normal / bounds pass) before the truncation. */
+void orc_set_inexact_mode(int mode);
 /* The same for an INT48 input (in_bits = 48), whose storage type is int64 (template_types.h:67-163); a stored
  * value with bit 47 set gets bits 48..63 set (value_extend64_impl, type_conversion.cpp:200-215), which changes
  * nothing for values inside the 48-bit range.  Needs scale32 = 0, hence apply_scale_16 (:122). */

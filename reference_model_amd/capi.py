@@ -36,6 +36,7 @@ EXPORTS = [
     "tmi_avg_pool2d", "tmi_max_pool2d", "tmi_pool2d_check",
     "tmi_conv2d_precise", "tmi_depthwise_conv2d_precise", "tmi_matmul_precise", "tmi_dot_product_check",
     "tmi_ctx_reserve_workspace", "tmi_transpose_conv2d_noalloc", "tmi_ctx_set_level", "tmi_clamp_fp",
+    "tmi_ctx_set_precise_mode", "tmi_ctx_workspace_bytes", "tmi_ctx_trim_workspace",
     "tmi_debug_launch_empty", "tmi_debug_tile_decode", "tmi_debug_last_launch_shape", "tmi_debug_stream",
 ]
 
@@ -140,6 +141,8 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_last_kernel.restype = ctypes.c_char_p
     lib.tmi_ctx_set_kernel_choice.argtypes = [vp, i32]
     lib.tmi_ctx_reserve_workspace.argtypes = [vp, ctypes.c_size_t]
+    lib.tmi_ctx_workspace_bytes.argtypes = [vp, ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    lib.tmi_ctx_trim_workspace.argtypes = [vp]
     lib.tmi_buf_alloc.argtypes = [vp, ctypes.c_size_t, ctypes.POINTER(vp)]
     lib.tmi_buf_free.argtypes = [vp, vp]
     lib.tmi_upload.argtypes = [vp, vp, vp, ctypes.c_size_t]
@@ -159,6 +162,7 @@ def load_library() -> ctypes.CDLL:
     lib.tmi_clamp.argtypes = [vp, i32, i64, vp, i32, i32, vp]
     lib.tmi_clamp_fp.argtypes = [vp, i32, i64, vp, ctypes.c_float, ctypes.c_float, i32, vp]
     lib.tmi_ctx_set_level.argtypes = [vp, ctypes.POINTER(Level)]
+    lib.tmi_ctx_set_precise_mode.argtypes = [vp, i32, i32, i32]
     lib.tmi_debug_launch_empty.argtypes = [vp, i32, i32, i32]
     lib.tmi_debug_last_launch_shape.argtypes = [ctypes.POINTER(ctypes.c_int32)]
     lib.tmi_debug_last_launch_shape.restype = None
@@ -329,6 +333,15 @@ class Context:
         return self._check(self.lib.tmi_transpose_conv2d_noalloc(self.handle, ctypes.byref(d), _ptr(inp), _ptr(w),
                                                                  _ptr(bias), in_zp, w_zp, _ptr(out)))
 
+    def workspace_bytes(self):
+        """(bytes of the scratch buffer in use, bytes of the outgrown blocks still held)"""
+        live, retired = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        self._check(self.lib.tmi_ctx_workspace_bytes(self.handle, ctypes.byref(live), ctypes.byref(retired)))
+        return live.value, retired.value
+
+    def trim_workspace(self) -> int:
+        return self._check(self.lib.tmi_ctx_trim_workspace(self.handle))
+
     def reserve_workspace(self, nbytes: int) -> int:
         return self._check(self.lib.tmi_ctx_reserve_workspace(self.handle, nbytes))
 
@@ -400,6 +413,10 @@ class Context:
 
     def launch_empty(self, grid, block, lds_bytes) -> int:
         return self._check(self.lib.tmi_debug_launch_empty(self.handle, grid, block, lds_bytes))
+
+    def set_precise_mode(self, precise=False, compliance=False, bounds=False):
+        """g_func_config.precise_mode / compliance_mode / bounds_mode as RESCALE's INEXACT_ROUND reads them"""
+        self._check(self.lib.tmi_ctx_set_precise_mode(self.handle, int(precise), int(compliance), int(bounds)))
 
     def set_level(self, level=LEVEL_NONE):
         lv = Level(*level)

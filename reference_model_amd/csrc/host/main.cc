@@ -202,7 +202,7 @@ int main(int argc, char** argv)
         ModelRunner runner(0);
         if (!fusion)
             runner.disableFusion();
-        runner.setPreciseMode(precise, run == 1);
+        runner.setPreciseMode(precise, run == 1, precise && desc.bounds_file_required);
         runner.setLevel(level);
         st = runner.initialize(block);
         if (st != GraphStatus::TOSA_VALID)

@@ -1171,7 +1171,10 @@ GraphStatus ModelRunner::initialize(const BasicBlock& block)
     sgt->precise_mode  = precise_mode;
     sgt->bounds_mode   = bounds_mode;
     if (sgt->ctx)
+    {
         tmi_ctx_set_level(sgt->ctx, &level);
+        tmi_ctx_set_precise_mode(sgt->ctx, precise_mode, compliance_mode, bounds_mode);
+    }
     if (sgt->initializeGraph() || sgt->linkTensorsAndNodes() || sgt->validateGraph())
         return sgt->getGraphStatus() == GraphStatus::TOSA_VALID ? GraphStatus::TOSA_ERROR : sgt->getGraphStatus();
     return sgt->getGraphStatus();

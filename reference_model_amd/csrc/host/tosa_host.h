@@ -227,13 +227,17 @@ public:
     int getOutput(const std::string& name, uint8_t* raw, size_t size);
     SubgraphTraverser* traverser() { return sgt.get(); }
     void disableFusion() { fusion = false; }
-    void setPreciseMode(bool precise, bool bounds) { precise_mode = precise, bounds_mode = bounds; }
+    // compliance: a compliance test in precise mode (main.cpp:109-115); RESCALE's INEXACT_ROUND reads it
+    void setPreciseMode(bool precise, bool bounds, bool compliance = false)
+    {
+        precise_mode = precise, bounds_mode = bounds, compliance_mode = compliance;
+    }
     // g_func_config.tosa_level (func_config.h:63-66); all zero = NONE
     void setLevel(const tmi_level_t& l) { level = l; }
 
 private:
     int device_id;
-    bool fusion = true, precise_mode = false, bounds_mode = false;
+    bool fusion = true, precise_mode = false, bounds_mode = false, compliance_mode = false;
     tmi_level_t level = { 0, 0, 0, 0, 0 };
     std::unique_ptr<SubgraphTraverser> sgt;
 };

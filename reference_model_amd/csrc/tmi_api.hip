@@ -53,10 +53,12 @@ struct tmi_ctx
     void* workspace       = nullptr;    // scratch for operand re-layout (MATMUL's transposed B)
     size_t workspace_size = 0;
     std::vector<void*> retired;         // outgrown scratch blocks: captured graphs may still name them
+    size_t retired_bytes  = 0;          // their sizes, summed
     unsigned char* static_scratch = nullptr;    // this device's copy of the library's static scratch array
     uint32_t last_flags   = 0;
     uint32_t host_flags   = 0;          // conditions found on the host since the last sync (TMI_FLAG_LEVEL)
     tmi_level_t level     = { 0, 0, 0, 0, 0 };    // all zero: no level configured (func_config_t::NONE)
+    int32_t inexact_mode  = 1;          // how INEXACT_ROUND is evaluated: RescaleParams::inexact_round
     int32_t kernel_choice = 0;
     std::string last_error;
     const char* last_kernel = "";
@@ -141,7 +143,7 @@ int after_launch(tmi_ctx* ctx, const char* kernel_name)
 // enqueued, and HIP graphs captured from earlier calls, still name it.  Growing is refused while the stream is
 // being captured (an allocation cannot be part of a graph): the caller sizes the buffer with an eager call of
 // the same operator first, or uses tmi_ctx_reserve_workspace().
-int ensure_workspace(tmi_ctx* ctx, size_t bytes)
+int ensure_workspace(tmi_ctx* ctx, size_t bytes, bool exact = false)
 {
     if (bytes <= ctx->workspace_size)
         return TMI_VALID;
@@ -149,12 +151,24 @@ int ensure_workspace(tmi_ctx* ctx, size_t bytes)
     if (hipStreamIsCapturing(ctx->stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
         return fail(ctx, "the context's scratch buffer would have to grow to %zu bytes during stream capture: "
                          "call tmi_ctx_reserve_workspace first", bytes);
+    // An operator that outgrows the block gets at least twice the old size, so the blocks kept for launches and graphs
+    // that may still name them sum to less than the live block (a request of its own size, from
+    // tmi_ctx_reserve_workspace, is taken as it is).
+    size_t want = exact || bytes >= 2 * ctx->workspace_size ? bytes : 2 * ctx->workspace_size;
     void* block = nullptr;
-    TMI_HIP(ctx, hipMalloc(&block, bytes));
+    if (hipMalloc(&block, want) != hipSuccess)
+    {
+        (void)hipGetLastError();
+        want = bytes;    // no room for the doubled block: the request itself
+        TMI_HIP(ctx, hipMalloc(&block, want));
+    }
     if (ctx->workspace)
+    {
         ctx->retired.push_back(ctx->workspace);
+        ctx->retired_bytes += ctx->workspace_size;
+    }
     ctx->workspace      = block;
-    ctx->workspace_size = bytes;
+    ctx->workspace_size = want;
     return TMI_VALID;
 }
 
@@ -198,7 +212,7 @@ int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool d
     // the accumulator type is part of the operator's type signature (op_factory.h:97-118, tensor_ops.cpp:2219-2251):
     // INT32 for INT8 operands, FP32 for floating point; FP16 accumulation of FP16 operands exists in the reference and
     // is not built here
-    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1 || d->OH < 0 ||
         d->OW < 0)
@@ -348,7 +362,7 @@ int validate_rescale(tmi_ctx* ctx, const tmi_rescale_desc_t* r, int32_t rank, in
     p.qmax          = out_u ? (i8out ? 255 : 65535) : (i8out ? 127 : (i16out ? 32767 : INT32_MAX));
     p.scale32       = r->scale32 != 0;
     p.double_round  = r->rounding_mode == TMI_ROUND_DOUBLE;
-    p.inexact_round = r->rounding_mode == TMI_ROUND_INEXACT;
+    p.inexact_round = r->rounding_mode == TMI_ROUND_INEXACT ? (uint8_t)ctx->inexact_mode : 0;
     p.per_channel   = r->per_channel != 0;
     p.in_bits       = (uint8_t)dtype_bits(r->in_dtype);
     p.in_unsigned   = in_u;
@@ -582,6 +596,14 @@ int tmi_ctx_set_level(tmi_ctx_t* ctx, const tmi_level_t* level)
     return TMI_VALID;
 }
 
+int tmi_ctx_set_precise_mode(tmi_ctx_t* ctx, int32_t precise_mode, int32_t compliance_mode, int32_t bounds_mode)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    ctx->inexact_mode = !precise_mode ? 1 : (!compliance_mode ? 2 : (bounds_mode ? 4 : 3));
+    return TMI_VALID;
+}
+
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
     if (!ctx || choice < 0 || choice > 4)
@@ -639,7 +661,31 @@ int tmi_ctx_reserve_workspace(tmi_ctx_t* ctx, size_t bytes)
     if (!ctx)
         return TMI_ERROR;
     TMI_HIP(ctx, hipSetDevice(ctx->device));
-    return ensure_workspace(ctx, bytes);
+    return ensure_workspace(ctx, bytes, true);
+}
+
+int tmi_ctx_workspace_bytes(const tmi_ctx_t* ctx, size_t* live, size_t* retired)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    if (live)
+        *live = ctx->workspace_size;
+    if (retired)
+        *retired = ctx->retired_bytes;
+    return TMI_VALID;
+}
+
+int tmi_ctx_trim_workspace(tmi_ctx_t* ctx)
+{
+    if (!ctx)
+        return TMI_ERROR;
+    TMI_HIP(ctx, hipSetDevice(ctx->device));
+    TMI_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    for (void* b : ctx->retired)
+        (void)hipFree(b);
+    ctx->retired.clear();
+    ctx->retired_bytes = 0;
+    return TMI_VALID;
 }
 
 int tmi_buf_alloc(tmi_ctx_t* ctx, size_t bytes, void** out_dev)
@@ -731,7 +777,7 @@ static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* 
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
-    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1)
         return fail(ctx, "%s: negative tensor dimension", op);
@@ -871,7 +917,7 @@ static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
-    if (d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))
+    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->ID < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KD < 1 || d->KH < 1 ||
         d->KW < 1)
@@ -1221,7 +1267,7 @@ static int validate_pool(tmi_ctx* ctx, const char* op, const tmi_pool_desc_t* d,
     const bool is_fp  = d->dtype == TMI_FP16 || d->dtype == TMI_BF16 || d->dtype == TMI_FP32;
     if (!is_int && !is_fp)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
-    if (avg && d->acc_dtype != (is_int ? TMI_INT32 : TMI_FP32))
+    if (avg && d->acc_dtype != 0 && d->acc_dtype != (is_int ? TMI_INT32 : TMI_FP32))
         return fail(ctx, "%s: accumulator type not supported for this configuration of operator", op);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->C < 0)
         return fail(ctx, "%s: negative tensor dimension", op);

@@ -63,6 +63,8 @@ struct RescaleParams
     int32_t out_zp;            // sign/zero-extended output zero point
     int32_t qmin, qmax;        // clip range of the output type
     int32_t clamp_min, clamp_max;
+    // inexact_round: 0 SINGLE / DOUBLE rounding; 1 INEXACT_ROUND in FP32; 2 in FP64 (precise mode); 3 / 4 the same moved to the
+    // lower / upper edge of the compliance error bound (normal / bounds pass)
     uint8_t scale32, double_round, inexact_round, per_channel;
     uint8_t in_bits, in_unsigned, has_clamp, enabled;
     // Set by the host when the input is a signed INT32 value with zero input_zp, scale32 is on and the
@@ -144,7 +146,7 @@ __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t
 {
     const int64_t v = value_extend(stored, p.in_bits, p.in_unsigned) - (int64_t)p.in_zp;
     int32_t scaled;
-    if (p.inexact_round)
+    if (p.inexact_round == 1)
     {
         const float t = (float)v * (float)m;
         const float u = rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
@@ -152,6 +154,20 @@ __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t
         // returns INT32_MIN for every such value (the conversion instruction's "integer indefinite"), and so does
         // this one, rather than the saturated value the device's own conversion would give.
         scaled = (u >= -2147483648.0f && u < 2147483648.0f) ? (int32_t)u : INT32_MIN;
+    }
+    else if (p.inexact_round)
+    {
+        // INEXACT_ROUND in precise mode (type_conversion.cpp:326-346): the scaled value in FP64, truncated; in compliance
+        // mode it is first moved to the edge of the error bound that the specification grants an FP32 implementation,
+        // the lower edge in the normal pass (3) and the upper edge in the bounds pass (4).
+        double x = (double)v * (double)m * ldexp(1.0, -s);
+        if (p.inexact_round >= 3)
+        {
+            const double with_zp = x + (double)p.out_zp;
+            const double bound   = 0.5 + (3.0 * fabs(x) + fabs(with_zp)) * ldexp(1.0, -24);
+            x                    = p.inexact_round == 4 ? floor(x + bound) : ceil(x - bound);
+        }
+        scaled = (x > -2147483649.0 && x < 2147483648.0) ? (int32_t)x : INT32_MIN;    // the same convention as above
     }
     else if (p.scale32)
         scaled = apply_scale_32((int32_t)v, m, s, p.double_round, flags);

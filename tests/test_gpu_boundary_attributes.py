@@ -104,6 +104,13 @@ def test_accumulator_types_that_are_not_built_are_refused(ctx):
     with pytest.raises(TmiError, match="accumulator"):
         ctx.conv2d(bad_i, ctx.upload(xi), ctx.upload(wi), ctx.upload(bi), 0, 0, ctx.empty((1, 4, 4, 8), capi.INT32))
 
+    # a descriptor zeroed by a caller that predates the field: 0 stands for the operand type's accumulator
+    zeroed = ctx.conv_desc(capi.INT8, capi.INT32, xi.shape, 8, 3, 3, (4, 4), (0, 0, 0, 0), (1, 1), (1, 1), 8, acc_dtype=0)
+    assert zeroed.acc_dtype == 0
+    oi = ctx.empty((1, 4, 4, 8), capi.INT32)
+    ctx.conv2d(zeroed, ctx.upload(xi), ctx.upload(wi), ctx.upload(bi), 0, 0, oi)
+    assert ctx.sync() == capi.VALID and np.array_equal(oi.numpy(), oracle.conv2d("i8", xi, wi, bi))
+
     td = capi.TconvDesc()
     td.in_dtype, td.out_dtype = capi.INT8, capi.INT32
     assert td.acc_dtype == capi.INT32
@@ -207,3 +214,32 @@ def test_floating_point_clamp_refuses_a_nan_or_inverted_range(ctx):
     with pytest.raises(TmiError):
         ctx.clamp_fp(capi.INT8, 4, x, 0.0, 1.0, 1, out)
     ctx.clamp_fp(capi.FP32, 0, None, 0.0, 1.0, 1, None)               # an empty tensor is a no-op
+
+
+@pytest.mark.parametrize("mode", [(False, False, False), (True, False, False), (True, True, False), (True, True, True)],
+                         ids=["fp32", "precise", "compliance", "compliance-bounds"])
+@pytest.mark.parametrize("in_dtype,out_dtype,out_zp", [(np.int8, np.int8, -100), (np.int32, np.int16, 0), (np.int16, np.int32, 0)])
+def test_inexact_round_in_precise_mode_matches_the_oracle(ctx, mode, in_dtype, out_dtype, out_zp):
+    """INEXACT_ROUND as the reference evaluates it in precise mode (type_conversion.cpp:326-346): FP64 maths truncated,
+    and under compliance mode the lower (normal pass) or upper (bounds pass) edge of the error bound"""
+    precise, compliance, bounds = mode
+    oracle_mode = 0 if not precise else (1 if not compliance else (3 if bounds else 2))
+    rng = np.random.default_rng(oracle_mode + 10 * np.dtype(in_dtype).itemsize)
+    info = np.iinfo(in_dtype)
+    x = rng.integers(max(info.min, -(1 << 24)), min(info.max, 1 << 24), (37, 24)).astype(in_dtype)
+    # scales that leave most results inside the output range, so that the rounding is what decides them
+    mult = rng.integers(1 << 29 if in_dtype == np.int8 else 1 << 20, 1 << 31, 24).astype(np.int32)
+    shift = (rng.integers(30, 34, 24) if in_dtype == np.int8 else rng.integers(28 if in_dtype == np.int32 else 20, 45, 24)).astype(np.int8)
+    mult[0], shift[0] = 1 << 30, 31    # halves: the ties are where the edges of the compliance bound leave rint()
+    in_zp = 5 if in_dtype == np.int8 else 0
+    kw = dict(in_zp=in_zp, out_zp=out_zp, out_dtype=out_dtype, rounding_mode=capi.ROUND_INEXACT)
+    want, wst = oracle.rescale(x, mult, shift, inexact_mode=oracle_mode, **kw)
+    ctx.set_precise_mode(precise, compliance, bounds)
+    try:
+        got, st = gpu_ops.rescale(ctx, x, mult, shift, **kw)
+    finally:
+        ctx.set_precise_mode()
+    assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    if precise and (not compliance or in_dtype == np.int8):    # differs from FP32 maths, or the setting did not arrive
+        plain, _ = oracle.rescale(x, mult, shift, **kw)
+        assert not np.array_equal(plain, want)

@@ -282,7 +282,22 @@ def test_benchmark_fp16_conv_and_bf16_matmul_errors_at_full_size(ctx):
         ksb = dp.kernel_size_bound(kh * kw * ic, "fp16")
         r = ctx.dot_product_check(capi.FP16, int(np.prod(shape)), imp, ref, bnd, ksb)
         assert ctx.sync() == capi.VALID and r.compliant
-        st = dp.check(imp.numpy(), ref.numpy(), bnd.numpy(), "fp16", ksb)
+        ref_h, bnd_h = ref.numpy(), bnd.numpy()
+        # one whole image of the fp64 reference and of the bound against the oracle's own loop nest (its OpenMP build:
+        # the same C source on all host cores), element for element: the reference the check above divides by is the
+        # oracle's, not only the library's
+        img = 11
+        x64, w64, b64 = (c[k].astype(np.float64) for k in ("x", "w", "bias"))
+        oracle.set_parallel(True)
+        try:
+            ref_o = oracle.conv2d("f64", x64[img:img + 1], w64, b64, c["pad"], c["stride"], c["dilation"])
+            bnd_o = oracle.conv2d("f64", x64[img:img + 1], w64, b64, c["pad"], c["stride"], c["dilation"], abs_mode=True)
+        finally:
+            oracle.set_parallel(False)
+        assert np.array_equal(ref_h[img:img + 1], ref_o) and np.array_equal(bnd_h[img:img + 1], bnd_o)
+        one = dp.check(imp.numpy()[img:img + 1], ref_o, bnd_o, "fp16", ksb)
+        assert one["ok"], one
+        st = dp.check(imp.numpy(), ref_h, bnd_h, "fp16", ksb)
         print("fp16 CONV2D [16,28,28,256]x[256,3,3,256]:", st)
         assert st["ok"] and st["max_ulp"] <= 32 and st["max_ulp_conditioned"] <= 1.0
         assert st["max_rel_to_bound"] <= 2.0 ** -12          # half an fp16 ULP of the sum of absolute products

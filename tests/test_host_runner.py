@@ -329,6 +329,35 @@ def test_int48_rescale_graph(tmp_path):
 
 
 @pytest.mark.gpu
+def test_inexact_round_rescale_in_precise_and_compliance_mode(tmp_path):
+    """--precise_mode=1 reaches an INEXACT_ROUND RESCALE (type_conversion.cpp:326-346): FP64 maths truncated; on a
+    compliance descriptor the normal pass writes the lower edge of the error bound and the bounds pass the upper one"""
+    rng = np.random.default_rng(11)
+    x = rng.integers(-128, 128, (4, 9, 16)).astype(np.int8)
+    mult = rng.integers(1 << 24, 1 << 30, 16).astype(np.int32)
+    shift = rng.integers(26, 31, 16).astype(np.int8)
+    mult[0], shift[0] = 1 << 30, 31    # halves: on ties the two edges of the compliance bound differ
+    kw = dict(in_zp=2, out_zp=-9, out_dtype=np.int8, rounding_mode=oracle.ROUND_INEXACT)
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("mult", [16], np.int32, mult), W.tensor("shift", [16], np.int8, shift),
+          W.tensor("izp", [1], np.int8, [2]), W.tensor("ozp", [1], np.int8, [-9]), W.tensor("y", x.shape, np.int8)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("mult", "shift", "izp", "ozp")]
+    ops.append(W.operator(R.OP_RESCALE, ["x", "mult", "shift", "izp", "ozp"], ["y"], W.rescale_attr(rounding_mode=2)))
+    desc = _write_case(tmp_path, W.graph(ts, ops, ["x"], ["y"]), {"x": x}, ["y"])
+    want = {m: oracle.rescale(x, mult, shift, inexact_mode=m, **kw)[0] for m in (0, 1, 2, 3)}
+    assert not np.array_equal(want[0], want[1]) and not np.array_equal(want[2], want[3])
+    r = _run(desc)
+    assert r.returncode == 0 and np.array_equal(np.load(tmp_path / "y_out.npy"), want[0])
+    r = _run(desc, "--precise_mode=1")
+    assert r.returncode == 0 and np.array_equal(np.load(tmp_path / "y_out.npy"), want[1])
+    meta = dict(json.loads(open(desc).read()), test_requirements={"bounds_file_required": True})
+    open(desc, "w").write(json.dumps(meta))
+    r = _run(desc, "--precise_mode=1")
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(tmp_path / "y_out.npy"), want[2])
+    assert np.array_equal(np.load(tmp_path / "bounds_y_out.npy"), want[3])
+
+
+@pytest.mark.gpu
 def test_precise_mode_writes_fp64_results_and_bounds(tmp_path):
     """--precise_mode=1 on a compliance-style descriptor (test_requirements.bounds_file_required): the fp16 CONV2D is
     evaluated in fp64, then once more over absolute values into bounds_<ofm_file> (reference: main.cpp:109-121,

@@ -1,11 +1,13 @@
 """tmi_transpose_conv2d_noalloc: the entry point that allocates nothing (its re-laid-out operands live in the
 library's static device array) against tmi_transpose_conv2d on the same operands, bit for bit, on two calls in a
-row, the second with a smaller input; and its refusal of operands beyond the array's size."""
+row, the second with a smaller input, and (integers) against the CPU oracle; that it leaves the context's scratch
+buffer unallocated; and its refusal of operands beyond the array's size."""
 from __future__ import annotations
 
 import numpy as np
 import pytest
 
+import oracle
 from reference_model_amd import Context, capi
 
 pytestmark = pytest.mark.gpu
@@ -38,16 +40,20 @@ def _operands(rng, shape, oc, k, fp):
 
 
 def _run_both(ctx, x, w, b, dt, in_zp, w_zp, out_pad, stride):
+    """the entry point that allocates nothing first, on a context whose scratch buffer must stay unallocated; then the
+    ordinary entry point, which allocates one"""
     d = _desc(x, w, b, out_pad, stride, dt)
     tx, tw, tb = ctx.upload(x, dt), ctx.upload(w, dt), ctx.upload(b)
     np_out = np.int32 if dt == capi.INT8 else np.float16
     shape = (d.N, d.OH, d.OW, d.OC)
     want_t, got_t = ctx.empty(shape, d.out_dtype, np_out), ctx.empty(shape, d.out_dtype, np_out)
-    ctx.transpose_conv2d(d, tx, tw, tb, in_zp, w_zp, want_t)
-    want_kernel = ctx.last_kernel
-    assert ctx.sync() == capi.VALID
+    before = ctx.workspace_bytes()
     ctx.transpose_conv2d_noalloc(d, tx, tw, tb, in_zp, w_zp, got_t)
-    assert ctx.last_kernel == want_kernel
+    noalloc_kernel = ctx.last_kernel
+    assert ctx.sync() == capi.VALID
+    assert ctx.workspace_bytes() == before, "the entry point that allocates nothing grew the context's scratch buffer"
+    ctx.transpose_conv2d(d, tx, tw, tb, in_zp, w_zp, want_t)
+    assert ctx.last_kernel == noalloc_kernel
     assert ctx.sync() == capi.VALID
     want, got = want_t.numpy(), got_t.numpy()
     for t in (tx, tw, tb, want_t, got_t):
@@ -63,13 +69,21 @@ def test_noalloc_matches_transpose_conv2d_twice(fp):
     rng = np.random.default_rng(20260 + fp)
     ctx = Context(0)
     try:
-        for shape, oc, out_pad, stride in (((2, 13, 11, 48), 40, (0, 1, 1, 0), (2, 2)),
-                                           ((1, 5, 7, 48), 24, (1, 0, 0, 0), (2, 3))):
+        assert ctx.workspace_bytes() == (0, 0)
+        # the third layer has unit stride: no holes, only the flipped weights go through the static array
+        for i, (shape, oc, out_pad, stride) in enumerate((((2, 13, 11, 48), 40, (0, 1, 1, 0), (2, 2)),
+                                                          ((1, 5, 7, 48), 24, (1, 0, 0, 0), (2, 3)),
+                                                          ((2, 9, 8, 48), 32, (0, 0, 1, 1), (1, 1)))):
             x, w, b, dt, in_zp, w_zp = _operands(rng, shape, oc, 3, fp)
             want, got = _run_both(ctx, x, w, b, dt, in_zp, w_zp, out_pad, stride)
             assert want.shape == got.shape and want.size > 0
             assert np.array_equal(want.view(np.uint8), got.view(np.uint8)), (
                 f"{shape}: {int(np.count_nonzero(want != got))} of {want.size} elements differ")
+            if not fp:
+                ref = oracle.transpose_conv2d("i8", x, w, b, out_pad, stride, in_zp, w_zp)
+                assert np.array_equal(got, ref), f"{shape}: differs from the oracle"
+            if i == 0:
+                assert ctx.workspace_bytes()[0] > 0    # the ordinary entry point did allocate
     finally:
         ctx.close()
 
