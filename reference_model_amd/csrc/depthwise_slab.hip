@@ -283,8 +283,6 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                 // one shift for all 64 channels: the high-word form with its constants in scalar registers
                 const int64_t rnd = (int64_t(1) << (s_uni - 1)) + (a.rp.double_round ? (int64_t(1) << 30) : 0) +
                                     ((int64_t)a.rp.out_zp << s_uni);
-                const int32_t hi_p  = (int32_t)(rnd >> 32);
-                const uint32_t lo_p = (uint32_t)rnd;
                 const int sh        = s_uni - 32;
                 int32_t cm[16];
 #pragma unroll
@@ -297,13 +295,13 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                 {
 #pragma unroll
                     for (int e = 0; e < 16; e++)
-                        r[e] = clamp_med3(high_word_rescale<true>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+                        r[e] = clamp_med3(high_word_rescale64<true>(acc[e], cm[e], rnd, sh), a.rp.lo, a.rp.hi);
                 }
                 else
                 {
 #pragma unroll
                     for (int e = 0; e < 16; e++)
-                        r[e] = clamp_med3(high_word_rescale<false>(acc[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
+                        r[e] = clamp_med3(high_word_rescale64<false>(acc[e], cm[e], rnd, sh), a.rp.lo, a.rp.hi);
                 }
             }
             else if (s_uni == -2)
@@ -314,7 +312,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                     for (int e = 0; e < 16; e++)
                     {
                         const HighWordScale c = tab_hw[clc + e];
-                        r[e] = clamp_med3(high_word_rescale<true>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                        r[e] = clamp_med3(high_word_rescale64<true>(acc[e], c), a.rp.lo, a.rp.hi);
                     }
                 }
                 else
@@ -323,7 +321,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                     for (int e = 0; e < 16; e++)
                     {
                         const HighWordScale c = tab_hw[clc + e];
-                        r[e] = clamp_med3(high_word_rescale<false>(acc[e], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
+                        r[e] = clamp_med3(high_word_rescale64<false>(acc[e], c), a.rp.lo, a.rp.hi);
                     }
                 }
             }

@@ -15,7 +15,8 @@ struct alignas(sizeof(T) * N) Pack
     T v[N];
 };
 
-template <typename InT, typename OutT, int VEC>
+// PRECISE: the FP64 forms of INEXACT_ROUND (precise mode), which the other instantiation does not hold.
+template <typename InT, typename OutT, int VEC, bool PRECISE>
 __global__ __launch_bounds__(256) void rescale_vec_kernel(RescaleParams p, const InT* __restrict__ in,
                                                           OutT* __restrict__ out, int64_t n_vec, int32_t C,
                                                           uint32_t* flag_word)
@@ -33,14 +34,14 @@ __global__ __launch_bounds__(256) void rescale_vec_kernel(RescaleParams p, const
         {
             const int32_t m = load_multiplier(p, c0 + j);
             const int32_t s = load_shift(p, c0 + j);
-            r.v[j]          = (OutT)rescale_value(p, a.v[j], m, s, flags);
+            r.v[j]          = (OutT)rescale_value<PRECISE>(p, a.v[j], m, s, flags);
         }
         reinterpret_cast<Pack<OutT, VEC>*>(out)[i] = r;
     }
     raise_flags(flag_word, flags);
 }
 
-template <typename InT, typename OutT>
+template <typename InT, typename OutT, bool PRECISE>
 __global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, const InT* __restrict__ in,
                                                              OutT* __restrict__ out, int64_t n, int32_t C,
                                                              uint32_t* flag_word)
@@ -52,7 +53,7 @@ __global__ __launch_bounds__(256) void rescale_scalar_kernel(RescaleParams p, co
         const int c     = (int)(i % C);
         const int32_t m = load_multiplier(p, c);
         const int32_t s = load_shift(p, c);
-        out[i]          = (OutT)rescale_value(p, in[i], m, s, flags);
+        out[i]          = (OutT)rescale_value<PRECISE>(p, in[i], m, s, flags);
     }
     raise_flags(flag_word, flags);
 }
@@ -233,15 +234,26 @@ static const char* launch_rescale_t(hipStream_t st, const RescaleParams& p, cons
     const bool aligned = ((uintptr_t)in % (sizeof(InT) * VEC) == 0) && ((uintptr_t)out % (sizeof(OutT) * VEC) == 0);
     if (n == 0)
         return "rescale_empty";
+    const bool precise = p.inexact_round >= 2;
     if (aligned && C % VEC == 0)
     {
         const int64_t n_vec = n / VEC;
-        hipLaunchKernelGGL((rescale_vec_kernel<InT, OutT, VEC>), dim3(grid_for(n_vec)), dim3(256), 0, st, p,
-                           (const InT*)in, (OutT*)out, n_vec, C, flag_word);
-        return "rescale_vec";
+        if (precise)
+            hipLaunchKernelGGL((rescale_vec_kernel<InT, OutT, VEC, true>), dim3(grid_for(n_vec)), dim3(256), 0, st, p,
+                               (const InT*)in, (OutT*)out, n_vec, C, flag_word);
+        else
+            hipLaunchKernelGGL((rescale_vec_kernel<InT, OutT, VEC, false>), dim3(grid_for(n_vec)), dim3(256), 0, st, p,
+                               (const InT*)in, (OutT*)out, n_vec, C, flag_word);
+        return precise ? "rescale_vec_precise" : "rescale_vec";
     }
-    hipLaunchKernelGGL((rescale_scalar_kernel<InT, OutT>), dim3(grid_for(n)), dim3(256), 0, st, p, (const InT*)in,
-                       (OutT*)out, n, C, flag_word);
+    if (precise)
+        hipLaunchKernelGGL((rescale_scalar_kernel<InT, OutT, true>), dim3(grid_for(n)), dim3(256), 0, st, p,
+                           (const InT*)in, (OutT*)out, n, C, flag_word);
+    else
+        hipLaunchKernelGGL((rescale_scalar_kernel<InT, OutT, false>), dim3(grid_for(n)), dim3(256), 0, st, p,
+                           (const InT*)in, (OutT*)out, n, C, flag_word);
+    if (precise)
+        return "rescale_scalar_precise";
     return "rescale_scalar";
 }
 

@@ -1028,6 +1028,31 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev, false);
 }
 
+// The fused operators under INEXACT_ROUND in precise mode: the convolution's INT32 results go to the scratch buffer and
+// the stand-alone RESCALE kernel, the only one that holds the FP64 forms, converts them.  (The convolution kernels keep
+// their epilogues free of FP64 code; precise mode is the reference's checking mode, not a path to be fast on.)
+static int run_conv_then_rescale(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in,
+                                 const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                                 int32_t out_dtype, void* out)
+{
+    ConvGeom g;
+    int rc = validate_conv(ctx, op, d, depthwise, in_zp, w_zp, g);
+    if (rc != TMI_VALID)
+        return rc;
+    const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
+    if (total > 0 && !out)
+        return fail(ctx, "%s: null tensor pointer", op);
+    rc = ensure_workspace(ctx, (size_t)(total > 0 ? total : 1) * sizeof(int32_t));
+    if (rc != TMI_VALID)
+        return rc;
+    RescaleParams none{};
+    rc = run_conv(ctx, op, depthwise, d, in, w, bias, in_zp, w_zp, none, TMI_INT32, ctx->workspace);
+    if (rc != TMI_VALID || total == 0)
+        return rc;
+    const char* name = launch_rescale(ctx->stream, rp, TMI_INT32, out_dtype, ctx->workspace, out, total, g.OC, ctx->flags_dev);
+    return after_launch(ctx, name);
+}
+
 int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev)
 {
@@ -1052,6 +1077,9 @@ int tmi_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const voi
                                     clamp_min, clamp_max, rp);
     if (rc != TMI_VALID)
         return rc;
+    if (rp.inexact_round >= 2)
+        return run_conv_then_rescale(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp,
+                                     r->out_dtype, out_dev);
     return run_conv(ctx, "OpConv2d", false, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp, r->out_dtype, out_dev);
 }
 
@@ -1070,6 +1098,9 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
                                     clamp_min, clamp_max, rp);
     if (rc != TMI_VALID)
         return rc;
+    if (rp.inexact_round >= 2)
+        return run_conv_then_rescale(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp,
+                                     r->out_dtype, out_dev);
     return run_conv(ctx, "OpDepthwiseConv2d", true, d, in_dev, weight_dev, bias_dev, in_zp, w_zp, rp, r->out_dtype,
                     out_dev);
 }

@@ -141,21 +141,17 @@ __device__ __forceinline__ int32_t apply_scale_16(int64_t value, int32_t multipl
 
 // The rescale_func lambda of OpRescale::eval (type_conversion.cpp:305-370) followed by the optional
 // CLAMP (arith_util.h:389-413).  `stored` is the raw stored input value, `m`/`s` the channel's constants.
+//
+// PRECISE chooses which INEXACT_ROUND forms the instantiation holds: false, the integer roundings and FP32 (inexact_round
+// 0 and 1); true, only the FP64 forms of precise mode (2, 3, 4).  A kernel is built for one or the other and the host
+// picks it by RescaleParams::inexact_round, so that the integer kernels carry no FP64 code.
+template <bool PRECISE = false>
 __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t stored, int32_t m, int32_t s,
                                                  uint32_t& flags)
 {
     const int64_t v = value_extend(stored, p.in_bits, p.in_unsigned) - (int64_t)p.in_zp;
     int32_t scaled;
-    if (p.inexact_round == 1)
-    {
-        const float t = (float)v * (float)m;
-        const float u = rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
-        // Outside the int32 range the reference's cast (type_conversion.cpp:323) is undefined; an x86-64 build of it
-        // returns INT32_MIN for every such value (the conversion instruction's "integer indefinite"), and so does
-        // this one, rather than the saturated value the device's own conversion would give.
-        scaled = (u >= -2147483648.0f && u < 2147483648.0f) ? (int32_t)u : INT32_MIN;
-    }
-    else if (p.inexact_round)
+    if constexpr (PRECISE)
     {
         // INEXACT_ROUND in precise mode (type_conversion.cpp:326-346): the scaled value in FP64, truncated; in compliance
         // mode it is first moved to the edge of the error bound that the specification grants an FP32 implementation,
@@ -167,7 +163,17 @@ __device__ __forceinline__ int32_t rescale_value(const RescaleParams& p, int64_t
             const double bound   = 0.5 + (3.0 * fabs(x) + fabs(with_zp)) * ldexp(1.0, -24);
             x                    = p.inexact_round == 4 ? floor(x + bound) : ceil(x - bound);
         }
-        scaled = (x > -2147483649.0 && x < 2147483648.0) ? (int32_t)x : INT32_MIN;    // the same convention as above
+        // outside int32: the same convention as for the FP32 form below
+        scaled = (x > -2147483649.0 && x < 2147483648.0) ? (int32_t)x : INT32_MIN;
+    }
+    else if (p.inexact_round)
+    {
+        const float t = (float)v * (float)m;
+        const float u = rintf(t * ldexpf(1.0f, -s));    // 2^-s is exact
+        // Outside the int32 range the reference's cast (type_conversion.cpp:323) is undefined; an x86-64 build of it
+        // returns INT32_MIN for every such value (the conversion instruction's "integer indefinite"), and so does
+        // this one, rather than the saturated value the device's own conversion would give.
+        scaled = (u >= -2147483648.0f && u < 2147483648.0f) ? (int32_t)u : INT32_MIN;
     }
     else if (p.scale32)
         scaled = apply_scale_32((int32_t)v, m, s, p.double_round, flags);
@@ -222,18 +228,18 @@ __device__ __forceinline__ int zp_fold_max_shift(int32_t out_zp)
 // test of apply_scale_32 cannot fire.  rnd(v) = R for v >= 0 and R - 2^31 for v < 0 when double rounding, with
 // R = 2^(s-1) + 2^30 + output_zp * 2^s: the low word of R is 2^30, so the low word of rnd(v) is R.lo | (sign << 31)
 // and its high word R.hi + (v >> 31).  Without double rounding rnd(v) = R = 2^(s-1) + output_zp * 2^s.
-struct HighWordScale
+struct alignas(16) HighWordScale
 {
-    int32_t m;      // multiplier
-    int32_t hi;     // R >> 32
-    int32_t sh;     // s - 32
     uint32_t lo;    // low word of R
+    int32_t hi;     // R >> 32: next to the low word, the two are the 64-bit addend of the multiply-add
+    int32_t m;      // multiplier
+    int32_t sh;     // s - 32
 };
 
 __device__ __forceinline__ HighWordScale make_high_word_scale(const ChannelScale& c, int32_t out_zp)
 {
     const int64_t r = c.rnd_pos + ((int64_t)out_zp << c.s);
-    return HighWordScale{ c.m, (int32_t)(r >> 32), c.s - 32, (uint32_t)r };
+    return HighWordScale{ (uint32_t)r, (int32_t)(r >> 32), c.m, c.s - 32 };
 }
 
 template <bool DOUBLE_ROUND>
@@ -247,6 +253,29 @@ __device__ __forceinline__ int32_t high_word_rescale(int32_t v, int32_t m, int32
     }
     const int64_t pr = (int64_t)v * (int64_t)m + (int64_t)(((uint64_t)(uint32_t)hi << 32) | lo);
     return (int32_t)(pr >> 32) >> sh;
+}
+
+// The same with the rounding term as one 64-bit value R (a scalar, or the lo / hi pair of a HighWordScale): v * m + R is
+// one multiply-add, and with double rounding a second one takes the 2^31 off again for a negative value,
+// (v >>> 31) * -2^31 + (v * m + R), instead of the three instructions that patch the sign into the two words of R.
+// (64-bit multiply-adds issue at the full rate on gfx950.)
+template <bool DOUBLE_ROUND>
+__device__ __forceinline__ int32_t high_word_rescale64(int32_t v, int32_t m, int64_t rnd, int32_t sh)
+{
+    int64_t pr = (int64_t)v * (int64_t)m + rnd;
+    if (DOUBLE_ROUND)
+    {
+        const int32_t neg = (int32_t)((uint32_t)v >> 31);
+        uint64_t carry;
+        asm("v_mad_i64_i32 %0, %1, %2, %3, %4" : "=v"(pr), "=s"(carry) : "v"(neg), "v"(INT32_MIN), "v"(pr));
+    }
+    return (int32_t)(pr >> 32) >> sh;
+}
+
+template <bool DOUBLE_ROUND>
+__device__ __forceinline__ int32_t high_word_rescale64(int32_t v, const HighWordScale& c)
+{
+    return high_word_rescale64<DOUBLE_ROUND>(v, c.m, (int64_t)(((uint64_t)(uint32_t)c.hi << 32) | c.lo), c.sh);
 }
 
 // The same for a rounding term that does not depend on the value's sign (single rounding, or double rounding where a

@@ -243,3 +243,34 @@ def test_inexact_round_in_precise_mode_matches_the_oracle(ctx, mode, in_dtype, o
     if precise and (not compliance or in_dtype == np.int8):    # differs from FP32 maths, or the setting did not arrive
         plain, _ = oracle.rescale(x, mult, shift, **kw)
         assert not np.array_equal(plain, want)
+
+
+@pytest.mark.parametrize("depthwise", [False, True])
+@pytest.mark.parametrize("mode", [(True, False, False), (True, True, True)])
+def test_fused_rescale_with_inexact_round_in_precise_mode(ctx, depthwise, mode):
+    """the fused entry points under precise mode: the convolution's INT32 results are converted by the stand-alone
+    RESCALE kernel in FP64 (type_conversion.cpp:326-346), as the reference's two operators in a row would"""
+    precise, compliance, bounds = mode
+    oracle_mode = 1 if not compliance else (3 if bounds else 2)
+    rng = np.random.default_rng(91 + oracle_mode + depthwise)
+    c = 16
+    x = rng.integers(-128, 128, (2, 9, 11, c), dtype=np.int8)
+    w = rng.integers(-128, 128, (3, 3, c, 1) if depthwise else (24, 3, 3, c), dtype=np.int8)
+    oc = c if depthwise else 24
+    bias = rng.integers(-2000, 2000, oc).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    shift = rng.integers(38 if depthwise else 42, 46, oc).astype(np.int8)
+    kw = dict(pad=(1, 1, 1, 1), in_zp=-3, w_zp=0)
+    acc = (oracle.depthwise_conv2d if depthwise else oracle.conv2d)("i8", x, w, bias, **kw)
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=4, out_dtype=np.int8, rounding_mode=capi.ROUND_INEXACT,
+                               inexact_mode=oracle_mode)
+    ctx.set_precise_mode(precise, compliance, bounds)
+    try:
+        got, st = gpu_ops.conv2d(ctx, x, w, bias, depthwise=depthwise, **kw,
+                                 rescale=dict(mult=mult, shift=shift, out_zp=4, rounding_mode=capi.ROUND_INEXACT))
+    finally:
+        ctx.set_precise_mode()
+    assert ctx.last_kernel in ("rescale_vec_precise", "rescale_scalar_precise")
+    assert wst == st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(want)) > 20    # not clipped away
+
