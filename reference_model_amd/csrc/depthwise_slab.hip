@@ -415,7 +415,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
         best_th = last.th, best_tw = last.tw, best_nw = last.nw;
     else
     {
-        int64_t best_cost = 0, best_busy = 0;
+        int64_t best_cost = 0, best_busy = 0, best_moved = 0;
         for (int th = 1; th <= g.OH && th <= 128; th++)
             for (int tw = 1; tw <= g.OW && th * tw <= 128; tw++)
             {
@@ -436,12 +436,15 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
                     const int64_t loads = (slots / 64 + nw) / nw, turns = (units + nw - 1) / nw;
                     // per workgroup: a fixed part, the loads a wave issues, the units a wave works through
                     const int64_t cost = rounds * (60 + 5 * loads + 30 * turns);
-                    // equal cost: the shape that keeps more of the 256 CUs busy, then the larger tile (measured on the
-                    // MobileNet layer: 7x15 tiles on 256 CUs 5.47 us, 8x14 tiles on 224 CUs 5.70 us)
-                    const int64_t busy = tiles < 256 ? tiles : 256;
+                    // equal cost: the shape that keeps more of the 256 CUs busy, then the one that moves the fewest
+                    // chunks into LDS over the whole layer, then the larger tile (measured on the MobileNet layer, us:
+                    // 7x15 and 14x7 tiles on 256 CUs 5.06 and 5.01, 7x17 5.23, 8x14 tiles on 224 CUs 5.16)
+                    const int64_t busy = tiles < 256 ? tiles : 256, moved = tiles * slots;
                     if (!best_th || cost < best_cost ||
-                        (cost == best_cost && (busy > best_busy || (busy == best_busy && th * tw > best_th * best_tw))))
-                        best_th = th, best_tw = tw, best_nw = nw, best_cost = cost, best_busy = busy;
+                        (cost == best_cost &&
+                         (busy > best_busy ||
+                          (busy == best_busy && (moved < best_moved || (moved == best_moved && th * tw > best_th * best_tw))))))
+                        best_th = th, best_tw = tw, best_nw = nw, best_cost = cost, best_busy = busy, best_moved = moved;
                 }
             }
         memcpy(last.key, key, sizeof(key));

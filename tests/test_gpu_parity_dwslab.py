@@ -48,7 +48,7 @@ def test_depthwise_mfma_int32_bit_exact(ctx, shape, in_zp):
     n, ih, iw, c, pad, stride, dil = shape
     x, w, bias = _operands(shape, ih * iw + c)
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True)
-    assert st == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8"
+    assert st == capi.VALID and ctx.last_kernel in ("depthwise_mfma_i8", "depthwise_mfma_pipe_i8")
     assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0))
 
 
@@ -65,7 +65,7 @@ def test_depthwise_mfma_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
     clamp = (-100, 110) if out_dtype == np.int8 else None
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=0, depthwise=True,
                              rescale=dict(mult=mult, shift=shift, out_zp=out_zp, out_dtype=out_dtype), clamp=clamp)
-    assert ctx.last_kernel == "depthwise_mfma_i8_rescale"
+    assert ctx.last_kernel in ("depthwise_mfma_i8_rescale", "depthwise_mfma_pipe_i8_rescale")
     acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, in_zp=zps[0], w_zp=0)
     want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp, out_dtype=out_dtype)
     if clamp is not None:
@@ -79,7 +79,7 @@ def test_depthwise_mfma_config4_full_size(ctx):
     c = cases.c4()
     got, st = gpu_ops.conv2d(ctx, c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"], c["in_zp"], c["w_zp"],
                              depthwise=True, rescale=dict(mult=c["mult"], shift=c["shift"], out_zp=c["out_zp"]))
-    assert ctx.last_kernel == "depthwise_mfma_i8_rescale" and st == capi.VALID
+    assert ctx.last_kernel in ("depthwise_mfma_i8_rescale", "depthwise_mfma_pipe_i8_rescale") and st == capi.VALID
     acc = oracle.depthwise_conv2d("i8", c["x"], c["w"], c["bias"], c["pad"], c["stride"], c["dilation"],
                                   in_zp=c["in_zp"], w_zp=c["w_zp"])
     want, wst = oracle.rescale(acc, c["mult"], c["shift"], out_zp=c["out_zp"])
@@ -100,7 +100,7 @@ def test_depthwise_mfma_one_shift_for_all_channels_and_single_rounding(ctx):
             assert st == wst == capi.VALID and np.array_equal(got, want)
     # bias of length 1 (tensor_ops.cpp:1191-1197)
     got, st = gpu_ops.conv2d(ctx, x, w, np.array([777], np.int32), shape[4], in_zp=5, w_zp=0, depthwise=True)
-    assert st == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8"
+    assert st == capi.VALID and ctx.last_kernel in ("depthwise_mfma_i8", "depthwise_mfma_pipe_i8")
     assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, np.array([777], np.int32), shape[4], in_zp=5, w_zp=0))
 
 
@@ -141,7 +141,7 @@ def test_automatic_choice_takes_the_matrix_core_kernel_for_its_layers():
         shape = (2, 28, 28, 96, (0, 1, 0, 1), (2, 2), (1, 1))
         x, w, bias = _operands(shape, 3)
         got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=4, depthwise=True)
-        assert st == capi.VALID and c.last_kernel == "depthwise_mfma_i8"
+        assert st == capi.VALID and c.last_kernel in ("depthwise_mfma_i8", "depthwise_mfma_pipe_i8")
         c.set_kernel_choice(capi.KERNEL_MFMA)
         other, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=4, depthwise=True)
         assert st == capi.VALID and c.last_kernel == "depthwise_dot4_i8" and np.array_equal(got, other)
@@ -178,7 +178,7 @@ def test_depthwise_mfma_epilogue_form_borders(ctx, name, shifts, mode, out_dtype
     mult[:4] = [(1 << 31) - 1, 1 << 30, 0, 1]
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, in_zp=-3, w_zp=0, depthwise=True,
                              rescale=dict(mult=mult, shift=shift, out_zp=out_zp, out_dtype=out_dtype, rounding_mode=mode))
-    assert ctx.last_kernel == "depthwise_mfma_i8_rescale"
+    assert ctx.last_kernel in ("depthwise_mfma_i8_rescale", "depthwise_mfma_pipe_i8_rescale")
     acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, in_zp=-3, w_zp=0)
     want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp, out_dtype=out_dtype, rounding_mode=mode)
     assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))

@@ -69,7 +69,7 @@ def test_depthwise_mfma_random_geometry(ctx, seed):
     bias = rng.integers(-(1 << 16), 1 << 16, c).astype(np.int32)
     acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True)
-    assert st == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8"
+    assert st == capi.VALID and ctx.last_kernel in ("depthwise_mfma_i8", "depthwise_mfma_pipe_i8")
     assert np.array_equal(got, acc), (ih, iw, c, pad, stride, dil)
     mult = rng.integers(1 << 30, 1 << 31, c).astype(np.int32)
     shift = rng.integers(33, 40, c).astype(np.int8) if seed % 3 else np.full(c, 35, np.int8)
@@ -77,7 +77,7 @@ def test_depthwise_mfma_random_geometry(ctx, seed):
     got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True,
                              rescale=dict(mult=mult, shift=shift, out_zp=out_zp))
     want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp)
-    assert st == wst == capi.VALID and ctx.last_kernel == "depthwise_mfma_i8_rescale"
+    assert st == wst == capi.VALID and ctx.last_kernel in ("depthwise_mfma_i8_rescale", "depthwise_mfma_pipe_i8_rescale")
     assert np.array_equal(got, want), (ih, iw, c, pad, stride, dil)
 
 
