@@ -429,7 +429,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
                 const int64_t rounds   = (tiles + 255) / 256;
                 // A single round of workgroups (one per CU) is as fast as its slowest wave: up to 16 waves, so that a
                 // wave has one unit.  With more rounds two workgroups of at most 8 waves share a CU and overlap.
-                for (int nw = 4; nw <= (rounds == 1 ? 16 : 8); nw += 2)
+                for (int nw = (rounds == 1 ? 16 : 8); nw >= 4; nw -= 2)    // equal cost: the larger workgroup
                 {
                     if (nw * 64 < C)    // the first C lanes build the per-channel tables
                         continue;
