@@ -39,12 +39,12 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
 
 PEAK = {"int8_mfma": 5000.0, "f16_mfma": 2500.0, "hbm": 8000.0}  # TOP/s, TFLOP/s, GB/s (MI355X, published)
 # rocprofv3 summary under profiles/ that holds the HBM traffic of each configuration's dominant kernel
-PROFILE_OF = {"c3": "conv2d_slab_i8_rescale_c3_resnet3x3", "c2": "matmul_gemm_i8_c2_8x1024",
+PROFILE_OF = {"c3": "conv2d_slab_wreg_i8_rescale_c3_resnet3x3", "c2": "matmul_gemm_i8_c2_8x1024",
               "c4": "depthwise_mfma_i8_rescale_c4_mobilenet", "c5a": "gemm_mfma_f16_c5a_3x3_256",
               "c5b": "matmul_gemm_bf16_c5b_4x2048x4096", "maxpool": "max_pool2d_i8_32x112x112x64",
               "avgpool": "avg_pool2d_i8_32x112x112x64", "tconv": "transpose_conv2d_slab_i8_8x28x28x128",
               "conv3d": "conv3d_slab_i8_2x16x28x28x32", "rescale": "rescale_fast_i32_to_i8_64x56x56x64",
-              "c4x8": "depthwise_mfma_i8_rescale_64x112x112x96", "c3x4": "conv2d_slab_i8_rescale_32x56x56x64"}
+              "c4x8": "depthwise_mfma_i8_rescale_64x112x112x96", "c3x4": "conv2d_slab_wreg_i8_rescale_32x56x56x64"}
 
 
 def measured_traffic(cfg, kernel):
