@@ -113,8 +113,9 @@ def test_rescale_dtype_matrix(ctx, in_dt, out_dt, in_u, out_u, in_zp, out_zp, sc
 
 @pytest.mark.parametrize("in_dt", [np.int8, np.int16, np.int32])
 @pytest.mark.parametrize("out_dt,out_zp", [(np.int8, 60), (np.int16, 0), (np.int32, 0)])
-def test_rescale_inexact_round_with_products_beyond_int32(ctx, in_dt, out_dt, out_zp):
-    """INEXACT_ROUND over the whole input range with shifts small enough for float(value) * float(multiplier) * 2^-shift
+def test_rescale_inexact_round_beyond_int32_is_reference_undefined_x86_64_convention(ctx, in_dt, out_dt, out_zp):
+    """Not a parity test for the elements it is named after: an agreement between device and oracle on a convention.
+    INEXACT_ROUND over the whole input range with shifts small enough for float(value) * float(multiplier) * 2^-shift
     to leave int32: the reference's cast is undefined there, its x86-64 builds return INT32_MIN, and the device
     returns the same (not its own saturating conversion), so results and status agree element for element"""
     rng = np.random.default_rng(np.dtype(in_dt).itemsize * 10 + np.dtype(out_dt).itemsize)

@@ -195,7 +195,24 @@ def test_rescale_random_configurations(ctx, block):
             got, st = None, capi.ERROR
         assert st == wst, (seed, ctx.last_kernel, shape, in_dt, kw)
         if wst == oracle.VALID:
-            assert np.array_equal(got.view(want.dtype), want), (seed, ctx.last_kernel, shape, in_dt, kw)
+            got = got.view(want.dtype)
+            if mode == capi.ROUND_INEXACT:
+                # Where float(value) * float(multiplier) * 2^-shift leaves int32 the reference's cast is undefined
+                # (type_conversion.cpp:323); device and oracle share the x86-64 convention there, which is an agreement
+                # between the two and not parity with the reference: those elements are kept out of the parity claim.
+                bits = 8 * np.dtype(in_dt).itemsize
+                v = x.astype(np.int64)
+                if in_u:
+                    v = v & ((1 << bits) - 1)
+                v = v - kw["in_zp"]
+                m = np.broadcast_to(np.asarray(mult, np.int64), (nm,)) if nm > 1 else np.full(C, int(mult[0]), np.int64)
+                sh = np.broadcast_to(np.asarray(shift, np.int64), (nm,)) if nm > 1 else np.full(C, int(shift[0]), np.int64)
+                t = np.rint(v.astype(np.float32) * m.astype(np.float32) * np.exp2(-sh.astype(np.float32)))
+                defined = (t >= -2147483648.0) & (t < 2147483648.0)
+                assert np.array_equal(got[defined], want[defined]), (seed, ctx.last_kernel, shape, in_dt, kw)
+                assert np.array_equal(got[~defined], want[~defined]), ("x86-64 convention", seed, shape, in_dt, kw)
+            else:
+                assert np.array_equal(got, want), (seed, ctx.last_kernel, shape, in_dt, kw)
         seen[wst] += 1
     assert seen[oracle.VALID] >= 20 and seen[oracle.ERROR] >= 5
 

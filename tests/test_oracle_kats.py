@@ -171,7 +171,7 @@ def test_rescale_inexact_round_literals():  # type_conversion_tests.cpp:385-405
     assert st == oracle.VALID and out.tolist() == [114]
 
 
-def test_rescale_inexact_round_is_float_arithmetic_and_names_its_overflow_value():
+def test_rescale_inexact_round_is_float_arithmetic_and_beyond_int32_reference_undefined_x86_64_convention():
     """INEXACT_ROUND is float(value) * float(multiplier) * 2^-shift rounded to nearest even (type_conversion.cpp:320-323),
     checked against numpy float32; a product outside int32 makes the reference's cast undefined, and the value its
     x86-64 builds return, INT32_MIN, is what the oracle states"""
