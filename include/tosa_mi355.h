@@ -52,7 +52,8 @@ enum
     TMI_INT8  = 3,
     TMI_INT16 = 4,
     TMI_INT32 = 5,
-    TMI_INT48 = 6, /* RESCALE input only; one int64 per element, as the reference stores it */
+    TMI_INT48 = 6, /* one int64 per element, as the reference stores it: RESCALE input, and the bias, accumulator and
+                      output of the INT16 convolutions and MATMUL */
     TMI_FP32  = 7,
     TMI_FP16  = 8,
     TMI_BF16  = 9
@@ -171,8 +172,9 @@ typedef struct
     int32_t stride[2];   /* y, x */
     int32_t dilation[2]; /* y, x */
     int32_t bias_len;    /* 1 (broadcast) or OC */
-    int32_t acc_dtype;   /* the attribute's acc_type: TMI_INT32 for INT8 operands, TMI_FP32 for floating point; 0 (a
-                            descriptor zeroed by a caller that predates the field) means that default.  The reference
+    int32_t acc_dtype;   /* the attribute's acc_type: TMI_INT32 for INT8 operands, TMI_INT48 for INT16 operands,
+                            TMI_FP32 for floating point; 0 (a descriptor zeroed by a caller that predates the field)
+                            means that default.  The reference
                             also instantiates FP16 accumulation of FP16 operands (op_factory.h:97-118), which is not
                             built: TMI_ERROR */
 } tmi_conv_desc_t;
@@ -243,16 +245,22 @@ typedef struct
 /* OpConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:723-882 (checks :120-226, :690-720).
  * INT8 x INT8 -> INT32 with int32 accumulation, or FP16 / BF16 / FP32 with fp32 accumulation and an output
  * of the input type (the instantiations at :2220-2229; FP32 runs on the one-element-per-lane kernels, in the
- * reference's summation order).  in_zp / w_zp are the values of operands 3 and 4 (must be 0 for non-INT8). */
+ * reference's summation order).  INT16 x INT8 -> INT48 (:2225; d->in_dtype TMI_INT16, weights INT8, bias and
+ * output one int64 per element, the sum kept in 64 bits and REQUIREd to lie within 48 bits, :875-879) runs on a
+ * one-element-per-lane kernel.  in_zp / w_zp are the values of operands 3 and 4: in_zp must be 0 unless the
+ * input is INT8, w_zp unless the weights are (:804-811). */
 int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
-/* OpDepthwiseConv2d::eval, reference_model/src/ops/tensor_ops.cpp:1172-1334.  M = d->OC / d->IC. */
+/* OpDepthwiseConv2d::eval, reference_model/src/ops/tensor_ops.cpp:1172-1334.  M = d->OC / d->IC.  The same
+ * element types as tmi_conv2d (the instantiations at :2242-2251; INT16 x INT8 -> INT48 at :2247, clip :1325-1329). */
 int tmi_depthwise_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
 /* OpMatMul::eval, reference_model/src/ops/tensor_ops.cpp:1423-1492 (checks :1347-1420).
- * in_dtype TMI_INT8 -> INT32 output; TMI_FP16 / TMI_BF16 / TMI_FP32 -> FP32 output (fp32 accumulation). */
+ * in_dtype TMI_INT8 -> INT32 output; TMI_INT16 -> INT48 output (one int64 per element, zero points must be 0,
+ * the 48-bit REQUIRE of :1485-1489; the instantiation at :2257); TMI_FP16 / TMI_BF16 / TMI_FP32 -> FP32 output
+ * (fp32 accumulation). */
 int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W, const void* a_dev,
                const void* b_dev, int32_t a_zp, int32_t b_zp, void* out_dev);
 

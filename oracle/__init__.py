@@ -124,6 +124,7 @@ def _check(rc, allow=(VALID,)):
 _KINDS = {
     "i8": (np.int8, np.int32, np.int32),      # element dtype, bias dtype, output dtype
     "i32": (np.int32, np.int32, np.int32),
+    "i16": (np.int16, np.int64, np.int64),    # INT16 x INT8 (MATMUL: x INT16) -> INT48 in its int64 storage
     "f32": (np.float32, np.float32, np.float32),
     "f64": (np.float64, np.float64, np.float64),
 }
@@ -137,17 +138,17 @@ def _abs_code(abs_mode, local_bound):
 
 def conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in_zp=0, w_zp=0,
            abs_mode=False, out_hw=None, local_bound=True):
-    """CONV2D.  inp NHWC, w OHWI, bias [1] or [OC].  kind in i8/i32/f32/f64."""
+    """CONV2D.  inp NHWC, w OHWI, bias [1] or [OC].  kind in i8/i32/i16/f32/f64 (i16: INT8 weights, INT48 results)."""
     et, bt, ot = _KINDS[kind]
-    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    inp, w, bias = _c(inp, et), _c(w, np.int8 if kind == "i16" else et), _c(bias, bt)
     oc, kh, kw, _ = w.shape
     s = _shape(inp, kh, kw, oc, bias, pad, stride, dilation, out_hw)
     if w.shape[3] != inp.shape[3]:
         raise OracleStatus(ERROR)
     out = np.zeros((s.N, max(s.OH, 0), max(s.OW, 0), oc), dtype=ot)
     L = lib()
-    if kind in ("i8", "i32"):
-        fn = L.orc_conv2d_i8 if kind == "i8" else L.orc_conv2d_i32
+    if kind in ("i8", "i32", "i16"):
+        fn = {"i8": L.orc_conv2d_i8, "i32": L.orc_conv2d_i32, "i16": L.orc_conv2d_i16}[kind]
         rc = fn(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp), ctypes.c_int32(w_zp),
                 _ptr(out))
     elif kind == "f32":
@@ -163,15 +164,15 @@ def depthwise_conv2d(kind, inp, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilati
                      abs_mode=False, out_hw=None, local_bound=True):
     """DEPTHWISE_CONV2D.  inp NHWC, w [KH,KW,C,M], bias [1] or [C*M]."""
     et, bt, ot = _KINDS[kind]
-    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    inp, w, bias = _c(inp, et), _c(w, np.int8 if kind == "i16" else et), _c(bias, bt)
     kh, kw, c, m = w.shape
     if c != inp.shape[3]:
         raise OracleStatus(ERROR)
     s = _shape(inp, kh, kw, c * m, bias, pad, stride, dilation, out_hw)
     out = np.zeros((s.N, max(s.OH, 0), max(s.OW, 0), c * m), dtype=ot)
     L = lib()
-    if kind in ("i8", "i32"):
-        fn = L.orc_depthwise_i8 if kind == "i8" else L.orc_depthwise_i32
+    if kind in ("i8", "i32", "i16"):
+        fn = {"i8": L.orc_depthwise_i8, "i32": L.orc_depthwise_i32, "i16": L.orc_depthwise_i16}[kind]
         rc = fn(ctypes.byref(s), ctypes.c_int32(m), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp),
                 ctypes.c_int32(w_zp), _ptr(out))
     elif kind == "f32":
@@ -269,8 +270,8 @@ def matmul(kind, a, b, a_zp=0, b_zp=0, abs_mode=False):
     out = np.zeros((n, h, w), dtype=ot)
     L = lib()
     dims = [ctypes.c_int32(v) for v in (n, h, c, w)]
-    if kind in ("i8", "i32"):
-        fn = L.orc_matmul_i8 if kind == "i8" else L.orc_matmul_i32
+    if kind in ("i8", "i32", "i16"):
+        fn = {"i8": L.orc_matmul_i8, "i32": L.orc_matmul_i32, "i16": L.orc_matmul_i16}[kind]
         rc = fn(*dims, _ptr(a), _ptr(b), ctypes.c_int32(a_zp), ctypes.c_int32(b_zp), _ptr(out))
     elif kind == "f32":
         rc = L.orc_matmul_f32(*dims, _ptr(a), _ptr(b), _ptr(out))

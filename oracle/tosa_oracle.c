@@ -129,6 +129,7 @@ int orc_conv_check(const orc_conv_shape_t* s, int32_t depthwise_m)
 #define ORC_ABS_F64(v) fabs(v)
 
 ORC_DEFINE_CONV2D(conv2d_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_CONV2D(conv2d_i64_impl, int64_t, ORC_ABS_I32)
 ORC_DEFINE_CONV2D(conv2d_f32_impl, float, ORC_ABS_F32)
 ORC_DEFINE_CONV2D(conv2d_f64_impl, double, ORC_ABS_F64)
 
@@ -168,6 +169,49 @@ int orc_conv2d_i8(const orc_conv_shape_t* s, const int8_t* in, const int8_t* w, 
     int rc        = (in32 && w32) ? orc_conv2d_i32(s, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
     free(in32);
     free(w32);
+    return rc;
+}
+
+/* INT16 x INT8 -> INT48 (tensor_ops.cpp:2225): the accumulator type is int64 (template_types.h:109), the input zero
+ * point must be zero for a tensor that is not INT8 (:805), the weights keep theirs, and the result is clipped to 48 bits
+ * (:875-879).  The same loop nest as above on operands widened to the accumulator type. */
+static int64_t* widen_i16_to_i64(const int16_t* p, size_t n)
+{
+    int64_t* r = (int64_t*)malloc(sizeof(int64_t) * n + 8);
+    if (r)
+        for (size_t i = 0; i < n; i++)
+            r[i] = (int64_t)p[i];
+    return r;
+}
+
+static int64_t* widen_i8_to_i64(const int8_t* p, size_t n)
+{
+    int64_t* r = (int64_t*)malloc(sizeof(int64_t) * n + 8);
+    if (r)
+        for (size_t i = 0; i < n; i++)
+            r[i] = (int64_t)p[i];
+    return r;
+}
+
+static void clip_int48(int64_t* p, size_t n)
+{
+    const int64_t lo = -((int64_t)1 << 47), hi = ((int64_t)1 << 47) - 1;
+    for (size_t i = 0; i < n; i++)
+        p[i] = p[i] < lo ? lo : (p[i] > hi ? hi : p[i]);
+}
+
+int orc_conv2d_i16(const orc_conv_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias, int32_t in_zp,
+                   int32_t w_zp, int64_t* out)
+{
+    if (orc_conv_check(s, 0) != ORC_VALID || in_zp != 0)
+        return ORC_ERROR;
+    int64_t* in64 = widen_i16_to_i64(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int64_t* w64  = widen_i8_to_i64(w, (size_t)s->OC * s->KH * s->KW * s->IC);
+    int rc        = (in64 && w64) ? conv2d_i64_impl(s, in64, w64, bias, 0, (int64_t)w_zp, 0, out) : ORC_ERROR;
+    if (rc == ORC_VALID)
+        clip_int48(out, (size_t)s->N * s->OH * s->OW * s->OC);
+    free(in64);
+    free(w64);
     return rc;
 }
 
@@ -428,6 +472,7 @@ int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const 
     }
 
 ORC_DEFINE_DEPTHWISE(depthwise_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_DEPTHWISE(depthwise_i64_impl, int64_t, ORC_ABS_I32)
 ORC_DEFINE_DEPTHWISE(depthwise_f32_impl, float, ORC_ABS_F32)
 ORC_DEFINE_DEPTHWISE(depthwise_f64_impl, double, ORC_ABS_F64)
 
@@ -447,6 +492,22 @@ int orc_depthwise_i8(const orc_conv_shape_t* s, int32_t M, const int8_t* in, con
     int rc        = (in32 && w32) ? orc_depthwise_i32(s, M, in32, w32, bias, in_zp, w_zp, out) : ORC_ERROR;
     free(in32);
     free(w32);
+    return rc;
+}
+
+/* INT16 x INT8 -> INT48 (tensor_ops.cpp:2247; the clip at :1325-1329) */
+int orc_depthwise_i16(const orc_conv_shape_t* s, int32_t M, const int16_t* in, const int8_t* w, const int64_t* bias,
+                      int32_t in_zp, int32_t w_zp, int64_t* out)
+{
+    if (M < 1 || orc_conv_check(s, M) != ORC_VALID || in_zp != 0)
+        return ORC_ERROR;
+    int64_t* in64 = widen_i16_to_i64(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int64_t* w64  = widen_i8_to_i64(w, (size_t)s->KH * s->KW * s->IC * M);
+    int rc        = (in64 && w64) ? depthwise_i64_impl(s, M, in64, w64, bias, 0, (int64_t)w_zp, 0, out) : ORC_ERROR;
+    if (rc == ORC_VALID)
+        clip_int48(out, (size_t)s->N * s->OH * s->OW * s->OC);
+    free(in64);
+    free(w64);
     return rc;
 }
 
@@ -510,6 +571,7 @@ int orc_depthwise_f64(const orc_conv_shape_t* s, int32_t M, const double* in, co
     }
 
 ORC_DEFINE_MATMUL(matmul_i32_impl, int32_t, ORC_ABS_I32)
+ORC_DEFINE_MATMUL(matmul_i64_impl, int64_t, ORC_ABS_I32)
 ORC_DEFINE_MATMUL(matmul_f32_impl, float, ORC_ABS_F32)
 ORC_DEFINE_MATMUL(matmul_f64_impl, double, ORC_ABS_F64)
 
@@ -527,6 +589,23 @@ int orc_matmul_i8(int32_t N, int32_t H, int32_t C, int32_t W, const int8_t* a, c
     int rc       = (a32 && b32) ? orc_matmul_i32(N, H, C, W, a32, b32, a_zp, b_zp, out) : ORC_ERROR;
     free(a32);
     free(b32);
+    return rc;
+}
+
+/* INT16 x INT16 -> INT48 (tensor_ops.cpp:2257): zero points must be zero for tensors that are not INT8 (:1433-1434),
+ * int64 accumulation, the result clipped to 48 bits (:1485-1489) */
+int orc_matmul_i16(int32_t N, int32_t H, int32_t C, int32_t W, const int16_t* a, const int16_t* b, int32_t a_zp,
+                   int32_t b_zp, int64_t* out)
+{
+    if (a_zp != 0 || b_zp != 0)
+        return ORC_ERROR;
+    int64_t* a64 = widen_i16_to_i64(a, (size_t)N * H * C);
+    int64_t* b64 = widen_i16_to_i64(b, (size_t)N * C * W);
+    int rc       = (a64 && b64) ? matmul_i64_impl(N, H, C, W, a64, b64, 0, 0, 0, out) : ORC_ERROR;
+    if (rc == ORC_VALID)
+        clip_int48(out, (size_t)N * H * W);
+    free(a64);
+    free(b64);
     return rc;
 }
 

@@ -87,6 +87,11 @@ int orc_conv2d_i8(const orc_conv_shape_t* s, const int8_t* in, const int8_t* w, 
 /* DEPTHWISE_CONV2D, weight [KH,KW,IC,M], out channel = ic*M + m. */
 int orc_depthwise_i32(const orc_conv_shape_t* s, int32_t M, const int32_t* in, const int32_t* w,
                       const int32_t* bias, int32_t in_zp, int32_t w_zp, int32_t* out);
+/* INT16 x INT8 -> INT48 CONV2D / DEPTHWISE_CONV2D: int64 bias and results, clipped to 48 bits; input_zp must be 0 */
+int orc_conv2d_i16(const orc_conv_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias, int32_t in_zp,
+                   int32_t w_zp, int64_t* out);
+int orc_depthwise_i16(const orc_conv_shape_t* s, int32_t M, const int16_t* in, const int8_t* w, const int64_t* bias,
+                      int32_t in_zp, int32_t w_zp, int64_t* out);
 int orc_depthwise_i8(const orc_conv_shape_t* s, int32_t M, const int8_t* in, const int8_t* w, const int32_t* bias,
                      int32_t in_zp, int32_t w_zp, int32_t* out);
 int orc_depthwise_f32(const orc_conv_shape_t* s, int32_t M, const float* in, const float* w, const float* bias,
@@ -140,6 +145,9 @@ int orc_matmul_i32(int32_t N, int32_t H, int32_t C, int32_t W, const int32_t* a,
                    int32_t b_zp, int32_t* out);
 int orc_matmul_i8(int32_t N, int32_t H, int32_t C, int32_t W, const int8_t* a, const int8_t* b, int32_t a_zp,
                   int32_t b_zp, int32_t* out);
+/* INT16 x INT16 -> INT48 (int64 results clipped to 48 bits) */
+int orc_matmul_i16(int32_t N, int32_t H, int32_t C, int32_t W, const int16_t* a, const int16_t* b, int32_t a_zp,
+                   int32_t b_zp, int64_t* out);
 int orc_matmul_f32(int32_t N, int32_t H, int32_t C, int32_t W, const float* a, const float* b, float* out);
 int orc_matmul_f64(int32_t N, int32_t H, int32_t C, int32_t W, const double* a, const double* b, int abs_mode,
                    double* out);

@@ -210,7 +210,7 @@ class DeviceTensor:
         self.ptr = ctx._alloc(self.nbytes)
 
     def numpy(self) -> np.ndarray:
-        dt = self.np_dtype or {INT8: np.int8, INT16: np.int16, INT32: np.int32, FP32: np.float32,
+        dt = self.np_dtype or {INT8: np.int8, INT16: np.int16, INT32: np.int32, INT48: np.int64, FP32: np.float32,
                                FP16: np.float16, BF16: np.uint16, F64: np.float64}[self.dtype]
         out = np.empty(self.shape, dtype=dt)
         self.ctx._check(self.ctx.lib.tmi_download(self.ctx.handle, out.ctypes.data_as(ctypes.c_void_p),
@@ -297,7 +297,7 @@ class Context:
     def conv_desc(in_dtype, out_dtype, in_shape, oc, kh, kw, out_hw, pad, stride, dilation, bias_len,
                   acc_dtype=None) -> ConvDesc:
         d = ConvDesc()
-        d.acc_dtype = acc_dtype if acc_dtype is not None else (INT32 if in_dtype == INT8 else FP32)
+        d.acc_dtype = acc_dtype if acc_dtype is not None else (INT32 if in_dtype == INT8 else (INT48 if in_dtype == INT16 else FP32))
         d.in_dtype, d.out_dtype = in_dtype, out_dtype
         d.N, d.IH, d.IW, d.IC = in_shape
         d.OC, d.KH, d.KW = oc, kh, kw

@@ -192,6 +192,80 @@ __global__ __launch_bounds__(256) void matmul_direct_kernel(int32_t N, int32_t H
     }
 }
 
+// INT16 x INT8 -> INT48 convolutions and INT16 x INT16 -> INT48 MATMUL (tensor_ops.cpp:2225, 2247, 2257): accumulator,
+// bias and result are int64, the reference's storage of INT48, and the result is clipped to 48 bits at the end
+// (tensor_ops.cpp:875-879, 1325-1329, 1485-1489).  The input zero point is zero by rule (only INT8 tensors have one);
+// the INT8 weights' need not be.  One output element per lane, loops in the reference's order.
+__device__ __forceinline__ int64_t clip_int48(int64_t v)
+{
+    const int64_t lo = -(int64_t(1) << 47), hi = (int64_t(1) << 47) - 1;
+    return v < lo ? lo : (v > hi ? hi : v);
+}
+
+template <bool DEPTHWISE>
+__global__ __launch_bounds__(256) void conv_i16_direct_kernel(ConvGeom g, const int16_t* __restrict__ in,
+                                                              const int8_t* __restrict__ w,
+                                                              const int64_t* __restrict__ bias, int32_t w_zp,
+                                                              int64_t* __restrict__ out)
+{
+    const int64_t total  = (int64_t)g.N * g.OH * g.OW * g.OC;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride)
+    {
+        const int oc = (int)(idx % g.OC);
+        int64_t t    = idx / g.OC;
+        const int ox = (int)(t % g.OW);
+        t /= g.OW;
+        const int oy = (int)(t % g.OH);
+        const int n  = (int)(t / g.OH);
+        int64_t acc  = 0;
+        for (int ky = 0; ky < g.KH; ky++)
+        {
+            const int y = oy * g.stride_y + ky * g.dil_y - g.pad_top;
+            if (y < 0 || y >= g.IH)
+                continue;
+            for (int kx = 0; kx < g.KW; kx++)
+            {
+                const int x = ox * g.stride_x + kx * g.dil_x - g.pad_left;
+                if (x < 0 || x >= g.IW)
+                    continue;
+                const int64_t ib = (((int64_t)n * g.IH + y) * g.IW + x) * g.IC;
+                if constexpr (DEPTHWISE)
+                {
+                    const int ic = oc / g.M, km = oc % g.M;
+                    acc += (int64_t)in[ib + ic] * (int64_t)((int32_t)w[(((int64_t)ky * g.KW + kx) * g.IC + ic) * g.M + km] - w_zp);
+                }
+                else
+                {
+                    const int64_t wb = (((int64_t)oc * g.KH + ky) * g.KW + kx) * g.IC;
+                    for (int ic = 0; ic < g.IC; ic++)
+                        acc += (int64_t)in[ib + ic] * (int64_t)((int32_t)w[wb + ic] - w_zp);
+                }
+            }
+        }
+        out[idx] = clip_int48(bias[g.bias_len == 1 ? 0 : oc] + acc);
+    }
+}
+
+__global__ __launch_bounds__(256) void matmul_i16_direct_kernel(int32_t N, int32_t H, int32_t C, int32_t W,
+                                                                const int16_t* __restrict__ a,
+                                                                const int16_t* __restrict__ b, int64_t* __restrict__ out)
+{
+    const int64_t total  = (int64_t)N * H * W;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride)
+    {
+        const int x = (int)(idx % W);
+        int64_t t   = idx / W;
+        const int h = (int)(t % H);
+        const int n = (int)(t / H);
+        int64_t acc = 0;
+        for (int c = 0; c < C; c++)
+            acc += (int64_t)a[((int64_t)n * H + h) * C + c] * (int64_t)b[((int64_t)n * C + c) * W + x];
+        out[idx] = clip_int48(acc);
+    }
+}
+
 static int grid_for(int64_t work_items)
 {
     int64_t blocks = (work_items + 255) / 256;
@@ -278,6 +352,32 @@ const char* launch_matmul_direct(hipStream_t st, int32_t in_dtype, int32_t N, in
         return "matmul_direct_f32";
     }
     return nullptr;
+}
+
+const char* launch_conv_i16_direct(hipStream_t st, bool depthwise, const ConvGeom& g, const void* in, const void* w,
+                                   const void* bias, int32_t w_zp, void* out)
+{
+    const int64_t total = (int64_t)g.N * g.OH * g.OW * g.OC;
+    if (total == 0)
+        return "conv_direct_empty";
+    if (depthwise)
+        hipLaunchKernelGGL((conv_i16_direct_kernel<true>), dim3(grid_for(total)), dim3(256), 0, st, g, (const int16_t*)in,
+                           (const int8_t*)w, (const int64_t*)bias, w_zp, (int64_t*)out);
+    else
+        hipLaunchKernelGGL((conv_i16_direct_kernel<false>), dim3(grid_for(total)), dim3(256), 0, st, g, (const int16_t*)in,
+                           (const int8_t*)w, (const int64_t*)bias, w_zp, (int64_t*)out);
+    return depthwise ? "depthwise_direct_i16_i48" : "conv2d_direct_i16_i48";
+}
+
+const char* launch_matmul_i16_direct(hipStream_t st, int32_t N, int32_t H, int32_t C, int32_t W, const void* a, const void* b,
+                                     void* out)
+{
+    const int64_t total = (int64_t)N * H * W;
+    if (total == 0)
+        return "matmul_direct_empty";
+    hipLaunchKernelGGL(matmul_i16_direct_kernel, dim3(grid_for(total)), dim3(256), 0, st, N, H, C, W, (const int16_t*)a,
+                       (const int16_t*)b, (int64_t*)out);
+    return "matmul_direct_i16_i48";
 }
 
 }    // namespace tmi

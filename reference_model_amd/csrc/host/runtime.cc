@@ -221,7 +221,8 @@ public:
             validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 4, 4))
             return 1;
-        if (inputs[1]->getDtype() != inputs[0]->getDtype())
+        // the weights have the input's type, except that INT16 inputs come with INT8 weights (tensor_ops.cpp:2225, 2247)
+        if (inputs[1]->getDtype() != (inputs[0]->getDtype() == DType_INT16 ? DType_INT8 : inputs[0]->getDtype()))
             return error("weight data type not supported for this configuration of operator");
         tmi_conv_desc_t d;
         if (fill_desc(d))
@@ -433,7 +434,7 @@ int ConvBase::eval()
     if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
         return error("zero-point operands must be available on the host");
     SubgraphTraverser* s = parent_sgt;
-    if (s->precise_mode && inputs[0]->getDtype() != DType_INT8)
+    if (s->precise_mode && inputs[0]->getDtype() != DType_INT8 && inputs[0]->getDtype() != DType_INT16)
     {
         // precise mode (tensor_ops.cpp:790-802, :1245-1257): fp64 accumulation, fp64 result
         outputs[0]->precise = true;
@@ -734,9 +735,12 @@ public:
         if (inputs[3]->shape[0] != 1)
             return error("OpMatMul: 'b_zp' zero point shape should be [1]");
         const DType in = a->getDtype();
-        if (b->getDtype() != in || !(in == DType_INT8 || in == DType_FP16 || in == DType_BF16 || in == DType_FP32))
+        // the instantiations of tensor_ops.cpp:2256-2261 that the library has: INT8 -> INT32, INT16 -> INT48, floating
+        // point -> FP32
+        if (b->getDtype() != in ||
+            !(in == DType_INT8 || in == DType_INT16 || in == DType_FP16 || in == DType_BF16 || in == DType_FP32))
             return error("OpMatMul: input data type not supported for this configuration of operator");
-        if (o->getDtype() != (in == DType_INT8 ? DType_INT32 : DType_FP32))
+        if (o->getDtype() != (in == DType_INT8 ? DType_INT32 : (in == DType_INT16 ? DType_INT48 : DType_FP32)))
             return error("OpMatMul: Output data type not supported for this configuration of operator");
         return 0;
     }
@@ -747,7 +751,7 @@ public:
             return error("zero-point operands must be available on the host");
         const Tensor *a = inputs[0], *b = inputs[1];
         SubgraphTraverser* s = parent_sgt;
-        if (s->precise_mode && a->getDtype() != DType_INT8)
+        if (s->precise_mode && a->getDtype() != DType_INT8 && a->getDtype() != DType_INT16)
         {
             // precise mode (tensor_ops.cpp:1436-1443)
             outputs[0]->precise = true;

@@ -204,15 +204,18 @@ int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool d
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 && d->in_dtype != TMI_FP32)
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 &&
+        d->in_dtype != TMI_FP32)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
-    const int32_t want_out = d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype;
+    // INT16 inputs come with INT8 weights and INT48 accumulator, bias and result (tensor_ops.cpp:2225, 2247)
+    const int32_t want_out = d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : d->in_dtype);
     if (d->out_dtype != want_out)
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
     // the accumulator type is part of the operator's type signature (op_factory.h:97-118, tensor_ops.cpp:2219-2251):
-    // INT32 for INT8 operands, FP32 for floating point; FP16 accumulation of FP16 operands exists in the reference and
-    // is not built here
-    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
+    // INT32 for INT8 operands, INT48 for INT16, FP32 for floating point; FP16 accumulation of FP16 operands exists in the
+    // reference and is not built here
+    const int32_t want_acc = d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : TMI_FP32);
+    if (d->acc_dtype != 0 && d->acc_dtype != want_acc)    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1 || d->OH < 0 ||
         d->OW < 0)
@@ -248,7 +251,7 @@ int validate_conv(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* d, bool d
         return fail(ctx, "%s: bias channel mismatch %d != %d", op, d->bias_len, d->OC);
     if (d->in_dtype != TMI_INT8 && in_zp != 0)
         return fail(ctx, "%s: Input zero point must be zero for non int8_t data", op);
-    if (d->in_dtype != TMI_INT8 && w_zp != 0)
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && w_zp != 0)    // INT16 inputs have INT8 weights
         return fail(ctx, "%s: Weight zero point must be zero for non int8_t data", op);
     if (in_zp < -128 || in_zp > 127 || w_zp < -128 || w_zp > 127)
         return fail(ctx, "%s: zero point outside the int8 range", op);
@@ -419,6 +422,12 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     {
         ctx->last_kernel = "empty";
         return TMI_VALID;
+    }
+    if (d->in_dtype == TMI_INT16)
+    {
+        if (rp.enabled)
+            return fail(ctx, "%s: the fused rescale needs an INT8 convolution", op);
+        return after_launch(ctx, launch_conv_i16_direct(ctx->stream, depthwise, g, in, w, bias, w_zp, out));
     }
     if (depthwise && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
         name = launch_depthwise_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
@@ -1110,7 +1119,7 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
 {
     if (!ctx)
         return TMI_ERROR;
-    if (in_dtype != TMI_INT8 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16 && in_dtype != TMI_FP32)
+    if (in_dtype != TMI_INT8 && in_dtype != TMI_INT16 && in_dtype != TMI_FP16 && in_dtype != TMI_BF16 && in_dtype != TMI_FP32)
         return fail(ctx, "OpMatMul: input data type not supported for this configuration of operator");
     if (N < 0 || H < 0 || C < 0 || W < 0)
         return fail(ctx, "OpMatMul: negative tensor dimension");
@@ -1130,6 +1139,8 @@ int tmi_matmul(tmi_ctx_t* ctx, int32_t in_dtype, int32_t N, int32_t H, int32_t C
         ctx->last_kernel = "empty";
         return TMI_VALID;
     }
+    if (in_dtype == TMI_INT16)    // INT16 x INT16 -> INT48 (tensor_ops.cpp:2257): int64 results
+        return after_launch(ctx, launch_matmul_i16_direct(ctx->stream, N, H, C, W, a_dev, b_dev, out_dev));
     const char* name = nullptr;
     if (ctx->kernel_choice != 1 && C > 0 && in_dtype != TMI_FP32)
     {

@@ -184,6 +184,11 @@ const char* launch_conv3d_operands(hipStream_t st, int32_t row_bytes, int32_t OC
 const char* launch_depthwise_vec(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
                                  const void* in, const void* w, const void* bias, int32_t in_zp, int32_t w_zp,
                                  const RescaleParams& rp, void* out, uint32_t* flag_word);
+// INT16 x INT8 -> INT48 CONV2D / DEPTHWISE_CONV2D and INT16 x INT16 -> INT48 MATMUL (int64 bias and results)
+const char* launch_conv_i16_direct(hipStream_t st, bool depthwise, const ConvGeom& g, const void* in, const void* w,
+                                   const void* bias, int32_t w_zp, void* out);
+const char* launch_matmul_i16_direct(hipStream_t st, int32_t N, int32_t H, int32_t C, int32_t W, const void* a, const void* b,
+                                     void* out);
 const char* launch_matmul_direct(hipStream_t st, int32_t in_dtype, int32_t N, int32_t H, int32_t C, int32_t W,
                                  const void* a, const void* b, int32_t a_zp, int32_t b_zp, void* out);
 

@@ -15,7 +15,7 @@ def _conv_common(ctx, x, w_shape_khkwoc, bias, pad, stride, dilation, in_dtype, 
     kh, kw, oc = w_shape_khkwoc
     if out_hw is None:
         out_hw = oracle.conv_out_hw(x.shape[1], x.shape[2], kh, kw, pad, stride, dilation) or (0, 0)
-    out_dtype = capi.INT32 if in_dtype == capi.INT8 else in_dtype
+    out_dtype = capi.INT32 if in_dtype == capi.INT8 else (capi.INT48 if in_dtype == capi.INT16 else in_dtype)
     d = ctx.conv_desc(in_dtype, out_dtype, x.shape, oc, kh, kw, out_hw, pad, stride, dilation, bias.shape[0])
     return d, out_hw, out_dtype
 
@@ -32,11 +32,14 @@ def conv2d(ctx, x, w, bias, pad=(0, 0, 0, 0), stride=(1, 1), dilation=(1, 1), in
     else:
         oc, kh, kw, _ = w.shape
     d, out_hw, out_dtype = _conv_common(ctx, x, (kh, kw, oc), bias, pad, stride, dilation, in_dtype, out_hw)
-    tx, tw, tb = ctx.upload(x, in_dtype), ctx.upload(w, in_dtype), ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
+    # INT16 inputs come with INT8 weights and an INT48 bias (int64)
+    tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, capi.INT8 if in_dtype == capi.INT16 else in_dtype)
+    tb = ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
     shape = (x.shape[0], out_hw[0], out_hw[1], oc)
     try:
         if rescale is None:
-            np_out = {capi.INT32: np.int32, capi.FP16: np.float16, capi.BF16: np.uint16, capi.FP32: np.float32}[out_dtype]
+            np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16,
+                      capi.FP32: np.float32}[out_dtype]
             to = ctx.empty(shape, out_dtype, np_out)
             fn = ctx.depthwise_conv2d if depthwise else ctx.conv2d
             fn(d, tx, tw, tb, in_zp, w_zp, to)
@@ -64,7 +67,7 @@ def matmul(ctx, a, b, a_zp=0, b_zp=0, dtype=None):
     n, h, c = a.shape
     w = b.shape[2]
     ta, tb = ctx.upload(a, in_dtype), ctx.upload(b, in_dtype)
-    to = ctx.empty((n, h, w), capi.INT32 if in_dtype == capi.INT8 else capi.FP32)
+    to = ctx.empty((n, h, w), capi.INT32 if in_dtype == capi.INT8 else (capi.INT48 if in_dtype == capi.INT16 else capi.FP32))
     try:
         ctx.matmul(in_dtype, n, h, c, w, ta, tb, a_zp, b_zp, to)
         st = ctx.sync()

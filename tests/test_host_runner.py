@@ -329,6 +329,53 @@ def test_int48_rescale_graph(tmp_path):
 
 
 @pytest.mark.gpu
+def test_int16_convolution_and_matmul_graphs(tmp_path):
+    """the 16-bit instantiations (tensor_ops.cpp:2225, 2247, 2257): INT16 x INT8 -> INT48 CONV2D and DEPTHWISE_CONV2D whose
+    result a RESCALE takes back to INT16, and INT16 x INT16 -> INT48 MATMUL; INT48 tensors are int64 .npy files, INT48
+    constants 6 bytes per element"""
+    rng = np.random.default_rng(21)
+    x = rng.integers(-32768, 32768, (2, 9, 8, 12)).astype(np.int16)
+    w = rng.integers(-128, 128, (6, 3, 3, 12)).astype(np.int8)
+    wd = rng.integers(-128, 128, (3, 3, 12, 1)).astype(np.int8)
+    bias = rng.integers(-(1 << 30), 1 << 30, 6).astype(np.int64)
+    biasd = rng.integers(-(1 << 30), 1 << 30, 12).astype(np.int64)
+    mult = rng.integers(1 << 13, 1 << 15, 6).astype(np.int16)
+    shift = rng.integers(24, 30, 6).astype(np.int8)
+    acc = oracle.conv2d("i16", x, w, bias, (1, 1, 1, 1), w_zp=2)
+    accd = oracle.depthwise_conv2d("i16", x, wd, biasd, (1, 1, 1, 1))
+    want, st = oracle.rescale(acc, mult, shift, out_dtype=np.int16, scale32=False, rounding_mode=oracle.ROUND_SINGLE)
+    assert st == oracle.VALID and len(np.unique(want)) > 100
+    ts = [W.tensor("x", x.shape, np.int16), W.tensor("w", w.shape, np.int8, w), W.tensor("wd", wd.shape, np.int8, wd),
+          W.tensor("bias", [6], np.int64, bias), W.tensor("biasd", [12], np.int64, biasd),
+          W.tensor("izp", [1], np.int16, [0]), W.tensor("wzp", [1], np.int8, [2]), W.tensor("wzp0", [1], np.int8, [0]),
+          W.tensor("acc", [2, 9, 8, 6], np.int64), W.tensor("accd", [2, 9, 8, 12], np.int64),
+          W.tensor("mult", [6], np.int16, mult), W.tensor("shift", [6], np.int8, shift),
+          W.tensor("rizp", [1], np.int64, [0]), W.tensor("rozp", [1], np.int16, [0]), W.tensor("y", [2, 9, 8, 6], np.int16)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "wd", "bias", "biasd", "izp", "wzp", "wzp0", "mult", "shift", "rizp", "rozp")]
+    ops.append(W.operator(R.OP_CONV2D, ["x", "w", "bias", "izp", "wzp"], ["acc"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1), acc_type=6)))
+    ops.append(W.operator(R.OP_DEPTHWISE_CONV2D, ["x", "wd", "biasd", "izp", "wzp0"], ["accd"],
+                          W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1), acc_type=6)))
+    ops.append(W.operator(R.OP_RESCALE, ["acc", "mult", "shift", "rizp", "rozp"], ["y"], W.rescale_attr(scale32=False, rounding_mode=1)))
+    r = _run(_write_case(tmp_path, W.graph(ts, ops, ["x"], ["y", "accd"]), {"x": x}, ["y", "accd"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(tmp_path / "y_out.npy"), want)
+    got_d = np.load(tmp_path / "accd_out.npy")
+    assert got_d.dtype == np.int64 and np.array_equal(got_d, accd)
+
+    a = rng.integers(-32768, 32768, (2, 20, 33)).astype(np.int16)
+    b = rng.integers(-32768, 32768, (2, 33, 7)).astype(np.int16)
+    ts = [W.tensor("a", a.shape, np.int16), W.tensor("b", b.shape, np.int16), W.tensor("azp", [1], np.int16, [0]),
+          W.tensor("bzp", [1], np.int16, [0]), W.tensor("o", [2, 20, 7], np.int64)]
+    ops = [W.operator(R.OP_CONST, [], ["azp"]), W.operator(R.OP_CONST, [], ["bzp"]),
+           W.operator(R.OP_MATMUL, ["a", "b", "azp", "bzp"], ["o"])]
+    d2 = tmp_path / "mm"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops, ["a", "b"], ["o"]), {"a": a, "b": b}, ["o"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d2 / "o_out.npy"), oracle.matmul("i16", a, b))
+
+
+@pytest.mark.gpu
 def test_inexact_round_rescale_in_precise_and_compliance_mode(tmp_path):
     """--precise_mode=1 reaches an INEXACT_ROUND RESCALE (type_conversion.cpp:326-346): FP64 maths truncated; on a
     compliance descriptor the normal pass writes the lower edge of the error bound and the bounds pass the upper one"""
