@@ -505,7 +505,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 // few as it can: with one shift for all channels the requantisation of a pixel tile is dealt over the K steps of the
 // wave's next one, four instructions per output element, and the fragments of the next tile are requested in the last
 // steps of the current one.
-template <bool ZA>
+template <bool ZA, bool VL>
 __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
 {
     constexpr int KH = 3, KW = 3, CH = 4;    // 3x3 taps of 64 input channels: 18 weight fragments, 72 registers
@@ -573,19 +573,37 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
     const uint32_t lbase = (uint32_t)(uintptr_t)lds;
     if (wave < LWAVES)
     {
+        constexpr int WB = (WLOADS + LWAVES - 1) / LWAVES;
+        v4i tw[VL ? WB : 1];
         {
             // Weights: LDS row r is channel r of the block, slot s = (row, chunk) reads byte 16 (s - row) of the block's
             // weights; seven loads on are 448 slots.  Whatever lies past the block's last channel is clamped to its last chunk.
             const int rows       = a.OC - oc0 < 64 ? a.OC - oc0 : 64;
             const uint32_t limit = (uint32_t)rows * (TAPS * KB) - 16u;
             const uint8_t* wb    = a.w + (size_t)oc0 * (TAPS * KB);
-            for (int l = wave; l < WLOADS; l += LWAVES)
+            if constexpr (VL)
             {
-                const int s0       = l * 64 + lane;
-                const int row0     = s0 / RW;
-                const uint32_t off = 16u * (uint32_t)(s0 - row0);
-                slab_load_off(off < limit ? off : limit, wb, lbase + l * 1024);
+                // through registers: the wave's five or six loads are in flight together (loads into LDS leave a wave
+                // one at a time), and are written to LDS after its patch loads have been issued
+#pragma unroll
+                for (int j = 0; j < WB; j++)
+                {
+                    const int l        = wave + j * LWAVES;
+                    const int s0       = l * 64 + lane;
+                    const int row0     = s0 / RW;
+                    const uint32_t off = 16u * (uint32_t)(s0 - row0);
+                    if (l < WLOADS)
+                        tw[j] = *reinterpret_cast<const v4i*>(wb + (off < limit ? off : limit));
+                }
             }
+            else
+                for (int l = wave; l < WLOADS; l += LWAVES)
+                {
+                    const int s0       = l * 64 + lane;
+                    const int row0     = s0 / RW;
+                    const uint32_t off = 16u * (uint32_t)(s0 - row0);
+                    slab_load_off(off < limit ? off : limit, wb, lbase + l * 1024);
+                }
         }
         {
             const uint8_t* in_n = a.in + (size_t)n * (a.IH * a.IW) * KB;
@@ -608,6 +626,16 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
                 r += a.step_chunk, py += a.step_row;
                 if (r >= a.pitch)
                     r -= a.pitch, py++;
+            }
+        }
+        if constexpr (VL)
+        {
+#pragma unroll
+            for (int j = 0; j < WB; j++)
+            {
+                const int l = wave + j * LWAVES;
+                if (l < WLOADS)
+                    *reinterpret_cast<v4i*>(lds + l * 1024 + lane * 16) = tw[j];
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -959,7 +987,13 @@ static bool launch_slab_wreg(hipStream_t st, const SlabArgs& a, int grid, int ld
         last_launch_shape[0] = grid, last_launch_shape[1] = 512, last_launch_shape[2] = lds_bytes;
         return true;
     };
-    return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true>) : launch(conv2d_slab_wreg_kernel<false>);
+    // Weight loads through registers from five pixel tiles per workgroup on.  Measured on MI355X, us per launch with the
+    // loads into LDS / through registers, [N,56,56,64]->64: N = 4 3.59 / 3.68, 8 4.04 / 4.09, 10 4.55 / 4.57, 12 4.70 / 4.60,
+    // 16 5.25 / 5.10, 20 5.67 / 5.56, 32 6.96 / 6.64, 64 11.0 / 10.47.
+    const bool vl = (a.TH * a.TW + 31) / 32 >= 5;
+    if (vl)
+        return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true, true>) : launch(conv2d_slab_wreg_kernel<false, true>);
+    return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true, false>) : launch(conv2d_slab_wreg_kernel<false, false>);
 }
 
 template <int KH, int KW, int CH>
