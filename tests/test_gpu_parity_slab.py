@@ -177,24 +177,27 @@ def test_slab_tile_width_follows_the_number_of_tiles(ctx):
     assert grid_of(32, 57, 2) > 32 * 29 * 29 // 252 * 2    # stride 2: tiles of at most 124 pixels
 
 
-@pytest.mark.parametrize("n,hw,shifts", [(8, 56, "uniform"), (32, 56, "uniform"), (32, 56, "mixed"), (5, 50, "uniform"),
-                                         (40, 28, "mixed"), (3, 112, "uniform")])
-def test_slab_weights_in_registers_form_on_large_tiles(ctx, n, hw, shifts):
+@pytest.mark.parametrize("n,hw,shifts,oc", [(8, 56, "uniform", 64), (32, 56, "uniform", 64), (32, 56, "mixed", 64),
+                                            (5, 50, "uniform", 64), (40, 28, "mixed", 64), (3, 112, "uniform", 64),
+                                            (16, 56, "uniform", 80), (12, 56, "mixed", 48)])
+def test_slab_weights_in_registers_form_on_large_tiles(ctx, n, hw, shifts, oc):
     """fused 3x3 layers with 64 input channels: one workgroup per CU walks a tile of several hundred pixels with the
     weights in registers; with one shift for all channels the requantisation of a pixel tile runs inside the K loop of
-    the next one, otherwise (mixed shifts) after its own"""
+    the next one, otherwise (mixed shifts) after its own.  From five pixel tiles per workgroup on the weight slab is
+    loaded through registers (32 and 16 images of 56 x 56, 3 of 112 x 112; with 80 and 48 output channels a channel block
+    of 16 and 48 weight rows, whose loads past the last row are clamped)"""
     rng = np.random.default_rng(n * hw)
     x = rng.integers(-128, 128, (n, hw, hw, 64)).astype(np.int8)
-    w = np.clip(np.rint(rng.normal(0, 30, (64, 3, 3, 64))), -127, 127).astype(np.int8)
-    bias = np.rint(rng.normal(0, 1 << 14, 64)).astype(np.int32)
-    mult = rng.integers(1 << 30, 1 << 31, 64).astype(np.int32)
-    shift = np.full(64, 38, np.int8) if shifts == "uniform" else rng.integers(31, 41, 64).astype(np.int8)
+    w = np.clip(np.rint(rng.normal(0, 30, (oc, 3, 3, 64))), -127, 127).astype(np.int8)
+    bias = np.rint(rng.normal(0, 1 << 14, oc)).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    shift = np.full(oc, 38, np.int8) if shifts == "uniform" else rng.integers(31, 41, oc).astype(np.int8)
     c = dict(x=x, w=w, bias=bias, in_zp=-7, pad=(1, 1, 1, 1), stride=(1, 1), dilation=(1, 1), mult=mult, shift=shift,
              out_zp=2, clamp=(0, 127))
     got, st, want, wst = _fused(ctx, c, np.int8)
     assert ctx.last_kernel == "conv2d_slab_wreg_i8_rescale" and st == wst
     assert np.array_equal(got, want), int(np.count_nonzero(got != want))
-    if hw == 56 and n in (8, 32):
+    if hw == 56 and n in (8, 32) and oc == 64:
         assert ctx.last_launch_shape()[0] == 256    # one round of workgroups: 7 x 14 and 7 x 56 pixels each
 
 
