@@ -449,20 +449,22 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (ctx->kernel_choice == 0 && !rp.enabled && g.KH * g.KW == 1 && total > (int64_t(1) << 21))
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
                                     pad_page, ctx->flags_dev);
-        // Tiny int8 layers: the patch kernel's set-up (4.4 us for a layer of one workgroup, 1.8 more with the fused
-        // RESCALE and 1.8 more when the channel vector is not made of 16-byte chunks) exceeds what the one-result-per-lane
-        // kernel takes, 2.6 us plus the longer of a lane's chain of K multiply-adds (90 ns each) and the whole layer at
-        // 1000 multiply-adds per ns.  us patch kernel / direct kernel (graph replays, fused): [1,32,32,8]->16 1x1 8.0 / 3.05,
-        // [1,64,64,8]->16 8.1 / 3.1, [8,32,32,8]->32 6.5 / 4.2, [1,32,32,16]->16 6.2 / 3.7, 3x3 [1,32,32,3]->16 7.7 / 5.1,
-        // [1,112,112,3]->32 stride 2 6.7 / 5.7; the other way: [1,14,14,8]->16 3x3 8.0 / 8.5, [1,224,224,3]->32 stride 2
-        // 7.6 / 12.0, [8,56,56,8]->64 1x1 6.7 / 12.9, [1,56,56,24]->144 8.3 / 10.1.
+        // Tiny int8 layers: the patch kernel's set-up (4.4 us for a layer of a few workgroups, 1.8 more with the fused
+        // RESCALE, 0.5 more when the channel vector is staged by 4- or 8-byte words and 1.8 when by bytes) exceeds what
+        // the one-result-per-lane kernel takes, 2.6 us plus the longer of a lane's chain of K multiply-adds (90 ns each)
+        // and the whole layer at 1000 multiply-adds per ns.  us patch kernel / direct kernel (graph replays, fused):
+        // [1,32,32,8]->16 1x1 6.6 / 3.1, [1,64,64,8]->16 6.7 / 3.2, [8,32,32,8]->32 5.1 / 4.2, [1,32,32,16]->16 6.2 / 3.7,
+        // [4,16,16,24]->48 6.5 / 4.2, 3x3 [1,32,32,3]->16 7.7 / 5.1, [1,112,112,3]->32 stride 2 6.9 / 5.8, int32 results
+        // [2,32,32,8]->16 4.7 / 2.8, [1,32,32,16]->16 4.4 / 3.4; the other way: 3x3 [1,14,14,8]->16 6.7 / 8.5,
+        // [1,28,28,12]->32 5.3 / 11.5, [1,224,224,3]->32 stride 2 7.7 / 11.9, 1x1 [8,56,56,8]->64 5.4 / 12.8,
+        // [1,56,56,24]->144 6.3 / 9.9.
         if (ctx->kernel_choice == 0 && d->in_dtype == TMI_INT8)
         {
             const double k      = (double)g.KH * g.KW * g.IC;
-            const double chain  = 0.09 * k, whole = (double)total * k / 1000.0 * 1e-3;
+            const double chain  = 0.09 * k, whole = (double)total * k * 1e-6;
             const double direct = 2.6 + (chain > whole ? chain : whole);
-            const double patch  = 4.4 + ((g.IC & 15) ? 1.8 : 0.0) + (rp.enabled ? 1.8 : 0.0);
-            if (direct + 0.8 < patch)
+            const double patch  = 4.4 + ((g.IC & 15) == 0 ? 0.0 : ((g.IC & 3) == 0 ? 0.5 : 1.8)) + (rp.enabled ? 1.8 : 0.0);
+            if (direct + 0.3 < patch)
                 name = launch_conv2d_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                             ctx->flags_dev);
         }

@@ -51,6 +51,24 @@ def test_conv2d_i8_mfma_bit_exact(ctx, shape, zps):
     assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
 
 
+@pytest.mark.parametrize("ic", [6, 12, 20, 40, 72, 104, 200])
+@pytest.mark.parametrize("taps,stride", [(1, 1), (3, 1), (3, 2)])
+def test_conv2d_i8_channel_vectors_of_words(ctx, ic, taps, stride):
+    """channel vectors that are not whole 16-byte chunks are staged by 8-byte words (40, 72, 104, 200 channels), 4-byte
+    words (12, 20) or bytes (6), over one channel block or several (72 and more)"""
+    rng = np.random.default_rng(ic * 10 + taps + stride)
+    pad = (taps // 2,) * 4
+    x = rng.integers(-128, 128, (2, 11, 13, ic)).astype(np.int8)
+    w = rng.integers(-128, 128, (24, taps, taps, ic)).astype(np.int8)
+    bias = rng.integers(-65536, 65536, 24).astype(np.int32)
+    oh, ow = (11 + 2 * pad[0] - taps) // stride + 1, (13 + 2 * pad[0] - taps) // stride + 1
+    x = x[:, :(oh - 1) * stride + taps - 2 * pad[0], :(ow - 1) * stride + taps - 2 * pad[0]]
+    want = oracle.conv2d("i8", x, w, bias, pad, (stride, stride), (1, 1), in_zp=-5, w_zp=2)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, (stride, stride), (1, 1), in_zp=-5, w_zp=2)
+    assert ctx.last_kernel == "conv2d_mfma_i8"
+    assert st == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+
+
 @pytest.mark.parametrize("shape", MFMA_SHAPES[5:9])
 def test_conv2d_i8_mfma_broadcast_bias(ctx, shape):
     n, ih, iw, ic, oc, kh, kw, pad, stride, dil = shape
@@ -196,6 +214,33 @@ def test_conv2d_fp_mfma_within_dot_product_bound(ctx, kind, shape):
     # tolerance: |imp-ref| <= 2*ksb * max(bnd*2^-(1+frac), normal_min) per element, sum err^2 <= 1.6*ksb*T
     assert st == capi.VALID and res["ok"], res
     assert res["max_ulp"] <= 2.0, res  # fp32 accumulation: the result is the correctly rounded value +- 1 ulp
+
+
+@pytest.mark.parametrize("kind", ["fp16", "bf16"])
+@pytest.mark.parametrize("ic", [3, 6, 10, 20, 36])
+def test_conv2d_fp_channel_vectors_of_words(ctx, kind, ic):
+    """16-bit channel vectors of 6 bytes (staged by bytes), 12 and 20 (4-byte words), 40 and 72 (8-byte words)"""
+    rng = np.random.default_rng(900 + ic)
+    pad, stride, dil = (1, 1, 1, 1), (1, 1), (1, 1)
+    x = rng.normal(0, 1, (2, 9, 10, ic)).astype(np.float32)
+    w = rng.normal(0, 1 / np.sqrt(9 * ic), (20, 3, 3, ic)).astype(np.float32)
+    b = rng.normal(0, 0.1, 20).astype(np.float32)
+    if kind == "fp16":
+        xs, ws, bs = x.astype(np.float16), w.astype(np.float16), b.astype(np.float16)
+        xf, wf, bf = (v.astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.FP16
+    else:
+        xs, ws, bs = (cases.float_to_bf16_bits(v) for v in (x, w, b))
+        xf, wf, bf = (cases.bf16_bits_to_float(v).astype(np.float64) for v in (xs, ws, bs))
+        dtype = capi.BF16
+    ref = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil)
+    bnd = oracle.conv2d("f64", xf, wf, bf, pad, stride, dil, abs_mode=True)
+    got, st = gpu_ops.conv2d(ctx, xs, ws, bs, pad, stride, dil, dtype=dtype)
+    assert ctx.last_kernel == ("conv2d_mfma_f16" if kind == "fp16" else "conv2d_mfma_bf16")
+    imp = got.astype(np.float64) if kind == "fp16" else cases.bf16_bits_to_float(got).astype(np.float64)
+    res = dp.check(imp, ref, bnd, kind, dp.kernel_size_bound(9 * ic, kind))
+    # tolerance: the DOT_PRODUCT bound of the reference's verifier, and at most 2 ulp of the output type
+    assert st == capi.VALID and res["ok"] and res["max_ulp"] <= 2.0, res
 
 
 # ---- GEMM-sized work: the 128-channel x 256-pixel workgroup shape and pipelined channel blocks ---------------
