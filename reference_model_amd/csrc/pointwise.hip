@@ -1,0 +1,351 @@
+// Pointwise (1x1, unit stride, no padding) int8 CONV2D with few input channels, with or without the fused RESCALE
+// (+ CLAMP): the layers of MobileNet-like networks that expand or project 16 ... 160 channels.
+//
+//   out[p][oc] = sum_ic (in[p][ic] - input_zp) * w[oc][ic] + bias[oc]      (tensor_ops.cpp:843-882 with one tap)
+//
+// Such a layer moves more bytes than it multiplies, and a workgroup that stages operands in LDS and meets at barriers
+// spends its time on that set-up.  Here nothing is staged and no wave waits for another: a wave owns one tile of 32
+// output channels for its whole life.  It fetches its weight fragments (K steps x 16 bytes per lane) straight from global
+// memory into the registers the matrix instruction reads, derives sum(w) from them (dot products with a word of ones),
+// builds the 32 channels' RESCALE constants in a wave-private piece of LDS, and then walks pixel tiles of 32: the pixel
+// fragments come straight from global memory as well (a lane reads 16 bytes of its pixel's channel vector; two tiles
+// ahead are in flight), K steps of v_mfma_i32_32x32x32_i8 start from
+// bias - input_zp * sum(w), and a lane requantises and stores the 16 consecutive channels of one pixel it ends up with.
+// Waves that share pixel tiles (the channel tiles of one pixel tile) are neighbours in a workgroup, so the pixel bytes
+// they all read come from HBM once.
+//
+// weight_zp must be 0 (the usual case for int8 weights); IC is a multiple of 8 from 16 to 160 and OC a multiple of 8.  The
+// K bytes past IC (the rest of the last K step of 32) are zeros in the weight fragments, so whatever the pixel fragment
+// holds there contributes nothing.
+#include <type_traits>
+
+#include "tmi_mfma.h"
+
+namespace tmi
+{
+
+struct PointwiseArgs
+{
+    const uint8_t* in;
+    const int8_t* w;
+    const int32_t* bias;
+    void* out;
+    uint32_t* flag_word;
+    RescaleParams rp;
+    int32_t P, IC, OC;    // pixels (N * OH * OW), input and output channels
+    int32_t za, bias_len;
+    int32_t out_kind;    // 0: int32 accumulators, 1: int8 through the RESCALE, 2: int16 through the RESCALE
+    int32_t n_oct;       // channel tiles of 32
+    int32_t n_pt;        // pixel tiles of 32
+    int32_t n_groups;    // groups of n_oct waves; group q takes the pixel tiles q, q + n_groups, ...
+    FastDiv div_oct;
+};
+
+constexpr int kPointwiseWaves   = 4;
+constexpr int kPointwiseWaveLds = 32 * (int)sizeof(HighWordScale) + 32 * 8 + 32 * 4;
+
+// apply_scale_32 + output_zp + clip (+ CLAMP) from the multiplier and the (validated) shift alone: fast_rescale() with
+// its per-channel constants worked out on the spot, for the channel tiles whose shifts rule out the high-word form.  Few
+// registers matter more here than few instructions.
+__device__ __forceinline__ int32_t rescale_from_shift(int32_t v, int32_t m, int32_t s, bool double_round, int32_t out_zp,
+                                                      int32_t lo, int32_t hi, uint32_t& flags)
+{
+    if (s <= 31)
+    {
+        const int32_t high = 1 << (s - 1);
+        if (v < -high || v >= high)
+            flags |= TMI_FLAG_SCALE_VALUE;
+    }
+    int64_t round = int64_t(1) << (s - 1);
+    if (double_round && s > 31)
+        round += v >= 0 ? (int64_t(1) << 30) : -(int64_t(1) << 30);
+    const int64_t p = (int64_t)v * (int64_t)m + round;
+    int32_t r       = (int32_t)(p >> s) + out_zp;
+    r               = r < lo ? lo : r;
+    return r > hi ? hi : r;
+}
+
+template <int KSTEPS, bool ZA>
+__global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void pointwise_i8_kernel(PointwiseArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kPointwiseWaves][kPointwiseWaveLds];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const uint32_t g = blockIdx.x * kPointwiseWaves + wave;
+    if (g >= (uint32_t)(a.n_groups * a.n_oct))
+        return;
+    const int q = (int)fdiv(g, a.div_oct), oct = (int)g - q * a.n_oct;
+    const int G = a.n_groups;
+    HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(lds[wave]);
+    v2i* tab_ms           = reinterpret_cast<v2i*>(tab_hw + 32);    // multiplier and validated shift
+    int32_t* wave_start   = reinterpret_cast<int32_t*>(tab_ms + 32);
+
+    // ---- pixel fragments: lane (li, lh) holds bytes [32 s + 16 lh, + 16) of pixel 32 pt + li ---------------------------
+    // (channel vectors of whole 16-byte chunks, or of 8-byte pieces: 24, 40, 56 ... channels, fetched 8 bytes at a time)
+    const bool by8 = (a.IC & 8) != 0;
+    auto load_pixels = [&](v4i (&fb)[KSTEPS], int pt) {
+        int p = pt * 32 + li;
+        p     = p < a.P ? p : a.P - 1;    // a pixel past the end: the last one again, never stored
+        const uint8_t* row = a.in + (size_t)p * a.IC;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++)
+        {
+            const int k0 = 32 * s + 16 * lh;
+            if (!by8)
+                fb[s] = *reinterpret_cast<const v4i*>(row + (k0 < a.IC ? k0 : 0));    // past IC: any bytes, times zero weights
+            else
+            {
+                const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
+                const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
+                fb[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
+            }
+        }
+    };
+    v4i fb0[KSTEPS], fb1[KSTEPS];
+    load_pixels(fb0, q);
+    if (q + G < a.n_pt)
+        load_pixels(fb1, q + G);
+
+    // ---- weight fragments: MFMA operand row li is channel 16 * ((li >> 2) & 1) + 4 * (li >> 3) + (li & 3) of the tile, so
+    // that a lane's 16 accumulators are 16 consecutive channels of its pixel -------------------------------------------
+    const int wr = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
+    const int ch = oct * 32 + wr;
+    v4i fa[KSTEPS];
+    {
+        const int8_t* row = a.w + (size_t)(ch < a.OC ? ch : a.OC - 1) * a.IC;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++)
+        {
+            const int k0 = 32 * s + 16 * lh;
+            const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
+            const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
+            const bool r = ch < a.OC;
+            fa[s]        = v4i{ r && k0 < a.IC ? lo.x : 0, r && k0 < a.IC ? lo.y : 0, r && k0 + 8 < a.IC ? hi.x : 0,
+                         r && k0 + 8 < a.IC ? hi.y : 0 };
+        }
+    }
+    // ---- per-channel constants: lane li (both halves alike) derives those of channel 32 oct + li ------------------------
+    uint32_t flags = 0;
+    int form       = 0;    // 1: every channel of the tile takes the high-word form of the requantisation
+    {
+        const int oc  = oct * 32 + li;
+        const bool ok = oc < a.OC;
+        const int occ = ok ? oc : oct * 32;
+        int32_t b     = a.bias[a.bias_len == 1 ? 0 : (ch < a.OC ? ch : oct * 32)];    // of the row this lane holds weights of
+        if (a.rp.enabled)
+        {
+            const int32_t m_raw   = load_multiplier(a.rp, occ);
+            const int32_t s_raw   = load_shift(a.rp, occ);
+            const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
+            const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
+            const int s_min       = a.rp.double_round ? 33 : 32;
+            form                  = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0;
+            if (lh == 0)
+            {
+                tab_ms[li] = v2i{ cs.m, cs.s };
+                tab_hw[li] = make_high_word_scale(cs, a.rp.out_zp);
+            }
+        }
+        if constexpr (ZA)
+        {
+            int sum = 0;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+                sum += dot4_ones(fa[s]);
+            sum += __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, sum);
+            b = (int32_t)((uint32_t)b - (uint32_t)a.za * (uint32_t)sum);
+        }
+        if (lh == 0)
+            wave_start[wr] = ch < a.OC ? b : 0;
+        __builtin_amdgcn_wave_barrier();    // the wave's own LDS accesses complete in order
+    }
+    v16i start;
+#pragma unroll
+    for (int gq = 0; gq < 4; gq++)
+    {
+        const v4i b4 = *reinterpret_cast<const v4i*>(wave_start + 16 * lh + 4 * gq);
+        start[4 * gq] = b4[0], start[4 * gq + 1] = b4[1], start[4 * gq + 2] = b4[2], start[4 * gq + 3] = b4[3];
+    }
+    const int oc_lane = oct * 32 + 16 * lh;                        // first of the lane's 16 channels
+    int cnt           = a.OC - oc_lane;                            // how many of them exist: 16, 8 or none (OC is a multiple of 8)
+    cnt               = cnt < 0 ? 0 : (cnt > 16 ? 16 : cnt);
+    const bool whole  = (a.OC & 15) == 0;                          // int8 rows of whole 16-byte pieces
+    const int32_t v_lo = a.rp.lo, v_hi = a.rp.hi;
+
+    // FORM 0: int32 results; 1: the high-word requantisation; 2: the general form
+    auto run = [&](auto FORM, auto DOUBLE) {
+        constexpr int kForm    = decltype(FORM)::value;
+        constexpr bool kDouble = decltype(DOUBLE)::value;
+        auto tile = [&](const v4i (&fb)[KSTEPS], int pt) {
+            // The constants of the lane's 16 channels are read from the wave's table for every tile (32 lanes read one
+            // address: four LDS cycles a read) rather than held in 64 registers, which would halve the waves a SIMD holds;
+            // the offset is hidden from the compiler so that it does not move the reads out of the loop over the tiles.
+            int first = 16 * lh;
+            asm volatile("" : "+v"(first));
+            const HighWordScale* hw = tab_hw + first;
+            const v2i* ms           = tab_ms + first;
+            v16i acc = start;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
+            const int p      = pt * 32 + li;
+            const bool store = p < a.P && cnt > 0;
+            const size_t at  = (size_t)(p < a.P ? p : 0) * a.OC + oc_lane;
+            if constexpr (kForm == 0)
+            {
+                int32_t* o = reinterpret_cast<int32_t*>(a.out) + at;
+                if (store)
+                {
+#pragma unroll
+                    for (int gq = 0; gq < 4; gq++)
+                        if (4 * gq < cnt)
+                            *reinterpret_cast<v4i*>(o + 4 * gq) = v4i{ acc[4 * gq], acc[4 * gq + 1], acc[4 * gq + 2], acc[4 * gq + 3] };
+                }
+                return;
+            }
+            int32_t r[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+            {
+                if constexpr (kForm == 1)
+                    r[e] = clamp_med3(high_word_rescale64<kDouble>(acc[e], hw[e]), v_lo, v_hi);
+                else
+                {
+                    // (elements that are not stored raise nothing)
+                    uint32_t f = 0;
+                    const v2i c = ms[e];
+                    r[e]        = rescale_from_shift(acc[e], c.x, c.y, a.rp.double_round != 0, a.rp.out_zp, v_lo, v_hi, f);
+                    flags |= (store && e < cnt) ? f : 0u;
+                }
+                if ((e & 3) == 3)
+                    __builtin_amdgcn_sched_barrier(0);    // four elements' constants at a time: the registers are few
+            }
+            if (a.out_kind == 1)
+            {
+                v4i pk;
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++)
+                {
+                    const int lo2 = __builtin_amdgcn_perm(r[4 * gq + 1], r[4 * gq], 0x0c0c0400);
+                    const int hi2 = __builtin_amdgcn_perm(r[4 * gq + 3], r[4 * gq + 2], 0x04000c0c);
+                    pk[gq]        = lo2 | hi2;
+                }
+                int8_t* o = reinterpret_cast<int8_t*>(a.out) + at;
+                if (store)
+                {
+                    if (whole)
+                        *reinterpret_cast<v4i*>(o) = pk;
+                    else
+                    {
+                        *reinterpret_cast<v2i*>(o) = v2i{ pk[0], pk[1] };
+                        if (cnt > 8)
+                            *reinterpret_cast<v2i*>(o + 8) = v2i{ pk[2], pk[3] };
+                    }
+                }
+            }
+            else
+            {
+                v4i pk, pk2;
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++)
+                {
+                    pk[gq]  = (r[2 * gq] & 0xffff) | ((r[2 * gq + 1] & 0xffff) << 16);
+                    pk2[gq] = (r[8 + 2 * gq] & 0xffff) | ((r[8 + 2 * gq + 1] & 0xffff) << 16);
+                }
+                int16_t* o = reinterpret_cast<int16_t*>(a.out) + at;
+                if (store)
+                {
+                    *reinterpret_cast<v4i*>(o) = pk;
+                    if (cnt > 8)
+                        *reinterpret_cast<v4i*>(o + 8) = pk2;
+                }
+            }
+        };
+        // two pixel tiles are in flight while one is multiplied
+        for (int pt = q; pt < a.n_pt; pt += 2 * G)
+        {
+            tile(fb0, pt);
+            if (pt + 2 * G < a.n_pt)
+                load_pixels(fb0, pt + 2 * G);
+            if (pt + G < a.n_pt)
+            {
+                tile(fb1, pt + G);
+                if (pt + 3 * G < a.n_pt)
+                    load_pixels(fb1, pt + 3 * G);
+            }
+        }
+    };
+    if (!a.rp.enabled)
+        run(std::integral_constant<int, 0>{}, std::false_type{});
+    else if (form == 1)
+        a.rp.double_round ? run(std::integral_constant<int, 1>{}, std::true_type{})
+                          : run(std::integral_constant<int, 1>{}, std::false_type{});
+    else
+        run(std::integral_constant<int, 2>{}, std::false_type{});
+    raise_flags(a.flag_word, flags);
+}
+
+template <int KSTEPS>
+static bool launch_pointwise(hipStream_t st, const PointwiseArgs& a, int grid)
+{
+    if (a.za != 0)
+        hipLaunchKernelGGL((pointwise_i8_kernel<KSTEPS, true>), dim3(grid), dim3(kPointwiseWaves * 64), 0, st, a);
+    else
+        hipLaunchKernelGGL((pointwise_i8_kernel<KSTEPS, false>), dim3(grid), dim3(kPointwiseWaves * 64), 0, st, a);
+    return true;
+}
+
+// nullptr when the layer is not one this kernel takes.
+const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                                    const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                                    void* out, uint32_t* flag_word)
+{
+    if (in_dtype != TMI_INT8 || g.KH != 1 || g.KW != 1 || g.stride_y != 1 || g.stride_x != 1 || g.pad_top != 0 ||
+        g.pad_left != 0 || g.OH != g.IH || g.OW != g.IW || w_zp != 0 || !flag_word)
+        return nullptr;
+    if ((g.IC & 7) || g.IC < 16 || g.IC > 160 || (g.OC & 7) || g.OC < 8 || g.OC > 4096)
+        return nullptr;
+    if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
+        return nullptr;
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out) & 15) || ((uintptr_t)bias & 3))
+        return nullptr;
+    const int64_t P = (int64_t)g.N * g.OH * g.OW;
+    if (P < 1 || P * g.IC >= (int64_t(1) << 31) || P * g.OC >= (int64_t(1) << 31))
+        return nullptr;
+
+    PointwiseArgs a{};
+    a.in = (const uint8_t*)in, a.w = (const int8_t*)w, a.bias = (const int32_t*)bias, a.out = out;
+    a.flag_word = flag_word, a.rp = rp;
+    a.P = (int32_t)P, a.IC = g.IC, a.OC = g.OC, a.za = in_zp, a.bias_len = g.bias_len;
+    a.out_kind = !rp.enabled ? 0 : (out_dtype == TMI_INT8 ? 1 : 2);
+    a.n_oct    = (g.OC + 31) / 32;
+    a.n_pt     = (int32_t)((P + 31) / 32);
+    // as many groups as there are pixel tiles, up to the waves the 256 CUs hold at once (12 each up to 64 input channels,
+    // 8 beyond: the fragments of two pixel tiles in flight take the registers)
+    const int per_cu     = g.IC <= 64 ? 12 : 8;
+    const int max_groups = 256 * per_cu / a.n_oct > 0 ? 256 * per_cu / a.n_oct : 1;
+    a.n_groups = a.n_pt < max_groups ? a.n_pt : max_groups;
+    a.div_oct  = make_fastdiv((uint32_t)a.n_oct);
+    const int64_t waves = (int64_t)a.n_groups * a.n_oct;
+    if (!fastdiv_exact_up_to((uint64_t)waves + kPointwiseWaves, (uint32_t)a.n_oct))
+        return nullptr;
+    const int grid   = (int)((waves + kPointwiseWaves - 1) / kPointwiseWaves);
+    const int ksteps = (g.IC + 31) / 32;
+    bool ok          = false;
+    switch (ksteps)
+    {
+        case 1: ok = launch_pointwise<1>(st, a, grid); break;
+        case 2: ok = launch_pointwise<2>(st, a, grid); break;
+        case 3: ok = launch_pointwise<3>(st, a, grid); break;
+        case 4: ok = launch_pointwise<4>(st, a, grid); break;
+        case 5: ok = launch_pointwise<5>(st, a, grid); break;
+        default: break;
+    }
+    if (!ok)
+        return nullptr;
+    last_launch_shape[0] = grid, last_launch_shape[1] = kPointwiseWaves * 64, last_launch_shape[2] = kPointwiseWaves * kPointwiseWaveLds;
+    return rp.enabled ? "conv2d_pointwise_i8_rescale" : "conv2d_pointwise_i8";
+}
+
+}    // namespace tmi

@@ -449,6 +449,19 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (ctx->kernel_choice == 0 && !rp.enabled && g.KH * g.KW == 1 && total > (int64_t(1) << 21))
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
                                     pad_page, ctx->flags_dev);
+        // Pointwise int8 layers with up to 112 input channels: the kernel that keeps a wave on one tile of 32 output channels
+        // and takes both operands straight from global memory, before every other (us slab or patch kernel / pointwise
+        // kernel, graph replays, fused RESCALE: [8,112,112,16]->96 16.6 / 6.4, [8,112,112,32]->16 9.0 / 3.4, [8,56,56,96]->24
+        // 7.5 / 2.8, [8,28,28,32]->192 4.9 / 2.9, [8,56,56,80]->80 10.0 / 3.8, [8,28,28,112]->224 6.3 / 3.7, [8,56,56,64]->64
+        // 3.5 / 3.3, [8,56,56,64]->256 6.4 / 5.5, [32,56,56,64]->256 18.0 / 12.6, [32,56,56,96]->192 16.4 / 11.3, [8,14,14,64]->384
+        // 3.3 / 2.8, [1,32,32,16]->16 3.7 (one result per lane) / 2.5; int32 results [8,56,56,96]->24 7.6 / 2.8, [8,112,112,16]->96
+        // 21.0 / 15.9, [8,56,56,64]->64 4.9 / 4.6).  With 128 input channels the slab kernel leads ([8,28,28,128]->512
+        // 4.9 / 6.0, [8,56,56,128]->128 5.1 / 6.1) and this kernel takes what that one declines; with 144 and 160 there is
+        // only the patch kernel to beat ([8,56,56,144]->24 10.2 / 3.1, [8,7,7,160]->960 5.4 / 3.2).  Large int32 results
+        // stay with the GEMM kernel above ([8,56,56,64]->256 8.1 / 11.8, [8,28,28,128]->512 6.3 / 8.9).
+        if (!name && ctx->kernel_choice == 0 && g.IC <= 112)
+            name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                           ctx->flags_dev);
         // Tiny int8 layers: the patch kernel's set-up (4.4 us for a layer of a few workgroups, 1.8 more with the fused
         // RESCALE, 0.5 more when the channel vector is staged by 4- or 8-byte words and 1.8 when by bytes) exceeds what
         // the one-result-per-lane kernel takes, 2.6 us plus the longer of a lane's chain of K multiply-adds (90 ns each)
@@ -458,7 +471,7 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // [2,32,32,8]->16 4.7 / 2.8, [1,32,32,16]->16 4.4 / 3.4; the other way: 3x3 [1,14,14,8]->16 6.7 / 8.5,
         // [1,28,28,12]->32 5.3 / 11.5, [1,224,224,3]->32 stride 2 7.7 / 11.9, 1x1 [8,56,56,8]->64 5.4 / 12.8,
         // [1,56,56,24]->144 6.3 / 9.9.
-        if (ctx->kernel_choice == 0 && d->in_dtype == TMI_INT8)
+        if (!name && ctx->kernel_choice == 0 && d->in_dtype == TMI_INT8)
         {
             const double k      = (double)g.KH * g.KW * g.IC;
             const double chain  = 0.09 * k, whole = (double)total * k * 1e-6;
@@ -471,6 +484,9 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (!name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
+        if (!name && (ctx->kernel_choice == 5 || ctx->kernel_choice == 0))    // (the layers it leads on were tried above)
+            name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                           ctx->flags_dev);
         if (!name && gemm_1st)
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
                                     pad_page, ctx->flags_dev);
@@ -634,7 +650,7 @@ int tmi_ctx_set_precise_mode(tmi_ctx_t* ctx, int32_t precise_mode, int32_t compl
 
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
-    if (!ctx || choice < 0 || choice > 4)
+    if (!ctx || choice < 0 || choice > 5)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;

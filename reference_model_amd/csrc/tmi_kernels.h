@@ -90,6 +90,12 @@ extern thread_local int32_t last_launch_shape[3];
 // a kernel without work: the cost of one launch of this grid, block and dynamic LDS size
 const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t lds_bytes);
 
+// pointwise.hip: int8 CONV2D 1x1 (unit stride, no padding) with 16 ... 160 input channels in multiples of 8 and
+// weight_zp 0; a wave per tile of 32 output channels, operands straight from global memory into registers
+const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                                    const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                                    void* out, uint32_t* flag_word);
+
 // direct.hip: one output element per lane, any legal shape.  out_dtype is the stored output type
 // (INT32 without rescale; the rescale output type with it; FP16/BF16/FP32 for floating point).
 const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,

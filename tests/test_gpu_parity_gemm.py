@@ -439,7 +439,11 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (16, 56, 56, 64, 128, 3, 1, 2), "conv2d_mfma_f16"),    # 98 tiles: the patch kernel
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_f16"),          # pointwise with two blocks of K
     (capi.INT8, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_i8"),           # int8 pointwise, int32 results, 6.4 M of them: before the slab kernel
-    (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_slab_i8"),          # the same with 1.6 M results: the slab kernel
+    (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_pointwise_i8"),     # the same with 1.6 M results: the pointwise kernel
+    (capi.INT8, (8, 28, 28, 128, 128, 1, 0), "conv2d_slab_i8"),        # 128 input channels: the slab kernel
+    (capi.INT8, (8, 28, 28, 128, 24, 1, 0), "conv2d_pointwise_i8"),    # too few output channels for it: the pointwise kernel
+    (capi.INT8, (8, 56, 56, 16, 96, 1, 0), "conv2d_pointwise_i8"),     # int8 pointwise with a short channel vector
+    (capi.INT8, (8, 28, 28, 144, 32, 1, 0), "conv2d_pointwise_i8"),    # 144 input channels: no slab kernel
 ])
 def test_automatic_kernel_choice(dtype, shape, kernel):
     n, ih, iw, ic, oc, k, pad = shape[:7]
@@ -459,7 +463,7 @@ def test_automatic_kernel_choice(dtype, shape, kernel):
         got, st = gpu_ops.conv2d(c, x, w, b, pads, (stride, stride), dtype=dtype)
         assert st == capi.VALID and c.last_kernel == kernel
         # the kernel not chosen, where it takes the shape at all
-        c.set_kernel_choice(capi.KERNEL_GEMM if kernel.startswith("conv2d") else capi.KERNEL_MFMA)
+        c.set_kernel_choice(capi.KERNEL_GEMM if kernel.startswith("conv2d") and "pointwise" not in kernel else capi.KERNEL_MFMA)
         try:
             other, st = gpu_ops.conv2d(c, x, w, b, pads, (stride, stride), dtype=dtype)
         except TmiError:
