@@ -38,6 +38,7 @@ struct PointwiseArgs
     int32_t n_oct;       // channel tiles of 32
     int32_t n_pt;        // pixel tiles of 32
     int32_t n_groups;    // groups of n_oct waves; group q takes the pixel tiles q, q + n_groups, ...
+    int32_t ksw;         // the form that splits K over a workgroup's waves: K steps per wave
     FastDiv div_oct;
 };
 
@@ -286,6 +287,202 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
     raise_flags(a.flag_word, flags);
 }
 
+// The same layers with long channel vectors (up to 2048 input channels): the four waves of a workgroup share one tile of
+// 32 output channels x 32 pixels and split K between them, a quarter each, again with both operands straight from global
+// memory into registers - all loads of a tile are in flight at once, so a tile costs one trip to memory however deep K is.
+// Each wave's accumulators start from its share of bias - input_zp * sum(w) (the bias with the first wave); the four
+// partial tiles meet in LDS (16 KB, two buffers, one barrier per tile), and every wave requantises and stores a quarter of
+// the tile: 4 consecutive channels per lane.  What a projection layer of a small image offers is few tiles and a long
+// reduction (8 x 7 x 7 pixels x 512 channels over K = 2048: 208 tiles of 64 K steps), which this form spreads over 832
+// waves where a 128 x 128 GEMM tile would keep 32 CUs busy.
+constexpr int kSplitWaves = 4;
+
+template <int KS, bool ZA>
+__global__ __launch_bounds__(kSplitWaves * 64, 2) void pointwise_ksplit_i8_kernel(PointwiseArgs a)
+{
+    // [two buffers x 4 waves x 4 quarters x 64 lanes x 16 bytes][32 x HighWordScale][32 x (m, s)][4 waves x 32 start values][form]
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * 16384 + 32 * 16 + 32 * 8 + kSplitWaves * 128 + 16];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const uint32_t g = blockIdx.x;
+    const int q = (int)fdiv(g, a.div_oct), oct = (int)g - q * a.n_oct;
+    const int G = a.n_groups;
+    HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(lds + 2 * 16384);
+    v2i* tab_ms           = reinterpret_cast<v2i*>(tab_hw + 32);
+    int32_t* wave_start   = reinterpret_cast<int32_t*>(tab_ms + 32) + wave * 32;
+    int32_t* form_word    = reinterpret_cast<int32_t*>(tab_ms + 32) + kSplitWaves * 32;
+    const int ksw = a.ksw;                     // K steps of a wave's share (at most KS)
+    const int kbase = wave * ksw * 32;         // first K byte of the share
+    const bool by8 = (a.IC & 8) != 0;
+
+    auto load_pixels = [&](v4i (&fb)[KS], int pt) {
+        int p = pt * 32 + li;
+        p     = p < a.P ? p : a.P - 1;
+        const uint8_t* row = a.in + (size_t)p * a.IC;
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+        {
+            const int k0 = kbase + 32 * s + 16 * lh;
+            if (s < ksw)    // (a test per step, not a loop exit: the register array keeps constant indices)
+            {
+                if (!by8)
+                    fb[s] = *reinterpret_cast<const v4i*>(row + (k0 < a.IC ? k0 : 0));
+                else
+                {
+                    const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
+                    const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
+                    fb[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
+                }
+            }
+        }
+    };
+    v4i fb[KS];
+    load_pixels(fb, q);
+
+    const int wr = 4 * (li & 4) + ((li >> 1) & 12) + (li & 3);
+    const int ch = oct * 32 + wr;
+    v4i fa[KS];
+    {
+        const int8_t* row = a.w + (size_t)(ch < a.OC ? ch : a.OC - 1) * a.IC;
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+        {
+            const int k0 = kbase + 32 * s + 16 * lh;
+            if (s < ksw)
+            {
+                const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
+                const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
+                const bool r = ch < a.OC;
+                fa[s]        = v4i{ r && k0 < a.IC ? lo.x : 0, r && k0 < a.IC ? lo.y : 0, r && k0 + 8 < a.IC ? hi.x : 0,
+                             r && k0 + 8 < a.IC ? hi.y : 0 };
+            }
+        }
+    }
+    uint32_t flags = 0;
+    if (wave == 0)
+    {
+        // the first wave derives the constants of the tile's 32 channels for all four
+        const int oc  = oct * 32 + li;
+        const bool ok = oc < a.OC;
+        const int occ = ok ? oc : oct * 32;
+        if (a.rp.enabled)
+        {
+            const int32_t m_raw   = load_multiplier(a.rp, occ);
+            const int32_t s_raw   = load_shift(a.rp, occ);
+            const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
+            const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
+            const int s_min       = a.rp.double_round ? 33 : 32;
+            const int form        = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0;
+            if (lh == 0)
+            {
+                tab_ms[li] = v2i{ cs.m, cs.s };
+                tab_hw[li] = make_high_word_scale(cs, a.rp.out_zp);
+            }
+            if (lane == 0)
+                *form_word = form;
+        }
+    }
+    {
+        int32_t b = wave == 0 ? a.bias[a.bias_len == 1 ? 0 : (ch < a.OC ? ch : oct * 32)] : 0;
+        if constexpr (ZA)
+        {
+            int sum = 0;
+#pragma unroll
+            for (int s = 0; s < KS; s++)
+                if (s < ksw)
+                    sum += dot4_ones(fa[s]);
+            sum += __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, sum);
+            b = (int32_t)((uint32_t)b - (uint32_t)a.za * (uint32_t)sum);
+        }
+        if (lh == 0)
+            wave_start[wr] = ch < a.OC ? b : 0;
+        __builtin_amdgcn_wave_barrier();
+    }
+    v16i start;
+#pragma unroll
+    for (int gq = 0; gq < 4; gq++)
+    {
+        const v4i b4 = *reinterpret_cast<const v4i*>(wave_start + 16 * lh + 4 * gq);
+        start[4 * gq] = b4[0], start[4 * gq + 1] = b4[1], start[4 * gq + 2] = b4[2], start[4 * gq + 3] = b4[3];
+    }
+    const int oc_lane = oct * 32 + 16 * lh + 4 * wave;    // first of the 4 channels this lane requantises and stores
+    const bool ch_ok  = oc_lane < a.OC;                   // OC is a multiple of 8: the four are in or out together
+    const int32_t v_lo = a.rp.lo, v_hi = a.rp.hi;
+    int buf = 0;
+    for (int pt = q; pt < a.n_pt; pt += G)
+    {
+        v16i acc = start;
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+            if (s < ksw)
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
+        if (pt + G < a.n_pt)
+            load_pixels(fb, pt + G);    // in flight across the exchange and the requantisation
+        // the partial tiles meet in LDS: [wave][quarter][lane] of 16 bytes
+        uint8_t* red = lds + buf * 16384;
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++)
+            *reinterpret_cast<v4i*>(red + ((wave * 4 + gq) * 64 + lane) * 16) = v4i{ acc[4 * gq], acc[4 * gq + 1], acc[4 * gq + 2], acc[4 * gq + 3] };
+        __syncthreads();    // also publishes the first wave's tables
+        v4i sum = *reinterpret_cast<const v4i*>(red + ((0 * 4 + wave) * 64 + lane) * 16);
+#pragma unroll
+        for (int w2 = 1; w2 < kSplitWaves; w2++)
+        {
+            const v4i o = *reinterpret_cast<const v4i*>(red + ((w2 * 4 + wave) * 64 + lane) * 16);
+            sum.x += o.x, sum.y += o.y, sum.z += o.z, sum.w += o.w;
+        }
+        buf ^= 1;
+        const int p      = pt * 32 + li;
+        const bool store = p < a.P && ch_ok;
+        const size_t at  = (size_t)(p < a.P ? p : 0) * a.OC + (ch_ok ? oc_lane : 0);
+        if (a.out_kind == 0)
+        {
+            if (store)
+                *reinterpret_cast<v4i*>(reinterpret_cast<int32_t*>(a.out) + at) = sum;
+            continue;
+        }
+        const int form = *form_word;
+        int32_t r[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+        {
+            const int c = 16 * lh + 4 * wave + j;
+            if (form == 1)
+                r[j] = a.rp.double_round ? clamp_med3(high_word_rescale64<true>(sum[j], tab_hw[c]), v_lo, v_hi)
+                                         : clamp_med3(high_word_rescale64<false>(sum[j], tab_hw[c]), v_lo, v_hi);
+            else
+            {
+                uint32_t f   = 0;
+                const v2i ms = tab_ms[c];
+                r[j]         = rescale_from_shift(sum[j], ms.x, ms.y, a.rp.double_round != 0, a.rp.out_zp, v_lo, v_hi, f);
+                flags |= store ? f : 0u;
+            }
+        }
+        if (a.out_kind == 1)
+        {
+            const int lo2 = __builtin_amdgcn_perm(r[1], r[0], 0x0c0c0400);
+            const int hi2 = __builtin_amdgcn_perm(r[3], r[2], 0x04000c0c);
+            if (store)
+                *reinterpret_cast<int*>(reinterpret_cast<int8_t*>(a.out) + at) = lo2 | hi2;
+        }
+        else if (store)
+            *reinterpret_cast<v2i*>(reinterpret_cast<int16_t*>(a.out) + at) =
+                v2i{ (r[0] & 0xffff) | ((r[1] & 0xffff) << 16), (r[2] & 0xffff) | ((r[3] & 0xffff) << 16) };
+    }
+    raise_flags(a.flag_word, flags);
+}
+
+template <int KS>
+static bool launch_pointwise_ksplit(hipStream_t st, const PointwiseArgs& a, int grid)
+{
+    if (a.za != 0)
+        hipLaunchKernelGGL((pointwise_ksplit_i8_kernel<KS, true>), dim3(grid), dim3(kSplitWaves * 64), 0, st, a);
+    else
+        hipLaunchKernelGGL((pointwise_ksplit_i8_kernel<KS, false>), dim3(grid), dim3(kSplitWaves * 64), 0, st, a);
+    return true;
+}
+
 template <int KSTEPS>
 static bool launch_pointwise(hipStream_t st, const PointwiseArgs& a, int grid)
 {
@@ -304,7 +501,7 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
     if (in_dtype != TMI_INT8 || g.KH != 1 || g.KW != 1 || g.stride_y != 1 || g.stride_x != 1 || g.pad_top != 0 ||
         g.pad_left != 0 || g.OH != g.IH || g.OW != g.IW || w_zp != 0 || !flag_word)
         return nullptr;
-    if ((g.IC & 7) || g.IC < 16 || g.IC > 160 || (g.OC & 7) || g.OC < 8 || g.OC > 4096)
+    if ((g.IC & 7) || g.IC < 16 || g.IC > 2048 || (g.OC & 7) || g.OC < 8 || g.OC > 4096)
         return nullptr;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
         return nullptr;
@@ -321,12 +518,33 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
     a.out_kind = !rp.enabled ? 0 : (out_dtype == TMI_INT8 ? 1 : 2);
     a.n_oct    = (g.OC + 31) / 32;
     a.n_pt     = (int32_t)((P + 31) / 32);
+    a.div_oct  = make_fastdiv((uint32_t)a.n_oct);
+    if (g.IC > 160)
+    {
+        // K split over the four waves of a workgroup; a workgroup per tile up to 8 workgroups on each CU
+        const int ksteps = (g.IC + 31) / 32;
+        a.ksw            = (ksteps + kSplitWaves - 1) / kSplitWaves;
+        const int max_groups = 2048 / a.n_oct > 0 ? 2048 / a.n_oct : 1;
+        a.n_groups       = a.n_pt < max_groups ? a.n_pt : max_groups;
+        const int grid   = a.n_groups * a.n_oct;
+        if (!fastdiv_exact_up_to((uint64_t)grid, (uint32_t)a.n_oct))
+            return nullptr;
+        if (a.ksw <= 2)
+            launch_pointwise_ksplit<2>(st, a, grid);
+        else if (a.ksw <= 4)
+            launch_pointwise_ksplit<4>(st, a, grid);
+        else if (a.ksw <= 8)
+            launch_pointwise_ksplit<8>(st, a, grid);
+        else
+            launch_pointwise_ksplit<16>(st, a, grid);
+        last_launch_shape[0] = grid, last_launch_shape[1] = kSplitWaves * 64, last_launch_shape[2] = 34064;
+        return rp.enabled ? "conv2d_pointwise_ksplit_i8_rescale" : "conv2d_pointwise_ksplit_i8";
+    }
     // as many groups as there are pixel tiles, up to the waves the 256 CUs hold at once (12 each up to 64 input channels,
     // 8 beyond: the fragments of two pixel tiles in flight take the registers)
     const int per_cu     = g.IC <= 64 ? 12 : 8;
     const int max_groups = 256 * per_cu / a.n_oct > 0 ? 256 * per_cu / a.n_oct : 1;
     a.n_groups = a.n_pt < max_groups ? a.n_pt : max_groups;
-    a.div_oct  = make_fastdiv((uint32_t)a.n_oct);
     const int64_t waves = (int64_t)a.n_groups * a.n_oct;
     if (!fastdiv_exact_up_to((uint64_t)waves + kPointwiseWaves, (uint32_t)a.n_oct))
         return nullptr;

@@ -459,7 +459,18 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // 4.9 / 6.0, [8,56,56,128]->128 5.1 / 6.1) and this kernel takes what that one declines; with 144 and 160 there is
         // only the patch kernel to beat ([8,56,56,144]->24 10.2 / 3.1, [8,7,7,160]->960 5.4 / 3.2).  Large int32 results
         // stay with the GEMM kernel above ([8,56,56,64]->256 8.1 / 11.8, [8,28,28,128]->512 6.3 / 8.9).
-        if (!name && ctx->kernel_choice == 0 && g.IC <= 112)
+        // With more than 160 input channels the pointwise kernel splits K over the four waves of a workgroup, one workgroup
+        // per tile of 32 x 32 results: the better form while the layer is small (at most 450 M multiply-adds) and the GEMM
+        // kernel would have few tiles of 128 x 128 for the chip, or does not take the layer (fewer than 64 output channels,
+        // channel vectors that are not multiples of 64 bytes).  us GEMM or patch kernel / this form, fused RESCALE:
+        // [8,28,28,192]->32 9.2 / 3.2, [8,14,14,384]->64 7.4 / 3.9, [8,14,14,576]->96 8.2 / 4.3, [8,7,7,960]->320 9.7 / 4.8,
+        // [8,7,7,320]->1280 7.4 / 4.6, [8,14,14,1024]->256 (26 tiles) 10.1 / 8.4, [8,7,7,2048]->512 (16) 14.2 / 8.8; ties at
+        // [8,28,28,512]->128 (49 tiles) 8.1 / 8.4 and [8,7,7,512]->2048 (64) 8.1 / 8.2; the other way: [8,56,56,256]->64 (196)
+        // 7.4 / 10.0, [8,14,14,256]->1024 (104) 7.2 / 9.9, [8,56,56,256]->128 7.6 / 13.2, [8,14,14,1024]->512 10.1 / 15.2.
+        const int64_t pixels   = (int64_t)g.N * g.OH * g.OW;
+        const int64_t tiles128 = ((pixels + 127) / 128) * ((g.OC + 127) / 128);
+        const bool deep_first  = g.IC > 160 && total * g.IC <= 450000000ll && (tiles128 <= 48 || g.OC < 64 || (g.IC & 63));
+        if (!name && ctx->kernel_choice == 0 && (g.IC <= 112 || deep_first))
             name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                            ctx->flags_dev);
         // Tiny int8 layers: the patch kernel's set-up (4.4 us for a layer of a few workgroups, 1.8 more with the fused
@@ -484,7 +495,7 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (!name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
-        if (!name && (ctx->kernel_choice == 5 || ctx->kernel_choice == 0))    // (the layers it leads on were tried above)
+        if (!name && (ctx->kernel_choice == 5 || (ctx->kernel_choice == 0 && g.IC <= 160)))    // (the layers it leads on were tried above)
             name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                            ctx->flags_dev);
         if (!name && gemm_1st)

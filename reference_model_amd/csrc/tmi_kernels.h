@@ -90,8 +90,9 @@ extern thread_local int32_t last_launch_shape[3];
 // a kernel without work: the cost of one launch of this grid, block and dynamic LDS size
 const char* launch_empty(hipStream_t st, int32_t grid, int32_t block, int32_t lds_bytes);
 
-// pointwise.hip: int8 CONV2D 1x1 (unit stride, no padding) with 16 ... 160 input channels in multiples of 8 and
-// weight_zp 0; a wave per tile of 32 output channels, operands straight from global memory into registers
+// pointwise.hip: int8 CONV2D 1x1 (unit stride, no padding) with 16 ... 2048 input channels in multiples of 8 and
+// weight_zp 0; a wave per tile of 32 output channels (from 168 input channels on: four waves that split K), operands
+// straight from global memory into registers
 const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                     const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                     void* out, uint32_t* flag_word);

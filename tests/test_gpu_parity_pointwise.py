@@ -1,10 +1,12 @@
-"""The int8 pointwise kernel (CONV2D 1x1, unit stride, 16 ... 160 input channels in multiples of 8) through the C ABI, bit
-for bit against the CPU oracle (tensor_ops.cpp:843-882 with one tap, then type_conversion.cpp:224-421): every number of K
-steps, channel tiles that are ragged by 8 or 16 channels, pixel counts either side of a tile of 32, all three result types,
-the three forms of its requantisation and the REQUIRE conditions of apply_scale_32."""
+"""The int8 pointwise kernels (CONV2D 1x1, unit stride, 16 ... 2048 input channels in multiples of 8; from 168 on the form
+that splits K over the waves of a workgroup) through the C ABI, bit for bit against the CPU oracle (tensor_ops.cpp:843-882
+with one tap, then type_conversion.cpp:224-421): every number of K steps, channel tiles that are ragged by 8 or 16
+channels, pixel counts either side of a tile of 32, all three result types, the forms of the requantisation and the
+REQUIRE conditions of apply_scale_32."""
 import numpy as np
 import pytest
 
+import cases
 import gpu_ops
 import oracle
 from reference_model_amd import Context, TmiError, capi
@@ -112,7 +114,7 @@ def test_pointwise_broadcast_bias_and_per_tensor_scale(ctx):
 
 def test_pointwise_declines_what_it_does_not_take(ctx):
     rng = np.random.default_rng(9)
-    for shape, kw in [((1, 4, 4, 20, 16), {}), ((1, 4, 4, 8, 16), {}), ((1, 4, 4, 176, 16), {}), ((1, 4, 4, 32, 12), {}), ((1, 4, 4, 32, 16), dict(w_zp=1))]:
+    for shape, kw in [((1, 4, 4, 20, 16), {}), ((1, 4, 4, 8, 16), {}), ((1, 4, 4, 2056, 16), {}), ((1, 4, 4, 32, 12), {}), ((1, 4, 4, 32, 16), dict(w_zp=1))]:
         n, h, w, ic, oc = shape
         x, wt, bias = _operands(rng, n, h, w, ic, oc)
         with pytest.raises(TmiError, match="no MFMA / vector kernel is eligible"):
@@ -120,3 +122,48 @@ def test_pointwise_declines_what_it_does_not_take(ctx):
     x, wt, bias = _operands(rng, 1, 5, 5, 32, 16)
     with pytest.raises(TmiError, match="no MFMA / vector kernel is eligible"):
         gpu_ops.conv2d(ctx, x, wt, bias, stride=(2, 2), in_zp=0, w_zp=0)
+
+
+@pytest.mark.parametrize("ic", [168, 192, 256, 264, 320, 384, 520, 576, 960, 1024, 1032, 1280, 2048])
+@pytest.mark.parametrize("oc", [8, 24, 64, 160])
+def test_pointwise_split_k_int32_and_fused(ctx, ic, oc):
+    """long channel vectors: the four waves of a workgroup take a quarter of K each (2, 4, 8 or 16 K steps a wave, the last
+    wave's share ragged or empty) and meet in LDS"""
+    rng = np.random.default_rng(ic * 7 + oc)
+    x, wt, bias = _operands(rng, 2, 5, 9, ic, oc)
+    acc = oracle.conv2d("i8", x, wt, bias, in_zp=-9, w_zp=0)
+    got, st = gpu_ops.conv2d(ctx, x, wt, bias, in_zp=-9, w_zp=0)
+    assert ctx.last_kernel == "conv2d_pointwise_ksplit_i8"
+    assert st == capi.VALID and np.array_equal(got, acc), int(np.count_nonzero(got != acc))
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    shift = rng.integers(40, 46, oc).astype(np.int8)
+    for out_dtype, out_zp in ((np.int8, 7), (np.int16, 0)):
+        want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp, out_dtype=out_dtype)
+        got, st = gpu_ops.conv2d(ctx, x, wt, bias, in_zp=-9, w_zp=0, rescale=dict(mult=mult, shift=shift, out_zp=out_zp, out_dtype=out_dtype))
+        assert ctx.last_kernel == "conv2d_pointwise_ksplit_i8_rescale"
+        assert st == wst == capi.VALID and np.array_equal(got, want), int(np.count_nonzero(got != want))
+    assert len(np.unique(got)) > 50
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 256, 64), (1, 1, 33, 384, 24), (8, 14, 14, 1024, 256), (8, 7, 7, 2048, 512),
+                                   (8, 56, 56, 256, 64), (8, 14, 14, 384, 96)])
+@pytest.mark.parametrize("shifts", ["33 to 40", "mixed with small"])
+def test_pointwise_split_k_layers_and_forms(ctx, shape, shifts):
+    """projection layers of ResNet-50 and MobileNetV2 at batch 8 (several pixel tiles per workgroup on the largest), one
+    pixel, a tile and one pixel; the high-word and the general form of the requantisation with zero input_zp and without"""
+    n, h, w, ic, oc = shape
+    rng = np.random.default_rng(n * h + ic + len(shifts))
+    x, wt, bias = _operands(rng, n, h, w, ic, oc)
+    small = shifts != "33 to 40"
+    if small:
+        wt = rng.integers(-1, 2, wt.shape).astype(np.int8)
+        bias = rng.integers(-200, 200, oc).astype(np.int32)
+    shift = (rng.integers(33, 41, oc) if not small else np.where(np.arange(oc) % 40 < 32, rng.integers(33, 40, oc),
+                                                                 rng.integers(22, 33, oc))).astype(np.int8)
+    mult = rng.integers(1 << 30, 1 << 31, oc).astype(np.int32)
+    for in_zp in (0, 6):
+        acc = cases.conv2d_exact_blas(x, wt, bias, (0, 0, 0, 0), (1, 1), (1, 1), in_zp, 0)
+        want, wst = oracle.rescale(acc, mult, shift, out_zp=-1)
+        got, st = gpu_ops.conv2d(ctx, x, wt, bias, in_zp=in_zp, w_zp=0, rescale=dict(mult=mult, shift=shift, out_zp=-1))
+        assert ctx.last_kernel == "conv2d_pointwise_ksplit_i8_rescale"
+        assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))
