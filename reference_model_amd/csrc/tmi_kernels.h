@@ -97,6 +97,12 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
                                     const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                     void* out, uint32_t* flag_word);
 
+// conv_ksplit.hip: small int8 CONV2D layers with taps and a long reduction (IC a multiple of 32, weight_zp 0): a workgroup
+// per tile of 32 x 32 results, K split over its waves, operands straight from global memory into registers
+const char* launch_conv2d_ksplit(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                                 const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
+                                 void* out, const void* pad_page, uint32_t* flag_word);
+
 // direct.hip: one output element per lane, any legal shape.  out_dtype is the stored output type
 // (INT32 without rescale; the rescale output type with it; FP16/BF16/FP32 for floating point).
 const char* launch_conv2d_direct(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g,
