@@ -88,20 +88,28 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
         const int oy  = row - n * a.OH;
         const int iy0 = oy * a.sy - a.pad_top, ix0 = ox * a.sx - a.pad_left;
         const uint8_t* img = a.in + (size_t)n * a.IH * a.IW * a.IC;
+        // the wave's first step is decoded with divisions, the following ones by stepping (scalar work, the same for all lanes)
+        int tap = (int)fdiv((uint32_t)step0, a.div_spt);
+        int cs  = step0 - tap * a.spt;    // which 32 channels of the tap
+        int ky  = (int)fdiv((uint32_t)tap, a.div_kw);
+        int kx  = tap - ky * a.KW;
 #pragma unroll
         for (int s = 0; s < KS; s++)
         {
-            const int step = step0 + s;
-            if (s < ksw && step < a.steps)    // (a test per step, not a loop exit: the register array keeps constant indices)
+            if (s < ksw && step0 + s < a.steps)    // (a test per step, not a loop exit: the register array keeps constant indices)
             {
-                const int tap = (int)fdiv((uint32_t)step, a.div_spt);
-                const int c0  = (step - tap * a.spt) * 32 + 16 * lh;
-                const int ky  = (int)fdiv((uint32_t)tap, a.div_kw);
-                const int kx  = tap - ky * a.KW;
                 const int iy = iy0 + ky * a.dy, ix = ix0 + kx * a.dx;
-                const bool inside = (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
-                const uint8_t* src = inside ? img + ((size_t)(iy * a.IW + ix) * a.IC + c0) : a.pad_page + 16 * lh;
+                const bool inside  = (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+                const uint32_t off = (uint32_t)((iy * a.IW + ix) * a.IC + cs * 32 + 16 * lh);    // one image is below 2^31 bytes
+                const uint8_t* src = inside ? img + off : a.pad_page + 16 * lh;
                 fb[s]              = *reinterpret_cast<const v4i*>(src);
+            }
+            cs++;
+            if (cs == a.spt)
+            {
+                cs = 0, kx++;
+                if (kx == a.KW)
+                    kx = 0, ky++;
             }
         }
     };
@@ -113,18 +121,16 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
     const int ch = oct * 32 + wr;
     v4i fa[KS];
     {
-        const int8_t* row = a.w + (size_t)(ch < a.OC ? ch : a.OC - 1) * kbytes;
+        // one 32-bit offset per lane; the steps are the instruction's offset field (the weights are below 2^31 bytes)
+        const uint32_t woff = (uint32_t)((ch < a.OC ? ch : a.OC - 1) * kbytes + step0 * 32 + 16 * lh);
 #pragma unroll
         for (int s = 0; s < KS; s++)
         {
-            const int step = step0 + s;
-            if (s < ksw && step < a.steps)
-            {
-                const v4i v = *reinterpret_cast<const v4i*>(row + step * 32 + 16 * lh);
-                fa[s]       = ch < a.OC ? v : v4i{ 0, 0, 0, 0 };
-            }
+            if (s < ksw && step0 + s < a.steps)
+                fa[s] = *reinterpret_cast<const v4i*>(a.w + woff + s * 32);
         }
     }
+    // (rows past OC are zeroed further down, once, so that no load is waited for before the next one is issued)
     uint32_t flags = 0;
     if (wave == 0)
     {
@@ -149,6 +155,12 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
                 *form_word = form;
         }
     }
+    if (ch >= a.OC)
+    {
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+            fa[s] = v4i{ 0, 0, 0, 0 };
+    }
     {
         int32_t b = wave == 0 ? a.bias[a.bias_len == 1 ? 0 : (ch < a.OC ? ch : oct * 32)] : 0;
         if constexpr (ZA)
@@ -165,19 +177,25 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
             wave_start[wr] = ch < a.OC ? b : 0;
         __builtin_amdgcn_wave_barrier();    // the wave's own LDS accesses complete in order
     }
-    v16i start;
+    // (a tile's start values are read from the wave's table again for every tile: the registers are needed for the loads)
+    auto start_values = [&]() {
+        int first = 16 * lh;
+        asm volatile("" : "+v"(first));    // (hidden from the compiler, which would otherwise keep them across the loop)
+        v16i start;
 #pragma unroll
-    for (int gq = 0; gq < 4; gq++)
-    {
-        const v4i b4 = *reinterpret_cast<const v4i*>(wave_start + 16 * lh + 4 * gq);
-        start[4 * gq] = b4[0], start[4 * gq + 1] = b4[1], start[4 * gq + 2] = b4[2], start[4 * gq + 3] = b4[3];
-    }
+        for (int gq = 0; gq < 4; gq++)
+        {
+            const v4i b4 = *reinterpret_cast<const v4i*>(wave_start + first + 4 * gq);
+            start[4 * gq] = b4[0], start[4 * gq + 1] = b4[1], start[4 * gq + 2] = b4[2], start[4 * gq + 3] = b4[3];
+        }
+        return start;
+    };
     const int oc_lane = oct * 32 + 16 * lh + 4 * (wave & 3);    // first of the 4 channels a lane of waves 0 .. 3 stores
     const bool ch_ok  = oc_lane < a.OC;                         // OC is a multiple of 8: the four are in or out together
     const int32_t v_lo = a.rp.lo, v_hi = a.rp.hi;
     for (int pt = q; pt < a.n_pt; pt += G)
     {
-        v16i acc = start;
+        v16i acc = start_values();
 #pragma unroll
         for (int s = 0; s < KS; s++)
             if (s < ksw && step0 + s < a.steps)

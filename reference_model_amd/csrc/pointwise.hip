@@ -121,9 +121,16 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
             const int k0 = 32 * s + 16 * lh;
             const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
             const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
-            const bool r = ch < a.OC;
-            fa[s]        = v4i{ r && k0 < a.IC ? lo.x : 0, r && k0 < a.IC ? lo.y : 0, r && k0 + 8 < a.IC ? hi.x : 0,
-                         r && k0 + 8 < a.IC ? hi.y : 0 };
+            fa[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
+        }
+        // what lies past IC or past OC is zeroed once all loads have been issued (a test in the loop above would wait for
+        // every load before the next)
+#pragma unroll
+        for (int s = 0; s < KSTEPS; s++)
+        {
+            const int k0  = 32 * s + 16 * lh;
+            const bool r0 = ch < a.OC && k0 < a.IC, r1 = ch < a.OC && k0 + 8 < a.IC;
+            fa[s]         = v4i{ r0 ? fa[s].x : 0, r0 ? fa[s].y : 0, r1 ? fa[s].z : 0, r1 ? fa[s].w : 0 };
         }
     }
     // ---- per-channel constants: lane li (both halves alike) derives those of channel 32 oct + li ------------------------
@@ -353,10 +360,17 @@ __global__ __launch_bounds__(kSplitWaves * 64, 2) void pointwise_ksplit_i8_kerne
             {
                 const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
                 const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
-                const bool r = ch < a.OC;
-                fa[s]        = v4i{ r && k0 < a.IC ? lo.x : 0, r && k0 < a.IC ? lo.y : 0, r && k0 + 8 < a.IC ? hi.x : 0,
-                             r && k0 + 8 < a.IC ? hi.y : 0 };
+                fa[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
             }
+        }
+        // what lies past IC or past OC is zeroed once all loads have been issued
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+        {
+            const int k0  = kbase + 32 * s + 16 * lh;
+            const bool r0 = ch < a.OC && k0 < a.IC, r1 = ch < a.OC && k0 + 8 < a.IC;
+            if (s < ksw)
+                fa[s] = v4i{ r0 ? fa[s].x : 0, r0 ? fa[s].y : 0, r1 ? fa[s].z : 0, r1 ? fa[s].w : 0 };
         }
     }
     uint32_t flags = 0;
