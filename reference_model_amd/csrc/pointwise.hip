@@ -40,6 +40,12 @@ struct PointwiseArgs
     int32_t n_groups;    // groups of n_oct waves; group q takes the pixel tiles q, q + n_groups, ...
     int32_t ksw;         // the form that splits K over a workgroup's waves: K steps per wave
     FastDiv div_oct;
+    // The first layer of a network (STEM): `in` is a copy of the image with its padding materialised, rows of row_bytes
+    // bytes; a K step is one row of taps, the KW * IC (at most 32) contiguous bytes under it; `w` holds 32 bytes per
+    // (channel, tap row), so IC above is 32 * KH for the weight loads
+    int32_t row_bytes, rows, OH, OW;     // padded image: bytes per row, rows per image
+    int32_t step_y, step_x, step_k;      // bytes from one output row / output pixel / tap row to the next
+    FastDiv div_ow, div_oh;
 };
 
 constexpr int kPointwiseWaves   = 4;
@@ -66,7 +72,7 @@ __device__ __forceinline__ int32_t rescale_from_shift(int32_t v, int32_t m, int3
     return r > hi ? hi : r;
 }
 
-template <int KSTEPS, bool ZA>
+template <int KSTEPS, bool ZA, bool STEM = false>
 __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void pointwise_i8_kernel(PointwiseArgs a)
 {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kPointwiseWaves][kPointwiseWaveLds];
@@ -88,6 +94,20 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
     auto load_pixels = [&](v4i (&fb)[KSTEPS], int pt) {
         int p = pt * 32 + li;
         p     = p < a.P ? p : a.P - 1;    // a pixel past the end: the last one again, never stored
+        if constexpr (STEM)
+        {
+            // 16 of the 32 bytes that start under the window's tap (ky, 0): KW * IC of them are the row of taps, the rest
+            // meets zero weights; the address has no alignment (the compiler is told so and chooses the load)
+            const int r  = (int)fdiv((uint32_t)p, a.div_ow);    // n * OH + oy
+            const int ox = p - r * a.OW;
+            const int n  = (int)fdiv((uint32_t)r, a.div_oh);
+            const int oy = r - n * a.OH;
+            const uint8_t* win = a.in + (uint32_t)((n * a.rows) * a.row_bytes + oy * a.step_y + ox * a.step_x + 16 * lh);
+#pragma unroll
+            for (int s = 0; s < KSTEPS; s++)
+                __builtin_memcpy(&fb[s], win + s * a.step_k, 16);
+            return;
+        }
         const uint8_t* row = a.in + (size_t)p * a.IC;
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++)
@@ -578,6 +598,149 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
         return nullptr;
     last_launch_shape[0] = grid, last_launch_shape[1] = kPointwiseWaves * 64, last_launch_shape[2] = kPointwiseWaves * kPointwiseWaveLds;
     return rp.enabled ? "conv2d_pointwise_i8_rescale" : "conv2d_pointwise_i8";
+}
+
+// ---- the first layer of a network: 3 x 3 ... 7 x 7 taps over at most 4 channels -------------------------------------------
+//
+// With 3 input channels a tap is 3 bytes and the whole row of taps of a 7 x 7 window 21 contiguous bytes of the image: a
+// K step of the matrix instruction (32 bytes) per tap row, read where it lies.  What stands in the way is the padding (a
+// window at the border reads input_zp for the pixels outside) and the weight layout; a first launch writes the image with
+// its padding materialised (rows of (IW + pad_left + pad_right) * IC bytes, input_zp outside) and the weights as 32 bytes
+// per (channel, tap row), zeros behind the KW * IC that exist, into the caller's scratch buffer; the pointwise kernel above
+// then runs with a wave per tile of 32 output channels, K steps = tap rows (STEM).  dilation_x must be 1.
+struct StemPrepArgs
+{
+    const uint8_t* in;
+    const int8_t* w;
+    uint8_t* padded;
+    int8_t* wrep;
+    int32_t N, IH, IW, IC, OC, KH, KW;
+    int32_t rows, row_bytes, pad_top, pad_left, za;
+    int32_t image_words, weight_words;    // 4-byte words of the padded images / of the weight rows
+    FastDiv div_rw, div_rows, div_ic;
+};
+
+__global__ __launch_bounds__(256) void stem_prepass_kernel(StemPrepArgs a)
+{
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < (uint32_t)a.image_words)
+    {
+        const uint32_t rw = (uint32_t)a.row_bytes / 4;
+        const uint32_t r  = fdiv(i, a.div_rw);    // n * rows + y
+        const uint32_t b0 = (i - r * rw) * 4;     // first of the word's four bytes in the row
+        const uint32_t n  = fdiv(r, a.div_rows);
+        const int iy      = (int)(r - n * a.rows) - a.pad_top;
+        uint32_t word     = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+        {
+            const uint32_t x = fdiv(b0 + k, a.div_ic);
+            const int c      = (int)(b0 + k - x * a.IC);
+            const int ix     = (int)x - a.pad_left;
+            int v            = a.za;
+            if (n < (uint32_t)a.N && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW)    // (n = N: the spare bytes behind the last image)
+                v = a.in[((size_t)(n * a.IH + iy) * a.IW + ix) * a.IC + c];
+            word |= (uint32_t)(v & 0xff) << (8 * k);
+        }
+        reinterpret_cast<uint32_t*>(a.padded)[i] = word;
+        return;
+    }
+    const uint32_t j = i - a.image_words;
+    if (j < (uint32_t)a.weight_words)
+    {
+        const uint32_t row = j >> 3;    // (channel, tap row): 32 bytes, 8 words
+        const int b0       = (int)(j & 7) * 4;
+        const int len      = a.KW * a.IC;
+        uint32_t word      = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (b0 + k < len)
+                word |= (uint32_t)(a.w[(size_t)row * len + b0 + k] & 0xff) << (8 * k);
+        reinterpret_cast<uint32_t*>(a.wrep)[j] = word;
+    }
+}
+
+template <int KSTEPS>
+static void launch_stem(hipStream_t st, const PointwiseArgs& a, int grid)
+{
+    if (a.za != 0)
+        hipLaunchKernelGGL((pointwise_i8_kernel<KSTEPS, true, true>), dim3(grid), dim3(kPointwiseWaves * 64), 0, st, a);
+    else
+        hipLaunchKernelGGL((pointwise_i8_kernel<KSTEPS, false, true>), dim3(grid), dim3(kPointwiseWaves * 64), 0, st, a);
+}
+
+// Bytes of scratch the first-layer form needs for this layer, or 0 when it does not take it.
+size_t conv2d_stem_scratch_bytes(int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, int32_t w_zp, const RescaleParams& rp)
+{
+    if (in_dtype != TMI_INT8 || w_zp != 0 || g.IC < 1 || g.IC > 4 || g.KW * g.IC > 32 || g.dil_x != 1)
+        return 0;
+    if ((g.KH != 3 && g.KH != 5 && g.KH != 7) || g.KW < 2 || (g.OC & 7) || g.OC < 8 || g.OC > 4096)
+        return 0;
+    if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
+        return 0;
+    // rows and columns the windows reach: what the declared output size needs, not more than the padded image
+    const int64_t rows = (int64_t)(g.OH - 1) * g.stride_y + (int64_t)(g.KH - 1) * g.dil_y + 1;
+    const int64_t cols = (int64_t)(g.OW - 1) * g.stride_x + g.KW;
+    const int64_t row_bytes = (cols * g.IC + 3) / 4 * 4;
+    const int64_t image = (int64_t)g.N * rows * row_bytes;
+    if (image + 64 >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
+        return 0;
+    return (size_t)((image + 64 + 255) / 256 * 256 + (int64_t)g.OC * g.KH * 32);
+}
+
+// nullptr when the layer is not one this form takes; `scratch` holds conv2d_stem_scratch_bytes() bytes, 256-byte aligned.
+const char* launch_conv2d_stem(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                               const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, void* out,
+                               void* scratch, uint32_t* flag_word)
+{
+    if (!conv2d_stem_scratch_bytes(in_dtype, out_dtype, g, w_zp, rp) || !scratch || !flag_word)
+        return nullptr;
+    if ((((uintptr_t)out | (uintptr_t)scratch) & 15) || ((uintptr_t)bias & 3))
+        return nullptr;
+    const int rows = (g.OH - 1) * g.stride_y + (g.KH - 1) * g.dil_y + 1;
+    const int cols = (g.OW - 1) * g.stride_x + g.KW;
+    const int row_bytes = (cols * g.IC + 3) / 4 * 4;
+    const int64_t image = (int64_t)g.N * rows * row_bytes;
+    StemPrepArgs pa{};
+    pa.in = (const uint8_t*)in, pa.w = (const int8_t*)w;
+    pa.padded = (uint8_t*)scratch, pa.wrep = (int8_t*)scratch + (image + 64 + 255) / 256 * 256;
+    pa.N = g.N, pa.IH = g.IH, pa.IW = g.IW, pa.IC = g.IC, pa.OC = g.OC, pa.KH = g.KH, pa.KW = g.KW;
+    pa.rows = rows, pa.row_bytes = row_bytes, pa.pad_top = g.pad_top, pa.pad_left = g.pad_left, pa.za = in_zp;
+    pa.image_words = (int32_t)((image + 64) / 4), pa.weight_words = g.OC * g.KH * 8;
+    pa.div_rw = make_fastdiv((uint32_t)(row_bytes / 4)), pa.div_rows = make_fastdiv((uint32_t)rows);
+    pa.div_ic = make_fastdiv((uint32_t)g.IC);
+    // (the 64 bytes behind the last image belong to no row: they are written as a row past the last image would be)
+    if (!fastdiv_exact_up_to((uint64_t)pa.image_words, (uint32_t)(row_bytes / 4)) ||
+        !fastdiv_exact_up_to((uint64_t)pa.image_words / (row_bytes / 4) + 1, (uint32_t)rows) ||
+        !fastdiv_exact_up_to((uint64_t)row_bytes + 4, (uint32_t)g.IC))
+        return nullptr;
+    const int64_t P = (int64_t)g.N * g.OH * g.OW;
+    PointwiseArgs a{};
+    a.in = pa.padded, a.w = pa.wrep, a.bias = (const int32_t*)bias, a.out = out, a.flag_word = flag_word, a.rp = rp;
+    a.P = (int32_t)P, a.IC = g.KH * 32, a.OC = g.OC, a.za = in_zp, a.bias_len = g.bias_len;
+    a.out_kind = !rp.enabled ? 0 : (out_dtype == TMI_INT8 ? 1 : 2);
+    a.n_oct = (g.OC + 31) / 32, a.n_pt = (int32_t)((P + 31) / 32);
+    a.div_oct = make_fastdiv((uint32_t)a.n_oct);
+    a.row_bytes = row_bytes, a.rows = rows, a.OH = g.OH, a.OW = g.OW;
+    a.step_y = g.stride_y * row_bytes, a.step_x = g.stride_x * g.IC, a.step_k = g.dil_y * row_bytes;
+    a.div_ow = make_fastdiv((uint32_t)g.OW), a.div_oh = make_fastdiv((uint32_t)g.OH);
+    const int max_groups = 256 * 8 / a.n_oct > 0 ? 256 * 8 / a.n_oct : 1;
+    a.n_groups = a.n_pt < max_groups ? a.n_pt : max_groups;
+    const int64_t waves = (int64_t)a.n_groups * a.n_oct;
+    if (!fastdiv_exact_up_to((uint64_t)waves + kPointwiseWaves, (uint32_t)a.n_oct) || !fastdiv_exact_up_to((uint64_t)P, (uint32_t)g.OW) ||
+        !fastdiv_exact_up_to((uint64_t)P / g.OW + 1, (uint32_t)g.OH))
+        return nullptr;
+    const int prep_grid = (pa.image_words + pa.weight_words + 255) / 256;
+    hipLaunchKernelGGL(stem_prepass_kernel, dim3(prep_grid), dim3(256), 0, st, pa);
+    const int grid = (int)((waves + kPointwiseWaves - 1) / kPointwiseWaves);
+    if (g.KH == 3)
+        launch_stem<3>(st, a, grid);
+    else if (g.KH == 5)
+        launch_stem<5>(st, a, grid);
+    else
+        launch_stem<7>(st, a, grid);
+    last_launch_shape[0] = grid, last_launch_shape[1] = kPointwiseWaves * 64, last_launch_shape[2] = kPointwiseWaves * kPointwiseWaveLds;
+    return rp.enabled ? "conv2d_stem_i8_rescale" : "conv2d_stem_i8";
 }
 
 }    // namespace tmi

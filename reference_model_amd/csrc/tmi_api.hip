@@ -505,6 +505,24 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (!name && g.KH * g.KW > 1 && (ctx->kernel_choice == 5 || (ctx->kernel_choice == 0 && split_first)))
             name = launch_conv2d_ksplit(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                         ctx->flags_dev);
+        // First layers (at most 4 input channels, 3 x 3 ... 7 x 7 taps): a pre-pass into the scratch buffer and the pointwise
+        // kernel with a K step per row of taps, unless an operand of this call lies in that buffer already.
+        if (!name && (ctx->kernel_choice == 5 || ctx->kernel_choice == 0))
+        {
+            const size_t need = conv2d_stem_scratch_bytes(d->in_dtype, out_dtype, g, w_zp, rp);
+            auto in_scratch   = [&](const void* p) {
+                return ctx->workspace && (const uint8_t*)p >= (const uint8_t*)ctx->workspace &&
+                       (const uint8_t*)p < (const uint8_t*)ctx->workspace + ctx->workspace_size;
+            };
+            if (need && !in_scratch(in) && !in_scratch(w) && !in_scratch(out) && !in_scratch(bias))
+            {
+                rc = ensure_workspace(ctx, need);
+                if (rc != TMI_VALID)
+                    return rc;
+                name = launch_conv2d_stem(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                          ctx->workspace, ctx->flags_dev);
+            }
+        }
         if (!name && (ctx->kernel_choice == 5 || (ctx->kernel_choice == 0 && g.IC <= 160)))    // (the layers it leads on were tried above)
             name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                            ctx->flags_dev);

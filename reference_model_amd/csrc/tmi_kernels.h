@@ -97,6 +97,14 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
                                     const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                     void* out, uint32_t* flag_word);
 
+// pointwise.hip, first layers: int8 CONV2D with 3 x 3 ... 7 x 7 taps over at most 4 channels (KW * IC <= 32, dilation_x 1,
+// weight_zp 0) as a pre-pass into `scratch` (padding materialised, weights as 32 bytes per tap row) plus the pointwise
+// kernel with a K step per tap row.  conv2d_stem_scratch_bytes() is 0 for a layer the form does not take.
+size_t conv2d_stem_scratch_bytes(int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, int32_t w_zp, const RescaleParams& rp);
+const char* launch_conv2d_stem(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                               const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, void* out,
+                               void* scratch, uint32_t* flag_word);
+
 // conv_ksplit.hip: small int8 CONV2D layers with taps and a long reduction (IC a multiple of 32, weight_zp 0): a workgroup
 // per tile of 32 x 32 results, K split over its waves, operands straight from global memory into registers
 const char* launch_conv2d_ksplit(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
