@@ -76,6 +76,7 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
     int32_t* form_word    = reinterpret_cast<int32_t*>(tab_ms + 32) + NW * 32;
     const int ksw   = a.ksw;
     const int step0 = wave * ksw;    // first K step of the wave's share
+    const int nvalid = a.steps - step0 < ksw ? (a.steps - step0 > 0 ? a.steps - step0 : 0) : ksw;    // steps of the share that exist
     const int kbytes = a.steps * 32; // bytes of a weight row
 
     // ---- pixel fragments: lane (li, lh) holds bytes [16 lh, + 16) of the 32 channels of step s under the step's tap ------
@@ -88,28 +89,38 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
         const int oy  = row - n * a.OH;
         const int iy0 = oy * a.sy - a.pad_top, ix0 = ox * a.sx - a.pad_left;
         const uint8_t* img = a.in + (size_t)n * a.IH * a.IW * a.IC;
-        // the wave's first step is decoded with divisions, the following ones by stepping (scalar work, the same for all lanes)
+        // A wave with one wave on its SIMD issues an instruction every eight clocks or so, so what a step costs is its
+        // instruction count: the tap's pixel is worked out once per tap (the wave's first step with divisions, the following
+        // taps by stepping: scalar work, the same for all lanes) and a step inside a tap is a load and an addition.
         int tap = (int)fdiv((uint32_t)step0, a.div_spt);
         int cs  = step0 - tap * a.spt;    // which 32 channels of the tap
         int ky  = (int)fdiv((uint32_t)tap, a.div_kw);
         int kx  = tap - ky * a.KW;
+        const uint8_t* cur = nullptr;
+        uint32_t inc       = 0;
+        auto at_tap        = [&]() {
+            const int iy = iy0 + ky * a.dy, ix = ix0 + kx * a.dx;
+            const bool inside  = (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
+            const uint32_t off = (uint32_t)((iy * a.IW + ix) * a.IC + cs * 32 + 16 * lh);    // one image is below 2^31 bytes
+            cur                = inside ? img + off : a.pad_page + 16 * lh;
+            inc                = inside ? 32u : 0u;    // outside the image every step reads the page of input_zp bytes
+        };
+        at_tap();
 #pragma unroll
         for (int s = 0; s < KS; s++)
         {
-            if (s < ksw && step0 + s < a.steps)    // (a test per step, not a loop exit: the register array keeps constant indices)
+            if (s < nvalid)    // (a test per step, not a loop exit: the register array keeps constant indices)
             {
-                const int iy = iy0 + ky * a.dy, ix = ix0 + kx * a.dx;
-                const bool inside  = (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
-                const uint32_t off = (uint32_t)((iy * a.IW + ix) * a.IC + cs * 32 + 16 * lh);    // one image is below 2^31 bytes
-                const uint8_t* src = inside ? img + off : a.pad_page + 16 * lh;
-                fb[s]              = *reinterpret_cast<const v4i*>(src);
-            }
-            cs++;
-            if (cs == a.spt)
-            {
-                cs = 0, kx++;
-                if (kx == a.KW)
-                    kx = 0, ky++;
+                fb[s] = *reinterpret_cast<const v4i*>(cur);
+                cur += inc;
+                cs++;
+                if (cs == a.spt)
+                {
+                    cs = 0, kx++;
+                    if (kx == a.KW)
+                        kx = 0, ky++;
+                    at_tap();
+                }
             }
         }
     };
@@ -126,7 +137,7 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
 #pragma unroll
         for (int s = 0; s < KS; s++)
         {
-            if (s < ksw && step0 + s < a.steps)
+            if (s < nvalid)
                 fa[s] = *reinterpret_cast<const v4i*>(a.w + woff + s * 32);
         }
     }
@@ -168,7 +179,7 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
             int sum = 0;
 #pragma unroll
             for (int s = 0; s < KS; s++)
-                if (s < ksw && step0 + s < a.steps)
+                if (s < nvalid)
                     sum += dot4_ones(fa[s]);
             sum += __builtin_amdgcn_ds_bpermute((lane ^ 32) * 4, sum);
             b = (int32_t)((uint32_t)b - (uint32_t)a.za * (uint32_t)sum);
@@ -198,7 +209,7 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
         v16i acc = start_values();
 #pragma unroll
         for (int s = 0; s < KS; s++)
-            if (s < ksw && step0 + s < a.steps)
+            if (s < nvalid)
                 acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[s], acc, 0, 0, 0);
         if (pt + G < a.n_pt)
             load_pixels(fb, pt + G);    // in flight across the exchange and the requantisation
