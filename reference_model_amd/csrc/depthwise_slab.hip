@@ -388,7 +388,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
 {
     if (in_dtype != TMI_INT8 || g.M != 1 || g.KH != 3 || g.KW != 3 || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
-    if ((g.IC & 15) || g.IC < 32 || g.IC > 512 || g.OC != g.IC)
+    if ((g.IC & 15) || g.IC < 32 || g.IC > 1024 || g.OC != g.IC)
         return nullptr;
     if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
         return nullptr;

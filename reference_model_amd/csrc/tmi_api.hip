@@ -429,7 +429,16 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
             return fail(ctx, "%s: the fused rescale needs an INT8 convolution", op);
         return after_launch(ctx, launch_conv_i16_direct(ctx->stream, depthwise, g, in, w, bias, w_zp, out));
     }
-    if (depthwise && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
+    // Small depthwise layers: the vector kernel (a lane per four channels of a pixel, no LDS, no barrier) costs 3.15 us plus
+    // 4.4 us per million results, the matrix-core kernel 3.3 us plus 3.7 ns per channel (its per-channel tables) and next
+    // to nothing per result.  us matrix-core / vector kernel, 3x3, fused RESCALE: [8,14,14,384] stride 2 4.3 / 3.3,
+    // [8,7,7,512] 4.9 / 3.4, [8,7,7,960] 6.8 / 4.1, [2,14,14,576] 5.1 / 3.8, [4,14,14,576] 5.3 / 4.8, [1,28,28,192] 3.8 / 3.4,
+    // [8,10,10,672] 5.6 / 5.0; the other way: [1,56,56,144] 3.9 / 4.3, [8,14,14,576] 5.3 / 7.2, [8,14,14,1024] 7.1 / 7.5,
+    // [8,28,28,384] 4.8 / 9.5, [32,14,14,576] 5.8 / 14.7.
+    if (depthwise && ctx->kernel_choice == 0 && total < 34000 + 850 * (int64_t)g.IC)
+        name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                    ctx->flags_dev);
+    if (depthwise && !name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
         name = launch_depthwise_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                      ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);
     if (depthwise && !name && ctx->kernel_choice != 1 && ctx->kernel_choice != 4)

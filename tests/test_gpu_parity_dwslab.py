@@ -30,6 +30,9 @@ DW_SHAPES = [  # n, ih, iw, c, pad, stride, dilation
     (2, 24, 24, 64, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilation 2
     (2, 33, 31, 64, (1, 1, 0, 0), (2, 1), (1, 1)),      # stride 2 x 1, no horizontal padding
     (40, 9, 9, 96, (1, 1, 1, 1), (1, 1), (1, 1)),       # many small images
+    (2, 14, 14, 576, (1, 1, 1, 1), (1, 1), (1, 1)),     # 18 channel blocks: more channels than eight waves have lanes
+    (2, 7, 7, 960, (1, 1, 1, 1), (1, 1), (1, 1)),       # 30 channel blocks
+    (1, 10, 10, 1024, (0, 1, 0, 1), (2, 2), (1, 1)),    # the most channels the kernel takes
 ]
 
 
@@ -138,7 +141,13 @@ def test_depthwise_mfma_refuses_what_it_cannot_take(ctx):
 def test_automatic_choice_takes_the_matrix_core_kernel_for_its_layers():
     c = Context(0)
     try:
-        shape = (2, 28, 28, 96, (0, 1, 0, 1), (2, 2), (1, 1))
+        # a small layer (37 632 results of 96 channels) goes to the vector kernel, whose set-up is the shorter one
+        small = (2, 28, 28, 96, (0, 1, 0, 1), (2, 2), (1, 1))
+        x, w, bias = _operands(small, 3)
+        got, st = gpu_ops.conv2d(c, x, w, bias, small[4], small[5], in_zp=4, depthwise=True)
+        assert st == capi.VALID and c.last_kernel == "depthwise_dot4_i8"
+        assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, small[4], small[5], in_zp=4, w_zp=0))
+        shape = (8, 56, 56, 96, (0, 1, 0, 1), (2, 2), (1, 1))
         x, w, bias = _operands(shape, 3)
         got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=4, depthwise=True)
         assert st == capi.VALID and c.last_kernel in ("depthwise_mfma_i8", "depthwise_mfma_pipe_i8")
