@@ -5,7 +5,7 @@
 //                        + bias[oc]                                                     (tensor_ops.cpp:828-882)
 //
 // Such a layer has few output tiles (8 x 14 x 14 pixels x 256 channels: 26 tiles of 128 x 128) and K = 2304 ... 4608, so a
-// kernel that gives a workgroup a large tile keeps a tenth of the chip busy.  Here a workgroup of NW waves (4 or 8) owns a
+// kernel that gives a workgroup a large tile keeps a tenth of the chip busy.  Here a workgroup of NW waves (4, 8 or 16) owns a
 // tile of 32 output channels x 32 pixels and splits the K steps (ky, kx, 32 channels) between its waves; both operands go
 // straight from global memory into the registers the matrix instruction reads - the weight rows are K-contiguous as they
 // lie, a pixel fragment is 16 bytes of the input pixel under the step's tap, or of the context's page of input_zp bytes
@@ -13,7 +13,7 @@
 // from its share of bias - input_zp * sum(w); the partial tiles meet in LDS and the first four waves requantise and store
 // a quarter of the tile each (4 consecutive channels per lane).
 //
-// weight_zp must be 0, IC a multiple of 32, OC a multiple of 8, and a wave's share at most 18 K steps.
+// weight_zp must be 0, IC a multiple of 32, OC a multiple of 8, and K at most 160 steps (16 waves of 10).
 #include "tmi_mfma.h"
 
 namespace tmi
@@ -60,10 +60,10 @@ __device__ __forceinline__ int32_t split_rescale_from_shift(int32_t v, int32_t m
 }
 
 template <int KS, int NW, bool ZA>
-__global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArgs a)
+__global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 2) void conv_ksplit_i8_kernel(ConvSplitArgs a)
 {
     // [NW waves x 4 quarters x 64 lanes x 16 bytes][32 x HighWordScale][32 x (m, s)][NW waves x 32 start values][form]
-    __shared__ __attribute__((aligned(16))) uint8_t lds[NW * 4096 + 32 * 16 + 32 * 8 + NW * 128 + 16];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int li = lane & 31, lh = lane >> 5;
@@ -269,14 +269,23 @@ __global__ __launch_bounds__(NW * 64, 2) void conv_ksplit_i8_kernel(ConvSplitArg
     raise_flags(a.flag_word, flags);
 }
 
-template <int KS, int NW>
-static void launch_conv_ksplit(hipStream_t st, const ConvSplitArgs& a, int grid)
+template <int KS, int NW, bool ZA>
+static bool launch_conv_ksplit_za(hipStream_t st, const ConvSplitArgs& a, int grid)
 {
-    if (a.za != 0)
-        hipLaunchKernelGGL((conv_ksplit_i8_kernel<KS, NW, true>), dim3(grid), dim3(NW * 64), 0, st, a);
-    else
-        hipLaunchKernelGGL((conv_ksplit_i8_kernel<KS, NW, false>), dim3(grid), dim3(NW * 64), 0, st, a);
-    last_launch_shape[0] = grid, last_launch_shape[1] = NW * 64, last_launch_shape[2] = NW * 4096 + 32 * 24 + NW * 128 + 16;
+    constexpr int lds_bytes = NW * 4096 + 32 * 16 + 32 * 8 + NW * 128 + 16;
+    static LdsLimit granted{};
+    auto kern = conv_ksplit_i8_kernel<KS, NW, ZA>;
+    if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
+        return false;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds_bytes, st, a);
+    last_launch_shape[0] = grid, last_launch_shape[1] = NW * 64, last_launch_shape[2] = lds_bytes;
+    return true;
+}
+
+template <int KS, int NW>
+static bool launch_conv_ksplit(hipStream_t st, const ConvSplitArgs& a, int grid)
+{
+    return a.za != 0 ? launch_conv_ksplit_za<KS, NW, true>(st, a, grid) : launch_conv_ksplit_za<KS, NW, false>(st, a, grid);
 }
 
 // nullptr when the layer is not one this kernel takes.
@@ -297,10 +306,11 @@ const char* launch_conv2d_ksplit(hipStream_t st, int32_t in_dtype, int32_t out_d
     if (P < 1 || (int64_t)g.N * g.IH * g.IW * g.IC >= (int64_t(1) << 31) || P * g.OC >= (int64_t(1) << 31) ||
         (int64_t)g.OC * taps * g.IC >= (int64_t(1) << 31))
         return nullptr;
+    // 4, 8 or 16 waves a workgroup: at most 10 K steps a wave (a wave's time is its instruction count)
     const int steps = taps * (g.IC / 32);
-    const int nw    = steps > 72 ? 8 : 4;
+    const int nw    = steps > 80 ? 16 : (steps > 40 ? 8 : 4);
     const int ksw   = (steps + nw - 1) / nw;
-    if (ksw > 18)
+    if (ksw > 10)
         return nullptr;
 
     ConvSplitArgs a{};
@@ -323,22 +333,15 @@ const char* launch_conv2d_ksplit(hipStream_t st, int32_t in_dtype, int32_t out_d
         !fastdiv_exact_up_to((uint64_t)P / g.OW + 1, (uint32_t)g.OH) || !fastdiv_exact_up_to((uint64_t)steps, (uint32_t)a.spt) ||
         !fastdiv_exact_up_to((uint64_t)taps, (uint32_t)g.KW))
         return nullptr;
+    bool ok;
     if (nw == 4)
-    {
-        if (ksw <= 4)
-            launch_conv_ksplit<4, 4>(st, a, grid);
-        else if (ksw <= 10)
-            launch_conv_ksplit<10, 4>(st, a, grid);
-        else
-            launch_conv_ksplit<18, 4>(st, a, grid);
-    }
+        ok = ksw <= 4 ? launch_conv_ksplit<4, 4>(st, a, grid) : launch_conv_ksplit<10, 4>(st, a, grid);
+    else if (nw == 8)
+        ok = launch_conv_ksplit<10, 8>(st, a, grid);
     else
-    {
-        if (ksw <= 10)
-            launch_conv_ksplit<10, 8>(st, a, grid);
-        else
-            launch_conv_ksplit<18, 8>(st, a, grid);
-    }
+        ok = launch_conv_ksplit<10, 16>(st, a, grid);
+    if (!ok)
+        return nullptr;
     return rp.enabled ? "conv2d_ksplit_i8_rescale" : "conv2d_ksplit_i8";
 }
 

@@ -507,10 +507,10 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // Layers with taps that are small and deep (at most 32 tiles of 128 x 128 results, at most 1 G multiply-adds) and
         // not the slab kernel's: a workgroup per tile of 32 x 32 results with K split over its waves, before the patch and
         // GEMM kernels, which would keep a tenth of the chip busy.  us patch kernel / this kernel, 3x3, fused RESCALE:
-        // [8,14,14,256]->256 14.3 / 11.4, [8,28,28,256]->256 stride 2 16.2 / 11.4, [8,7,7,512]->512 21.1 / 11.0,
-        // [8,14,14,512]->512 stride 2 22.5 / 11.0, [8,14,14,160]->160 13.6 / 5.0, [1,14,14,256]->256 14.2 / 7.5; the other
-        // way beyond: [12,14,14,256]->256 (38 tiles) 14.4 / 15.9, [16,..] 14.5 / 19.5 (the GEMM kernel's patch form 17.1),
-        // [4,28,28,256]->256 14.4 / 19.6, [8,14,14,384]->384 (2.1 G multiply-adds) 18.8 / 25.2.
+        // [8,14,14,256]->256 14.3 / 10.8, [8,28,28,256]->256 stride 2 16.2 / 10.8, [8,7,7,512]->512 21.1 / 10.8,
+        // [8,14,14,512]->512 stride 2 22.5 / 10.8, [8,14,14,160]->160 13.6 / 4.5, [1,14,14,256]->256 14.2 / 6.9; the other
+        // way beyond: [12,14,14,256]->256 (38 tiles) 14.4 / 14.9, [16,..] 14.5 / 18.5 (the GEMM kernel's patch form 17.1),
+        // [4,28,28,256]->256 14.4 / 19.6, [8,14,14,384]->384 (2.1 G multiply-adds) 18.8 / 24.1.
         const bool split_first = g.KH * g.KW > 1 && tiles128 <= 32 && total * g.IC * g.KH * g.KW <= 1000000000ll;
         if (!name && g.KH * g.KW > 1 && (ctx->kernel_choice == 5 || (ctx->kernel_choice == 0 && split_first)))
             name = launch_conv2d_ksplit(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,

@@ -1,6 +1,6 @@
 """The int8 CONV2D kernel that splits K over the waves of a workgroup (small layers with taps and a long reduction) through
 the C ABI, bit for bit against the CPU oracle (tensor_ops.cpp:828-882, then type_conversion.cpp:224-421): tap counts, strides,
-dilations and paddings, every share of K steps per wave, four and eight waves, ragged channel tiles, all result types and
+dilations and paddings, every share of K steps per wave, four, eight and sixteen waves, ragged channel tiles, all result types and
 both forms of the requantisation."""
 import numpy as np
 import pytest
@@ -26,12 +26,12 @@ SHAPES = [
     (2, 7, 7, 32, 8, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),         # 9 K steps on four waves: shares of 3, 3, 3, 0
     (2, 9, 8, 64, 24, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),        # 18 steps: 5, 5, 5, 3
     (1, 14, 14, 128, 40, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 36 steps: 9 each
-    (2, 14, 14, 256, 72, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 72 steps: 18 each
-    (2, 7, 7, 512, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),       # 144 steps on eight waves: 18 each
-    (1, 9, 9, 288, 16, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1)),       # 81 steps on eight waves: 11 x 7 + 4
+    (2, 14, 14, 256, 72, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),     # 72 steps on eight waves: 9 each
+    (2, 7, 7, 512, 64, 3, 3, (1, 1, 1, 1), (1, 1), (1, 1)),       # 144 steps on sixteen waves: 9 each
+    (1, 9, 9, 288, 16, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1)),       # 81 steps on sixteen waves: 6 x 13 + 3, two waves without a share
     (2, 14, 12, 64, 32, 3, 3, (1, 0, 1, 0), (2, 2), (1, 1)),      # stride 2
     (1, 12, 12, 96, 48, 3, 3, (2, 2, 2, 2), (1, 1), (2, 2)),      # dilation 2
-    (1, 10, 11, 64, 16, 5, 5, (2, 2, 2, 2), (1, 1), (1, 1)),      # 50 steps
+    (1, 10, 11, 64, 16, 5, 5, (2, 2, 2, 2), (1, 1), (1, 1)),      # 50 steps on eight waves: 7 x 7 + 1
     (1, 6, 40, 160, 8, 1, 3, (0, 0, 1, 1), (1, 1), (1, 1)),       # 1 x 3 taps, 15 steps
     (3, 5, 5, 32, 104, 2, 2, (0, 1, 0, 1), (1, 1), (1, 1)),       # 4 steps, one each; four channel tiles, the last of 8
 ]
