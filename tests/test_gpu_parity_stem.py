@@ -97,3 +97,32 @@ def test_stem_declines_what_it_does_not_take(ctx):
         w = rng.integers(-128, 128, (oc, k, k, ic)).astype(np.int8)
         with pytest.raises(TmiError, match="no MFMA / vector kernel is eligible"):
             gpu_ops.conv2d(ctx, x, w, np.zeros(oc, np.int32), (0, 0, 0, 0), (1, 1), dil, in_zp=0, w_zp=w_zp)
+
+
+def test_stem_form_is_skipped_when_the_result_lies_in_the_scratch_buffer():
+    """a fused first layer under precise mode is the convolution into the context's scratch buffer plus the stand-alone
+    RESCALE (type_conversion.cpp:326-346): the first-layer form, which needs that buffer for its own copies, stands back;
+    before and after, the same layer takes it"""
+    rng = np.random.default_rng(12)
+    x = rng.integers(-128, 128, (4, 64, 60, 3), dtype=np.int8)    # (large enough not to be left to the one-result-per-lane kernel)
+    w = rng.integers(-128, 128, (16, 3, 3, 3), dtype=np.int8)
+    bias = rng.integers(-2000, 2000, 16).astype(np.int32)
+    mult = rng.integers(1 << 30, 1 << 31, 16).astype(np.int32)
+    shift = rng.integers(36, 40, 16).astype(np.int8)
+    kw = dict(pad=(1, 1, 1, 1), in_zp=-3, w_zp=0)
+    acc = oracle.conv2d("i8", x, w, bias, **kw)
+    c = Context(0)
+    try:
+        got, st = gpu_ops.conv2d(c, x, w, bias, **kw)
+        assert c.last_kernel == "conv2d_stem_i8" and st == capi.VALID and np.array_equal(got, acc)
+        want, wst = oracle.rescale(acc, mult, shift, out_zp=4, rounding_mode=capi.ROUND_INEXACT, inexact_mode=1)
+        c.set_precise_mode(1, 0, 0)
+        got, st = gpu_ops.conv2d(c, x, w, bias, **kw, rescale=dict(mult=mult, shift=shift, out_zp=4, rounding_mode=capi.ROUND_INEXACT))
+        c.set_precise_mode()
+        assert c.last_kernel in ("rescale_vec_precise", "rescale_scalar_precise")
+        assert st == wst == capi.VALID and np.array_equal(got, want)
+        want, wst = oracle.rescale(acc, mult, shift, out_zp=4)
+        got, st = gpu_ops.conv2d(c, x, w, bias, **kw, rescale=dict(mult=mult, shift=shift, out_zp=4))
+        assert c.last_kernel == "conv2d_stem_i8_rescale" and st == wst == capi.VALID and np.array_equal(got, want)
+    finally:
+        c.close()
