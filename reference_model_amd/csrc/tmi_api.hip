@@ -401,10 +401,12 @@ int validate_fused_rescale(tmi_ctx* ctx, const char* op, const tmi_conv_desc_t* 
     return TMI_VALID;
 }
 
-// check_level: false for the CONV2D that TRANSPOSE_CONV2D / CONV3D are evaluated as (their own limits were checked)
+// check_level: false for the CONV2D that TRANSPOSE_CONV2D / CONV3D are evaluated as (their own limits were checked).
+// own_scratch: false when the caller holds operands of its own in a scratch buffer (the context's or the static one of
+// the entry point that allocates nothing): then no kernel that would grow or write the context's buffer is chosen.
 int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t* d, const void* in, const void* w,
              const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp, int32_t out_dtype, void* out,
-             bool check_level = true)
+             bool check_level = true, bool own_scratch = true)
 {
     ConvGeom g;
     int rc = validate_conv(ctx, op, d, depthwise, in_zp, w_zp, g);
@@ -517,7 +519,7 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
                                         ctx->flags_dev);
         // First layers (at most 4 input channels, 3 x 3 ... 7 x 7 taps): a pre-pass into the scratch buffer and the pointwise
         // kernel with a K step per row of taps, unless an operand of this call lies in that buffer already.
-        if (!name && (ctx->kernel_choice == 5 || ctx->kernel_choice == 0))
+        if (!name && own_scratch && (ctx->kernel_choice == 5 || ctx->kernel_choice == 0))
         {
             const size_t need = conv2d_stem_scratch_bytes(d->in_dtype, out_dtype, g, w_zp, rp);
             auto in_scratch   = [&](const void* p) {
@@ -982,7 +984,7 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
                 : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
         return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
-                    d->out_dtype, out_dev, false);
+                    d->out_dtype, out_dev, false, false);
 }
 
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
@@ -1118,7 +1120,8 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
     if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
                                 d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
         return fail(ctx, "%s: operand re-layout launch failed", op);
-    return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev, false);
+    return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev, false,
+                    false);
 }
 
 // The fused operators under INEXACT_ROUND in precise mode: the convolution's INT32 results go to the scratch buffer and

@@ -88,6 +88,25 @@ def test_noalloc_matches_transpose_conv2d_twice(fp):
         ctx.close()
 
 
+@pytest.mark.parametrize("ic", [3, 4])
+def test_noalloc_stays_off_the_kernel_that_needs_the_contexts_buffer(ic):
+    """At most 4 input channels, 3 x 3 taps, weight zero point 0: as a CONV2D this layer goes to the first-layer
+    kernel, whose pre-pass writes the context's scratch buffer (growing it on demand).  Reached from
+    TRANSPOSE_CONV2D the convolution must take another kernel: its operands lie in scratch memory already, and the
+    entry point that allocates nothing may not grow anything."""
+    rng = np.random.default_rng(977 + ic)
+    ctx = Context(0)
+    try:
+        assert ctx.workspace_bytes() == (0, 0)
+        for shape, oc, out_pad, stride in (((2, 9, 7, ic), 16, (0, 1, 1, 0), (2, 2)), ((1, 6, 5, ic), 8, (0, 0, 0, 0), (1, 1))):
+            x, w, b, dt, in_zp, _ = _operands(rng, shape, oc, 3, False)
+            want, got = _run_both(ctx, x, w, b, dt, in_zp, 0, out_pad, stride)
+            assert np.array_equal(want, got)
+            assert np.array_equal(got, oracle.transpose_conv2d("i8", x, w, b, out_pad, stride, in_zp, 0))
+    finally:
+        ctx.close()
+
+
 def test_noalloc_refuses_operands_beyond_the_static_array():
     """The input with its stride holes alone exceeds TMI_NOALLOC_SCRATCH_BYTES: TMI_ERROR, nothing launched (the
     operand pointers are never dereferenced: they are small valid buffers)."""
