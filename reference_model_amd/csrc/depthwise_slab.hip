@@ -411,6 +411,9 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     static thread_local Choice last = { { 0, 0, 0, 0, 0, 0, 0, 0 }, 0, 0, 0 };
     const int32_t key[8] = { g.N, g.OH, g.OW, C, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
     int best_th = 0, best_tw = 0, best_nw = 0;
+    // weights, both forms of the requantisation constants, multipliers, bias terms, the table waves' shifts
+    const int table_bytes = 9 * C * 4 + C * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + C * 8 + 32;
+    constexpr int lds_max = 160 * 1024;
     if (memcmp(key, last.key, sizeof(key)) == 0)
         best_th = last.th, best_tw = last.tw, best_nw = last.nw;
     else
@@ -422,7 +425,8 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
                 const int ph = (th - 1) * g.stride_y + 2 * g.dil_y + 1;
                 const int pw = (tw - 1) * g.stride_x + 2 * g.dil_x + 1;
                 const int64_t slots = (int64_t)ph * (pw * ppitch + 15);
-                if (slots >= (1 << 16) || slots * 16 > 96 * 1024)
+                // (the patch is rounded up to whole rounds of 64 slots, and a row may take up to 15 chunks of padding)
+                if (slots >= (1 << 16) || slots * 16 > 96 * 1024 || slots * 16 + 1024 + table_bytes > lds_max)
                     continue;
                 const int units        = ((th * tw + 31) / 32) * n_cblk;
                 const int64_t tiles    = (int64_t)g.N * ((g.OH + th - 1) / th) * ((g.OW + tw - 1) / tw);
@@ -489,7 +493,9 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_cblk = make_fastdiv((uint32_t)n_cblk);
     const int p_loads   = (a.PH * a.pitch + 63) / 64;
-    const int lds_bytes = p_loads * 1024 + 9 * C * 4 + C * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + C * 8 + 32;
+    const int lds_bytes = p_loads * 1024 + table_bytes;
+    if (lds_bytes > lds_max)
+        return nullptr;
     bool ok;
     if (in_zp != 0)
         ok = rp.enabled ? launch_dwslab_kernel<true, true>(st, a, (int)grid, per_round, lds_bytes)

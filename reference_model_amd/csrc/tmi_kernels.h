@@ -28,7 +28,10 @@ inline bool ensure_dynamic_lds(const void* kernel, size_t bytes, LdsLimit& lim)
     if (bytes <= lim.done[dev].load(std::memory_order_acquire))
         return true;
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess)
+    {
+        (void)hipGetLastError();    // the caller goes on to another kernel, whose launch must not inherit this error
         return false;
+    }
     lim.done[dev].store(bytes, std::memory_order_release);
     return true;
 }

@@ -33,6 +33,7 @@ DW_SHAPES = [  # n, ih, iw, c, pad, stride, dilation
     (2, 14, 14, 576, (1, 1, 1, 1), (1, 1), (1, 1)),     # 18 channel blocks: more channels than eight waves have lanes
     (2, 7, 7, 960, (1, 1, 1, 1), (1, 1), (1, 1)),       # 30 channel blocks
     (1, 10, 10, 1024, (0, 1, 0, 1), (2, 2), (1, 1)),    # the most channels the kernel takes
+    (3, 29, 33, 1024, (0, 2, 0, 2), (1, 1), (1, 1)),    # ... whose tables leave 66 KB of the LDS for the patch
 ]
 
 
@@ -157,6 +158,20 @@ def test_automatic_choice_takes_the_matrix_core_kernel_for_its_layers():
         c.set_kernel_choice(capi.KERNEL_AUTO)
         got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=4, w_zp=2, depthwise=True)
         assert st == capi.VALID and c.last_kernel == "depthwise_dot4_i8"    # weight zero point: the vector kernel
+    finally:
+        c.close()
+
+
+def test_a_kernel_that_declines_leaves_no_error_for_the_next_one():
+    """1024 channels on more than 256 tiles: the matrix-core kernel has no shape for the layer (eight waves do not
+    have a lane per channel) and the vector kernel runs it; nothing of the first attempt may show in the call's status."""
+    c = Context(0)
+    try:
+        shape = (8, 40, 40, 1024, (1, 1, 1, 1), (1, 1), (1, 1))
+        x, w, bias = _operands(shape, 11)
+        got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=-128, depthwise=True)
+        assert st == capi.VALID and c.last_kernel.startswith("depthwise_")
+        assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, shape[4], shape[5], in_zp=-128, w_zp=0))
     finally:
         c.close()
 
