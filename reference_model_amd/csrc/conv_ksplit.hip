@@ -324,8 +324,13 @@ const char* launch_conv2d_ksplit(hipStream_t st, int32_t in_dtype, int32_t out_d
     a.n_oct    = (g.OC + 31) / 32;
     a.n_pt     = (int32_t)((P + 31) / 32);
     a.steps = steps, a.spt = g.IC / 32, a.ksw = ksw;
-    const int max_groups = 2048 / a.n_oct > 0 ? 2048 / a.n_oct : 1;
-    a.n_groups = a.n_pt < max_groups ? a.n_pt : max_groups;
+    // At most one workgroup per CU, each walking its pixel tiles with the weight fragments in registers (us for a
+    // workgroup per tile / at most 256 workgroups, 3x3, fused RESCALE: [8,14,14,256]->256 10.9 / 9.0, [16,14,14,256]->256
+    // 18.5 / 12.8, [4,28,28,256]->256 19.6 / 12.9, [8,14,14,384]->384 24.1 / 15.3; 320 workgroups: 17.0 and 23.0 on the last
+    // two, 192: 14.8 and 18.2).
+    const int max_groups = 256 / a.n_oct > 0 ? 256 / a.n_oct : 1;
+    const int per_group  = (a.n_pt + max_groups - 1) / max_groups;    // pixel tiles a workgroup walks: the same for all
+    a.n_groups = (a.n_pt + per_group - 1) / per_group;
     a.div_oct = make_fastdiv((uint32_t)a.n_oct), a.div_spt = make_fastdiv((uint32_t)a.spt);
     a.div_kw = make_fastdiv((uint32_t)g.KW), a.div_ow = make_fastdiv((uint32_t)g.OW), a.div_oh = make_fastdiv((uint32_t)g.OH);
     const int grid = a.n_groups * a.n_oct;

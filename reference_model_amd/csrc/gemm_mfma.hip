@@ -1389,6 +1389,12 @@ bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g)
     // 66.2 / 49.5; with 32 channels the two tie ([16,112,112,32]->128 stride 2 13.2 / 13.4).
     if (in_dtype != TMI_INT8 && g.IC >= 64 && g.OC >= 96 && tiles >= 196)
         return true;
+    // int8 layers below 120 tiles: the patch kernel, whose set-up is the shorter one (us patch kernel / this kernel's patch
+    // form, 3x3, fused RESCALE: [4,28,28,256]->256 (50 tiles) 14.5 / 17.3, [8,28,28,256]->256 (98) 15.0 / 17.3,
+    // [32,14,14,256]->256 15.2 / 17.3, [16,14,14,512]->512 (100) 23.6 / 26.7, [8,14,14,384]->384 18.8 / 24.1; int32 results
+    // [8,28,28,256]->256 15.8 / 16.3; from 147 tiles on the other way: [12,28,28,256]->256 18.1 / 17.5, [16,..] 19.7 / 18.1).
+    if (in_dtype == TMI_INT8 && tiles < 120)
+        return false;
     int rows, patch_h, patch_w;
     const int icb = g.IC * (in_dtype == TMI_INT8 ? 1 : 2);
     return patch_form_geometry(g.OH, g.OW, g.KH, g.KW, g.stride_y, g.stride_x, g.dil_y, g.dil_x, icb, g.OC, rows,

@@ -378,9 +378,15 @@ __global__ __launch_bounds__(kSplitWaves * 64, 2) void pointwise_ksplit_i8_kerne
             const int k0 = kbase + 32 * s + 16 * lh;
             if (s < ksw)
             {
-                const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
-                const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
-                fa[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
+                // (a load instruction costs the memory pipeline the same for 8 or 16 bytes a lane)
+                if (!by8)
+                    fa[s] = *reinterpret_cast<const v4i*>(row + (k0 < a.IC ? k0 : 0));
+                else
+                {
+                    const v2i lo = *reinterpret_cast<const v2i*>(row + (k0 < a.IC ? k0 : 0));
+                    const v2i hi = *reinterpret_cast<const v2i*>(row + (k0 + 8 < a.IC ? k0 + 8 : 0));
+                    fa[s]        = v4i{ lo.x, lo.y, hi.x, hi.y };
+                }
             }
         }
         // what lies past IC or past OC is zeroed once all loads have been issued
@@ -555,11 +561,16 @@ const char* launch_conv2d_pointwise(hipStream_t st, int32_t in_dtype, int32_t ou
     a.div_oct  = make_fastdiv((uint32_t)a.n_oct);
     if (g.IC > 160)
     {
-        // K split over the four waves of a workgroup; a workgroup per tile up to 8 workgroups on each CU
+        // K split over the four waves of a workgroup.  A workgroup walks several pixel tiles with its weight fragments in
+        // registers once the layer has more than 640 tiles: about two workgroups per CU is where the weight loads saved and
+        // the tiles a workgroup works through one after the other balance (us for 1 / 2 / 3 / 4 tiles a workgroup, fused
+        // RESCALE: [8,28,28,512]->128 6.8 / 6.5 / 7.0 / -, [8,14,14,1024]->512 10.6 / 8.6 / 9.2 / 8.8, [8,28,28,512]->256
+        // 11.1 / 9.0 / 8.8 / 9.2, [8,56,56,256]->64 8.7 / - / 7.0 / 7.5, [8,14,14,256]->1024 8.3 / - / 6.7 / 7.4).
         const int ksteps = (g.IC + 31) / 32;
         a.ksw            = (ksteps + kSplitWaves - 1) / kSplitWaves;
-        const int max_groups = 2048 / a.n_oct > 0 ? 2048 / a.n_oct : 1;
-        a.n_groups       = a.n_pt < max_groups ? a.n_pt : max_groups;
+        const int max_groups = 640 / a.n_oct > 0 ? 640 / a.n_oct : 1;
+        const int per_group = (a.n_pt + max_groups - 1) / max_groups;    // pixel tiles a workgroup walks: the same for all
+        a.n_groups       = (a.n_pt + per_group - 1) / per_group;
         const int grid   = a.n_groups * a.n_oct;
         if (!fastdiv_exact_up_to((uint64_t)grid, (uint32_t)a.n_oct))
             return nullptr;

@@ -470,17 +470,21 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // 4.9 / 6.0, [8,56,56,128]->128 5.1 / 6.1) and this kernel takes what that one declines; with 144 and 160 there is
         // only the patch kernel to beat ([8,56,56,144]->24 10.2 / 3.1, [8,7,7,160]->960 5.4 / 3.2).  Large int32 results
         // stay with the GEMM kernel above ([8,56,56,64]->256 8.1 / 11.8, [8,28,28,128]->512 6.3 / 8.9).
-        // With more than 160 input channels the pointwise kernel splits K over the four waves of a workgroup, one workgroup
-        // per tile of 32 x 32 results: the better form while the layer is small (at most 450 M multiply-adds) and the GEMM
-        // kernel would have few tiles of 128 x 128 for the chip, or does not take the layer (fewer than 64 output channels,
-        // channel vectors that are not multiples of 64 bytes).  us GEMM or patch kernel / this form, fused RESCALE:
-        // [8,28,28,192]->32 9.2 / 3.2, [8,14,14,384]->64 7.4 / 3.9, [8,14,14,576]->96 8.2 / 4.3, [8,7,7,960]->320 9.7 / 4.8,
-        // [8,7,7,320]->1280 7.4 / 4.6, [8,14,14,1024]->256 (26 tiles) 10.1 / 8.4, [8,7,7,2048]->512 (16) 14.2 / 8.8; ties at
-        // [8,28,28,512]->128 (49 tiles) 8.1 / 8.4 and [8,7,7,512]->2048 (64) 8.1 / 8.2; the other way: [8,56,56,256]->64 (196)
-        // 7.4 / 10.0, [8,14,14,256]->1024 (104) 7.2 / 9.9, [8,56,56,256]->128 7.6 / 13.2, [8,14,14,1024]->512 10.1 / 15.2.
+        // With more than 160 input channels the pointwise kernel splits K over the four waves of a workgroup, a workgroup
+        // per tile of 32 x 32 results (or per few of them): the better form while the layer is small, up to 500 M
+        // multiply-adds on at most 1600 such tiles, or up to 900 M where the GEMM kernel would have at most 64 tiles of
+        // 128 x 128 for the chip.  us GEMM kernel / this form, fused RESCALE: [8,28,28,192]->32 9.2 / 3.3, [8,14,14,384]->64
+        // 7.4 / 3.8, [8,7,7,960]->320 9.7 / 4.3, [8,7,7,320]->1280 7.4 / 4.2, [8,14,14,1024]->256 10.0 / 6.9, [8,7,7,2048]->512
+        // 14.2 / 7.5, [8,28,28,512]->128 8.1 / 6.5, [8,7,7,512]->2048 8.0 / 6.4, [8,14,14,256]->1024 7.2 / 6.7, [8,56,56,256]->64
+        // 7.1 / 7.0, [8,28,28,256]->256 7.1 / 6.7, [32,14,14,384]->96 7.6 / 5.3, [8,28,28,256]->128 7.0 / 5.3, [32,7,7,960]->320
+        // 9.7 / 5.7; 500 - 900 M: [8,14,14,1024]->512 (52 tiles) 10.0 / 8.6, [8,28,28,1024]->128 (49) 10.1 / 8.7, [8,14,14,2048]->256
+        // (26) 14.2 / 11.0; the other way: [8,28,28,192]->384 (2352 small tiles) 7.0 / 7.6, [8,28,28,512]->256 (98 tiles of
+        // 128 x 128) 8.2 / 8.8, [8,14,14,768]->768 (78) 9.1 / 10.1, [8,56,56,256]->128 7.4 / 10.5.
         const int64_t pixels   = (int64_t)g.N * g.OH * g.OW;
         const int64_t tiles128 = ((pixels + 127) / 128) * ((g.OC + 127) / 128);
-        const bool deep_first  = g.IC > 160 && total * g.IC <= 450000000ll && (tiles128 <= 48 || g.OC < 64 || (g.IC & 63));
+        const int64_t tiles32  = ((pixels + 31) / 32) * ((g.OC + 31) / 32);
+        const int64_t macs     = total * g.IC * g.KH * g.KW;
+        const bool deep_first  = g.IC > 160 && ((macs <= 500000000ll && tiles32 <= 1600) || (macs <= 900000000ll && tiles128 <= 64));
         if (!name && ctx->kernel_choice == 0 && (g.IC <= 112 || deep_first))
             name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                            ctx->flags_dev);
@@ -506,14 +510,18 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         if (!name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
-        // Layers with taps that are small and deep (at most 32 tiles of 128 x 128 results, at most 1 G multiply-adds) and
-        // not the slab kernel's: a workgroup per tile of 32 x 32 results with K split over its waves, before the patch and
-        // GEMM kernels, which would keep a tenth of the chip busy.  us patch kernel / this kernel, 3x3, fused RESCALE:
-        // [8,14,14,256]->256 14.3 / 10.8, [8,28,28,256]->256 stride 2 16.2 / 10.8, [8,7,7,512]->512 21.1 / 10.8,
-        // [8,14,14,512]->512 stride 2 22.5 / 10.8, [8,14,14,160]->160 13.6 / 4.5, [1,14,14,256]->256 14.2 / 6.9; the other
-        // way beyond: [12,14,14,256]->256 (38 tiles) 14.4 / 14.9, [16,..] 14.5 / 18.5 (the GEMM kernel's patch form 17.1),
-        // [4,28,28,256]->256 14.4 / 19.6, [8,14,14,384]->384 (2.1 G multiply-adds) 18.8 / 24.1.
-        const bool split_first = g.KH * g.KW > 1 && tiles128 <= 32 && total * g.IC * g.KH * g.KW <= 1000000000ll;
+        // Layers with taps that are small and deep (at most 2.4 G multiply-adds on at most 64 tiles of 128 x 128 results, or
+        // on at most 100 from 160 input channels on) and not the slab kernel's: workgroups that own tiles of 32 x 32 results
+        // with K split over their waves, before the patch and GEMM kernels, which would keep a fraction of the chip busy.
+        // us patch kernel / this kernel, 3x3, fused RESCALE: [8,14,14,256]->256 14.3 / 9.0, [8,28,28,256]->256 stride 2
+        // 16.2 / 9.1, [8,7,7,512]->512 21.1 / 10.8, [8,14,14,512]->512 stride 2 22.5 / 10.8, [8,14,14,160]->160 13.6 / 4.5,
+        // [1,14,14,256]->256 14.2 / 6.9, [16,14,14,256]->256 (50 tiles) 14.4 / 12.8, [20,14,14,256]->256 (62) 14.5 / 12.8,
+        // [8,14,14,384]->384 18.8 / 15.2, [8,14,14,256]->512 14.5 / 12.8, [8,14,14,512]->256 23.2 / 15.7, [16,7,7,512]->512
+        // 21.2 / 15.1, [8,14,14,320]->320 16.6 / 8.8, [8,28,28,160]->160 (98) 13.8 / 9.2, [8,28,28,192]->192 (98) 12.1 / 11.4,
+        // 5x5 [8,14,14,192]->192 31.1 / 11.1, [8,56,56,32]->32 stride 2 6.8 / 3.9; ties at [24,14,14,256]->256 (74 tiles, 2.8 G)
+        // 14.6 / 15.0 and [32,7,7,512]->512 21.2 / 21.8; the other way: [32,14,14,256]->256 (98, 3.7 G) 15.2 / 18.7,
+        // [16,14,14,512]->512 23.6 / 34.2, [8,56,56,32]->64 (196) 5.3 / 11.9, [8,112,112,32]->32 8.1 / 19.5.
+        const bool split_first = g.KH * g.KW > 1 && macs <= 2400000000ll && (tiles128 <= 64 || (g.IC >= 160 && tiles128 <= 100));
         if (!name && g.KH * g.KW > 1 && (ctx->kernel_choice == 5 || (ctx->kernel_choice == 0 && split_first)))
             name = launch_conv2d_ksplit(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                         ctx->flags_dev);
