@@ -257,7 +257,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
             // most 0 for a multiplier >= 0), so that form skips the sign test (bit 8).
             const int relu = a.rp.double_round && a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
             if (lane == 0)
-                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? -2 : -1);
+                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? (relu ? -3 : -2) : -1);
         }
         tab_m[lane] = m;
         tab_b[lane] = ok ? b : 0;
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         int32_t r[16];
         const int form  = __builtin_amdgcn_readfirstlane(*uni_shift);
         const int s_uni = form >= 0 ? (form & 255) : form;
-        const int relu  = form >= 0 ? (form >> 8) : 0;
+        const int relu  = form >= 0 ? (form >> 8) : (form == -3);    // (-3: the per-channel high-word form without the sign test)
         if (s_uni >= 0)
         {
             // one shift for every channel: the high-word form with its constants in scalar registers
@@ -425,9 +425,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                     r[e] = clamp_med3(high_word_rescale<false>(acck[e], cm[e], hi_p, lo_p, sh), a.rp.lo, a.rp.hi);
             }
         }
-        else if (s_uni == -2)
+        else if (s_uni <= -2)
         {
-            if (a.rp.double_round)
+            if (a.rp.double_round && !relu)
             {
 #pragma unroll
                 for (int e = 0; e < 16; e++)
@@ -659,7 +659,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
             tab_hw[lane]    = make_high_word_scale(cs, a.rp.out_zp);
             const int relu = a.rp.double_round && a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
             if (lane == 0)
-                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? -2 : -1);
+                *uni_shift = uni ? (s_first | (relu << 8)) : (folds ? (relu ? -3 : -2) : -1);
             tab_m[lane] = cs.m;
         }
         tab_b[lane] = ok ? a.bias[a.bias_len == 1 ? 0 : occ] : 0;
@@ -911,8 +911,9 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
                         pk2[2 * g - 4] = w0, pk2[2 * g - 3] = w1;
                 }
             };
-            if (form == -2)
+            if (form <= -2)
             {
+                const bool sign_test = a.rp.double_round && form == -2;    // (-3: a negative value is clamped away either way)
 #pragma unroll
                 for (int g = 0; g < 4; g++)
                 {
@@ -921,7 +922,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
                     for (int j = 0; j < 4; j++)
                     {
                         const HighWordScale c = tab_hw[ocl + 4 * g + j];
-                        r[j] = a.rp.double_round ? clamp_med3(high_word_rescale<true>(acc[4 * g + j], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi)
+                        r[j] = sign_test ? clamp_med3(high_word_rescale<true>(acc[4 * g + j], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi)
                                                  : clamp_med3(high_word_rescale<false>(acc[4 * g + j], c.m, c.hi, c.lo, c.sh), a.rp.lo, a.rp.hi);
                     }
                     pack(g, r);

@@ -156,7 +156,10 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 2) void conv_ksplit_i8_kern
             const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
             const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
             const int s_min       = a.rp.double_round ? 33 : 32;
-            const int form        = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0;
+            // bit 0: the high-word form for all 32 channels; bit 1: no sign test in it (a negative value is clamped away
+            // with either rounding term: the result's lower limit is at or above output_zp and no multiplier is negative)
+            const int form = (__all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0) |
+                             (a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0) ? 2 : 0);
             if (lh == 0)
             {
                 tab_ms[li] = v2i{ cs.m, cs.s };
@@ -244,9 +247,9 @@ __global__ __launch_bounds__(NW * 64, NW == 16 ? 4 : 2) void conv_ksplit_i8_kern
         for (int j = 0; j < 4; j++)
         {
             const int c = 16 * lh + 4 * wave + j;
-            if (form == 1)
-                r[j] = a.rp.double_round ? clamp_med3(high_word_rescale64<true>(sum[j], tab_hw[c]), v_lo, v_hi)
-                                         : clamp_med3(high_word_rescale64<false>(sum[j], tab_hw[c]), v_lo, v_hi);
+            if (form & 1)
+                r[j] = (a.rp.double_round && !(form & 2)) ? clamp_med3(high_word_rescale64<true>(sum[j], tab_hw[c]), v_lo, v_hi)
+                                                          : clamp_med3(high_word_rescale64<false>(sum[j], tab_hw[c]), v_lo, v_hi);
             else
             {
                 uint32_t f   = 0;

@@ -170,16 +170,20 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
             //   to ride in the 64-bit rounding term: 16 bytes of constants per channel, no value-range test (-2);
             //   the same with one shift for all 64 channels: rounding term and shift are scalars (the shift itself);
             //   anything else: fast_rescale() with its range test and a 64-bit shift (-1).
+            // With double rounding a value below zero takes a rounding term 2^31 smaller; where the result is clamped at or
+            // above output_zp anyway, a negative value ends at the lower limit with either term (the scaled value is at
+            // most 0 for a multiplier >= 0), and the first two forms skip the sign test (bit 8 of the shift; -3).
             const int s_min = a.rp.double_round ? 33 : 32;
             const int folds = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp));
             const int uni   = folds && __all(cs.s == s_first);
+            const int relu  = a.rp.double_round && a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
             if (tab_lane)
             {
                 tab_cs[tid] = cs;
                 tab_hw[tid] = make_high_word_scale(cs, a.rp.out_zp);
             }
             if (lane == 0)
-                uni_shift[wave] = uni ? s_first : (folds ? -2 : -1);
+                uni_shift[wave] = uni ? (s_first | (relu << 8)) : (folds ? (relu ? -3 : -2) : -1);
         }
         if (tab_lane)
         {
@@ -277,10 +281,12 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
         else
         {
             int32_t r[16];
-            const int s_uni = __builtin_amdgcn_readfirstlane(uni_shift[c0 >> 6]);    // the form of this block's group
-            if (s_uni >= 0)
+            const int s_form = __builtin_amdgcn_readfirstlane(uni_shift[c0 >> 6]);    // the form of this block's group
+            const bool sign_test = a.rp.double_round && (s_form >= 0 ? (s_form >> 8) == 0 : s_form == -2);
+            if (s_form >= 0)
             {
                 // one shift for all 64 channels: the high-word form with its constants in scalar registers
+                const int s_uni   = s_form & 255;
                 const int64_t rnd = (int64_t(1) << (s_uni - 1)) + (a.rp.double_round ? (int64_t(1) << 30) : 0) +
                                     ((int64_t)a.rp.out_zp << s_uni);
                 const int sh        = s_uni - 32;
@@ -291,7 +297,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                     const v4i m4 = *reinterpret_cast<const v4i*>(tab_m + clc + 4 * q);
                     cm[4 * q] = m4[0], cm[4 * q + 1] = m4[1], cm[4 * q + 2] = m4[2], cm[4 * q + 3] = m4[3];
                 }
-                if (a.rp.double_round)
+                if (sign_test)
                 {
 #pragma unroll
                     for (int e = 0; e < 16; e++)
@@ -304,9 +310,9 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
                         r[e] = clamp_med3(high_word_rescale64<false>(acc[e], cm[e], rnd, sh), a.rp.lo, a.rp.hi);
                 }
             }
-            else if (s_uni == -2)
+            else if (s_form <= -2)
             {
-                if (a.rp.double_round)
+                if (sign_test)
                 {
 #pragma unroll
                     for (int e = 0; e < 16; e++)

@@ -156,6 +156,10 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
     // ---- per-channel constants: lane li (both halves alike) derives those of channel 32 oct + li ------------------------
     uint32_t flags = 0;
     int form       = 0;    // 1: every channel of the tile takes the high-word form of the requantisation
+    // With double rounding a value below zero takes a rounding term 2^31 smaller; where the result is clamped at or above
+    // output_zp anyway, a negative value ends at the lower limit with either term (the scaled value is at most 0 for a
+    // multiplier >= 0), and the high-word form needs no sign test.
+    bool sign_free = false;
     {
         const int oc  = oct * 32 + li;
         const bool ok = oc < a.OC;
@@ -169,6 +173,7 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
             const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
             const int s_min       = a.rp.double_round ? 33 : 32;
             form                  = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0;
+            sign_free             = a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0);
             if (lh == 0)
             {
                 tab_ms[li] = v2i{ cs.m, cs.s };
@@ -307,8 +312,8 @@ __global__ __launch_bounds__(kPointwiseWaves * 64, KSTEPS <= 2 ? 3 : 2) void poi
     if (!a.rp.enabled)
         run(std::integral_constant<int, 0>{}, std::false_type{});
     else if (form == 1)
-        a.rp.double_round ? run(std::integral_constant<int, 1>{}, std::true_type{})
-                          : run(std::integral_constant<int, 1>{}, std::false_type{});
+        (a.rp.double_round && !sign_free) ? run(std::integral_constant<int, 1>{}, std::true_type{})
+                                          : run(std::integral_constant<int, 1>{}, std::false_type{});
     else
         run(std::integral_constant<int, 2>{}, std::false_type{});
     raise_flags(a.flag_word, flags);
@@ -413,7 +418,10 @@ __global__ __launch_bounds__(kSplitWaves * 64, 2) void pointwise_ksplit_i8_kerne
             const int32_t s_first = __builtin_amdgcn_readfirstlane(s_raw);
             const ChannelScale cs = make_channel_scale(ok ? m_raw : 0, ok ? s_raw : s_first, a.rp.double_round != 0, flags);
             const int s_min       = a.rp.double_round ? 33 : 32;
-            const int form        = __all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0;
+            // bit 0: the high-word form for all 32 channels; bit 1: no sign test in it (a negative value is clamped away
+            // with either rounding term: the result's lower limit is at or above output_zp and no multiplier is negative)
+            const int form = (__all(cs.s >= s_min && cs.s <= zp_fold_max_shift(a.rp.out_zp)) ? 1 : 0) |
+                             (a.rp.lo >= a.rp.out_zp && __all(cs.m >= 0) ? 2 : 0);
             if (lh == 0)
             {
                 tab_ms[li] = v2i{ cs.m, cs.s };
@@ -488,9 +496,9 @@ __global__ __launch_bounds__(kSplitWaves * 64, 2) void pointwise_ksplit_i8_kerne
         for (int j = 0; j < 4; j++)
         {
             const int c = 16 * lh + 4 * wave + j;
-            if (form == 1)
-                r[j] = a.rp.double_round ? clamp_med3(high_word_rescale64<true>(sum[j], tab_hw[c]), v_lo, v_hi)
-                                         : clamp_med3(high_word_rescale64<false>(sum[j], tab_hw[c]), v_lo, v_hi);
+            if (form & 1)
+                r[j] = (a.rp.double_round && !(form & 2)) ? clamp_med3(high_word_rescale64<true>(sum[j], tab_hw[c]), v_lo, v_hi)
+                                                          : clamp_med3(high_word_rescale64<false>(sum[j], tab_hw[c]), v_lo, v_hi);
             else
             {
                 uint32_t f   = 0;
