@@ -997,10 +997,15 @@ static bool launch_slab_wreg(hipStream_t st, const SlabArgs& a, int grid, int ld
     return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true, false>) : launch(conv2d_slab_wreg_kernel<false, false>);
 }
 
-template <int KH, int KW, int CH>
+template <int KH, int KW, int CH, bool WIDE_TOO = true>
 static bool launch_slab_taps(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, bool fused, bool wide)
 {
-    if (wide)
+    if constexpr (!WIDE_TOO)
+    {
+        if (wide)
+            return false;
+    }
+    else if (wide)
     {
         if (a.za != 0)
             return fused ? launch_slab_kernel<KH, KW, CH, true, true, false, 1, 2>(st, a, grid, lds_bytes)
@@ -1022,7 +1027,12 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                const SlabDepth* c3d)
 {
     const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
-    if (in_dtype != TMI_INT8 || (g.IC != 64 && g.IC != 96 && g.IC != 128) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
+    // 64, 96 or 128 input channels; pointwise layers also the common counts from 160 to 1024 (64 weight rows of 1024 bytes
+    // and a patch of 62 pixels still fit the LDS; the K loop is unrolled, so each count is an instantiation of its own)
+    const bool deep11 = k11 && !tc && !c3d &&
+                        (g.IC == 160 || g.IC == 192 || g.IC == 256 || g.IC == 320 || g.IC == 384 || g.IC == 480 || g.IC == 512 ||
+                         g.IC == 576 || g.IC == 768 || g.IC == 960 || g.IC == 1024);
+    if (in_dtype != TMI_INT8 || ((g.IC != 64 && g.IC != 96 && g.IC != 128) && !deep11) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
         return nullptr;
     if (tc && (!k33 || rp.enabled || tc->up_y < 1 || tc->up_x < 1 || g.stride_y != 1 || g.stride_x != 1))
         return nullptr;
@@ -1125,7 +1135,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
         else
         {
             search(124, 600);
-            if (best_th && best_rounds > 1 && g.stride_y == 1 && g.stride_x == 1 && plain)
+            if (best_th && best_rounds > 1 && g.stride_y == 1 && g.stride_x == 1 && plain && ch <= 16)
             {
                 const int th1 = best_th, tw1 = best_tw;
                 search(252, 1100);
@@ -1224,6 +1234,24 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
         ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused, wide)
                      : (ch == 6 ? launch_slab_taps<3, 3, 6>(st, a, (int)grid, lds_bytes, fused, wide)
                                 : launch_slab_taps<3, 3, 8>(st, a, (int)grid, lds_bytes, fused, wide));
+    else if (ch > 8)
+    {
+        switch (ch)    // (one accumulator tile per wave beyond 256 channels: see the tile search)
+        {
+            case 10: ok = launch_slab_taps<1, 1, 10>(st, a, (int)grid, lds_bytes, fused, wide); break;
+            case 12: ok = launch_slab_taps<1, 1, 12>(st, a, (int)grid, lds_bytes, fused, wide); break;
+            case 16: ok = launch_slab_taps<1, 1, 16>(st, a, (int)grid, lds_bytes, fused, wide); break;
+            case 20: ok = launch_slab_taps<1, 1, 20, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 24: ok = launch_slab_taps<1, 1, 24, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 30: ok = launch_slab_taps<1, 1, 30, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 32: ok = launch_slab_taps<1, 1, 32, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 36: ok = launch_slab_taps<1, 1, 36, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 48: ok = launch_slab_taps<1, 1, 48, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 60: ok = launch_slab_taps<1, 1, 60, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            case 64: ok = launch_slab_taps<1, 1, 64, false>(st, a, (int)grid, lds_bytes, fused, false); break;
+            default: ok = false; break;
+        }
+    }
     else
         ok = ch == 4 ? launch_slab_taps<1, 1, 4>(st, a, (int)grid, lds_bytes, fused, wide)
                      : (ch == 6 ? launch_slab_taps<1, 1, 6>(st, a, (int)grid, lds_bytes, fused, wide)

@@ -457,7 +457,7 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // whole lines, before the slab kernel (us slab / GEMM, host clock: [8,56,56,64]->256 12.8 / 8.8,
         // [32,56,56,64]->256 35.9 / 21.6, [8,28,28,128]->512 8.3 / 6.6, [32,28,28,128]->512 24.0 / 14.5; smaller ones
         // and every layer with the fused RESCALE are the slab kernel's: 5.3 / 5.5, fused 6.9 / 10.1, 19.6 / 28.3).
-        if (ctx->kernel_choice == 0 && !rp.enabled && g.KH * g.KW == 1 && total > (int64_t(1) << 21))
+        if (ctx->kernel_choice == 0 && !rp.enabled && g.KH * g.KW == 1 && total > (int64_t(1) << 21) && g.IC <= 128)
             name = launch_gemm_mfma(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, 0, 0,
                                     pad_page, ctx->flags_dev);
         // Pointwise int8 layers with up to 112 input channels: the kernel that keeps a wave on one tile of 32 output channels
@@ -485,6 +485,24 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         const int64_t tiles32  = ((pixels + 31) / 32) * ((g.OC + 31) / 32);
         const int64_t macs     = total * g.IC * g.KH * g.KW;
         const bool deep_first  = g.IC > 160 && ((macs <= 500000000ll && tiles32 <= 1600) || (macs <= 900000000ll && tiles128 <= 64));
+        // Pointwise layers with 160 ... 1024 input channels (the counts the slab kernel is instantiated for): its weight slab,
+        // 64 rows of up to 1 KB, and a patch of 62 ... 124 pixels fit the LDS as those of 3 x 3 taps on 64 channels do, so it
+        // comes before all of these - up to 256 channels at every size, beyond while the layer fits one round of
+        // workgroups (900 M multiply-adds): a workgroup then takes 75 ... 135 KB of LDS, one fits a CU, and from the second
+        // round on the GEMM kernel leads.  us slab / K-split pointwise / GEMM kernel, fused RESCALE:
+        // [8,56,56,256]->64 4.2 / 7.0 / 7.2, [32,..] 7.7 / 17.6 / 19.9, [8,56,56,256]->128 5.7 / 10.6 / 7.4, [32,..] 16.7 / 30.0 / 21.7,
+        // [8,56,56,256]->512 16.8 / 28.7 / 19.2, [8,14,14,256]->1024 4.1 / 6.8 / 7.1, [32,..] 7.6 / 16.0 / 11.1, [1,14,14,256]->1024
+        // 3.4 / 3.5 / 6.9; [8,28,28,512]->128 4.2 / 6.6 / 8.1, [16,..] 4.9 / 9.5 / 8.2, [8,28,28,512]->256 4.9 / 8.9 / 8.2,
+        // [8,7,7,512]->2048 4.2 / 6.6 / 8.1, [1,7,7,512]->512 3.6 / 4.0 / -, [8,14,14,1024]->256 4.7 / 6.8 / 10.0, [8,14,14,1024]->512
+        // 5.1 / 8.7 / 10.0, [8,28,28,192]->64 3.3 / 3.7 / 6.6, [8,56,56,192]->64 3.8 / 6.3 / 6.9, [8,28,28,384]->192 4.3 / 7.0 / 7.7,
+        // [8,28,28,192]->384 5.1 / 7.8 / 7.0, [32,14,14,384]->96 4.0 / 5.4 / 7.5; the other way: [32,28,28,512]->128 (1.6 G)
+        // 10.8 / 15.8 / 8.5, [16,28,28,512]->256 10.8 / 15.8 / 8.5, [32,7,7,512]->2048 10.7 / 13.0 / 8.5, [8,28,28,512]->1024
+        // 20.1 / 22.7 / 12.9, [32,14,14,1024]->256 11.9 / 16.1 / 10.2.  int32 results: [32,56,56,256]->64 15.0 / 17.3 / 17.3,
+        // [8,14,14,256]->1024 5.6 / 6.1 / 6.0, [8,14,14,1024]->256 4.4 / 6.3 / 8.3.
+        const bool slab_deep = g.KH * g.KW == 1 && g.IC > 128 && g.IC <= 1024 && (g.IC <= 256 || macs <= 900000000ll);
+        if (!name && ctx->kernel_choice == 0 && slab_deep)
+            name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
+                                      ctx->flags_dev);
         if (!name && ctx->kernel_choice == 0 && (g.IC <= 112 || deep_first))
             name = launch_conv2d_pointwise(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                            ctx->flags_dev);
@@ -507,7 +525,8 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
                 name = launch_conv2d_direct(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                             ctx->flags_dev);
         }
-        if (!name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
+        // (left open, the slab kernel's layers with more than 128 input channels are the ones tried above)
+        if (!name && (ctx->kernel_choice == 4 || (ctx->kernel_choice == 0 && g.IC <= 128)))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
         // Layers with taps that are small and deep (at most 2.4 G multiply-adds on at most 64 tiles of 128 x 128 results, or

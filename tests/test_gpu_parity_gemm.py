@@ -428,8 +428,10 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (4, 28, 28, 256, 256, 3, 1), "gemm_mfma_f16_patch"),   # 56 tiles of four output rows: enough for the patch form
     (capi.INT8, (16, 14, 14, 256, 256, 3, 1), "conv2d_ksplit_i8"),     # 50 tiles, 1.8 G multiply-adds: K split over the waves of small workgroups
     (capi.INT8, (32, 14, 14, 256, 256, 3, 1), "conv2d_mfma_i8"),       # 98 tiles, 3.7 G: too much for that, too few tiles for the GEMM kernel
-    (capi.INT8, (8, 14, 14, 1024, 512, 1, 0), "conv2d_pointwise_ksplit_i8"),    # pointwise, 822 M multiply-adds on 52 tiles
-    (capi.INT8, (8, 28, 28, 512, 256, 1, 0), "gemm_mfma_i8"),          # the same on 98 tiles: the GEMM kernel
+    (capi.INT8, (8, 14, 14, 1024, 512, 1, 0), "conv2d_slab_i8"),       # pointwise on 1024 channels, one round of workgroups: the slab kernel
+    (capi.INT8, (8, 7, 7, 2048, 512, 1, 0), "conv2d_pointwise_ksplit_i8"),    # 2048 channels, 411 M multiply-adds on 16 tiles: K split over waves
+    (capi.INT8, (8, 28, 28, 512, 256, 1, 0), "conv2d_slab_i8"),        # pointwise on 512 channels, one round of workgroups: the slab kernel
+    (capi.INT8, (16, 28, 28, 512, 256, 1, 0), "gemm_mfma_i8"),         # two rounds: the GEMM kernel
     (capi.FP16, (2, 28, 28, 256, 256, 3, 1), "conv2d_mfma_f16"),       # 28 tiles: too few
     (capi.FP16, (1, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_f16"),       # pointwise with 16 tiles: still the GEMM kernel
     (capi.FP16, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_f16"),          # 3x3, no patch form (49 pixels a tile), 100 tiles

@@ -125,10 +125,24 @@ def test_slab_conv_fused_rescale_bit_exact(ctx, shape, zps, out_dtype):
     (3, 17, 13, 64, 80, (1, 0, 0, 2), (1, 1)),          # padding on a pointwise layer: the border is bias only
     (9, 61, 47, 64, 192, (0, 0, 0, 0), (1, 1)),         # two accumulator tiles per wave, ragged tiles
     (5, 33, 35, 128, 320, (1, 0, 0, 2), (1, 1)),        # the same with padding and five channel blocks
+    (2, 28, 28, 256, 64, (0, 0, 0, 0), (1, 1)),         # 256 input channels: 8 K steps, 17 chunks per patch pixel
+    (3, 14, 14, 256, 208, (0, 0, 0, 0), (1, 1)),        # ... four channel blocks, the last of 16
+    (2, 28, 28, 512, 128, (0, 0, 0, 0), (1, 1)),        # 512 input channels: 16 K steps
+    (2, 15, 13, 512, 80, (0, 0, 1, 1), (2, 2)),         # ... with a stride and padding
+    (9, 40, 40, 256, 64, (0, 0, 0, 0), (1, 1)),         # 256 channels, two accumulator tiles per wave
+    (2, 14, 14, 160, 64, (0, 0, 0, 0), (1, 1)),         # every other channel count the kernel is built for: 5 K steps
+    (10, 38, 38, 192, 48, (0, 0, 0, 0), (1, 1)),        # ... 6, two accumulator tiles per wave
+    (2, 14, 14, 320, 96, (0, 0, 0, 0), (1, 1)),         # ... 10
+    (2, 15, 14, 384, 64, (1, 1, 0, 0), (1, 1)),         # ... 12
+    (2, 14, 14, 480, 112, (0, 0, 0, 0), (1, 1)),        # ... 15
+    (2, 14, 14, 576, 96, (0, 0, 0, 0), (1, 1)),         # ... 18
+    (2, 9, 14, 768, 64, (0, 0, 0, 0), (1, 1)),          # ... 24
+    (2, 7, 7, 960, 160, (0, 0, 0, 0), (1, 1)),          # ... 30
+    (3, 14, 14, 1024, 144, (0, 0, 0, 0), (1, 1)),       # ... 32 K steps of a weight row of 1 KB, tiles of 62 pixels
 ])
 @pytest.mark.parametrize("in_zp", [0, -7])
 def test_slab_pointwise_layers_bit_exact(ctx, shape, in_zp):
-    """1x1 taps with 64 or 128 input channels: too little K for the GEMM kernel, one or two MFMA steps here"""
+    """1x1 taps with 64 ... 512 input channels: little K for the GEMM kernel, 2 ... 16 MFMA steps here"""
     n, ih, iw, ic, oc, pad, stride = shape
     rng = np.random.default_rng(ih * oc + ic)
     x = rng.integers(-128, 128, (n, ih, iw, ic)).astype(np.int8)
