@@ -133,7 +133,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
             const int iy = y0 + py, ix = x0 + px;
             const bool img = py < a.PH && px < a.PW && (unsigned)iy < (unsigned)a.IH && (unsigned)ix < (unsigned)a.IW;
             const int cc   = ch < a.cpp ? ch : 0;    // the spare chunk of a pixel reads its first one
-            const uint8_t* src = img ? in_n + (uint32_t)(__umul24(__umul24(iy, a.IW) + ix, C) + cc * 16)
+            const uint8_t* src = img ? in_n + mad_u24(mad_u24((uint32_t)iy, (uint32_t)a.IW, (uint32_t)ix), (uint32_t)C, (uint32_t)(cc * 16))
                                      : a.pad_page + (cc & 3) * 16;
             dwslab_load(src, dst);
             dst += nwaves * 1024;

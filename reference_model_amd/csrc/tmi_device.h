@@ -29,6 +29,16 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f)
     return f.d <= 1 ? n : __umulhi(n, f.magic);
 }
 
+// a * b + c on the 24-bit multiplier with three 32-bit operands (a and b below 2^24).  Left to the compiler, a * b + c
+// becomes a 64-bit multiply-add whose addend's upper half is whatever register is at hand, and where that register is the
+// destination of a load in flight, the instruction - and every load the wave has yet to issue - waits for that load.
+__device__ __forceinline__ uint32_t mad_u24(uint32_t a, uint32_t b, uint32_t c)
+{
+    uint32_t r;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // The same quotient on the host (the multiply-high written out).
 inline uint32_t fdiv_host(uint32_t n, FastDiv f)
 {
