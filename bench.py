@@ -80,7 +80,8 @@ def main() -> int:
                     help="times the region of --steps steps is run; the median repeat is reported "
                          "(default: enough repeats for 10000 steps, between 5 and 500)")
     ap.add_argument("--copy-mib", type=int, default=1024, help="buffer size of --config copy")
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy", "launch_floor"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy", "launch_floor", "networks"])
+    ap.add_argument("--batch", type=int, default=8, help="images per layer of --config networks")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     ap.add_argument("--no-named-configs", action="store_true",
                     help="default configuration only: skip the short GPU legs of the other named configurations")
@@ -162,6 +163,76 @@ def main() -> int:
             out[name] = {"GB_per_s": round(moved / t / 1e9, 1), "us": round(t * 1e6, 2), "bytes_moved": moved,
                          "frac_of_8TBps": round(moved / t / 8e12, 4)}
         print(json.dumps(out))
+        ctx.close()
+        return 0
+    if cfg == "networks":
+        # Beyond the named configurations: the int8 layers of ResNet-50 (the first and a following block of every stage)
+        # and MobileNetV2 (every block), CONV2D or DEPTHWISE_CONV2D with the fused per-channel RESCALE under the library's
+        # own kernel choice, each timed alone by graph replay.  "floor" is the launch floor plus the larger of ops / 5 POP/s and bytes / 8 TB/s.
+        N, rng, layers = args.batch, np.random.default_rng(cases.SEED), []
+        layers.append(("r50 conv1 7x7 s2", False, 224, 3, 64, 7, 2))
+        for hw, cin, mid, cout, s in ((56, 64, 64, 256, 1), (56, 256, 64, 256, 1), (56, 256, 128, 512, 2), (28, 512, 128, 512, 1),
+                                      (28, 512, 256, 1024, 2), (14, 1024, 256, 1024, 1), (14, 1024, 512, 2048, 2), (7, 2048, 512, 2048, 1)):
+            layers.append(("r50 1x1 %d->%d @%d" % (cin, mid, hw), False, hw, cin, mid, 1, 1))
+            layers.append(("r50 3x3 %d s%d @%d" % (mid, s, hw), False, hw, mid, mid, 3, s))
+            layers.append(("r50 1x1 %d->%d @%d" % (mid, cout, hw // s), False, hw // s, mid, cout, 1, 1))
+        layers.append(("mbv2 conv1 3x3 s2", False, 224, 3, 32, 3, 2))
+        layers.append(("mbv2 dw 32 s1 @112", True, 112, 32, 32, 3, 1))
+        layers.append(("mbv2 1x1 32->16 @112", False, 112, 32, 16, 1, 1))
+        for hw, cin, e, cout, s in ((112, 16, 96, 24, 2), (56, 24, 144, 24, 1), (56, 24, 144, 32, 2), (28, 32, 192, 32, 1),
+                                    (28, 32, 192, 64, 2), (14, 64, 384, 64, 1), (14, 64, 384, 96, 1), (14, 96, 576, 96, 1),
+                                    (14, 96, 576, 160, 2), (7, 160, 960, 160, 1), (7, 160, 960, 320, 1)):
+            layers.append(("mbv2 1x1 %d->%d @%d" % (cin, e, hw), False, hw, cin, e, 1, 1))
+            layers.append(("mbv2 dw %d s%d @%d" % (e, s, hw), True, hw, e, e, 3, s))
+            layers.append(("mbv2 1x1 %d->%d @%d" % (e, cout, hw // s), False, hw // s, e, cout, 1, 1))
+        layers.append(("mbv2 1x1 320->1280 @7", False, 7, 320, 1280, 1, 1))
+        launch_floor_us, rows = 1.67, []
+        for name, depthwise, hw, ic, oc, k, s in layers:
+            p = k // 2
+            oh = (hw + 2 * p - k) // s + 1
+            ih = (oh - 1) * s + k - 2 * p    # exact output size
+            x = to_dev(rng.integers(-128, 128, (N, ih, ih, ic), dtype=np.int8))
+            w = to_dev(rng.integers(-128, 128, (k, k, ic, 1) if depthwise else (oc, k, k, ic), dtype=np.int8))
+            macs = N * oh * oh * oc * k * k * (1 if depthwise else ic)
+            b = to_dev(rng.integers(-1000, 1000, oc, dtype=np.int32))
+            m = to_dev(rng.integers(1 << 29, 1 << 30, oc, dtype=np.int32))
+            sh = to_dev(np.full(oc, 38, np.int8))
+            out = torch.empty((N, oh, oh, oc), dtype=torch.int8, device=dev)
+            d = ctx.conv_desc(capi.INT8, capi.INT32, (N, ih, ih, ic), oc, k, k, (oh, oh), (p, p, p, p), (s, s), (1, 1), oc)
+            r = ctx.rescale_desc(capi.INT32, capi.INT8, oc, oc, 0, 3, True, capi.ROUND_DOUBLE, True)
+            fn = ctx.depthwise_conv2d_rescale_clamp if depthwise else ctx.conv2d_rescale_clamp
+
+            def step():
+                fn(d, x, w, b, -3, 0, r, m, sh, out, None)
+            for _ in range(5):
+                step()
+            torch.cuda.synchronize()
+            kernel = ctx.last_kernel
+            g, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+            side.wait_stream(stream)
+            with torch.cuda.graph(g, stream=side):
+                ctx.set_stream(side.cuda_stream)
+                for _ in range(50):
+                    step()
+            ctx.set_stream(stream.cuda_stream)
+            g.replay()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(15):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1) * 20.0)
+            us = sorted(ts)[len(ts) // 2]
+            nbytes = x.numel() + w.numel() + out.numel() + 9 * oc
+            floor = launch_floor_us + max(2 * macs / 5e15, nbytes / 8e12) * 1e6
+            rows.append({"layer": name, "us": round(us, 2), "floor_us": round(floor, 2), "kernel": kernel})
+        print(json.dumps({"metric": "sum over 62 int8 layers of ResNet-50 and MobileNetV2, each timed alone",
+                          "unit": "us", "value": round(sum(r["us"] for r in rows), 1), "higher_is_better": False,
+                          "floor_us": round(sum(r["floor_us"] for r in rows), 1), "batch": N, "n_gpus": 1, "data": "synthetic",
+                          "dtype": "int8", "config": {"workload": "int8 CONV2D / DEPTHWISE_CONV2D + RESCALE, per layer", "layers": rows}}))
         ctx.close()
         return 0
     def make_workload(cfg):
