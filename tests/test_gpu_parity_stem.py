@@ -33,6 +33,9 @@ SHAPES = [
     (2, 12, 40, 3, 72, 3, 7, (1, 1, 3, 3), (1, 3), (1, 1)),      # 3 x 7 taps, horizontal stride 3
     (1, 7, 7, 4, 8, 7, 7, (0, 0, 0, 0), (1, 1), (1, 1)),         # one output pixel per image
     (5, 6, 6, 3, 8, 3, 3, (0, 0, 0, 0), (1, 1), (1, 1)),         # no padding
+    (2, 9, 30, 1, 16, 3, 11, (1, 1, 5, 5), (1, 1), (1, 1)),      # 11 taps a row: the copy keeps a pixel per byte
+    (1, 11, 27, 2, 8, 5, 9, (2, 2, 4, 4), (2, 2), (1, 1)),       # 9 taps of 2 channels: a pixel every 2 bytes
+    (1, 12, 29, 4, 24, 3, 8, (1, 1, 3, 4), (1, 1), (1, 1)),      # 8 taps of 4 channels: a row of taps fills the K step
 ]
 
 
