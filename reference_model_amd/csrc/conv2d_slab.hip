@@ -92,9 +92,12 @@ __device__ __forceinline__ void slab_barrier()
 // NPT: accumulator tiles (of 32 columns) per wave.  Two of them share every weight fragment, which cuts the LDS
 // traffic of the K loop by a quarter; the workgroup's tile is then up to 252 pixels, which only pays when the layer
 // has more tiles than the chip has CUs.
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1>
+// T: int8_t, or _Float16 / bf16_t: the same loads and LDS layout on channel vectors of CH * 8 values, fp32 accumulators that
+// start at the bias, results rounded to T (tensor_ops.cpp:828-882 with fp32 accumulation); no zero points, no RESCALE.
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1, typename T = int8_t>
 __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
 {
+    static_assert(Mma<T>::is_int || (!ZA && !FUSED && !TC && KD == 1), "floating point: plain CONV2D only");
     // one field of every cache line of the arguments up front: a single scalar-cache round trip
     // every scalar argument the kernel reads, named once so that they are fetched together at the top (fields
     // first needed later are otherwise loaded one at a time, each with its own wait)
@@ -230,7 +233,11 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         const int oc    = oc0 + lane;
         const bool ok   = oc < a.OC;
         const int occ   = ok ? oc : 0;
-        const int32_t b = a.bias[a.bias_len == 1 ? 0 : occ];
+        int32_t b;    // the accumulator's start value: an int32, or the bits of a float
+        if constexpr (Mma<T>::is_int)
+            b = a.bias[a.bias_len == 1 ? 0 : occ];
+        else
+            b = __float_as_int(load_as_float<T>(a.bias, a.bias_len == 1 ? 0 : occ));
         int32_t m       = 0;
         if constexpr (FUSED)
         {
@@ -290,7 +297,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     }
     // The accumulators start at the bias of the lane's 16 channels (the zero-point column at zero).
     const int ocl = oct * 32 + 16 * lh;    // first of the lane's 16 channels inside the block
-    v16i acc[NPT];
+    typename Mma<T>::acc_t acc[NPT];
 #pragma unroll
     for (int k = 0; k < NPT; k++)
     {
@@ -299,7 +306,14 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
         for (int q = 0; q < 4; q++)
         {
             const v4i b4 = *reinterpret_cast<const v4i*>(b16 + 4 * q);
-            acc[k][4 * q] = b4[0], acc[k][4 * q + 1] = b4[1], acc[k][4 * q + 2] = b4[2], acc[k][4 * q + 3] = b4[3];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                if constexpr (Mma<T>::is_int)
+                    acc[k][4 * q + j] = b4[j];
+                else
+                    acc[k][4 * q + j] = __int_as_float(b4[j]);
+            }
         }
     }
     const bool wave_active = pxt * WPIX < P;                     // wave-uniform
@@ -349,7 +363,7 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
                 request(s + DEPTH);
 #pragma unroll
             for (int k = 0; k < NPT; k++)
-                acc[k] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[s], fb[k][s], acc[k], 0, 0, 0);
+                acc[k] = Mma<T>::mma(fa[s], fb[k][s], acc[k]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -376,12 +390,29 @@ __global__ __launch_bounds__(512) void conv2d_slab_kernel(SlabArgs a)
     {
     if (k > 0 && !second_active)
         break;
-    const v16i& acck = acc[k];
+    const auto& acck = acc[k];
     const int oy = oy0 + ty[k], ox = ox0 + tx[k];
     const bool pix_ok  = p_in_tile[k] && wave_active && oy < a.OH && ox < a.OW;
     // the tensor has fewer than 2^31 elements (checked by the launcher): 32-bit arithmetic, scalar where it can be
     const size_t obase = (uint32_t)(((n * a.OH + oy) * a.OW + ox) * a.OC + oc0 + ocl);
-    if constexpr (!FUSED)
+    if constexpr (!Mma<T>::is_int)
+    {
+        // 16 consecutive channels of one pixel, rounded to the tensor's type: 32 bytes
+        if (pix_ok && chan_ok)
+        {
+            union
+            {
+                T e[16];
+                v4i q[2];
+            } u;
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                store_from_float(&u.e[e], acck[e]);
+            v4i* o = reinterpret_cast<v4i*>(reinterpret_cast<T*>(a.out) + obase);
+            o[0] = u.q[0], o[1] = u.q[1];
+        }
+    }
+    else if constexpr (!FUSED)
     {
         if (pix_ok && chan_ok)
         {
@@ -966,10 +997,10 @@ __global__ __launch_bounds__(512) void conv2d_slab_wreg_kernel(SlabArgs a)
 
 thread_local int32_t last_launch_shape[3] = { 0, 0, 0 };
 
-template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1>
+template <int KH, int KW, int CH, bool ZA, bool FUSED, bool TC = false, int KD = 1, int NPT = 1, typename T = int8_t>
 static bool launch_slab_kernel(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes)
 {
-    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC, KD, NPT>;
+    auto kern              = conv2d_slab_kernel<KH, KW, CH, ZA, FUSED, TC, KD, NPT, T>;
     static LdsLimit granted{};
     if (!ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (size_t)lds_bytes, granted))
         return false;
@@ -995,6 +1026,22 @@ static bool launch_slab_wreg(hipStream_t st, const SlabArgs& a, int grid, int ld
     if (vl)
         return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true, true>) : launch(conv2d_slab_wreg_kernel<false, true>);
     return a.za != 0 ? launch(conv2d_slab_wreg_kernel<true, false>) : launch(conv2d_slab_wreg_kernel<false, false>);
+}
+
+// the floating-point instantiations: fp16 (kind 1) or bf16 (kind 2)
+template <int KH, int KW, int CH, bool WIDE_TOO = true>
+static bool launch_slab_taps_fp(hipStream_t st, const SlabArgs& a, int grid, int lds_bytes, int kind, bool wide)
+{
+    if constexpr (WIDE_TOO)
+    {
+        if (wide)
+            return kind == 1 ? launch_slab_kernel<KH, KW, CH, false, false, false, 1, 2, _Float16>(st, a, grid, lds_bytes)
+                             : launch_slab_kernel<KH, KW, CH, false, false, false, 1, 2, bf16_t>(st, a, grid, lds_bytes);
+    }
+    else if (wide)
+        return false;
+    return kind == 1 ? launch_slab_kernel<KH, KW, CH, false, false, false, 1, 1, _Float16>(st, a, grid, lds_bytes)
+                     : launch_slab_kernel<KH, KW, CH, false, false, false, 1, 1, bf16_t>(st, a, grid, lds_bytes);
 }
 
 template <int KH, int KW, int CH, bool WIDE_TOO = true>
@@ -1027,12 +1074,19 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                                const SlabDepth* c3d)
 {
     const bool k33 = g.KH == 3 && g.KW == 3, k11 = g.KH == 1 && g.KW == 1;
-    // 64, 96 or 128 input channels; pointwise layers also the common counts from 160 to 1024 (64 weight rows of 1024 bytes
-    // and a patch of 62 pixels still fit the LDS; the K loop is unrolled, so each count is an instantiation of its own)
+    // fp16 / bf16: plain CONV2D without zero points; what counts below is the bytes of a channel vector
+    const int fp = in_dtype == TMI_FP16 ? 1 : (in_dtype == TMI_BF16 ? 2 : 0);
+    if (fp && (tc || c3d || rp.enabled || out_dtype != in_dtype || in_zp != 0 || ((uintptr_t)bias & 1)))
+        return nullptr;
+    const int icb = g.IC * (fp ? 2 : 1);
+    // channel vectors of 64, 96 or 128 bytes; pointwise layers also the common sizes from 160 to 1024 bytes (64 weight rows
+    // of 1024 bytes and a patch of 62 pixels still fit the LDS; the K loop is unrolled, so each size is an instantiation of
+    // its own, and floating point has a few less)
     const bool deep11 = k11 && !tc && !c3d &&
-                        (g.IC == 160 || g.IC == 192 || g.IC == 256 || g.IC == 320 || g.IC == 384 || g.IC == 480 || g.IC == 512 ||
-                         g.IC == 576 || g.IC == 768 || g.IC == 960 || g.IC == 1024);
-    if (in_dtype != TMI_INT8 || ((g.IC != 64 && g.IC != 96 && g.IC != 128) && !deep11) || !(k33 || k11) || w_zp != 0 || !pad_page || !flag_word)
+                        (icb == 160 || icb == 192 || icb == 256 || icb == 320 || icb == 384 || icb == 512 || icb == 768 || icb == 1024 ||
+                         (!fp && (icb == 480 || icb == 576 || icb == 960)));
+    if ((in_dtype != TMI_INT8 && !fp) || ((icb != 64 && icb != 96 && icb != 128) && !deep11) || !(k33 || k11) || w_zp != 0 || !pad_page ||
+        !flag_word)
         return nullptr;
     if (tc && (!k33 || rp.enabled || tc->up_y < 1 || tc->up_x < 1 || g.stride_y != 1 || g.stride_x != 1))
         return nullptr;
@@ -1044,13 +1098,13 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
             return nullptr;
     }
     const int taps = g.KH * g.KW;
-    if (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32)
+    if (!fp && (rp.enabled ? (!rp.fast || (out_dtype != TMI_INT8 && out_dtype != TMI_INT16)) : out_dtype != TMI_INT32))
         return nullptr;
     if (g.OC < 48 || g.OC > 65536 || (g.OC & 15) || g.N < 1 || g.OH < 1 || g.OW < 1)
         return nullptr;
-    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || ((uintptr_t)bias & 3))
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)out | (uintptr_t)pad_page) & 15) || (!fp && ((uintptr_t)bias & 3)))
         return nullptr;
-    if ((int64_t)g.N * g.IH * g.IW * g.IC >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
+    if ((int64_t)g.N * g.IH * g.IW * icb >= (int64_t(1) << 31) || (int64_t)g.N * g.OH * g.OW * g.OC >= (int64_t(1) << 31))
         return nullptr;
 
     // The tile: at most 124 pixels (four tiles of 31 pixels, one per wave and channel tile).  A workgroup moves the
@@ -1065,7 +1119,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     // a single round of the small tiles is faster with them ([8,56,56,64]->64 4.3 / 5.1, [16,28,28,128]->128 5.5 / 6.4),
     // and so is stride 2, whose patch grows with the tile ([32,57,57,128]->64 9.5 / 11.7).
     const int n_ocb = (g.OC + 63) / 64;
-    const int ch = g.IC / 16, rp_chunks = ch + 1;    // chunks of a channel vector; chunks per patch pixel in LDS
+    const int ch = icb / 16, rp_chunks = ch + 1;    // chunks of a channel vector; chunks per patch pixel in LDS
     struct TileChoice
     {
         int32_t key[8];
@@ -1183,7 +1237,7 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
     a.div_tiles_x = make_fastdiv((uint32_t)a.tiles_x), a.div_tiles_y = make_fastdiv((uint32_t)a.tiles_y);
     a.div_ocb = make_fastdiv((uint32_t)n_ocb);
     const int w_loads = taps * ch + 1, p_loads = (a.PH * a.pitch + 63) / 64;
-    const int ones_bytes = (g.KH - 1) * g.dil_y * a.pitch * 16 + (g.KW - 1) * g.dil_x * rp_chunks * 16 + g.IC;
+    const int ones_bytes = (g.KH - 1) * g.dil_y * a.pitch * 16 + (g.KW - 1) * g.dil_x * rp_chunks * 16 + icb;
     const int lds_bytes  = (w_loads + p_loads) * 1024 + ones_bytes + 64 * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + 64 * 4 + 80 * 4 + 16;
     const bool fused = rp.enabled != 0;
     bool ok;
@@ -1229,6 +1283,32 @@ const char* launch_conv2d_slab(hipStream_t st, int32_t in_dtype, int32_t out_dty
                          : (ch == 6 ? launch_slab_kernel<3, 3, 6, false, false, true>(st, a, (int)grid, lds_bytes)
                                     : launch_slab_kernel<3, 3, 8, false, false, true>(st, a, (int)grid, lds_bytes));
         return ok ? "transpose_conv2d_slab_i8" : nullptr;
+    }
+    if (fp)
+    {
+        if (k33)
+            ok = ch == 4 ? launch_slab_taps_fp<3, 3, 4>(st, a, (int)grid, lds_bytes, fp, wide)
+                         : (ch == 6 ? launch_slab_taps_fp<3, 3, 6>(st, a, (int)grid, lds_bytes, fp, wide)
+                                    : launch_slab_taps_fp<3, 3, 8>(st, a, (int)grid, lds_bytes, fp, wide));
+        else
+            switch (ch)
+            {
+                case 4: ok = launch_slab_taps_fp<1, 1, 4>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 6: ok = launch_slab_taps_fp<1, 1, 6>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 8: ok = launch_slab_taps_fp<1, 1, 8>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 10: ok = launch_slab_taps_fp<1, 1, 10>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 12: ok = launch_slab_taps_fp<1, 1, 12>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 16: ok = launch_slab_taps_fp<1, 1, 16>(st, a, (int)grid, lds_bytes, fp, wide); break;
+                case 20: ok = launch_slab_taps_fp<1, 1, 20, false>(st, a, (int)grid, lds_bytes, fp, false); break;
+                case 24: ok = launch_slab_taps_fp<1, 1, 24, false>(st, a, (int)grid, lds_bytes, fp, false); break;
+                case 32: ok = launch_slab_taps_fp<1, 1, 32, false>(st, a, (int)grid, lds_bytes, fp, false); break;
+                case 48: ok = launch_slab_taps_fp<1, 1, 48, false>(st, a, (int)grid, lds_bytes, fp, false); break;
+                case 64: ok = launch_slab_taps_fp<1, 1, 64, false>(st, a, (int)grid, lds_bytes, fp, false); break;
+                default: ok = false; break;
+            }
+        if (!ok)
+            return nullptr;
+        return fp == 1 ? "conv2d_slab_f16" : "conv2d_slab_bf16";
     }
     if (k33)
         ok = ch == 4 ? launch_slab_taps<3, 3, 4>(st, a, (int)grid, lds_bytes, fused, wide)

@@ -499,8 +499,23 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
         // 10.8 / 15.8 / 8.5, [16,28,28,512]->256 10.8 / 15.8 / 8.5, [32,7,7,512]->2048 10.7 / 13.0 / 8.5, [8,28,28,512]->1024
         // 20.1 / 22.7 / 12.9, [32,14,14,1024]->256 11.9 / 16.1 / 10.2.  int32 results: [32,56,56,256]->64 15.0 / 17.3 / 17.3,
         // [8,14,14,256]->1024 5.6 / 6.1 / 6.0, [8,14,14,1024]->256 4.4 / 6.3 / 8.3.
-        const bool slab_deep = g.KH * g.KW == 1 && g.IC > 128 && g.IC <= 1024 && (g.IC <= 256 || macs <= 900000000ll);
+        const bool slab_deep = d->in_dtype == TMI_INT8 && g.KH * g.KW == 1 && g.IC > 128 && g.IC <= 1024 && (g.IC <= 256 || macs <= 900000000ll);
         if (!name && ctx->kernel_choice == 0 && slab_deep)
+            name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
+                                      ctx->flags_dev);
+        // fp16 / bf16 on the slab kernel (channel vectors of 64 ... 128 bytes under 3 x 3 taps, up to 1024 bytes under 1 x 1):
+        // every 3 x 3 layer it takes, and the pointwise ones up to 1.6 M results - beyond, the GEMM kernel's whole-line stores
+        // win.  us patch or GEMM kernel / slab kernel, fp16: 3x3 [8,56,56,64]->64 7.2 / 4.8, ->128 8.4 / 6.9, stride 2 10.3 / 4.1,
+        // [32,56,56,64]->64 18.7 / 12.7, [8,56,56,32]->64 4.8 / 3.8, [8,28,28,48]->96 7.0 / 3.7; 1x1 [8,28,28,256]->128 4.2 / 3.6,
+        // [8,14,14,512]->256 5.0 / 4.0, [1,14,14,512]->512 4.9 / 3.5, [8,28,28,96]->192 3.7 / 3.2, [8,56,56,256]->64 4.6 / 4.4,
+        // [8,14,14,256]->1024 4.5 / 4.4; the other way: [8,28,28,128]->512 (3.2 M results) 4.7 / 5.3, [8,56,56,64]->256 6.2 / 6.7,
+        // [32,28,28,256]->128 5.4 / 7.7, [32,56,56,64]->256 15.8 / 20.4.  Large 3 x 3 layers: stride 1 [2,160,160,64]->128 17.2 / 13.9,
+        // [8,160,160,64]->96 50.9 / 47.7, [8,56,56,64]->256 16.6 / 13.9, [16,28,28,64]->256 8.5 / 7.5; with a stride the patch grows
+        // with the tile, and from 160 tiles of 128 x 128 on the GEMM kernel leads: [16,56,56,64]->128 stride 2 (98 tiles) 9.5 / 7.7,
+        // [32,..] (196) 10.3 / 13.2, [64,..] 17.3 / 25.0, [32,56,56,64]->256 17.0 / 24.8.
+        const bool fp16b = d->in_dtype == TMI_FP16 || d->in_dtype == TMI_BF16;
+        const bool fp_slab33 = g.KH * g.KW == 9 && !(g.stride_y * g.stride_x > 1 && tiles128 >= 160);
+        if (!name && ctx->kernel_choice == 0 && fp16b && (fp_slab33 || (g.KH * g.KW == 1 && total <= 1600000)))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
         if (!name && ctx->kernel_choice == 0 && (g.IC <= 112 || deep_first))
@@ -526,7 +541,7 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
                                             ctx->flags_dev);
         }
         // (left open, the slab kernel's layers with more than 128 input channels are the ones tried above)
-        if (!name && (ctx->kernel_choice == 4 || (ctx->kernel_choice == 0 && g.IC <= 128)))
+        if (!name && (ctx->kernel_choice == 4 || (ctx->kernel_choice == 0 && g.IC <= 128 && d->in_dtype == TMI_INT8)))
             name = launch_conv2d_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out, pad_page,
                                       ctx->flags_dev);
         // Layers with taps that are small and deep (at most 2.4 G multiply-adds on at most 64 tiles of 128 x 128 results, or

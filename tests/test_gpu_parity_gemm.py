@@ -436,12 +436,12 @@ def test_conv2d_fused_rescale_gemm_reports_require_conditions(ctx):
     (capi.FP16, (1, 14, 14, 1024, 1024, 1, 0), "gemm_mfma_f16"),       # pointwise with 16 tiles: still the GEMM kernel
     (capi.FP16, (64, 7, 7, 512, 512, 3, 1), "gemm_mfma_f16"),          # 3x3, no patch form (49 pixels a tile), 100 tiles
     (capi.FP16, (32, 7, 7, 512, 512, 3, 1), "conv2d_mfma_f16"),        # the same with 52 tiles: the patch kernel
-    (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_mfma_f16"),         # 3x3 fp16, IC 64, too few output channels for the patch form
-    (capi.FP16, (8, 56, 56, 64, 128, 3, 1), "gemm_mfma_f16_patch"),    # the same with 128: the GEMM kernel's patch form
-    (capi.FP16, (32, 56, 56, 64, 128, 3, 1, 2), "gemm_mfma_f16"),      # and with stride 2, 196 tiles: its taps form
+    (capi.FP16, (8, 56, 56, 64, 64, 3, 1), "conv2d_slab_f16"),         # 3x3 fp16 on 128-byte channel vectors: the slab kernel
+    (capi.FP16, (8, 56, 56, 64, 128, 3, 1), "conv2d_slab_f16"),        # the same with 128 output channels
+    (capi.FP16, (32, 56, 56, 64, 128, 3, 1, 2), "gemm_mfma_f16"),      # and with stride 2, 196 tiles: the GEMM kernel's taps form
     (capi.FP16, (16, 56, 56, 128, 64, 3, 1), "conv2d_mfma_f16"),       # 128 channels in, 64 out: half of the GEMM kernel's tile empty
     (capi.FP16, (16, 56, 56, 128, 96, 3, 1), "gemm_mfma_f16"),         # 96 out
-    (capi.FP16, (16, 56, 56, 64, 128, 3, 1, 2), "conv2d_mfma_f16"),    # 98 tiles: the patch kernel
+    (capi.FP16, (16, 56, 56, 64, 128, 3, 1, 2), "conv2d_slab_f16"),    # 98 tiles: the slab kernel
     (capi.FP16, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_f16"),          # pointwise with two blocks of K
     (capi.INT8, (8, 56, 56, 64, 256, 1, 0), "gemm_mfma_i8"),           # int8 pointwise, int32 results, 6.4 M of them: before the slab kernel
     (capi.INT8, (8, 56, 56, 64, 64, 1, 0), "conv2d_pointwise_i8"),     # the same with 1.6 M results: the pointwise kernel
