@@ -405,9 +405,10 @@ int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank,
 
 /* Forces a kernel family for the following operator calls: 0 = automatic choice, 1 = direct (one output
  * element per lane, any shape), 2 = MFMA implicit-GEMM ("patch") kernel, 3 = MFMA GEMM kernel with direct
- * loads into LDS (CONV2D and MATMUL), 4 = the kernels that load operands straight into LDS for small int8 layers (CONV2D 3x3 / 1x1 with 64 or 128
- * input channels, DEPTHWISE_CONV2D 3x3), 5 = the int8 kernels that take both operands straight from global memory (CONV2D 1x1 with 16 ... 2048 input channels;
- * small deep layers with taps);
+ * loads into LDS (CONV2D and MATMUL), 4 = the kernels that hold a weight slab and an input patch in LDS (CONV2D 3x3 / 1x1
+ * on channel vectors of 64 ... 128 bytes, 1x1 on up to 1024 bytes, int8 / fp16 / bf16; int8 DEPTHWISE_CONV2D 3x3),
+ * 5 = the int8 kernels that take both operands straight from global memory (CONV2D 1x1 with 16 ... 2048 input
+ * channels; small deep layers with taps; first layers with at most 4 channels);
  * 2, 3, 4 and 5 return TMI_ERROR if the shape is not eligible.  Used by the parity tests to check every kernel on the
  * same operands. */
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
