@@ -437,7 +437,12 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     // [8,7,7,512] 4.9 / 3.4, [8,7,7,960] 6.8 / 4.1, [2,14,14,576] 5.1 / 3.8, [4,14,14,576] 5.3 / 4.8, [1,28,28,192] 3.8 / 3.4,
     // [8,10,10,672] 5.6 / 5.0; the other way: [1,56,56,144] 3.9 / 4.3, [8,14,14,576] 5.3 / 7.2, [8,14,14,1024] 7.1 / 7.5,
     // [8,28,28,384] 4.8 / 9.5, [32,14,14,576] 5.8 / 14.7.
-    if (depthwise && ctx->kernel_choice == 0 && total < 34000 + 850 * (int64_t)g.IC)
+    // fp16 / bf16 depthwise layers with channels in multiples of 8: the vector kernel (us one-result-per-lane kernel / this
+    // one, fp16 3x3: [8,112,112,96] stride 2 25.6 / 8.1, [8,112,112,32] 31.0 / 8.6, [8,56,56,144] 31.6 / 10.7, [8,28,28,192]
+    // 11.4 / 5.6, [8,14,14,576] 9.4 / 5.2, [64,112,112,96] stride 2 182 / 38.5)
+    if (depthwise && ctx->kernel_choice != 1 && !rp.enabled && (d->in_dtype == TMI_FP16 || d->in_dtype == TMI_BF16))
+        name = launch_depthwise_fp_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, out);
+    if (depthwise && !name && ctx->kernel_choice == 0 && total < 34000 + 850 * (int64_t)g.IC)
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
     if (depthwise && !name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))

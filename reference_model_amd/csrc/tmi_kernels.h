@@ -181,6 +181,10 @@ const char* launch_gemm_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype
                              void* out, int64_t w_batch_stride, int64_t w_kmajor_stride = 0,
                              const void* pad_page = nullptr, uint32_t* flag_word = nullptr);
 
+// fp16 / bf16 DEPTHWISE_CONV2D, 8 channels per lane (depthwise_fp.hip); nullptr when the layer is not eligible.
+const char* launch_depthwise_fp_vec(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
+                                    const void* w, const void* bias, void* out);
+
 // conv2d_mfma.hip: implicit GEMM on the matrix cores with the fused epilogue; nullptr when not eligible.
 const char* launch_conv2d_mfma(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
