@@ -408,8 +408,9 @@ int tmi_rescale_check(tmi_ctx_t* ctx, const tmi_rescale_desc_t* r, int32_t rank,
  * loads into LDS (CONV2D and MATMUL), 4 = the kernels that hold a weight slab and an input patch in LDS (CONV2D 3x3 / 1x1
  * on channel vectors of 64 ... 128 bytes, 1x1 on up to 1024 bytes, int8 / fp16 / bf16; int8 DEPTHWISE_CONV2D 3x3),
  * 5 = the int8 kernels that take both operands straight from global memory (CONV2D 1x1 with 16 ... 2048 input
- * channels; small deep layers with taps; first layers with at most 4 channels);
- * 2, 3, 4 and 5 return TMI_ERROR if the shape is not eligible.  Used by the parity tests to check every kernel on the
+ * channels; small deep layers with taps; first layers with at most 4 channels), 6 = the int8 DEPTHWISE_CONV2D 3x3
+ * kernel whose waves load the pixel operand of the matrix instruction straight from global memory;
+ * 2, 3, 4, 5 and 6 return TMI_ERROR if the shape is not eligible.  Used by the parity tests to check every kernel on the
  * same operands. */
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice);
 

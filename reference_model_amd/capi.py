@@ -18,7 +18,7 @@ VALID, UNPREDICTABLE, ERROR = 0, 1, 2
 INT8, INT16, INT32, INT48, FP32, FP16, BF16 = 3, 4, 5, 6, 7, 8, 9
 ROUND_SINGLE, ROUND_INEXACT, ROUND_DOUBLE = 1, 2, 3
 FLAG_SCALE_MULTIPLIER, FLAG_SCALE_SHIFT, FLAG_SCALE_VALUE, FLAG_SCALE_RESULT, FLAG_ZP_RESULT = 1, 2, 4, 8, 16
-KERNEL_AUTO, KERNEL_DIRECT, KERNEL_MFMA, KERNEL_GEMM, KERNEL_SLAB, KERNEL_POINTWISE = 0, 1, 2, 3, 4, 5
+KERNEL_AUTO, KERNEL_DIRECT, KERNEL_MFMA, KERNEL_GEMM, KERNEL_SLAB, KERNEL_POINTWISE, KERNEL_STREAM = 0, 1, 2, 3, 4, 5, 6
 
 F64 = -64  # host-side tag of the fp64 buffers of the precise / bounds passes (not a TOSA element type)
 DTYPE_SIZE = {INT8: 1, INT16: 2, INT32: 4, INT48: 8, FP32: 4, FP16: 2, BF16: 2, F64: 8}

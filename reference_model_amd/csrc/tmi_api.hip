@@ -445,10 +445,13 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     if (depthwise && !name && ctx->kernel_choice == 0 && total < 34000 + 850 * (int64_t)g.IC)
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
+    if (depthwise && !name && ctx->kernel_choice == 6)
+        name = launch_depthwise_stream(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
+                                       ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);
     if (depthwise && !name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
         name = launch_depthwise_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                      ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);
-    if (depthwise && !name && ctx->kernel_choice != 1 && ctx->kernel_choice != 4)
+    if (depthwise && !name && ctx->kernel_choice != 1 && ctx->kernel_choice != 4 && ctx->kernel_choice != 6)
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
     if (!depthwise && ctx->kernel_choice != 1)
@@ -748,7 +751,7 @@ int tmi_ctx_set_precise_mode(tmi_ctx_t* ctx, int32_t precise_mode, int32_t compl
 
 int tmi_ctx_set_kernel_choice(tmi_ctx_t* ctx, int32_t choice)
 {
-    if (!ctx || choice < 0 || choice > 5)
+    if (!ctx || choice < 0 || choice > 6)
         return TMI_ERROR;
     ctx->kernel_choice = choice;
     return TMI_VALID;

@@ -32,6 +32,8 @@ LAYERS = [
     (capi.KERNEL_SLAB, (2, 20, 20, 128, 96, 1, 0, 1), False, "conv2d_slab_i8_rescale"),
     (capi.KERNEL_SLAB, (2, 21, 21, 96, 96, 3, 1, 1), True, "depthwise_mfma_i8_rescale"),
     (capi.KERNEL_SLAB, (1, 15, 15, 320, 320, 3, 1, 2), True, "depthwise_mfma_i8_rescale"),
+    (capi.KERNEL_STREAM, (2, 21, 21, 96, 96, 3, 1, 1), True, "depthwise_stream_i8_rescale"),
+    (capi.KERNEL_STREAM, (1, 15, 15, 336, 336, 3, 1, 2), True, "depthwise_stream_i8_rescale"),
 ]
 
 
