@@ -445,9 +445,16 @@ int run_conv(tmi_ctx* ctx, const char* op, bool depthwise, const tmi_conv_desc_t
     if (depthwise && !name && ctx->kernel_choice == 0 && total < 34000 + 850 * (int64_t)g.IC)
         name = launch_depthwise_vec(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                     ctx->flags_dev);
-    if (depthwise && !name && ctx->kernel_choice == 6)
+    // Layers with at most 48 channels and 1.6 M results or more: the kernel whose waves load the pixel operand straight from
+    // global memory (a pixel is one or two 32-byte pieces, neighbouring lanes read neighbouring memory; us LDS-patch kernel /
+    // this one, fused RESCALE: [8,112,112,32] 6.5 / 5.3, [32,...] 16.8 / 11.9, [64,...] 29.9 / 20.8, stride 2 11.9 / 8.6,
+    // [64,56,56,32] 10.8 / 7.8, [64,56,56,48] 13.4 / 11.7, [8,150,150,32] 9.9 / 6.4; the other way: [4,112,112,32] 4.2 / 4.1
+    // is the border, [8,56,56,32] 3.6 / 3.9, [8,56,56,48] 3.9 / 4.1).  With 64 channels and more a load instruction takes 32
+    // bytes out of every pixel and the L1 looks up a line per lane: [64,112,112,64] 40.8 / 43.4, [64,112,112,96] stride 2
+    // 23.0 / 28.7, [32,28,28,384] 10.1 / 20.4.
+    if (depthwise && !name && (ctx->kernel_choice == 6 || (ctx->kernel_choice == 0 && g.IC <= 48 && total >= 1600000)))
         name = launch_depthwise_stream(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
-                                       ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);
+                                       ctx->flags_dev);
     if (depthwise && !name && (ctx->kernel_choice == 0 || ctx->kernel_choice == 4))
         name = launch_depthwise_slab(ctx->stream, d->in_dtype, out_dtype, g, in, w, bias, in_zp, w_zp, rp, out,
                                      ctx->pages_dev + (in_zp & 255) * 64, ctx->flags_dev);

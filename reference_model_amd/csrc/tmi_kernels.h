@@ -167,11 +167,12 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
                                   const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
                                   void* out, const void* pad_page, uint32_t* flag_word);
 
-// depthwise_stream.hip: the same layers with both operands in registers (the pixel operand loaded straight from global
-// memory, no LDS, no barrier; a wave keeps one channel block and walks pixel tiles); nullptr for anything else.
+// depthwise_stream.hip: the same layers with the pixel operand loaded straight from global memory into the matrix
+// instruction's registers (no patch in LDS; a wave keeps a group of channel blocks and walks pixel tiles with the next
+// tile's loads in flight); nullptr for anything else.
 const char* launch_depthwise_stream(hipStream_t st, int32_t in_dtype, int32_t out_dtype, const ConvGeom& g, const void* in,
                                     const void* w, const void* bias, int32_t in_zp, int32_t w_zp, const RescaleParams& rp,
-                                    void* out, const void* pad_page, uint32_t* flag_word);
+                                    void* out, uint32_t* flag_word);
 
 // gemm_mfma.hip: whether a CONV2D left to automatic choice tries the GEMM kernel before the patch kernel.
 bool gemm_mfma_preferred(int32_t in_dtype, const ConvGeom& g);

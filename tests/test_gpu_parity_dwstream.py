@@ -175,3 +175,17 @@ def test_depthwise_stream_epilogue_form_borders(ctx, name, shifts, mode, out_dty
     assert st == wst and np.array_equal(got, want), (st, wst, int(np.count_nonzero(got != want)))
     if small and out_dtype == np.int16:
         assert len(np.unique(got)) > 50
+
+
+def test_automatic_choice_takes_this_kernel_for_large_layers_with_few_channels():
+    c = Context(0)
+    try:
+        for shape, kernel in [((4, 112, 112, 32, (1, 1, 1, 1), (1, 1), (1, 1)), "depthwise_stream_i8"),
+                              ((9, 56, 56, 48, (0, 1, 0, 1), (1, 1), (1, 1)), "depthwise_mfma_i8"),     # 1.3 M results
+                              ((2, 112, 112, 64, (1, 1, 1, 1), (1, 1), (1, 1)), "depthwise_mfma_i8")]:  # 64 channels
+            x, w, bias = _operands(shape, 21)
+            got, st = gpu_ops.conv2d(c, x, w, bias, shape[4], shape[5], in_zp=-9, depthwise=True)
+            assert st == capi.VALID and c.last_kernel == kernel
+            assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, shape[4], shape[5], in_zp=-9, w_zp=0))
+    finally:
+        c.close()
