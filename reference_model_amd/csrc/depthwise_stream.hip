@@ -84,6 +84,7 @@ __global__ __launch_bounds__(512) void depthwise_stream_kernel(DwStreamArgs a)
     // loads the tensor's first bytes instead and is replaced by input_zp before use; the return value has bit t set when
     // tap t is a real one.
     const bool lane_has_channels = G > 1 || g_ok[0];    // (with G > 1 the launcher takes whole groups only)
+    const bool all_channels      = G > 1 || c0 + 32 <= C;
     auto request = [&](int p, v4i(&fb)[TAPS][G]) -> uint32_t {
         const uint32_t trow = fdiv((uint32_t)p, a.div_tiles_x);
         const int txi       = p - trow * a.tiles_x;
@@ -91,9 +92,26 @@ __global__ __launch_bounds__(512) void depthwise_stream_kernel(DwStreamArgs a)
         const int tyi       = trow - n * a.tiles_y;
         const int oy = tyi * th + ty, ox = txi * tw + tx;
         const int iy0 = oy * a.sy - a.pad_top, ix0 = ox * a.sx - a.pad_left;
-        const bool px_ok = lane_has_channels && oy < a.OH && ox < a.OW;
         // the tensor has fewer than 2^31 bytes (checked by the launcher)
         const uint32_t base = (uint32_t)(((n * a.IH + iy0) * a.IW + ix0) * C + cl);
+        // a tile whose pixels all exist and whose windows all lie inside the image (a test on scalars): nine additions
+        const int ty0 = tyi * th, tx0 = txi * tw;
+        const bool inside = all_channels && ty0 + th <= a.OH && tx0 + tw <= a.OW && ty0 * a.sy >= a.pad_top &&
+                            tx0 * a.sx >= a.pad_left && (ty0 + th - 1) * a.sy - a.pad_top + 2 * a.dy < a.IH &&
+                            (tx0 + tw - 1) * a.sx - a.pad_left + 2 * a.dx < a.IW;
+        if (inside)
+        {
+#pragma unroll
+            for (int t = 0; t < TAPS; t++)
+            {
+                const uint32_t voff = base + (uint32_t)((t / 3) * row_step + (t % 3) * col_step);
+#pragma unroll
+                for (int g = 0; g < G; g++)
+                    fb[t][g] = *reinterpret_cast<const v4i*>(a.in + voff + 32 * g);
+            }
+            return 0x1ffu;
+        }
+        const bool px_ok = lane_has_channels && oy < a.OH && ox < a.OW;
         bool rok[3], cok[3];
 #pragma unroll
         for (int k = 0; k < 3; k++)
@@ -402,8 +420,8 @@ const char* launch_depthwise_stream(hipStream_t st, int32_t in_dtype, int32_t ou
     a.n_tiles       = (int32_t)n_tiles;
     a.tiles_per_part = (int32_t)((n_tiles + 7) / 8);
     // eight waves per workgroup; a CU holds one workgroup (two waves per SIMD: a wave of the fused kernel holds 190 to 254
-    // registers), with single blocks two (126 registers), and a part of the layer has 32 CUs
-    constexpr int NW = 8;
+    // registers), with single blocks two (at most 128 registers), and a part of the layer has 32 CUs
+    constexpr int NW      = 8;
     const int64_t wgs_max = G == 1 ? 64 : 32;
     int64_t wgs = ((int64_t)a.tiles_per_part * n_grp + NW - 1) / NW;
     wgs         = wgs < wgs_max ? wgs : wgs_max;
