@@ -44,7 +44,7 @@ PROFILE_OF = {"c3": "conv2d_slab_wreg_i8_rescale_c3_resnet3x3", "c2": "matmul_ge
               "c5b": "matmul_gemm_bf16_c5b_4x2048x4096", "maxpool": "max_pool2d_i8_32x112x112x64",
               "avgpool": "avg_pool2d_i8_32x112x112x64", "tconv": "transpose_conv2d_slab_i8_8x28x28x128",
               "conv3d": "conv3d_slab_i8_2x16x28x28x32", "rescale": "rescale_fast_i32_to_i8_64x56x56x64",
-              "c4x8": "depthwise_mfma_i8_rescale_64x112x112x96", "c3x4": "conv2d_slab_wreg_i8_rescale_32x56x56x64"}
+              "c4x8": "depthwise_mfma_i8_rescale_64x112x112x96", "dw32": "depthwise_stream_i8_rescale_64x112x112x32", "c3x4": "conv2d_slab_wreg_i8_rescale_32x56x56x64"}
 
 
 def measured_traffic(cfg, kernel):
@@ -80,7 +80,7 @@ def main() -> int:
                     help="times the region of --steps steps is run; the median repeat is reported "
                          "(default: enough repeats for 10000 steps, between 5 and 500)")
     ap.add_argument("--copy-mib", type=int, default=1024, help="buffer size of --config copy")
-    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy", "launch_floor", "networks"])
+    ap.add_argument("--config", default="c3", choices=["c1", "c2", "c3", "c3x4", "c4", "c5a", "c5b", "rescale", "c4x8", "dw32", "tconv", "conv3d", "maxpool", "avgpool", "precise", "copy", "launch_floor", "networks"])
     ap.add_argument("--batch", type=int, default=8, help="images per layer of --config networks")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     ap.add_argument("--no-named-configs", action="store_true",
@@ -352,10 +352,10 @@ def main() -> int:
                      cpu_fraction=frac, result=lambda: out[:1].cpu().numpy(), dtype="int8",
                      metric="int8 %s TOPS; %% int8 MFMA peak; bit-exact" % cfg.upper(), unit="TOPS", bound="mfma",
                      peak=PEAK["int8_mfma"], runit="TOP/s", workload="INT8 " + name)
-        elif cfg in ("c1", "c3", "c3x4", "c4", "c4x8"):
+        elif cfg in ("c1", "c3", "c3x4", "c4", "c4x8", "dw32"):
             c = {"c1": cases.c1, "c3": cases.c3, "c3x4": lambda: cases.c3(n=32), "c4": cases.c4,
-                 "c4x8": lambda: cases.c4(n=64)}[cfg]()
-            depthwise = cfg in ("c4", "c4x8")
+                 "c4x8": lambda: cases.c4(n=64), "dw32": lambda: cases.c4(n=64, c=32, stride=1)}[cfg]()
+            depthwise = cfg in ("c4", "c4x8", "dw32")
             n, ih, iw, ic = c["x"].shape
             if depthwise:
                 kh, kw, _, m = c["w"].shape
@@ -403,6 +403,9 @@ def main() -> int:
                                   "RESCALE (shift 34..40, double_round), fused")
                 if cfg == "c4x8":    # the same layer at eight times the batch: the kernel's rate without the launch floor
                     W["workload"] = W["workload"].replace("[8,112,112,96]", "[64,112,112,96]") + " (8x the named batch)"
+                if cfg == "dw32":    # the network's first depthwise layer, 64 images: no named configuration
+                    W["workload"] = "INT8 DEPTHWISE_CONV2D [64,112,112,32] 3x3 s1 pad 1 + per-channel RESCALE (shift 34..40, " \
+                                    "double_round), fused (MobileNetV2's first depthwise layer; not a named configuration)"
         elif cfg in ("c2", "c5b"):
             c = cases.c2() if cfg == "c2" else cases.c5_matmul()
             n, h, k = c["a"].shape

@@ -45,9 +45,17 @@ def c3(n=8, hw=56, ic=64, oc=64):
         shift=np.full(oc, 38, np.int8), out_zp=0, clamp=(0, 127))
 
 
-def c4(n=8, hw=112, c=96):
-    """INT8 DEPTHWISE_CONV2D MobileNetV2-style [8,112,112,96], stride 2, pad [0,1,0,1], per-channel RESCALE."""
+def c4(n=8, hw=112, c=96, stride=2):
+    """INT8 DEPTHWISE_CONV2D MobileNetV2-style [8,112,112,96], stride 2, pad [0,1,0,1], per-channel RESCALE
+    (stride 1: pad 1 all round, the network's first depthwise layer when c is 32)."""
     r = rng_for(4)
+    d = _c4(r, n, hw, c)
+    if stride == 1:
+        d.update(pad=(1, 1, 1, 1), stride=(1, 1))
+    return d
+
+
+def _c4(r, n, hw, c):
     return dict(
         x=r.integers(-128, 128, (n, hw, hw, c)).astype(np.int8),
         w=r.integers(-127, 128, (3, 3, c, 1)).astype(np.int8),

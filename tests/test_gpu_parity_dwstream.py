@@ -189,3 +189,43 @@ def test_automatic_choice_takes_this_kernel_for_large_layers_with_few_channels()
             assert np.array_equal(got, oracle.depthwise_conv2d("i8", x, w, bias, shape[4], shape[5], in_zp=-9, w_zp=0))
     finally:
         c.close()
+
+
+def _geometry(rng):
+    """a legal (ih, iw, pad, stride, dilation) for 3x3 taps: (ih - 1 + pad - 2 * dilation) % stride == 0"""
+    while True:
+        stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        dil = (int(rng.integers(1, 4)), int(rng.integers(1, 3)))
+        pad = tuple(int(v) for v in rng.integers(0, 4, 4))
+        oh, ow = int(rng.integers(1, 70)), int(rng.integers(1, 70))
+        ih = (oh - 1) * stride[0] + 2 * dil[0] + 1 - pad[0] - pad[1]
+        iw = (ow - 1) * stride[1] + 2 * dil[1] + 1 - pad[2] - pad[3]
+        if ih >= 1 and iw >= 1:
+            return ih, iw, pad, stride, dil
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_depthwise_stream_random_geometry(ctx, seed):
+    """random strides, dilations, paddings (wider than the taps reach, too), image shapes from a single pixel to many tiles
+    per wave, and channel counts that give groups of one, two and three blocks and a ragged last block"""
+    rng = np.random.default_rng(7000 + seed)
+    ih, iw, pad, stride, dil = _geometry(rng)
+    n = int(rng.choice([1, 2, 3, 5, 33]))
+    c = int(rng.choice([32, 48, 64, 80, 96, 128, 144, 192, 288]))
+    in_zp = int(rng.integers(-128, 128))
+    x = rng.integers(-128, 128, (n, ih, iw, c)).astype(np.int8)
+    w = rng.integers(-128, 128, (3, 3, c, 1)).astype(np.int8)
+    bias = rng.integers(-(1 << 16), 1 << 16, c if seed % 5 else 1).astype(np.int32)
+    acc = oracle.depthwise_conv2d("i8", x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0)
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True)
+    assert st == capi.VALID and ctx.last_kernel == "depthwise_stream_i8"
+    assert np.array_equal(got, acc), (n, ih, iw, c, pad, stride, dil)
+    mult = rng.integers(1 << 30, 1 << 31, c).astype(np.int32)
+    shift = rng.integers(33, 40, c).astype(np.int8) if seed % 3 else np.full(c, 35, np.int8)
+    out_zp = int(rng.integers(-20, 20))
+    out_dtype = np.int16 if seed % 4 == 3 else np.int8
+    got, st = gpu_ops.conv2d(ctx, x, w, bias, pad, stride, dil, in_zp=in_zp, w_zp=0, depthwise=True,
+                             rescale=dict(mult=mult, shift=shift, out_zp=out_zp if out_dtype == np.int8 else 0, out_dtype=out_dtype))
+    want, wst = oracle.rescale(acc, mult, shift, out_zp=out_zp if out_dtype == np.int8 else 0, out_dtype=out_dtype)
+    assert st == wst == capi.VALID and ctx.last_kernel == "depthwise_stream_i8_rescale"
+    assert np.array_equal(got, want), (n, ih, iw, c, pad, stride, dil)
