@@ -247,6 +247,15 @@ __global__ __launch_bounds__(512) void depthwise_stream_kernel(DwStreamArgs a)
         }
         __builtin_amdgcn_sched_barrier(0);
         // ---- the next tile's loads ---------------------------------------------------------------------------------------
+        // They land in the registers the matrix instructions above read.  A matrix instruction runs for 16 passes after it
+        // has been issued and nothing orders a later load's data behind its operand reads (a load of a line that the L1 holds,
+        // issued right behind the matrix instruction of its tap, was seen to replace the operand's last bytes in time to
+        // change the product), so the requests wait for a value of the last matrix instruction's result.
+        {
+            const int done = __builtin_amdgcn_readfirstlane(acc[G - 1][15]);
+            asm volatile("" ::"s"(done));
+        }
+        __builtin_amdgcn_sched_barrier(0);
         const int pn        = pt + a.n_streams;
         const bool has_next = pn < pt_end;
         if (has_next)
