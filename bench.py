@@ -85,6 +85,9 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing and the parity check")
     ap.add_argument("--no-named-configs", action="store_true",
                     help="default configuration only: skip the short GPU legs of the other named configurations")
+    ap.add_argument("--kernel-choice", type=int, default=0,
+                    help="tmi_ctx_set_kernel_choice for the measured operator (0: the library's own choice; the profiles of "
+                         "one layer under two kernels use it)")
     ap.add_argument("--eager", action="store_true",
                     help="issue every step from the host instead of replaying HIP graphs of the steps")
     args = ap.parse_args()
@@ -106,6 +109,8 @@ def main() -> int:
     ctx = Context(0)
     stream = torch.cuda.current_stream()
     ctx.set_stream(stream.cuda_stream)
+    if args.kernel_choice:
+        ctx.set_kernel_choice(args.kernel_choice)
 
     def the_oracle():
         # the CPU oracle is the checker and the CPU baseline: nothing before the timed region touches it
