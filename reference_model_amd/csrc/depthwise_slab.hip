@@ -83,7 +83,7 @@ __global__ __launch_bounds__(1024) void depthwise_slab_kernel(DwSlabArgs a)
     HighWordScale* tab_hw = reinterpret_cast<HighWordScale*>(tab_cs + C);
     int32_t* tab_m       = reinterpret_cast<int32_t*>(tab_hw + C);
     int32_t* tab_b       = tab_m + C;
-    int32_t* uni_shift   = tab_b + C;    // 8 words
+    int32_t* uni_shift   = tab_b + C;    // a word per table wave: 16
 
     uint32_t bid = blockIdx.x;
     if (a.xcd_remap)
@@ -418,7 +418,7 @@ const char* launch_depthwise_slab(hipStream_t st, int32_t in_dtype, int32_t out_
     const int32_t key[8] = { g.N, g.OH, g.OW, C, g.stride_y, g.stride_x, g.dil_y, g.dil_x };
     int best_th = 0, best_tw = 0, best_nw = 0;
     // weights, both forms of the requantisation constants, multipliers, bias terms, the table waves' shifts
-    const int table_bytes = 9 * C * 4 + C * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + C * 8 + 32;
+    const int table_bytes = 9 * C * 4 + C * (int)(sizeof(ChannelScale) + sizeof(HighWordScale)) + C * 8 + 64;
     constexpr int lds_max = 160 * 1024;
     if (memcmp(key, last.key, sizeof(key)) == 0)
         best_th = last.th, best_tw = last.tw, best_nw = last.nw;
