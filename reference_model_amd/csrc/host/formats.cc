@@ -11,6 +11,10 @@
 //   MaxPool2dAttribute        0 kernel, 1 stride, 2 pad, 3 nan_mode
 //   RescaleAttribute  0 scale32, 1 rounding_mode, 2 per_channel, 3 input_unsigned, 4 output_unsigned
 //   ClampAttribute    0 min_val[ubyte], 1 max_val[ubyte], 2 nan_mode
+// The numbers of the Conv2d, Rescale and tensor / operator tables are confirmed by the reference's example graphs.  Those of
+// the TransposeConv2d, pooling and Clamp attributes have no stored graph to confirm them; they follow the argument order in
+// which the reference's test generator hands the fields to the serializer (verif/generator/tosa_test_gen.py:910, 974,
+// 1239, 1522), the correspondence that the confirmed Conv2dAttribute (:1065) and RescaleAttribute (:2290) show.
 #include <cstdio>
 #include <cstring>
 #include <fstream>
