@@ -29,6 +29,7 @@ size_t dtype_size(DType t)
 {
     switch (t)
     {
+        case DType_INT4:    // one value per byte in memory and in .npy files; two per byte in a .tosa payload
         case DType_INT8:
             return 1;
         case DType_INT16:
@@ -314,6 +315,7 @@ const char* npy_descr_for(DType t)
 {
     switch (t)
     {
+        case DType_INT4:
         case DType_INT8:
             return "|i1";
         case DType_INT16:

@@ -25,6 +25,7 @@ bool Tensor::scalar_value(int32_t& v) const
         return false;
     switch (dtype)
     {
+        case DType_INT4:
         case DType_INT8:
             v = (int8_t)host[0];
             return true;
@@ -222,7 +223,9 @@ public:
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 4, 4))
             return 1;
         // the weights have the input's type, except that INT16 inputs come with INT8 weights (tensor_ops.cpp:2225, 2247)
-        if (inputs[1]->getDtype() != (inputs[0]->getDtype() == DType_INT16 ? DType_INT8 : inputs[0]->getDtype()))
+        // and INT8 inputs may come with INT4 weights (:2224, :2246: the same arithmetic on values of -8 ... 7)
+        if (inputs[1]->getDtype() != (inputs[0]->getDtype() == DType_INT16 ? DType_INT8 : inputs[0]->getDtype()) &&
+            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))
             return error("weight data type not supported for this configuration of operator");
         tmi_conv_desc_t d;
         if (fill_desc(d))
@@ -433,6 +436,8 @@ int ConvBase::eval()
     int32_t in_zp = 0, w_zp = 0;
     if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
         return error("zero-point operands must be available on the host");
+    if (inputs[1]->getDtype() == DType_INT4 && w_zp != 0)    // tensor_ops.cpp:811, :1241
+        return error("Weight zero point must be zero for non int8_t data");
     SubgraphTraverser* s = parent_sgt;
     if (s->precise_mode && inputs[0]->getDtype() != DType_INT8 && inputs[0]->getDtype() != DType_INT16)
     {
@@ -526,7 +531,8 @@ public:
             validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 4, 4))
             return 1;
-        if (inputs[1]->getDtype() != inputs[0]->getDtype())
+        if (inputs[1]->getDtype() != inputs[0]->getDtype() &&
+            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (tensor_ops.cpp:2235, 2258)
             return error("weight data type not supported for this configuration of operator");
         tmi_tconv_desc_t d;
         if (fill_desc(d))
@@ -547,6 +553,8 @@ public:
         int32_t in_zp = 0, w_zp = 0;
         if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
             return error("zero-point operands must be available on the host");
+        if (inputs[1]->getDtype() == DType_INT4 && w_zp != 0)    // tensor_ops.cpp:1037, :2119
+            return error("Weight zero point must be zero for non int8_t data");
         SubgraphTraverser* s = parent_sgt;
         if (call(tmi_transpose_conv2d(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]),
                                       in_zp, w_zp, s->device_out(outputs[0]))))
@@ -675,7 +683,8 @@ public:
             validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 5, 5))
             return 1;
-        if (inputs[1]->getDtype() != inputs[0]->getDtype())
+        if (inputs[1]->getDtype() != inputs[0]->getDtype() &&
+            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (tensor_ops.cpp:2235, 2258)
             return error("weight data type not supported for this configuration of operator");
         tmi_conv3d_desc_t d;
         if (fill_desc(d))
@@ -696,6 +705,8 @@ public:
         int32_t in_zp = 0, w_zp = 0;
         if (!inputs[3]->scalar_value(in_zp) || !inputs[4]->scalar_value(w_zp))
             return error("zero-point operands must be available on the host");
+        if (inputs[1]->getDtype() == DType_INT4 && w_zp != 0)    // tensor_ops.cpp:1037, :2119
+            return error("Weight zero point must be zero for non int8_t data");
         SubgraphTraverser* s = parent_sgt;
         if (call(tmi_conv3d(s->ctx, &d, s->device(inputs[0]), s->device(inputs[1]), s->device(inputs[2]), in_zp, w_zp,
                             s->device_out(outputs[0]))))
@@ -832,8 +843,12 @@ int SubgraphTraverser::initializeGraph()
         {
             // an INT48 element takes 6 bytes in the serialized payload and one int64 in memory
             // (reference: subgraph_traverser.cpp:652-656, ConvertU8toI48)
+            // an INT4 element takes half a byte in the payload, the first of a pair in the low half, and one int8 in memory
+            // (reference: subgraph_traverser.cpp:625-630, ConvertU8toI4 of the serialization library, whose source the
+            // reference does not hold: the pair order is that library's published one, with no stored graph to confirm it)
             const bool i48      = d.dtype == DType_INT48;
-            const size_t stored = i48 ? (size_t)t->getElementCount() * 6 : t->bytes();
+            const bool i4       = d.dtype == DType_INT4;
+            const size_t stored = i48 ? (size_t)t->getElementCount() * 6 : (i4 ? ((size_t)t->getElementCount() + 1) / 2 : t->bytes());
             if (d.data.size() < stored)
             {
                 last_message = "tensor " + d.name + ": constant payload shorter than the tensor";
@@ -851,6 +866,15 @@ int SubgraphTraverser::initializeGraph()
                     if (v & 0x800000000000ull)
                         v |= 0xFFFF000000000000ull;
                     memcpy(t->host.data() + e * 8, &v, 8);
+                }
+            }
+            else if (i4)
+            {
+                t->host.resize(t->bytes());
+                for (size_t e = 0; e < (size_t)t->getElementCount(); e++)
+                {
+                    const uint8_t nib = (uint8_t)((d.data[e / 2] >> (4 * (e & 1))) & 0xf);
+                    t->host[e]        = (uint8_t)(int8_t)((nib & 8) ? (int)nib - 16 : (int)nib);
                 }
             }
             else

@@ -376,6 +376,66 @@ def test_int16_convolution_and_matmul_graphs(tmp_path):
 
 
 @pytest.mark.gpu
+def test_int4_weight_graphs(tmp_path):
+    """INT8 x INT4 -> INT32 (tensor_ops.cpp:2224, 2246): the weights are constants of two values to a byte
+    (subgraph_traverser.cpp:625-630) and the arithmetic is that of int8 weights; an odd element count leaves half a byte
+    unused; a weight zero point other than 0 is an error (tensor_ops.cpp:811)"""
+    rng = np.random.default_rng(44)
+    x = rng.integers(-128, 128, (2, 7, 9, 5)).astype(np.int8)
+    w = rng.integers(-8, 8, (3, 3, 3, 5)).astype(np.int8)         # 135 values: 67 and a half bytes
+    wd = rng.integers(-8, 8, (3, 3, 5, 2)).astype(np.int8)
+    bias = rng.integers(-1000, 1000, 3).astype(np.int32)
+    biasd = rng.integers(-1000, 1000, 10).astype(np.int32)
+    assert w.min() == -8 and w.max() == 7
+    acc = oracle.conv2d("i8", x, w, bias, (1, 1, 1, 1), in_zp=-5)
+    accd = oracle.depthwise_conv2d("i8", x, wd, biasd, (1, 1, 1, 1), in_zp=-5)
+    ts = [W.tensor("x", x.shape, np.int8), W.tensor("w", w.shape, np.int8, w, int4=True),
+          W.tensor("wd", wd.shape, np.int8, wd, int4=True), W.tensor("bias", [3], np.int32, bias),
+          W.tensor("biasd", [10], np.int32, biasd), W.tensor("izp", [1], np.int8, [-5]),
+          W.tensor("wzp", [1], np.int8, [0], int4=True), W.tensor("wzp3", [1], np.int8, [3], int4=True),
+          W.tensor("acc", [2, 7, 9, 3], np.int32), W.tensor("accd", [2, 7, 9, 10], np.int32)]
+    consts = [W.operator(R.OP_CONST, [], [n]) for n in ("w", "wd", "bias", "biasd", "izp", "wzp", "wzp3")]
+    ops = consts + [W.operator(R.OP_CONV2D, ["x", "w", "bias", "izp", "wzp"], ["acc"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1))),
+                    W.operator(R.OP_DEPTHWISE_CONV2D, ["x", "wd", "biasd", "izp", "wzp"], ["accd"],
+                               W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1)))]
+    r = _run(_write_case(tmp_path, W.graph(ts, ops, ["x"], ["acc", "accd"]), {"x": x}, ["acc", "accd"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(tmp_path / "acc_out.npy"), acc)
+    assert np.array_equal(np.load(tmp_path / "accd_out.npy"), accd)
+    ops = consts + [W.operator(R.OP_CONV2D, ["x", "w", "bias", "izp", "wzp3"], ["acc"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1)))]
+    d2 = tmp_path / "zp"
+    d2.mkdir()
+    r = _run(_write_case(d2, W.graph(ts, ops, ["x"], ["acc"]), {"x": x}, ["acc"]))
+    assert r.returncode == 2 and "Weight zero point must be zero for non int8_t data" in r.stderr
+    # TRANSPOSE_CONV2D and CONV3D with INT4 weights (tensor_ops.cpp:2235, 2258)
+    wt = rng.integers(-8, 8, (4, 3, 3, 5)).astype(np.int8)
+    bt = rng.integers(-500, 500, 4).astype(np.int32)
+    acct = oracle.transpose_conv2d("i8", x, wt, bt, (0, 1, -1, 0), (2, 2), in_zp=-5, w_zp=0)
+    x3 = rng.integers(-128, 128, (1, 4, 5, 5, 8)).astype(np.int8)
+    w3 = rng.integers(-8, 8, (4, 2, 3, 3, 8)).astype(np.int8)
+    pad3, one3 = (1, 0, 1, 1, 1, 1), (1, 1, 1)
+    acc3 = oracle.conv3d("i8", x3, w3, bt, pad3, one3, one3, in_zp=-5, w_zp=0)
+    ts3 = [W.tensor("x", x.shape, np.int8), W.tensor("x3", x3.shape, np.int8), W.tensor("wt", wt.shape, np.int8, wt, int4=True),
+           W.tensor("w3", w3.shape, np.int8, w3, int4=True), W.tensor("bt", [4], np.int32, bt), W.tensor("izp", [1], np.int8, [-5]),
+           W.tensor("wzp", [1], np.int8, [0], int4=True), W.tensor("ot", acct.shape, np.int32), W.tensor("o3", acc3.shape, np.int32)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("wt", "w3", "bt", "izp", "wzp")]
+    ops.append(W.operator(10, ["x", "wt", "bt", "izp", "wzp"], ["ot"], W.transpose_conv_attr((0, 1, -1, 0), (2, 2))))
+    ops.append(W.operator(4, ["x3", "w3", "bt", "izp", "wzp"], ["o3"], W.conv_attr(pad3, one3, one3)))
+    d4 = tmp_path / "t3"
+    d4.mkdir()
+    r = _run(_write_case(d4, W.graph(ts3, ops, ["x", "x3"], ["ot", "o3"]), {"x": x, "x3": x3}, ["ot", "o3"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d4 / "ot_out.npy"), acct) and np.array_equal(np.load(d4 / "o3_out.npy"), acc3)
+    # INT4 is a weight type only: as a convolution's input it is refused
+    ts2 = [W.tensor("x", x.shape, np.int8, int4=True)] + ts[1:]
+    ops = consts + [W.operator(R.OP_CONV2D, ["x", "w", "bias", "izp", "wzp"], ["acc"], W.conv_attr((1, 1, 1, 1), (1, 1), (1, 1)))]
+    d3 = tmp_path / "in4"
+    d3.mkdir()
+    r = _run(_write_case(d3, W.graph(ts2, ops, ["x"], ["acc"]), {"x": x}, ["acc"]))
+    assert r.returncode == 2
+
+
+@pytest.mark.gpu
 def test_inexact_round_rescale_in_precise_and_compliance_mode(tmp_path):
     """--precise_mode=1 reaches an INEXACT_ROUND RESCALE (type_conversion.cpp:326-346): FP64 maths truncated; on a
     compliance descriptor the normal pass writes the lower edge of the error bound and the bounds pass the upper one"""

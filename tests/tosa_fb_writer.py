@@ -111,12 +111,18 @@ class Writer:
         return bytes(self.buf)
 
 
-def tensor(name, shape, dtype, data=None):
-    f = [(0, None, string(name)), (1, None, vector("i", shape)), (2, "I", DTYPE_CODE[np.dtype(dtype)])]
+def tensor(name, shape, dtype, data=None, int4=False):
+    """int4: an INT4 tensor (DType 2) from int8 values of -8 ... 7, two to a byte, the first of a pair in the low half"""
+    f = [(0, None, string(name)), (1, None, vector("i", shape)), (2, "I", 2 if int4 else DTYPE_CODE[np.dtype(dtype)])]
     if data is not None:
         arr = np.ascontiguousarray(data, dtype=dtype)
-        # INT48 (int64 here) is serialized as the low 6 bytes of every element
-        raw = arr.view(np.uint8).reshape(-1, 8)[:, :6].tobytes() if arr.dtype == np.int64 else arr.tobytes()
+        if int4:
+            nib = (arr.reshape(-1).astype(np.int16) & 0xF).astype(np.uint8)
+            nib = np.concatenate([nib, np.zeros(len(nib) & 1, np.uint8)])
+            raw = (nib[0::2] | (nib[1::2] << 4)).astype(np.uint8).tobytes()
+        else:
+            # INT48 (int64 here) is serialized as the low 6 bytes of every element
+            raw = arr.view(np.uint8).reshape(-1, 8)[:, :6].tobytes() if arr.dtype == np.int64 else arr.tobytes()
         raw += b"\0" * (-len(raw) % 8)
         f.append((3, None, vector("B", raw)))
     return table(f)
