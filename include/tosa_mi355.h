@@ -247,8 +247,10 @@ typedef struct
  * of the input type (the instantiations at :2220-2229; FP32 runs on the one-element-per-lane kernels, in the
  * reference's summation order).  INT16 x INT8 -> INT48 (:2225; d->in_dtype TMI_INT16, weights INT8, bias and
  * output one int64 per element, the sum kept in 64 bits and REQUIREd to lie within 48 bits, :875-879) runs on a
- * one-element-per-lane kernel.  in_zp / w_zp are the values of operands 3 and 4: in_zp must be 0 unless the
- * input is INT8, w_zp unless the weights are (:804-811). */
+ * one-element-per-lane kernel.  INT8 x INT4 -> INT32 (:2224) is the INT8 call with the weights handed over as one
+ * int8 value of -8 ... 7 per element and w_zp = 0, which the caller checks (the library cannot tell such weights from INT8
+ * ones).  in_zp / w_zp are the values of operands 3 and 4: in_zp must be 0 unless the input is INT8, w_zp unless the
+ * weights are (:804-811). */
 int tmi_conv2d(tmi_ctx_t* ctx, const tmi_conv_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
