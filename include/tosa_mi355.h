@@ -303,7 +303,8 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
 /* OpTransposeConv2d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:2058-2197 (checks :1982-2056).
  * Evaluated as a stride-1 CONV2D with flipped taps over the input with stride-1 holes filled with input_zp.
  * INT8 with 3x3 taps, 64 / 96 / 128 input channels and w_zp 0 reads both operands in place (holes and flip are
- * part of the kernel's addressing); otherwise the re-laid-out operands live in the context's scratch buffer. */
+ * part of the kernel's addressing); otherwise the re-laid-out operands live in the context's scratch buffer.
+ * Element types as tmi_conv2d: INT8 -> INT32, FP16 / BF16, and INT16 x INT8 -> INT48 (:2291; clip :2190-2194). */
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
@@ -325,7 +326,8 @@ int tmi_transpose_conv2d_noalloc(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, cons
 /* OpConv3d<In,W,Acc,Out>::eval, reference_model/src/ops/tensor_ops.cpp:935-1120 (checks :901-933, :120-226).
  * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side.  INT8 with 3x3 taps in
  * the plane, KD*IC = 64 / 96 / 128 (IC 32 or 64) and w_zp 0 reads both operands in place; otherwise the gathered
- * input and the permuted weights live in the context's scratch buffer. */
+ * input and the permuted weights live in the context's scratch buffer.  Element types as tmi_conv2d: INT8 -> INT32,
+ * FP16 / BF16, and INT16 x INT8 -> INT48 (:2237; clip :1113-1117). */
 int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 

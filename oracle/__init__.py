@@ -208,7 +208,7 @@ def conv3d_out_dhw(idhw, kdhw, pad, stride, dilation):
 
 def _dispatch(prefix, kind, s, inp, w, bias, in_zp, w_zp, abs_mode, out):
     L = lib()
-    if kind in ("i8", "i32"):
+    if kind in ("i8", "i32", "i16"):
         rc = getattr(L, f"{prefix}_{kind}")(ctypes.byref(s), _ptr(inp), _ptr(w), _ptr(bias), ctypes.c_int32(in_zp),
                                             ctypes.c_int32(w_zp), _ptr(out))
     elif kind == "f32":
@@ -222,9 +222,9 @@ def _dispatch(prefix, kind, s, inp, w, bias, in_zp, w_zp, abs_mode, out):
 
 def conv3d(kind, inp, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), in_zp=0, w_zp=0,
            abs_mode=False, out_dhw=None):
-    """CONV3D.  inp [N,D,H,W,C], w [OC,KD,KH,KW,C], bias [1] or [OC]."""
+    """CONV3D.  inp [N,D,H,W,C], w [OC,KD,KH,KW,C], bias [1] or [OC].  kind i16: INT8 weights, INT48 results."""
     et, bt, ot = _KINDS[kind]
-    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    inp, w, bias = _c(inp, et), _c(w, np.int8 if kind == "i16" else et), _c(bias, bt)
     if w.shape[4] != inp.shape[4]:
         raise OracleStatus(ERROR)
     if out_dhw is None:
@@ -241,9 +241,9 @@ def conv3d(kind, inp, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1
 
 def transpose_conv2d(kind, inp, w, bias, out_pad=(0, 0, 0, 0), stride=(1, 1), in_zp=0, w_zp=0, abs_mode=False,
                      out_hw=None):
-    """TRANSPOSE_CONV2D.  inp NHWC, w OHWI, bias [1] or [OC]."""
+    """TRANSPOSE_CONV2D.  inp NHWC, w OHWI, bias [1] or [OC].  kind i16: INT8 weights, INT48 results."""
     et, bt, ot = _KINDS[kind]
-    inp, w, bias = _c(inp, et), _c(w, et), _c(bias, bt)
+    inp, w, bias = _c(inp, et), _c(w, np.int8 if kind == "i16" else et), _c(bias, bt)
     if w.shape[3] != inp.shape[3]:
         raise OracleStatus(ERROR)
     n, ih, iw, ic = inp.shape

@@ -318,6 +318,24 @@ int orc_conv3d_i8(const orc_conv3d_shape_t* s, const int8_t* in, const int8_t* w
     return rc;
 }
 
+/* INT16 x INT8 -> INT48 (tensor_ops.cpp:2237): as orc_conv2d_i16; zero-point rule :1031, 48-bit clip :1113-1117 */
+ORC_DEFINE_CONV3D(conv3d_i64_impl, int64_t, ORC_ABS_I32)
+
+int orc_conv3d_i16(const orc_conv3d_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias, int32_t in_zp,
+                   int32_t w_zp, int64_t* out)
+{
+    if (orc_conv3d_check(s) != ORC_VALID || in_zp != 0)
+        return ORC_ERROR;
+    int64_t* in64 = widen_i16_to_i64(in, (size_t)s->N * s->ID * s->IH * s->IW * s->IC);
+    int64_t* w64  = widen_i8_to_i64(w, (size_t)s->OC * s->KD * s->KH * s->KW * s->IC);
+    int rc        = (in64 && w64) ? conv3d_i64_impl(s, in64, w64, bias, 0, (int64_t)w_zp, 0, out) : ORC_ERROR;
+    if (rc == ORC_VALID)
+        clip_int48(out, (size_t)s->N * s->OD * s->OH * s->OW * s->OC);
+    free(in64);
+    free(w64);
+    return rc;
+}
+
 /* ------------------------------------------------------------------------------------------------
  * OpTransposeConv2d (tensor_ops.cpp:1982-2197): out_pad > -kernel (:2037-2041), output size
  * (IH-1)*stride + out_pad + kernel (:2043-2053); eval: for every output element and tap (ky,kx) the
@@ -402,6 +420,24 @@ int orc_transpose_conv2d_f64(const orc_tconv_shape_t* s, const double* in, const
                              int abs_mode, double* out)
 {
     return tconv_f64_impl(s, in, w, bias, 0.0, 0.0, abs_mode, out);
+}
+
+/* INT16 x INT8 -> INT48 (tensor_ops.cpp:2291): as orc_conv2d_i16; zero-point rule :2115, 48-bit clip :2190-2194 */
+ORC_DEFINE_TCONV(tconv_i64_impl, int64_t, ORC_ABS_I32)
+
+int orc_transpose_conv2d_i16(const orc_tconv_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias,
+                             int32_t in_zp, int32_t w_zp, int64_t* out)
+{
+    if (orc_tconv_check(s) != ORC_VALID || in_zp != 0)
+        return ORC_ERROR;
+    int64_t* in64 = widen_i16_to_i64(in, (size_t)s->N * s->IH * s->IW * s->IC);
+    int64_t* w64  = widen_i8_to_i64(w, (size_t)s->OC * s->KH * s->KW * s->IC);
+    int rc        = (in64 && w64) ? tconv_i64_impl(s, in64, w64, bias, 0, (int64_t)w_zp, 0, out) : ORC_ERROR;
+    if (rc == ORC_VALID)
+        clip_int48(out, (size_t)s->N * s->OH * s->OW * s->OC);
+    free(in64);
+    free(w64);
+    return rc;
 }
 
 int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias,

@@ -115,6 +115,8 @@ int orc_conv3d_i32(const orc_conv3d_shape_t* s, const int32_t* in, const int32_t
                    int32_t in_zp, int32_t w_zp, int32_t* out);
 int orc_conv3d_i8(const orc_conv3d_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias, int32_t in_zp,
                   int32_t w_zp, int32_t* out);
+int orc_conv3d_i16(const orc_conv3d_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias, int32_t in_zp,
+                   int32_t w_zp, int64_t* out);
 int orc_conv3d_f32(const orc_conv3d_shape_t* s, const float* in, const float* w, const float* bias, float* out);
 int orc_conv3d_f64(const orc_conv3d_shape_t* s, const double* in, const double* w, const double* bias, int abs_mode,
                    double* out);
@@ -135,6 +137,8 @@ int orc_transpose_conv2d_i32(const orc_tconv_shape_t* s, const int32_t* in, cons
                              int32_t in_zp, int32_t w_zp, int32_t* out);
 int orc_transpose_conv2d_i8(const orc_tconv_shape_t* s, const int8_t* in, const int8_t* w, const int32_t* bias,
                             int32_t in_zp, int32_t w_zp, int32_t* out);
+int orc_transpose_conv2d_i16(const orc_tconv_shape_t* s, const int16_t* in, const int8_t* w, const int64_t* bias,
+                             int32_t in_zp, int32_t w_zp, int64_t* out);
 int orc_transpose_conv2d_f32(const orc_tconv_shape_t* s, const float* in, const float* w, const float* bias,
                              float* out);
 int orc_transpose_conv2d_f64(const orc_tconv_shape_t* s, const double* in, const double* w, const double* bias,

@@ -64,7 +64,7 @@ class TconvDesc(ctypes.Structure):
         # the accumulator type follows the operand type unless it is set explicitly afterwards
         super().__setattr__(name, value)
         if name == "in_dtype":
-            super().__setattr__("acc_dtype", INT32 if value == INT8 else FP32)
+            super().__setattr__("acc_dtype", INT32 if value == INT8 else (INT48 if value == INT16 else FP32))
 
 
 class Conv3dDesc(ctypes.Structure):
@@ -76,7 +76,7 @@ class Conv3dDesc(ctypes.Structure):
     def __setattr__(self, name, value):
         super().__setattr__(name, value)
         if name == "in_dtype":
-            super().__setattr__("acc_dtype", INT32 if value == INT8 else FP32)
+            super().__setattr__("acc_dtype", INT32 if value == INT8 else (INT48 if value == INT16 else FP32))
 
 
 class PoolDesc(ctypes.Structure):

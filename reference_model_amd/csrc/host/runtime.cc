@@ -531,8 +531,8 @@ public:
             validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 4, 4))
             return 1;
-        if (inputs[1]->getDtype() != inputs[0]->getDtype() &&
-            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (tensor_ops.cpp:2235, 2258)
+        if (inputs[1]->getDtype() != (inputs[0]->getDtype() == DType_INT16 ? DType_INT8 : inputs[0]->getDtype()) &&    // INT16 x INT8 (:2237, :2291)
+            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (:2235, :2289)
             return error("weight data type not supported for this configuration of operator");
         tmi_tconv_desc_t d;
         if (fill_desc(d))
@@ -683,8 +683,8 @@ public:
             validateRequiredRank(inputs[2], 1, 1) || validateRequiredRank(inputs[3], 1, 1) ||
             validateRequiredRank(inputs[4], 1, 1) || validateRequiredRank(outputs[0], 5, 5))
             return 1;
-        if (inputs[1]->getDtype() != inputs[0]->getDtype() &&
-            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (tensor_ops.cpp:2235, 2258)
+        if (inputs[1]->getDtype() != (inputs[0]->getDtype() == DType_INT16 ? DType_INT8 : inputs[0]->getDtype()) &&    // INT16 x INT8 (:2237, :2291)
+            !(inputs[0]->getDtype() == DType_INT8 && inputs[1]->getDtype() == DType_INT4))    // INT8 x INT4 (:2235, :2289)
             return error("weight data type not supported for this configuration of operator");
         tmi_conv3d_desc_t d;
         if (fill_desc(d))

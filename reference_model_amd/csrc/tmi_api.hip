@@ -925,11 +925,13 @@ static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* 
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48 (tensor_ops.cpp:2269), FP16 / BF16 with fp32 accumulation
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
-    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
+    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : d->in_dtype)))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
-    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
+    if (d->acc_dtype != 0 &&
+        d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : TMI_FP32)))    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KH < 1 || d->KW < 1)
         return fail(ctx, "%s: negative tensor dimension", op);
@@ -947,8 +949,11 @@ static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* 
                     (long long)H, (long long)W);
     if (d->bias_len != d->OC && d->bias_len != 1)
         return fail(ctx, "%s: bias channels mismatch %d != %d", op, d->bias_len, d->OC);
-    if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
-        return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    // tensor_ops.cpp:2115-2119; INT16 inputs come with INT8 weights, which keep their zero point
+    if (d->in_dtype != TMI_INT8 && in_zp != 0)
+        return fail(ctx, "%s: Input zero point must be zero for non int8_t data", op);
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && w_zp != 0)
+        return fail(ctx, "%s: Weight zero point must be zero for non int8_t data", op);
     return TMI_VALID;
 }
 
@@ -994,6 +999,7 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
     // the equivalent CONV2D: flipped taps, stride 1, pads KH-1+out_pad, input with holes between its pixels
     const int eb         = dtype_bits(d->in_dtype) / 8;
     const int row_bytes  = d->IC * eb;
+    const int w_row_bytes = d->in_dtype == TMI_INT16 ? d->IC : row_bytes;    // INT16 inputs come with INT8 weights
     const bool holes     = d->stride[0] > 1 || d->stride[1] > 1;
     const int32_t UH     = (d->IH - 1) * d->stride[0] + 1, UW = (d->IW - 1) * d->stride[1] + 1;
     tmi_conv_desc_t c{};
@@ -1017,7 +1023,7 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
         if (name)
             return after_launch(ctx, name);
     }
-    const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * row_bytes);
+    const size_t w_bytes = align256((size_t)d->OC * d->KH * d->KW * w_row_bytes);
     const size_t u_bytes = holes ? align256((size_t)d->N * UH * UW * row_bytes) : 0;
     uint8_t* w_flip = nullptr;
     if (static_only)
@@ -1036,9 +1042,16 @@ static int run_transpose_conv2d(tmi_ctx* ctx, bool static_only, const tmi_tconv_
         w_flip = (uint8_t*)ctx->workspace;
     }
     uint8_t* u      = w_flip + w_bytes;
-    if (!(holes ? launch_tconv_operands(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip, d->N, d->IH, d->IW,
-                                        d->stride[0], d->stride[1], in_zp, in_dev, u)
-                : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
+    if (w_row_bytes != row_bytes)
+    {
+        // operands of different element sizes: one launch each (the input zero point of INT16 data is 0)
+        if (!launch_flip_taps(ctx->stream, w_row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip) ||
+            (holes && !launch_upsample(ctx->stream, row_bytes, d->N, d->IH, d->IW, d->stride[0], d->stride[1], 0, in_dev, u)))
+            return fail(ctx, "%s: operand re-layout launch failed", op);
+    }
+    else if (!(holes ? launch_tconv_operands(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip, d->N, d->IH, d->IW,
+                                             d->stride[0], d->stride[1], in_zp, in_dev, u)
+                     : launch_flip_taps(ctx->stream, row_bytes, d->OC, d->KH, d->KW, weight_dev, w_flip)))
         return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, holes ? (const void*)u : in_dev, w_flip, bias_dev, in_zp, w_zp, none,
                     d->out_dtype, out_dev, false, false);
@@ -1065,11 +1078,13 @@ static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48 (tensor_ops.cpp:2237), FP16 / BF16 with fp32 accumulation
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
-    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : d->in_dtype))
+    if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : d->in_dtype)))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
-    if (d->acc_dtype != 0 && d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : TMI_FP32))    // 0: the operand type's default
+    if (d->acc_dtype != 0 &&
+        d->acc_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : TMI_FP32)))    // 0: the operand type's default
         return fail(ctx, "%s: accumulator type %d not supported for this configuration of operator", op, d->acc_dtype);
     if (d->N < 0 || d->ID < 0 || d->IH < 0 || d->IW < 0 || d->IC < 0 || d->OC < 0 || d->KD < 1 || d->KH < 1 ||
         d->KW < 1)
@@ -1096,8 +1111,11 @@ static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t
                     (long long)(full_w / d->stride[2] + 1));
     if (d->bias_len != d->OC && d->bias_len != 1)
         return fail(ctx, "%s: bias channel mismatch %d != %d", op, d->bias_len, d->OC);
-    if (d->in_dtype != TMI_INT8 && (in_zp != 0 || w_zp != 0))
-        return fail(ctx, "%s: zero points must be zero for non int8_t data", op);
+    // tensor_ops.cpp:1031-1037; INT16 inputs come with INT8 weights, which keep their zero point
+    if (d->in_dtype != TMI_INT8 && in_zp != 0)
+        return fail(ctx, "%s: Input zero point must be zero for non int8_t data", op);
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && w_zp != 0)
+        return fail(ctx, "%s: Weight zero point must be zero for non int8_t data", op);
     return TMI_VALID;
 }
 
@@ -1167,15 +1185,24 @@ int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, c
         if (name)
             return after_launch(ctx, name);
     }
-    const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * row_bytes);
+    const int w_row_bytes = d->in_dtype == TMI_INT16 ? d->IC : row_bytes;    // INT16 inputs come with INT8 weights
+    const size_t w_bytes = align256((size_t)d->OC * d->KD * d->KH * d->KW * w_row_bytes);
     const size_t g_bytes = align256((size_t)d->N * d->OD * d->IH * d->IW * d->KD * row_bytes);
     rc                   = ensure_workspace(ctx, w_bytes + g_bytes);
     if (rc != TMI_VALID)
         return rc;
     uint8_t* w_perm = (uint8_t*)ctx->workspace;
     uint8_t* gath   = w_perm + w_bytes;
-    if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID, d->OD,
-                                d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
+    if (w_row_bytes != row_bytes)
+    {
+        // operands of different element sizes: one launch each (the input zero point of INT16 data is 0)
+        if (!launch_permute_w3d(ctx->stream, w_row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm) ||
+            !launch_gather_depth(ctx->stream, row_bytes, d->N, d->ID, d->OD, d->KD, d->IH * d->IW, d->stride[0], d->dilation[0],
+                                 d->pad[0], 0, in_dev, gath))
+            return fail(ctx, "%s: operand re-layout launch failed", op);
+    }
+    else if (!launch_conv3d_operands(ctx->stream, row_bytes, d->OC, d->KD, d->KH * d->KW, weight_dev, w_perm, d->N, d->ID,
+                                     d->OD, d->IH * d->IW, d->stride[0], d->dilation[0], d->pad[0], in_zp, in_dev, gath))
         return fail(ctx, "%s: operand re-layout launch failed", op);
     return run_conv(ctx, op, false, &c, gath, w_perm, bias_dev, in_zp, w_zp, none, d->out_dtype, out_dev, false,
                     false);

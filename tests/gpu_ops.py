@@ -120,14 +120,16 @@ def transpose_conv2d(ctx, x, w, bias, out_pad=(0, 0, 0, 0), stride=(1, 1), in_zp
     if out_hw is None:
         out_hw = ((ih - 1) * stride[0] + out_pad[0] + out_pad[1] + kh, (iw - 1) * stride[1] + out_pad[2] + out_pad[3] + kw)
     d = capi.TconvDesc()
-    d.in_dtype, d.out_dtype = in_dtype, capi.INT32 if in_dtype == capi.INT8 else in_dtype
+    d.in_dtype = in_dtype
+    d.out_dtype = capi.INT32 if in_dtype == capi.INT8 else (capi.INT48 if in_dtype == capi.INT16 else in_dtype)
     d.N, d.IH, d.IW, d.IC, d.OC, d.KH, d.KW = n, ih, iw, ic, oc, kh, kw
     d.OH, d.OW = out_hw
     d.out_pad[:], d.stride[:] = list(out_pad), list(stride)
     d.bias_len = bias.shape[0]
-    tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, in_dtype)
+    # INT16 inputs come with INT8 weights and an INT48 bias (int64)
+    tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, capi.INT8 if in_dtype == capi.INT16 else in_dtype)
     tb = ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
-    np_out = {capi.INT32: np.int32, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
+    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
     try:
         to = ctx.empty((n, max(out_hw[0], 0), max(out_hw[1], 0), oc), d.out_dtype, np_out)
         ctx.transpose_conv2d(d, tx, tw, tb, in_zp, w_zp, to)
@@ -147,14 +149,16 @@ def conv3d(ctx, x, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), 
     if out_dhw is None:
         out_dhw = oracle.conv3d_out_dhw((idp, ih, iw), (kd, kh, kw), pad, stride, dilation) or (0, 0, 0)
     d = capi.Conv3dDesc()
-    d.in_dtype, d.out_dtype = in_dtype, capi.INT32 if in_dtype == capi.INT8 else in_dtype
+    d.in_dtype = in_dtype
+    d.out_dtype = capi.INT32 if in_dtype == capi.INT8 else (capi.INT48 if in_dtype == capi.INT16 else in_dtype)
     d.N, d.ID, d.IH, d.IW, d.IC, d.OC, d.KD, d.KH, d.KW = n, idp, ih, iw, ic, oc, kd, kh, kw
     d.OD, d.OH, d.OW = out_dhw
     d.pad[:], d.stride[:], d.dilation[:] = list(pad), list(stride), list(dilation)
     d.bias_len = bias.shape[0]
-    tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, in_dtype)
+    # INT16 inputs come with INT8 weights and an INT48 bias (int64)
+    tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, capi.INT8 if in_dtype == capi.INT16 else in_dtype)
     tb = ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
-    np_out = {capi.INT32: np.int32, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
+    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
     try:
         to = ctx.empty((n,) + tuple(out_dhw) + (oc,), d.out_dtype, np_out)
         ctx.conv3d(d, tx, tw, tb, in_zp, w_zp, to)

@@ -104,3 +104,52 @@ def test_int16_argument_rules(ctx):
                                  ctx.empty((1, 4, 4, 2), capi.INT8, np.int8))
     for t in list(ctx._owned):
         ctx._free(t)
+
+
+@pytest.mark.parametrize("geom", [((2, 6, 7, 16), (8, 3, 3, 16), (0, 1, -1, 0), (2, 2)), ((1, 9, 5, 12), (5, 2, 4, 12), (1, 1, 0, 2), (1, 3)),
+                                  ((3, 4, 4, 40), (24, 3, 3, 40), (0, 0, 0, 0), (1, 1))])
+@pytest.mark.parametrize("w_zp", [0, 9])
+def test_transpose_conv2d_int16_to_int48(ctx, geom, w_zp):
+    """INT16 x INT8 -> INT48 TRANSPOSE_CONV2D (tensor_ops.cpp:2291): tap flip and hole insertion on operands of two element
+    sizes, then the 64-bit one-result-per-lane kernel"""
+    xs, ws, out_pad, stride = geom
+    rng = np.random.default_rng(xs[1] * 7 + ws[0])
+    x = rng.integers(-32768, 32768, xs).astype(np.int16)
+    w = rng.integers(-128, 128, ws).astype(np.int8)
+    bias = rng.integers(-(1 << 40), 1 << 40, ws[0]).astype(np.int64)
+    got, st = gpu_ops.transpose_conv2d(ctx, x, w, bias, out_pad, stride, w_zp=w_zp)
+    assert st == capi.VALID and got.dtype == np.int64
+    assert np.array_equal(got, oracle.transpose_conv2d("i16", x, w, bias, out_pad, stride, w_zp=w_zp))
+
+
+@pytest.mark.parametrize("geom", [((1, 4, 5, 5, 8), (4, 2, 3, 3, 8), (1, 0, 1, 1, 1, 1), (1, 1, 1), (1, 1, 1)),
+                                  ((2, 6, 7, 4, 12), (6, 3, 1, 2, 12), (1, 2, 0, 0, 1, 0), (2, 1, 1), (1, 2, 1)),
+                                  ((1, 3, 9, 9, 32), (16, 1, 3, 3, 32), (0, 0, 1, 1, 1, 1), (1, 2, 2), (1, 1, 1))])
+@pytest.mark.parametrize("w_zp", [0, -3])
+def test_conv3d_int16_to_int48(ctx, geom, w_zp):
+    """INT16 x INT8 -> INT48 CONV3D (tensor_ops.cpp:2237): depth gather and weight permutation on operands of two element
+    sizes, then the 64-bit one-result-per-lane kernel"""
+    xs, ws, pad, stride, dil = geom
+    rng = np.random.default_rng(xs[2] * 5 + ws[0])
+    x = rng.integers(-32768, 32768, xs).astype(np.int16)
+    w = rng.integers(-128, 128, ws).astype(np.int8)
+    bias = rng.integers(-(1 << 40), 1 << 40, 1 if ws[0] == 6 else ws[0]).astype(np.int64)
+    got, st = gpu_ops.conv3d(ctx, x, w, bias, pad, stride, dil, w_zp=w_zp)
+    assert st == capi.VALID and got.dtype == np.int64
+    assert np.array_equal(got, oracle.conv3d("i16", x, w, bias, pad, stride, dil, w_zp=w_zp))
+
+
+def test_transpose_conv2d_and_conv3d_int16_rules(ctx):
+    x = np.zeros((1, 3, 3, 4), np.int16)
+    w = np.zeros((2, 2, 2, 4), np.int8)
+    with pytest.raises(TmiError, match="Input zero point must be zero"):
+        gpu_ops.transpose_conv2d(ctx, x, w, np.zeros(2, np.int64), in_zp=1)
+    with pytest.raises(TmiError, match="Input zero point must be zero"):
+        gpu_ops.conv3d(ctx, x[None], w[:, None], np.zeros(2, np.int64), in_zp=-1)
+    lim = (1 << 47) - 1
+    one = np.full((1, 1, 1, 8), 32767, np.int16)
+    wt = np.full((1, 1, 1, 8), 127, np.int8)
+    got, st = gpu_ops.transpose_conv2d(ctx, one, wt, np.array([lim], np.int64))
+    assert st == capi.VALID and got.ravel().tolist() == [lim]
+    got, st = gpu_ops.conv3d(ctx, -one[None], wt[None], np.array([-lim - 1], np.int64))
+    assert st == capi.VALID and got.ravel().tolist() == [-lim - 1]

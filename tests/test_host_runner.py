@@ -362,6 +362,26 @@ def test_int16_convolution_and_matmul_graphs(tmp_path):
     got_d = np.load(tmp_path / "accd_out.npy")
     assert got_d.dtype == np.int64 and np.array_equal(got_d, accd)
 
+    # TRANSPOSE_CONV2D and CONV3D on INT16 (tensor_ops.cpp:2237, 2291)
+    wt = rng.integers(-128, 128, (4, 3, 2, 12)).astype(np.int8)
+    bt = rng.integers(-(1 << 40), 1 << 40, 4).astype(np.int64)
+    acct = oracle.transpose_conv2d("i16", x, wt, bt, (0, 1, -1, 0), (2, 2), w_zp=2)
+    x3 = rng.integers(-32768, 32768, (1, 4, 5, 5, 8)).astype(np.int16)
+    w3 = rng.integers(-128, 128, (4, 2, 3, 3, 8)).astype(np.int8)
+    pad3, one3 = (1, 0, 1, 1, 1, 1), (1, 1, 1)
+    acc3 = oracle.conv3d("i16", x3, w3, bt, pad3, one3, one3, w_zp=2)
+    ts = [W.tensor("x", x.shape, np.int16), W.tensor("x3", x3.shape, np.int16), W.tensor("wt", wt.shape, np.int8, wt),
+          W.tensor("w3", w3.shape, np.int8, w3), W.tensor("bt", [4], np.int64, bt), W.tensor("izp", [1], np.int16, [0]),
+          W.tensor("wzp", [1], np.int8, [2]), W.tensor("ot", acct.shape, np.int64), W.tensor("o3", acc3.shape, np.int64)]
+    ops = [W.operator(R.OP_CONST, [], [n]) for n in ("wt", "w3", "bt", "izp", "wzp")]
+    ops.append(W.operator(10, ["x", "wt", "bt", "izp", "wzp"], ["ot"], W.transpose_conv_attr((0, 1, -1, 0), (2, 2), acc_type=6)))
+    ops.append(W.operator(4, ["x3", "w3", "bt", "izp", "wzp"], ["o3"], W.conv_attr(pad3, one3, one3, acc_type=6)))
+    d3 = tmp_path / "t3"
+    d3.mkdir()
+    r = _run(_write_case(d3, W.graph(ts, ops, ["x", "x3"], ["ot", "o3"]), {"x": x, "x3": x3}, ["ot", "o3"]))
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.load(d3 / "ot_out.npy"), acct) and np.array_equal(np.load(d3 / "o3_out.npy"), acc3)
+
     a = rng.integers(-32768, 32768, (2, 20, 33)).astype(np.int16)
     b = rng.integers(-32768, 32768, (2, 33, 7)).astype(np.int16)
     ts = [W.tensor("a", a.shape, np.int16), W.tensor("b", b.shape, np.int16), W.tensor("azp", [1], np.int16, [0]),
