@@ -304,7 +304,8 @@ int tmi_depthwise_conv2d_rescale_clamp(tmi_ctx_t* ctx, const tmi_conv_desc_t* d,
  * Evaluated as a stride-1 CONV2D with flipped taps over the input with stride-1 holes filled with input_zp.
  * INT8 with 3x3 taps, 64 / 96 / 128 input channels and w_zp 0 reads both operands in place (holes and flip are
  * part of the kernel's addressing); otherwise the re-laid-out operands live in the context's scratch buffer.
- * Element types as tmi_conv2d: INT8 -> INT32, FP16 / BF16, and INT16 x INT8 -> INT48 (:2291; clip :2190-2194). */
+ * Element types as tmi_conv2d: INT8 -> INT32, FP16 / BF16 / FP32 (FP32 on the one-element-per-lane kernel, the sum in
+ * the order of the equivalent CONV2D, not the reference's scatter order), INT16 x INT8 -> INT48 (:2291; clip :2190-2194). */
 int tmi_transpose_conv2d(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, const void* in_dev, const void* weight_dev,
                          const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 
@@ -327,7 +328,8 @@ int tmi_transpose_conv2d_noalloc(tmi_ctx_t* ctx, const tmi_tconv_desc_t* d, cons
  * Evaluated as a CONV2D over N*OD images whose channels are the KD depth taps side by side.  INT8 with 3x3 taps in
  * the plane, KD*IC = 64 / 96 / 128 (IC 32 or 64) and w_zp 0 reads both operands in place; otherwise the gathered
  * input and the permuted weights live in the context's scratch buffer.  Element types as tmi_conv2d: INT8 -> INT32,
- * FP16 / BF16, and INT16 x INT8 -> INT48 (:2237; clip :1113-1117). */
+ * FP16 / BF16 / FP32 (FP32 on the one-element-per-lane kernel, the depth taps innermost in the sum), and INT16 x INT8 ->
+ * INT48 (:2237; clip :1113-1117). */
 int tmi_conv3d(tmi_ctx_t* ctx, const tmi_conv3d_desc_t* d, const void* in_dev, const void* weight_dev,
                const void* bias_dev, int32_t in_zp, int32_t w_zp, void* out_dev);
 

@@ -925,8 +925,9 @@ static int validate_tconv(tmi_ctx* ctx, const char* op, const tmi_tconv_desc_t* 
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48 (tensor_ops.cpp:2269), FP16 / BF16 with fp32 accumulation
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48, FP16 / BF16 / FP32 with fp32 accumulation (tensor_ops.cpp:2286-2291)
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 &&
+        d->in_dtype != TMI_FP32)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : d->in_dtype)))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);
@@ -1078,8 +1079,9 @@ static int validate_conv3d(tmi_ctx* ctx, const char* op, const tmi_conv3d_desc_t
 {
     if (!d)
         return fail(ctx, "%s: null descriptor", op);
-    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48 (tensor_ops.cpp:2237), FP16 / BF16 with fp32 accumulation
-    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16)
+    // INT8 x INT8 -> INT32, INT16 x INT8 -> INT48, FP16 / BF16 / FP32 with fp32 accumulation (tensor_ops.cpp:2232-2237)
+    if (d->in_dtype != TMI_INT8 && d->in_dtype != TMI_INT16 && d->in_dtype != TMI_FP16 && d->in_dtype != TMI_BF16 &&
+        d->in_dtype != TMI_FP32)
         return fail(ctx, "%s: input data type not supported for this configuration of operator", op);
     if (d->out_dtype != (d->in_dtype == TMI_INT8 ? TMI_INT32 : (d->in_dtype == TMI_INT16 ? TMI_INT48 : d->in_dtype)))
         return fail(ctx, "%s: Output data type not supported for this configuration of operator", op);

@@ -129,7 +129,7 @@ def transpose_conv2d(ctx, x, w, bias, out_pad=(0, 0, 0, 0), stride=(1, 1), in_zp
     # INT16 inputs come with INT8 weights and an INT48 bias (int64)
     tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, capi.INT8 if in_dtype == capi.INT16 else in_dtype)
     tb = ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
-    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
+    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16, capi.FP32: np.float32}[d.out_dtype]
     try:
         to = ctx.empty((n, max(out_hw[0], 0), max(out_hw[1], 0), oc), d.out_dtype, np_out)
         ctx.transpose_conv2d(d, tx, tw, tb, in_zp, w_zp, to)
@@ -158,7 +158,7 @@ def conv3d(ctx, x, w, bias, pad=(0,) * 6, stride=(1, 1, 1), dilation=(1, 1, 1), 
     # INT16 inputs come with INT8 weights and an INT48 bias (int64)
     tx, tw = ctx.upload(x, in_dtype), ctx.upload(w, capi.INT8 if in_dtype == capi.INT16 else in_dtype)
     tb = ctx.upload(bias, None if bias.dtype != np.uint16 else in_dtype)
-    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16}[d.out_dtype]
+    np_out = {capi.INT32: np.int32, capi.INT48: np.int64, capi.FP16: np.float16, capi.BF16: np.uint16, capi.FP32: np.float32}[d.out_dtype]
     try:
         to = ctx.empty((n,) + tuple(out_dhw) + (oc,), d.out_dtype, np_out)
         ctx.conv3d(d, tx, tw, tb, in_zp, w_zp, to)

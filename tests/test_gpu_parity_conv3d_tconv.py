@@ -171,6 +171,31 @@ def test_fp16_variants_within_dot_product_bound(ctx):
     assert st == capi.VALID and res["ok"], res
 
 
+def test_fp32_variants_within_dot_product_bound(ctx):
+    """FP32 TRANSPOSE_CONV2D and CONV3D (tensor_ops.cpp:2234, 2288) run as a CONV2D on re-laid-out operands: the order of
+    the sum is not the reference's (it scatters TRANSPOSE_CONV2D tap by tap and walks CONV3D's depth taps first), so the
+    test is the DOT_PRODUCT bound against the fp64 oracle, and closeness to the oracle's fp32 loop nest"""
+    rng = np.random.default_rng(13)
+    x = rng.normal(0, 1, (2, 6, 5, 24)).astype(np.float32)
+    w = rng.normal(0, 0.1, (10, 3, 2, 24)).astype(np.float32)
+    b = rng.normal(0, 0.1, 10).astype(np.float32)
+    got, st = gpu_ops.transpose_conv2d(ctx, x, w, b, (0, 1, -1, 1), (2, 3))
+    ref = oracle.transpose_conv2d("f64", x, w, b, (0, 1, -1, 1), (2, 3))
+    bnd = oracle.transpose_conv2d("f64", x, w, b, (0, 1, -1, 1), (2, 3), abs_mode=True)
+    res = dp.check(got.astype(np.float64), ref, bnd, "fp32", dp.kernel_size_bound(6 * 24, "fp32", has_bias=True))
+    assert st == capi.VALID and got.dtype == np.float32 and res["ok"], res
+    assert np.allclose(got, oracle.transpose_conv2d("f32", x, w, b, (0, 1, -1, 1), (2, 3)), rtol=1e-4, atol=1e-5)
+    x3 = rng.normal(0, 1, (1, 4, 5, 5, 12)).astype(np.float32)
+    w3 = rng.normal(0, 0.1, (6, 2, 3, 3, 12)).astype(np.float32)
+    b3 = rng.normal(0, 0.1, 1).astype(np.float32)
+    got, st = gpu_ops.conv3d(ctx, x3, w3, b3, (0, 0, 1, 1, 1, 1))
+    ref = oracle.conv3d("f64", x3, w3, b3, (0, 0, 1, 1, 1, 1))
+    bnd = oracle.conv3d("f64", x3, w3, b3, (0, 0, 1, 1, 1, 1), abs_mode=True)
+    res = dp.check(got.astype(np.float64), ref, bnd, "fp32", dp.kernel_size_bound(18 * 12, "fp32", has_bias=True))
+    assert st == capi.VALID and got.dtype == np.float32 and res["ok"], res
+    assert np.allclose(got, oracle.conv3d("f32", x3, w3, b3, (0, 0, 1, 1, 1, 1)), rtol=1e-4, atol=1e-5)
+
+
 def test_shape_rules_are_errors(ctx):
     x, w, b = np.zeros((1, 2, 2, 1), np.int8), np.zeros((1, 3, 3, 1), np.int8), np.zeros(1, np.int32)
     with pytest.raises(TmiError) as e:
